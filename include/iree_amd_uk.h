@@ -1,0 +1,394 @@
+/*
+ * iree_amd_uk.h - C ABI of the MI355X (gfx950) data-tiled matmul microkernels.
+ *
+ * This is the boundary a host runtime binds to: plain C, plain pointers and
+ * sizes, no C++ or torch types. Every entry point mirrors one public entry point
+ * of the reference microkernel library (runtime/src/iree/builtins/ukernel/ in
+ * the IREE tree, cited per function as REF <file>:<line>) with the same argument
+ * order and meaning. Two things differ, because the work runs on a GPU:
+ *
+ *   - buffer pointers are DEVICE pointers (hipMalloc'ed or otherwise visible to
+ *     the current HIP device); the *_host variants at the end take host
+ *     pointers and stage through device memory;
+ *   - the trailing `cpu_data` argument of the reference is kept (and ignored) so
+ *     that argument lists stay positionally identical, and one extra trailing
+ *     `void* stream` (a hipStream_t, NULL = the null stream) is appended.
+ *     Launches are asynchronous on that stream.
+ *
+ * All offsets, strides and sizes are in ELEMENTS, not bytes, as in the
+ * reference. Every function that can fail returns an int: 0 on success, else
+ * one of the IREE_AMD_UK_STATUS_* codes (numerically the low 5 bits of
+ * iree_status_code_t, REF runtime/src/iree/hal/local/executable_plugin.h:221-259)
+ * and the call has launched nothing. The reference validates only in debug
+ * builds (REF mmt4d.c:12-48, pack.c:51-103, unpack.c:32-81); this library always
+ * validates.
+ */
+#ifndef IREE_AMD_UK_H_
+#define IREE_AMD_UK_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#if defined(_WIN32)
+#define IREE_AMD_UK_EXPORT
+#else
+#define IREE_AMD_UK_EXPORT __attribute__((visibility("default")))
+#endif
+
+typedef int64_t iree_amd_uk_index_t; /* REF common.h:269-275 (iree_uk_index_t) */
+
+/*===------------------------------------------------------------------------===
+ * Status codes (subset of iree_status_code_t that this library returns).
+ *===------------------------------------------------------------------------===*/
+#define IREE_AMD_UK_STATUS_OK 0
+#define IREE_AMD_UK_STATUS_INVALID_ARGUMENT 3
+#define IREE_AMD_UK_STATUS_NOT_FOUND 5
+#define IREE_AMD_UK_STATUS_FAILED_PRECONDITION 9
+#define IREE_AMD_UK_STATUS_OUT_OF_RANGE 11
+#define IREE_AMD_UK_STATUS_UNIMPLEMENTED 12
+#define IREE_AMD_UK_STATUS_INTERNAL 13
+#define IREE_AMD_UK_STATUS_UNAVAILABLE 14
+
+/*===------------------------------------------------------------------------===
+ * Flag words. Numerically identical to REF exported_bits.h:29-106, which the
+ * reference declares "set in stone" (exported_bits.h:15-17).
+ *===------------------------------------------------------------------------===*/
+
+/* mmt4d: low byte = (lhs, rhs, out) element type tuple. REF exported_bits.h:29-41 */
+#define IREE_AMD_UK_FLAG_MMT4D_TYPE_MASK 0xFF
+#define IREE_AMD_UK_FLAG_MMT4D_TYPE_NONE 0x00
+#define IREE_AMD_UK_FLAG_MMT4D_TYPE_F32F32F32 0x01
+#define IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32 0x02
+#define IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F32 0x03
+#define IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F16 0x04
+#define IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16F32 0x05
+#define IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16BF16 0x06
+#define IREE_AMD_UK_FLAG_MMT4D_TYPE_S16S16S32 0x07
+#define IREE_AMD_UK_FLAG_MMT4D_TYPE_S16U4S32 0x08
+#define IREE_AMD_UK_FLAG_MMT4D_TYPE_S16S8S32 0x09
+#define IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S4S32 0x0A
+/* Extension: the reference enum ends at 0x0A (END = 0x0B, exported_bits.h:41).
+ * fp8 e4m3fn x e4m3fn -> f32 takes the next free value. Operand decoding follows
+ * OCP/IEEE e4m3fn (subnormals kept), which is what the gfx950 fp8 MFMAs do; the
+ * reference's scalar helper flushes subnormals (REF base/internal/math.h:322). */
+#define IREE_AMD_UK_FLAG_MMT4D_TYPE_F8E4M3F8E4M3F32 0x0B
+#define IREE_AMD_UK_FLAG_MMT4D_TYPE_END 0x0C
+
+/* mmt4d bit flags. REF exported_bits.h:44-46 */
+#define IREE_AMD_UK_FLAG_MMT4D_ACCUMULATE 0x100
+#define IREE_AMD_UK_FLAG_MMT4D_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION 0x200
+#define IREE_AMD_UK_FLAG_MMT4D_SKIP_INTERMEDIATE_ROUNDINGS 0x400
+
+/* iree_amd_uk_mmt4d_info result bits. REF exported_bits.h:49 */
+#define IREE_AMD_UK_FLAG_MMT4D_INFO_HAVE_ARCHITECTURE_SPECIFIC_TILE_FUNCTION 0x1
+
+/* pack. REF exported_bits.h:56-66 */
+#define IREE_AMD_UK_FLAG_PACK_TYPE_MASK 0xFF
+#define IREE_AMD_UK_FLAG_PACK_TYPE_NONE 0x00
+#define IREE_AMD_UK_FLAG_PACK_TYPE_F32F32 0x01
+#define IREE_AMD_UK_FLAG_PACK_TYPE_I8I8 0x02 /* also used for 1-byte fp8 */
+#define IREE_AMD_UK_FLAG_PACK_TYPE_I32I32 0x03
+#define IREE_AMD_UK_FLAG_PACK_TYPE_F16F16 0x04
+#define IREE_AMD_UK_FLAG_PACK_TYPE_BF16BF16 0x05
+#define IREE_AMD_UK_FLAG_PACK_TRANSPOSE_INNER 0x100
+#define IREE_AMD_UK_FLAG_PACK_TRANSPOSE_OUTER 0x200
+
+/* unpack. REF exported_bits.h:73-83 (0x02 is reserved, no I8 unpack) */
+#define IREE_AMD_UK_FLAG_UNPACK_TYPE_MASK 0xFF
+#define IREE_AMD_UK_FLAG_UNPACK_TYPE_NONE 0x00
+#define IREE_AMD_UK_FLAG_UNPACK_TYPE_F32F32 0x01
+#define IREE_AMD_UK_FLAG_UNPACK_TYPE_I32I32 0x03
+#define IREE_AMD_UK_FLAG_UNPACK_TYPE_F16F16 0x04
+#define IREE_AMD_UK_FLAG_UNPACK_TYPE_BF16BF16 0x05
+#define IREE_AMD_UK_FLAG_UNPACK_TRANSPOSE_INNER 0x100
+#define IREE_AMD_UK_FLAG_UNPACK_TRANSPOSE_OUTER 0x200
+
+/* query_tile_sizes. REF exported_bits.h:91-106 */
+#define IREE_AMD_UK_FLAG_QUERY_TILE_SIZES_OPERAND_ROLE_MASK 0xFF
+#define IREE_AMD_UK_FLAG_QUERY_TILE_SIZES_OPERAND_ROLE_NONE 0x00
+#define IREE_AMD_UK_FLAG_QUERY_TILE_SIZES_OPERAND_ROLE_LHS 0x01
+#define IREE_AMD_UK_FLAG_QUERY_TILE_SIZES_OPERAND_ROLE_RHS 0x02
+#define IREE_AMD_UK_FLAG_QUERY_TILE_SIZES_OPERAND_ROLE_RESULT 0x03
+#define IREE_AMD_UK_FLAG_QUERY_TILE_SIZES_OPERATION_MASK 0xFF00
+#define IREE_AMD_UK_FLAG_QUERY_TILE_SIZES_OPERATION_NONE 0x0000
+#define IREE_AMD_UK_FLAG_QUERY_TILE_SIZES_OPERATION_MATMUL_F32F32F32 0x0100
+#define IREE_AMD_UK_FLAG_QUERY_TILE_SIZES_OPERATION_MATMUL_I8I8I32 0x0200
+#define IREE_AMD_UK_FLAG_QUERY_TILE_SIZES_OPERATION_MATMUL_F16F16F32 0x0300
+#define IREE_AMD_UK_FLAG_QUERY_TILE_SIZES_OPERATION_MATMUL_F16F16F16 0x0400
+#define IREE_AMD_UK_FLAG_QUERY_TILE_SIZES_OPERATION_MATMUL_BF16BF16F32 0x0500
+#define IREE_AMD_UK_FLAG_QUERY_TILE_SIZES_OPERATION_MATMUL_BF16BF16BF16 0x0600
+/* Extension (no reference counterpart): fp8 e4m3fn matmul. */
+#define IREE_AMD_UK_FLAG_QUERY_TILE_SIZES_OPERATION_MATMUL_F8E4M3F8E4M3F32 0x0B00
+
+/*===------------------------------------------------------------------------===
+ * mmt4d
+ *
+ *   out[i][j][i0][j0] (+)= sum_k sum_k0 lhs[i][k][i0][k0] * rhs[j][k][j0][k0]
+ *
+ * for i<M, j<N, k<K (M, N, K are OUTER tile counts), i0<M0, j0<N0, k0<K0. The
+ * three inner dimensions of every operand are contiguous; `*_stride0` is the
+ * distance in elements between consecutive outermost indices and need not be
+ * tight. 4-bit RHS elements are packed two per byte, even k0 in the low nibble
+ * (REF mmt4d_tile_generic.c:37-44,132-135). M==0, N==0 or (K==0 with
+ * ACCUMULATE) return without touching `out`; K==0 without ACCUMULATE zero-fills
+ * (REF mmt4d.c:105-113).
+ *===------------------------------------------------------------------------===*/
+
+/* Field order = REF mmt4d_internal.h:14-32 (iree_uk_mmt4d_params_t). */
+typedef struct iree_amd_uk_mmt4d_params_t {
+  const void* lhs_buffer;
+  iree_amd_uk_index_t lhs_offset;
+  iree_amd_uk_index_t lhs_stride0;
+  const void* rhs_buffer;
+  iree_amd_uk_index_t rhs_offset;
+  iree_amd_uk_index_t rhs_stride0;
+  void* out_buffer;
+  iree_amd_uk_index_t out_offset;
+  iree_amd_uk_index_t out_stride0;
+  iree_amd_uk_index_t M;
+  iree_amd_uk_index_t N;
+  iree_amd_uk_index_t K;
+  int32_t M0;
+  int32_t N0;
+  int32_t K0;
+  uint32_t flags;
+  const uint64_t* cpu_data; /* accepted, ignored */
+} iree_amd_uk_mmt4d_params_t;
+
+/* Replaces REF mmt4d.h:14-21 / mmt4d.c:151-177 (iree_uk_mmt4d). */
+IREE_AMD_UK_EXPORT int iree_amd_uk_mmt4d(
+    const void* lhs_buffer, iree_amd_uk_index_t lhs_offset,
+    iree_amd_uk_index_t lhs_stride0, const void* rhs_buffer,
+    iree_amd_uk_index_t rhs_offset, iree_amd_uk_index_t rhs_stride0,
+    void* out_buffer, iree_amd_uk_index_t out_offset,
+    iree_amd_uk_index_t out_stride0, iree_amd_uk_index_t M,
+    iree_amd_uk_index_t N, iree_amd_uk_index_t K, int32_t M0, int32_t N0,
+    int32_t K0, uint32_t flags, const uint64_t* cpu_data, void* stream);
+
+/* Replaces REF mmt4d_internal.h:34 / mmt4d.c:115-141 (iree_uk_mmt4d_p). */
+IREE_AMD_UK_EXPORT int iree_amd_uk_mmt4d_p(
+    const iree_amd_uk_mmt4d_params_t* params, void* stream);
+
+/* Replaces REF mmt4d.h:23-25 / mmt4d.c:179-185 (iree_uk_mmt4d_info): bit 0 set
+ * when a gfx950 MFMA kernel (not the generic one) serves this type and tile. */
+IREE_AMD_UK_EXPORT uint32_t iree_amd_uk_mmt4d_info(int32_t M0, int32_t N0,
+                                                   int32_t K0, uint32_t flags,
+                                                   const uint64_t* cpu_data);
+
+/*===------------------------------------------------------------------------===
+ * pack: row-major (strided) 2-D source -> 4-D tiled destination with padding.
+ *
+ * With (O0,O1,T0,T1) = out_size0..3 and destination strides
+ * (out_stride0, T0*T1, T1, 1); TRANSPOSE_OUTER swaps (O0,O1) and their strides,
+ * TRANSPOSE_INNER swaps (T0,T1) and their strides; then for every
+ * a<O0,b<O1,c<T0,d<T1 the element (a,b,c,d) receives in[a*T0+c][b*T1+d] when that
+ * is inside in_size0 x in_size1 and the low element-bits of `padding_value`
+ * otherwise (REF tools/pack_test.c:13-71, pack.h:16-25). out_stride1 must equal
+ * out_size2*out_size3 (REF pack.c:72). Any out_size == 0 writes nothing
+ * (REF pack.c:106-109).
+ *===------------------------------------------------------------------------===*/
+
+/* Field order = REF pack_internal.h:12-30 (iree_uk_pack_params_t). */
+typedef struct iree_amd_uk_pack_params_t {
+  const void* in_buffer;
+  iree_amd_uk_index_t in_offset;
+  iree_amd_uk_index_t in_stride0;
+  iree_amd_uk_index_t in_stride1;
+  void* out_buffer;
+  iree_amd_uk_index_t out_offset;
+  iree_amd_uk_index_t out_stride0;
+  iree_amd_uk_index_t out_stride1;
+  iree_amd_uk_index_t in_size0;
+  iree_amd_uk_index_t in_size1;
+  iree_amd_uk_index_t out_size0;
+  iree_amd_uk_index_t out_size1;
+  iree_amd_uk_index_t out_size2;
+  iree_amd_uk_index_t out_size3;
+  uint64_t padding_value;
+  uint32_t flags;
+  const uint64_t* cpu_data; /* accepted, ignored */
+} iree_amd_uk_pack_params_t;
+
+/* Replaces REF pack.h:26-34 / pack.c:325-352 (iree_uk_pack). */
+IREE_AMD_UK_EXPORT int iree_amd_uk_pack(
+    const void* in_buffer, iree_amd_uk_index_t in_offset,
+    iree_amd_uk_index_t in_stride0, iree_amd_uk_index_t in_stride1,
+    void* out_buffer, iree_amd_uk_index_t out_offset,
+    iree_amd_uk_index_t out_stride0, iree_amd_uk_index_t out_stride1,
+    iree_amd_uk_index_t in_size0, iree_amd_uk_index_t in_size1,
+    iree_amd_uk_index_t out_size0, iree_amd_uk_index_t out_size1,
+    iree_amd_uk_index_t out_size2, iree_amd_uk_index_t out_size3,
+    uint64_t padding_value, uint32_t flags, const uint64_t* cpu_data,
+    void* stream);
+
+/* Replaces REF pack_internal.h:32 / pack.c:315-323 (iree_uk_pack_p). */
+IREE_AMD_UK_EXPORT int iree_amd_uk_pack_p(
+    const iree_amd_uk_pack_params_t* params, void* stream);
+
+/*===------------------------------------------------------------------------===
+ * unpack: inverse of pack without padding. Copies only elements inside
+ * out_size0 x out_size1; every other destination element is left untouched
+ * (REF tools/unpack_test.c:13-58). in_stride1 must equal in_size2*in_size3
+ * (REF unpack.c:49). out_size0 == 0 or out_size1 == 0 writes nothing
+ * (REF unpack.c:84-86).
+ *===------------------------------------------------------------------------===*/
+
+/* Field order = REF unpack_internal.h:12-29 (iree_uk_unpack_params_t). */
+typedef struct iree_amd_uk_unpack_params_t {
+  const void* in_buffer;
+  iree_amd_uk_index_t in_offset;
+  iree_amd_uk_index_t in_stride0;
+  iree_amd_uk_index_t in_stride1;
+  void* out_buffer;
+  iree_amd_uk_index_t out_offset;
+  iree_amd_uk_index_t out_stride0;
+  iree_amd_uk_index_t out_stride1;
+  iree_amd_uk_index_t in_size0;
+  iree_amd_uk_index_t in_size1;
+  iree_amd_uk_index_t in_size2;
+  iree_amd_uk_index_t in_size3;
+  iree_amd_uk_index_t out_size0;
+  iree_amd_uk_index_t out_size1;
+  uint32_t flags;
+  const uint64_t* cpu_data; /* accepted, ignored */
+} iree_amd_uk_unpack_params_t;
+
+/* Replaces REF unpack.h:17-25 / unpack.c:259-285 (iree_uk_unpack). */
+IREE_AMD_UK_EXPORT int iree_amd_uk_unpack(
+    const void* in_buffer, iree_amd_uk_index_t in_offset,
+    iree_amd_uk_index_t in_stride0, iree_amd_uk_index_t in_stride1,
+    void* out_buffer, iree_amd_uk_index_t out_offset,
+    iree_amd_uk_index_t out_stride0, iree_amd_uk_index_t out_stride1,
+    iree_amd_uk_index_t in_size0, iree_amd_uk_index_t in_size1,
+    iree_amd_uk_index_t in_size2, iree_amd_uk_index_t in_size3,
+    iree_amd_uk_index_t out_size0, iree_amd_uk_index_t out_size1,
+    uint32_t flags, const uint64_t* cpu_data, void* stream);
+
+/* Replaces REF unpack_internal.h:31 / unpack.c:249-257 (iree_uk_unpack_p). */
+IREE_AMD_UK_EXPORT int iree_amd_uk_unpack_p(
+    const iree_amd_uk_unpack_params_t* params, void* stream);
+
+/*===------------------------------------------------------------------------===
+ * query_tile_sizes_2d: (operation, operand role) -> (tile_size0, tile_size1).
+ * LHS -> (M0,K0), RHS -> (N0,K0), RESULT -> (M0,N0) of the matmul tile chosen
+ * for gfx950 (REF query_tile_sizes.c:43-63 for the role mapping). `size0` /
+ * `size1` are the operand's own dimensions (INT64_MIN = dynamic): a static M
+ * (LHS/RESULT size0) or N (RHS size0, RESULT size1) below 32 narrows that tile
+ * dimension to the next power of two >= the size, as the reference's
+ * compile-time chooser does for narrow matmuls
+ * (REF compiler/src/iree/compiler/Codegen/Common/CPU/CPUMaterializeEncodingPass.cpp:284-377).
+ *===------------------------------------------------------------------------===*/
+
+/* REF query_tile_sizes.h:18-23 */
+typedef struct iree_amd_uk_query_tile_sizes_2d_params_t {
+  uint32_t flags;
+  iree_amd_uk_index_t size0;
+  iree_amd_uk_index_t size1;
+  const uint64_t* cpu_data; /* accepted, ignored */
+} iree_amd_uk_query_tile_sizes_2d_params_t;
+
+/* REF query_tile_sizes.h:25-28 */
+typedef struct iree_amd_uk_query_tile_sizes_2d_out_params_t {
+  iree_amd_uk_index_t tile_size0;
+  iree_amd_uk_index_t tile_size1;
+} iree_amd_uk_query_tile_sizes_2d_out_params_t;
+
+/* Replaces REF query_tile_sizes.h:29-31 / query_tile_sizes.c:65-75. Host-only,
+ * touches no device. Returns INVALID_ARGUMENT for an unknown operation/role. */
+IREE_AMD_UK_EXPORT int iree_amd_uk_query_tile_sizes_2d(
+    const iree_amd_uk_query_tile_sizes_2d_params_t* params,
+    iree_amd_uk_query_tile_sizes_2d_out_params_t* out_params);
+
+/*===------------------------------------------------------------------------===
+ * Grouped int4-weight dequantising matmul (the dispatch that quantised LLM
+ * inference lowers to; there is no reference ukernel for it, the semantics are
+ * the fused dequantisation + matmul pattern of
+ * REF compiler/src/iree/compiler/GlobalOptimization/FuseDequantizationMatmul.cpp:53-159
+ * and GlobalOptimization/test/fuse_dequantization_matmul.mlir:127-158):
+ *
+ *   out[m][n] = sum_g sum_k  x[m][g*gs+k] * ((float)w[n][g][k] - zp[n][g]) * s[n][g]
+ *
+ * x: f16 [M][K] row-major. w: unsigned 4-bit [N][K], two per byte, even k in the
+ * low nibble (REF tests/e2e/linalg/subbyte_to_fp.mlir, mmt4d_tile_generic.c:132-135).
+ * scales: f16 [N][K/gs]. zero points: either f16 [N][K/gs] (the reference's
+ * form: a floating tensor subtracted after uitofp) or packed uint4 [N][K/gs]
+ * (two per byte, even group in the low nibble) when ..._ZP_U4 is set. f32
+ * accumulation, result rounded to f16 once (RNE). out: f16 [M][N] row-major.
+ * Requires K % group_size == 0, group_size % 32 == 0, 1 <= M.
+ *===------------------------------------------------------------------------===*/
+#define IREE_AMD_UK_FLAG_DEQUANT_MATMUL_ZP_F16 0x0
+#define IREE_AMD_UK_FLAG_DEQUANT_MATMUL_ZP_U4 0x1
+
+IREE_AMD_UK_EXPORT int iree_amd_uk_dequant_matmul_i4(
+    const void* x_buffer, const void* w_buffer, const void* scale_buffer,
+    const void* zp_buffer, void* out_buffer, iree_amd_uk_index_t M,
+    iree_amd_uk_index_t N, iree_amd_uk_index_t K,
+    iree_amd_uk_index_t group_size, uint32_t flags, void* stream);
+
+/*===------------------------------------------------------------------------===
+ * Pieces of the fp8 Llama-style MLP block (no reference ukernel; the pattern is
+ * REF compiler/src/iree/compiler/GlobalOptimization/FuseSiluHorizontalMatmul.cpp:32-82,113-140:
+ * h = silu(x Wg^T) * (x Wu^T), y = h Wd^T, silu(g) = g / (1 + exp(-g))).
+ *===------------------------------------------------------------------------===*/
+
+/* out_fp8[i] = e4m3fn_rne(clamp(in_f16[i] * inv_scale, +-448)), n elements.
+ * Conversion is OCP e4m3fn round-to-nearest-even with saturation (values above
+ * 448 in magnitude clamp to +-448 instead of the reference helper's NaN,
+ * REF base/internal/math.h:363-423); NaN stays NaN. */
+IREE_AMD_UK_EXPORT int iree_amd_uk_quantize_f16_to_f8e4m3(
+    const void* in_f16, void* out_fp8, iree_amd_uk_index_t n, float inv_scale,
+    void* stream);
+
+/* out_fp8[m][n] = e4m3fn( silu(gate[m][n]*gate_scale) * (up[m][n]*up_scale)
+ *                          * inv_out_scale ), gate/up f32 row-major [rows][cols]
+ * with row pitch `ld` elements. */
+IREE_AMD_UK_EXPORT int iree_amd_uk_silu_mul_quantize(
+    const void* gate_f32, const void* up_f32, void* out_fp8,
+    iree_amd_uk_index_t rows, iree_amd_uk_index_t cols, iree_amd_uk_index_t ld,
+    float gate_scale, float up_scale, float inv_out_scale, void* stream);
+
+/*===------------------------------------------------------------------------===
+ * Thin device ABI, so that a pure-C host (the HAL executable plugin) needs no
+ * HIP headers. Mirrors the handful of driver calls the reference's own HIP HAL
+ * driver resolves at run time
+ * (REF runtime/src/iree/hal/drivers/hip/dynamic_symbol_tables.h).
+ *===------------------------------------------------------------------------===*/
+IREE_AMD_UK_EXPORT int iree_amd_uk_device_count(int* out_count);
+IREE_AMD_UK_EXPORT int iree_amd_uk_device_set(int ordinal);
+IREE_AMD_UK_EXPORT int iree_amd_uk_device_malloc(void** out_ptr, uint64_t bytes);
+IREE_AMD_UK_EXPORT int iree_amd_uk_device_free(void* ptr);
+IREE_AMD_UK_EXPORT int iree_amd_uk_memcpy_h2d(void* dst, const void* src,
+                                              uint64_t bytes, void* stream);
+IREE_AMD_UK_EXPORT int iree_amd_uk_memcpy_d2h(void* dst, const void* src,
+                                              uint64_t bytes, void* stream);
+IREE_AMD_UK_EXPORT int iree_amd_uk_stream_create(void** out_stream);
+IREE_AMD_UK_EXPORT int iree_amd_uk_stream_destroy(void* stream);
+IREE_AMD_UK_EXPORT int iree_amd_uk_stream_synchronize(void* stream);
+/* Human-readable text of the calling thread's last non-OK status ("" if none). */
+IREE_AMD_UK_EXPORT const char* iree_amd_uk_last_error(void);
+/* Library version: (major << 16) | minor. */
+IREE_AMD_UK_EXPORT uint32_t iree_amd_uk_version(void);
+
+/*===------------------------------------------------------------------------===
+ * Host-pointer variants: same parameter structs, but every buffer is a HOST
+ * pointer (what IREE's local-task/local-sync HAL hands an import,
+ * REF samples/custom_dispatch/cpu/plugin/README.md:90-97). Each call stages the
+ * touched byte ranges to device memory, runs the device entry point above,
+ * copies the destination range back and synchronises before returning.
+ * Reentrant; safe to call concurrently from several threads.
+ *===------------------------------------------------------------------------===*/
+IREE_AMD_UK_EXPORT int iree_amd_uk_mmt4d_host(
+    const iree_amd_uk_mmt4d_params_t* params);
+IREE_AMD_UK_EXPORT int iree_amd_uk_pack_host(
+    const iree_amd_uk_pack_params_t* params);
+IREE_AMD_UK_EXPORT int iree_amd_uk_unpack_host(
+    const iree_amd_uk_unpack_params_t* params);
+
+#ifdef __cplusplus
+} /* extern "C" */
+#endif
+
+#endif /* IREE_AMD_UK_H_ */

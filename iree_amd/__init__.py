@@ -1,0 +1,22 @@
+"""MI355X (gfx950) implementation of IREE's data-tiled matmul microkernels.
+
+The product is the C-ABI shared library built from ``iree_amd/csrc`` (declared in
+``include/iree_amd_uk.h``). This package is the thin Python host mirror of the
+reference's ukernel entry points (``iree_uk_pack`` / ``iree_uk_mmt4d`` /
+``iree_uk_unpack`` / ``iree_uk_query_tile_sizes_2d``) over that library; torch is
+used only to own device memory and streams.
+"""
+from . import flags  # noqa: F401
+from ._lib import load_library, library_path  # noqa: F401
+from .ukernel import (  # noqa: F401
+    UkError,
+    dequant_matmul_i4,
+    matmul_data_tiled,
+    mmt4d,
+    mmt4d_info,
+    pack,
+    quantize_f16_to_f8e4m3,
+    query_tile_sizes_2d,
+    silu_mul_quantize,
+    unpack,
+)

@@ -1,0 +1,559 @@
+// C-ABI entry points of the gfx950 ukernel library (include/iree_amd_uk.h):
+// argument packing, validation, early returns, kernel selection, the thin
+// device ABI and the host-pointer staging variants. No kernels live here.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "uk_common.h"
+
+namespace uk {
+
+static thread_local char g_last_error[512] = "";
+
+int fail(int status, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_last_error, sizeof g_last_error, fmt, ap);
+  va_end(ap);
+  return status;
+}
+
+int check_hip(hipError_t err, const char* what) {
+  if (err == hipSuccess) return 0;
+  int status = IREE_AMD_UK_STATUS_INTERNAL;
+  if (err == hipErrorNoDevice || err == hipErrorInvalidDevice ||
+      err == hipErrorNotInitialized || err == hipErrorInsufficientDriver) {
+    status = IREE_AMD_UK_STATUS_UNAVAILABLE;
+  } else if (err == hipErrorOutOfMemory) {
+    status = 8;  // RESOURCE_EXHAUSTED
+  }
+  return fail(status, "%s: %s", what, hipGetErrorString(err));
+}
+
+bool mmt4d_type_info(uint32_t flags, Mmt4dTypeInfo* out) {
+  switch (flags & IREE_AMD_UK_FLAG_MMT4D_TYPE_MASK) {
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F32F32F32: *out = {32, 32, 4}; return true;
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32: *out = {8, 8, 4}; return true;
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F32: *out = {16, 16, 4}; return true;
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F16: *out = {16, 16, 2}; return true;
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16F32: *out = {16, 16, 4}; return true;
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16BF16: *out = {16, 16, 2}; return true;
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_S16S16S32: *out = {16, 16, 4}; return true;
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_S16U4S32: *out = {16, 4, 4}; return true;
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_S16S8S32: *out = {16, 8, 4}; return true;
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S4S32: *out = {8, 4, 4}; return true;
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F8E4M3F8E4M3F32: *out = {8, 8, 4}; return true;
+    default: return false;
+  }
+}
+
+int pack_elem_bytes(uint32_t flags) {
+  switch (flags & IREE_AMD_UK_FLAG_PACK_TYPE_MASK) {
+    case IREE_AMD_UK_FLAG_PACK_TYPE_F32F32:
+    case IREE_AMD_UK_FLAG_PACK_TYPE_I32I32: return 4;
+    case IREE_AMD_UK_FLAG_PACK_TYPE_F16F16:
+    case IREE_AMD_UK_FLAG_PACK_TYPE_BF16BF16: return 2;
+    case IREE_AMD_UK_FLAG_PACK_TYPE_I8I8: return 1;
+    default: return 0;
+  }
+}
+
+int unpack_elem_bytes(uint32_t flags) {
+  // Same table minus the 1-byte type, which the reference reserves but does
+  // not define for unpack (exported_bits.h:75-79).
+  if ((flags & IREE_AMD_UK_FLAG_UNPACK_TYPE_MASK) == IREE_AMD_UK_FLAG_PACK_TYPE_I8I8)
+    return 0;
+  return pack_elem_bytes(flags);
+}
+
+static bool fits_i32(int64_t v) { return v >= 0 && v <= 0x7FFFFFFFll; }
+static bool fits_i16(int64_t v) { return v >= 0 && v <= 0x7FFFll; }
+
+// Mirrors the asserts of the reference's iree_uk_mmt4d_validate (mmt4d.c:12-48).
+int validate_mmt4d(const iree_amd_uk_mmt4d_params_t& p) {
+  const uint32_t known =
+      IREE_AMD_UK_FLAG_MMT4D_TYPE_MASK | IREE_AMD_UK_FLAG_MMT4D_ACCUMULATE |
+      IREE_AMD_UK_FLAG_MMT4D_SKIP_INTERMEDIATE_ROUNDINGS |
+      IREE_AMD_UK_FLAG_MMT4D_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION;
+  if (p.flags & ~known)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "mmt4d: unknown flag bits 0x%x", p.flags & ~known);
+  Mmt4dTypeInfo ti;
+  if (!mmt4d_type_info(p.flags, &ti))
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "mmt4d: unknown type 0x%x", p.flags & 0xFF);
+  if (!fits_i32(p.M) || !fits_i32(p.N) || !fits_i32(p.K))
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "mmt4d: M/N/K outside [0, 2^31)");
+  if (!fits_i16(p.M0) || !fits_i16(p.N0) || !fits_i16(p.K0))
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "mmt4d: M0/N0/K0 outside [0, 2^15)");
+  if ((p.K0 * ti.lhs_bits) % 8 || (p.K0 * ti.rhs_bits) % 8)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "mmt4d: K0 rows are not whole bytes");
+  if ((p.lhs_stride0 * ti.lhs_bits) % 8 || (p.rhs_stride0 * ti.rhs_bits) % 8 ||
+      (p.lhs_offset * ti.lhs_bits) % 8 || (p.rhs_offset * ti.rhs_bits) % 8)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "mmt4d: sub-byte stride/offset not on a byte boundary");
+  return 0;
+}
+
+// Mirrors iree_uk_pack_validate (pack.c:51-103). The reference also caps one
+// tile at 4 KiB because of its stack temporary (pack.c:9-49); the GPU kernels
+// have no such buffer, so larger tiles are accepted here.
+int validate_pack(const iree_amd_uk_pack_params_t& p) {
+  const uint32_t known = IREE_AMD_UK_FLAG_PACK_TYPE_MASK |
+                         IREE_AMD_UK_FLAG_PACK_TRANSPOSE_INNER |
+                         IREE_AMD_UK_FLAG_PACK_TRANSPOSE_OUTER;
+  if (p.flags & ~known)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "pack: unknown flag bits 0x%x", p.flags & ~known);
+  if (!pack_elem_bytes(p.flags))
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "pack: unknown type 0x%x", p.flags & 0xFF);
+  if (p.in_size0 < 0 || p.in_size1 < 0 || p.out_size0 < 0 || p.out_size1 < 0 ||
+      p.out_size2 < 0 || p.out_size3 < 0 || p.in_stride0 < 0 ||
+      p.in_stride1 < 0 || p.out_stride0 < 0)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "pack: negative size or stride");
+  if (p.out_stride1 != p.out_size2 * p.out_size3)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "pack: out_stride1 must equal out_size2*out_size3");
+  int64_t o0 = p.out_size0, o1 = p.out_size1, t0 = p.out_size2, t1 = p.out_size3;
+  if (p.flags & IREE_AMD_UK_FLAG_PACK_TRANSPOSE_OUTER) { int64_t t = o0; o0 = o1; o1 = t; }
+  if (p.flags & IREE_AMD_UK_FLAG_PACK_TRANSPOSE_INNER) { int64_t t = t0; t0 = t1; t1 = t; }
+  if (o0 * t0 < p.in_size0 || o1 * t1 < p.in_size1)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "pack: tiled shape does not cover the source");
+  return 0;
+}
+
+// Mirrors iree_uk_unpack_validate (unpack.c:31-81).
+int validate_unpack(const iree_amd_uk_unpack_params_t& p) {
+  const uint32_t known = IREE_AMD_UK_FLAG_UNPACK_TYPE_MASK |
+                         IREE_AMD_UK_FLAG_UNPACK_TRANSPOSE_INNER |
+                         IREE_AMD_UK_FLAG_UNPACK_TRANSPOSE_OUTER;
+  if (p.flags & ~known)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "unpack: unknown flag bits 0x%x", p.flags & ~known);
+  if (!unpack_elem_bytes(p.flags))
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "unpack: unknown type 0x%x", p.flags & 0xFF);
+  if (p.in_size0 < 0 || p.in_size1 < 0 || p.in_size2 < 0 || p.in_size3 < 0 ||
+      p.out_size0 < 0 || p.out_size1 < 0 || p.in_stride0 < 0 ||
+      p.out_stride0 < 0 || p.out_stride1 < 0)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "unpack: negative size or stride");
+  if (p.in_stride1 != p.in_size2 * p.in_size3)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "unpack: in_stride1 must equal in_size2*in_size3");
+  int64_t o0 = p.in_size0, o1 = p.in_size1, t0 = p.in_size2, t1 = p.in_size3;
+  if (p.flags & IREE_AMD_UK_FLAG_UNPACK_TRANSPOSE_OUTER) { int64_t t = o0; o0 = o1; o1 = t; }
+  if (p.flags & IREE_AMD_UK_FLAG_UNPACK_TRANSPOSE_INNER) { int64_t t = t0; t0 = t1; t1 = t; }
+  if (o0 * t0 < p.out_size0 || o1 * t1 < p.out_size1)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "unpack: tiled shape does not cover the destination");
+  return 0;
+}
+
+int device_cu_count() {
+  static int cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (!cached[dev]) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}
+
+// The tile the gfx950 kernels are built around, per operation:
+// M0 = N0 = 32 (one MFMA 32x32 block) and K0 = half the K extent of one MFMA,
+// i.e. exactly the 16 bytes one lane feeds the instruction, so that a packed
+// tile is already in MFMA operand register order.
+struct MatmulTile { int M0, N0, K0; };
+static bool matmul_tile_for_op(uint32_t op, MatmulTile* t) {
+  switch (op) {
+    case IREE_AMD_UK_FLAG_QUERY_TILE_SIZES_OPERATION_MATMUL_I8I8I32:
+      *t = {32, 32, 16}; return true;
+    case IREE_AMD_UK_FLAG_QUERY_TILE_SIZES_OPERATION_MATMUL_F16F16F32:
+    case IREE_AMD_UK_FLAG_QUERY_TILE_SIZES_OPERATION_MATMUL_F16F16F16:
+    case IREE_AMD_UK_FLAG_QUERY_TILE_SIZES_OPERATION_MATMUL_BF16BF16F32:
+    case IREE_AMD_UK_FLAG_QUERY_TILE_SIZES_OPERATION_MATMUL_BF16BF16BF16:
+      *t = {32, 32, 8}; return true;
+    case IREE_AMD_UK_FLAG_QUERY_TILE_SIZES_OPERATION_MATMUL_F8E4M3F8E4M3F32:
+      *t = {32, 32, 16}; return true;
+    case IREE_AMD_UK_FLAG_QUERY_TILE_SIZES_OPERATION_MATMUL_F32F32F32:
+      *t = {32, 32, 4}; return true;
+    default: return false;
+  }
+}
+
+// Narrow dimension handling: a static size below the full tile shrinks the tile
+// to the next power of two that holds it (the reference's compile-time chooser
+// accepts padding up to that power of two and no further,
+// CPUMaterializeEncodingPass.cpp:343-353).
+static int narrow(int full, int64_t size) {
+  if (size < 0 || size >= full) return full;  // dynamic (INT64_MIN) or wide
+  int t = 1;
+  while (t < size) t <<= 1;
+  return t < full ? t : full;
+}
+
+}  // namespace uk
+
+using namespace uk;
+
+//===----------------------------------------------------------------------===//
+// mmt4d
+//===----------------------------------------------------------------------===//
+
+extern "C" int iree_amd_uk_mmt4d_p(const iree_amd_uk_mmt4d_params_t* params,
+                                   void* stream) {
+  if (!params) return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "mmt4d: null params");
+  const iree_amd_uk_mmt4d_params_t& p = *params;
+  UK_RETURN_IF_ERROR(validate_mmt4d(p));
+  // Early return exactly as the reference (mmt4d.c:105-113).
+  if (p.M == 0 || p.N == 0 ||
+      (p.K == 0 && (p.flags & IREE_AMD_UK_FLAG_MMT4D_ACCUMULATE)))
+    return 0;
+  if (p.M0 == 0 || p.N0 == 0) return 0;  // empty tiles: nothing to write
+  if (!p.lhs_buffer && p.K && p.K0) return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "mmt4d: null lhs");
+  if (!p.rhs_buffer && p.K && p.K0) return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "mmt4d: null rhs");
+  if (!p.out_buffer) return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "mmt4d: null out");
+  hipStream_t s = (hipStream_t)stream;
+  if (mmt4d_mfma_supported(p.flags, p.M0, p.N0, p.K0)) {
+    int st = launch_mmt4d_mfma(p, s);
+    if (st != IREE_AMD_UK_STATUS_NOT_FOUND) return st;
+  }
+  if (!(p.flags & IREE_AMD_UK_FLAG_MMT4D_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION)) {
+    // The reference asserts here (mmt4d.c:128-138); a release build would
+    // crash on a null tile function. Report instead.
+    return fail(IREE_AMD_UK_STATUS_UNIMPLEMENTED,
+                "mmt4d: no gfx950 MFMA kernel for type 0x%x tile %dx%dx%d (or "
+                "operands not 16-byte aligned) and generic fallback not allowed",
+                p.flags & 0xFF, p.M0, p.N0, p.K0);
+  }
+  return launch_mmt4d_generic(p, s);
+}
+
+extern "C" int iree_amd_uk_mmt4d(
+    const void* lhs_buffer, iree_amd_uk_index_t lhs_offset,
+    iree_amd_uk_index_t lhs_stride0, const void* rhs_buffer,
+    iree_amd_uk_index_t rhs_offset, iree_amd_uk_index_t rhs_stride0,
+    void* out_buffer, iree_amd_uk_index_t out_offset,
+    iree_amd_uk_index_t out_stride0, iree_amd_uk_index_t M,
+    iree_amd_uk_index_t N, iree_amd_uk_index_t K, int32_t M0, int32_t N0,
+    int32_t K0, uint32_t flags, const uint64_t* cpu_data, void* stream) {
+  iree_amd_uk_mmt4d_params_t p = {lhs_buffer, lhs_offset, lhs_stride0,
+                                  rhs_buffer, rhs_offset, rhs_stride0,
+                                  out_buffer, out_offset, out_stride0,
+                                  M, N, K, M0, N0, K0, flags, cpu_data};
+  return iree_amd_uk_mmt4d_p(&p, stream);
+}
+
+extern "C" uint32_t iree_amd_uk_mmt4d_info(int32_t M0, int32_t N0, int32_t K0,
+                                           uint32_t flags,
+                                           const uint64_t* cpu_data) {
+  (void)cpu_data;
+  return mmt4d_mfma_supported(flags, M0, N0, K0)
+             ? IREE_AMD_UK_FLAG_MMT4D_INFO_HAVE_ARCHITECTURE_SPECIFIC_TILE_FUNCTION
+             : 0u;
+}
+
+//===----------------------------------------------------------------------===//
+// pack / unpack
+//===----------------------------------------------------------------------===//
+
+extern "C" int iree_amd_uk_pack_p(const iree_amd_uk_pack_params_t* params,
+                                  void* stream) {
+  if (!params) return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "pack: null params");
+  const iree_amd_uk_pack_params_t& p = *params;
+  UK_RETURN_IF_ERROR(validate_pack(p));
+  // Early return as the reference (pack.c:106-109).
+  if (p.out_size0 == 0 || p.out_size1 == 0 || p.out_size2 == 0 || p.out_size3 == 0)
+    return 0;
+  if (!p.out_buffer) return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "pack: null out");
+  if (!p.in_buffer && p.in_size0 && p.in_size1)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "pack: null in");
+  return launch_pack(p, (hipStream_t)stream);
+}
+
+extern "C" int iree_amd_uk_pack(
+    const void* in_buffer, iree_amd_uk_index_t in_offset,
+    iree_amd_uk_index_t in_stride0, iree_amd_uk_index_t in_stride1,
+    void* out_buffer, iree_amd_uk_index_t out_offset,
+    iree_amd_uk_index_t out_stride0, iree_amd_uk_index_t out_stride1,
+    iree_amd_uk_index_t in_size0, iree_amd_uk_index_t in_size1,
+    iree_amd_uk_index_t out_size0, iree_amd_uk_index_t out_size1,
+    iree_amd_uk_index_t out_size2, iree_amd_uk_index_t out_size3,
+    uint64_t padding_value, uint32_t flags, const uint64_t* cpu_data,
+    void* stream) {
+  iree_amd_uk_pack_params_t p = {in_buffer, in_offset, in_stride0, in_stride1,
+                                 out_buffer, out_offset, out_stride0, out_stride1,
+                                 in_size0, in_size1, out_size0, out_size1,
+                                 out_size2, out_size3, padding_value, flags,
+                                 cpu_data};
+  return iree_amd_uk_pack_p(&p, stream);
+}
+
+extern "C" int iree_amd_uk_unpack_p(const iree_amd_uk_unpack_params_t* params,
+                                    void* stream) {
+  if (!params) return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "unpack: null params");
+  const iree_amd_uk_unpack_params_t& p = *params;
+  UK_RETURN_IF_ERROR(validate_unpack(p));
+  // Early return as the reference (unpack.c:84-86).
+  if (p.out_size0 == 0 || p.out_size1 == 0) return 0;
+  if (!p.out_buffer || !p.in_buffer)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "unpack: null buffer");
+  return launch_unpack(p, (hipStream_t)stream);
+}
+
+extern "C" int iree_amd_uk_unpack(
+    const void* in_buffer, iree_amd_uk_index_t in_offset,
+    iree_amd_uk_index_t in_stride0, iree_amd_uk_index_t in_stride1,
+    void* out_buffer, iree_amd_uk_index_t out_offset,
+    iree_amd_uk_index_t out_stride0, iree_amd_uk_index_t out_stride1,
+    iree_amd_uk_index_t in_size0, iree_amd_uk_index_t in_size1,
+    iree_amd_uk_index_t in_size2, iree_amd_uk_index_t in_size3,
+    iree_amd_uk_index_t out_size0, iree_amd_uk_index_t out_size1,
+    uint32_t flags, const uint64_t* cpu_data, void* stream) {
+  iree_amd_uk_unpack_params_t p = {in_buffer, in_offset, in_stride0, in_stride1,
+                                   out_buffer, out_offset, out_stride0, out_stride1,
+                                   in_size0, in_size1, in_size2, in_size3,
+                                   out_size0, out_size1, flags, cpu_data};
+  return iree_amd_uk_unpack_p(&p, stream);
+}
+
+//===----------------------------------------------------------------------===//
+// query_tile_sizes_2d
+//===----------------------------------------------------------------------===//
+
+extern "C" int iree_amd_uk_query_tile_sizes_2d(
+    const iree_amd_uk_query_tile_sizes_2d_params_t* params,
+    iree_amd_uk_query_tile_sizes_2d_out_params_t* out_params) {
+  if (!params || !out_params)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "query_tile_sizes: null params");
+  MatmulTile t;
+  if (!matmul_tile_for_op(params->flags & IREE_AMD_UK_FLAG_QUERY_TILE_SIZES_OPERATION_MASK, &t))
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "query_tile_sizes: unknown operation 0x%x",
+                params->flags & IREE_AMD_UK_FLAG_QUERY_TILE_SIZES_OPERATION_MASK);
+  // Role mapping of the reference (query_tile_sizes.c:43-63).
+  switch (params->flags & IREE_AMD_UK_FLAG_QUERY_TILE_SIZES_OPERAND_ROLE_MASK) {
+    case IREE_AMD_UK_FLAG_QUERY_TILE_SIZES_OPERAND_ROLE_LHS:
+      out_params->tile_size0 = narrow(t.M0, params->size0);
+      out_params->tile_size1 = t.K0;
+      return 0;
+    case IREE_AMD_UK_FLAG_QUERY_TILE_SIZES_OPERAND_ROLE_RHS:
+      out_params->tile_size0 = narrow(t.N0, params->size0);
+      out_params->tile_size1 = t.K0;
+      return 0;
+    case IREE_AMD_UK_FLAG_QUERY_TILE_SIZES_OPERAND_ROLE_RESULT:
+      out_params->tile_size0 = narrow(t.M0, params->size0);
+      out_params->tile_size1 = narrow(t.N0, params->size1);
+      return 0;
+    default:
+      return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "query_tile_sizes: unknown operand role 0x%x",
+                  params->flags & IREE_AMD_UK_FLAG_QUERY_TILE_SIZES_OPERAND_ROLE_MASK);
+  }
+}
+
+//===----------------------------------------------------------------------===//
+// int4 dequant matmul, fp8 helpers
+//===----------------------------------------------------------------------===//
+
+extern "C" int iree_amd_uk_dequant_matmul_i4(
+    const void* x_buffer, const void* w_buffer, const void* scale_buffer,
+    const void* zp_buffer, void* out_buffer, iree_amd_uk_index_t M,
+    iree_amd_uk_index_t N, iree_amd_uk_index_t K,
+    iree_amd_uk_index_t group_size, uint32_t flags, void* stream) {
+  if (flags & ~1u) return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "dequant_matmul_i4: unknown flag bits");
+  if (M < 0 || N < 0 || K < 0 || group_size <= 0)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "dequant_matmul_i4: bad sizes");
+  if (K % group_size || group_size % 32)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT,
+                "dequant_matmul_i4: need K %% group_size == 0 and group_size %% 32 == 0");
+  if (M == 0 || N == 0) return 0;
+  if (!x_buffer || !w_buffer || !scale_buffer || !zp_buffer || !out_buffer)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "dequant_matmul_i4: null buffer");
+  return launch_dequant_matmul_i4(x_buffer, w_buffer, scale_buffer, zp_buffer,
+                                  out_buffer, M, N, K, group_size, flags,
+                                  (hipStream_t)stream);
+}
+
+extern "C" int iree_amd_uk_quantize_f16_to_f8e4m3(const void* in_f16,
+                                                  void* out_fp8,
+                                                  iree_amd_uk_index_t n,
+                                                  float inv_scale, void* stream) {
+  if (n < 0) return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "quantize: negative n");
+  if (n == 0) return 0;
+  if (!in_f16 || !out_fp8) return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "quantize: null buffer");
+  return launch_quantize_f16_to_f8e4m3(in_f16, out_fp8, n, inv_scale, (hipStream_t)stream);
+}
+
+extern "C" int iree_amd_uk_silu_mul_quantize(
+    const void* gate_f32, const void* up_f32, void* out_fp8,
+    iree_amd_uk_index_t rows, iree_amd_uk_index_t cols, iree_amd_uk_index_t ld,
+    float gate_scale, float up_scale, float inv_out_scale, void* stream) {
+  if (rows < 0 || cols < 0 || ld < cols)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "silu_mul_quantize: bad sizes");
+  if (rows == 0 || cols == 0) return 0;
+  if (!gate_f32 || !up_f32 || !out_fp8)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "silu_mul_quantize: null buffer");
+  return launch_silu_mul_quantize(gate_f32, up_f32, out_fp8, rows, cols, ld,
+                                  gate_scale, up_scale, inv_out_scale,
+                                  (hipStream_t)stream);
+}
+
+//===----------------------------------------------------------------------===//
+// Thin device ABI
+//===----------------------------------------------------------------------===//
+
+extern "C" int iree_amd_uk_device_count(int* out_count) {
+  if (!out_count) return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "device_count: null");
+  *out_count = 0;
+  hipError_t e = hipGetDeviceCount(out_count);
+  if (e == hipErrorNoDevice) { *out_count = 0; return 0; }
+  return check_hip(e, "hipGetDeviceCount");
+}
+extern "C" int iree_amd_uk_device_set(int ordinal) {
+  return check_hip(hipSetDevice(ordinal), "hipSetDevice");
+}
+extern "C" int iree_amd_uk_device_malloc(void** out_ptr, uint64_t bytes) {
+  if (!out_ptr) return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "device_malloc: null");
+  *out_ptr = nullptr;
+  if (!bytes) return 0;
+  return check_hip(hipMalloc(out_ptr, bytes), "hipMalloc");
+}
+extern "C" int iree_amd_uk_device_free(void* ptr) {
+  if (!ptr) return 0;
+  return check_hip(hipFree(ptr), "hipFree");
+}
+extern "C" int iree_amd_uk_memcpy_h2d(void* dst, const void* src, uint64_t bytes, void* stream) {
+  if (!bytes) return 0;
+  return check_hip(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, (hipStream_t)stream), "hipMemcpyAsync(h2d)");
+}
+extern "C" int iree_amd_uk_memcpy_d2h(void* dst, const void* src, uint64_t bytes, void* stream) {
+  if (!bytes) return 0;
+  return check_hip(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, (hipStream_t)stream), "hipMemcpyAsync(d2h)");
+}
+extern "C" int iree_amd_uk_stream_create(void** out_stream) {
+  if (!out_stream) return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "stream_create: null");
+  hipStream_t s = nullptr;
+  // Default priority on purpose: mixed stream priorities are not used.
+  UK_RETURN_IF_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+  *out_stream = (void*)s;
+  return 0;
+}
+extern "C" int iree_amd_uk_stream_destroy(void* stream) {
+  if (!stream) return 0;
+  return check_hip(hipStreamDestroy((hipStream_t)stream), "hipStreamDestroy");
+}
+extern "C" int iree_amd_uk_stream_synchronize(void* stream) {
+  return check_hip(hipStreamSynchronize((hipStream_t)stream), "hipStreamSynchronize");
+}
+extern "C" const char* iree_amd_uk_last_error(void) { return g_last_error; }
+extern "C" uint32_t iree_amd_uk_version(void) { return (0u << 16) | 1u; }
+
+//===----------------------------------------------------------------------===//
+// Host-pointer variants: stage the touched element ranges through device
+// memory. Each call owns its device buffers and one stream, so concurrent
+// calls from several host threads do not share state.
+//===----------------------------------------------------------------------===//
+
+namespace {
+
+struct Staging {
+  hipStream_t stream = nullptr;
+  void* dev[3] = {nullptr, nullptr, nullptr};
+  ~Staging() {
+    for (void* d : dev)
+      if (d) (void)hipFree(d);
+    if (stream) (void)hipStreamDestroy(stream);
+  }
+  int init() { return check_hip(hipStreamCreateWithFlags(&stream, hipStreamNonBlocking), "hipStreamCreate"); }
+  // Uploads [host + byte_off, +bytes) into a fresh device buffer `slot`.
+  int upload(int slot, const void* host, int64_t byte_off, int64_t bytes, bool copy) {
+    if (bytes <= 0) return 0;
+    UK_RETURN_IF_HIP(hipMalloc(&dev[slot], (size_t)bytes));
+    if (copy)
+      UK_RETURN_IF_HIP(hipMemcpyAsync(dev[slot], (const char*)host + byte_off, (size_t)bytes,
+                                      hipMemcpyHostToDevice, stream));
+    return 0;
+  }
+  int download(int slot, void* host, int64_t byte_off, int64_t bytes) {
+    if (bytes <= 0) return 0;
+    UK_RETURN_IF_HIP(hipMemcpyAsync((char*)host + byte_off, dev[slot], (size_t)bytes,
+                                    hipMemcpyDeviceToHost, stream));
+    return check_hip(hipStreamSynchronize(stream), "hipStreamSynchronize");
+  }
+};
+
+// Bytes spanned by `rows` rows of `row_elems` contiguous elements, `stride`
+// elements apart, for an element of `bits` bits.
+int64_t span_bytes(int64_t rows, int64_t stride, int64_t row_elems, int bits) {
+  if (rows <= 0 || row_elems <= 0) return 0;
+  return (((rows - 1) * stride + row_elems) * bits + 7) / 8;
+}
+
+}  // namespace
+
+extern "C" int iree_amd_uk_mmt4d_host(const iree_amd_uk_mmt4d_params_t* params) {
+  if (!params) return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "mmt4d_host: null params");
+  iree_amd_uk_mmt4d_params_t p = *params;
+  UK_RETURN_IF_ERROR(validate_mmt4d(p));
+  if (p.M == 0 || p.N == 0 || (p.K == 0 && (p.flags & IREE_AMD_UK_FLAG_MMT4D_ACCUMULATE))) return 0;
+  if (p.M0 == 0 || p.N0 == 0) return 0;
+  Mmt4dTypeInfo ti;
+  mmt4d_type_info(p.flags, &ti);
+  const int64_t lhs_bytes = span_bytes(p.M, p.lhs_stride0, p.K * p.M0 * p.K0, ti.lhs_bits);
+  const int64_t rhs_bytes = span_bytes(p.N, p.rhs_stride0, p.K * p.N0 * p.K0, ti.rhs_bits);
+  const int64_t out_bytes = span_bytes(p.M, p.out_stride0, p.N * p.M0 * p.N0, ti.out_bytes * 8);
+  const bool out_tight = p.out_stride0 == p.N * p.M0 * p.N0;
+  const bool need_out_in = (p.flags & IREE_AMD_UK_FLAG_MMT4D_ACCUMULATE) || !out_tight;
+  Staging st;
+  UK_RETURN_IF_ERROR(st.init());
+  UK_RETURN_IF_ERROR(st.upload(0, p.lhs_buffer, p.lhs_offset * ti.lhs_bits / 8, lhs_bytes, true));
+  UK_RETURN_IF_ERROR(st.upload(1, p.rhs_buffer, p.rhs_offset * ti.rhs_bits / 8, rhs_bytes, true));
+  UK_RETURN_IF_ERROR(st.upload(2, p.out_buffer, p.out_offset * ti.out_bytes, out_bytes, need_out_in));
+  void* host_out = p.out_buffer;
+  const int64_t host_out_off = p.out_offset * ti.out_bytes;
+  p.lhs_buffer = st.dev[0]; p.lhs_offset = 0;
+  p.rhs_buffer = st.dev[1]; p.rhs_offset = 0;
+  p.out_buffer = st.dev[2]; p.out_offset = 0;
+  UK_RETURN_IF_ERROR(iree_amd_uk_mmt4d_p(&p, st.stream));
+  return st.download(2, host_out, host_out_off, out_bytes);
+}
+
+extern "C" int iree_amd_uk_pack_host(const iree_amd_uk_pack_params_t* params) {
+  if (!params) return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "pack_host: null params");
+  iree_amd_uk_pack_params_t p = *params;
+  UK_RETURN_IF_ERROR(validate_pack(p));
+  if (p.out_size0 == 0 || p.out_size1 == 0 || p.out_size2 == 0 || p.out_size3 == 0) return 0;
+  const int es = pack_elem_bytes(p.flags);
+  const int64_t in_row = p.in_size1 > 0 ? (p.in_size1 - 1) * p.in_stride1 + 1 : 0;
+  const int64_t in_bytes = span_bytes(p.in_size0, p.in_stride0, in_row, es * 8);
+  const int64_t out_bytes = span_bytes(p.out_size0, p.out_stride0, p.out_size1 * p.out_stride1, es * 8);
+  const bool out_tight = p.out_stride0 == p.out_size1 * p.out_stride1;
+  Staging st;
+  UK_RETURN_IF_ERROR(st.init());
+  UK_RETURN_IF_ERROR(st.upload(0, p.in_buffer, p.in_offset * es, in_bytes, true));
+  UK_RETURN_IF_ERROR(st.upload(2, p.out_buffer, p.out_offset * es, out_bytes, !out_tight));
+  void* host_out = p.out_buffer;
+  const int64_t host_out_off = p.out_offset * es;
+  p.in_buffer = st.dev[0]; p.in_offset = 0;
+  p.out_buffer = st.dev[2]; p.out_offset = 0;
+  UK_RETURN_IF_ERROR(iree_amd_uk_pack_p(&p, st.stream));
+  return st.download(2, host_out, host_out_off, out_bytes);
+}
+
+extern "C" int iree_amd_uk_unpack_host(const iree_amd_uk_unpack_params_t* params) {
+  if (!params) return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "unpack_host: null params");
+  iree_amd_uk_unpack_params_t p = *params;
+  UK_RETURN_IF_ERROR(validate_unpack(p));
+  if (p.out_size0 == 0 || p.out_size1 == 0) return 0;
+  const int es = unpack_elem_bytes(p.flags);
+  const int64_t in_bytes = span_bytes(p.in_size0, p.in_stride0, p.in_size1 * p.in_stride1, es * 8);
+  const int64_t out_row = (p.out_size1 - 1) * p.out_stride1 + 1;
+  const int64_t out_bytes = span_bytes(p.out_size0, p.out_stride0, out_row, es * 8);
+  // The destination may have gaps (strides) the kernel must not disturb: start
+  // from the caller's bytes unless the destination is dense.
+  const bool out_dense = p.out_stride1 == 1 && p.out_stride0 == p.out_size1;
+  Staging st;
+  UK_RETURN_IF_ERROR(st.init());
+  UK_RETURN_IF_ERROR(st.upload(0, p.in_buffer, p.in_offset * es, in_bytes, true));
+  UK_RETURN_IF_ERROR(st.upload(2, p.out_buffer, p.out_offset * es, out_bytes, !out_dense));
+  void* host_out = p.out_buffer;
+  const int64_t host_out_off = p.out_offset * es;
+  p.in_buffer = st.dev[0]; p.in_offset = 0;
+  p.out_buffer = st.dev[2]; p.out_offset = 0;
+  UK_RETURN_IF_ERROR(iree_amd_uk_unpack_p(&p, st.stream));
+  return st.download(2, host_out, host_out_off, out_bytes);
+}

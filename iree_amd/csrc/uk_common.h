@@ -1,0 +1,83 @@
+// Shared declarations of the gfx950 ukernel library (internal, C++/HIP only).
+//
+// The public boundary is include/iree_amd_uk.h. Everything here is private to
+// the .hip translation units: error plumbing, element-type tables and the
+// launch functions each kernel file exports to uk_api.hip.
+#ifndef IREE_AMD_CSRC_UK_COMMON_H_
+#define IREE_AMD_CSRC_UK_COMMON_H_
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "iree_amd_uk.h"
+
+namespace uk {
+
+// Records a message for iree_amd_uk_last_error() on this thread and returns
+// `status`, so call sites read `return fail(STATUS, "...")`.
+int fail(int status, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+
+// Converts a hipError_t of a runtime call or of a kernel launch to a status.
+int check_hip(hipError_t err, const char* what);
+
+#define UK_RETURN_IF_HIP(expr)                                   \
+  do {                                                           \
+    int uk_status_ = ::uk::check_hip((expr), #expr);             \
+    if (uk_status_) return uk_status_;                           \
+  } while (0)
+
+#define UK_RETURN_IF_ERROR(expr)       \
+  do {                                 \
+    int uk_status_ = (expr);           \
+    if (uk_status_) return uk_status_; \
+  } while (0)
+
+// Element-type facts of an mmt4d type tuple.
+struct Mmt4dTypeInfo {
+  int lhs_bits;
+  int rhs_bits;
+  int out_bytes;
+};
+// Returns false for an unknown type value.
+bool mmt4d_type_info(uint32_t flags, Mmt4dTypeInfo* out);
+// 0 for an unknown / unsupported type value.
+int pack_elem_bytes(uint32_t flags);
+int unpack_elem_bytes(uint32_t flags);
+
+// Validation shared by the device and the host-pointer entry points.
+int validate_mmt4d(const iree_amd_uk_mmt4d_params_t& p);
+int validate_pack(const iree_amd_uk_pack_params_t& p);
+int validate_unpack(const iree_amd_uk_unpack_params_t& p);
+
+// Kernel launchers (each defined next to its kernels). All assume validated
+// parameters and non-degenerate sizes.
+int launch_mmt4d_generic(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s);
+// Returns true when a MFMA kernel exists for (type, M0, N0, K0).
+bool mmt4d_mfma_supported(uint32_t flags, int M0, int N0, int K0);
+// Also needs alignment / stride properties of the actual call; returns
+// NOT_FOUND (without recording an error) when the call must take the generic
+// kernel instead.
+int launch_mmt4d_mfma(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s);
+
+int launch_pack(const iree_amd_uk_pack_params_t& p, hipStream_t s);
+int launch_unpack(const iree_amd_uk_unpack_params_t& p, hipStream_t s);
+
+int launch_dequant_matmul_i4(const void* x, const void* w, const void* scale,
+                             const void* zp, void* out, int64_t M, int64_t N,
+                             int64_t K, int64_t group_size, uint32_t flags,
+                             hipStream_t s);
+int launch_quantize_f16_to_f8e4m3(const void* in, void* out, int64_t n,
+                                  float inv_scale, hipStream_t s);
+int launch_silu_mul_quantize(const void* gate, const void* up, void* out,
+                             int64_t rows, int64_t cols, int64_t ld,
+                             float gate_scale, float up_scale,
+                             float inv_out_scale, hipStream_t s);
+
+// Number of compute units of the current device (cached per device).
+int device_cu_count();
+
+__host__ __device__ static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+}  // namespace uk
+
+#endif  // IREE_AMD_CSRC_UK_COMMON_H_

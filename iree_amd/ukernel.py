@@ -1,0 +1,212 @@
+"""Host mirror of the reference's ukernel entry points over the C-ABI library.
+
+Function names, argument names and meaning follow
+runtime/src/iree/builtins/ukernel/{mmt4d.h:14-21, pack.h:26-34, unpack.h:17-25,
+query_tile_sizes.h:29-31} of the reference; buffers are torch CUDA tensors used
+only as owners of device memory (their ``data_ptr()`` is the base pointer,
+offsets and strides are in elements exactly as in the reference). Work is
+enqueued on torch's current stream. Errors from the library raise ``UkError``.
+"""
+import ctypes as C
+
+import torch
+
+from . import flags as F
+from ._lib import (Mmt4dParams, PackParams, QueryOutParams, QueryParams,
+                   UnpackParams, load_library)
+
+
+class UkError(RuntimeError):
+    def __init__(self, status, message):
+        super().__init__(f"iree_amd_uk status {status}: {message}")
+        self.status = status
+
+
+def _check(status):
+    if status != 0:
+        msg = load_library().iree_amd_uk_last_error()
+        raise UkError(status, msg.decode() if msg else "")
+
+
+def _ptr(t):
+    if t is None:
+        return None
+    if not t.is_cuda:
+        raise ValueError("ukernel buffers must be CUDA (HIP) tensors")
+    return C.c_void_p(t.data_ptr())
+
+
+def _stream(stream):
+    if stream is None:
+        stream = torch.cuda.current_stream()
+    return C.c_void_p(stream.cuda_stream)
+
+
+def mmt4d(lhs_buffer, rhs_buffer, out_buffer, M, N, K, M0, N0, K0, flags, *,
+          lhs_offset=0, lhs_stride0=None, rhs_offset=0, rhs_stride0=None,
+          out_offset=0, out_stride0=None, stream=None):
+    """iree_uk_mmt4d (reference mmt4d.h:14-21). Strides default to tight."""
+    if lhs_stride0 is None:
+        lhs_stride0 = K * M0 * K0
+    if rhs_stride0 is None:
+        rhs_stride0 = K * N0 * K0
+    if out_stride0 is None:
+        out_stride0 = N * M0 * N0
+    lib = load_library()
+    _check(lib.iree_amd_uk_mmt4d(
+        _ptr(lhs_buffer), lhs_offset, lhs_stride0, _ptr(rhs_buffer), rhs_offset,
+        rhs_stride0, _ptr(out_buffer), out_offset, out_stride0, M, N, K, M0, N0,
+        K0, flags, None, _stream(stream)))
+
+
+def mmt4d_info(M0, N0, K0, flags):
+    """iree_uk_mmt4d_info (reference mmt4d.h:23-25)."""
+    return load_library().iree_amd_uk_mmt4d_info(M0, N0, K0, flags, None)
+
+
+def pack(in_buffer, out_buffer, in_size0, in_size1, out_size0, out_size1,
+         out_size2, out_size3, padding_value, flags, *, in_offset=0,
+         in_stride0=None, in_stride1=1, out_offset=0, out_stride0=None,
+         out_stride1=None, stream=None):
+    """iree_uk_pack (reference pack.h:26-34). Strides default to tight."""
+    if in_stride0 is None:
+        in_stride0 = in_size1 * in_stride1
+    if out_stride1 is None:
+        out_stride1 = out_size2 * out_size3
+    if out_stride0 is None:
+        out_stride0 = out_size1 * out_stride1
+    lib = load_library()
+    _check(lib.iree_amd_uk_pack(
+        _ptr(in_buffer), in_offset, in_stride0, in_stride1, _ptr(out_buffer),
+        out_offset, out_stride0, out_stride1, in_size0, in_size1, out_size0,
+        out_size1, out_size2, out_size3, padding_value & 0xFFFFFFFFFFFFFFFF,
+        flags, None, _stream(stream)))
+
+
+def unpack(in_buffer, out_buffer, in_size0, in_size1, in_size2, in_size3,
+           out_size0, out_size1, flags, *, in_offset=0, in_stride0=None,
+           in_stride1=None, out_offset=0, out_stride0=None, out_stride1=1,
+           stream=None):
+    """iree_uk_unpack (reference unpack.h:17-25). Strides default to tight."""
+    if in_stride1 is None:
+        in_stride1 = in_size2 * in_size3
+    if in_stride0 is None:
+        in_stride0 = in_size1 * in_stride1
+    if out_stride0 is None:
+        out_stride0 = out_size1 * out_stride1
+    lib = load_library()
+    _check(lib.iree_amd_uk_unpack(
+        _ptr(in_buffer), in_offset, in_stride0, in_stride1, _ptr(out_buffer),
+        out_offset, out_stride0, out_stride1, in_size0, in_size1, in_size2,
+        in_size3, out_size0, out_size1, flags, None, _stream(stream)))
+
+
+_INT64_MIN = -(1 << 63)
+
+
+def query_tile_sizes_2d(flags, size0=_INT64_MIN, size1=_INT64_MIN):
+    """iree_uk_query_tile_sizes_2d (reference query_tile_sizes.h:29-31).
+    Returns (tile_size0, tile_size1). Needs no device."""
+    p = QueryParams(flags=flags, size0=size0, size1=size1, cpu_data=None)
+    o = QueryOutParams()
+    _check(load_library().iree_amd_uk_query_tile_sizes_2d(C.byref(p), C.byref(o)))
+    return int(o.tile_size0), int(o.tile_size1)
+
+
+def dequant_matmul_i4(x, w, scale, zp, out, M, N, K, group_size, flags=0,
+                      stream=None):
+    """Grouped int4-weight dequantising matmul (see include/iree_amd_uk.h)."""
+    _check(load_library().iree_amd_uk_dequant_matmul_i4(
+        _ptr(x), _ptr(w), _ptr(scale), _ptr(zp), _ptr(out), M, N, K, group_size,
+        flags, _stream(stream)))
+
+
+def quantize_f16_to_f8e4m3(inp, out, n, inv_scale, stream=None):
+    _check(load_library().iree_amd_uk_quantize_f16_to_f8e4m3(
+        _ptr(inp), _ptr(out), n, inv_scale, _stream(stream)))
+
+
+def silu_mul_quantize(gate, up, out, rows, cols, ld, gate_scale, up_scale,
+                      inv_out_scale, stream=None):
+    _check(load_library().iree_amd_uk_silu_mul_quantize(
+        _ptr(gate), _ptr(up), _ptr(out), rows, cols, ld, gate_scale, up_scale,
+        inv_out_scale, _stream(stream)))
+
+
+# ---------------------------------------------------------------------------
+# The reference's end-to-end chain: pack LHS, pack RHS (inner+outer transposed),
+# [pack accumulator], mmt4d, unpack
+# (runtime/src/iree/builtins/ukernel/tools/e2e_matmul_benchmark.c:173-186,
+# parameters built as at :208-285).
+# ---------------------------------------------------------------------------
+
+_MMT4D_TO_QUERY_OP = {
+    F.MMT4D_TYPE_F32F32F32: F.QUERY_OP_MATMUL_F32F32F32,
+    F.MMT4D_TYPE_S8S8S32: F.QUERY_OP_MATMUL_I8I8I32,
+    F.MMT4D_TYPE_F16F16F32: F.QUERY_OP_MATMUL_F16F16F32,
+    F.MMT4D_TYPE_F16F16F16: F.QUERY_OP_MATMUL_F16F16F16,
+    F.MMT4D_TYPE_BF16BF16F32: F.QUERY_OP_MATMUL_BF16BF16F32,
+    F.MMT4D_TYPE_BF16BF16BF16: F.QUERY_OP_MATMUL_BF16BF16BF16,
+    F.MMT4D_TYPE_F8E4M3F8E4M3F32: F.QUERY_OP_MATMUL_F8E4M3F8E4M3F32,
+}
+_IN_PACK_TYPE = {
+    F.MMT4D_TYPE_F32F32F32: F.PACK_TYPE_F32F32,
+    F.MMT4D_TYPE_S8S8S32: F.PACK_TYPE_I8I8,
+    F.MMT4D_TYPE_F16F16F32: F.PACK_TYPE_F16F16,
+    F.MMT4D_TYPE_F16F16F16: F.PACK_TYPE_F16F16,
+    F.MMT4D_TYPE_BF16BF16F32: F.PACK_TYPE_BF16BF16,
+    F.MMT4D_TYPE_BF16BF16BF16: F.PACK_TYPE_BF16BF16,
+    F.MMT4D_TYPE_F8E4M3F8E4M3F32: F.PACK_TYPE_I8I8,
+}
+_OUT_PACK_TYPE = {
+    F.MMT4D_TYPE_F32F32F32: F.PACK_TYPE_F32F32,
+    F.MMT4D_TYPE_S8S8S32: F.PACK_TYPE_I32I32,
+    F.MMT4D_TYPE_F16F16F32: F.PACK_TYPE_F32F32,
+    F.MMT4D_TYPE_F16F16F16: F.PACK_TYPE_F16F16,
+    F.MMT4D_TYPE_BF16BF16F32: F.PACK_TYPE_F32F32,
+    F.MMT4D_TYPE_BF16BF16BF16: F.PACK_TYPE_BF16BF16,
+    F.MMT4D_TYPE_F8E4M3F8E4M3F32: F.PACK_TYPE_F32F32,
+}
+
+
+def _ceil_div(a, b):
+    return -(-a // b)
+
+
+def matmul_data_tiled(a, b, c, M, N, K, mmt4d_type, *, accumulate=False,
+                      tile=None, workspace=None):
+    """Row-major C[M][N] (+)= A[M][K] * B[K][N] through pack -> mmt4d -> unpack.
+
+    ``a``/``b``/``c`` are flat CUDA tensors holding the row-major matrices with
+    the element types of ``mmt4d_type``. ``tile`` = (M0, N0, K0); by default the
+    tile the library's query_tile_sizes_2d reports for gfx950. ``workspace`` may
+    carry pre-allocated packed buffers as a dict {"lhs","rhs","out"}.
+    Returns the dict of packed buffers used (so callers can reuse them).
+    """
+    if tile is None:
+        op = _MMT4D_TO_QUERY_OP[mmt4d_type]
+        M0, K0 = query_tile_sizes_2d(op | F.QUERY_ROLE_LHS, M, K)
+        N0, _ = query_tile_sizes_2d(op | F.QUERY_ROLE_RHS, N, K)
+    else:
+        M0, N0, K0 = tile
+    M1, N1, K1 = _ceil_div(M, M0), _ceil_div(N, N0), _ceil_div(K, K0)
+    in_type = _IN_PACK_TYPE[mmt4d_type]
+    out_type = _OUT_PACK_TYPE[mmt4d_type]
+    ws = workspace if workspace is not None else {}
+    if "lhs" not in ws:
+        ws["lhs"] = torch.empty(M1 * K1 * M0 * K0, dtype=a.dtype, device=a.device)
+    if "rhs" not in ws:
+        ws["rhs"] = torch.empty(N1 * K1 * N0 * K0, dtype=b.dtype, device=b.device)
+    if "out" not in ws:
+        ws["out"] = torch.empty(M1 * N1 * M0 * N0, dtype=c.dtype, device=c.device)
+    pack(a, ws["lhs"], M, K, M1, K1, M0, K0, 0, in_type)
+    pack(b, ws["rhs"], K, N, N1, K1, N0, K0, 0,
+         in_type | F.PACK_TRANSPOSE_INNER | F.PACK_TRANSPOSE_OUTER)
+    mm_flags = mmt4d_type | F.MMT4D_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION | \
+        F.MMT4D_SKIP_INTERMEDIATE_ROUNDINGS
+    if accumulate:
+        pack(c, ws["out"], M, N, M1, N1, M0, N0, 0, out_type)
+        mm_flags |= F.MMT4D_ACCUMULATE
+    mmt4d(ws["lhs"], ws["rhs"], ws["out"], M1, N1, K1, M0, N0, K0, mm_flags)
+    unpack(ws["out"], c, M1, N1, M0, N0, M, N, out_type)
+    return ws

@@ -1,0 +1,166 @@
+"""The C-ABI library loads, exports every symbol include/iree_amd_uk.h
+declares, agrees with the reference's flag values, and its host-only entry
+points (validation, tile-size query, info) behave - all without a GPU."""
+import ctypes as C
+import os
+import re
+import subprocess
+import tempfile
+
+import pytest
+
+import iree_amd
+from iree_amd import flags as F
+from iree_amd._lib import (Mmt4dParams, PackParams, QueryOutParams, QueryParams,
+                           UnpackParams)
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "iree_amd_uk.h")
+
+
+def _header_text():
+    with open(HEADER) as f:
+        return f.read()
+
+
+def test_every_declared_symbol_is_exported():
+    text = re.sub(r"/\*.*?\*/", "", _header_text(), flags=re.S)
+    names = re.findall(r"IREE_AMD_UK_EXPORT\s+[\w\s\*]+?\b(iree_amd_uk_\w+)\s*\(", text)
+    assert len(names) >= 24, names
+    lib = iree_amd.load_library()
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in the header but not exported"
+
+
+# Values of the reference's exported_bits.h:29-106 ("set in stone"), as data.
+REFERENCE_FLAG_VALUES = {
+    "MMT4D_TYPE_F32F32F32": 0x01, "MMT4D_TYPE_S8S8S32": 0x02, "MMT4D_TYPE_F16F16F32": 0x03,
+    "MMT4D_TYPE_F16F16F16": 0x04, "MMT4D_TYPE_BF16BF16F32": 0x05, "MMT4D_TYPE_BF16BF16BF16": 0x06,
+    "MMT4D_TYPE_S16S16S32": 0x07, "MMT4D_TYPE_S16U4S32": 0x08, "MMT4D_TYPE_S16S8S32": 0x09,
+    "MMT4D_TYPE_S8S4S32": 0x0A, "MMT4D_ACCUMULATE": 0x100,
+    "MMT4D_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION": 0x200, "MMT4D_SKIP_INTERMEDIATE_ROUNDINGS": 0x400,
+    "MMT4D_INFO_HAVE_ARCHITECTURE_SPECIFIC_TILE_FUNCTION": 0x1,
+    "PACK_TYPE_F32F32": 1, "PACK_TYPE_I8I8": 2, "PACK_TYPE_I32I32": 3, "PACK_TYPE_F16F16": 4,
+    "PACK_TYPE_BF16BF16": 5, "PACK_TRANSPOSE_INNER": 0x100, "PACK_TRANSPOSE_OUTER": 0x200,
+    "UNPACK_TYPE_F32F32": 1, "UNPACK_TYPE_I32I32": 3, "UNPACK_TYPE_F16F16": 4,
+    "UNPACK_TYPE_BF16BF16": 5, "UNPACK_TRANSPOSE_INNER": 0x100, "UNPACK_TRANSPOSE_OUTER": 0x200,
+    "QUERY_TILE_SIZES_OPERAND_ROLE_LHS": 1, "QUERY_TILE_SIZES_OPERAND_ROLE_RHS": 2,
+    "QUERY_TILE_SIZES_OPERAND_ROLE_RESULT": 3,
+    "QUERY_TILE_SIZES_OPERATION_MATMUL_F32F32F32": 0x100,
+    "QUERY_TILE_SIZES_OPERATION_MATMUL_I8I8I32": 0x200,
+    "QUERY_TILE_SIZES_OPERATION_MATMUL_F16F16F32": 0x300,
+    "QUERY_TILE_SIZES_OPERATION_MATMUL_F16F16F16": 0x400,
+    "QUERY_TILE_SIZES_OPERATION_MATMUL_BF16BF16F32": 0x500,
+    "QUERY_TILE_SIZES_OPERATION_MATMUL_BF16BF16BF16": 0x600,
+}
+
+
+def test_flag_values_equal_the_reference():
+    defs = dict(re.findall(r"#define IREE_AMD_UK_FLAG_(\w+)\s+(0x[0-9A-Fa-f]+|\d+)", _header_text()))
+    for name, val in REFERENCE_FLAG_VALUES.items():
+        assert int(defs[name], 0) == val, name
+    # the Python mirror agrees with the header
+    py = {"QUERY_ROLE_LHS": "QUERY_TILE_SIZES_OPERAND_ROLE_LHS",
+          "QUERY_OP_MATMUL_I8I8I32": "QUERY_TILE_SIZES_OPERATION_MATMUL_I8I8I32",
+          "QUERY_OP_MATMUL_F16F16F32": "QUERY_TILE_SIZES_OPERATION_MATMUL_F16F16F32"}
+    for name in dir(F):
+        hname = py.get(name, name)
+        if hname in defs and isinstance(getattr(F, name), int):
+            assert getattr(F, name) == int(defs[hname], 0), name
+    # flag words the reference's compiler tests pin
+    # (Codegen/Common/CPU/test/lower_to_ukernel_ops.mlir:212 and the blog walkthrough)
+    assert (F.MMT4D_TYPE_F16F16F16 | F.MMT4D_ACCUMULATE | F.MMT4D_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION |
+            F.MMT4D_SKIP_INTERMEDIATE_ROUNDINGS) == 1796
+    assert (F.MMT4D_TYPE_F32F32F32 | F.MMT4D_ACCUMULATE | F.MMT4D_SKIP_INTERMEDIATE_ROUNDINGS) == 1281
+
+
+def test_struct_layout_matches_the_c_header():
+    src = r'''
+#include <stdio.h>
+#include <stddef.h>
+#include "iree_amd_uk.h"
+int main(void) {
+  printf("%zu %zu %zu %zu %zu\n", sizeof(iree_amd_uk_mmt4d_params_t), sizeof(iree_amd_uk_pack_params_t),
+         sizeof(iree_amd_uk_unpack_params_t), sizeof(iree_amd_uk_query_tile_sizes_2d_params_t),
+         sizeof(iree_amd_uk_query_tile_sizes_2d_out_params_t));
+  printf("%zu %zu %zu %zu\n", offsetof(iree_amd_uk_mmt4d_params_t, M0), offsetof(iree_amd_uk_mmt4d_params_t, flags),
+         offsetof(iree_amd_uk_pack_params_t, padding_value), offsetof(iree_amd_uk_unpack_params_t, flags));
+  return 0;
+}'''
+    with tempfile.TemporaryDirectory() as d:
+        c = os.path.join(d, "t.c")
+        with open(c, "w") as f:
+            f.write(src)
+        exe = os.path.join(d, "t")
+        subprocess.check_call(["gcc", "-std=c99", "-pedantic", "-Wall", "-Werror", "-I",
+                               os.path.join(ROOT, "include"), c, "-o", exe])
+        out = subprocess.check_output([exe]).decode().split()
+    sizes = [int(x) for x in out]
+    assert sizes[:5] == [C.sizeof(Mmt4dParams), C.sizeof(PackParams), C.sizeof(UnpackParams),
+                         C.sizeof(QueryParams), C.sizeof(QueryOutParams)]
+    assert sizes[5:] == [Mmt4dParams.M0.offset, Mmt4dParams.flags.offset,
+                         PackParams.padding_value.offset, UnpackParams.flags.offset]
+
+
+def test_query_tile_sizes_roles_and_narrowing():
+    q = iree_amd.query_tile_sizes_2d
+    # (M0, N0, K0) per operation: one 32x32 MFMA block, K0 = the 16 bytes a lane feeds it
+    for op, (m0, n0, k0) in [(F.QUERY_OP_MATMUL_I8I8I32, (32, 32, 16)),
+                             (F.QUERY_OP_MATMUL_F16F16F32, (32, 32, 8)),
+                             (F.QUERY_OP_MATMUL_BF16BF16F32, (32, 32, 8)),
+                             (F.QUERY_OP_MATMUL_F8E4M3F8E4M3F32, (32, 32, 16))]:
+        assert q(op | F.QUERY_ROLE_LHS) == (m0, k0)
+        assert q(op | F.QUERY_ROLE_RHS) == (n0, k0)
+        assert q(op | F.QUERY_ROLE_RESULT) == (m0, n0)
+        # role mapping equals the reference's (query_tile_sizes.c:43-63) via the oracle
+        import ukref
+        t0, t1 = C.c_int64(), C.c_int64()
+        for role in (F.QUERY_ROLE_LHS, F.QUERY_ROLE_RHS, F.QUERY_ROLE_RESULT):
+            assert ukref.oracle().oracle_query_role_tile(role, m0, n0, k0, C.byref(t0), C.byref(t1)) == 0
+            assert q(op | role) == (t0.value, t1.value)
+    # narrow static sizes shrink to the next power of two, never below 1
+    op = F.QUERY_OP_MATMUL_F16F16F32
+    assert q(op | F.QUERY_ROLE_LHS, 1, 4096) == (1, 8)
+    assert q(op | F.QUERY_ROLE_LHS, 7, 4096) == (8, 8)
+    assert q(op | F.QUERY_ROLE_LHS, 17, 4096) == (32, 8)
+    assert q(op | F.QUERY_ROLE_RESULT, 8, 3) == (8, 4)
+    assert q(op | F.QUERY_ROLE_RHS, 4096, 4096) == (32, 8)
+    with pytest.raises(iree_amd.UkError) as e:
+        q(0x0700 | F.QUERY_ROLE_LHS)
+    assert e.value.status == F.STATUS_INVALID_ARGUMENT
+    with pytest.raises(iree_amd.UkError):
+        q(op | 0x7)
+
+
+def test_mmt4d_info_reports_mfma_tiles():
+    have = F.MMT4D_INFO_HAVE_ARCHITECTURE_SPECIFIC_TILE_FUNCTION
+    assert iree_amd.mmt4d_info(32, 32, 8, F.MMT4D_TYPE_F16F16F32) == have
+    assert iree_amd.mmt4d_info(32, 32, 16, F.MMT4D_TYPE_F16F16F32) == have
+    assert iree_amd.mmt4d_info(32, 32, 16, F.MMT4D_TYPE_S8S8S32) == have
+    assert iree_amd.mmt4d_info(32, 32, 32, F.MMT4D_TYPE_S8S8S32) == have
+    assert iree_amd.mmt4d_info(16, 16, 1, F.MMT4D_TYPE_F16F16F32) == 0
+    assert iree_amd.mmt4d_info(32, 32, 8, F.MMT4D_TYPE_S16S16S32) == 0
+
+
+def test_validation_happens_before_any_device_work():
+    """Invalid calls are rejected and degenerate calls return OK without a GPU
+    (no compute is attempted in this test)."""
+    lib = iree_amd.load_library()
+    one = C.c_void_p(16)
+    # unknown flag bits / unknown type / bad sub-byte K0 (reference mmt4d.c:12-48)
+    assert lib.iree_amd_uk_mmt4d(one, 0, 8, one, 0, 8, one, 0, 8, 1, 1, 1, 2, 2, 2, 0x802, None, None) == 3
+    assert lib.iree_amd_uk_mmt4d(one, 0, 8, one, 0, 8, one, 0, 8, 1, 1, 1, 2, 2, 2, 0x0C, None, None) == 3
+    assert lib.iree_amd_uk_mmt4d(one, 0, 8, one, 0, 8, one, 0, 8, 1, 1, 1, 2, 2, 3, F.MMT4D_TYPE_S8S4S32, None, None) == 3
+    assert lib.iree_amd_uk_mmt4d(one, 0, 8, one, 0, 8, one, 0, 8, 1, 1, 1, 40000, 2, 2, 2, None, None) == 3
+    assert b"M0/N0/K0" in lib.iree_amd_uk_last_error()
+    # early returns (reference mmt4d.c:105-113)
+    assert lib.iree_amd_uk_mmt4d(None, 0, 8, None, 0, 8, None, 0, 8, 0, 5, 7, 2, 2, 2, 2, None, None) == 0
+    assert lib.iree_amd_uk_mmt4d(None, 0, 8, None, 0, 8, None, 0, 8, 5, 7, 0, 2, 2, 2, 2 | 0x100, None, None) == 0
+    # pack: out_stride1 must be the tile size (reference pack.c:72); I8 unpack does not exist
+    assert lib.iree_amd_uk_pack(one, 0, 4, 1, one, 0, 99, 7, 2, 4, 1, 2, 2, 2, 0, 1, None, None) == 3
+    assert lib.iree_amd_uk_pack(one, 0, 4, 1, one, 0, 8, 4, 5, 4, 1, 2, 2, 2, 0, 1, None, None) == 3
+    assert lib.iree_amd_uk_pack(None, 0, 4, 1, None, 0, 8, 4, 0, 0, 0, 2, 2, 2, 0, 1, None, None) == 0
+    assert lib.iree_amd_uk_unpack(one, 0, 8, 4, one, 0, 4, 1, 1, 2, 2, 2, 2, 4, 2, None, None) == 3
+    assert lib.iree_amd_uk_unpack(None, 0, 8, 4, None, 0, 4, 1, 1, 2, 2, 2, 0, 4, 1, None, None) == 0
+    assert lib.iree_amd_uk_dequant_matmul_i4(one, one, one, one, one, 1, 8, 100, 32, 0, None) == 3
+    assert lib.iree_amd_uk_version() >= 1

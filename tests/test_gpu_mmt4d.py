@@ -1,0 +1,249 @@
+"""GPU parity of mmt4d against the oracle through the C ABI. Integer types are
+bit-exact; float types are bit-exact on the reference's small-integer inputs
+(every partial sum exact, tools/mmt4d_test.c:430-436) and within 1e-2 relative
+or 1e-3 absolute of the f64-accumulated oracle on N(0,1) inputs."""
+import ctypes as C
+import hashlib
+import itertools
+import json
+import os
+
+import numpy as np
+import pytest
+
+import gpucase
+import ukref
+from iree_amd import flags as F
+from iree_amd import synth
+from test_oracle_mmt4d import REF_TYPES, SHAPES, TILES
+
+pytestmark = pytest.mark.gpu
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "golden.json")
+RTOL, ATOL = 1e-2, 1e-3   # the stated tolerance for f16 / fp8 / int4 results
+
+
+@pytest.mark.parametrize("type_flag", REF_TYPES + [F.MMT4D_TYPE_F8E4M3F8E4M3F32])
+def test_reference_test_matrix_bit_exact(uk, cuda, type_flag):
+    rng = np.random.default_rng(3000 + type_flag)
+    tiles = TILES.get(type_flag, [(3, 5, 8), (32, 32, 16)])
+    for tile in tiles:
+        M0, N0, K0 = tile
+        for (M, N, K), acc in itertools.product(SHAPES, (False, True)):
+            if type_flag in (F.MMT4D_TYPE_F16F16F16, F.MMT4D_TYPE_BF16BF16BF16) and K * K0 > 24:
+                continue
+            case = ukref.Mmt4dCase(rng, type_flag, M, N, K, M0, N0, K0, accumulate=acc,
+                                   loose_strides=bool(rng.integers(0, 2)),
+                                   offsets=bool(rng.integers(0, 2)))
+            got = gpucase.run_mmt4d(case)
+            want = case.run_oracle(ukref.F16_IEEE)
+            assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), \
+                (hex(type_flag), tile, (M, N, K), acc)
+
+
+MFMA_TILES = [(F.MMT4D_TYPE_S8S8S32, 32, 32, 16), (F.MMT4D_TYPE_S8S8S32, 32, 32, 32),
+              (F.MMT4D_TYPE_F16F16F32, 32, 32, 8), (F.MMT4D_TYPE_F16F16F32, 32, 32, 16),
+              (F.MMT4D_TYPE_BF16BF16F32, 32, 32, 8), (F.MMT4D_TYPE_BF16BF16F32, 32, 32, 16)]
+# outer shapes chosen to hit: single tile, ragged macro tiles in M and N, K
+# tails that are not whole LDS stages, both macro-tile variants, > 8 XCD slices
+MFMA_SHAPES = [(1, 1, 2), (1, 1, 8), (3, 2, 6), (5, 7, 10), (9, 4, 18), (8, 8, 8),
+               (17, 9, 4), (4, 33, 2), (20, 20, 12)]
+
+
+@pytest.mark.parametrize("type_flag,M0,N0,K0", MFMA_TILES)
+def test_mfma_kernels_bit_exact_on_exact_inputs(uk, cuda, type_flag, M0, N0, K0):
+    assert uk.mmt4d_info(M0, N0, K0, type_flag) == 1
+    rng = np.random.default_rng(4000 + type_flag + K0)
+    for (M, N, K), acc in itertools.product(MFMA_SHAPES, (False, True)):
+        case = ukref.Mmt4dCase(rng, type_flag, M, N, K, M0, N0, K0, accumulate=acc)
+        got = gpucase.run_mmt4d(case)
+        want = case.run_oracle(ukref.F16_IEEE)
+        assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), \
+            (hex(type_flag), (M0, N0, K0), (M, N, K), acc)
+        # The same call without the generic-fallback permission must also be
+        # served (it is an MFMA tile) and give the same bits.
+        got2 = gpucase.run_mmt4d(case, flags=case.flags & ~F.MMT4D_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION)
+        assert np.array_equal(got2.view(np.uint8), want.view(np.uint8))
+    # loose strides that keep 16-byte alignment stay on the MFMA path; odd ones
+    # and odd offsets fall back to the generic kernel - both must be right
+    for loose, offs in [(True, False), (False, True), (True, True)]:
+        case = ukref.Mmt4dCase(rng, type_flag, 5, 3, 6, M0, N0, K0, accumulate=True,
+                               loose_strides=loose, offsets=offs)
+        assert np.array_equal(gpucase.run_mmt4d(case), case.run_oracle(ukref.F16_IEEE))
+    case = ukref.Mmt4dCase(rng, type_flag, 5, 3, 6, M0, N0, K0)
+    case.lhs_stride0 += 64
+    case.rhs_stride0 += 32
+    case.out_stride0 += 16
+    case.lhs = np.resize(case.lhs, case.lhs.size + 5 * 64)
+    case.rhs = np.resize(case.rhs, case.rhs.size + 3 * 32)
+    case.out_init = np.resize(case.out_init, case.out_init.size + 5 * 16)
+    assert np.array_equal(gpucase.run_mmt4d(case), case.run_oracle(ukref.F16_IEEE))
+
+
+def test_without_fallback_permission_unserved_tiles_are_refused(uk, cuda):
+    rng = np.random.default_rng(1)
+    case = ukref.Mmt4dCase(rng, F.MMT4D_TYPE_S8S8S32, 2, 2, 2, 9, 6, 3)
+    with pytest.raises(uk.UkError) as e:
+        gpucase.run_mmt4d(case, flags=F.MMT4D_TYPE_S8S8S32)
+    assert e.value.status == F.STATUS_UNIMPLEMENTED
+
+
+@pytest.mark.parametrize("K0", [8, 16])
+def test_f16_normal_inputs_within_tolerance(uk, cuda, K0):
+    """f16 x f16 -> f32 on N(0,1)/sqrt(K) inputs, with and without accumulate,
+    against the f64-accumulated oracle: |got - want| <= 1e-3 + 1e-2 |want|."""
+    rng = np.random.default_rng(6)
+    M, N, K = 6, 5, 512 // K0
+    scale = 1.0 / np.sqrt(K * K0)
+
+    def gen(rng, tf, which, n):
+        if which == 2:
+            return rng.standard_normal(n).astype(np.float32)
+        return (rng.standard_normal(n) * scale).astype(np.float16).view(np.uint16)
+
+    for acc in (False, True):
+        case = ukref.Mmt4dCase(rng, F.MMT4D_TYPE_F16F16F32, M, N, K, 32, 32, K0,
+                               accumulate=acc, generator=gen)
+        got = case.written_region(gpucase.run_mmt4d(case))
+        want = case.written_region(case.run_oracle(f64=True))
+        assert np.all(np.abs(got - want) <= ATOL + RTOL * np.abs(want))
+        # and in practice far tighter than the stated tolerance
+        assert np.max(np.abs(got - want)) < 1e-5
+
+
+def _pack_chain_oracle_i8(A, B, M, N, K):
+    want = np.zeros((M, N), np.int32)
+    assert ukref.oracle().oracle_matmul_rowmajor(ukref.ptr(A), ukref.ptr(B), ukref.ptr(want),
+                                                 M, N, K, F.MMT4D_TYPE_S8S8S32) == 0
+    return want
+
+
+@pytest.mark.parametrize("M,N,K", [(1024, 1024, 1024), (123, 456, 789), (81, 19, 41), (1, 1000, 1000)])
+def test_i8_matmul_through_pack_mmt4d_unpack(uk, cuda, M, N, K):
+    """linalg.matmul i8 x i8 -> i32 through data tiling, bit-exact against a
+    plain row-major integer matmul (shapes: the 1024^3 configuration and ragged
+    shapes from the reference's e2e generator,
+    tests/e2e/matmul/generate_e2e_matmul_tests.py:134-177)."""
+    import torch
+    A = synth.uniform_int8(1, M * K)
+    B = synth.uniform_int8(2, K * N)
+    c = torch.zeros(M * N, dtype=torch.int32, device="cuda")
+    uk.matmul_data_tiled(torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda(), c,
+                         M, N, K, F.MMT4D_TYPE_S8S8S32)
+    torch.cuda.synchronize()
+    got = c.cpu().numpy().reshape(M, N)
+    want = _pack_chain_oracle_i8(A, B, M, N, K)
+    assert np.array_equal(got, want)
+    if (M, N, K) == (1024, 1024, 1024):
+        with open(GOLDEN) as f:
+            golden = json.load(f)
+        assert hashlib.sha256(got.tobytes()).hexdigest() == golden["matmul_i8_1024_sha256"]
+
+
+def test_i8_matmul_accumulates_into_seeded_c(uk, cuda):
+    import torch
+    M, N, K = 200, 100, 300
+    A, B = synth.uniform_int8(1, M * K), synth.uniform_int8(2, K * N)
+    c0 = (synth.splitmix64(3, M * N) >> np.uint64(44)).astype(np.int64).astype(np.int32)
+    c = torch.from_numpy(c0.copy()).cuda()
+    uk.matmul_data_tiled(torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda(), c,
+                         M, N, K, F.MMT4D_TYPE_S8S8S32, accumulate=True)
+    want = c0.reshape(M, N) + _pack_chain_oracle_i8(A, B, M, N, K)
+    assert np.array_equal(c.cpu().numpy().reshape(M, N), want)
+
+
+def _sampled_f64_rows(A, B, rows, K, N):
+    return A[rows].astype(np.float64) @ B.astype(np.float64)
+
+
+@pytest.mark.parametrize("accumulate", [False, True])
+def test_f16_4096_cubed_through_pack_mmt4d_unpack(uk, cuda, accumulate):
+    """The headline configuration at full size: f16 4096^3 with N(0,1)/sqrt(K)
+    inputs (second run accumulating into a seeded f32 C). Checked three ways:
+    64 sampled rows against an f64 product (the stated tolerance), the
+    checksum identity sum(C) = colsum(A) . rowsum(B), and bit-equality with the
+    oracle on 4 whole output tiles."""
+    import torch
+    M = N = K = 4096
+    A = synth.normal_f16(1, M * K, 1.0 / 64).reshape(M, K)
+    B = synth.normal_f16(2, K * N, 1.0 / 64).reshape(K, N)
+    C0 = synth.normal_f32(3, M * N).reshape(M, N) if accumulate else np.zeros((M, N), np.float32)
+    c = torch.from_numpy(C0.copy().reshape(-1)).cuda()
+    ws = uk.matmul_data_tiled(torch.from_numpy(A.reshape(-1).view(np.int16)).cuda().view(torch.float16),
+                              torch.from_numpy(B.reshape(-1).view(np.int16)).cuda().view(torch.float16),
+                              c, M, N, K, F.MMT4D_TYPE_F16F16F32, accumulate=accumulate)
+    torch.cuda.synchronize()
+    got = c.cpu().numpy().reshape(M, N)
+    rows = (synth.splitmix64(9, 64) % np.uint64(M)).astype(np.int64)
+    want = _sampled_f64_rows(A, B, rows, K, N) + C0[rows]
+    err = np.abs(got[rows] - want)
+    assert np.all(err <= ATOL + RTOL * np.abs(want)), float(err.max())
+    assert float(err.max()) < 5e-5
+    total = got.astype(np.float64).sum()
+    ident = A.astype(np.float64).sum(axis=0) @ B.astype(np.float64).sum(axis=1) + C0.astype(np.float64).sum()
+    assert abs(total - ident) <= 1e-6 * np.abs(got).astype(np.float64).sum()
+    # packed-layout check of whole tiles against the oracle's f32 tile function
+    M0, N0, K0 = 32, 32, 8
+    lhs = ws["lhs"].cpu().numpy().view(np.uint16)
+    rhs = ws["rhs"].cpu().numpy().view(np.uint16)
+    out = ws["out"].cpu().numpy()
+    K1, N1 = K // K0, N // N0
+    from iree_amd._lib import Mmt4dParams
+    for (i, j) in [(0, 0), (5, 77), (127, 127), (64, 3)]:
+        tile = np.zeros(M0 * N0, np.float32)
+        if accumulate:
+            tile[:] = C0[i * M0:(i + 1) * M0, j * N0:(j + 1) * N0].reshape(-1)
+        p = Mmt4dParams(ukref.ptr(lhs).value, i * K1 * M0 * K0, K1 * M0 * K0,
+                        ukref.ptr(rhs).value, j * K1 * N0 * K0, K1 * N0 * K0,
+                        ukref.ptr(tile).value, 0, M0 * N0, 1, 1, K1, M0, N0, K0,
+                        F.MMT4D_TYPE_F16F16F32 | (F.MMT4D_ACCUMULATE if accumulate else 0), None)
+        assert ukref.oracle().oracle_mmt4d_f64(C.byref(p)) == 0
+        g = out[(i * N1 + j) * M0 * N0:][:M0 * N0]
+        assert np.all(np.abs(g - tile) <= ATOL + RTOL * np.abs(tile))
+
+
+def test_i8_4096_cubed_mmt4d_invariants(uk, cuda):
+    """i8 4096^3 (the integer metric run) on packed operands: exact checksum
+    identity in integers, and 6 whole tiles bit-equal to the oracle."""
+    import torch
+    M1 = N1 = 128
+    M0 = N0 = 32
+    K0, K1 = 16, 256
+    lhs = synth.uniform_int8(1, M1 * K1 * M0 * K0)
+    rhs = synth.uniform_int8(2, N1 * K1 * N0 * K0)
+    out = torch.empty(M1 * N1 * M0 * N0, dtype=torch.int32, device="cuda")
+    uk.mmt4d(torch.from_numpy(lhs).cuda(), torch.from_numpy(rhs).cuda(), out, M1, N1, K1, M0, N0, K0,
+             F.MMT4D_TYPE_S8S8S32)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    L = lhs.reshape(M1, K1, M0, K0).astype(np.int64)
+    R = rhs.reshape(N1, K1, N0, K0).astype(np.int64)
+    ident = int((L.sum(axis=(0, 2)) * R.sum(axis=(0, 2))).sum())
+    assert int(got.astype(np.int64).sum()) == ident
+    for (i, j) in [(0, 0), (1, 126), (127, 127), (63, 64), (100, 7), (8, 8)]:
+        want = np.einsum("kac,kbc->ab", L[i], R[j]).astype(np.int32).reshape(-1)
+        assert np.array_equal(got[(i * N1 + j) * 1024:][:1024], want), (i, j)
+
+
+def test_host_pointer_variants(uk, cuda):
+    """iree_amd_uk_{pack,mmt4d,unpack}_host: the entry points the HAL plugin's
+    imports call with host buffers."""
+    lib = uk.load_library()
+    rng = np.random.default_rng(12)
+    for tf, tile in [(F.MMT4D_TYPE_S8S8S32, (32, 32, 16)), (F.MMT4D_TYPE_F16F16F32, (4, 6, 5))]:
+        case = ukref.Mmt4dCase(rng, tf, 3, 4, 6, *tile, accumulate=True, loose_strides=True, offsets=True)
+        out = case.out_init.copy()
+        p = case.params(ukref.ptr(case.lhs).value, ukref.ptr(case.rhs).value, ukref.ptr(out).value)
+        assert lib.iree_amd_uk_mmt4d_host(C.byref(p)) == 0
+        assert np.array_equal(out, case.run_oracle())
+    pc = ukref.PackCase(rng, F.PACK_TYPE_F16F16, 3, 5, 32, 16, pad="one_incomplete_tile",
+                        loose_strides=True, offsets=True)
+    out = pc.out_init.copy()
+    p = pc.params(ukref.ptr(pc.inp).value, ukref.ptr(out).value)
+    assert lib.iree_amd_uk_pack_host(C.byref(p)) == 0
+    assert np.array_equal(out, pc.run_oracle())
+    ucase = ukref.UnpackCase(rng, F.UNPACK_TYPE_I32I32, 3, 5, 32, 32, pad="one_incomplete_tile",
+                             loose_strides=True, offsets=True, out_stride1=2)
+    out = ucase.out_init.copy()
+    p = ucase.params(ukref.ptr(ucase.inp).value, ukref.ptr(out).value)
+    assert lib.iree_amd_uk_unpack_host(C.byref(p)) == 0
+    assert np.array_equal(out, ucase.run_oracle())

@@ -1,0 +1,109 @@
+"""GPU parity of pack / unpack against the oracle, bit-exact, through the C ABI:
+the reference's own test matrix (tools/pack_test.c:137-246,
+tools/unpack_test.c:123-218) plus the gfx950 tile shapes, which take the
+streaming kernels, and the full-size bandwidth workload (f16 8191x5001 <-> 32x16)."""
+import hashlib
+import itertools
+import json
+import os
+
+import numpy as np
+import pytest
+
+import gpucase
+import ukref
+from iree_amd import flags as F
+from iree_amd import synth
+from test_oracle_pack import OUTER, PACK_TILES, PADS, UNPACK_TILES
+
+pytestmark = pytest.mark.gpu
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "golden.json")
+
+
+@pytest.mark.parametrize("type_flag,t0,t1", PACK_TILES)
+def test_pack_matches_oracle(uk, cuda, type_flag, t0, t1):
+    rng = np.random.default_rng(131 * type_flag + 7 * t0 + t1)
+    for (o0, o1), ti, to, pad in itertools.product(OUTER, (0, 1), (0, 1), PADS):
+        for aligned in (False, True):
+            # `aligned`: tight strides, zero offsets, unit inner stride -> the
+            # streaming kernel where the tile shape allows it
+            case = ukref.PackCase(rng, type_flag, o0, o1, t0, t1, transpose_inner=ti,
+                                  transpose_outer=to, pad=pad,
+                                  loose_strides=(not aligned) and bool(rng.integers(0, 2)),
+                                  offsets=not aligned,
+                                  in_stride1=1 if aligned else 1 + int(rng.integers(0, 2)))
+            got = gpucase.run_pack(case)
+            assert np.array_equal(got, case.run_oracle()), (o0, o1, ti, to, pad, aligned)
+
+
+@pytest.mark.parametrize("type_flag,t0,t1", UNPACK_TILES)
+def test_unpack_matches_oracle(uk, cuda, type_flag, t0, t1):
+    rng = np.random.default_rng(117 * type_flag + 5 * t0 + t1)
+    for (o0, o1), ti, to, pad in itertools.product(OUTER, (0, 1), (0, 1), PADS):
+        for aligned in (False, True):
+            case = ukref.UnpackCase(rng, type_flag, o0, o1, t0, t1, transpose_inner=ti,
+                                    transpose_outer=to, pad=pad,
+                                    loose_strides=(not aligned) and bool(rng.integers(0, 2)),
+                                    offsets=not aligned,
+                                    out_stride1=1 if aligned else 1 + int(rng.integers(0, 2)))
+            got = gpucase.run_unpack(case)
+            # compares the WHOLE destination buffer: elements outside the
+            # matrix (stride gaps, the tail) must be untouched
+            assert np.array_equal(got, case.run_oracle()), (o0, o1, ti, to, pad, aligned)
+
+
+@pytest.mark.parametrize("type_flag,t0,t1,rows,cols", [
+    (F.PACK_TYPE_F16F16, 32, 16, 333, 1001),   # odd row pitch: 2-byte aligned rows
+    (F.PACK_TYPE_F16F16, 32, 8, 95, 257),
+    (F.PACK_TYPE_I8I8, 32, 16, 129, 1003),     # 1-byte aligned rows
+    (F.PACK_TYPE_I8I8, 32, 32, 64, 4096),
+    (F.PACK_TYPE_F32F32, 32, 32, 70, 515),
+    (F.PACK_TYPE_I32I32, 8, 4, 37, 123),
+    (F.PACK_TYPE_BF16BF16, 16, 64, 100, 700),
+])
+def test_streaming_shapes_with_ragged_edges(uk, cuda, type_flag, t0, t1, rows, cols):
+    rng = np.random.default_rng(rows * cols)
+    for to in (0, 1):
+        o0, o1 = -(-rows // t0), -(-cols // t1)
+        case = ukref.PackCase(rng, type_flag, o0, o1, t0, t1, transpose_outer=to,
+                              in_size=(rows, cols))
+        packed = gpucase.run_pack(case)
+        assert np.array_equal(packed, case.run_oracle()), (to,)
+        if type_flag != F.PACK_TYPE_I8I8:
+            ucase = ukref.UnpackCase(rng, type_flag, o0, o1, t0, t1, transpose_outer=to,
+                                     out_size=(rows, cols))
+            assert np.array_equal(gpucase.run_unpack(ucase), ucase.run_oracle()), (to,)
+
+
+def test_full_size_f16_8191x5001_pack_unpack_round_trip(uk, cuda):
+    """The bandwidth workload at its real size: packed bytes equal the oracle's
+    (and the committed SHA-256 produced by the reference library), the padded
+    row and columns hold the padding value, and unpack restores the source."""
+    import torch
+    R, Cc, T0, T1 = 8191, 5001, 32, 16
+    O0, O1 = -(-R // T0), -(-Cc // T1)
+    x = synth.uniform_pm1_f16(1, R * Cc).view(np.uint16)
+    xd = torch.from_numpy(x.view(np.int16)).cuda()
+    packed = torch.full((O0 * O1 * T0 * T1,), 0x5A5A, dtype=torch.int16, device="cuda")
+    uk.pack(xd, packed, R, Cc, O0, O1, T0, T1, 0, F.PACK_TYPE_F16F16)
+    back = torch.full((R * Cc + 64,), 0x1234, dtype=torch.int16, device="cuda")
+    uk.unpack(packed, back, O0, O1, T0, T1, R, Cc, F.UNPACK_TYPE_F16F16)
+    torch.cuda.synchronize()
+    got = packed.cpu().numpy().view(np.uint16)
+    # oracle at full size (a few hundred ms of C)
+    import ctypes as C
+    from iree_amd._lib import PackParams
+    want = np.full(O0 * O1 * T0 * T1, 0x5A5A, np.uint16)
+    p = PackParams(ukref.ptr(x).value, 0, Cc, 1, ukref.ptr(want).value, 0, O1 * T0 * T1, T0 * T1,
+                   R, Cc, O0, O1, T0, T1, 0, F.PACK_TYPE_F16F16, None)
+    assert ukref.oracle().oracle_pack(C.byref(p)) == 0
+    assert np.array_equal(got, want)
+    with open(GOLDEN) as f:
+        golden = json.load(f)
+    assert hashlib.sha256(got.tobytes()).hexdigest() == golden["pack_f16_8191x5001_32x16_sha256"]
+    t = got.reshape(O0, O1, T0, T1)
+    assert not t[-1, :, R - (O0 - 1) * T0:, :].any()      # 1 padded row
+    assert not t[:, -1, :, Cc - (O1 - 1) * T1:].any()     # 7 padded columns
+    b = back.cpu().numpy().view(np.uint16)
+    assert np.array_equal(b[:R * Cc], x)
+    assert (b[R * Cc:] == 0x1234).all()
