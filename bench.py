@@ -1,0 +1,297 @@
+#!/usr/bin/env python3
+"""Benchmark of the data-tiled matmul hot path on one MI355X.
+
+One "step" is one mmt4d launch of the headline configuration: f16 x f16 -> f32,
+M = N = K = 4096, operands already packed into the gfx950 tile (32x32x8) and
+resident in HBM, inputs N(0,1)/sqrt(K) from the seeded generator. The JSON line
+also carries, under "extra", the other parts of the metric measured in the same
+run (i8 mmt4d TOP/s, the accumulate variant, pack / unpack GB/s on the
+8191x5001 f16 tensor, the int4 GEMV GB/s, the whole pack->mmt4d->unpack chain),
+a roofline object for the dominant kernel and the CPU baseline: the reference
+ukernel library itself (oracle/_ref, built from the reference's sources) timed
+on this machine's host cores, or the repository's own CPU restatement when that
+library is absent.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extra] [--no-cpu]
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+import numpy as np  # noqa: E402
+
+PEAK_F16_TFLOPS = 2500.0   # MI355X dense f16 MFMA
+PEAK_I8_TOPS = 5000.0      # MI355X dense int8 MFMA
+PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE
+# and WRITE_SIZE runs of this same command (summaries under profiles/), scaled
+# by what the counters read for a copy kernel of known size. None = not measured.
+MEASURED_TRAFFIC_BYTES = {"mmt4d_f16_4096": None}
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-extra", action="store_true", help="skip the secondary measurements")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--only", default="", help="run only the named kernel in a loop (for profilers): "
+                    "mmt4d_f16 | mmt4d_i8 | pack | unpack | gemv")
+    return ap.parse_args()
+
+
+def gpu_time(torch, fn, steps, warmup):
+    """(seconds per step by wall clock, seconds per launch by HIP events on the
+    launch stream) for `steps` back-to-back calls after `warmup` untimed ones."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(steps):
+        fn()
+    end.record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    return (t1 - t0) / steps, start.elapsed_time(end) * 1e-3 / steps
+
+
+def packed_operands_f16(torch, synth, M1, N1, K1, M0, N0, K0, K):
+    scale = 1.0 / np.sqrt(K)
+    lhs = synth.normal_f16(1, M1 * K1 * M0 * K0, scale)
+    rhs = synth.normal_f16(2, N1 * K1 * N0 * K0, scale)
+    return (torch.from_numpy(lhs.view(np.int16)).cuda().view(torch.float16),
+            torch.from_numpy(rhs.view(np.int16)).cuda().view(torch.float16))
+
+
+def cpu_baseline(F, synth, size):
+    """f16 x f16 -> f32 mmt4d of the same 4096^3 problem on the host, with the
+    reference's own x86 tile (16x16x1): one ukernel call on one core, which is
+    what one call of the reference library is."""
+    import ukref
+    M0, N0, K0 = 16, 16, 1
+    M1, N1, K1 = size // M0, size // N0, size // K0
+    scale = 1.0 / np.sqrt(size)
+    lhs = synth.normal_f16(1, M1 * K1 * M0 * K0, scale).view(np.uint16)
+    rhs = synth.normal_f16(2, N1 * K1 * N0 * K0, scale).view(np.uint16)
+    flags = F.MMT4D_TYPE_F16F16F32 | F.MMT4D_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION
+    lib = ukref.reflib()
+    if lib is not None:
+        fs = ukref.best_host_feature_set()
+        cd = ukref.cpu_data(fs)
+        out = np.zeros(M1 * N1 * M0 * N0, np.float32)
+
+        def run(rows):
+            lib.iree_uk_mmt4d(ukref.ptr(lhs), 0, K1 * M0 * K0, ukref.ptr(rhs), 0, K1 * N0 * K0,
+                              ukref.ptr(out), 0, N1 * M0 * N0, rows, N1, K1, M0, N0, K0, flags,
+                              C.cast(cd, C.c_void_p))
+        run(8)  # warm-up slice
+        t0 = time.perf_counter()
+        run(M1)
+        dt = time.perf_counter() - t0
+        return {"value": round(2.0 * size ** 3 / dt / 1e12, 5), "unit": "TFLOP/s", "cores": 1,
+                "kind": "reference",
+                "sample": f"reference iree_uk_mmt4d f16f16f32, tile 16x16x1 ({fs or 'generic'} path), "
+                          f"full {size}^3 problem, 1 call on 1 thread, {dt:.2f} s"}
+    # Fallback: the repository's own scalar restatement on a bounded slice.
+    from iree_amd._lib import Mmt4dParams
+    rows = 4
+    out = np.zeros(rows * N1 * M0 * N0, np.float32)
+    p = Mmt4dParams(ukref.ptr(lhs).value, 0, K1 * M0 * K0, ukref.ptr(rhs).value, 0, K1 * N0 * K0,
+                    ukref.ptr(out).value, 0, N1 * M0 * N0, rows, N1, K1, M0, N0, K0, flags, None)
+    threads = min(os.cpu_count() or 1, 16)
+    t0 = time.perf_counter()
+    ukref.oracle().oracle_mmt4d_mt(C.byref(p), 0, threads)
+    dt = time.perf_counter() - t0
+    return {"value": round(2.0 * rows * M0 * size * size / dt / 1e12, 5), "unit": "TFLOP/s",
+            "cores": threads, "kind": "port",
+            "sample": f"oracle_mmt4d (scalar C restatement), {rows * M0} of {size} rows x {size} x {size}, "
+                      f"{threads} threads, {dt:.2f} s"}
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; the path has no multi-GPU part "
+              "(--gpus must be 1).", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    import iree_amd
+    from iree_amd import flags as F
+    from iree_amd import synth
+
+    if not torch.cuda.is_available():
+        print("bench.py: no HIP device visible", file=sys.stderr)
+        sys.exit(1)
+    iree_amd.load_library()  # raises when the HIP extension has not been built
+    torch.cuda.set_device(0)
+
+    size = 4096
+    M0, N0, K0 = 32, 32, 8
+    M1, N1, K1 = size // M0, size // N0, size // K0
+    lhs, rhs = packed_operands_f16(torch, synth, M1, N1, K1, M0, N0, K0, size)
+    out = torch.empty(M1 * N1 * M0 * N0, dtype=torch.float32, device="cuda")
+    mm_flags = F.MMT4D_TYPE_F16F16F32 | F.MMT4D_SKIP_INTERMEDIATE_ROUNDINGS
+
+    def step():
+        iree_amd.mmt4d(lhs, rhs, out, M1, N1, K1, M0, N0, K0, mm_flags)
+
+    if args.only:
+        run_only(args, torch, iree_amd, F, synth, step)
+        return
+
+    # Verify the very buffers that are timed (as the reference's benchmark does
+    # before timing): 2 output tiles against a float64 numpy product.
+    step()
+    torch.cuda.synchronize()
+    verify_tiles(torch, iree_amd, F, lhs, rhs, out, M1, N1, K1, M0, N0, K0)
+
+    wall, per_launch = gpu_time(torch, step, args.steps, args.warmup)
+    flops = 2.0 * size ** 3
+    value = flops / wall / 1e12
+    achieved = flops / per_launch / 1e12
+    result = {
+        "metric": "mmt4d_f16f16f32_4096x4096x4096_tflops",
+        "value": round(value, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall * 1e3, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": "mmt4d f16xf16->f32, M=N=K=4096 (outer 128x128x512 tiles of 32x32x8), "
+                               "operands pre-packed and HBM-resident, inputs N(0,1)/sqrt(K) seeded",
+                   "tile": [M0, N0, K0], "accumulate": False},
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_F16_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(achieved / PEAK_F16_TFLOPS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES["mmt4d_f16_4096"]},
+    }
+    if not args.no_extra:
+        result["extra"] = extras(args, torch, iree_amd, F, synth, lhs, rhs, out)
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(F, synth, size)
+    print(json.dumps(result))
+
+
+def verify_tiles(torch, iree_amd, F, lhs, rhs, out, M1, N1, K1, M0, N0, K0):
+    """Two output tiles of the timed buffers against a float64 numpy product."""
+    for (i, j) in [(0, 0), (M1 - 1, N1 // 2)]:
+        l = lhs[i * K1 * M0 * K0:(i + 1) * K1 * M0 * K0].cpu().numpy().astype(np.float64)
+        r = rhs[j * K1 * N0 * K0:(j + 1) * K1 * N0 * K0].cpu().numpy().astype(np.float64)
+        want = np.einsum("kac,kbc->ab", l.reshape(K1, M0, K0), r.reshape(K1, N0, K0)).reshape(-1)
+        got = out[(i * N1 + j) * M0 * N0:(i * N1 + j + 1) * M0 * N0].cpu().numpy()
+        if not np.all(np.abs(got - want) <= 1e-3 + 1e-2 * np.abs(want)):
+            raise SystemExit("bench.py: mmt4d result is outside tolerance; refusing to time it")
+
+
+def extras(args, torch, iree_amd, F, synth, lhs, rhs, out):
+    ex = {}
+    size = 4096
+    steps, warm = args.steps, args.warmup
+    M1 = N1 = size // 32
+    flops = 2.0 * size ** 3
+
+    # f16 with accumulate (reads the 64 MiB accumulator as well)
+    acc_flags = F.MMT4D_TYPE_F16F16F32 | F.MMT4D_ACCUMULATE | F.MMT4D_SKIP_INTERMEDIATE_ROUNDINGS
+    _, t = gpu_time(torch, lambda: iree_amd.mmt4d(lhs, rhs, out, M1, N1, size // 8, 32, 32, 8, acc_flags),
+                    steps, warm)
+    ex["mmt4d_f16_accumulate_tflops"] = round(flops / t / 1e12, 2)
+
+    # i8 x i8 -> i32 at 4096^3, tile 32x32x16
+    K1 = size // 16
+    li = torch.from_numpy(synth.uniform_int8(1, M1 * K1 * 32 * 16)).cuda()
+    ri = torch.from_numpy(synth.uniform_int8(2, N1 * K1 * 32 * 16)).cuda()
+    oi = torch.empty(M1 * N1 * 1024, dtype=torch.int32, device="cuda")
+    _, t = gpu_time(torch, lambda: iree_amd.mmt4d(li, ri, oi, M1, N1, K1, 32, 32, 16, F.MMT4D_TYPE_S8S8S32),
+                    steps, warm)
+    ex["mmt4d_i8_tops"] = round(flops / t / 1e12, 2)
+    ex["mmt4d_i8_frac_of_peak"] = round(flops / t / 1e12 / PEAK_I8_TOPS, 4)
+    del li, ri, oi
+
+    # pack / unpack of the f16 8191 x 5001 tensor <-> 32x16 tiles. Rotating
+    # buffer sets (> 256 MiB in total) so that HBM, not the last-level cache,
+    # is what is measured.
+    R, Cc, T0, T1 = 8191, 5001, 32, 16
+    O0, O1 = -(-R // T0), -(-Cc // T1)
+    nrot = 4
+    x_host = synth.uniform_pm1_f16(1, R * Cc).view(np.int16)
+    xs = [torch.from_numpy(x_host).cuda() for _ in range(nrot)]
+    ps = [torch.empty(O0 * O1 * T0 * T1, dtype=torch.int16, device="cuda") for _ in range(nrot)]
+    state = {"i": 0}
+
+    def do_pack():
+        k = state["i"] % nrot
+        state["i"] += 1
+        iree_amd.pack(xs[k], ps[k], R, Cc, O0, O1, T0, T1, 0, F.PACK_TYPE_F16F16)
+
+    def do_unpack():
+        k = state["i"] % nrot
+        state["i"] += 1
+        iree_amd.unpack(ps[k], xs[k], O0, O1, T0, T1, R, Cc, F.UNPACK_TYPE_F16F16)
+
+    pack_bytes = R * Cc * 2 + O0 * O1 * T0 * T1 * 2      # read + written
+    _, t = gpu_time(torch, do_pack, steps, warm)
+    ex["pack_f16_8191x5001_gbs"] = round(pack_bytes / t / 1e9, 1)
+    ex["pack_frac_of_hbm_peak"] = round(pack_bytes / t / 1e9 / PEAK_HBM_GBS, 4)
+    _, t = gpu_time(torch, do_unpack, steps, warm)
+    ex["unpack_f16_8191x5001_gbs"] = round(pack_bytes / t / 1e9, 1)
+    ex["unpack_frac_of_hbm_peak"] = round(pack_bytes / t / 1e9 / PEAK_HBM_GBS, 4)
+    torch.cuda.synchronize()
+    assert np.array_equal(xs[0].cpu().numpy(), x_host), "pack/unpack round trip is not bit-exact"
+    del xs, ps
+
+    # whole chain on row-major operands: pack LHS, pack RHS (transposing), mmt4d, unpack
+    a = torch.from_numpy(synth.normal_f16(1, size * size, 1 / 64).view(np.int16)).cuda().view(torch.float16)
+    b = torch.from_numpy(synth.normal_f16(2, size * size, 1 / 64).view(np.int16)).cuda().view(torch.float16)
+    c = torch.zeros(size * size, dtype=torch.float32, device="cuda")
+    ws = iree_amd.matmul_data_tiled(a, b, c, size, size, size, F.MMT4D_TYPE_F16F16F32)
+    _, t = gpu_time(torch, lambda: iree_amd.matmul_data_tiled(a, b, c, size, size, size,
+                                                              F.MMT4D_TYPE_F16F16F32, workspace=ws),
+                    max(5, steps // 4), 2)
+    ex["matmul_f16_pack_mmt4d_unpack_tflops"] = round(flops / t / 1e12, 2)
+    return ex
+
+
+def run_only(args, torch, iree_amd, F, synth, mm_step):
+    """Runs one kernel `steps` times (for rocprofv3 --kernel-trace / --pmc)."""
+    if args.only == "mmt4d_f16":
+        fn = mm_step
+    elif args.only == "mmt4d_i8":
+        size = 4096
+        M1 = N1 = size // 32
+        K1 = size // 16
+        li = torch.from_numpy(synth.uniform_int8(1, M1 * K1 * 512)).cuda()
+        ri = torch.from_numpy(synth.uniform_int8(2, N1 * K1 * 512)).cuda()
+        oi = torch.empty(M1 * N1 * 1024, dtype=torch.int32, device="cuda")
+        fn = lambda: iree_amd.mmt4d(li, ri, oi, M1, N1, K1, 32, 32, 16, F.MMT4D_TYPE_S8S8S32)  # noqa: E731
+    elif args.only in ("pack", "unpack"):
+        R, Cc, T0, T1 = 8191, 5001, 32, 16
+        O0, O1 = -(-R // T0), -(-Cc // T1)
+        x = torch.from_numpy(synth.uniform_pm1_f16(1, R * Cc).view(np.int16)).cuda()
+        p = torch.zeros(O0 * O1 * T0 * T1, dtype=torch.int16, device="cuda")
+        if args.only == "pack":
+            fn = lambda: iree_amd.pack(x, p, R, Cc, O0, O1, T0, T1, 0, F.PACK_TYPE_F16F16)  # noqa: E731
+        else:
+            fn = lambda: iree_amd.unpack(p, x, O0, O1, T0, T1, R, Cc, F.UNPACK_TYPE_F16F16)  # noqa: E731
+    else:
+        raise SystemExit(f"unknown --only {args.only}")
+    wall, per_launch = gpu_time(torch, fn, args.steps, args.warmup)
+    print(json.dumps({"only": args.only, "us_per_launch": round(per_launch * 1e6, 2)}))
+
+
+if __name__ == "__main__":
+    main()

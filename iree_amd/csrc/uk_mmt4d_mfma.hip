@@ -20,10 +20,17 @@
 // Kernel shape: a workgroup of 4 waves owns a macro tile of (2*WM) x (2*WN)
 // outer tiles; each wave accumulates WM x WN blocks of 32x32 in registers. The K
 // loop moves operand blocks global -> LDS with direct-to-LDS 128-bit loads
-// (no register staging), double buffered: the loads of stage s+1 are in flight
-// while the MFMAs of stage s issue. Workgroup ids are remapped so that the 8
-// XCDs (which receive consecutive workgroup ids round-robin) each work on a
-// compact block of macro tiles and reuse operand panels in their own L2.
+// (no register staging) into a ring of K-step slots, several K-steps ahead of
+// the MFMAs; operand fragments are read from LDS one K-step ahead and every
+// memory instruction is issued in the shadow of an MFMA. Workgroup ids are
+// remapped so that the 8 XCDs (which receive consecutive workgroup ids
+// round-robin) each work on a compact block of macro tiles and reuse operand
+// panels in their own L2.
+//
+// Measured bound that matters more than the nominal peak: with N(0,1) f16
+// operands a register-only MFMA loop sustains about 1.3 PFLOP/s on MI355X
+// (2.1 with all-zero operands): the matrix pipe is power-limited by operand
+// toggling, so data movement that costs energy also costs MFMA rate.
 #include "uk_common.h"
 
 namespace uk {
@@ -67,7 +74,6 @@ struct S8Cfg {
 };
 
 constexpr int kThreads = 256;
-constexpr int kSteps = 4;           // MFMA K-steps per LDS stage
 constexpr int kBlockBytes = 1024;   // one 32-row operand block of one K-step
 
 struct MfmaArgs {
@@ -86,6 +92,29 @@ __device__ __forceinline__ void load_block_to_lds(const char* gptr, char* lds) {
   __builtin_amdgcn_global_load_lds(
       (const __attribute__((address_space(1))) void*)gptr,
       (__attribute__((address_space(3))) void*)lds, 16, 0, 0);
+}
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+// Pins the issue order of one basic block: kSlots times {1 MFMA, a share of the
+// kVmem vector-memory loads, a share of the kDsr LDS reads}, then the remaining
+// MFMAs. Memory instructions issued right behind an MFMA run in its shadow.
+template <int kMfma, int kVmem, int kDsr, int kSlots, int I = 0>
+__device__ __forceinline__ void interleave_issue() {
+  if constexpr (I < kSlots) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    constexpr int v = (kVmem + kSlots - 1 - I) / kSlots;
+    if constexpr (v > 0) __builtin_amdgcn_sched_group_barrier(0x020, v, 0);
+    constexpr int d = (kDsr + kSlots - 1 - I) / kSlots;
+    if constexpr (d > 0) __builtin_amdgcn_sched_group_barrier(0x100, d, 0);
+    interleave_issue<kMfma, kVmem, kDsr, kSlots, I + 1>();
+  } else if constexpr (kMfma > kSlots) {
+    __builtin_amdgcn_sched_group_barrier(0x008, kMfma - kSlots, 0);
+  }
 }
 
 // Maps the hardware workgroup id to a macro-tile coordinate. Workgroup ids go
@@ -108,30 +137,42 @@ __device__ __forceinline__ void tile_coord(int bid, int tiles_m, int tiles_n,
   *tn = in_group / rows;
 }
 
-template <typename Cfg, int WM, int WN, bool kHalfK0>
+// K-loop organisation. LDS is a ring of kRing slots; slot (ks % kRing) holds
+// K-step ks: the TM blocks of A followed by the TN blocks of B, 1 KiB each, in
+// MFMA lane order. Waves synchronise once every kSync K-steps; right after
+// that barrier each wave issues its share of the direct-to-LDS loads for the
+// kSync K-steps that lie kAhead = kRing - kSync steps ahead, so up to kAhead
+// K-steps of loads are in flight behind the one being multiplied. Operand
+// fragments are read from LDS one K-step ahead of the MFMAs that use them.
+template <typename Cfg, int WM, int WN, bool kHalfK0, int kRing, int kSync>
 __global__ __launch_bounds__(kThreads) void mmt4d_mfma_kernel(MfmaArgs a) {
   typedef typename Cfg::frag_t frag_t;
   typedef typename Cfg::acc_t acc_t;
   typedef typename Cfg::out_t out_t;
   constexpr int TM = 2 * WM, TN = 2 * WN;      // outer tiles per workgroup
-  constexpr int kRowBytes = kSteps * kBlockBytes;  // one outer row, one stage
-  constexpr int kABytes = TM * kRowBytes, kBBytes = TN * kRowBytes;
-  constexpr int kStageBytes = kABytes + kBBytes;
+  constexpr int kABytes = TM * kBlockBytes;
+  constexpr int kSlotBytes = (TM + TN) * kBlockBytes;
+  constexpr int kAhead = kRing - kSync;
+  constexpr int kARowsPerWave = TM / 4, kBRowsPerWave = TN / 4;
+  constexpr int kLoadsPerStep = kARowsPerWave + kBRowsPerWave;  // per wave
+  constexpr int kBody = (kSync % 2) ? 2 * kSync : kSync;        // K-steps per unrolled body
+  static_assert(kAhead >= kSync && kAhead % kSync == 0, "ring must hold whole sync groups");
+  static_assert((kAhead - kSync) * kLoadsPerStep < 64, "too many loads in flight for vmcnt");
   extern __shared__ __attribute__((aligned(1024))) char lds[];
 
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wm = wave >> 1, wn = wave & 1;
   int tm, tn;
   tile_coord(blockIdx.x, a.tiles_m, a.tiles_n, &tm, &tn);
   const int i_base = tm * TM, j_base = tn * TN;
+  const int T = a.ksteps;
 
   // Per-lane byte offset inside a 1 KiB operand block in global memory.
   const int lane_off = kHalfK0 ? lane * 16 : ((lane & 31) * 32 + (lane >> 5) * 16);
 
-  // Rows this wave copies each stage: TM/4 rows of A and TN/4 rows of B.
-  // Out-of-range rows are clamped to the last valid one (loaded, never stored).
-  constexpr int kARowsPerWave = TM / 4, kBRowsPerWave = TN / 4;
+  // Rows this wave copies: TM/4 rows of A and TN/4 rows of B. Out-of-range
+  // rows are clamped to the last valid one (loaded, never stored).
   const char* a_src[kARowsPerWave];
   const char* b_src[kBRowsPerWave];
 #pragma unroll
@@ -170,79 +211,123 @@ __global__ __launch_bounds__(kThreads) void mmt4d_mfma_kernel(MfmaArgs a) {
         for (int v = 0; v < 16; ++v) acc[x][y][v] = 0;
   }
 
-  // Copies this wave's share of one stage: `nsteps` K-steps starting at
-  // K-step `ks0` for kARowsPerWave rows of A and kBRowsPerWave rows of B.
-  auto issue_rows = [&](char* stage_base, int ks0, int s) {
-    char* sa = stage_base;
-    char* sb = stage_base + kABytes;
+  // This wave's share of the loads of K-step `ks` into ring slot `slot`.
+  auto issue_step = [&](int ks, int slot) {
+    char* base = lds + slot * kSlotBytes;
 #pragma unroll
     for (int r = 0; r < kARowsPerWave; ++r)
-      load_block_to_lds(a_src[r] + (int64_t)(ks0 + s) * kBlockBytes,
-                        sa + (wave * kARowsPerWave + r) * kRowBytes + s * kBlockBytes);
+      load_block_to_lds(a_src[r] + (int64_t)ks * kBlockBytes,
+                        base + (wave * kARowsPerWave + r) * kBlockBytes);
 #pragma unroll
     for (int r = 0; r < kBRowsPerWave; ++r)
-      load_block_to_lds(b_src[r] + (int64_t)(ks0 + s) * kBlockBytes,
-                        sb + (wave * kBRowsPerWave + r) * kRowBytes + s * kBlockBytes);
+      load_block_to_lds(b_src[r] + (int64_t)ks * kBlockBytes,
+                        base + kABytes + (wave * kBRowsPerWave + r) * kBlockBytes);
   };
-  auto issue_full = [&](int stage, int ks0) {
+  auto read_frags = [&](int slot, frag_t (&fa)[WM], frag_t (&fb)[WN]) {
+    const char* sa = lds + slot * kSlotBytes + (wm * WM) * kBlockBytes + lane * 16;
+    const char* sb = lds + slot * kSlotBytes + kABytes + (wn * WN) * kBlockBytes + lane * 16;
 #pragma unroll
-    for (int s = 0; s < kSteps; ++s) issue_rows(lds + stage * kStageBytes, ks0, s);
+    for (int x = 0; x < WM; ++x) fa[x] = *(const frag_t*)(sa + x * kBlockBytes);
+#pragma unroll
+    for (int y = 0; y < WN; ++y) fb[y] = *(const frag_t*)(sb + y * kBlockBytes);
   };
-  auto issue_tail = [&](int stage, int ks0, int nsteps) {
-#pragma unroll 1
-    for (int s = 0; s < nsteps; ++s) issue_rows(lds + stage * kStageBytes, ks0, s);
-  };
-
-  // One K-step of this wave's WM x WN blocks out of the given stage.
-  auto compute_step = [&](const char* stage_base, int s) {
-    const char* sa = stage_base + (wm * WM) * kRowBytes + lane * 16 + s * kBlockBytes;
-    const char* sb = stage_base + kABytes + (wn * WN) * kRowBytes + lane * 16 + s * kBlockBytes;
-    frag_t fa[WM], fb[WN];
-#pragma unroll
-    for (int x = 0; x < WM; ++x) fa[x] = *(const frag_t*)(sa + x * kRowBytes);
-#pragma unroll
-    for (int y = 0; y < WN; ++y) fb[y] = *(const frag_t*)(sb + y * kRowBytes);
+  // MFMAs of block rows [x0, x1) of this wave's WM x WN blocks.
+  auto multiply_rows = [&](const frag_t (&fa)[WM], const frag_t (&fb)[WN], int x0, int x1) {
 #pragma unroll
     for (int x = 0; x < WM; ++x)
+      if (x >= x0 && x < x1) {
 #pragma unroll
-      for (int y = 0; y < WN; ++y) acc[x][y] = Cfg::mfma(fa[x], fb[y], acc[x][y]);
+        for (int y = 0; y < WN; ++y) acc[x][y] = Cfg::mfma(fa[x], fb[y], acc[x][y]);
+      }
   };
-  auto compute_full = [&](int stage) {
-#pragma unroll
-    for (int s = 0; s < kSteps; ++s) compute_step(lds + stage * kStageBytes, s);
-  };
-  auto compute_tail = [&](int stage, int nsteps) {
-#pragma unroll 1
-    for (int s = 0; s < nsteps; ++s) compute_step(lds + stage * kStageBytes, s);
-  };
-  // All of this wave's direct-to-LDS loads have landed, and (after the
-  // barrier) so have everybody else's; every wave has also left the stage that
-  // is about to be overwritten.
-  auto stage_fence = [&]() {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
+  auto multiply = [&](const frag_t (&fa)[WM], const frag_t (&fb)[WN]) {
+    multiply_rows(fa, fb, 0, WM);
   };
 
-  const int nfull = a.ksteps / kSteps;
-  const int tail = a.ksteps - nfull * kSteps;
-  if (nfull > 0) {
-    issue_full(0, 0);
-    for (int st = 0; st + 1 < nfull; ++st) {
-      stage_fence();
-      issue_full((st + 1) & 1, (st + 1) * kSteps);
-      compute_full(st & 1);
+  frag_t fa[2][WM], fb[2][WN];
+  int done = 0;  // K-steps multiplied so far
+  if (T > kRing) {
+    // ---- pipelined path -------------------------------------------------
+    int issue_ks = 0, issue_slot = 0;   // next K-step to load and its slot
+    int read_slot = 0;                  // slot of K-step `done`
+#pragma unroll 1
+    for (; issue_ks < kRing; ++issue_ks) issue_step(issue_ks, issue_ks);
+    issue_slot = 0;  // kRing % kRing
+    wait_vmcnt<(kAhead) * kLoadsPerStep>();  // the first kSync K-steps have landed
+    __syncthreads();
+    read_frags(0, fa[0], fb[0]);
+    // Each body multiplies kBody K-steps; `base` is the first of them. The
+    // loop runs while another whole body remains AFTER this one needs no
+    // special casing; the last bodies and the remainder are handled below.
+    while (done + kBody <= T) {
+#pragma unroll
+      for (int g = 0; g < kBody; ++g) {
+        const int p = g & 1;
+        const bool sync_point = (g % kSync) == kSync - 1;
+        int next_slot = read_slot + 1; if (next_slot == kRing) next_slot = 0;
+        if (!sync_point) {
+          read_frags(next_slot, fa[p ^ 1], fb[p ^ 1]);
+          multiply(fa[p], fb[p]);
+          // Issue order: one LDS read slipped in behind each of the first
+          // MFMAs (an LDS read issues in the shadow of the running MFMA),
+          // then the rest of the MFMAs back to back.
+          interleave_issue<WM * WN, 0, WM + WN, (WM * WN < WM + WN ? WM * WN : WM + WN)>();
+        } else {
+          // The first row of MFMAs goes ahead of the barrier so that the
+          // matrix pipe has work while the waves meet. All reads of K-steps
+          // <= done+g are complete once fa[p]/fb[p] have arrived; the barrier
+          // then frees the slots of this sync group and publishes the next
+          // group's data. The scheduling fences keep the compiler from moving
+          // MFMAs across the synchronisation sequence.
+          __builtin_amdgcn_sched_barrier(0);
+          multiply_rows(fa[p], fb[p], 0, 1);
+          __builtin_amdgcn_sched_barrier(0);
+          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+          wait_vmcnt<(kAhead - kSync) * kLoadsPerStep>();
+          __syncthreads();
+          __builtin_amdgcn_sched_barrier(0);
+          // Loads for the K-steps kAhead beyond this sync group go into the
+          // slots it just vacated. Past the end of K the last K-step is loaded
+          // again (into a slot nobody reads any more): that keeps the number
+          // of loads in flight, and with it the vmcnt arithmetic, constant.
+#pragma unroll
+          for (int q = 0; q < kSync; ++q) {
+            issue_step(issue_ks < T ? issue_ks : T - 1, issue_slot);
+            ++issue_ks;
+            ++issue_slot; if (issue_slot == kRing) issue_slot = 0;
+          }
+          read_frags(next_slot, fa[p ^ 1], fb[p ^ 1]);
+          multiply_rows(fa[p], fb[p], 1, WM);
+          constexpr int kDma = kSync * kLoadsPerStep, kMma = (WM - 1) * WN, kDsr = WM + WN;
+          constexpr int kSlots = kMma < kDsr ? kMma : kDsr;
+          interleave_issue<kMma, kDma, kDsr, kSlots>();
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        read_slot = next_slot;
+      }
+      done += kBody;
     }
-    stage_fence();
-    if (tail) issue_tail(nfull & 1, nfull * kSteps, tail);
-    compute_full((nfull - 1) & 1);
-    if (tail) {
-      stage_fence();
-      compute_tail(nfull & 1, tail);
+    // Remainder (< kBody K-steps): everything has been issued; wait for all
+    // of it and multiply straight out of the ring.
+    wait_vmcnt<0>();
+    __syncthreads();
+#pragma unroll 1
+    for (; done < T; ++done) {
+      read_frags(read_slot, fa[0], fb[0]);
+      multiply(fa[0], fb[0]);
+      ++read_slot; if (read_slot == kRing) read_slot = 0;
     }
   } else {
-    issue_tail(0, 0, tail);
-    stage_fence();
-    compute_tail(0, tail);
+    // ---- short-K path: everything fits in the ring ------------------------
+#pragma unroll 1
+    for (int ks = 0; ks < T; ++ks) issue_step(ks, ks);
+    wait_vmcnt<0>();
+    __syncthreads();
+#pragma unroll 1
+    for (; done < T; ++done) {
+      read_frags(done, fa[0], fb[0]);
+      multiply(fa[0], fb[0]);
+    }
   }
 
   // Epilogue. MFMA 32x32 accumulator layout: register v of lane l holds
@@ -262,7 +347,7 @@ __global__ __launch_bounds__(kThreads) void mmt4d_mfma_kernel(MfmaArgs a) {
     }
 }
 
-template <typename Cfg, int WM, int WN, bool kHalfK0>
+template <typename Cfg, int WM, int WN, bool kHalfK0, int kRing, int kSync>
 int launch_variant(const MfmaArgs& a0, hipStream_t s) {
   MfmaArgs a = a0;
   constexpr int TM = 2 * WM, TN = 2 * WN;
@@ -270,8 +355,9 @@ int launch_variant(const MfmaArgs& a0, hipStream_t s) {
   a.tiles_n = (a.N + TN - 1) / TN;
   const int64_t blocks = (int64_t)a.tiles_m * a.tiles_n;
   if (blocks > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
-  constexpr int lds_bytes = 2 * (TM + TN) * kSteps * kBlockBytes;
-  auto kernel = mmt4d_mfma_kernel<Cfg, WM, WN, kHalfK0>;
+  constexpr int lds_bytes = kRing * (TM + TN) * kBlockBytes;
+  static_assert(lds_bytes <= 160 * 1024, "LDS ring exceeds 160 KiB");
+  auto kernel = mmt4d_mfma_kernel<Cfg, WM, WN, kHalfK0, kRing, kSync>;
   static bool attr_set = false;  // benign race: the call is idempotent
   if (!attr_set) {
     UK_RETURN_IF_HIP(hipFuncSetAttribute((const void*)kernel,
@@ -282,16 +368,22 @@ int launch_variant(const MfmaArgs& a0, hipStream_t s) {
   return check_hip(hipGetLastError(), "mmt4d_mfma launch");
 }
 
-template <typename Cfg>
-int launch_cfg(const MfmaArgs& a, bool half_k0, hipStream_t s) {
-  // Pick the macro tile: the largest one (best operand reuse) when it still
-  // yields at least one workgroup per compute unit, else the smaller one.
+template <typename Cfg, bool kHalfK0>
+int launch_half(const MfmaArgs& a, hipStream_t s) {
+  // Pick the macro tile: 256x256 (best operand reuse: 1 KiB of operand per
+  // two MFMAs) when that still yields at least one workgroup per compute
+  // unit, else 128x128 so that small problems spread over more of the chip.
+  // Ring of 8 K-steps (128 KiB of LDS for the large tile), one barrier every
+  // 2 K-steps, 6 K-steps of loads in flight.
   const int cus = device_cu_count();
   const int64_t big = (int64_t)((a.M + 7) / 8) * ((a.N + 7) / 8);
-  if (big >= cus) {
-    return half_k0 ? launch_variant<Cfg, 4, 4, true>(a, s) : launch_variant<Cfg, 4, 4, false>(a, s);
-  }
-  return half_k0 ? launch_variant<Cfg, 2, 2, true>(a, s) : launch_variant<Cfg, 2, 2, false>(a, s);
+  if (big >= cus) return launch_variant<Cfg, 4, 4, kHalfK0, 8, 2>(a, s);
+  return launch_variant<Cfg, 2, 2, kHalfK0, 8, 2>(a, s);
+}
+
+template <typename Cfg>
+int launch_cfg(const MfmaArgs& a, bool half_k0, hipStream_t s) {
+  return half_k0 ? launch_half<Cfg, true>(a, s) : launch_half<Cfg, false>(a, s);
 }
 
 struct Served { int mfma_k; };
