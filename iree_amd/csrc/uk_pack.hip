@@ -96,10 +96,30 @@ __global__ __launch_bounds__(256) void unpack_generic_kernel(PackArgs a) {
 //   cpr  = chunks per tile row  = tile_cols / CE
 //   a "row of chunks" of the matrix has ceil(m_size1 / CE) chunks; chunk j of
 //   matrix row r lives in tile column j / cpr, tile row r % tile_rows.
+// All per-lane index arithmetic is 32-bit; divisions by run-time constants go
+// through a precomputed multiply-shift. The grid's y dimension walks the outer
+// rows of tiles (pack) or groups of matrix rows (unpack).
 //---------------------------------------------------------------------------
 
 constexpr int kStreamThreads = 256;
-constexpr int kStreamUnroll = 4;
+constexpr int kStreamUnroll = 2;
+
+// n / d for 0 <= n < 2^31 and a fixed d >= 1: (n * mul) >> shift.
+struct FastDiv {
+  uint32_t mul, shift, d;
+  __device__ __forceinline__ uint32_t div(uint32_t n) const {
+    return d == 1 ? n : (uint32_t)(((uint64_t)n * mul) >> shift);
+  }
+};
+FastDiv make_fastdiv(uint32_t d) {
+  FastDiv f;
+  f.d = d;
+  uint32_t l = 0;
+  while ((1ull << l) < d) ++l;
+  f.shift = 31 + l;
+  f.mul = (uint32_t)(((1ull << f.shift) + d - 1) / d);  // < 2^32 for d >= 2
+  return f;
+}
 
 struct StreamArgs {
   const char* mat;
@@ -109,23 +129,227 @@ struct StreamArgs {
   int64_t t_stride_row, t_stride_col;   // elements between tiles along matrix rows / cols
   int tile_rows, tile_cols;             // matrix orientation (== stored order)
   int cpr;                              // chunks per tile row
+  uint32_t chunks_per_row;              // ceil(m_size1 / CE)
+  uint32_t padded_chunks_per_row;       // outer_cols * cpr
+  int64_t padded_rows;                  // outer_rows * tile_rows
+  int64_t t_stride_row_bytes, t_stride_col_bytes;
+  int log2_tile_rows, log2_cpr;         // valid when both are powers of two
+  int pow2;
+  FastDiv by_cpr, by_tile_rows;
   uint64_t padding;
-  int64_t units;                        // work units (see kernels)
 };
 
-// pack: a work unit is one wave-sized run of 64 consecutive chunks of the tiled
-// buffer inside one outer row of tiles; a wave takes kStreamUnroll consecutive
-// runs. Consecutive chunks run along (tile column, tile row, chunk in row), so
-// 64 chunks are 1 KiB of contiguous destination.
-template <int ES>
+// Both kernels walk the MATRIX in blocks of 8 rows x 8 chunks (128 bytes of
+// each row) per wave instruction: lane = (row in block) * 8 + (chunk in block).
+// On the matrix side every row segment is 128 contiguous bytes; on the tiled
+// side the 8 rows of one tile column are contiguous as well (8 tile rows of
+// cpr chunks each), so neither side moves less than a cache line at a time.
+// A wave takes kStreamUnroll vertically adjacent blocks; the 4 waves of a
+// workgroup take 4 horizontally adjacent column strips. (Measured on MI355X:
+// two blocks per wave beat four and eight - more waves in flight matter more
+// than more bytes per wave.)
+constexpr int kBlockRows = 8, kBlockChunks = 8;
+
+// Position of matrix element (row r, chunk column j) in the tiled buffer, in
+// bytes from the buffer start. kPow2: tile_rows and cpr are powers of two (every
+// gfx950 tile shape is) and the divisions become shifts.
+template <bool kPow2>
+__device__ __forceinline__ int64_t tiled_chunk_offset(const StreamArgs& a, int64_t r, uint32_t j) {
+  int64_t panel;
+  uint32_t trow, tile_col, h;
+  if (kPow2) {
+    panel = r >> a.log2_tile_rows;
+    trow = (uint32_t)r & (a.tile_rows - 1);
+    tile_col = j >> a.log2_cpr;
+    h = j & (a.cpr - 1);
+  } else {
+    if (r < 0x7FFFFFFF) {
+      panel = a.by_tile_rows.div((uint32_t)r);
+      trow = (uint32_t)r - (uint32_t)panel * a.tile_rows;
+    } else {
+      panel = r / a.tile_rows;
+      trow = (uint32_t)(r - panel * a.tile_rows);
+    }
+    tile_col = a.by_cpr.div(j);
+    h = j - tile_col * a.cpr;
+  }
+  return panel * a.t_stride_row_bytes + (int64_t)tile_col * a.t_stride_col_bytes +
+         (int64_t)(trow * a.cpr + h) * 16;
+}
+
+template <int ES, bool kPow2>
 __global__ __launch_bounds__(kStreamThreads) void pack_stream_kernel(StreamArgs a) {
   constexpr int CE = 16 / ES;
   typedef typename Chunk<ES>::aligned_t src_vec_t;
-  const int lane = threadIdx.x & 63;
-  const int64_t wave = ((int64_t)blockIdx.x * kStreamThreads + threadIdx.x) >> 6;
-  const int64_t chunks_per_tile = (int64_t)a.tile_rows * a.cpr;
-  const int64_t chunks_per_panel = a.outer_cols * chunks_per_tile;
-  const int64_t runs_per_panel = ceil_div(chunks_per_panel, 64);
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t j0 = (blockIdx.x * 4 + wave) * kBlockChunks;   // first chunk column of the wave
+  if (j0 >= a.padded_chunks_per_row) return;
+  const uint32_t j = j0 + (lane & 7);
+  const int64_t c = (int64_t)j * CE;
+  const int64_t row_groups = ceil_div(a.padded_rows, kBlockRows * kStreamUnroll);
+  // Wave-uniform: every chunk of the strip lies wholly inside the matrix.
+  const bool cols_inside = (int64_t)(j0 + kBlockChunks) * CE <= a.m_size1;
+  for (int64_t rg = blockIdx.y; rg < row_groups; rg += gridDim.y) {
+    const int64_t r0 = rg * kStreamUnroll * kBlockRows;
+    if (cols_inside && r0 + kStreamUnroll * kBlockRows <= a.m_size0) {
+      // Interior: straight-line code, all loads in flight before the stores.
+      u32x4 v[kStreamUnroll];
+#pragma unroll
+      for (int u = 0; u < kStreamUnroll; ++u) {
+        const int64_t r = r0 + u * kBlockRows + (lane >> 3);
+        v[u] = *(const src_vec_t*)(a.mat + (r * a.m_stride0 + c) * ES);
+      }
+#pragma unroll
+      for (int u = 0; u < kStreamUnroll; ++u) {
+        const int64_t r = r0 + u * kBlockRows + (lane >> 3);
+        *(u32x4*)(a.tiled + tiled_chunk_offset<kPow2>(a, r, j)) = v[u];
+      }
+      continue;
+    }
+    // Edge: per-lane predicates, padding, and a byte-wise tail for the chunk
+    // that straddles the right edge (never reading past it).
+    u32x4 pad_vec;
+    {
+      uint64_t p = a.padding;
+      if (ES == 1) { p &= 0xFF; p |= p << 8; p |= p << 16; p |= p << 32; }
+      if (ES == 2) { p &= 0xFFFF; p |= p << 16; p |= p << 32; }
+      if (ES == 4) { p &= 0xFFFFFFFFull; p |= p << 32; }
+      pad_vec = u32x4{(uint32_t)p, (uint32_t)(p >> 32), (uint32_t)p, (uint32_t)(p >> 32)};
+    }
+    if (j >= a.padded_chunks_per_row) continue;
+#pragma unroll 1
+    for (int u = 0; u < kStreamUnroll; ++u) {
+      const int64_t r = r0 + u * kBlockRows + (lane >> 3);
+      if (r >= a.padded_rows) continue;
+      u32x4 v = pad_vec;
+      if (r < a.m_size0 && c < a.m_size1) {
+        const char* src = a.mat + (r * a.m_stride0 + c) * ES;
+        if (c + CE <= a.m_size1) {
+          v = *(const src_vec_t*)src;
+        } else {
+          union { u32x4 vec; uint8_t b[16]; } tmp;
+          tmp.vec = pad_vec;
+          const int valid = (int)(a.m_size1 - c) * ES;
+          for (int i = 0; i < valid; ++i) tmp.b[i] = ((const uint8_t*)src)[i];
+          v = tmp.vec;
+        }
+      }
+      *(u32x4*)(a.tiled + tiled_chunk_offset<kPow2>(a, r, j)) = v;
+    }
+  }
+}
+
+template <int ES, bool kPow2>
+__global__ __launch_bounds__(kStreamThreads) void unpack_stream_kernel(StreamArgs a) {
+  constexpr int CE = 16 / ES;
+  typedef typename Chunk<ES>::aligned_t dst_vec_t;
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t j0 = (blockIdx.x * 4 + wave) * kBlockChunks;
+  if (j0 >= a.chunks_per_row) return;
+  const uint32_t j = j0 + (lane & 7);
+  const int64_t c = (int64_t)j * CE;
+  const int64_t row_groups = ceil_div(a.m_size0, kBlockRows * kStreamUnroll);
+  const bool cols_inside = (int64_t)(j0 + kBlockChunks) * CE <= a.m_size1;
+  for (int64_t rg = blockIdx.y; rg < row_groups; rg += gridDim.y) {
+    const int64_t r0 = rg * kStreamUnroll * kBlockRows;
+    if (cols_inside && r0 + kStreamUnroll * kBlockRows <= a.m_size0) {
+      u32x4 v[kStreamUnroll];
+#pragma unroll
+      for (int u = 0; u < kStreamUnroll; ++u) {
+        const int64_t r = r0 + u * kBlockRows + (lane >> 3);
+        v[u] = *(const u32x4*)(a.tiled + tiled_chunk_offset<kPow2>(a, r, j));
+      }
+#pragma unroll
+      for (int u = 0; u < kStreamUnroll; ++u) {
+        const int64_t r = r0 + u * kBlockRows + (lane >> 3);
+        *(dst_vec_t*)((char*)a.mat + (r * a.m_stride0 + c) * ES) = v[u];
+      }
+      continue;
+    }
+    if (j >= a.chunks_per_row) continue;
+#pragma unroll 1
+    for (int u = 0; u < kStreamUnroll; ++u) {
+      const int64_t r = r0 + u * kBlockRows + (lane >> 3);
+      if (r >= a.m_size0) continue;
+      const u32x4 v = *(const u32x4*)(a.tiled + tiled_chunk_offset<kPow2>(a, r, j));
+      char* dst = (char*)a.mat + (r * a.m_stride0 + c) * ES;
+      if (c + CE <= a.m_size1) {
+        *(dst_vec_t*)dst = v;
+      } else {
+        union { u32x4 vec; uint8_t b[16]; } tmp;
+        tmp.vec = v;
+        const int valid = (int)(a.m_size1 - c) * ES;
+        for (int i = 0; i < valid; ++i) ((uint8_t*)dst)[i] = tmp.b[i];
+      }
+    }
+  }
+}
+
+// Power-of-two tile geometry (every gfx950 tile shape): the same 8x8 block walk
+// with all 64-bit address arithmetic done once per wave on the scalar unit and
+// only 32-bit offsets per lane. kPack selects the direction.
+struct Pow2Args {
+  const char* mat;
+  char* tiled;
+  int64_t m_size0, m_size1;             // elements
+  int64_t m_pitch_bytes;
+  int64_t t_stride_row_bytes, t_stride_col_bytes;
+  int64_t padded_rows;
+  uint32_t chunks_per_row, padded_chunks_per_row;
+  int log2_tile_rows, log2_cpr;
+  uint64_t padding;
+};
+
+template <int ES, bool kPack>
+__global__ __launch_bounds__(kStreamThreads) void stream_pow2_kernel(Pow2Args a) {
+  constexpr int CE = 16 / ES;
+  constexpr int kRows = kBlockRows * kStreamUnroll;
+  typedef typename Chunk<ES>::aligned_t mat_vec_t;
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t j0 = (blockIdx.x * 4 + wave) * kBlockChunks;
+  const uint32_t col_limit = kPack ? a.padded_chunks_per_row : a.chunks_per_row;
+  if (j0 >= col_limit) return;
+  const int64_t row_limit = kPack ? a.padded_rows : a.m_size0;
+  const int64_t r0 = (int64_t)blockIdx.y * kRows;
+  if (r0 >= row_limit) return;
+  const uint32_t tile_rows = 1u << a.log2_tile_rows, cpr = 1u << a.log2_cpr;
+  const uint32_t jl = lane & 7, rl = lane >> 3;
+  // Scalar bases of this wave's block on both sides.
+  const char* mat_base = a.mat + r0 * a.m_pitch_bytes + (int64_t)j0 * 16;
+  char* tiled_base = a.tiled + (r0 >> a.log2_tile_rows) * a.t_stride_row_bytes +
+                     (int64_t)(j0 >> a.log2_cpr) * a.t_stride_col_bytes;
+  const uint32_t trow0 = (uint32_t)r0 & (tile_rows - 1), h0 = j0 & (cpr - 1);
+  // Per-lane 32-bit offsets.
+  const uint32_t pitch = (uint32_t)a.m_pitch_bytes;
+  const uint32_t srow = (uint32_t)a.t_stride_row_bytes, scol = (uint32_t)a.t_stride_col_bytes;
+  uint32_t mat_off[kStreamUnroll], tiled_off[kStreamUnroll];
+#pragma unroll
+  for (int u = 0; u < kStreamUnroll; ++u) {
+    const uint32_t r = trow0 + u * kBlockRows + rl, j = h0 + jl;
+    mat_off[u] = (u * kBlockRows + rl) * pitch + jl * 16;
+    tiled_off[u] = (r >> a.log2_tile_rows) * srow + (j >> a.log2_cpr) * scol +
+                   (((r & (tile_rows - 1)) << a.log2_cpr) + (j & (cpr - 1))) * 16;
+  }
+  const bool interior = (int64_t)(j0 + kBlockChunks) * CE <= a.m_size1 && r0 + kRows <= a.m_size0;
+  if (interior) {
+    u32x4 v[kStreamUnroll];
+#pragma unroll
+    for (int u = 0; u < kStreamUnroll; ++u)
+      v[u] = kPack ? *(const mat_vec_t*)(mat_base + mat_off[u]) : *(const u32x4*)(tiled_base + tiled_off[u]);
+#pragma unroll
+    for (int u = 0; u < kStreamUnroll; ++u) {
+      if (kPack) *(u32x4*)(tiled_base + tiled_off[u]) = v[u];
+      else *(mat_vec_t*)((char*)mat_base + mat_off[u]) = v[u];
+    }
+    return;
+  }
+  // Edge blocks: per-lane predicates, padding (pack), byte-wise handling of the
+  // chunk that straddles the right edge.
+  if (j0 + jl >= col_limit) return;
+  const int64_t c = (int64_t)(j0 + jl) * CE;
   u32x4 pad_vec;
   {
     uint64_t p = a.padding;
@@ -134,113 +358,111 @@ __global__ __launch_bounds__(kStreamThreads) void pack_stream_kernel(StreamArgs 
     if (ES == 4) { p &= 0xFFFFFFFFull; p |= p << 32; }
     pad_vec = u32x4{(uint32_t)p, (uint32_t)(p >> 32), (uint32_t)p, (uint32_t)(p >> 32)};
   }
-  u32x4 v[kStreamUnroll];
-  char* dst[kStreamUnroll];
-#pragma unroll
+#pragma unroll 1
   for (int u = 0; u < kStreamUnroll; ++u) {
-    dst[u] = nullptr;
-    const int64_t unit = wave * kStreamUnroll + u;
-    if (unit >= a.units) continue;
-    const int64_t panel = unit / runs_per_panel;
-    const int64_t q = (unit - panel * runs_per_panel) * 64 + lane;  // chunk in panel
-    if (q >= chunks_per_panel) continue;
-    const int64_t tile_col = q / chunks_per_tile;
-    const int in_tile = (int)(q - tile_col * chunks_per_tile);
-    const int trow = in_tile / a.cpr, h = in_tile - trow * a.cpr;
-    const int64_t r = panel * a.tile_rows + trow;
-    const int64_t c = tile_col * a.tile_cols + (int64_t)h * CE;
-    dst[u] = a.tiled + (panel * a.t_stride_row + tile_col * a.t_stride_col +
-                        (int64_t)in_tile * CE) * ES;
-    v[u] = pad_vec;
-    if (r < a.m_size0 && c < a.m_size1) {
-      const char* src = a.mat + (r * a.m_stride0 + c) * ES;
-      if (c + CE <= a.m_size1) {
-        v[u] = *(const src_vec_t*)src;
-      } else {
-        // Chunk straddles the right edge: element-wise, never reading past it.
-        union { u32x4 vec; uint8_t b[16]; } tmp;
-        tmp.vec = pad_vec;
-        const int valid = (int)(a.m_size1 - c) * ES;
-        for (int i = 0; i < valid; ++i) tmp.b[i] = ((const uint8_t*)src)[i];
-        v[u] = tmp.vec;
-      }
-    }
-  }
-#pragma unroll
-  for (int u = 0; u < kStreamUnroll; ++u)
-    if (dst[u]) *(u32x4*)dst[u] = v[u];
-}
-
-// unpack: a work unit is 64 consecutive chunks of one matrix row; a wave takes
-// kStreamUnroll consecutive ROWS at the same columns (they sit in the same
-// tiles, hence the same source cache lines).
-template <int ES>
-__global__ __launch_bounds__(kStreamThreads) void unpack_stream_kernel(StreamArgs a) {
-  constexpr int CE = 16 / ES;
-  typedef typename Chunk<ES>::aligned_t dst_vec_t;
-  const int lane = threadIdx.x & 63;
-  const int64_t wave = ((int64_t)blockIdx.x * kStreamThreads + threadIdx.x) >> 6;
-  const int64_t chunks_per_row = ceil_div(a.m_size1, CE);
-  const int64_t runs_per_row = ceil_div(chunks_per_row, 64);
-  const int64_t row_groups = ceil_div(a.m_size0, kStreamUnroll);
-  if (wave >= row_groups * runs_per_row) return;
-  const int64_t rg = wave / runs_per_row;
-  const int64_t j = (wave - rg * runs_per_row) * 64 + lane;  // chunk in row
-  if (j >= chunks_per_row) return;
-  const int64_t c = j * CE;
-  const int64_t tile_col = j / a.cpr;
-  const int h = (int)(j - tile_col * a.cpr);
-  u32x4 v[kStreamUnroll];
-#pragma unroll
-  for (int u = 0; u < kStreamUnroll; ++u) {
-    const int64_t r = rg * kStreamUnroll + u;
-    if (r >= a.m_size0) continue;
-    const int64_t panel = r / a.tile_rows;
-    const int trow = (int)(r - panel * a.tile_rows);
-    const char* src = a.tiled + (panel * a.t_stride_row + tile_col * a.t_stride_col +
-                                 ((int64_t)trow * a.cpr + h) * CE) * ES;
-    v[u] = *(const u32x4*)src;
-  }
-#pragma unroll
-  for (int u = 0; u < kStreamUnroll; ++u) {
-    const int64_t r = rg * kStreamUnroll + u;
-    if (r >= a.m_size0) continue;
-    char* dst = (char*)a.mat + (r * a.m_stride0 + c) * ES;
-    if (c + CE <= a.m_size1) {
-      *(dst_vec_t*)dst = v[u];
+    const int64_t r = r0 + u * kBlockRows + rl;
+    if (r >= row_limit) continue;
+    const bool in_matrix = r < a.m_size0 && c < a.m_size1;
+    const int valid = in_matrix ? (c + CE <= a.m_size1 ? 16 : (int)(a.m_size1 - c) * ES) : 0;
+    union { u32x4 vec; uint8_t b[16]; } tmp;
+    if (kPack) {
+      tmp.vec = pad_vec;
+      if (valid == 16) tmp.vec = *(const mat_vec_t*)(mat_base + mat_off[u]);
+      else for (int i = 0; i < valid; ++i) tmp.b[i] = ((const uint8_t*)(mat_base + mat_off[u]))[i];
+      *(u32x4*)(tiled_base + tiled_off[u]) = tmp.vec;
     } else {
-      union { u32x4 vec; uint8_t b[16]; } tmp;
-      tmp.vec = v[u];
-      const int valid = (int)(a.m_size1 - c) * ES;
-      for (int i = 0; i < valid; ++i) ((uint8_t*)dst)[i] = tmp.b[i];
+      tmp.vec = *(const u32x4*)(tiled_base + tiled_off[u]);
+      if (valid == 16) *(mat_vec_t*)((char*)mat_base + mat_off[u]) = tmp.vec;
+      else for (int i = 0; i < valid; ++i) ((uint8_t*)mat_base + mat_off[u])[i] = tmp.b[i];
     }
   }
 }
 
-bool stream_eligible(int es, int64_t m_stride1, int transpose_inner, int tile_cols,
-                     const void* tiled, int64_t t_stride0, int64_t tile_elems) {
+// The 32-bit per-lane offsets of stream_pow2_kernel must not overflow.
+bool pow2_eligible(const StreamArgs& a, int es) {
+  if (!a.pow2) return false;
+  const int64_t rows = kBlockRows * kStreamUnroll;
+  const int64_t pitch = a.m_stride0 * es;
+  if (pitch * rows + 128 >= (1ll << 31)) return false;
+  const int64_t panels = rows / a.tile_rows + 2, cols = kBlockChunks / a.cpr + 2;
+  if (a.t_stride_row_bytes * panels + a.t_stride_col_bytes * cols + (1ll << 20) >= (1ll << 31)) return false;
+  if ((int64_t)a.tile_rows * a.cpr * 16 >= (1ll << 20)) return false;
+  return ceil_div(a.padded_rows, rows) <= 65535 && ceil_div(a.m_size0, rows) <= 65535;
+}
+
+template <int ES, bool kPack>
+int launch_stream_pow2(const StreamArgs& a, hipStream_t s) {
+  Pow2Args p;
+  p.mat = a.mat; p.tiled = a.tiled;
+  p.m_size0 = a.m_size0; p.m_size1 = a.m_size1; p.m_pitch_bytes = a.m_stride0 * ES;
+  p.t_stride_row_bytes = a.t_stride_row_bytes; p.t_stride_col_bytes = a.t_stride_col_bytes;
+  p.padded_rows = a.padded_rows;
+  p.chunks_per_row = a.chunks_per_row; p.padded_chunks_per_row = a.padded_chunks_per_row;
+  p.log2_tile_rows = a.log2_tile_rows; p.log2_cpr = a.log2_cpr;
+  p.padding = a.padding;
+  const int64_t cols = kPack ? a.padded_chunks_per_row : a.chunks_per_row;
+  const int64_t rows = kPack ? a.padded_rows : a.m_size0;
+  const int64_t bx = ceil_div(cols, 4 * kBlockChunks);
+  const int64_t by = ceil_div(rows, kBlockRows * kStreamUnroll);
+  if (bx > 0x7FFFFFFF || by > 65535 || bx < 1 || by < 1) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  hipLaunchKernelGGL((stream_pow2_kernel<ES, kPack>), dim3((unsigned)bx, (unsigned)by), dim3(kStreamThreads), 0, s, p);
+  return check_hip(hipGetLastError(), "stream_pow2 launch");
+}
+
+bool stream_eligible(int es, int64_t m_stride1, int transpose_inner, int64_t tile_rows,
+                     int64_t tile_cols, int64_t outer_cols, int64_t m_size1, const void* tiled,
+                     int64_t t_stride0, int64_t tile_elems) {
   const int ce = 16 / es;
-  return m_stride1 == 1 && !transpose_inner && tile_cols > 0 && tile_cols % ce == 0 &&
-         ((uintptr_t)tiled % 16) == 0 && (t_stride0 * es) % 16 == 0 &&
-         (tile_elems * es) % 16 == 0;
+  if (!(m_stride1 == 1 && !transpose_inner && tile_cols > 0 && tile_cols % ce == 0 &&
+        ((uintptr_t)tiled % 16) == 0 && (t_stride0 * es) % 16 == 0 && (tile_elems * es) % 16 == 0))
+    return false;
+  // 32-bit per-lane column arithmetic: chunks per row must stay below 2^31.
+  return tile_rows < (1ll << 31) && outer_cols * (tile_cols / ce) < (1ll << 31) &&
+         m_size1 / ce + 1 < (1ll << 31);
+}
+
+void fill_stream_geometry(StreamArgs* a, int es) {
+  const int ce = 16 / es;
+  a->cpr = a->tile_cols / ce;
+  a->chunks_per_row = (uint32_t)((a->m_size1 + ce - 1) / ce);
+  a->padded_chunks_per_row = (uint32_t)(a->outer_cols * a->cpr);
+  a->padded_rows = a->outer_rows * a->tile_rows;
+  a->t_stride_row_bytes = a->t_stride_row * es;
+  a->t_stride_col_bytes = a->t_stride_col * es;
+  a->by_cpr = make_fastdiv((uint32_t)a->cpr);
+  a->by_tile_rows = make_fastdiv((uint32_t)a->tile_rows);
+  auto is_pow2 = [](int v) { return v > 0 && (v & (v - 1)) == 0; };
+  a->pow2 = is_pow2(a->tile_rows) && is_pow2(a->cpr);
+  a->log2_tile_rows = a->log2_cpr = 0;
+  while ((1 << a->log2_tile_rows) < a->tile_rows) ++a->log2_tile_rows;
+  while ((1 << a->log2_cpr) < a->cpr) ++a->log2_cpr;
 }
 
 template <int ES>
 int launch_pack_stream(const StreamArgs& a, hipStream_t s) {
-  const int64_t waves = ceil_div(a.units, kStreamUnroll);
-  const int64_t blocks = ceil_div(waves, kStreamThreads / 64);
-  if (blocks > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
-  hipLaunchKernelGGL(pack_stream_kernel<ES>, dim3((unsigned)blocks), dim3(kStreamThreads), 0, s, a);
+  if (pow2_eligible(a, ES)) return launch_stream_pow2<ES, true>(a, s);
+  const int64_t bx = ceil_div(a.padded_chunks_per_row, 4 * kBlockChunks);
+  const int64_t row_groups = ceil_div(a.padded_rows, kBlockRows * kStreamUnroll);
+  const int64_t by = row_groups < 65535 ? row_groups : 65535;
+  if (bx > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  if (a.pow2)
+    hipLaunchKernelGGL((pack_stream_kernel<ES, true>), dim3((unsigned)bx, (unsigned)by), dim3(kStreamThreads), 0, s, a);
+  else
+    hipLaunchKernelGGL((pack_stream_kernel<ES, false>), dim3((unsigned)bx, (unsigned)by), dim3(kStreamThreads), 0, s, a);
   return check_hip(hipGetLastError(), "pack_stream launch");
 }
 
 template <int ES>
 int launch_unpack_stream(const StreamArgs& a, hipStream_t s) {
-  constexpr int CE = 16 / ES;
-  const int64_t waves = ceil_div(a.m_size0, kStreamUnroll) * ceil_div(ceil_div(a.m_size1, CE), 64);
-  const int64_t blocks = ceil_div(waves, kStreamThreads / 64);
-  if (blocks > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
-  hipLaunchKernelGGL(unpack_stream_kernel<ES>, dim3((unsigned)blocks), dim3(kStreamThreads), 0, s, a);
+  if (pow2_eligible(a, ES)) return launch_stream_pow2<ES, false>(a, s);
+  const int64_t bx = ceil_div(a.chunks_per_row, 4 * kBlockChunks);
+  const int64_t row_groups = ceil_div(a.m_size0, kBlockRows * kStreamUnroll);
+  const int64_t by = row_groups < 65535 ? row_groups : 65535;
+  if (bx > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  if (a.pow2)
+    hipLaunchKernelGGL((unpack_stream_kernel<ES, true>), dim3((unsigned)bx, (unsigned)by), dim3(kStreamThreads), 0, s, a);
+  else
+    hipLaunchKernelGGL((unpack_stream_kernel<ES, false>), dim3((unsigned)bx, (unsigned)by), dim3(kStreamThreads), 0, s, a);
   return check_hip(hipGetLastError(), "unpack_stream launch");
 }
 
@@ -266,7 +488,8 @@ int launch_pack(const iree_amd_uk_pack_params_t& p, hipStream_t s) {
   if (p.out_size2 > 0x7FFFFFFF || p.out_size3 > 0x7FFFFFFF || tile_elems > 0x7FFFFFFF)
     return fail(IREE_AMD_UK_STATUS_OUT_OF_RANGE, "pack: tile larger than 2^31 elements");
 
-  if (stream_eligible(es, p.in_stride1, ti, (int)p.out_size3, out, p.out_stride0, tile_elems)) {
+  if (stream_eligible(es, p.in_stride1, ti, p.out_size2, p.out_size3, to ? p.out_size0 : p.out_size1,
+                      p.in_size1, out, p.out_stride0, tile_elems)) {
     StreamArgs a;
     a.mat = in; a.tiled = out;
     a.m_size0 = p.in_size0; a.m_size1 = p.in_size1; a.m_stride0 = p.in_stride0;
@@ -275,10 +498,8 @@ int launch_pack(const iree_amd_uk_pack_params_t& p, hipStream_t s) {
     a.t_stride_row = to ? tile_elems : p.out_stride0;
     a.t_stride_col = to ? p.out_stride0 : tile_elems;
     a.tile_rows = (int)p.out_size2; a.tile_cols = (int)p.out_size3;
-    a.cpr = a.tile_cols / (16 / es);
     a.padding = p.padding_value;
-    const int64_t chunks_per_panel = a.outer_cols * (int64_t)a.tile_rows * a.cpr;
-    a.units = a.outer_rows * ceil_div(chunks_per_panel, 64);
+    fill_stream_geometry(&a, es);
     // With swapped outer dimensions consecutive tile columns are t_stride0
     // apart; the 1 KiB runs then only stay contiguous inside one tile, which
     // is still a whole number of chunks.
@@ -314,7 +535,8 @@ int launch_unpack(const iree_amd_uk_unpack_params_t& p, hipStream_t s) {
     return fail(IREE_AMD_UK_STATUS_OUT_OF_RANGE, "unpack: tile larger than 2^31 elements");
   if (tile_elems == 0) return 0;  // validated: then out sizes are 0 too
 
-  if (stream_eligible(es, p.out_stride1, ti, (int)p.in_size3, tiled, p.in_stride0, tile_elems)) {
+  if (stream_eligible(es, p.out_stride1, ti, p.in_size2, p.in_size3, to ? p.in_size0 : p.in_size1,
+                      p.out_size1, tiled, p.in_stride0, tile_elems)) {
     StreamArgs a;
     a.mat = mat; a.tiled = (char*)tiled;
     a.m_size0 = p.out_size0; a.m_size1 = p.out_size1; a.m_stride0 = p.out_stride0;
@@ -323,8 +545,8 @@ int launch_unpack(const iree_amd_uk_unpack_params_t& p, hipStream_t s) {
     a.t_stride_row = to ? tile_elems : p.in_stride0;
     a.t_stride_col = to ? p.in_stride0 : tile_elems;
     a.tile_rows = (int)p.in_size2; a.tile_cols = (int)p.in_size3;
-    a.cpr = a.tile_cols / (16 / es);
-    a.padding = 0; a.units = 0;
+    a.padding = 0;
+    fill_stream_geometry(&a, es);
     int st = es == 2 ? launch_unpack_stream<2>(a, s) : launch_unpack_stream<4>(a, s);
     if (st != IREE_AMD_UK_STATUS_NOT_FOUND) return st;
   }
