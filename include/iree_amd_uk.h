@@ -321,12 +321,31 @@ IREE_AMD_UK_EXPORT int iree_amd_uk_query_tile_sizes_2d(
  *===------------------------------------------------------------------------===*/
 #define IREE_AMD_UK_FLAG_DEQUANT_MATMUL_ZP_F16 0x0
 #define IREE_AMD_UK_FLAG_DEQUANT_MATMUL_ZP_U4 0x1
+/* Weights are in the pre-tiled layout that iree_amd_uk_pack_i4_weights
+ * produces: tiles of 32 columns (n) x 128 k, 2 KiB each, ordered
+ * [N/32][K/128]; inside a tile column c owns bytes [64c, 64c+64), in which the
+ * 16 dwords of the row-major span (8 nibbles each, even k in the low nibble)
+ * are transposed as a 4 x 4 matrix: dword q of 16-byte chunk j holds
+ * k = 32q + 8j .. 32q + 8j + 7. A 64-lane wave then reads 1 KiB of contiguous
+ * memory per load and every lane's four dwords feed four consecutive MFMAs.
+ * Needs N % 32 == 0 and K % 128 == 0. Without the flag the weights are
+ * row-major [N][K/2]; groups smaller than 128 are fast only from tiled weights. */
+#define IREE_AMD_UK_FLAG_DEQUANT_MATMUL_W_TILED 0x2
 
 IREE_AMD_UK_EXPORT int iree_amd_uk_dequant_matmul_i4(
     const void* x_buffer, const void* w_buffer, const void* scale_buffer,
     const void* zp_buffer, void* out_buffer, iree_amd_uk_index_t M,
     iree_amd_uk_index_t N, iree_amd_uk_index_t K,
     iree_amd_uk_index_t group_size, uint32_t flags, void* stream);
+
+/* Row-major [N][K/2] 4-bit weights -> the ..._W_TILED layout above (done once
+ * per weight matrix, like the reference's pack of a constant right-hand side
+ * at compile time, REF compiler/src/iree/compiler/GlobalOptimization/
+ * MaterializeHomogeneousEncodings.cpp). N % 32 == 0, K % 128 == 0; src and dst
+ * must not overlap. */
+IREE_AMD_UK_EXPORT int iree_amd_uk_pack_i4_weights(
+    const void* w_rowmajor, void* w_tiled, iree_amd_uk_index_t N,
+    iree_amd_uk_index_t K, void* stream);
 
 /*===------------------------------------------------------------------------===
  * Pieces of the fp8 Llama-style MLP block (no reference ukernel; the pattern is

@@ -15,6 +15,7 @@ from .ukernel import (  # noqa: F401
     mmt4d,
     mmt4d_info,
     pack,
+    pack_i4_weights,
     quantize_f16_to_f8e4m3,
     query_tile_sizes_2d,
     silu_mul_quantize,

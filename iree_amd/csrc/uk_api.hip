@@ -354,7 +354,7 @@ extern "C" int iree_amd_uk_dequant_matmul_i4(
     const void* zp_buffer, void* out_buffer, iree_amd_uk_index_t M,
     iree_amd_uk_index_t N, iree_amd_uk_index_t K,
     iree_amd_uk_index_t group_size, uint32_t flags, void* stream) {
-  if (flags & ~1u) return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "dequant_matmul_i4: unknown flag bits");
+  if (flags & ~3u) return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "dequant_matmul_i4: unknown flag bits");
   if (M < 0 || N < 0 || K < 0 || group_size <= 0)
     return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "dequant_matmul_i4: bad sizes");
   if (K % group_size || group_size % 32)
@@ -366,6 +366,20 @@ extern "C" int iree_amd_uk_dequant_matmul_i4(
   return launch_dequant_matmul_i4(x_buffer, w_buffer, scale_buffer, zp_buffer,
                                   out_buffer, M, N, K, group_size, flags,
                                   (hipStream_t)stream);
+}
+
+extern "C" int iree_amd_uk_pack_i4_weights(const void* w_rowmajor, void* w_tiled,
+                                           iree_amd_uk_index_t N, iree_amd_uk_index_t K,
+                                           void* stream) {
+  if (N < 0 || K < 0 || N % 32 || K % 128)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT,
+                "pack_i4_weights: need N %% 32 == 0 and K %% 128 == 0");
+  if (N == 0 || K == 0) return 0;
+  if (!w_rowmajor || !w_tiled)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "pack_i4_weights: null buffer");
+  if (((uintptr_t)w_rowmajor | (uintptr_t)w_tiled) % 4)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "pack_i4_weights: buffers must be 4-byte aligned");
+  return launch_pack_i4_weights(w_rowmajor, w_tiled, N, K, (hipStream_t)stream);
 }
 
 extern "C" int iree_amd_uk_quantize_f16_to_f8e4m3(const void* in_f16,

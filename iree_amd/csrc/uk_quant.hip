@@ -1,10 +1,452 @@
-// Placeholder translation unit: int4 dequant-matmul and fp8 helpers.
+// Grouped int4-weight dequantising matmul and the fp8 element-wise helpers.
+//
+//   out[m][n] = sum_g s[n][g] * sum_{k in g} x[m][k] * (w[n][k] - zp[n][g])
+//
+// (the fused dequantisation + matmul pattern of the reference's
+// compiler/src/iree/compiler/GlobalOptimization/FuseDequantizationMatmul.cpp:53-159;
+// f32 accumulation, one rounding to f16 at the end).
+//
+// Decode-shaped calls (a few rows of activations) are bound by the HBM stream of
+// the weights, 0.5 byte per weight, and the whole stream is only tens of
+// megabytes: the kernel is as much latency- as bandwidth-bound. The fast kernel
+// therefore:
+//   * reads each weight byte exactly once, 16 bytes per lane per load, through
+//     buffer loads that always have a whole tile of requests in flight: the
+//     request for slab i of the next tile is issued the moment slab i of the
+//     current tile has been consumed, and nothing in the loop waits for a load
+//     it has just issued (group parameters travel as raw bits and are only
+//     decoded when the weights that follow them in the queue have landed);
+//   * keeps the activations stationary in REGISTERS: the 8 waves of a
+//     workgroup each own one eighth of K and hold their slice of x as MFMA A
+//     operands for the whole kernel, so no LDS or cache bandwidth is spent on
+//     re-reading x (which would be 4 bytes per weight byte);
+//   * dequantises in registers ahead of the MFMA: a nibble n becomes the f16
+//     value 1024+n (or 1024+16n for the upper nibble of a byte, no shift
+//     needed) by OR-ing it into the mantissa of 0x6400, the offset and the zero
+//     point are removed with exact packed-f16 arithmetic, the small integers
+//     go through v_mfma_f32_16x16x32_f16 (products are exact), and the
+//     per-group f32 partial sums are scaled by s[n][g] with one f32 FMA per
+//     accumulator register (the lane owns column n, so the scale is a
+//     per-lane scalar);
+//   * sums the 8 K-slices through LDS in a fixed order (deterministic).
 #include "uk_common.h"
+
+#include <hip/hip_fp16.h>
+
 namespace uk {
-int launch_dequant_matmul_i4(const void*, const void*, const void*, const void*, void*, int64_t,
-                             int64_t, int64_t, int64_t, uint32_t, hipStream_t) {
-  return fail(IREE_AMD_UK_STATUS_UNIMPLEMENTED, "dequant_matmul_i4: not built yet");
+namespace {
+
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kWaves = 8;               // K-slices per workgroup
+constexpr int kThreads = kWaves * 64;
+
+struct I4Args {
+  const uint16_t* x;      // [M][K] f16
+  const uint8_t* w;       // u4, tiled or row-major
+  const uint16_t* scale;  // [N][G] f16
+  const void* zp;         // [N][G] f16 or packed u4
+  uint16_t* out;          // [M][N] f16
+  int M, N, K, G;
+  int log2_gs;            // group size = 1 << log2_gs
+  int zp_u4;
+  int tiled;
+  int n_tiles;            // ceil(N / 32)
+  int m_base;             // first activation row of this pass
+  // weight addressing of the fast kernel: byte offset of the 16 bytes that
+  // lane (nl, kc) reads for column c of tile nt in 128-k span s is
+  //   nt * K * 16 + s * span_stride + c * col_stride + kc * 16
+  uint32_t span_stride, col_stride;
+  uint32_t w_bytes;       // size of the weight buffer
+};
+
+// Position, in the tiled layout, of the byte that holds elements (n, k) and
+// (n, k+1), k even. A tile is 32 columns by 128 k (2 KiB): 64 bytes per column,
+// in which the 16 dwords of the row-major span are transposed as a 4 x 4
+// matrix, so that 16-byte chunk kc holds, as dword q, k = q*32 + kc*8 .. +8.
+__host__ __device__ inline size_t tiled_byte_index(int64_t n, int64_t k, int64_t K) {
+  const int64_t s = k >> 7, r = k & 127, q = r >> 5, kc = (r >> 3) & 3, j = r & 7;
+  return (size_t)((((n >> 5) * (K >> 7) + s) * 32 + (n & 31)) * 64 + kc * 16 + q * 4 + (j >> 1));
 }
+
+// 8 nibbles of one dword -> 8 small f16 integers (nibble - zero point), in the
+// k order [0,4,1,5,2,6,3,7] of the dword's nibbles (pairs (i, i+4) fall out of
+// one AND/OR); the activation operand is permuted the same way. `lo` is
+// 1024 + zp and `hi` 64 + zp as packed f16 pairs: 0x6400 | n is 1024 + n and
+// 0x6400 | (n << 4) is 1024 + 16 n, so (1024 + n) - lo and
+// (1024 + 16 n) / 16 - hi are both n - zp, every step exact for integer zp.
+__device__ __forceinline__ half8 dequant_dword(uint32_t w, half2v lo, half2v hi) {
+  union { uint32_t u; half2v h; } a, b, c, d;
+  const uint32_t w8 = w >> 8;
+  a.u = (w & 0x000F000Fu) | 0x64006400u;    // nibbles 0, 4
+  b.u = (w & 0x00F000F0u) | 0x64006400u;    // nibbles 1, 5 (x16)
+  c.u = (w8 & 0x000F000Fu) | 0x64006400u;   // nibbles 2, 6
+  d.u = (w8 & 0x00F000F0u) | 0x64006400u;   // nibbles 3, 7 (x16)
+  const half2v sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
+  const half2v r0 = a.h - lo, r1 = b.h * sixteenth - hi, r2 = c.h - lo, r3 = d.h * sixteenth - hi;
+  return half8{r0.x, r0.y, r1.x, r1.y, r2.x, r2.y, r3.x, r3.y};
+}
+
+// x[m][k .. k+8) (8 consecutive halves, 16 bytes) -> the same 8 halves in the
+// order [0,4,1,5,2,6,3,7].
+__device__ __forceinline__ half8 permute_x(u32x4 v) {
+  union { uint32_t u[4]; half8 h; } r;
+  // v.x = (h0,h1) v.y = (h2,h3) v.z = (h4,h5) v.w = (h6,h7)
+  r.u[0] = __builtin_amdgcn_perm(v.z, v.x, 0x05040100);  // (h0, h4)
+  r.u[1] = __builtin_amdgcn_perm(v.z, v.x, 0x07060302);  // (h1, h5)
+  r.u[2] = __builtin_amdgcn_perm(v.w, v.y, 0x05040100);  // (h2, h6)
+  r.u[3] = __builtin_amdgcn_perm(v.w, v.y, 0x07060302);  // (h3, h7)
+  return r.h;
+}
+
+// NB bytes (1 .. 16 naturally aligned, 32 aligned to 16) into NB/4 (at least 1) dwords.
+template <int NB>
+__device__ __forceinline__ void load_bits(const void* p, uint32_t* dst) {
+  if constexpr (NB == 1) dst[0] = *(const uint8_t*)p;
+  else if constexpr (NB == 2) dst[0] = *(const uint16_t*)p;
+  else if constexpr (NB == 4) dst[0] = *(const uint32_t*)p;
+  else if constexpr (NB == 8) { const u32x2 v = *(const u32x2*)p; dst[0] = v.x; dst[1] = v.y; }
+  else if constexpr (NB == 16) { const u32x4 v = *(const u32x4*)p; dst[0] = v.x; dst[1] = v.y; dst[2] = v.z; dst[3] = v.w; }
+  else { static_assert(NB == 32, "unsupported width"); load_bits<16>(p, dst); load_bits<16>((const uint8_t*)p + 16, dst + 4); }
+}
+
+// Work decomposition. A tile is 32 columns (n) of the output. Wave w of the
+// workgroup owns k in [w*KB*64, (w+1)*KB*64), walked in KB/2 spans of 128: in
+// one span lane (nl = l % 16, kc = l / 16) loads, for each half h of the
+// tile's columns, 16 bytes of column h*16+nl, so that one wave load
+// instruction moves a 16-column x 128-k slab (1 KiB, contiguous in the tiled
+// layout). Its 4 dwords feed 4 MFMAs 16x16x32 (A = x rows m, B = weight
+// columns n). Which k a dword holds depends on the layout: chunk (8 k) number
+// q*4 + kc of the span in the tiled layout, kc*4 + q in the row-major one; the
+// activation fragments are loaded to match (a.tiled), which in the tiled case
+// makes each wave load of x cover 64 contiguous bytes of 16 rows.
+//   MH       16-row halves of activations held (1: M <= 16, 2: M <= 32)
+//   kZpU4    zero points are packed uint4 (else f16)
+//   kLog2Gs  log2 of the group size, 5..8, or 9 for "at least the wave's K
+//            slice" (one group per wave and tile). A group never straddles
+//            MFMAs in the tiled layout (MFMA q covers k = q*32 .. +32 of the
+//            span); in the row-major one that only holds for groups of 128
+//            and more, so smaller groups are served from tiled weights only.
+template <int KB, int MH, bool kZpU4, int kLog2Gs>
+__global__ __launch_bounds__(kThreads) void dequant_matmul_i4_kernel(I4Args a) {
+  constexpr int SP = KB / 2;                 // spans of 128 k per wave
+  constexpr int L = kLog2Gs >= 9 ? 30 : kLog2Gs;
+  constexpr int GW = ((KB * 64) >> L) > 0 ? ((KB * 64) >> L) : 1;   // groups per wave slice
+  constexpr int SB = GW * 2;                 // bytes of scales per lane, tile and half
+  constexpr int ZB = kZpU4 ? (GW >= 2 ? GW / 2 : 1) : GW * 2;
+  constexpr int SW = (SB + 3) / 4, ZW = (ZB + 3) / 4;
+  __shared__ float partial[2][kWaves][2 * MH * 4][64];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int nl = lane & 15, kc = lane >> 4;
+  const int k_slice = wave * KB * 64;
+  const int g_first = k_slice >> a.log2_gs;  // first group of this wave's slice
+  const uint32_t tile_bytes = (uint32_t)a.K * 16;
+  const uint32_t voff = nl * a.col_stride + kc * 16;
+  const uint32_t soff_wave = wave * SP * a.span_stride;
+  const uint32_t half_stride = 16 * a.col_stride;
+
+  // Raw group parameters of this lane's two columns for the wave's K slice
+  // (zsh: position of a lone packed zero point inside its byte).
+  struct Meta { uint32_t s[2][SW], z[2][ZW], zsh[2]; };
+  auto load_meta = [&](int nt, Meta& m) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      int n = nt * 32 + h * 16 + nl;
+      n = n < a.N ? n : a.N - 1;
+      const size_t sg = (size_t)n * a.G + g_first;
+      load_bits<SB>(a.scale + sg, m.s[h]);
+      if (kZpU4) load_bits<ZB>((const uint8_t*)a.zp + (sg >> 1), m.z[h]);
+      else load_bits<ZB>((const uint16_t*)a.zp + sg, m.z[h]);
+      m.zsh[h] = (kZpU4 && GW == 1) ? (uint32_t)(sg & 1) * 4 : 0;
+    }
+  };
+  // Weights of one tile: loads past the end of the buffer (a tile after the
+  // last one, columns past N) return zeros without touching memory.
+  auto tile_rsrc = [&](int nt) {
+    const uint32_t off = (uint32_t)nt * tile_bytes;   // the host checked that this fits
+    const uint32_t left = nt < a.n_tiles ? a.w_bytes - off : 0;
+    return __builtin_amdgcn_make_buffer_rsrc((void*)(a.w + off), 0, left, 0x00020000);
+  };
+  auto load_slab = [&](__amdgpu_buffer_rsrc_t rsrc, int sp, int h) -> u32x4 {
+    return __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, soff_wave + sp * a.span_stride + h * half_stride, 0);
+  };
+
+  // ---- request the first tile's parameters and weights, then x -------------
+  int nt = blockIdx.x;
+  Meta meta_next;
+  u32x4 wreg[SP][2];
+  load_meta(nt < a.n_tiles ? nt : a.n_tiles - 1, meta_next);
+  {
+    const __amdgpu_buffer_rsrc_t rsrc = tile_rsrc(nt);
+#pragma unroll
+    for (int sp = 0; sp < SP; ++sp)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) wreg[sp][h] = load_slab(rsrc, sp, h);
+  }
+  __builtin_amdgcn_sched_barrier(0);   // keep the weight requests ahead of the x loads
+  // activations: rows m_base + mh*16 + nl, this wave's K slice, permuted; rows
+  // past M are read from the last row and zeroed.
+  half8 xf[MH][SP][4];
+  {
+    const int cq = a.tiled ? 32 : 8, ckc = a.tiled ? 8 : 32;   // chunk strides in k
+#pragma unroll
+    for (int mh = 0; mh < MH; ++mh) {
+      const int m = a.m_base + mh * 16 + nl;
+      const uint32_t keep = m < a.M ? 0xFFFFFFFFu : 0u;
+      const int mr = m < a.M ? m : a.M - 1;
+      const uint16_t* row = a.x + (size_t)mr * a.K + k_slice + kc * ckc;
+#pragma unroll
+      for (int sp = 0; sp < SP; ++sp)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          u32x4 v = *(const u32x4*)(row + sp * 128 + q * cq);
+          v.x &= keep; v.y &= keep; v.z &= keep; v.w &= keep;
+          xf[mh][sp][q] = permute_x(v);
+        }
+    }
+  }
+
+  int parity = 0;
+  for (; nt < a.n_tiles; nt += gridDim.x, parity ^= 1) {
+    const int next = nt + gridDim.x;
+    const Meta mt = meta_next;
+    load_meta(next < a.n_tiles ? next : a.n_tiles - 1, meta_next);
+    const __amdgpu_buffer_rsrc_t rsrc_next = tile_rsrc(next < a.n_tiles ? next : a.n_tiles);
+    __builtin_amdgcn_sched_barrier(0);
+    floatx4 acc[2][MH], part[2][MH];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int mh = 0; mh < MH; ++mh) acc[h][mh] = part[h][mh] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int sp = 0; sp < SP; ++sp) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const u32x4 wv = wreg[sp][h];
+        float sc = 0.f;
+        union { uint32_t u; half2v h; } lo, hi, zf;
+        lo.u = hi.u = zf.u = 0;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int k_lo = sp * 128 + q * 32;                 // within the wave's slice
+          const int g = k_lo >> L;
+          const bool group_start = kLog2Gs >= 9 ? k_lo == 0 : (k_lo & ((1 << L) - 1)) == 0;
+          const bool group_end = kLog2Gs >= 9 ? k_lo + 32 == KB * 64 : ((k_lo + 32) & ((1 << L) - 1)) == 0;
+          if (group_start || q == 0) {
+            // decode the group's parameters
+            const uint32_t sbits = (mt.s[h][g >> 1] >> ((g & 1) * 16)) & 0xFFFF;
+            sc = __half2float(__ushort_as_half((uint16_t)sbits));
+            // Packed uint4 zero points fold into the offsets (1024 + zp and
+            // 64 + zp are exact). f16 zero points may carry a fraction, which
+            // such a sum would round away: they are subtracted in a second step.
+            if (kZpU4) {
+              const uint32_t zb = (mt.z[h][g >> 3] >> ((g & 7) * 4 + mt.zsh[h])) & 0xF;
+              lo.u = 0x64006400u | zb | (zb << 16);
+              const _Float16 c = (_Float16)(float)(64 + zb);
+              hi.h = half2v{c, c};
+            } else {
+              const uint32_t zb = (mt.z[h][g >> 1] >> ((g & 1) * 16)) & 0xFFFF;
+              lo.u = 0x64006400u;
+              hi.h = half2v{(_Float16)64.0f, (_Float16)64.0f};
+              zf.u = zb | (zb << 16);
+            }
+          }
+          if (group_start) {
+#pragma unroll
+            for (int mh = 0; mh < MH; ++mh) part[h][mh] = floatx4{0.f, 0.f, 0.f, 0.f};
+          }
+          half8 wq = dequant_dword(wv[q], lo.h, hi.h);
+          if (!kZpU4) {
+            const half8 zsub2 = {zf.h.x, zf.h.x, zf.h.x, zf.h.x, zf.h.x, zf.h.x, zf.h.x, zf.h.x};
+            wq = wq - zsub2;
+          }
+#pragma unroll
+          for (int mh = 0; mh < MH; ++mh)
+            part[h][mh] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xf[mh][sp][q], wq, part[h][mh], 0, 0, 0);
+          if (group_end) {
+#pragma unroll
+            for (int mh = 0; mh < MH; ++mh)
+#pragma unroll
+              for (int r = 0; r < 4; ++r) acc[h][mh][r] = __builtin_fmaf(part[h][mh][r], sc, acc[h][mh][r]);
+          }
+        }
+        // The slab's registers are free: request the same slab of the next
+        // tile. The fences keep the requests in slab order, which is what
+        // makes every wait in the loop a wait for the OLDEST outstanding load.
+        __builtin_amdgcn_sched_barrier(0);
+        wreg[sp][h] = load_slab(rsrc_next, sp, h);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    // ---- sum the 8 K-slices in wave order and store ----------------------
+    float (*buf)[2 * MH * 4][64] = partial[parity];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int mh = 0; mh < MH; ++mh)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) buf[wave][(h * MH + mh) * 4 + r][lane] = acc[h][mh][r];
+    __syncthreads();
+#pragma unroll
+    for (int rep = 0; rep < MH; ++rep) {
+      const int flat = rep * kThreads + threadIdx.x;     // (h*MH + mh)*256 + r*64 + lane
+      const int l = flat & 63, slot = flat >> 6;         // slot = (h*MH + mh)*4 + r
+      float sum = 0.f;
+#pragma unroll
+      for (int w = 0; w < kWaves; ++w) sum += buf[w][slot][l];
+      const int r = slot & 3, hm = slot >> 2, h = hm / MH, mh = hm % MH;
+      const int m = a.m_base + mh * 16 + 4 * (l >> 4) + r;
+      const int n = nt * 32 + h * 16 + (l & 15);
+      if (m < a.M && n < a.N) a.out[(size_t)m * a.N + n] = __half_as_ushort(__float2half_rn(sum));
+    }
+    // The other half of `partial` is used by the next tile; this half is
+    // rewritten only two tiles later, after the next tile's barrier.
+  }
+}
+
+// Row-major [N][K/2] bytes -> the tiled layout (one thread per dword).
+__global__ __launch_bounds__(256) void pack_i4_weights_kernel(const uint32_t* src, uint32_t* dst,
+                                                              int64_t N, int64_t K) {
+  const int64_t total = N * K / 8;
+  for (int64_t d = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; d < total;
+       d += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t q = d & 3, kc = (d >> 2) & 3, c = (d >> 4) & 31, rest = d >> 9;
+    const int64_t spans = K >> 7, s = rest % spans, nt = rest / spans;
+    dst[d] = src[((nt * 32 + c) * K + s * 128 + q * 32 + kc * 8) >> 3];
+  }
+}
+
+// Reference-order fallback for every shape the MFMA kernel does not serve: one
+// thread per output element.
+__global__ __launch_bounds__(256) void dequant_matmul_i4_generic_kernel(I4Args a, int gs) {
+  const int64_t total = (int64_t)a.M * a.N;
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (int64_t)gridDim.x * blockDim.x) {
+    const int m = (int)(idx / a.N), n = (int)(idx - (int64_t)m * a.N);
+    float acc = 0.f;
+    for (int g = 0; g < a.G; ++g) {
+      const size_t sg = (size_t)n * a.G + g;
+      float zpv;
+      if (a.zp_u4) {
+        const uint8_t byte = ((const uint8_t*)a.zp)[sg >> 1];
+        zpv = (float)((sg & 1) ? (byte >> 4) : (byte & 0xF));
+      } else {
+        zpv = __half2float(__ushort_as_half(((const uint16_t*)a.zp)[sg]));
+      }
+      const float sc = __half2float(__ushort_as_half(a.scale[sg]));
+      float part = 0.f;
+      for (int kk = 0; kk < gs; ++kk) {
+        const int k = g * gs + kk;
+        const uint8_t byte = a.w[a.tiled ? tiled_byte_index(n, k, a.K) : ((size_t)n * a.K + k) >> 1];
+        const float q = (float)((k & 1) ? (byte >> 4) : (byte & 0xF));
+        part = __builtin_fmaf(__half2float(__ushort_as_half(a.x[(size_t)m * a.K + k])), q - zpv, part);
+      }
+      acc = __builtin_fmaf(part, sc, acc);
+    }
+    a.out[idx] = __half_as_ushort(__float2half_rn(acc));
+  }
+}
+
+template <int KB, int MH, bool kZpU4>
+void launch_one(const I4Args& a, int blocks, hipStream_t s) {
+  const dim3 g(blocks), b(kThreads);
+  switch (a.log2_gs) {
+    case 5: hipLaunchKernelGGL((dequant_matmul_i4_kernel<KB, MH, kZpU4, 5>), g, b, 0, s, a); break;
+    case 6: hipLaunchKernelGGL((dequant_matmul_i4_kernel<KB, MH, kZpU4, 6>), g, b, 0, s, a); break;
+    case 7: hipLaunchKernelGGL((dequant_matmul_i4_kernel<KB, MH, kZpU4, 7>), g, b, 0, s, a); break;
+    case 8: hipLaunchKernelGGL((dequant_matmul_i4_kernel<KB, MH, kZpU4, 8>), g, b, 0, s, a); break;
+    default: hipLaunchKernelGGL((dequant_matmul_i4_kernel<KB, MH, kZpU4, 9>), g, b, 0, s, a); break;
+  }
+}
+
+template <int KB>
+int launch_fast(I4Args a, hipStream_t s) {
+  const int cus = device_cu_count();
+  const int blocks = a.n_tiles < cus ? a.n_tiles : cus;
+  int m_base = 0;
+  while (m_base < a.M) {
+    a.m_base = m_base;
+    if (a.M - m_base > 16) {
+      if (a.zp_u4) launch_one<KB, 2, true>(a, blocks, s); else launch_one<KB, 2, false>(a, blocks, s);
+      m_base += 32;
+    } else {
+      if (a.zp_u4) launch_one<KB, 1, true>(a, blocks, s); else launch_one<KB, 1, false>(a, blocks, s);
+      m_base += 16;
+    }
+    UK_RETURN_IF_HIP(hipGetLastError());
+  }
+  return 0;
+}
+
+}  // namespace
+
+int launch_dequant_matmul_i4(const void* x, const void* w, const void* scale, const void* zp,
+                             void* out, int64_t M, int64_t N, int64_t K, int64_t group_size,
+                             uint32_t flags, hipStream_t s) {
+  if (M > 0x7FFFFFFF || N > 0x7FFFFFFF || K > 0x7FFFFFFF)
+    return fail(IREE_AMD_UK_STATUS_OUT_OF_RANGE, "dequant_matmul_i4: sizes beyond 2^31");
+  const bool tiled = (flags & IREE_AMD_UK_FLAG_DEQUANT_MATMUL_W_TILED) != 0;
+  if (tiled && (N % 32 || K % 128))
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT,
+                "dequant_matmul_i4: tiled weights need N %% 32 == 0 and K %% 128 == 0");
+  I4Args a;
+  a.x = (const uint16_t*)x; a.w = (const uint8_t*)w; a.scale = (const uint16_t*)scale;
+  a.zp = zp; a.out = (uint16_t*)out;
+  a.M = (int)M; a.N = (int)N; a.K = (int)K; a.G = (int)(K / group_size);
+  a.zp_u4 = (flags & IREE_AMD_UK_FLAG_DEQUANT_MATMUL_ZP_U4) != 0;
+  a.tiled = tiled;
+  a.n_tiles = (int)ceil_div(N, 32);
+  a.m_base = 0;
+  a.log2_gs = 0;
+  while ((1ll << a.log2_gs) < group_size) ++a.log2_gs;
+  const bool gs_pow2 = (1ll << a.log2_gs) == group_size;
+  a.span_stride = tiled ? 2048u : 64u;
+  a.col_stride = tiled ? 64u : (uint32_t)(K / 2);
+  // Fast path: K = 512 * KB for KB in {4, 8} (every wave owns KB blocks of 64),
+  // power-of-two groups (below 128 only from tiled weights, where a group never
+  // straddles an MFMA), a weight buffer that 32-bit offsets can address (plus
+  // one tile, for the offset of the tile after the last), 16-byte aligned
+  // operands, and group parameters aligned to what one wave slice loads at once.
+  const int64_t kb = K / 512;
+  const int64_t w_bytes = N * K / 2;
+  const bool k_ok = K % 512 == 0 && (kb == 4 || kb == 8);
+  const bool gs_ok = gs_pow2 && group_size >= (tiled ? 32 : 128);
+  const bool size_ok = w_bytes + K * 16 < (1ll << 32);
+  const bool aligned = ((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0 &&
+                       ((uintptr_t)scale % 16) == 0 && ((uintptr_t)zp % 16) == 0;
+  if (k_ok && gs_ok && size_ok && aligned) {
+    a.w_bytes = (uint32_t)w_bytes;
+    return kb == 4 ? launch_fast<4>(a, s) : launch_fast<8>(a, s);
+  }
+  const int64_t total = M * N;
+  int64_t blocks = ceil_div(total, 256);
+  const int64_t max_blocks = (int64_t)device_cu_count() * 32;
+  if (blocks > max_blocks) blocks = max_blocks;
+  hipLaunchKernelGGL(dequant_matmul_i4_generic_kernel, dim3((unsigned)blocks), dim3(256), 0, s, a,
+                     (int)group_size);
+  return check_hip(hipGetLastError(), "dequant_matmul_i4_generic launch");
+}
+
+int launch_pack_i4_weights(const void* src, void* dst, int64_t N, int64_t K, hipStream_t s) {
+  const int64_t total = N * K / 8;
+  if (total == 0) return 0;
+  int64_t blocks = ceil_div(total, 256);
+  const int64_t max_blocks = (int64_t)device_cu_count() * 32;
+  if (blocks > max_blocks) blocks = max_blocks;
+  hipLaunchKernelGGL(pack_i4_weights_kernel, dim3((unsigned)blocks), dim3(256), 0, s,
+                     (const uint32_t*)src, (uint32_t*)dst, N, K);
+  return check_hip(hipGetLastError(), "pack_i4_weights launch");
+}
+
+//===----------------------------------------------------------------------===//
+// fp8 helpers (placeholders until the fp8 path is built)
+//===----------------------------------------------------------------------===//
+
 int launch_quantize_f16_to_f8e4m3(const void*, void*, int64_t, float, hipStream_t) {
   return fail(IREE_AMD_UK_STATUS_UNIMPLEMENTED, "quantize: not built yet");
 }
@@ -12,4 +454,5 @@ int launch_silu_mul_quantize(const void*, const void*, void*, int64_t, int64_t, 
                              float, float, hipStream_t) {
   return fail(IREE_AMD_UK_STATUS_UNIMPLEMENTED, "silu_mul_quantize: not built yet");
 }
+
 }  // namespace uk

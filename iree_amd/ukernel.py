@@ -121,6 +121,12 @@ def dequant_matmul_i4(x, w, scale, zp, out, M, N, K, group_size, flags=0,
         flags, _stream(stream)))
 
 
+def pack_i4_weights(w_rowmajor, w_tiled, N, K, stream=None):
+    """Row-major [N][K/2] 4-bit weights -> the DEQUANT_MATMUL_W_TILED layout."""
+    _check(load_library().iree_amd_uk_pack_i4_weights(
+        _ptr(w_rowmajor), _ptr(w_tiled), N, K, _stream(stream)))
+
+
 def quantize_f16_to_f8e4m3(inp, out, n, inv_scale, stream=None):
     _check(load_library().iree_amd_uk_quantize_f16_to_f8e4m3(
         _ptr(inp), _ptr(out), n, inv_scale, _stream(stream)))

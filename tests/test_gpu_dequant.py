@@ -1,0 +1,113 @@
+"""GPU parity of the grouped int4 dequantising matmul against the f64 oracle:
+|got - want| <= 1e-3 + 1e-2 |want| (the stated tolerance for int4 results), on
+decode shapes (MFMA kernel) and on shapes only the generic kernel serves."""
+import numpy as np
+import pytest
+
+import ukref
+from iree_amd import flags as F
+from iree_amd import synth
+
+pytestmark = pytest.mark.gpu
+RTOL, ATOL = 1e-2, 1e-3
+
+
+def tile_weights(w_bytes, N, K):
+    """Row-major [N][K/2] nibble bytes -> the pre-tiled layout of the header:
+    [N/32][K/128][32 columns][4 chunks j][4 dwords q], dword (j, q) = row-major
+    dword 4q + j of the column's 64-byte span."""
+    d = w_bytes.view(np.uint32).reshape(N // 32, 32, K // 128, 4, 4)   # [nt][c][s][q][j]
+    return np.ascontiguousarray(d.transpose(0, 2, 1, 4, 3)).reshape(-1).view(np.uint8)
+
+
+def run_case(uk, M, N, K, gs, zp_u4, tiled, seed=0, frac_zp=False):
+    import torch
+    G = K // gs
+    x = synth.normal_f16(seed + 1, M * K)
+    w = synth.uniform_u4_packed(seed + 2, N * K)
+    s = synth.uniform_f16(seed + 4, N * G, 0.005, 0.02)
+    if zp_u4:
+        zp = synth.uniform_u4_packed(seed + 5, N * G)
+        if zp.size * 2 < N * G + 1:
+            zp = np.concatenate([zp, np.zeros(1, np.uint8)])
+    else:
+        zi = (synth.splitmix64(seed + 5, N * G) >> np.uint64(60)).astype(np.float32)
+        if frac_zp:
+            zi = zi + 0.5
+        zp = zi.astype(np.float16)
+    want = np.zeros(M * N, np.uint16)
+    assert ukref.oracle().oracle_dequant_matmul_i4(
+        ukref.ptr(x.view(np.uint16)), ukref.ptr(w), ukref.ptr(s.view(np.uint16)),
+        ukref.ptr(zp.view(np.uint8) if zp_u4 else zp.view(np.uint16)), ukref.ptr(want),
+        M, N, K, gs, int(zp_u4)) == 0
+    wd = tile_weights(w, N, K) if tiled else w
+    flags = (F.DEQUANT_MATMUL_ZP_U4 if zp_u4 else 0) | (F.DEQUANT_MATMUL_W_TILED if tiled else 0)
+    out = torch.full((M * N,), 0x7E00, dtype=torch.int16, device="cuda")
+    uk.dequant_matmul_i4(torch.from_numpy(x.view(np.int16)).cuda(), torch.from_numpy(wd).cuda(),
+                         torch.from_numpy(s.view(np.int16)).cuda(),
+                         torch.from_numpy(zp.view(np.uint8)).cuda(), out, M, N, K, gs, flags)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy().view(np.float16).astype(np.float64)
+    wantf = want.view(np.float16).astype(np.float64)
+    err = np.abs(got - wantf)
+    assert np.all(err <= ATOL + RTOL * np.abs(wantf)), (M, N, K, gs, zp_u4, tiled, float(err.max()))
+    return float(err.max()), float(np.abs(wantf).max())
+
+
+@pytest.mark.parametrize("M", [1, 8, 32])
+@pytest.mark.parametrize("tiled", [False, True])
+def test_decode_shape_llama_ffn(uk, cuda, M, tiled):
+    """The decode configuration: K = 4096, N = 14336, groups of 128, f16 scales,
+    packed uint4 zero points."""
+    err, mag = run_case(uk, M, 14336, 4096, 128, True, tiled)
+    # f32 accumulation of exact products: far inside the stated tolerance
+    assert err <= 4e-3 * max(1.0, mag) / 8
+
+
+@pytest.mark.parametrize("K,gs", [(1024, 32), (1024, 64), (2048, 32), (2048, 64), (2048, 128), (2048, 256),
+                                  (2048, 2048), (4096, 32), (4096, 64), (4096, 256), (4096, 512),
+                                  (4096, 1024), (4096, 4096)])
+@pytest.mark.parametrize("zp_u4", [False, True])
+def test_mfma_kernel_group_sizes_and_zero_point_forms(uk, cuda, K, gs, zp_u4):
+    for M, N, tiled in [(3, 96, True), (32, 64, False), (40, 100, False), (17, 160, True)]:
+        run_case(uk, M, N, K, gs, zp_u4, tiled, seed=K + gs)
+
+
+def test_fractional_f16_zero_points(uk, cuda):
+    run_case(uk, 5, 64, 2048, 128, False, False, seed=3, frac_zp=True)
+    run_case(uk, 5, 64, 2048, 128, False, True, seed=4, frac_zp=True)
+
+
+@pytest.mark.parametrize("M,N,K,gs", [(2, 10, 96, 32), (5, 33, 192, 96), (1, 7, 640, 64), (3, 64, 1536, 128)])
+def test_generic_kernel_shapes(uk, cuda, M, N, K, gs):
+    for zp_u4 in (False, True):
+        run_case(uk, M, N, K, gs, zp_u4, False, seed=M * N)
+    if N % 32 == 0 and K % 128 == 0:
+        run_case(uk, M, N, K, gs, True, True, seed=M * N + 1)
+
+
+def test_pack_i4_weights_matches_the_documented_layout(uk, cuda):
+    import torch
+    for N, K in [(32, 128), (96, 512), (14336, 4096)]:
+        w = synth.uniform_u4_packed(N + K, N * K)
+        dst = torch.zeros(N * K // 2, dtype=torch.uint8, device="cuda")
+        uk.pack_i4_weights(torch.from_numpy(w).cuda(), dst, N, K)
+        torch.cuda.synchronize()
+        assert np.array_equal(dst.cpu().numpy(), tile_weights(w, N, K)), (N, K)
+    with pytest.raises(uk.UkError):
+        uk.pack_i4_weights(dst, dst, 48, 128)
+    with pytest.raises(uk.UkError):
+        uk.pack_i4_weights(dst, dst, 32, 192)
+
+
+def test_invalid_arguments(uk, cuda):
+    import torch
+    t = torch.zeros(64, dtype=torch.int16, device="cuda")
+    with pytest.raises(uk.UkError) as e:
+        uk.dequant_matmul_i4(t, t, t, t, t, 1, 8, 100, 32)       # K % group_size != 0
+    assert e.value.status == F.STATUS_INVALID_ARGUMENT
+    with pytest.raises(uk.UkError):
+        uk.dequant_matmul_i4(t, t, t, t, t, 1, 8, 128, 48)       # group_size % 32 != 0
+    with pytest.raises(uk.UkError):
+        uk.dequant_matmul_i4(t, t, t, t, t, 1, 8, 128, 32, F.DEQUANT_MATMUL_W_TILED)  # N % 32
+    uk.dequant_matmul_i4(t, t, t, t, t, 0, 8, 128, 32)           # M == 0: nothing to do
