@@ -263,6 +263,33 @@ def extras(args, torch, iree_amd, F, synth, lhs, rhs, out):
                                                               F.MMT4D_TYPE_F16F16F32, workspace=ws),
                     max(5, steps // 4), 2)
     ex["matmul_f16_pack_mmt4d_unpack_tflops"] = round(flops / t / 1e12, 2)
+    del a, b, c, ws
+
+    # grouped int4 dequant matmul, decode shapes (K = 4096, N = 14336, groups of
+    # 128, f16 scales, packed uint4 zero points, pre-tiled weights). Ten weight
+    # sets (294 MB) rotate so that the weights come from HBM.
+    Nq, Kq, gs = 14336, 4096, 128
+    G = Kq // gs
+    nrot = 10
+    wq = [torch.from_numpy(synth.uniform_u4_packed(10 + i, Nq * Kq)).cuda() for i in range(nrot)]
+    sq = torch.from_numpy(synth.uniform_f16(30, Nq * G, 0.005, 0.02).view(np.int16)).cuda()
+    zq = torch.from_numpy(synth.uniform_u4_packed(31, Nq * G)).cuda()
+    qflags = F.DEQUANT_MATMUL_ZP_U4 | F.DEQUANT_MATMUL_W_TILED
+    for Mq in (1, 8, 32):
+        xq = torch.from_numpy(synth.normal_f16(40 + Mq, Mq * Kq).view(np.int16)).cuda()
+        oq = torch.empty(Mq * Nq, dtype=torch.int16, device="cuda")
+        qbytes = Nq * Kq // 2 + Nq * G * 2 + Nq * G // 2 + Mq * Kq * 2 + Mq * Nq * 2
+        state["i"] = 0
+
+        def do_q():
+            k = state["i"] % nrot
+            state["i"] += 1
+            iree_amd.dequant_matmul_i4(xq, wq[k], sq, zq, oq, Mq, Nq, Kq, gs, qflags)
+
+        _, t = gpu_time(torch, do_q, steps, warm)
+        ex[f"dequant_matmul_i4_m{Mq}_gbs"] = round(qbytes / t / 1e9, 1)
+        ex[f"dequant_matmul_i4_m{Mq}_us"] = round(t * 1e6, 2)
+    ex["dequant_matmul_i4_m1_frac_of_hbm_peak"] = round(ex["dequant_matmul_i4_m1_gbs"] / PEAK_HBM_GBS, 4)
     return ex
 
 

@@ -369,6 +369,25 @@ IREE_AMD_UK_EXPORT int iree_amd_uk_silu_mul_quantize(
     iree_amd_uk_index_t rows, iree_amd_uk_index_t cols, iree_amd_uk_index_t ld,
     float gate_scale, float up_scale, float inv_out_scale, void* stream);
 
+/* The same on data-tiled buffers, fusing the unpack of the gate/up result and
+ * the pack of the next left-hand side: `acc_tiled` is an mmt4d f32 result with
+ * 32x32 tiles (outer row pitch acc_stride0 ELEMENTS) whose outer columns
+ * [gate_tile0, gate_tile0+N1) hold gate and [up_tile0, up_tile0+N1) hold up;
+ * `out_tiled` receives e4m3 left-hand-side tiles 32x16 (outer row pitch
+ * out_stride0 elements), outer column 2j and 2j+1 from tile column j. M1 is the
+ * number of outer rows. Buffers 16-byte aligned. */
+IREE_AMD_UK_EXPORT int iree_amd_uk_silu_mul_quantize_tiled(
+    const void* acc_tiled, iree_amd_uk_index_t acc_stride0,
+    iree_amd_uk_index_t gate_tile0, iree_amd_uk_index_t up_tile0,
+    void* out_tiled, iree_amd_uk_index_t out_stride0, iree_amd_uk_index_t M1,
+    iree_amd_uk_index_t N1, float gate_scale, float up_scale,
+    float inv_out_scale, void* stream);
+
+/* buf[i] *= scale over n f32 elements, in place (applies the product of the
+ * per-tensor scales to an fp8 matmul result). */
+IREE_AMD_UK_EXPORT int iree_amd_uk_scale_f32(void* buf_f32, iree_amd_uk_index_t n,
+                                             float scale, void* stream);
+
 /*===------------------------------------------------------------------------===
  * Thin device ABI, so that a pure-C host (the HAL executable plugin) needs no
  * HIP headers. Mirrors the handful of driver calls the reference's own HIP HAL

@@ -9,6 +9,7 @@ used only to own device memory and streams.
 from . import flags  # noqa: F401
 from ._lib import load_library, library_path  # noqa: F401
 from .ukernel import (  # noqa: F401
+    Fp8Mlp,
     UkError,
     dequant_matmul_i4,
     matmul_data_tiled,
@@ -18,6 +19,8 @@ from .ukernel import (  # noqa: F401
     pack_i4_weights,
     quantize_f16_to_f8e4m3,
     query_tile_sizes_2d,
+    scale_f32,
     silu_mul_quantize,
+    silu_mul_quantize_tiled,
     unpack,
 )

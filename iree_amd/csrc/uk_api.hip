@@ -212,13 +212,18 @@ extern "C" int iree_amd_uk_mmt4d_p(const iree_amd_uk_mmt4d_params_t* params,
   if (mmt4d_mfma_supported(p.flags, p.M0, p.N0, p.K0)) {
     int st = launch_mmt4d_mfma(p, s);
     if (st != IREE_AMD_UK_STATUS_NOT_FOUND) return st;
+    // A gfx950 tile whose operands the MFMA kernel cannot take (not 16-byte
+    // aligned, or a K extent that is not whole MFMA steps): the tile is still
+    // an architecture tile, served by the element-wise kernel whether or not
+    // the caller allowed the generic fallback.
+    return launch_mmt4d_generic(p, s);
   }
   if (!(p.flags & IREE_AMD_UK_FLAG_MMT4D_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION)) {
     // The reference asserts here (mmt4d.c:128-138); a release build would
     // crash on a null tile function. Report instead.
     return fail(IREE_AMD_UK_STATUS_UNIMPLEMENTED,
-                "mmt4d: no gfx950 MFMA kernel for type 0x%x tile %dx%dx%d (or "
-                "operands not 16-byte aligned) and generic fallback not allowed",
+                "mmt4d: no gfx950 MFMA kernel for type 0x%x tile %dx%dx%d and "
+                "generic fallback not allowed",
                 p.flags & 0xFF, p.M0, p.N0, p.K0);
   }
   return launch_mmt4d_generic(p, s);
@@ -404,6 +409,38 @@ extern "C" int iree_amd_uk_silu_mul_quantize(
   return launch_silu_mul_quantize(gate_f32, up_f32, out_fp8, rows, cols, ld,
                                   gate_scale, up_scale, inv_out_scale,
                                   (hipStream_t)stream);
+}
+
+extern "C" int iree_amd_uk_silu_mul_quantize_tiled(
+    const void* acc_tiled, iree_amd_uk_index_t acc_stride0,
+    iree_amd_uk_index_t gate_tile0, iree_amd_uk_index_t up_tile0,
+    void* out_tiled, iree_amd_uk_index_t out_stride0, iree_amd_uk_index_t M1,
+    iree_amd_uk_index_t N1, float gate_scale, float up_scale,
+    float inv_out_scale, void* stream) {
+  if (M1 < 0 || N1 < 0 || gate_tile0 < 0 || up_tile0 < 0)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "silu_mul_quantize_tiled: bad sizes");
+  if (M1 == 0 || N1 == 0) return 0;
+  if (!acc_tiled || !out_tiled)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "silu_mul_quantize_tiled: null buffer");
+  const iree_amd_uk_index_t last = (gate_tile0 > up_tile0 ? gate_tile0 : up_tile0) + N1;
+  if (acc_stride0 < last * 1024 || out_stride0 < N1 * 1024)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT,
+                "silu_mul_quantize_tiled: outer row pitch smaller than the tiles of a row");
+  if (((uintptr_t)acc_tiled | (uintptr_t)out_tiled) % 16 || acc_stride0 % 4 || out_stride0 % 16)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT,
+                "silu_mul_quantize_tiled: buffers and pitches must be 16-byte aligned");
+  return launch_silu_mul_quantize_tiled(acc_tiled, acc_stride0, gate_tile0, up_tile0, out_tiled,
+                                        out_stride0, M1, N1, gate_scale, up_scale,
+                                        inv_out_scale, (hipStream_t)stream);
+}
+
+extern "C" int iree_amd_uk_scale_f32(void* buf_f32, iree_amd_uk_index_t n, float scale,
+                                     void* stream) {
+  if (n < 0) return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "scale_f32: negative n");
+  if (n == 0) return 0;
+  if (!buf_f32 || (uintptr_t)buf_f32 % 4)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "scale_f32: null or misaligned buffer");
+  return launch_scale_f32(buf_f32, n, scale, (hipStream_t)stream);
 }
 
 //===----------------------------------------------------------------------===//

@@ -73,6 +73,11 @@ int launch_silu_mul_quantize(const void* gate, const void* up, void* out,
                              int64_t rows, int64_t cols, int64_t ld,
                              float gate_scale, float up_scale,
                              float inv_out_scale, hipStream_t s);
+int launch_silu_mul_quantize_tiled(const void* acc, int64_t acc_stride0, int64_t gate_tile0,
+                                   int64_t up_tile0, void* out, int64_t out_stride0, int64_t M1,
+                                   int64_t N1, float gate_scale, float up_scale,
+                                   float inv_out_scale, hipStream_t s);
+int launch_scale_f32(void* buf, int64_t n, float scale, hipStream_t s);
 
 // Number of compute units of the current device (cached per device).
 int device_cu_count();

@@ -10,12 +10,17 @@
 //   f16 x f16 -> f32  v_mfma_f32_32x32x16_f16        16         8, 16
 //   bf16 x bf16 -> f32 v_mfma_f32_32x32x16_bf16      16         8, 16
 //   s8 x s8 -> s32    v_mfma_i32_32x32x32_i8         32         16, 32
+//   e4m3 x e4m3 -> f32 v_mfma_scale_f32_32x32x64_f8f6f4  64         16
 //
 // With K0 = half the MFMA's K extent, two consecutive K tiles of one outer row
 // ARE one MFMA operand in register order (lane l <-> bytes [16 l, 16 l + 16)),
 // so a 64-lane 128-bit load moves a 1 KiB operand block with perfectly linear
 // addressing. With K0 = the full extent the same 1 KiB holds one tile and the
-// lane <-> address map is (l % 32) * 32 + (l / 32) * 16.
+// lane <-> address map is (l % 32) * 32 + (l / 32) * 16. The fp8 instruction
+// takes 32 bytes per lane (k = 32 (l / 32) .. + 32 of row l % 32): four K0 = 16
+// tiles make one operand block of 2 KiB, moved as two 1 KiB halves in which
+// lanes 0-31 fetch one whole tile and lanes 32-63 the tile two further on, so
+// each half is again in lane order in LDS. (OCP e4m3fn, unit block scales.)
 //
 // Kernel shape: a workgroup of 4 waves owns a macro tile of (2*WM) x (2*WN)
 // outer tiles; each wave accumulates WM x WN blocks of 32x32 in registers. The K
@@ -39,6 +44,7 @@ namespace {
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef int int4v __attribute__((ext_vector_type(4)));
+typedef int int8v __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef int intx16 __attribute__((ext_vector_type(16)));
 
@@ -48,6 +54,7 @@ struct F16Cfg {
   typedef float out_t;
   static constexpr int kElemBytes = 2;
   static constexpr int kMfmaK = 16;
+  static constexpr int kSub = 1;   // 1 KiB pieces per operand block
   __device__ static acc_t mfma(frag_t a, frag_t b, acc_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
   }
@@ -58,6 +65,7 @@ struct BF16Cfg {
   typedef float out_t;
   static constexpr int kElemBytes = 2;
   static constexpr int kMfmaK = 16;
+  static constexpr int kSub = 1;
   __device__ static acc_t mfma(frag_t a, frag_t b, acc_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
@@ -68,13 +76,26 @@ struct S8Cfg {
   typedef int32_t out_t;
   static constexpr int kElemBytes = 1;
   static constexpr int kMfmaK = 32;
+  static constexpr int kSub = 1;
   __device__ static acc_t mfma(frag_t a, frag_t b, acc_t c) {
     return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
   }
 };
+struct F8Cfg {
+  typedef int8v frag_t;
+  typedef floatx16 acc_t;
+  typedef float out_t;
+  static constexpr int kElemBytes = 1;
+  static constexpr int kMfmaK = 64;
+  static constexpr int kSub = 2;
+  __device__ static acc_t mfma(frag_t a, frag_t b, acc_t c) {
+    // formats 0 / 0: both operands e4m3; block scales 0x7F = 2^0.
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+  }
+};
 
 constexpr int kThreads = 256;
-constexpr int kBlockBytes = 1024;   // one 32-row operand block of one K-step
+constexpr int kPieceBytes = 1024;   // what one 64-lane 128-bit load moves
 
 struct MfmaArgs {
   const char* lhs;  // offset applied
@@ -150,11 +171,13 @@ __global__ __launch_bounds__(kThreads) void mmt4d_mfma_kernel(MfmaArgs a) {
   typedef typename Cfg::acc_t acc_t;
   typedef typename Cfg::out_t out_t;
   constexpr int TM = 2 * WM, TN = 2 * WN;      // outer tiles per workgroup
+  constexpr int kSub = Cfg::kSub;
+  constexpr int kBlockBytes = kSub * kPieceBytes;   // one 32-row operand block of one K-step
   constexpr int kABytes = TM * kBlockBytes;
   constexpr int kSlotBytes = (TM + TN) * kBlockBytes;
   constexpr int kAhead = kRing - kSync;
   constexpr int kARowsPerWave = TM / 4, kBRowsPerWave = TN / 4;
-  constexpr int kLoadsPerStep = kARowsPerWave + kBRowsPerWave;  // per wave
+  constexpr int kLoadsPerStep = (kARowsPerWave + kBRowsPerWave) * kSub;  // per wave
   constexpr int kBody = (kSync % 2) ? 2 * kSync : kSync;        // K-steps per unrolled body
   static_assert(kAhead >= kSync && kAhead % kSync == 0, "ring must hold whole sync groups");
   static_assert((kAhead - kSync) * kLoadsPerStep < 64, "too many loads in flight for vmcnt");
@@ -168,8 +191,11 @@ __global__ __launch_bounds__(kThreads) void mmt4d_mfma_kernel(MfmaArgs a) {
   const int i_base = tm * TM, j_base = tn * TN;
   const int T = a.ksteps;
 
-  // Per-lane byte offset inside a 1 KiB operand block in global memory.
-  const int lane_off = kHalfK0 ? lane * 16 : ((lane & 31) * 32 + (lane >> 5) * 16);
+  // Per-lane byte offset inside an operand block in global memory (of its
+  // first piece; with two pieces the second lies one 512-byte tile further).
+  const int lane_off = kSub == 2 ? ((lane >> 5) * 1024 + (lane & 31) * 16)
+                       : kHalfK0 ? lane * 16 : ((lane & 31) * 32 + (lane >> 5) * 16);
+  constexpr int kPieceStride = 512;
 
   // Rows this wave copies: TM/4 rows of A and TN/4 rows of B. Out-of-range
   // rows are clamped to the last valid one (loaded, never stored).
@@ -216,20 +242,32 @@ __global__ __launch_bounds__(kThreads) void mmt4d_mfma_kernel(MfmaArgs a) {
     char* base = lds + slot * kSlotBytes;
 #pragma unroll
     for (int r = 0; r < kARowsPerWave; ++r)
-      load_block_to_lds(a_src[r] + (int64_t)ks * kBlockBytes,
-                        base + (wave * kARowsPerWave + r) * kBlockBytes);
+#pragma unroll
+      for (int j = 0; j < kSub; ++j)
+        load_block_to_lds(a_src[r] + (int64_t)ks * kBlockBytes + j * kPieceStride,
+                          base + (wave * kARowsPerWave + r) * kBlockBytes + j * kPieceBytes);
 #pragma unroll
     for (int r = 0; r < kBRowsPerWave; ++r)
-      load_block_to_lds(b_src[r] + (int64_t)ks * kBlockBytes,
-                        base + kABytes + (wave * kBRowsPerWave + r) * kBlockBytes);
+#pragma unroll
+      for (int j = 0; j < kSub; ++j)
+        load_block_to_lds(b_src[r] + (int64_t)ks * kBlockBytes + j * kPieceStride,
+                          base + kABytes + (wave * kBRowsPerWave + r) * kBlockBytes + j * kPieceBytes);
+  };
+  auto read_frag = [&](const char* p) -> frag_t {
+    if constexpr (kSub == 1) {
+      return *(const frag_t*)p;
+    } else {
+      const int4v lo = *(const int4v*)p, hi = *(const int4v*)(p + kPieceBytes);
+      return frag_t{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    }
   };
   auto read_frags = [&](int slot, frag_t (&fa)[WM], frag_t (&fb)[WN]) {
     const char* sa = lds + slot * kSlotBytes + (wm * WM) * kBlockBytes + lane * 16;
     const char* sb = lds + slot * kSlotBytes + kABytes + (wn * WN) * kBlockBytes + lane * 16;
 #pragma unroll
-    for (int x = 0; x < WM; ++x) fa[x] = *(const frag_t*)(sa + x * kBlockBytes);
+    for (int x = 0; x < WM; ++x) fa[x] = read_frag(sa + x * kBlockBytes);
 #pragma unroll
-    for (int y = 0; y < WN; ++y) fb[y] = *(const frag_t*)(sb + y * kBlockBytes);
+    for (int y = 0; y < WN; ++y) fb[y] = read_frag(sb + y * kBlockBytes);
   };
   // MFMAs of block rows [x0, x1) of this wave's WM x WN blocks.
   auto multiply_rows = [&](const frag_t (&fa)[WM], const frag_t (&fb)[WN], int x0, int x1) {
@@ -271,7 +309,8 @@ __global__ __launch_bounds__(kThreads) void mmt4d_mfma_kernel(MfmaArgs a) {
           // Issue order: one LDS read slipped in behind each of the first
           // MFMAs (an LDS read issues in the shadow of the running MFMA),
           // then the rest of the MFMAs back to back.
-          interleave_issue<WM * WN, 0, WM + WN, (WM * WN < WM + WN ? WM * WN : WM + WN)>();
+          constexpr int kReads = (WM + WN) * kSub;
+          interleave_issue<WM * WN, 0, kReads, (WM * WN < kReads ? WM * WN : kReads)>();
         } else {
           // The first row of MFMAs goes ahead of the barrier so that the
           // matrix pipe has work while the waves meet. All reads of K-steps
@@ -298,7 +337,7 @@ __global__ __launch_bounds__(kThreads) void mmt4d_mfma_kernel(MfmaArgs a) {
           }
           read_frags(next_slot, fa[p ^ 1], fb[p ^ 1]);
           multiply_rows(fa[p], fb[p], 1, WM);
-          constexpr int kDma = kSync * kLoadsPerStep, kMma = (WM - 1) * WN, kDsr = WM + WN;
+          constexpr int kDma = kSync * kLoadsPerStep, kMma = (WM - 1) * WN, kDsr = (WM + WN) * kSub;
           constexpr int kSlots = kMma < kDsr ? kMma : kDsr;
           interleave_issue<kMma, kDma, kDsr, kSlots>();
           __builtin_amdgcn_sched_barrier(0);
@@ -355,7 +394,7 @@ int launch_variant(const MfmaArgs& a0, hipStream_t s) {
   a.tiles_n = (a.N + TN - 1) / TN;
   const int64_t blocks = (int64_t)a.tiles_m * a.tiles_n;
   if (blocks > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
-  constexpr int lds_bytes = kRing * (TM + TN) * kBlockBytes;
+  constexpr int lds_bytes = kRing * (TM + TN) * Cfg::kSub * kPieceBytes;
   static_assert(lds_bytes <= 160 * 1024, "LDS ring exceeds 160 KiB");
   auto kernel = mmt4d_mfma_kernel<Cfg, WM, WN, kHalfK0, kRing, kSync>;
   static bool attr_set = false;  // benign race: the call is idempotent
@@ -377,7 +416,11 @@ int launch_half(const MfmaArgs& a, hipStream_t s) {
   // 2 K-steps, 6 K-steps of loads in flight.
   const int cus = device_cu_count();
   const int64_t big = (int64_t)((a.M + 7) / 8) * ((a.N + 7) / 8);
-  if (big >= cus) return launch_variant<Cfg, 4, 4, kHalfK0, 8, 2>(a, s);
+  // An fp8 K-step moves (and multiplies) twice as much: its large tile gets a
+  // ring of 5 K-steps (all 160 KiB of LDS) with a barrier every K-step, which
+  // is the same barrier rate and load lead in time.
+  constexpr int kRing = Cfg::kSub == 2 ? 5 : 8, kSync = Cfg::kSub == 2 ? 1 : 2;
+  if (big >= cus) return launch_variant<Cfg, 4, 4, kHalfK0, kRing, kSync>(a, s);
   return launch_variant<Cfg, 2, 2, kHalfK0, 8, 2>(a, s);
 }
 
@@ -393,10 +436,15 @@ bool served(uint32_t flags, int M0, int N0, int K0, Served* out) {
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F32:
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16F32: mfma_k = 16; break;
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32: mfma_k = 32; break;
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F8E4M3F8E4M3F32: mfma_k = 64; break;
     default: return false;
   }
   if (M0 != 32 || N0 != 32) return false;
-  if (K0 != mfma_k && K0 * 2 != mfma_k) return false;
+  if (mfma_k == 64) {
+    if (K0 != 16) return false;
+  } else if (K0 != mfma_k && K0 * 2 != mfma_k) {
+    return false;
+  }
   if (out) out->mfma_k = mfma_k;
   return true;
 }
@@ -436,6 +484,7 @@ int launch_mmt4d_mfma(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) {
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F32: return launch_cfg<F16Cfg>(a, half_k0, s);
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16F32: return launch_cfg<BF16Cfg>(a, half_k0, s);
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32: return launch_cfg<S8Cfg>(a, half_k0, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F8E4M3F8E4M3F32: return launch_half<F8Cfg, true>(a, s);
     default: return IREE_AMD_UK_STATUS_NOT_FOUND;
   }
 }

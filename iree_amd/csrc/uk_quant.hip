@@ -444,15 +444,187 @@ int launch_pack_i4_weights(const void* src, void* dst, int64_t N, int64_t K, hip
 }
 
 //===----------------------------------------------------------------------===//
-// fp8 helpers (placeholders until the fp8 path is built)
+// fp8 element-wise helpers of the MLP block. All of them are HBM streams:
+// 16-byte accesses, no reuse.
 //===----------------------------------------------------------------------===//
 
-int launch_quantize_f16_to_f8e4m3(const void*, void*, int64_t, float, hipStream_t) {
-  return fail(IREE_AMD_UK_STATUS_UNIMPLEMENTED, "quantize: not built yet");
+namespace {
+
+// f32 -> OCP e4m3fn, round to nearest even, saturating at +-448 (NaN stays NaN).
+__device__ __forceinline__ float clamp_e4m3(float x) {
+  const float c = __builtin_fminf(__builtin_fmaxf(x, -448.0f), 448.0f);
+  return x != x ? x : c;
 }
-int launch_silu_mul_quantize(const void*, const void*, void*, int64_t, int64_t, int64_t, float,
-                             float, float, hipStream_t) {
-  return fail(IREE_AMD_UK_STATUS_UNIMPLEMENTED, "silu_mul_quantize: not built yet");
+// Four floats -> four e4m3 bytes (first value in the low byte).
+__device__ __forceinline__ uint32_t pack4_e4m3(float a, float b, float c, float d) {
+  int v = 0;
+  v = __builtin_amdgcn_cvt_pk_fp8_f32(clamp_e4m3(a), clamp_e4m3(b), v, false);
+  v = __builtin_amdgcn_cvt_pk_fp8_f32(clamp_e4m3(c), clamp_e4m3(d), v, true);
+  return (uint32_t)v;
+}
+
+__device__ __forceinline__ float silu_mul(float g, float u) {
+  // g / (1 + exp(-g)) * u; exp(-g) overflows to +inf for g < -88, giving -0.
+  return __fdividef(g, 1.0f + __expf(-g)) * u;
+}
+
+__global__ __launch_bounds__(256) void quantize_f16_kernel(const uint16_t* in, uint8_t* out,
+                                                           int64_t n, float inv_scale) {
+  const int64_t n8 = n >> 3;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n8;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const u32x4 v = ((const u32x4*)in)[i];
+    float f[8];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      f[2 * j] = __half2float(__ushort_as_half((uint16_t)(v[j] & 0xFFFF))) * inv_scale;
+      f[2 * j + 1] = __half2float(__ushort_as_half((uint16_t)(v[j] >> 16))) * inv_scale;
+    }
+    ((u32x2*)out)[i] = u32x2{pack4_e4m3(f[0], f[1], f[2], f[3]), pack4_e4m3(f[4], f[5], f[6], f[7])};
+  }
+  // tail (n % 8 elements) and unaligned buffers: element-wise
+  if (blockIdx.x == 0) {
+    for (int64_t i = (n8 << 3) + threadIdx.x; i < n; i += blockDim.x) {
+      const float f = __half2float(__ushort_as_half(in[i])) * inv_scale;
+      out[i] = (uint8_t)(pack4_e4m3(f, 0.f, 0.f, 0.f) & 0xFF);
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void quantize_f16_scalar_kernel(const uint16_t* in, uint8_t* out,
+                                                                  int64_t n, float inv_scale) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const float f = __half2float(__ushort_as_half(in[i])) * inv_scale;
+    out[i] = (uint8_t)(pack4_e4m3(f, 0.f, 0.f, 0.f) & 0xFF);
+  }
+}
+
+// Row-major: thread = 4 consecutive columns of one row when everything is
+// 16-byte aligned (kVec), else one element.
+template <bool kVec>
+__global__ __launch_bounds__(256) void silu_mul_quantize_kernel(const float* gate, const float* up,
+                                                                uint8_t* out, int64_t rows,
+                                                                int64_t cols, int64_t ld, float gs,
+                                                                float us, float os) {
+  constexpr int V = kVec ? 4 : 1;
+  const int64_t per_row = cols / V, total = rows * per_row;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t r = i / per_row, c = (i - r * per_row) * V;
+    if constexpr (kVec) {
+      const floatx4 g = *(const floatx4*)(gate + r * ld + c), u = *(const floatx4*)(up + r * ld + c);
+      float h[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) h[j] = silu_mul(g[j] * gs, u[j] * us) * os;
+      *(uint32_t*)(out + r * cols + c) = pack4_e4m3(h[0], h[1], h[2], h[3]);
+    } else {
+      const float h = silu_mul(gate[r * ld + c] * gs, up[r * ld + c] * us) * os;
+      out[r * cols + c] = (uint8_t)(pack4_e4m3(h, 0.f, 0.f, 0.f) & 0xFF);
+    }
+  }
+}
+
+// Tiled: one wave per pair (gate tile, up tile) of 32x32 f32 accumulators;
+// lane l owns row l / 2, columns (l % 2) * 16 .. + 16: 64 contiguous bytes of
+// each input tile and 16 contiguous bytes of the output, which is the pair of
+// adjacent 32x16 e4m3 left-hand-side tiles (2j, 2j+1) of outer row i.
+__global__ __launch_bounds__(256) void silu_mul_quantize_tiled_kernel(
+    const float* acc, int64_t acc_stride0, int64_t gate_tile0, int64_t up_tile0, uint8_t* out,
+    int64_t out_stride0, int64_t M1, int64_t N1, float gs, float us, float os) {
+  const int lane = threadIdx.x & 63;
+  const int64_t pair = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (pair >= M1 * N1) return;
+  const int64_t i = pair / N1, j = pair - i * N1;
+  const float* g = acc + i * acc_stride0 + (gate_tile0 + j) * 1024 + lane * 16;
+  const float* u = acc + i * acc_stride0 + (up_tile0 + j) * 1024 + lane * 16;
+  uint32_t w[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const floatx4 gv = ((const floatx4*)g)[q], uv = ((const floatx4*)u)[q];
+    float h[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) h[e] = silu_mul(gv[e] * gs, uv[e] * us) * os;
+    w[q] = pack4_e4m3(h[0], h[1], h[2], h[3]);
+  }
+  uint8_t* o = out + i * out_stride0 + j * 1024 + (lane & 1) * 512 + (lane >> 1) * 16;
+  *(u32x4*)o = u32x4{w[0], w[1], w[2], w[3]};
+}
+
+template <bool kVec>
+__global__ __launch_bounds__(256) void scale_f32_kernel(float* buf, int64_t n, float scale) {
+  const int64_t n4 = kVec ? n >> 2 : 0;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    floatx4 v = ((floatx4*)buf)[i];
+    v[0] *= scale; v[1] *= scale; v[2] *= scale; v[3] *= scale;
+    ((floatx4*)buf)[i] = v;
+  }
+  for (int64_t i = (n4 << 2) + (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (int64_t)gridDim.x * blockDim.x)
+    buf[i] *= scale;
+}
+
+unsigned stream_blocks(int64_t work_items) {
+  int64_t blocks = ceil_div(work_items, (int64_t)256);
+  const int64_t max_blocks = (int64_t)device_cu_count() * 16;
+  if (blocks > max_blocks) blocks = max_blocks;
+  return (unsigned)(blocks < 1 ? 1 : blocks);
+}
+
+}  // namespace
+
+int launch_quantize_f16_to_f8e4m3(const void* in, void* out, int64_t n, float inv_scale,
+                                  hipStream_t s) {
+  if (((uintptr_t)in % 16) == 0 && ((uintptr_t)out % 8) == 0) {
+    hipLaunchKernelGGL(quantize_f16_kernel, dim3(stream_blocks(n / 8)), dim3(256), 0, s,
+                       (const uint16_t*)in, (uint8_t*)out, n, inv_scale);
+  } else {
+    hipLaunchKernelGGL(quantize_f16_scalar_kernel, dim3(stream_blocks(n)), dim3(256), 0, s,
+                       (const uint16_t*)in, (uint8_t*)out, n, inv_scale);
+  }
+  return check_hip(hipGetLastError(), "quantize_f16_to_f8e4m3 launch");
+}
+
+int launch_silu_mul_quantize(const void* gate, const void* up, void* out, int64_t rows,
+                             int64_t cols, int64_t ld, float gate_scale, float up_scale,
+                             float inv_out_scale, hipStream_t s) {
+  const bool vec = cols % 4 == 0 && ld % 4 == 0 && ((uintptr_t)gate % 16) == 0 &&
+                   ((uintptr_t)up % 16) == 0 && ((uintptr_t)out % 4) == 0;
+  if (vec) {
+    hipLaunchKernelGGL(silu_mul_quantize_kernel<true>, dim3(stream_blocks(rows * cols / 4)), dim3(256),
+                       0, s, (const float*)gate, (const float*)up, (uint8_t*)out, rows, cols, ld,
+                       gate_scale, up_scale, inv_out_scale);
+  } else {
+    hipLaunchKernelGGL(silu_mul_quantize_kernel<false>, dim3(stream_blocks(rows * cols)), dim3(256),
+                       0, s, (const float*)gate, (const float*)up, (uint8_t*)out, rows, cols, ld,
+                       gate_scale, up_scale, inv_out_scale);
+  }
+  return check_hip(hipGetLastError(), "silu_mul_quantize launch");
+}
+
+int launch_silu_mul_quantize_tiled(const void* acc, int64_t acc_stride0, int64_t gate_tile0,
+                                   int64_t up_tile0, void* out, int64_t out_stride0, int64_t M1,
+                                   int64_t N1, float gate_scale, float up_scale,
+                                   float inv_out_scale, hipStream_t s) {
+  const int64_t blocks = ceil_div(M1 * N1, (int64_t)4);
+  if (blocks > 0x7FFFFFFF)
+    return fail(IREE_AMD_UK_STATUS_OUT_OF_RANGE, "silu_mul_quantize_tiled: too many tiles");
+  hipLaunchKernelGGL(silu_mul_quantize_tiled_kernel, dim3((unsigned)blocks), dim3(256), 0, s,
+                     (const float*)acc, acc_stride0, gate_tile0, up_tile0, (uint8_t*)out,
+                     out_stride0, M1, N1, gate_scale, up_scale, inv_out_scale);
+  return check_hip(hipGetLastError(), "silu_mul_quantize_tiled launch");
+}
+
+int launch_scale_f32(void* buf, int64_t n, float scale, hipStream_t s) {
+  if ((uintptr_t)buf % 16 == 0) {
+    hipLaunchKernelGGL(scale_f32_kernel<true>, dim3(stream_blocks(n / 4)), dim3(256), 0, s,
+                       (float*)buf, n, scale);
+  } else {
+    hipLaunchKernelGGL(scale_f32_kernel<false>, dim3(stream_blocks(n)), dim3(256), 0, s, (float*)buf,
+                       n, scale);
+  }
+  return check_hip(hipGetLastError(), "scale_f32 launch");
 }
 
 }  // namespace uk

@@ -139,6 +139,17 @@ def silu_mul_quantize(gate, up, out, rows, cols, ld, gate_scale, up_scale,
         inv_out_scale, _stream(stream)))
 
 
+def silu_mul_quantize_tiled(acc, acc_stride0, gate_tile0, up_tile0, out, out_stride0,
+                            M1, N1, gate_scale, up_scale, inv_out_scale, stream=None):
+    _check(load_library().iree_amd_uk_silu_mul_quantize_tiled(
+        _ptr(acc), acc_stride0, gate_tile0, up_tile0, _ptr(out), out_stride0, M1, N1,
+        gate_scale, up_scale, inv_out_scale, _stream(stream)))
+
+
+def scale_f32(buf, n, scale, stream=None):
+    _check(load_library().iree_amd_uk_scale_f32(_ptr(buf), n, scale, _stream(stream)))
+
+
 # ---------------------------------------------------------------------------
 # The reference's end-to-end chain: pack LHS, pack RHS (inner+outer transposed),
 # [pack accumulator], mmt4d, unpack
@@ -216,3 +227,57 @@ def matmul_data_tiled(a, b, c, M, N, K, mmt4d_type, *, accumulate=False,
     mmt4d(ws["lhs"], ws["rhs"], ws["out"], M1, N1, K1, M0, N0, K0, mm_flags)
     unpack(ws["out"], c, M1, N1, M0, N0, M, N, out_type)
     return ws
+
+
+class Fp8Mlp:
+    """Llama-style MLP block ``y = (silu(x Wg^T) * (x Wu^T)) Wd^T`` on fp8 e4m3
+    operands with per-tensor f32 scales, as the chain of dispatches the
+    reference's patterns give (gate and up fused horizontally into one matmul,
+    compiler/src/iree/compiler/GlobalOptimization/FuseSiluHorizontalMatmul.cpp:113-140):
+
+        quantize x -> pack LHS -> mmt4d [gate|up] -> silu*up -> fp8 LHS tiles
+        -> mmt4d down -> unpack -> scale
+
+    Weights arrive as e4m3 bytes, row-major ``[N][K]`` (the transpose_b form),
+    and are packed once into right-hand-side tiles 32x16. ``sx``/``sh`` are the
+    static activation scales (value = code * scale), ``sg``/``su``/``sd`` the
+    weight scales. M, hidden and ffn must be multiples of 32.
+    """
+
+    def __init__(self, hidden, ffn, wg_q, wu_q, wd_q, sg, su, sd, sx, sh, max_tokens):
+        if hidden % 32 or ffn % 32 or max_tokens % 32:
+            raise ValueError("hidden, ffn and max_tokens must be multiples of 32")
+        self.hidden, self.ffn, self.max_tokens = hidden, ffn, max_tokens
+        self.sg, self.su, self.sd, self.sx, self.sh = sg, su, sd, sx, sh
+        dev = wg_q.device
+        u8 = torch.uint8
+        t = F.PACK_TYPE_I8I8
+        self.wgu = torch.empty(2 * ffn * hidden, dtype=u8, device=dev)
+        F1, H1 = ffn // 32, hidden // 32
+        # gate tiles occupy outer rows [0, F1), up tiles [F1, 2 F1)
+        pack(wg_q, self.wgu, ffn, hidden, F1, hidden // 16, 32, 16, 0, t)
+        pack(wu_q, self.wgu, ffn, hidden, F1, hidden // 16, 32, 16, 0, t,
+             out_offset=ffn * hidden)
+        self.wd = torch.empty(hidden * ffn, dtype=u8, device=dev)
+        pack(wd_q, self.wd, hidden, ffn, H1, ffn // 16, 32, 16, 0, t)
+        M = max_tokens
+        self.xq = torch.empty(M * hidden, dtype=u8, device=dev)
+        self.x_tiles = torch.empty(M * hidden, dtype=u8, device=dev)
+        self.acc = torch.empty(M * 2 * ffn, dtype=torch.float32, device=dev)
+        self.h_tiles = torch.empty(M * ffn, dtype=u8, device=dev)
+        self.acc2 = torch.empty(M * hidden, dtype=torch.float32, device=dev)
+
+    def __call__(self, x_f16, y_f32, M):
+        hidden, ffn = self.hidden, self.ffn
+        if M % 32 or M > self.max_tokens:
+            raise ValueError("M must be a multiple of 32 within max_tokens")
+        M1, F1, H1 = M // 32, ffn // 32, hidden // 32
+        mm = F.MMT4D_TYPE_F8E4M3F8E4M3F32
+        quantize_f16_to_f8e4m3(x_f16, self.xq, M * hidden, 1.0 / self.sx)
+        pack(self.xq, self.x_tiles, M, hidden, M1, hidden // 16, 32, 16, 0, F.PACK_TYPE_I8I8)
+        mmt4d(self.x_tiles, self.wgu, self.acc, M1, 2 * F1, hidden // 16, 32, 32, 16, mm)
+        silu_mul_quantize_tiled(self.acc, 2 * F1 * 1024, 0, F1, self.h_tiles, ffn * 32, M1, F1,
+                                self.sx * self.sg, self.sx * self.su, 1.0 / self.sh)
+        mmt4d(self.h_tiles, self.wd, self.acc2, M1, H1, ffn // 16, 32, 32, 16, mm)
+        unpack(self.acc2, y_f32, M1, H1, 32, 32, M, hidden, F.UNPACK_TYPE_F32F32)
+        scale_f32(y_f32, M * hidden, self.sh * self.sd)

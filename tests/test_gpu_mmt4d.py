@@ -42,11 +42,12 @@ def test_reference_test_matrix_bit_exact(uk, cuda, type_flag):
 
 MFMA_TILES = [(F.MMT4D_TYPE_S8S8S32, 32, 32, 16), (F.MMT4D_TYPE_S8S8S32, 32, 32, 32),
               (F.MMT4D_TYPE_F16F16F32, 32, 32, 8), (F.MMT4D_TYPE_F16F16F32, 32, 32, 16),
-              (F.MMT4D_TYPE_BF16BF16F32, 32, 32, 8), (F.MMT4D_TYPE_BF16BF16F32, 32, 32, 16)]
+              (F.MMT4D_TYPE_BF16BF16F32, 32, 32, 8), (F.MMT4D_TYPE_BF16BF16F32, 32, 32, 16),
+              (F.MMT4D_TYPE_F8E4M3F8E4M3F32, 32, 32, 16)]
 # outer shapes chosen to hit: single tile, ragged macro tiles in M and N, K
 # tails that are not whole LDS stages, both macro-tile variants, > 8 XCD slices
 MFMA_SHAPES = [(1, 1, 2), (1, 1, 8), (3, 2, 6), (5, 7, 10), (9, 4, 18), (8, 8, 8),
-               (17, 9, 4), (4, 33, 2), (20, 20, 12)]
+               (17, 9, 4), (4, 33, 2), (20, 20, 12), (9, 17, 28), (2, 3, 44)]
 
 
 @pytest.mark.parametrize("type_flag,M0,N0,K0", MFMA_TILES)
