@@ -29,6 +29,7 @@ import numpy as np  # noqa: E402
 
 PEAK_F16_TFLOPS = 2500.0   # MI355X dense f16 MFMA
 PEAK_I8_TOPS = 5000.0      # MI355X dense int8 MFMA
+PEAK_FP8_TFLOPS = 5000.0   # MI355X dense fp8 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE
@@ -290,6 +291,56 @@ def extras(args, torch, iree_amd, F, synth, lhs, rhs, out):
         ex[f"dequant_matmul_i4_m{Mq}_gbs"] = round(qbytes / t / 1e9, 1)
         ex[f"dequant_matmul_i4_m{Mq}_us"] = round(t * 1e6, 2)
     ex["dequant_matmul_i4_m1_frac_of_hbm_peak"] = round(ex["dequant_matmul_i4_m1_gbs"] / PEAK_HBM_GBS, 4)
+    del wq, sq, zq
+
+    # fp8 e4m3 x e4m3 -> f32 at 4096^3, tile 32x32x16 (codes of N(0,1) values)
+    K1 = size // 16
+    g = torch.Generator(device="cuda")
+    g.manual_seed(5)
+    src = torch.randn(size * size, generator=g, device="cuda", dtype=torch.float16)
+    l8 = torch.empty(size * size, dtype=torch.uint8, device="cuda")
+    r8 = torch.empty(size * size, dtype=torch.uint8, device="cuda")
+    iree_amd.quantize_f16_to_f8e4m3(src, l8, size * size, 1.0)
+    iree_amd.quantize_f16_to_f8e4m3(src.flip(0), r8, size * size, 0.5)
+    o8 = torch.empty(M1 * N1 * 1024, dtype=torch.float32, device="cuda")
+    _, t = gpu_time(torch, lambda: iree_amd.mmt4d(l8, r8, o8, M1, N1, K1, 32, 32, 16,
+                                                  F.MMT4D_TYPE_F8E4M3F8E4M3F32), steps, warm)
+    ex["mmt4d_fp8_tflops"] = round(flops / t / 1e12, 2)
+    ex["mmt4d_fp8_frac_of_peak"] = round(flops / t / 1e12 / PEAK_FP8_TFLOPS, 4)
+    del src, l8, r8, o8
+
+    # Llama-style MLP block on fp8 operands: 2048 tokens, hidden 4096, ffn 14336
+    # (weights N(0, 0.02) quantised per tensor with scale maxabs/448; static
+    # activation scales calibrated on this input, outside the timed region).
+    Mt, Hd, Ff = 2048, 4096, 14336
+    xm = torch.randn(Mt * Hd, generator=g, device="cuda", dtype=torch.float16)
+    wts, scales = [], []
+    for n_el in (Ff * Hd, Ff * Hd, Hd * Ff):
+        w = torch.randn(n_el, generator=g, device="cuda", dtype=torch.float32) * 0.02
+        sc = float(w.abs().max()) / 448.0
+        wq8 = torch.empty(n_el, dtype=torch.uint8, device="cuda")
+        iree_amd.quantize_f16_to_f8e4m3(w.to(torch.float16), wq8, n_el, 1.0 / sc)
+        wts.append(wq8)
+        scales.append(sc)
+        del w
+    sx = float(xm.float().abs().max()) / 448.0
+    mlp = iree_amd.Fp8Mlp(Hd, Ff, wts[0], wts[1], wts[2], scales[0], scales[1], scales[2], sx, 1.0,
+                          max_tokens=Mt)
+    del wts
+    ym = torch.empty(Mt * Hd, dtype=torch.float32, device="cuda")
+    # calibrate the scale of h = silu(g) * u from one pass with unit scale
+    mlp(xm, ym, Mt)
+    gu = mlp.acc.view(Mt // 32, 2 * Ff // 32, 32, 32)
+    gate = gu[:, :Ff // 32] * (sx * scales[0])
+    up = gu[:, Ff // 32:] * (sx * scales[1])
+    mlp.sh = float((torch.nn.functional.silu(gate) * up).abs().max()) / 448.0
+    del gu, gate, up
+    _, t = gpu_time(torch, lambda: mlp(xm, ym, Mt), max(5, steps // 4), 2)
+    mlp_flops = 3 * 2.0 * Mt * Hd * Ff
+    ex["mlp_fp8_m2048_tflops"] = round(mlp_flops / t / 1e12, 2)
+    ex["mlp_fp8_m2048_frac_of_peak"] = round(mlp_flops / t / 1e12 / PEAK_FP8_TFLOPS, 4)
+    ex["mlp_fp8_m2048_ms"] = round(t * 1e3, 3)
+    assert bool(torch.isfinite(ym).all()), "fp8 MLP produced non-finite values"
     return ex
 
 
