@@ -46,7 +46,7 @@ def parse_args():
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary measurements")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--only", default="", help="run only the named kernel in a loop (for profilers): "
-                    "mmt4d_f16 | mmt4d_i8 | pack | unpack | gemv")
+                    "mmt4d_f16 | mmt4d_i8 | mmt4d_fp8 | pack | unpack | dequant_i4 | copy")
     return ap.parse_args()
 
 
@@ -359,12 +359,52 @@ def run_only(args, torch, iree_amd, F, synth, mm_step):
     elif args.only in ("pack", "unpack"):
         R, Cc, T0, T1 = 8191, 5001, 32, 16
         O0, O1 = -(-R // T0), -(-Cc // T1)
-        x = torch.from_numpy(synth.uniform_pm1_f16(1, R * Cc).view(np.int16)).cuda()
-        p = torch.zeros(O0 * O1 * T0 * T1, dtype=torch.int16, device="cuda")
-        if args.only == "pack":
-            fn = lambda: iree_amd.pack(x, p, R, Cc, O0, O1, T0, T1, 0, F.PACK_TYPE_F16F16)  # noqa: E731
-        else:
-            fn = lambda: iree_amd.unpack(p, x, O0, O1, T0, T1, R, Cc, F.UNPACK_TYPE_F16F16)  # noqa: E731
+        # four buffer sets (656 MB), rotated, so that the 256 MiB last-level
+        # cache does not serve the reads
+        x_host = synth.uniform_pm1_f16(1, R * Cc).view(np.int16)
+        xs = [torch.from_numpy(x_host).cuda() for _ in range(4)]
+        ps = [torch.zeros(O0 * O1 * T0 * T1, dtype=torch.int16, device="cuda") for _ in range(4)]
+        st = {"i": 0}
+
+        def fn():
+            k = st["i"] % 4
+            st["i"] += 1
+            if args.only == "pack":
+                iree_amd.pack(xs[k], ps[k], R, Cc, O0, O1, T0, T1, 0, F.PACK_TYPE_F16F16)
+            else:
+                iree_amd.unpack(ps[k], xs[k], O0, O1, T0, T1, R, Cc, F.UNPACK_TYPE_F16F16)
+    elif args.only == "mmt4d_fp8":
+        size = 4096
+        M1 = N1 = size // 32
+        K1 = size // 16
+        src = torch.from_numpy(synth.normal_f16(5, size * size).view(np.int16)).cuda()
+        l8 = torch.empty(size * size, dtype=torch.uint8, device="cuda")
+        r8 = torch.empty(size * size, dtype=torch.uint8, device="cuda")
+        iree_amd.quantize_f16_to_f8e4m3(src, l8, size * size, 1.0)
+        iree_amd.quantize_f16_to_f8e4m3(src.flip(0), r8, size * size, 0.5)
+        o8 = torch.empty(M1 * N1 * 1024, dtype=torch.float32, device="cuda")
+        fn = lambda: iree_amd.mmt4d(l8, r8, o8, M1, N1, K1, 32, 32, 16, F.MMT4D_TYPE_F8E4M3F8E4M3F32)  # noqa: E731
+    elif args.only == "dequant_i4":
+        Nq, Kq, gs = 14336, 4096, 128
+        G = Kq // gs
+        wq = [torch.from_numpy(synth.uniform_u4_packed(10 + i, Nq * Kq)).cuda() for i in range(10)]
+        sq = torch.from_numpy(synth.uniform_f16(30, Nq * G, 0.005, 0.02).view(np.int16)).cuda()
+        zq = torch.from_numpy(synth.uniform_u4_packed(31, Nq * G)).cuda()
+        xq = torch.from_numpy(synth.normal_f16(41, Kq).view(np.int16)).cuda()
+        oq = torch.empty(Nq, dtype=torch.int16, device="cuda")
+        st = {"i": 0}
+
+        def fn():
+            k = st["i"] % 10
+            st["i"] += 1
+            iree_amd.dequant_matmul_i4(xq, wq[k], sq, zq, oq, 1, Nq, Kq, gs,
+                                       F.DEQUANT_MATMUL_ZP_U4 | F.DEQUANT_MATMUL_W_TILED)
+    elif args.only == "copy":
+        # a plain read-once / write-once kernel of known size (256 MiB each way):
+        # the yardstick that the FETCH_SIZE / WRITE_SIZE counters are scaled by
+        n = 64 * 1024 * 1024
+        buf = torch.ones(n, dtype=torch.float32, device="cuda")
+        fn = lambda: iree_amd.scale_f32(buf, n, 1.0)  # noqa: E731
     else:
         raise SystemExit(f"unknown --only {args.only}")
     wall, per_launch = gpu_time(torch, fn, args.steps, args.warmup)

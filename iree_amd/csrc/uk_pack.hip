@@ -299,6 +299,7 @@ struct Pow2Args {
   int64_t padded_rows;
   uint32_t chunks_per_row, padded_chunks_per_row;
   int log2_tile_rows, log2_cpr;
+  uint32_t blocks_x, blocks_y;   // logical grid; launched as blocks_x * blocks_y workgroups
   uint64_t padding;
 };
 
@@ -309,11 +310,24 @@ __global__ __launch_bounds__(kStreamThreads) void stream_pow2_kernel(Pow2Args a)
   typedef typename Chunk<ES>::aligned_t mat_vec_t;
   const uint32_t lane = threadIdx.x & 63;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const uint32_t j0 = (blockIdx.x * 4 + wave) * kBlockChunks;
+  // Workgroup ids go round-robin over the 8 XCDs, each with its own L2. Give
+  // XCD x the x-th contiguous slice of the row-major block sequence, so that
+  // blocks that share a cache line (rows are rarely line-aligned) meet in one L2.
+  uint32_t bx, by;
+  {
+    constexpr uint32_t kXcds = 8;
+    const uint32_t total = a.blocks_x * a.blocks_y;
+    const uint32_t per = total / kXcds, rem = total % kXcds;
+    const uint32_t xcd = blockIdx.x % kXcds, idx = blockIdx.x / kXcds;
+    const uint32_t logical = xcd * per + (xcd < rem ? xcd : rem) + idx;
+    by = logical / a.blocks_x;
+    bx = logical - by * a.blocks_x;
+  }
+  const uint32_t j0 = (bx * 4 + wave) * kBlockChunks;
   const uint32_t col_limit = kPack ? a.padded_chunks_per_row : a.chunks_per_row;
   if (j0 >= col_limit) return;
   const int64_t row_limit = kPack ? a.padded_rows : a.m_size0;
-  const int64_t r0 = (int64_t)blockIdx.y * kRows;
+  const int64_t r0 = (int64_t)by * kRows;
   if (r0 >= row_limit) return;
   const uint32_t tile_rows = 1u << a.log2_tile_rows, cpr = 1u << a.log2_cpr;
   const uint32_t jl = lane & 7, rl = lane >> 3;
@@ -387,7 +401,7 @@ bool pow2_eligible(const StreamArgs& a, int es) {
   const int64_t panels = rows / a.tile_rows + 2, cols = kBlockChunks / a.cpr + 2;
   if (a.t_stride_row_bytes * panels + a.t_stride_col_bytes * cols + (1ll << 20) >= (1ll << 31)) return false;
   if ((int64_t)a.tile_rows * a.cpr * 16 >= (1ll << 20)) return false;
-  return ceil_div(a.padded_rows, rows) <= 65535 && ceil_div(a.m_size0, rows) <= 65535;
+  return true;
 }
 
 template <int ES, bool kPack>
@@ -404,8 +418,9 @@ int launch_stream_pow2(const StreamArgs& a, hipStream_t s) {
   const int64_t rows = kPack ? a.padded_rows : a.m_size0;
   const int64_t bx = ceil_div(cols, 4 * kBlockChunks);
   const int64_t by = ceil_div(rows, kBlockRows * kStreamUnroll);
-  if (bx > 0x7FFFFFFF || by > 65535 || bx < 1 || by < 1) return IREE_AMD_UK_STATUS_NOT_FOUND;
-  hipLaunchKernelGGL((stream_pow2_kernel<ES, kPack>), dim3((unsigned)bx, (unsigned)by), dim3(kStreamThreads), 0, s, p);
+  if (bx < 1 || by < 1 || bx * by > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  p.blocks_x = (uint32_t)bx; p.blocks_y = (uint32_t)by;
+  hipLaunchKernelGGL((stream_pow2_kernel<ES, kPack>), dim3((unsigned)(bx * by)), dim3(kStreamThreads), 0, s, p);
   return check_hip(hipGetLastError(), "stream_pow2 launch");
 }
 
