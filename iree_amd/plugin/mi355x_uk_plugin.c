@@ -18,12 +18,18 @@
  * 252-274): field for field the reference's own iree_uk_*_params_t
  * (REF runtime/src/iree/builtins/ukernel/mmt4d_internal.h:14-32,
  * pack_internal.h:12-30, unpack_internal.h:12-29), which is also the layout of
- * iree_amd_uk_*_params_t. The import therefore passes the pointer straight
- * through. Buffers of a local-CPU HAL device are host memory, so the
- * host-pointer entry points are used (they stage through device memory).
+ * iree_amd_uk_*_params_t. Buffers of a local-CPU HAL device are host memory,
+ * so the host-pointer entry points are used (they stage through device memory).
  *
- * Imports are served under the names the compiler emits (iree_uk_*) and under
- * the mi355x_uk_* aliases used by example.mlir next to this file.
+ * Two spellings of each import, because results come first in the struct:
+ *   mi355x_uk_{mmt4d,pack,unpack}  the op has only its tensor result (which
+ *       bufferisation removes), as in example.mlir next to this file and in
+ *       REF samples/custom_dispatch/cpu/plugin/system_ukernel.mlir:50-62: the
+ *       struct IS the parameter struct.
+ *   iree_uk_{mmt4d,pack,unpack}    the op as the llvm-cpu lowering builds it,
+ *       with an extra i32 result (REF CPULowerToUKernels.cpp:157-168): the
+ *       struct is {int32 result; <padding to 8>; parameter struct}; the import
+ *       stores 0 into the result.
  *
  * Load parameters (--executable_plugin=path?key=value pairs reach load()):
  *   uk_library=<path>   the MI355X microkernel library; default: the
@@ -77,6 +83,29 @@ static int import_unpack(void* params, void* context, void* reserved) {
   (void)reserved;
   mi355x_plugin_t* plugin = (mi355x_plugin_t*)context;
   return report(plugin, "unpack", plugin->unpack((const iree_amd_uk_unpack_params_t*)params));
+}
+
+/* The llvm-cpu form: a leading i32 result, then the parameters at the next
+ * 8-byte boundary (the first parameter is a pointer). */
+typedef struct with_result_t {
+  int32_t result;
+  int32_t padding;
+  char params[];
+} with_result_t;
+static int import_mmt4d_r(void* params, void* context, void* reserved) {
+  with_result_t* w = (with_result_t*)params;
+  w->result = 0;
+  return import_mmt4d(w->params, context, reserved);
+}
+static int import_pack_r(void* params, void* context, void* reserved) {
+  with_result_t* w = (with_result_t*)params;
+  w->result = 0;
+  return import_pack(w->params, context, reserved);
+}
+static int import_unpack_r(void* params, void* context, void* reserved) {
+  with_result_t* w = (with_result_t*)params;
+  w->result = 0;
+  return import_unpack(w->params, context, reserved);
 }
 
 static int key_is(const iree_amd_hal_plugin_string_view_t* key, const char* name) {
@@ -158,8 +187,8 @@ static const struct {
   const char* name;
   iree_amd_hal_plugin_import_fn_t fn;
 } kImports[] = {
-    {"iree_uk_mmt4d", import_mmt4d},     {"iree_uk_pack", import_pack},
-    {"iree_uk_unpack", import_unpack},   {"mi355x_uk_mmt4d", import_mmt4d},
+    {"iree_uk_mmt4d", import_mmt4d_r},   {"iree_uk_pack", import_pack_r},
+    {"iree_uk_unpack", import_unpack_r}, {"mi355x_uk_mmt4d", import_mmt4d},
     {"mi355x_uk_pack", import_pack},     {"mi355x_uk_unpack", import_unpack},
 };
 

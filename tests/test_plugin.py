@@ -138,7 +138,7 @@ def test_load_resolve_unload_protocol(host):
     assert resolution == 1                                   # one optional import missing
     assert all(fns[:5]) and fns[5] is None
     assert all(c == self_ptr.value for c in ctxs[:5])
-    assert fns[0] == fns[3]                                  # alias of the same import
+    assert fns[0] != fns[3]                                  # two parameter layouts, see the GPU test
     # a required unknown import: NOT_FOUND, the known ones still resolved
     status, resolution, fns, _ = host.resolve(plugin, self_ptr, [b"iree_uk_mmt4d", b"other_symbol"])
     assert status == 5 and fns[0] and fns[1] is None
@@ -162,9 +162,19 @@ def test_imports_run_pack_mmt4d_unpack_on_host_buffers(host, uk, cuda):
     status, self_ptr = host.load(plugin, [(b"uk_library", _lib.library_path().encode())])
     assert status == 0
     status, _, fns, ctxs = host.resolve(plugin, self_ptr,
-                                        [b"iree_uk_pack", b"iree_uk_mmt4d", b"iree_uk_unpack"])
+                                        [b"mi355x_uk_pack", b"iree_uk_mmt4d", b"mi355x_uk_unpack"])
     assert status == 0
-    pack_fn, mmt4d_fn, unpack_fn = (IMPORT(f) for f in fns)
+    pack_fn, mmt4d_r_fn, unpack_fn = (IMPORT(f) for f in fns)
+
+    class Mmt4dWithResult(C.Structure):      # the llvm-cpu lowering's form: i32 result first
+        _fields_ = [("result", C.c_int32), ("params", _lib.Mmt4dParams)]
+    assert Mmt4dWithResult.params.offset == 8
+
+    def mmt4d_fn(addr, ctx, reserved):
+        w = Mmt4dWithResult(-1, C.cast(addr, C.POINTER(_lib.Mmt4dParams)).contents)
+        rc = mmt4d_r_fn(C.addressof(w), ctx, reserved)
+        assert w.result == 0
+        return rc
     M, N, K = 100, 70, 150
     M0, N0, K0 = 32, 32, 16
     M1, N1, K1 = -(-M // M0), -(-N // N0), -(-K // K0)
