@@ -165,8 +165,8 @@ __device__ __forceinline__ void tile_coord(int bid, int tiles_m, int tiles_n,
 // kSync K-steps that lie kAhead = kRing - kSync steps ahead, so up to kAhead
 // K-steps of loads are in flight behind the one being multiplied. Operand
 // fragments are read from LDS one K-step ahead of the MFMAs that use them.
-template <typename Cfg, int WM, int WN, bool kHalfK0, int kRing, int kSync>
-__global__ __launch_bounds__(kThreads) void mmt4d_mfma_kernel(MfmaArgs a) {
+template <typename Cfg, int WM, int WN, bool kHalfK0, int kRing, int kSync, int kWavesPerSimd = 1>
+__global__ __launch_bounds__(kThreads, kWavesPerSimd) void mmt4d_mfma_kernel(MfmaArgs a) {
   typedef typename Cfg::frag_t frag_t;
   typedef typename Cfg::acc_t acc_t;
   typedef typename Cfg::out_t out_t;
@@ -386,7 +386,7 @@ __global__ __launch_bounds__(kThreads) void mmt4d_mfma_kernel(MfmaArgs a) {
     }
 }
 
-template <typename Cfg, int WM, int WN, bool kHalfK0, int kRing, int kSync>
+template <typename Cfg, int WM, int WN, bool kHalfK0, int kRing, int kSync, int kWavesPerSimd = 1>
 int launch_variant(const MfmaArgs& a0, hipStream_t s) {
   MfmaArgs a = a0;
   constexpr int TM = 2 * WM, TN = 2 * WN;
@@ -396,7 +396,7 @@ int launch_variant(const MfmaArgs& a0, hipStream_t s) {
   if (blocks > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
   constexpr int lds_bytes = kRing * (TM + TN) * Cfg::kSub * kPieceBytes;
   static_assert(lds_bytes <= 160 * 1024, "LDS ring exceeds 160 KiB");
-  auto kernel = mmt4d_mfma_kernel<Cfg, WM, WN, kHalfK0, kRing, kSync>;
+  auto kernel = mmt4d_mfma_kernel<Cfg, WM, WN, kHalfK0, kRing, kSync, kWavesPerSimd>;
   static bool attr_set = false;  // benign race: the call is idempotent
   if (!attr_set) {
     UK_RETURN_IF_HIP(hipFuncSetAttribute((const void*)kernel,

@@ -26,9 +26,9 @@ namespace {
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 // 128-bit access to memory that is only element-aligned.
 template <int ES> struct Chunk;
-template <> struct Chunk<1> { typedef u32x4 aligned_t __attribute__((aligned(1))); };
-template <> struct Chunk<2> { typedef u32x4 aligned_t __attribute__((aligned(2))); };
-template <> struct Chunk<4> { typedef u32x4 aligned_t __attribute__((aligned(4))); };
+template <> struct Chunk<1> { typedef u32x4 aligned_t __attribute__((aligned(1))); typedef uint8_t elem_t; };
+template <> struct Chunk<2> { typedef u32x4 aligned_t __attribute__((aligned(2))); typedef uint16_t elem_t; };
+template <> struct Chunk<4> { typedef u32x4 aligned_t __attribute__((aligned(4))); typedef uint32_t elem_t; };
 
 struct PackArgs {
   const char* in;   // matrix (pack source / unpack destination), offset applied
@@ -424,6 +424,107 @@ int launch_stream_pow2(const StreamArgs& a, hipStream_t s) {
   return check_hip(hipGetLastError(), "stream_pow2 launch");
 }
 
+//---------------------------------------------------------------------------
+// Pack with transposed inner tiles (the right-hand side of a matmul given as
+// B[K][N]: every tile is stored column by column). A 16-byte chunk of the tiled
+// buffer is then CE = 16/ES consecutive matrix ROWS of one matrix column. One
+// thread builds one such chunk from CE element-sized loads and stores it with
+// one 128-bit store. Lanes of a wave take 64 consecutive matrix columns, so
+// every load instruction reads 64 consecutive elements of a row and the stores
+// of a wave are whole tiles (or whole rows of chunks of a tile); a wave walks
+// kTransUnroll consecutive row groups so that enough loads are in flight.
+//---------------------------------------------------------------------------
+constexpr int kTransUnroll = 4;
+
+struct TransArgs {
+  const char* mat;
+  char* tiled;
+  int64_t m_size0, m_size1, m_pitch_bytes;
+  int64_t row_groups;            // outer_rows * groups_per_tile
+  int64_t padded_cols;           // outer_cols * tile_cols
+  int64_t t_stride_orow_bytes, t_stride_ocol_bytes;
+  int tile_rows, tile_cols;      // matrix orientation: tile_rows = stored inner size
+  int groups_per_tile;           // tile_rows / CE
+  FastDiv by_tile_cols, by_groups;
+  uint32_t blocks_x, blocks_y;
+  uint64_t padding;
+};
+
+template <int ES>
+__global__ __launch_bounds__(256) void pack_transpose_kernel(TransArgs a) {
+  constexpr int CE = 16 / ES;
+  typedef typename Chunk<ES>::elem_t elem_t;
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  // Same XCD-compact block order as the streaming kernels.
+  uint32_t bx, by;
+  {
+    constexpr uint32_t kXcds = 8;
+    const uint32_t total = a.blocks_x * a.blocks_y;
+    const uint32_t per = total / kXcds, rem = total % kXcds;
+    const uint32_t xcd = blockIdx.x % kXcds, idx = blockIdx.x / kXcds;
+    const uint32_t logical = xcd * per + (xcd < rem ? xcd : rem) + idx;
+    by = logical / a.blocks_x;
+    bx = logical - by * a.blocks_x;
+  }
+  const int64_t c = (int64_t)bx * 64 + lane;                 // matrix column
+  const int64_t g0 = ((int64_t)by * 4 + wave) * kTransUnroll;  // first row group of this wave
+  if (g0 >= a.row_groups) return;
+  const bool col_in_tiles = c < a.padded_cols;
+  // where column c lands: tile column and row of the (transposed) tile
+  const uint32_t cc = col_in_tiles ? (uint32_t)c : 0;
+  const uint32_t ocol = a.by_tile_cols.div(cc), d2 = cc - ocol * a.tile_cols;
+  char* out_col = a.tiled + (int64_t)ocol * a.t_stride_ocol_bytes + (int64_t)d2 * a.tile_rows * ES;
+  const elem_t pad = (elem_t)a.padding;
+  const bool interior = (int64_t)(bx + 1) * 64 <= a.m_size1 &&
+                        (g0 + kTransUnroll) * CE <= a.m_size0 && g0 + kTransUnroll <= a.row_groups;
+  elem_t v[kTransUnroll][CE];
+  if (interior) {
+    const char* src = a.mat + g0 * CE * a.m_pitch_bytes + c * ES;
+#pragma unroll
+    for (int u = 0; u < kTransUnroll; ++u)
+#pragma unroll
+      for (int i = 0; i < CE; ++i) v[u][i] = *(const elem_t*)(src + (int64_t)(u * CE + i) * a.m_pitch_bytes);
+  } else {
+#pragma unroll
+    for (int u = 0; u < kTransUnroll; ++u)
+#pragma unroll
+      for (int i = 0; i < CE; ++i) {
+        const int64_t r = (g0 + u) * CE + i;
+        v[u][i] = (r < a.m_size0 && c < a.m_size1) ? *(const elem_t*)(a.mat + r * a.m_pitch_bytes + c * ES) : pad;
+      }
+  }
+  if (!col_in_tiles) return;
+#pragma unroll
+  for (int u = 0; u < kTransUnroll; ++u) {
+    const int64_t g = g0 + u;
+    if (g >= a.row_groups) break;
+    int64_t orow;
+    uint32_t grp;
+    if (g < 0x7FFFFFFF) {
+      orow = a.by_groups.div((uint32_t)g);
+      grp = (uint32_t)g - (uint32_t)orow * a.groups_per_tile;
+    } else {
+      orow = g / a.groups_per_tile;
+      grp = (uint32_t)(g - orow * a.groups_per_tile);
+    }
+    union { elem_t e[CE]; u32x4 vec; } chunk;
+#pragma unroll
+    for (int i = 0; i < CE; ++i) chunk.e[i] = v[u][i];
+    *(u32x4*)(out_col + orow * a.t_stride_orow_bytes + (int64_t)grp * 16) = chunk.vec;
+  }
+}
+
+template <int ES>
+int launch_pack_transpose(TransArgs a, hipStream_t s) {
+  const int64_t bx = ceil_div(a.padded_cols, (int64_t)64);
+  const int64_t by = ceil_div(a.row_groups, (int64_t)(4 * kTransUnroll));
+  if (bx < 1 || by < 1 || bx * by > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  a.blocks_x = (uint32_t)bx; a.blocks_y = (uint32_t)by;
+  hipLaunchKernelGGL((pack_transpose_kernel<ES>), dim3((unsigned)(bx * by)), dim3(256), 0, s, a);
+  return check_hip(hipGetLastError(), "pack_transpose launch");
+}
+
 bool stream_eligible(int es, int64_t m_stride1, int transpose_inner, int64_t tile_rows,
                      int64_t tile_cols, int64_t outer_cols, int64_t m_size1, const void* tiled,
                      int64_t t_stride0, int64_t tile_elems) {
@@ -521,6 +622,32 @@ int launch_pack(const iree_amd_uk_pack_params_t& p, hipStream_t s) {
     int st = es == 1 ? launch_pack_stream<1>(a, s)
            : es == 2 ? launch_pack_stream<2>(a, s)
                      : launch_pack_stream<4>(a, s);
+    if (st != IREE_AMD_UK_STATUS_NOT_FOUND) return st;
+  }
+
+  // Transposed inner tiles whose stored rows are whole 16-byte chunks.
+  const int ce = 16 / es;
+  if (ti && p.in_stride1 == 1 && p.out_size3 > 0 && p.out_size3 % ce == 0 && p.out_size2 > 0 &&
+      ((uintptr_t)out % 16) == 0 && (p.out_stride0 * es) % 16 == 0 && (tile_elems * es) % 16 == 0 &&
+      p.in_size1 < (1ll << 31) && (to ? p.out_size0 : p.out_size1) * p.out_size2 < (1ll << 31)) {
+    TransArgs a;
+    a.mat = in; a.tiled = out;
+    a.m_size0 = p.in_size0; a.m_size1 = p.in_size1; a.m_pitch_bytes = p.in_stride0 * es;
+    a.tile_rows = (int)p.out_size3; a.tile_cols = (int)p.out_size2;
+    a.groups_per_tile = a.tile_rows / ce;
+    const int64_t outer_rows = to ? p.out_size1 : p.out_size0;
+    const int64_t outer_cols = to ? p.out_size0 : p.out_size1;
+    a.row_groups = outer_rows * a.groups_per_tile;
+    a.padded_cols = outer_cols * a.tile_cols;
+    a.t_stride_orow_bytes = (to ? tile_elems : p.out_stride0) * es;
+    a.t_stride_ocol_bytes = (to ? p.out_stride0 : tile_elems) * es;
+    a.by_tile_cols = make_fastdiv((uint32_t)a.tile_cols);
+    a.by_groups = make_fastdiv((uint32_t)a.groups_per_tile);
+    a.padding = p.padding_value;
+    a.blocks_x = a.blocks_y = 0;
+    int st = es == 1 ? launch_pack_transpose<1>(a, s)
+           : es == 2 ? launch_pack_transpose<2>(a, s)
+                     : launch_pack_transpose<4>(a, s);
     if (st != IREE_AMD_UK_STATUS_NOT_FOUND) return st;
   }
 

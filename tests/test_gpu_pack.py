@@ -75,6 +75,29 @@ def test_streaming_shapes_with_ragged_edges(uk, cuda, type_flag, t0, t1, rows, c
             assert np.array_equal(gpucase.run_unpack(ucase), ucase.run_oracle()), (to,)
 
 
+@pytest.mark.parametrize("type_flag,tr,tc,rows,cols", [
+    (F.PACK_TYPE_F16F16, 8, 32, 1001, 333),    # f16 right-hand side: K0 = 8 rows x N0 = 32 columns
+    (F.PACK_TYPE_F16F16, 16, 32, 200, 95),     # two 16-byte row groups per tile
+    (F.PACK_TYPE_I8I8, 16, 32, 1003, 129),
+    (F.PACK_TYPE_I8I8, 32, 32, 4096, 64),
+    (F.PACK_TYPE_F32F32, 4, 32, 515, 70),
+    (F.PACK_TYPE_BF16BF16, 24, 5, 123, 77),    # odd tile width, three row groups
+])
+def test_transposing_pack_with_ragged_edges(uk, cuda, type_flag, tr, tc, rows, cols):
+    """Packs with transposed inner tiles (what the right-hand side B[K][N] of a
+    matmul needs): matrix tiles of tr rows x tc columns, stored column by column."""
+    rng = np.random.default_rng(rows + cols)
+    orows, ocols = -(-rows // tr), -(-cols // tc)
+    for to in (0, 1):
+        case = ukref.PackCase(rng, type_flag, orows, ocols, tr, tc, transpose_inner=1,
+                              transpose_outer=to, in_size=(rows, cols))
+        assert np.array_equal(gpucase.run_pack(case), case.run_oracle()), (to,)
+        loose = ukref.PackCase(rng, type_flag, orows, ocols, tr, tc, transpose_inner=1,
+                               transpose_outer=to, in_size=(rows, cols), loose_strides=True,
+                               offsets=True)
+        assert np.array_equal(gpucase.run_pack(loose), loose.run_oracle()), (to, "loose")
+
+
 def test_full_size_f16_8191x5001_pack_unpack_round_trip(uk, cuda):
     """The bandwidth workload at its real size: packed bytes equal the oracle's
     (and the committed SHA-256 produced by the reference library), the padded
