@@ -103,7 +103,8 @@ struct MfmaArgs {
   char* out;
   int64_t lhs_stride_bytes, rhs_stride_bytes, out_stride_bytes;
   int M, N;          // outer tile counts
-  int ksteps;        // number of MFMA K-steps = K * K0 / kMfmaK
+  int ksteps;        // whole MFMA K-steps = K * K0 / kMfmaK
+  int tail_tiles;    // K tiles left over after them (less than one MFMA's worth)
   int tiles_m, tiles_n;  // macro-tile grid
   int accumulate;
 };
@@ -369,6 +370,42 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void mmt4d_mfma_kernel(Mfm
     }
   }
 
+  // K tail: fewer K tiles than one MFMA consumes are left. Their fragments
+  // come straight from global memory, with zeros in the lanes (or lane halves)
+  // that stand for the missing tiles.
+  if (a.tail_tiles > 0) {
+    const int64_t tail_off = (int64_t)T * kBlockBytes;
+    auto tail_frag = [&](const char* block) -> frag_t {
+      const int4v zero = {0, 0, 0, 0};
+      if constexpr (kSub == 1) {
+        // (reached with K0 = half the MFMA extent only: lanes 32..63 hold the second tile)
+        const int4v v = (lane >> 5) < a.tail_tiles ? *(const int4v*)(block + lane * 16) : zero;
+        union { int4v i; frag_t f; } u;
+        u.i = v;
+        return u.f;
+      } else {
+        const int t0 = 2 * (lane >> 5);
+        const char* p = block + (lane >> 5) * 1024 + (lane & 31) * 16;
+        const int4v lo = t0 < a.tail_tiles ? *(const int4v*)p : zero;
+        const int4v hi = t0 + 1 < a.tail_tiles ? *(const int4v*)(p + kPieceStride) : zero;
+        return frag_t{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+      }
+    };
+#pragma unroll
+    for (int x = 0; x < WM; ++x) {
+      int i = i_base + wm * WM + x;
+      i = i < a.M ? i : a.M - 1;
+      fa[0][x] = tail_frag(a.lhs + (int64_t)i * a.lhs_stride_bytes + tail_off);
+    }
+#pragma unroll
+    for (int y = 0; y < WN; ++y) {
+      int j = j_base + wn * WN + y;
+      j = j < a.N ? j : a.N - 1;
+      fb[0][y] = tail_frag(a.rhs + (int64_t)j * a.rhs_stride_bytes + tail_off);
+    }
+    multiply(fa[0], fb[0]);
+  }
+
   // Epilogue. MFMA 32x32 accumulator layout: register v of lane l holds
   // row 8*(v/4) + 4*(l/32) + v%4, column l%32 of the block; one store
   // instruction therefore writes two full 128-byte rows of the tile.
@@ -462,8 +499,9 @@ int launch_mmt4d_mfma(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) {
   mmt4d_type_info(p.flags, &ti);
   const int eb = ti.lhs_bits / 8;
   const int64_t k_elems = p.K * p.K0;
-  // Whole MFMA K-steps only, and every operand block must be 16-byte aligned.
-  if (p.K == 0 || k_elems % sv.mfma_k) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  // Every operand block must be 16-byte aligned. K need not be whole MFMA
+  // steps: the kernel finishes with a partial step.
+  if (p.K == 0) return IREE_AMD_UK_STATUS_NOT_FOUND;
   const char* lhs = (const char*)p.lhs_buffer + p.lhs_offset * eb;
   const char* rhs = (const char*)p.rhs_buffer + p.rhs_offset * eb;
   if (((uintptr_t)lhs | (uintptr_t)rhs) % 16) return IREE_AMD_UK_STATUS_NOT_FOUND;
@@ -477,6 +515,7 @@ int launch_mmt4d_mfma(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) {
   a.out_stride_bytes = p.out_stride0 * ti.out_bytes;
   a.M = (int)p.M; a.N = (int)p.N;
   a.ksteps = (int)(k_elems / sv.mfma_k);
+  a.tail_tiles = (int)((k_elems % sv.mfma_k) / p.K0);
   a.tiles_m = a.tiles_n = 0;
   a.accumulate = (p.flags & IREE_AMD_UK_FLAG_MMT4D_ACCUMULATE) != 0;
   const bool half_k0 = p.K0 * 2 == sv.mfma_k;

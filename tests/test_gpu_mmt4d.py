@@ -47,7 +47,9 @@ MFMA_TILES = [(F.MMT4D_TYPE_S8S8S32, 32, 32, 16), (F.MMT4D_TYPE_S8S8S32, 32, 32,
 # outer shapes chosen to hit: single tile, ragged macro tiles in M and N, K
 # tails that are not whole LDS stages, both macro-tile variants, > 8 XCD slices
 MFMA_SHAPES = [(1, 1, 2), (1, 1, 8), (3, 2, 6), (5, 7, 10), (9, 4, 18), (8, 8, 8),
-               (17, 9, 4), (4, 33, 2), (20, 20, 12), (9, 17, 28), (2, 3, 44)]
+               (17, 9, 4), (4, 33, 2), (20, 20, 12), (9, 17, 28), (2, 3, 44),
+               # K tile counts that are not whole MFMA steps (a partial last step)
+               (2, 3, 1), (3, 2, 7), (9, 4, 19), (4, 5, 21), (2, 2, 3), (1, 2, 23), (8, 8, 13)]
 
 
 @pytest.mark.parametrize("type_flag,M0,N0,K0", MFMA_TILES)
