@@ -48,7 +48,7 @@ def parse_args():
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary measurements")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--only", default="", help="run only the named kernel in a loop (for profilers): "
-                    "mmt4d_f16 | mmt4d_i8 | mmt4d_fp8 | pack | unpack | dequant_i4 | copy")
+                    "mmt4d_f16 | mmt4d_i8 | mmt4d_fp8 | mlp_fp8 | pack | unpack | dequant_i4 | copy")
     return ap.parse_args()
 
 
@@ -201,6 +201,38 @@ def verify_tiles(torch, iree_amd, F, lhs, rhs, out, M1, N1, K1, M0, N0, K0):
             raise SystemExit("bench.py: mmt4d result is outside tolerance; refusing to time it")
 
 
+def make_fp8_mlp(torch, iree_amd):
+    """Llama-style MLP block on fp8 operands: 2048 tokens, hidden 4096, ffn 14336
+    (weights N(0, 0.02) quantised per tensor with scale maxabs/448; static
+    activation scales calibrated on this input, outside any timed region)."""
+    g = torch.Generator(device="cuda")
+    g.manual_seed(6)
+    Mt, Hd, Ff = 2048, 4096, 14336
+    xm = torch.randn(Mt * Hd, generator=g, device="cuda", dtype=torch.float16)
+    wts, scales = [], []
+    for n_el in (Ff * Hd, Ff * Hd, Hd * Ff):
+        w = torch.randn(n_el, generator=g, device="cuda", dtype=torch.float32) * 0.02
+        sc = float(w.abs().max()) / 448.0
+        wq8 = torch.empty(n_el, dtype=torch.uint8, device="cuda")
+        iree_amd.quantize_f16_to_f8e4m3(w.to(torch.float16), wq8, n_el, 1.0 / sc)
+        wts.append(wq8)
+        scales.append(sc)
+        del w
+    sx = float(xm.float().abs().max()) / 448.0
+    mlp = iree_amd.Fp8Mlp(Hd, Ff, wts[0], wts[1], wts[2], scales[0], scales[1], scales[2], sx, 1.0,
+                          max_tokens=Mt)
+    del wts
+    ym = torch.empty(Mt * Hd, dtype=torch.float32, device="cuda")
+    # calibrate the scale of h = silu(g) * u from one pass with unit scale
+    mlp(xm, ym, Mt)
+    gu = mlp.acc.view(Mt // 32, 2 * Ff // 32, 32, 32)
+    gate = gu[:, :Ff // 32] * (sx * scales[0])
+    up = gu[:, Ff // 32:] * (sx * scales[1])
+    mlp.sh = float((torch.nn.functional.silu(gate) * up).abs().max()) / 448.0
+    del gu, gate, up
+    return mlp, xm, ym, Mt, Hd, Ff
+
+
 def extras(args, torch, iree_amd, F, synth, lhs, rhs, out):
     ex = {}
     size = 4096
@@ -311,32 +343,7 @@ def extras(args, torch, iree_amd, F, synth, lhs, rhs, out):
     ex["mmt4d_fp8_frac_of_peak"] = round(flops / t / 1e12 / PEAK_FP8_TFLOPS, 4)
     del src, l8, r8, o8
 
-    # Llama-style MLP block on fp8 operands: 2048 tokens, hidden 4096, ffn 14336
-    # (weights N(0, 0.02) quantised per tensor with scale maxabs/448; static
-    # activation scales calibrated on this input, outside the timed region).
-    Mt, Hd, Ff = 2048, 4096, 14336
-    xm = torch.randn(Mt * Hd, generator=g, device="cuda", dtype=torch.float16)
-    wts, scales = [], []
-    for n_el in (Ff * Hd, Ff * Hd, Hd * Ff):
-        w = torch.randn(n_el, generator=g, device="cuda", dtype=torch.float32) * 0.02
-        sc = float(w.abs().max()) / 448.0
-        wq8 = torch.empty(n_el, dtype=torch.uint8, device="cuda")
-        iree_amd.quantize_f16_to_f8e4m3(w.to(torch.float16), wq8, n_el, 1.0 / sc)
-        wts.append(wq8)
-        scales.append(sc)
-        del w
-    sx = float(xm.float().abs().max()) / 448.0
-    mlp = iree_amd.Fp8Mlp(Hd, Ff, wts[0], wts[1], wts[2], scales[0], scales[1], scales[2], sx, 1.0,
-                          max_tokens=Mt)
-    del wts
-    ym = torch.empty(Mt * Hd, dtype=torch.float32, device="cuda")
-    # calibrate the scale of h = silu(g) * u from one pass with unit scale
-    mlp(xm, ym, Mt)
-    gu = mlp.acc.view(Mt // 32, 2 * Ff // 32, 32, 32)
-    gate = gu[:, :Ff // 32] * (sx * scales[0])
-    up = gu[:, Ff // 32:] * (sx * scales[1])
-    mlp.sh = float((torch.nn.functional.silu(gate) * up).abs().max()) / 448.0
-    del gu, gate, up
+    mlp, xm, ym, Mt, Hd, Ff = make_fp8_mlp(torch, iree_amd)
     _, t = gpu_time(torch, lambda: mlp(xm, ym, Mt), max(5, steps // 4), 2)
     mlp_flops = 3 * 2.0 * Mt * Hd * Ff
     ex["mlp_fp8_m2048_tflops"] = round(mlp_flops / t / 1e12, 2)
@@ -401,6 +408,9 @@ def run_only(args, torch, iree_amd, F, synth, mm_step):
             st["i"] += 1
             iree_amd.dequant_matmul_i4(xq, wq[k], sq, zq, oq, 1, Nq, Kq, gs,
                                        F.DEQUANT_MATMUL_ZP_U4 | F.DEQUANT_MATMUL_W_TILED)
+    elif args.only == "mlp_fp8":
+        mlp, xm, ym, Mt, _, _ = make_fp8_mlp(torch, iree_amd)
+        fn = lambda: mlp(xm, ym, Mt)  # noqa: E731
     elif args.only == "copy":
         # a plain read-once / write-once kernel of known size (256 MiB each way):
         # the yardstick that the FETCH_SIZE / WRITE_SIZE counters are scaled by

@@ -107,6 +107,7 @@ struct MfmaArgs {
   int tail_tiles;    // K tiles left over after them (less than one MFMA's worth)
   int tiles_m, tiles_n;  // macro-tile grid
   int accumulate;
+  int half_k0;       // K0 is half the MFMA's K extent (else the full extent)
 };
 
 __device__ __forceinline__ void load_block_to_lds(const char* gptr, char* lds) {
@@ -166,8 +167,10 @@ __device__ __forceinline__ void tile_coord(int bid, int tiles_m, int tiles_n,
 // kSync K-steps that lie kAhead = kRing - kSync steps ahead, so up to kAhead
 // K-steps of loads are in flight behind the one being multiplied. Operand
 // fragments are read from LDS one K-step ahead of the MFMAs that use them.
-template <typename Cfg, int WM, int WN, bool kHalfK0, int kRing, int kSync, int kWavesPerSimd = 1>
-__global__ __launch_bounds__(kThreads, kWavesPerSimd) void mmt4d_mfma_kernel(MfmaArgs a) {
+// kOcc: waves per SIMD the register allocation must leave room for (2 = two
+// workgroups of 4 waves resident on one compute unit).
+template <typename Cfg, int WM, int WN, int kRing, int kSync, int kOcc = 1>
+__global__ __launch_bounds__(kThreads, kOcc) void mmt4d_mfma_kernel(MfmaArgs a) {
   typedef typename Cfg::frag_t frag_t;
   typedef typename Cfg::acc_t acc_t;
   typedef typename Cfg::out_t out_t;
@@ -195,7 +198,7 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void mmt4d_mfma_kernel(Mfm
   // Per-lane byte offset inside an operand block in global memory (of its
   // first piece; with two pieces the second lies one 512-byte tile further).
   const int lane_off = kSub == 2 ? ((lane >> 5) * 1024 + (lane & 31) * 16)
-                       : kHalfK0 ? lane * 16 : ((lane & 31) * 32 + (lane >> 5) * 16);
+                       : a.half_k0 ? lane * 16 : ((lane & 31) * 32 + (lane >> 5) * 16);
   constexpr int kPieceStride = 512;
 
   // Rows this wave copies: TM/4 rows of A and TN/4 rows of B. Out-of-range
@@ -423,7 +426,7 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void mmt4d_mfma_kernel(Mfm
     }
 }
 
-template <typename Cfg, int WM, int WN, bool kHalfK0, int kRing, int kSync, int kWavesPerSimd = 1>
+template <typename Cfg, int WM, int WN, int kRing, int kSync, int kOcc = 1>
 int launch_variant(const MfmaArgs& a0, hipStream_t s) {
   MfmaArgs a = a0;
   constexpr int TM = 2 * WM, TN = 2 * WN;
@@ -433,7 +436,7 @@ int launch_variant(const MfmaArgs& a0, hipStream_t s) {
   if (blocks > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
   constexpr int lds_bytes = kRing * (TM + TN) * Cfg::kSub * kPieceBytes;
   static_assert(lds_bytes <= 160 * 1024, "LDS ring exceeds 160 KiB");
-  auto kernel = mmt4d_mfma_kernel<Cfg, WM, WN, kHalfK0, kRing, kSync, kWavesPerSimd>;
+  auto kernel = mmt4d_mfma_kernel<Cfg, WM, WN, kRing, kSync, kOcc>;
   static bool attr_set = false;  // benign race: the call is idempotent
   if (!attr_set) {
     UK_RETURN_IF_HIP(hipFuncSetAttribute((const void*)kernel,
@@ -444,26 +447,45 @@ int launch_variant(const MfmaArgs& a0, hipStream_t s) {
   return check_hip(hipGetLastError(), "mmt4d_mfma launch");
 }
 
-template <typename Cfg, bool kHalfK0>
-int launch_half(const MfmaArgs& a, hipStream_t s) {
-  // Pick the macro tile: 256x256 (best operand reuse: 1 KiB of operand per
-  // two MFMAs) when that still yields at least one workgroup per compute
-  // unit, else 128x128 so that small problems spread over more of the chip.
-  // Ring of 8 K-steps (128 KiB of LDS for the large tile), one barrier every
-  // 2 K-steps, 6 K-steps of loads in flight.
-  const int cus = device_cu_count();
-  const int64_t big = (int64_t)((a.M + 7) / 8) * ((a.N + 7) / 8);
-  // An fp8 K-step moves (and multiplies) twice as much: its large tile gets a
-  // ring of 5 K-steps (all 160 KiB of LDS) with a barrier every K-step, which
-  // is the same barrier rate and load lead in time.
-  constexpr int kRing = Cfg::kSub == 2 ? 5 : 8, kSync = Cfg::kSub == 2 ? 1 : 2;
-  if (big >= cus) return launch_variant<Cfg, 4, 4, kHalfK0, kRing, kSync>(a, s);
-  return launch_variant<Cfg, 2, 2, kHalfK0, 8, 2>(a, s);
-}
-
 template <typename Cfg>
-int launch_cfg(const MfmaArgs& a, bool half_k0, hipStream_t s) {
-  return half_k0 ? launch_half<Cfg, true>(a, s) : launch_half<Cfg, false>(a, s);
+int launch_cfg(const MfmaArgs& a, hipStream_t s) {
+  // Pick the macro tile. 256x256 (one workgroup per compute unit, all of its
+  // registers) has the best operand reuse: 1 KiB of operand per two MFMAs.
+  // 256x128 / 128x256 run two workgroups per compute unit, so one workgroup's
+  // output stores overlap the other's MFMAs, and they spread a problem over
+  // more compute units; 128x128 spreads small problems further still.
+  // Estimated cost of a variant, in units of one 32x32 block row of MFMAs:
+  // rounds of resident workgroups x work per workgroup / relative efficiency
+  // (measured on MI355X against the 256x256 tile's rate).
+  // LDS rings: 8 K-steps with a barrier every 2 for the single-occupancy
+  // tiles (fp8, whose K-step is twice as large: 5 with a barrier every step),
+  // 6 (fp8: 3) for the double-occupancy ones.
+  const int cus = device_cu_count();
+  struct Variant { int wm, wn, occ; double eff_alone, eff_full; };
+  static const Variant variants[4] = {
+      {4, 4, 1, 1.0, 1.0}, {4, 2, 2, 0.9, 0.95}, {2, 4, 2, 0.9, 0.95}, {2, 2, 2, 0.75, 0.8}};
+  int best = 0;
+  double best_cost = 0;
+  for (int v = 0; v < 4; ++v) {
+    const Variant& t = variants[v];
+    const int64_t tiles = (int64_t)ceil_div(a.M, 2 * t.wm) * ceil_div(a.N, 2 * t.wn);
+    const int64_t slots = (int64_t)t.occ * cus;
+    const double work = t.wm * t.wn;
+    double cost = (double)(tiles / slots) * t.occ * work / t.eff_full;
+    const int64_t rest = tiles % slots;
+    if (rest > 0) {
+      const int resident = (int)ceil_div(rest, (int64_t)cus);   // workgroups sharing a compute unit
+      cost += resident * work / (resident == t.occ ? t.eff_full : t.eff_alone);
+    }
+    if (v == 0 || cost < best_cost * 0.999) { best = v; best_cost = cost; }
+  }
+  constexpr bool kWide = Cfg::kSub == 2;
+  switch (best) {
+    case 0: return launch_variant<Cfg, 4, 4, kWide ? 5 : 8, kWide ? 1 : 2>(a, s);
+    case 1: return launch_variant<Cfg, 4, 2, kWide ? 3 : 6, kWide ? 1 : 2, 2>(a, s);
+    case 2: return launch_variant<Cfg, 2, 4, kWide ? 3 : 6, kWide ? 1 : 2, 2>(a, s);
+    default: return launch_variant<Cfg, 2, 2, 8, 2>(a, s);
+  }
 }
 
 struct Served { int mfma_k; };
@@ -518,12 +540,12 @@ int launch_mmt4d_mfma(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) {
   a.tail_tiles = (int)((k_elems % sv.mfma_k) / p.K0);
   a.tiles_m = a.tiles_n = 0;
   a.accumulate = (p.flags & IREE_AMD_UK_FLAG_MMT4D_ACCUMULATE) != 0;
-  const bool half_k0 = p.K0 * 2 == sv.mfma_k;
+  a.half_k0 = p.K0 * 2 == sv.mfma_k;
   switch (p.flags & IREE_AMD_UK_FLAG_MMT4D_TYPE_MASK) {
-    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F32: return launch_cfg<F16Cfg>(a, half_k0, s);
-    case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16F32: return launch_cfg<BF16Cfg>(a, half_k0, s);
-    case IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32: return launch_cfg<S8Cfg>(a, half_k0, s);
-    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F8E4M3F8E4M3F32: return launch_half<F8Cfg, true>(a, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F32: return launch_cfg<F16Cfg>(a, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16F32: return launch_cfg<BF16Cfg>(a, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32: return launch_cfg<S8Cfg>(a, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F8E4M3F8E4M3F32: return launch_cfg<F8Cfg>(a, s);
     default: return IREE_AMD_UK_STATUS_NOT_FOUND;
   }
 }

@@ -82,6 +82,21 @@ def test_mfma_kernels_bit_exact_on_exact_inputs(uk, cuda, type_flag, M0, N0, K0)
     assert np.array_equal(gpucase.run_mmt4d(case), case.run_oracle(ukref.F16_IEEE))
 
 
+@pytest.mark.parametrize("type_flag,K0", [(F.MMT4D_TYPE_F16F16F32, 8), (F.MMT4D_TYPE_S8S8S32, 16),
+                                          (F.MMT4D_TYPE_F8E4M3F8E4M3F32, 16)])
+@pytest.mark.parametrize("M,N", [(64, 128), (4, 2048), (128, 8), (64, 130)])
+def test_mfma_macro_tile_variants_bit_exact(uk, cuda, type_flag, K0, M, N):
+    """Outer shapes for which, on 256 compute units, the launcher prefers the
+    256x128, 128x256 and 256x256 macro tiles (the small shapes above all take
+    128x128), including ragged last tiles and a partial last K step."""
+    rng = np.random.default_rng(M * N + K0)
+    for K, acc in ((5, False), (12, True)):
+        case = ukref.Mmt4dCase(rng, type_flag, M, N, K, 32, 32, K0, accumulate=acc)
+        got = gpucase.run_mmt4d(case)
+        want = case.run_oracle(ukref.F16_IEEE)
+        assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), (hex(type_flag), M, N, K, acc)
+
+
 def test_without_fallback_permission_unserved_tiles_are_refused(uk, cuda):
     rng = np.random.default_rng(1)
     case = ukref.Mmt4dCase(rng, F.MMT4D_TYPE_S8S8S32, 2, 2, 2, 9, 6, 3)
