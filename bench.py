@@ -219,17 +219,20 @@ def make_fp8_mlp(torch, iree_amd):
         scales.append(sc)
         del w
     sx = float(xm.float().abs().max()) / 448.0
-    mlp = iree_amd.Fp8Mlp(Hd, Ff, wts[0], wts[1], wts[2], scales[0], scales[1], scales[2], sx, 1.0,
-                          max_tokens=Mt)
-    del wts
     ym = torch.empty(Mt * Hd, dtype=torch.float32, device="cuda")
-    # calibrate the scale of h = silu(g) * u from one pass with unit scale
-    mlp(xm, ym, Mt)
-    gu = mlp.acc.view(Mt // 32, 2 * Ff // 32, 32, 32)
+    # calibrate the scale of h = silu(g) * u from one unfused pass, which leaves
+    # the f32 gate/up values in memory
+    cal = iree_amd.Fp8Mlp(Hd, Ff, wts[0], wts[1], wts[2], scales[0], scales[1], scales[2], sx, 1.0,
+                          max_tokens=Mt, fused=False)
+    cal(xm, ym, Mt)
+    gu = cal.acc.view(Mt // 32, 2 * Ff // 32, 32, 32)
     gate = gu[:, :Ff // 32] * (sx * scales[0])
     up = gu[:, Ff // 32:] * (sx * scales[1])
-    mlp.sh = float((torch.nn.functional.silu(gate) * up).abs().max()) / 448.0
-    del gu, gate, up
+    sh = float((torch.nn.functional.silu(gate) * up).abs().max()) / 448.0
+    del gu, gate, up, cal
+    mlp = iree_amd.Fp8Mlp(Hd, Ff, wts[0], wts[1], wts[2], scales[0], scales[1], scales[2], sx, sh,
+                          max_tokens=Mt)
+    del wts
     return mlp, xm, ym, Mt, Hd, Ff
 
 

@@ -383,6 +383,28 @@ IREE_AMD_UK_EXPORT int iree_amd_uk_silu_mul_quantize_tiled(
     iree_amd_uk_index_t N1, float gate_scale, float up_scale,
     float inv_out_scale, void* stream);
 
+/* The gate/up matmul and the SiLU * up step in one kernel: an mmt4d (same
+ * operands and meaning as iree_amd_uk_mmt4d, tiles M0 = N0 = 32, types
+ * F16F16F32, BF16BF16F32 or F8E4M3F8E4M3F32 at the K0 of the tile-size query)
+ * whose right-hand side holds gate and up tiles INTERLEAVED along its outer
+ * dimension (outer row 2j = gate tile j, 2j+1 = up tile j; N counts both, so it
+ * is even), and whose epilogue stores
+ *   e4m3fn( silu(acc_gate * gate_scale) * (acc_up * up_scale) * inv_out_scale )
+ * as left-hand-side tiles 32x16 of the next matmul instead of the f32
+ * accumulators: out holds N/2 * 1024 bytes per outer row, out_offset and
+ * out_stride0 are in bytes. No accumulate flag. Operands must be 16-byte
+ * aligned (there is no element-wise fallback for this fused form:
+ * IREE_AMD_UK_STATUS_UNIMPLEMENTED otherwise). The f32 accumulators never
+ * reach memory, which saves writing and re-reading 8 bytes per output byte. */
+IREE_AMD_UK_EXPORT int iree_amd_uk_mmt4d_silu_mul_f8e4m3(
+    const void* lhs_buffer, iree_amd_uk_index_t lhs_offset,
+    iree_amd_uk_index_t lhs_stride0, const void* rhs_buffer,
+    iree_amd_uk_index_t rhs_offset, iree_amd_uk_index_t rhs_stride0,
+    void* out_buffer, iree_amd_uk_index_t out_offset,
+    iree_amd_uk_index_t out_stride0, iree_amd_uk_index_t M,
+    iree_amd_uk_index_t N, iree_amd_uk_index_t K, int32_t K0, uint32_t flags,
+    float gate_scale, float up_scale, float inv_out_scale, void* stream);
+
 /* buf[i] *= scale over n f32 elements, in place (applies the product of the
  * per-tensor scales to an fp8 matmul result). */
 IREE_AMD_UK_EXPORT int iree_amd_uk_scale_f32(void* buf_f32, iree_amd_uk_index_t n,

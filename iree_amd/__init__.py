@@ -15,6 +15,7 @@ from .ukernel import (  # noqa: F401
     matmul_data_tiled,
     mmt4d,
     mmt4d_info,
+    mmt4d_silu_mul_f8e4m3,
     pack,
     pack_i4_weights,
     quantize_f16_to_f8e4m3,

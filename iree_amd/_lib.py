@@ -107,6 +107,10 @@ def _declare(lib):
     lib.iree_amd_uk_silu_mul_quantize_tiled.restype = C.c_int
     lib.iree_amd_uk_silu_mul_quantize_tiled.argtypes = [vp, i64, i64, i64, vp, i64, i64, i64,
                                                          C.c_float, C.c_float, C.c_float, vp]
+    lib.iree_amd_uk_mmt4d_silu_mul_f8e4m3.restype = C.c_int
+    lib.iree_amd_uk_mmt4d_silu_mul_f8e4m3.argtypes = [vp, i64, i64, vp, i64, i64, vp, i64, i64,
+                                                       i64, i64, i64, i32, u32,
+                                                       C.c_float, C.c_float, C.c_float, vp]
     lib.iree_amd_uk_scale_f32.restype = C.c_int
     lib.iree_amd_uk_scale_f32.argtypes = [vp, i64, C.c_float, vp]
     lib.iree_amd_uk_device_count.restype = C.c_int

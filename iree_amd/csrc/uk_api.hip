@@ -434,6 +434,38 @@ extern "C" int iree_amd_uk_silu_mul_quantize_tiled(
                                         inv_out_scale, (hipStream_t)stream);
 }
 
+extern "C" int iree_amd_uk_mmt4d_silu_mul_f8e4m3(
+    const void* lhs_buffer, iree_amd_uk_index_t lhs_offset,
+    iree_amd_uk_index_t lhs_stride0, const void* rhs_buffer,
+    iree_amd_uk_index_t rhs_offset, iree_amd_uk_index_t rhs_stride0,
+    void* out_buffer, iree_amd_uk_index_t out_offset,
+    iree_amd_uk_index_t out_stride0, iree_amd_uk_index_t M,
+    iree_amd_uk_index_t N, iree_amd_uk_index_t K, int32_t K0, uint32_t flags,
+    float gate_scale, float up_scale, float inv_out_scale, void* stream) {
+  iree_amd_uk_mmt4d_params_t p = {lhs_buffer, lhs_offset, lhs_stride0,
+                                  rhs_buffer, rhs_offset, rhs_stride0,
+                                  out_buffer, out_offset, out_stride0,
+                                  M, N, K, 32, 32, K0, flags, nullptr};
+  UK_RETURN_IF_ERROR(validate_mmt4d(p));
+  if (flags & IREE_AMD_UK_FLAG_MMT4D_ACCUMULATE)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "mmt4d_silu_mul: accumulate is not supported");
+  if (N % 2) return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "mmt4d_silu_mul: N counts gate and up tiles and must be even");
+  if (out_stride0 < N / 2 * 1024)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "mmt4d_silu_mul: out_stride0 smaller than one outer row");
+  if (M == 0 || N == 0) return 0;
+  if (!lhs_buffer || !rhs_buffer || !out_buffer)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "mmt4d_silu_mul: null buffer");
+  int st = IREE_AMD_UK_STATUS_NOT_FOUND;
+  if (mmt4d_mfma_supported(flags, 32, 32, K0) &&
+      (flags & IREE_AMD_UK_FLAG_MMT4D_TYPE_MASK) != IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32)
+    st = launch_mmt4d_silu_mul_mfma(p, gate_scale, up_scale, inv_out_scale, (hipStream_t)stream);
+  if (st == IREE_AMD_UK_STATUS_NOT_FOUND)
+    return fail(IREE_AMD_UK_STATUS_UNIMPLEMENTED,
+                "mmt4d_silu_mul: needs an MFMA float type at its queried K0, K > 0 and "
+                "16-byte aligned operands");
+  return st;
+}
+
 extern "C" int iree_amd_uk_scale_f32(void* buf_f32, iree_amd_uk_index_t n, float scale,
                                      void* stream) {
   if (n < 0) return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "scale_f32: negative n");

@@ -58,6 +58,8 @@ bool mmt4d_mfma_supported(uint32_t flags, int M0, int N0, int K0);
 // NOT_FOUND (without recording an error) when the call must take the generic
 // kernel instead.
 int launch_mmt4d_mfma(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s);
+int launch_mmt4d_silu_mul_mfma(const iree_amd_uk_mmt4d_params_t& p, float gate_scale,
+                               float up_scale, float inv_out_scale, hipStream_t s);
 
 int launch_pack(const iree_amd_uk_pack_params_t& p, hipStream_t s);
 int launch_unpack(const iree_amd_uk_unpack_params_t& p, hipStream_t s);

@@ -37,6 +37,7 @@
 // (2.1 with all-zero operands): the matrix pipe is power-limited by operand
 // toggling, so data movement that costs energy also costs MFMA rate.
 #include "uk_common.h"
+#include "uk_fp8.h"
 
 namespace uk {
 namespace {
@@ -108,6 +109,9 @@ struct MfmaArgs {
   int tiles_m, tiles_n;  // macro-tile grid
   int accumulate;
   int half_k0;       // K0 is half the MFMA's K extent (else the full extent)
+  // fused SiLU * up epilogue only: scales of the gate and up accumulators and
+  // the inverse scale of the e4m3 result
+  float gate_scale, up_scale, inv_out_scale;
 };
 
 __device__ __forceinline__ void load_block_to_lds(const char* gptr, char* lds) {
@@ -169,7 +173,10 @@ __device__ __forceinline__ void tile_coord(int bid, int tiles_m, int tiles_n,
 // fragments are read from LDS one K-step ahead of the MFMAs that use them.
 // kOcc: waves per SIMD the register allocation must leave room for (2 = two
 // workgroups of 4 waves resident on one compute unit).
-template <typename Cfg, int WM, int WN, int kRing, int kSync, int kOcc = 1>
+// kSiluMul: instead of storing the accumulators, treat even outer columns as
+// gate and the following odd ones as up, and store e4m3(silu(gate) * up) as
+// left-hand-side tiles 32x16 of the next matmul (one byte per element).
+template <typename Cfg, int WM, int WN, int kRing, int kSync, int kOcc = 1, bool kSiluMul = false>
 __global__ __launch_bounds__(kThreads, kOcc) void mmt4d_mfma_kernel(MfmaArgs a) {
   typedef typename Cfg::frag_t frag_t;
   typedef typename Cfg::acc_t acc_t;
@@ -412,6 +419,36 @@ __global__ __launch_bounds__(kThreads, kOcc) void mmt4d_mfma_kernel(MfmaArgs a) 
   // Epilogue. MFMA 32x32 accumulator layout: register v of lane l holds
   // row 8*(v/4) + 4*(l/32) + v%4, column l%32 of the block; one store
   // instruction therefore writes two full 128-byte rows of the tile.
+  if constexpr (kSiluMul) {
+    static_assert(WN % 2 == 0, "gate/up pairs must not straddle waves");
+    // Block pair (y, y+1) -> 32x32 bytes, stored as the two 32x16 tiles
+    // (rows of 16 bytes) that the next matmul reads as left-hand side: column
+    // c of row r lies at (c / 16) * 512 + r * 16 + c % 16.
+    const int col = lane & 31;
+    const int col_off = (col >> 4) * 512 + (col & 15);
+#pragma unroll
+    for (int x = 0; x < WM; ++x)
+#pragma unroll
+      for (int y = 0; y < WN; y += 2) {
+        const int i = i_base + wm * WM + x, j = j_base + wn * WN + y;
+        if (i < a.M && j + 1 < a.N) {
+          uint8_t* t = (uint8_t*)a.out + (int64_t)i * a.out_stride_bytes + (int64_t)(j >> 1) * 1024 + col_off;
+#pragma unroll
+          for (int v = 0; v < 16; v += 4) {
+            float h[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              h[e] = silu_mul((float)acc[x][y][v + e] * a.gate_scale,
+                              (float)acc[x][y + 1][v + e] * a.up_scale) * a.inv_out_scale;
+            const uint32_t packed = pack4_e4m3(h[0], h[1], h[2], h[3]);
+            const int row = 8 * (v >> 2) + 4 * (lane >> 5);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) t[(row + e) * 16] = (uint8_t)(packed >> (8 * e));
+          }
+        }
+      }
+    return;
+  }
 #pragma unroll
   for (int x = 0; x < WM; ++x)
 #pragma unroll
@@ -426,7 +463,7 @@ __global__ __launch_bounds__(kThreads, kOcc) void mmt4d_mfma_kernel(MfmaArgs a) 
     }
 }
 
-template <typename Cfg, int WM, int WN, int kRing, int kSync, int kOcc = 1>
+template <typename Cfg, int WM, int WN, int kRing, int kSync, int kOcc = 1, bool kSiluMul = false>
 int launch_variant(const MfmaArgs& a0, hipStream_t s) {
   MfmaArgs a = a0;
   constexpr int TM = 2 * WM, TN = 2 * WN;
@@ -436,7 +473,7 @@ int launch_variant(const MfmaArgs& a0, hipStream_t s) {
   if (blocks > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
   constexpr int lds_bytes = kRing * (TM + TN) * Cfg::kSub * kPieceBytes;
   static_assert(lds_bytes <= 160 * 1024, "LDS ring exceeds 160 KiB");
-  auto kernel = mmt4d_mfma_kernel<Cfg, WM, WN, kRing, kSync, kOcc>;
+  auto kernel = mmt4d_mfma_kernel<Cfg, WM, WN, kRing, kSync, kOcc, kSiluMul>;
   static bool attr_set = false;  // benign race: the call is idempotent
   if (!attr_set) {
     UK_RETURN_IF_HIP(hipFuncSetAttribute((const void*)kernel,
@@ -447,7 +484,7 @@ int launch_variant(const MfmaArgs& a0, hipStream_t s) {
   return check_hip(hipGetLastError(), "mmt4d_mfma launch");
 }
 
-template <typename Cfg>
+template <typename Cfg, bool kSiluMul = false>
 int launch_cfg(const MfmaArgs& a, hipStream_t s) {
   // Pick the macro tile. 256x256 (one workgroup per compute unit, all of its
   // registers) has the best operand reuse: 1 KiB of operand per two MFMAs.
@@ -481,10 +518,10 @@ int launch_cfg(const MfmaArgs& a, hipStream_t s) {
   }
   constexpr bool kWide = Cfg::kSub == 2;
   switch (best) {
-    case 0: return launch_variant<Cfg, 4, 4, kWide ? 5 : 8, kWide ? 1 : 2>(a, s);
-    case 1: return launch_variant<Cfg, 4, 2, kWide ? 3 : 6, kWide ? 1 : 2, 2>(a, s);
-    case 2: return launch_variant<Cfg, 2, 4, kWide ? 3 : 6, kWide ? 1 : 2, 2>(a, s);
-    default: return launch_variant<Cfg, 2, 2, 8, 2>(a, s);
+    case 0: return launch_variant<Cfg, 4, 4, kWide ? 5 : 8, kWide ? 1 : 2, 1, kSiluMul>(a, s);
+    case 1: return launch_variant<Cfg, 4, 2, kWide ? 3 : 6, kWide ? 1 : 2, 2, kSiluMul>(a, s);
+    case 2: return launch_variant<Cfg, 2, 4, kWide ? 3 : 6, kWide ? 1 : 2, 2, kSiluMul>(a, s);
+    default: return launch_variant<Cfg, 2, 2, 8, 2, 1, kSiluMul>(a, s);
   }
 }
 
@@ -514,7 +551,9 @@ bool mmt4d_mfma_supported(uint32_t flags, int M0, int N0, int K0) {
   return served(flags, M0, N0, K0, nullptr);
 }
 
-int launch_mmt4d_mfma(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) {
+namespace {
+// Fills `a` from the parameters; NOT_FOUND when the MFMA kernels cannot take the call.
+int make_args(const iree_amd_uk_mmt4d_params_t& p, int out_elem_bytes, MfmaArgs* out_args) {
   Served sv;
   if (!served(p.flags, p.M0, p.N0, p.K0, &sv)) return IREE_AMD_UK_STATUS_NOT_FOUND;
   Mmt4dTypeInfo ti;
@@ -529,23 +568,52 @@ int launch_mmt4d_mfma(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) {
   if (((uintptr_t)lhs | (uintptr_t)rhs) % 16) return IREE_AMD_UK_STATUS_NOT_FOUND;
   if ((p.lhs_stride0 * eb) % 16 || (p.rhs_stride0 * eb) % 16) return IREE_AMD_UK_STATUS_NOT_FOUND;
   if (k_elems / sv.mfma_k > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
-  MfmaArgs a;
+  MfmaArgs& a = *out_args;
   a.lhs = lhs; a.rhs = rhs;
-  a.out = (char*)p.out_buffer + p.out_offset * ti.out_bytes;
+  a.out = (char*)p.out_buffer + p.out_offset * out_elem_bytes;
   a.lhs_stride_bytes = p.lhs_stride0 * eb;
   a.rhs_stride_bytes = p.rhs_stride0 * eb;
-  a.out_stride_bytes = p.out_stride0 * ti.out_bytes;
+  a.out_stride_bytes = p.out_stride0 * out_elem_bytes;
   a.M = (int)p.M; a.N = (int)p.N;
   a.ksteps = (int)(k_elems / sv.mfma_k);
   a.tail_tiles = (int)((k_elems % sv.mfma_k) / p.K0);
   a.tiles_m = a.tiles_n = 0;
   a.accumulate = (p.flags & IREE_AMD_UK_FLAG_MMT4D_ACCUMULATE) != 0;
   a.half_k0 = p.K0 * 2 == sv.mfma_k;
+  a.gate_scale = a.up_scale = a.inv_out_scale = 1.0f;
+  return 0;
+}
+}  // namespace
+
+int launch_mmt4d_mfma(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) {
+  Mmt4dTypeInfo ti;
+  mmt4d_type_info(p.flags, &ti);
+  MfmaArgs a;
+  const int st = make_args(p, ti.out_bytes, &a);
+  if (st) return st;
   switch (p.flags & IREE_AMD_UK_FLAG_MMT4D_TYPE_MASK) {
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F32: return launch_cfg<F16Cfg>(a, s);
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16F32: return launch_cfg<BF16Cfg>(a, s);
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32: return launch_cfg<S8Cfg>(a, s);
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_F8E4M3F8E4M3F32: return launch_cfg<F8Cfg>(a, s);
+    default: return IREE_AMD_UK_STATUS_NOT_FOUND;
+  }
+}
+
+// mmt4d whose epilogue is e4m3(silu(gate) * up): `p.N` counts gate AND up outer
+// columns (interleaved, so it is even); the output has N / 2 outer columns of
+// 1024 bytes and `out_offset` / `out_stride0` are in bytes.
+int launch_mmt4d_silu_mul_mfma(const iree_amd_uk_mmt4d_params_t& p, float gate_scale,
+                               float up_scale, float inv_out_scale, hipStream_t s) {
+  MfmaArgs a;
+  const int st = make_args(p, 1, &a);
+  if (st) return st;
+  a.gate_scale = gate_scale; a.up_scale = up_scale; a.inv_out_scale = inv_out_scale;
+  a.accumulate = 0;
+  switch (p.flags & IREE_AMD_UK_FLAG_MMT4D_TYPE_MASK) {
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F32: return launch_cfg<F16Cfg, true>(a, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16F32: return launch_cfg<BF16Cfg, true>(a, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F8E4M3F8E4M3F32: return launch_cfg<F8Cfg, true>(a, s);
     default: return IREE_AMD_UK_STATUS_NOT_FOUND;
   }
 }

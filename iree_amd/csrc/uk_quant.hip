@@ -30,6 +30,7 @@
 //     per-lane scalar);
 //   * sums the 8 K-slices through LDS in a fixed order (deterministic).
 #include "uk_common.h"
+#include "uk_fp8.h"
 
 #include <hip/hip_fp16.h>
 
@@ -449,24 +450,6 @@ int launch_pack_i4_weights(const void* src, void* dst, int64_t N, int64_t K, hip
 //===----------------------------------------------------------------------===//
 
 namespace {
-
-// f32 -> OCP e4m3fn, round to nearest even, saturating at +-448 (NaN stays NaN).
-__device__ __forceinline__ float clamp_e4m3(float x) {
-  const float c = __builtin_fminf(__builtin_fmaxf(x, -448.0f), 448.0f);
-  return x != x ? x : c;
-}
-// Four floats -> four e4m3 bytes (first value in the low byte).
-__device__ __forceinline__ uint32_t pack4_e4m3(float a, float b, float c, float d) {
-  int v = 0;
-  v = __builtin_amdgcn_cvt_pk_fp8_f32(clamp_e4m3(a), clamp_e4m3(b), v, false);
-  v = __builtin_amdgcn_cvt_pk_fp8_f32(clamp_e4m3(c), clamp_e4m3(d), v, true);
-  return (uint32_t)v;
-}
-
-__device__ __forceinline__ float silu_mul(float g, float u) {
-  // g / (1 + exp(-g)) * u; exp(-g) overflows to +inf for g < -88, giving -0.
-  return __fdividef(g, 1.0f + __expf(-g)) * u;
-}
 
 __global__ __launch_bounds__(256) void quantize_f16_kernel(const uint16_t* in, uint8_t* out,
                                                            int64_t n, float inv_scale) {

@@ -146,6 +146,24 @@ def silu_mul_quantize_tiled(acc, acc_stride0, gate_tile0, up_tile0, out, out_str
         gate_scale, up_scale, inv_out_scale, _stream(stream)))
 
 
+def mmt4d_silu_mul_f8e4m3(lhs_buffer, rhs_buffer, out_buffer, M, N, K, K0, flags,
+                          gate_scale, up_scale, inv_out_scale, *, lhs_offset=0,
+                          lhs_stride0=None, rhs_offset=0, rhs_stride0=None, out_offset=0,
+                          out_stride0=None, stream=None):
+    """mmt4d over interleaved gate/up right-hand-side tiles with the SiLU * up
+    product quantised to e4m3 in the epilogue (see include/iree_amd_uk.h)."""
+    if lhs_stride0 is None:
+        lhs_stride0 = K * 32 * K0
+    if rhs_stride0 is None:
+        rhs_stride0 = K * 32 * K0
+    if out_stride0 is None:
+        out_stride0 = N // 2 * 1024
+    _check(load_library().iree_amd_uk_mmt4d_silu_mul_f8e4m3(
+        _ptr(lhs_buffer), lhs_offset, lhs_stride0, _ptr(rhs_buffer), rhs_offset, rhs_stride0,
+        _ptr(out_buffer), out_offset, out_stride0, M, N, K, K0, flags,
+        gate_scale, up_scale, inv_out_scale, _stream(stream)))
+
+
 def scale_f32(buf, n, scale, stream=None):
     _check(load_library().iree_amd_uk_scale_f32(_ptr(buf), n, scale, _stream(stream)))
 
@@ -238,32 +256,42 @@ class Fp8Mlp:
         quantize x -> pack LHS -> mmt4d [gate|up] -> silu*up -> fp8 LHS tiles
         -> mmt4d down -> unpack -> scale
 
+    With ``fused`` (the default) the gate/up matmul and the SiLU * up step are one
+    kernel (``mmt4d_silu_mul_f8e4m3``) and the f32 gate/up values never reach memory.
+
     Weights arrive as e4m3 bytes, row-major ``[N][K]`` (the transpose_b form),
     and are packed once into right-hand-side tiles 32x16. ``sx``/``sh`` are the
     static activation scales (value = code * scale), ``sg``/``su``/``sd`` the
     weight scales. M, hidden and ffn must be multiples of 32.
     """
 
-    def __init__(self, hidden, ffn, wg_q, wu_q, wd_q, sg, su, sd, sx, sh, max_tokens):
+    def __init__(self, hidden, ffn, wg_q, wu_q, wd_q, sg, su, sd, sx, sh, max_tokens, fused=True):
         if hidden % 32 or ffn % 32 or max_tokens % 32:
             raise ValueError("hidden, ffn and max_tokens must be multiples of 32")
-        self.hidden, self.ffn, self.max_tokens = hidden, ffn, max_tokens
+        self.hidden, self.ffn, self.max_tokens, self.fused = hidden, ffn, max_tokens, fused
         self.sg, self.su, self.sd, self.sx, self.sh = sg, su, sd, sx, sh
         dev = wg_q.device
         u8 = torch.uint8
         t = F.PACK_TYPE_I8I8
         self.wgu = torch.empty(2 * ffn * hidden, dtype=u8, device=dev)
         F1, H1 = ffn // 32, hidden // 32
-        # gate tiles occupy outer rows [0, F1), up tiles [F1, 2 F1)
-        pack(wg_q, self.wgu, ffn, hidden, F1, hidden // 16, 32, 16, 0, t)
-        pack(wu_q, self.wgu, ffn, hidden, F1, hidden // 16, 32, 16, 0, t,
-             out_offset=ffn * hidden)
+        row = hidden * 32          # bytes of one outer row of right-hand-side tiles
+        if fused:
+            # gate tile row j at outer row 2j, up tile row j at 2j + 1
+            pack(wg_q, self.wgu, ffn, hidden, F1, hidden // 16, 32, 16, 0, t, out_stride0=2 * row)
+            pack(wu_q, self.wgu, ffn, hidden, F1, hidden // 16, 32, 16, 0, t, out_stride0=2 * row,
+                 out_offset=row)
+        else:
+            # gate tiles occupy outer rows [0, F1), up tiles [F1, 2 F1)
+            pack(wg_q, self.wgu, ffn, hidden, F1, hidden // 16, 32, 16, 0, t)
+            pack(wu_q, self.wgu, ffn, hidden, F1, hidden // 16, 32, 16, 0, t,
+                 out_offset=ffn * hidden)
         self.wd = torch.empty(hidden * ffn, dtype=u8, device=dev)
         pack(wd_q, self.wd, hidden, ffn, H1, ffn // 16, 32, 16, 0, t)
         M = max_tokens
         self.xq = torch.empty(M * hidden, dtype=u8, device=dev)
         self.x_tiles = torch.empty(M * hidden, dtype=u8, device=dev)
-        self.acc = torch.empty(M * 2 * ffn, dtype=torch.float32, device=dev)
+        self.acc = None if fused else torch.empty(M * 2 * ffn, dtype=torch.float32, device=dev)
         self.h_tiles = torch.empty(M * ffn, dtype=u8, device=dev)
         self.acc2 = torch.empty(M * hidden, dtype=torch.float32, device=dev)
 
@@ -275,9 +303,13 @@ class Fp8Mlp:
         mm = F.MMT4D_TYPE_F8E4M3F8E4M3F32
         quantize_f16_to_f8e4m3(x_f16, self.xq, M * hidden, 1.0 / self.sx)
         pack(self.xq, self.x_tiles, M, hidden, M1, hidden // 16, 32, 16, 0, F.PACK_TYPE_I8I8)
-        mmt4d(self.x_tiles, self.wgu, self.acc, M1, 2 * F1, hidden // 16, 32, 32, 16, mm)
-        silu_mul_quantize_tiled(self.acc, 2 * F1 * 1024, 0, F1, self.h_tiles, ffn * 32, M1, F1,
-                                self.sx * self.sg, self.sx * self.su, 1.0 / self.sh)
+        if self.fused:
+            mmt4d_silu_mul_f8e4m3(self.x_tiles, self.wgu, self.h_tiles, M1, 2 * F1, hidden // 16, 16, mm,
+                                  self.sx * self.sg, self.sx * self.su, 1.0 / self.sh)
+        else:
+            mmt4d(self.x_tiles, self.wgu, self.acc, M1, 2 * F1, hidden // 16, 32, 32, 16, mm)
+            silu_mul_quantize_tiled(self.acc, 2 * F1 * 1024, 0, F1, self.h_tiles, ffn * 32, M1, F1,
+                                    self.sx * self.sg, self.sx * self.su, 1.0 / self.sh)
         mmt4d(self.h_tiles, self.wd, self.acc2, M1, H1, ffn // 16, 32, 32, 16, mm)
         unpack(self.acc2, y_f32, M1, H1, 32, 32, M, hidden, F.UNPACK_TYPE_F32F32)
         scale_f32(y_f32, M * hidden, self.sh * self.sd)

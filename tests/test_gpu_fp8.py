@@ -230,10 +230,17 @@ def test_fp8_mlp_block_small(uk, cuda):
     sh = float(np.abs(h).max()) / 448.0
 
     dev = lambda a: torch.from_numpy(np.ascontiguousarray(a).reshape(-1)).cuda()  # noqa: E731
-    mlp = uk.Fp8Mlp(H, Fn, dev(wg_q), dev(wu_q), dev(wd_q), sg, su, sd, sx, sh, max_tokens=M)
+    mlp = uk.Fp8Mlp(H, Fn, dev(wg_q), dev(wu_q), dev(wd_q), sg, su, sd, sx, sh, max_tokens=M,
+                    fused=False)
     y = torch.zeros(M * H, dtype=torch.float32, device="cuda")
     mlp(dev(x.view(np.int16)), y, M)
+    # the fused gate/up + SiLU kernel: same accumulators, same arithmetic, same bits
+    fused = uk.Fp8Mlp(H, Fn, dev(wg_q), dev(wu_q), dev(wd_q), sg, su, sd, sx, sh, max_tokens=M)
+    y2 = torch.full((M * H,), 7.0, dtype=torch.float32, device="cuda")
+    fused(dev(x.view(np.int16)), y2, M)
     torch.cuda.synchronize()
+    assert np.array_equal(fused.h_tiles.cpu().numpy(), mlp.h_tiles.cpu().numpy())
+    assert np.array_equal(y2.cpu().numpy(), y.cpu().numpy())
     # x codes: bit-exact
     assert np.array_equal(mlp.xq.cpu().numpy().reshape(M, H), xq)
     # h codes (as LHS tiles 32x16 -> row-major)
@@ -255,3 +262,53 @@ def test_fp8_mlp_block_small(uk, cuda):
     got = y.cpu().numpy().reshape(M, H).astype(np.float64)
     assert np.all(np.abs(got - want) <= ATOL + RTOL * np.abs(want))
     assert np.max(np.abs(got - want)) <= 1e-4 * np.abs(want).max()
+
+
+@pytest.mark.parametrize("type_flag,K0", [(F.MMT4D_TYPE_F8E4M3F8E4M3F32, 16), (F.MMT4D_TYPE_F16F16F32, 8)])
+@pytest.mark.parametrize("M1,P,K1", [(1, 1, 4), (3, 5, 7), (9, 33, 12), (64, 64, 5)])
+def test_fused_gate_up_silu_matches_unfused(uk, cuda, type_flag, K0, M1, P, K1):
+    """mmt4d_silu_mul_f8e4m3 on interleaved gate/up tiles against plain mmt4d
+    followed by silu_mul_quantize_tiled on the de-interleaved accumulators:
+    identical bytes (ragged macro tiles, partial last K step, every tile variant
+    the launcher picks at these sizes), loose output pitch respected."""
+    import torch
+    rng = np.random.default_rng(M1 * 100 + P + K1)
+    n_l, n_r = M1 * K1 * 32 * K0, 2 * P * K1 * 32 * K0
+    if type_flag == F.MMT4D_TYPE_F16F16F32:
+        lhs = (rng.standard_normal(n_l) * 0.5).astype(np.float16).view(np.uint16)
+        rhs = (rng.standard_normal(n_r) * 0.5).astype(np.float16).view(np.uint16)
+    else:
+        lhs, rhs = quantize_np(rng.standard_normal(n_l)), quantize_np(rng.standard_normal(n_r))
+    dl, dr = torch.from_numpy(lhs.view(np.uint8)).cuda(), torch.from_numpy(rhs.view(np.uint8)).cuda()
+    gs, us, os_ = 0.8, 1.2, 0.7
+    pitch = P * 1024 + 64
+    fused = torch.full((M1 * pitch,), 0xEE, dtype=torch.uint8, device="cuda")
+    uk.mmt4d_silu_mul_f8e4m3(dl, dr, fused, M1, 2 * P, K1, K0, type_flag, gs, us, os_, out_stride0=pitch)
+    acc = torch.zeros(M1 * 2 * P * 1024, dtype=torch.float32, device="cuda")
+    uk.mmt4d(dl, dr, acc, M1, 2 * P, K1, 32, 32, K0, type_flag)
+    a4 = acc.view(M1, P, 2, 1024)
+    split = torch.cat([a4[:, :, 0], a4[:, :, 1]], dim=1).contiguous()     # [M1][gate tiles | up tiles]
+    want = torch.zeros(M1 * P * 1024, dtype=torch.uint8, device="cuda")
+    uk.silu_mul_quantize_tiled(split, 2 * P * 1024, 0, P, want, P * 1024, M1, P, gs, us, os_)
+    torch.cuda.synchronize()
+    got = fused.cpu().numpy().reshape(M1, pitch)
+    assert np.array_equal(got[:, :P * 1024].reshape(-1), want.cpu().numpy())
+    assert np.all(got[:, P * 1024:] == 0xEE)
+
+
+def test_fused_gate_up_silu_invalid_arguments(uk, cuda):
+    import torch
+    t = torch.zeros(4096, dtype=torch.uint8, device="cuda")
+    mm = F.MMT4D_TYPE_F8E4M3F8E4M3F32
+    with pytest.raises(uk.UkError) as e:
+        uk.mmt4d_silu_mul_f8e4m3(t, t, t, 1, 3, 4, 16, mm, 1.0, 1.0, 1.0)        # odd N
+    assert e.value.status == F.STATUS_INVALID_ARGUMENT
+    with pytest.raises(uk.UkError):
+        uk.mmt4d_silu_mul_f8e4m3(t, t, t, 1, 2, 4, 16, mm | F.MMT4D_ACCUMULATE, 1.0, 1.0, 1.0)
+    with pytest.raises(uk.UkError) as e:
+        uk.mmt4d_silu_mul_f8e4m3(t, t, t, 1, 2, 4, 16, F.MMT4D_TYPE_S8S8S32, 1.0, 1.0, 1.0)
+    assert e.value.status == F.STATUS_UNIMPLEMENTED
+    with pytest.raises(uk.UkError) as e:
+        uk.mmt4d_silu_mul_f8e4m3(t[1:], t, t, 1, 2, 4, 16, mm, 1.0, 1.0, 1.0)    # misaligned operand
+    assert e.value.status == F.STATUS_UNIMPLEMENTED
+    uk.mmt4d_silu_mul_f8e4m3(t, t, t, 0, 2, 4, 16, mm, 1.0, 1.0, 1.0)             # M == 0: nothing to do
