@@ -330,6 +330,26 @@ def extras(args, torch, iree_amd, F, synth, lhs, rhs, out):
     ex["dequant_matmul_i4_m1_frac_of_hbm_peak"] = round(ex["dequant_matmul_i4_m1_gbs"] / PEAK_HBM_GBS, 4)
     del wq, sq, zq
 
+    # f16 mmt4d with a narrow left-hand side (decode shape: one outer row of
+    # M0 x 8 tiles against 448 x 512 right-hand-side tiles = N 14336, K 4096);
+    # six right-hand sides (705 MB) rotate so that they come from HBM
+    Nn, Kn = 14336, 4096
+    rn = [torch.from_numpy(synth.normal_f16(50 + i, Nn * Kn, 1 / 64).view(np.int16)).cuda() for i in range(6)]
+    for M0 in (1, 8):
+        ln = torch.from_numpy(synth.normal_f16(60, M0 * Kn).view(np.int16)).cuda()
+        on = torch.empty(M0 * Nn, dtype=torch.float32, device="cuda")
+        state["i"] = 0
+
+        def do_n():
+            k = state["i"] % 6
+            state["i"] += 1
+            iree_amd.mmt4d(ln, rn[k], on, 1, Nn // 32, Kn // 8, M0, 32, 8, F.MMT4D_TYPE_F16F16F32)
+
+        _, t = gpu_time(torch, do_n, steps, warm)
+        ex[f"mmt4d_f16_narrow_m{M0}_gbs"] = round((Nn * Kn * 2 + M0 * Kn * 2 + M0 * Nn * 4) / t / 1e9, 1)
+    ex["mmt4d_f16_narrow_m1_frac_of_hbm_peak"] = round(ex["mmt4d_f16_narrow_m1_gbs"] / PEAK_HBM_GBS, 4)
+    del rn
+
     # fp8 e4m3 x e4m3 -> f32 at 4096^3, tile 32x32x16 (codes of N(0,1) values)
     K1 = size // 16
     g = torch.Generator(device="cuda")

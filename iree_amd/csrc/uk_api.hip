@@ -209,6 +209,13 @@ extern "C" int iree_amd_uk_mmt4d_p(const iree_amd_uk_mmt4d_params_t* params,
   if (!p.rhs_buffer && p.K && p.K0) return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "mmt4d: null rhs");
   if (!p.out_buffer) return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "mmt4d: null out");
   hipStream_t s = (hipStream_t)stream;
+  if (mmt4d_skinny_supported(p.flags, p.M0, p.N0, p.K0)) {
+    // Narrow left-hand-side tiles (a matrix of fewer than 32 rows): the
+    // streaming MFMA kernel, or the element-wise one for what it cannot take.
+    int st = launch_mmt4d_skinny(p, s);
+    if (st != IREE_AMD_UK_STATUS_NOT_FOUND) return st;
+    return launch_mmt4d_generic(p, s);
+  }
   if (mmt4d_mfma_supported(p.flags, p.M0, p.N0, p.K0)) {
     int st = launch_mmt4d_mfma(p, s);
     if (st != IREE_AMD_UK_STATUS_NOT_FOUND) return st;
@@ -248,7 +255,7 @@ extern "C" uint32_t iree_amd_uk_mmt4d_info(int32_t M0, int32_t N0, int32_t K0,
                                            uint32_t flags,
                                            const uint64_t* cpu_data) {
   (void)cpu_data;
-  return mmt4d_mfma_supported(flags, M0, N0, K0)
+  return (mmt4d_mfma_supported(flags, M0, N0, K0) || mmt4d_skinny_supported(flags, M0, N0, K0))
              ? IREE_AMD_UK_FLAG_MMT4D_INFO_HAVE_ARCHITECTURE_SPECIFIC_TILE_FUNCTION
              : 0u;
 }

@@ -54,6 +54,8 @@ int validate_unpack(const iree_amd_uk_unpack_params_t& p);
 int launch_mmt4d_generic(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s);
 // Returns true when a MFMA kernel exists for (type, M0, N0, K0).
 bool mmt4d_mfma_supported(uint32_t flags, int M0, int N0, int K0);
+bool mmt4d_skinny_supported(uint32_t flags, int M0, int N0, int K0);
+int launch_mmt4d_skinny(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s);
 // Also needs alignment / stride properties of the actual call; returns
 // NOT_FOUND (without recording an error) when the call must take the generic
 // kernel instead.

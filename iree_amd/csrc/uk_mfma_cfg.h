@@ -1,0 +1,67 @@
+// MFMA instruction wrappers shared by the matmul kernels: one struct per
+// element-type tuple giving the operand fragment type of one lane, the
+// accumulator type of a 32x32 block and the instruction.
+#ifndef IREE_AMD_UK_MFMA_CFG_H_
+#define IREE_AMD_UK_MFMA_CFG_H_
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace uk {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef int int4v __attribute__((ext_vector_type(4)));
+typedef int int8v __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef int intx16 __attribute__((ext_vector_type(16)));
+
+struct F16Cfg {
+  typedef half8 frag_t;
+  typedef floatx16 acc_t;
+  typedef float out_t;
+  static constexpr int kElemBytes = 2;
+  static constexpr int kMfmaK = 16;
+  static constexpr int kSub = 1;   // 1 KiB pieces per operand block
+  __device__ static acc_t mfma(frag_t a, frag_t b, acc_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+};
+struct BF16Cfg {
+  typedef bf16x8 frag_t;
+  typedef floatx16 acc_t;
+  typedef float out_t;
+  static constexpr int kElemBytes = 2;
+  static constexpr int kMfmaK = 16;
+  static constexpr int kSub = 1;
+  __device__ static acc_t mfma(frag_t a, frag_t b, acc_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+};
+struct S8Cfg {
+  typedef int4v frag_t;
+  typedef intx16 acc_t;
+  typedef int32_t out_t;
+  static constexpr int kElemBytes = 1;
+  static constexpr int kMfmaK = 32;
+  static constexpr int kSub = 1;
+  __device__ static acc_t mfma(frag_t a, frag_t b, acc_t c) {
+    return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
+  }
+};
+struct F8Cfg {
+  typedef int8v frag_t;
+  typedef floatx16 acc_t;
+  typedef float out_t;
+  static constexpr int kElemBytes = 1;
+  static constexpr int kMfmaK = 64;
+  static constexpr int kSub = 2;
+  __device__ static acc_t mfma(frag_t a, frag_t b, acc_t c) {
+    // formats 0 / 0: both operands e4m3; block scales 0x7F = 2^0.
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+  }
+};
+
+}  // namespace uk
+
+#endif  // IREE_AMD_UK_MFMA_CFG_H_

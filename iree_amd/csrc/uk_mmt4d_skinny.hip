@@ -1,0 +1,194 @@
+// mmt4d for narrow left-hand sides (a matrix with fewer than 32 rows: the
+// decode / GEMV shapes), on the matrix cores.
+//
+// The tile-size query narrows M0 to the next power of two that holds a static
+// M below 32 (the reference does the same, compiler/src/iree/compiler/Codegen/
+// Common/CPU/CPUMaterializeEncodingPass.cpp:343-353), so these calls arrive
+// with M = 1 outer row of M0 x K0 tiles, N0 = 32 and a long right-hand side:
+// the work is reading the right-hand side once, i.e. an HBM stream.
+//
+//   out[0][j][m0][n0] (+)= sum_k lhs[0][k][m0][k0] * rhs[j][k][n0][k0]
+//
+// A workgroup of 8 waves takes one outer column j at a time; wave w owns the
+// w-th eighth of the K steps and keeps its part of the left-hand side in
+// registers for the whole kernel, as the B operand of v_mfma_*_32x32 (column
+// m0 of the block, zero beyond M0). The right-hand side streams through a
+// rolling register buffer of 8 blocks of 1 KiB per wave (A operand: a packed
+// tile is already in operand order), the request for block q+8 issued as block
+// q is consumed, across tile boundaries, so the stream never drains. The 8
+// partial 32x32 blocks are summed through LDS in wave order (deterministic)
+// and rows m0 < M0 are stored.
+#include "uk_common.h"
+#include "uk_mfma_cfg.h"
+
+namespace uk {
+namespace {
+
+constexpr int kWaves = 8;
+constexpr int kThreads = kWaves * 64;
+constexpr int kDepth = 8;   // right-hand-side blocks in flight per wave
+
+struct SkinnyArgs {
+  const char* lhs;   // offsets applied
+  const char* rhs;
+  char* out;
+  int64_t rhs_stride_bytes, out_stride_elems;  // per outer column j
+  int N;             // outer columns
+  int M0;
+  int ksteps;        // MFMA K steps in total
+  int steps_per_wave;
+  int lhs_tile_bytes;  // M0 * K0 * element size
+  int half_k0;
+  int accumulate;
+};
+
+// SP: K steps per wave held in registers (compile-time bound; a.steps_per_wave <= SP).
+template <typename Cfg, int SP>
+__global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
+  typedef typename Cfg::frag_t frag_t;
+  typedef typename Cfg::acc_t acc_t;
+  typedef typename Cfg::out_t out_t;
+  static_assert(SP % kDepth == 0, "the rolling buffer must divide the steps of a tile");
+  __shared__ out_t partial[2][kWaves][16][64];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int m0 = lane & 31, kh = lane >> 5;
+  const int first = wave * a.steps_per_wave;
+  int count = a.ksteps - first;
+  count = count < 0 ? 0 : (count > a.steps_per_wave ? a.steps_per_wave : count);
+
+  // Right-hand side: lane offset inside a 1 KiB block, block of (j, step).
+  const int lane_off = a.half_k0 ? lane * 16 : ((lane & 31) * 32 + (lane >> 5) * 16);
+  const char* rhs_lane = a.rhs + (int64_t)first * 1024 + lane_off;
+  // Steps past this wave's count read the wave's first block again (a valid
+  // address) and are multiplied by a zero left-hand side.
+  auto load_block = [&](int j, int sp) -> frag_t {
+    const int s = sp < count ? sp : 0;
+    const int jj = j < a.N ? j : a.N - 1;
+    union { int4v i; frag_t f; } u;
+    u.i = *(const int4v*)(rhs_lane + (int64_t)jj * a.rhs_stride_bytes + (int64_t)s * 1024);
+    return u.f;
+  };
+
+  // ---- first blocks of the first tile, then the left-hand side -------------
+  int j = blockIdx.x;
+  frag_t ring[kDepth];
+#pragma unroll
+  for (int d = 0; d < kDepth; ++d) ring[d] = load_block(j, d);
+  __builtin_amdgcn_sched_barrier(0);
+  frag_t xf[SP];
+#pragma unroll
+  for (int sp = 0; sp < SP; ++sp) {
+    const int s = first + (sp < count ? sp : 0);
+    // K tile(s) of step s: two tiles of K0 = half the MFMA extent, or one.
+    const int64_t off = a.half_k0 ? ((int64_t)(2 * s + kh) * a.lhs_tile_bytes + m0 * 16)
+                                  : ((int64_t)s * a.lhs_tile_bytes + m0 * 32 + kh * 16);
+    int4v v = {0, 0, 0, 0};
+    if (m0 < a.M0 && sp < count) v = *(const int4v*)(a.lhs + off);
+    union { int4v i; frag_t f; } u;
+    u.i = v;
+    xf[sp] = u.f;
+  }
+
+  int parity = 0;
+  for (; j < a.N; j += gridDim.x, parity ^= 1) {
+    const int next = j + gridDim.x;
+    acc_t acc;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[v] = 0;
+#pragma unroll
+    for (int sp = 0; sp < SP; ++sp) {
+      acc = Cfg::mfma(ring[sp % kDepth], xf[sp], acc);
+      // refill the slot: kDepth steps ahead, wrapping into the next tile
+      __builtin_amdgcn_sched_barrier(0);
+      ring[sp % kDepth] = sp + kDepth < SP ? load_block(j, sp + kDepth) : load_block(next, sp + kDepth - SP);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // ---- sum the 8 K slices in wave order and store -----------------------
+    out_t (*buf)[16][64] = partial[parity];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) buf[wave][v][lane] = acc[v];
+    __syncthreads();
+    out_t* tile = (out_t*)a.out + (int64_t)j * a.out_stride_elems;
+#pragma unroll
+    for (int rep = 0; rep < 2; ++rep) {
+      const int flat = rep * kThreads + threadIdx.x;   // v * 64 + lane
+      const int l = flat & 63, v = flat >> 6;
+      const int mm = l & 31, nn = 8 * (v >> 2) + 4 * (l >> 5) + (v & 3);
+      if (mm < a.M0) {
+        out_t sum = a.accumulate ? tile[mm * 32 + nn] : (out_t)0;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) sum += buf[w][v][l];
+        tile[mm * 32 + nn] = sum;
+      }
+    }
+    // The other half of `partial` serves the next tile; this half is rewritten
+    // two tiles later, after the next tile's barrier.
+  }
+}
+
+template <typename Cfg>
+int launch_cfg(SkinnyArgs a, hipStream_t s) {
+  const int cus = device_cu_count();
+  const int blocks = a.N < cus ? a.N : cus;
+  const int per = (a.ksteps + kWaves - 1) / kWaves;
+  a.steps_per_wave = per;
+  if (per <= 8) hipLaunchKernelGGL((mmt4d_skinny_kernel<Cfg, 8>), dim3(blocks), dim3(kThreads), 0, s, a);
+  else if (per <= 16) hipLaunchKernelGGL((mmt4d_skinny_kernel<Cfg, 16>), dim3(blocks), dim3(kThreads), 0, s, a);
+  else if (per <= 32) hipLaunchKernelGGL((mmt4d_skinny_kernel<Cfg, 32>), dim3(blocks), dim3(kThreads), 0, s, a);
+  else return IREE_AMD_UK_STATUS_NOT_FOUND;
+  return check_hip(hipGetLastError(), "mmt4d_skinny launch");
+}
+
+int mfma_k_of(uint32_t flags) {
+  switch (flags & IREE_AMD_UK_FLAG_MMT4D_TYPE_MASK) {
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F32:
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16F32: return 16;
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32: return 32;
+    default: return 0;
+  }
+}
+
+}  // namespace
+
+// Narrow tiles served: M0 < 32, N0 = 32, K0 = half or all of the MFMA's K extent.
+bool mmt4d_skinny_supported(uint32_t flags, int M0, int N0, int K0) {
+  const int mk = mfma_k_of(flags);
+  return mk && M0 >= 1 && M0 < 32 && N0 == 32 && (K0 == mk || K0 * 2 == mk);
+}
+
+int launch_mmt4d_skinny(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) {
+  if (!mmt4d_skinny_supported(p.flags, p.M0, p.N0, p.K0)) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  const int mk = mfma_k_of(p.flags);
+  Mmt4dTypeInfo ti;
+  mmt4d_type_info(p.flags, &ti);
+  const int eb = ti.lhs_bits / 8;
+  const int64_t k_elems = p.K * p.K0;
+  // One outer row, whole MFMA steps, a K that fits the register-resident
+  // left-hand side (8 waves x 32 steps), 16-byte aligned operands.
+  if (p.M != 1 || p.K == 0 || k_elems % mk || k_elems / mk > kWaves * 32 || p.N > 0x7FFFFFFF)
+    return IREE_AMD_UK_STATUS_NOT_FOUND;
+  const char* lhs = (const char*)p.lhs_buffer + p.lhs_offset * eb;
+  const char* rhs = (const char*)p.rhs_buffer + p.rhs_offset * eb;
+  if (((uintptr_t)lhs | (uintptr_t)rhs) % 16 || (p.rhs_stride0 * eb) % 16 || (p.M0 * p.K0 * eb) % 16)
+    return IREE_AMD_UK_STATUS_NOT_FOUND;
+  SkinnyArgs a;
+  a.lhs = lhs; a.rhs = rhs;
+  a.out = (char*)p.out_buffer + p.out_offset * ti.out_bytes;
+  a.rhs_stride_bytes = p.rhs_stride0 * eb;
+  a.out_stride_elems = (int64_t)p.M0 * 32;   // consecutive outer columns of the single outer row
+  a.N = (int)p.N; a.M0 = p.M0;
+  a.ksteps = (int)(k_elems / mk);
+  a.steps_per_wave = 0;
+  a.lhs_tile_bytes = p.M0 * p.K0 * eb;
+  a.half_k0 = p.K0 * 2 == mk;
+  a.accumulate = (p.flags & IREE_AMD_UK_FLAG_MMT4D_ACCUMULATE) != 0;
+  switch (p.flags & IREE_AMD_UK_FLAG_MMT4D_TYPE_MASK) {
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F32: return launch_cfg<F16Cfg>(a, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16F32: return launch_cfg<BF16Cfg>(a, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32: return launch_cfg<S8Cfg>(a, s);
+    default: return IREE_AMD_UK_STATUS_NOT_FOUND;
+  }
+}
+
+}  // namespace uk

@@ -97,6 +97,34 @@ def test_mfma_macro_tile_variants_bit_exact(uk, cuda, type_flag, K0, M, N):
         assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), (hex(type_flag), M, N, K, acc)
 
 
+@pytest.mark.parametrize("type_flag,K0", [(F.MMT4D_TYPE_F16F16F32, 8), (F.MMT4D_TYPE_F16F16F32, 16),
+                                          (F.MMT4D_TYPE_BF16BF16F32, 8), (F.MMT4D_TYPE_S8S8S32, 16),
+                                          (F.MMT4D_TYPE_S8S8S32, 32)])
+def test_narrow_lhs_tiles_bit_exact(uk, cuda, type_flag, K0):
+    """Narrow left-hand-side tiles (M0 < 32, one outer row: the decode shapes
+    the tile-size query hands out for a static M below 32) run the streaming
+    MFMA kernel: K step counts that fill 8, 16 and 32 register slots per wave,
+    ragged splits over the 8 waves, more outer columns than compute units,
+    accumulate. Calls that kernel does not take (two outer rows, an odd K tile
+    count, a K beyond the register-resident range) must give the same bits
+    through the element-wise kernel."""
+    rng = np.random.default_rng(7000 + type_flag + K0)
+    mfma_k = 32 if type_flag == F.MMT4D_TYPE_S8S8S32 else 16
+    tps = mfma_k // K0                      # K tiles per MFMA step
+    for M0 in (1, 2, 4, 8, 16):
+        assert uk.mmt4d_info(M0, 32, K0, type_flag) == 1
+        for N, steps, acc in ((1, 1, False), (5, 8, True), (300, 13, False), (3, 70, True),
+                              (7, 128, False), (2, 255, True)):
+            case = ukref.Mmt4dCase(rng, type_flag, 1, N, steps * tps, M0, 32, K0, accumulate=acc)
+            got = gpucase.run_mmt4d(case, flags=case.flags & ~F.MMT4D_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION)
+            assert np.array_equal(got.view(np.uint8), case.run_oracle(ukref.F16_IEEE).view(np.uint8)), \
+                (hex(type_flag), M0, K0, N, steps, acc)
+    for M, N, K in ((2, 3, 4 * tps), (1, 3, 2 * tps + (1 if tps > 1 else 0)), (1, 2, 260 * tps)):
+        case = ukref.Mmt4dCase(rng, type_flag, M, N, K, 8, 32, K0, accumulate=True,
+                               loose_strides=True, offsets=True)
+        assert np.array_equal(gpucase.run_mmt4d(case), case.run_oracle(ukref.F16_IEEE)), (M, N, K)
+
+
 def test_without_fallback_permission_unserved_tiles_are_refused(uk, cuda):
     rng = np.random.default_rng(1)
     case = ukref.Mmt4dCase(rng, F.MMT4D_TYPE_S8S8S32, 2, 2, 2, 9, 6, 3)
