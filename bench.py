@@ -30,6 +30,7 @@ import numpy as np  # noqa: E402
 PEAK_F16_TFLOPS = 2500.0   # MI355X dense f16 MFMA
 PEAK_I8_TOPS = 5000.0      # MI355X dense int8 MFMA
 PEAK_FP8_TFLOPS = 5000.0   # MI355X dense fp8 MFMA
+PEAK_F32_TFLOPS = 157.3    # MI355X dense f32 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE
@@ -259,6 +260,16 @@ def extras(args, torch, iree_amd, F, synth, lhs, rhs, out):
     ex["mmt4d_i8_tops"] = round(flops / t / 1e12, 2)
     ex["mmt4d_i8_frac_of_peak"] = round(flops / t / 1e12 / PEAK_I8_TOPS, 4)
     del li, ri, oi
+
+    # f32 x f32 -> f32 at 4096^3, tile 32x32x4 (the reference's primary type)
+    K1 = size // 4
+    lf = torch.from_numpy(synth.normal_f32(1, M1 * K1 * 32 * 4, 1 / 64)).cuda()
+    rf = torch.from_numpy(synth.normal_f32(2, N1 * K1 * 32 * 4, 1 / 64)).cuda()
+    _, t = gpu_time(torch, lambda: iree_amd.mmt4d(lf, rf, out, M1, N1, K1, 32, 32, 4, F.MMT4D_TYPE_F32F32F32),
+                    max(5, steps // 4), 2)
+    ex["mmt4d_f32_tflops"] = round(flops / t / 1e12, 2)
+    ex["mmt4d_f32_frac_of_peak"] = round(flops / t / 1e12 / PEAK_F32_TFLOPS, 4)
+    del lf, rf
 
     # pack / unpack of the f16 8191 x 5001 tensor <-> 32x16 tiles. Rotating
     # buffer sets (> 256 MiB in total) so that HBM, not the last-level cache,

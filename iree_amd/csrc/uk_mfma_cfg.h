@@ -13,6 +13,7 @@ typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef int int4v __attribute__((ext_vector_type(4)));
 typedef int int8v __attribute__((ext_vector_type(8)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef int intx16 __attribute__((ext_vector_type(16)));
 
@@ -36,6 +37,33 @@ struct BF16Cfg {
   static constexpr int kSub = 1;
   __device__ static acc_t mfma(frag_t a, frag_t b, acc_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+};
+// f16 / bf16 results: f32 accumulation, one rounding (to nearest even) when the
+// accumulators are stored, which is the reference's arithmetic when
+// IREE_UK_FLAG_MMT4D_SKIP_INTERMEDIATE_ROUNDINGS is set
+// (runtime/src/iree/builtins/ukernel/mmt4d_tile_generic.c:229-286, 289-376).
+struct F16F16Cfg : F16Cfg {
+  typedef _Float16 out_t;
+};
+struct BF16BF16Cfg : BF16Cfg {
+  typedef __bf16 out_t;
+};
+// f32: v_mfma_f32_32x32x2_f32 takes one float per lane (row l % 32, k = l / 32).
+// A lane's 16 bytes are 4 consecutive k of its row, so element e of lanes 0..31
+// and element e of lanes 32..63 form the k pair of the e-th of four
+// instructions; both operands pair the same way, so every k meets its partner.
+struct F32Cfg {
+  typedef floatx4 frag_t;
+  typedef floatx16 acc_t;
+  typedef float out_t;
+  static constexpr int kElemBytes = 4;
+  static constexpr int kMfmaK = 8;
+  static constexpr int kSub = 1;
+  __device__ static acc_t mfma(frag_t a, frag_t b, acc_t c) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) c = __builtin_amdgcn_mfma_f32_32x32x2f32(a[e], b[e], c, 0, 0, 0);
+    return c;
   }
 };
 struct S8Cfg {

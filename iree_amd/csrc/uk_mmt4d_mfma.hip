@@ -10,6 +10,8 @@
 //   f16 x f16 -> f32  v_mfma_f32_32x32x16_f16        16         8, 16
 //   bf16 x bf16 -> f32 v_mfma_f32_32x32x16_bf16      16         8, 16
 //   s8 x s8 -> s32    v_mfma_i32_32x32x32_i8         32         16, 32
+//   f32 x f32 -> f32  4 x v_mfma_f32_32x32x2_f32      8          4, 8
+//   f16 -> f16, bf16 -> bf16 (intermediate roundings skipped): as -> f32, rounded on store
 //   e4m3 x e4m3 -> f32 v_mfma_scale_f32_32x32x64_f8f6f4  64         16
 //
 // With K0 = half the MFMA's K extent, two consecutive K tiles of one outer row
@@ -479,6 +481,14 @@ bool served(uint32_t flags, int M0, int N0, int K0, Served* out) {
   switch (flags & IREE_AMD_UK_FLAG_MMT4D_TYPE_MASK) {
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F32:
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16F32: mfma_k = 16; break;
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F16:
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16BF16:
+      // f32 accumulation with one final rounding is only the reference's
+      // arithmetic when intermediate roundings are skipped
+      if (!(flags & IREE_AMD_UK_FLAG_MMT4D_SKIP_INTERMEDIATE_ROUNDINGS)) return false;
+      mfma_k = 16;
+      break;
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F32F32F32: mfma_k = 8; break;
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32: mfma_k = 32; break;
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_F8E4M3F8E4M3F32: mfma_k = 64; break;
     default: return false;
@@ -544,6 +554,9 @@ int launch_mmt4d_mfma(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) {
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16F32: return launch_cfg<BF16Cfg>(a, s);
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32: return launch_cfg<S8Cfg>(a, s);
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_F8E4M3F8E4M3F32: return launch_cfg<F8Cfg>(a, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F32F32F32: return launch_cfg<F32Cfg>(a, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F16: return launch_cfg<F16F16Cfg>(a, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16BF16: return launch_cfg<BF16BF16Cfg>(a, s);
     default: return IREE_AMD_UK_STATUS_NOT_FOUND;
   }
 }

@@ -43,7 +43,10 @@ def test_reference_test_matrix_bit_exact(uk, cuda, type_flag):
 MFMA_TILES = [(F.MMT4D_TYPE_S8S8S32, 32, 32, 16), (F.MMT4D_TYPE_S8S8S32, 32, 32, 32),
               (F.MMT4D_TYPE_F16F16F32, 32, 32, 8), (F.MMT4D_TYPE_F16F16F32, 32, 32, 16),
               (F.MMT4D_TYPE_BF16BF16F32, 32, 32, 8), (F.MMT4D_TYPE_BF16BF16F32, 32, 32, 16),
-              (F.MMT4D_TYPE_F8E4M3F8E4M3F32, 32, 32, 16)]
+              (F.MMT4D_TYPE_F8E4M3F8E4M3F32, 32, 32, 16),
+              (F.MMT4D_TYPE_F32F32F32, 32, 32, 4), (F.MMT4D_TYPE_F32F32F32, 32, 32, 8),
+              # f16 / bf16 results: on the matrix cores when intermediate roundings are skipped
+              (F.MMT4D_TYPE_F16F16F16, 32, 32, 8), (F.MMT4D_TYPE_BF16BF16BF16, 32, 32, 16)]
 # outer shapes chosen to hit: single tile, ragged macro tiles in M and N, K
 # tails that are not whole LDS stages, both macro-tile variants, > 8 XCD slices
 MFMA_SHAPES = [(1, 1, 2), (1, 1, 8), (3, 2, 6), (5, 7, 10), (9, 4, 18), (8, 8, 8),
@@ -54,7 +57,7 @@ MFMA_SHAPES = [(1, 1, 2), (1, 1, 8), (3, 2, 6), (5, 7, 10), (9, 4, 18), (8, 8, 8
 
 @pytest.mark.parametrize("type_flag,M0,N0,K0", MFMA_TILES)
 def test_mfma_kernels_bit_exact_on_exact_inputs(uk, cuda, type_flag, M0, N0, K0):
-    assert uk.mmt4d_info(M0, N0, K0, type_flag) == 1
+    assert uk.mmt4d_info(M0, N0, K0, type_flag | F.MMT4D_SKIP_INTERMEDIATE_ROUNDINGS) == 1
     rng = np.random.default_rng(4000 + type_flag + K0)
     for (M, N, K), acc in itertools.product(MFMA_SHAPES, (False, True)):
         case = ukref.Mmt4dCase(rng, type_flag, M, N, K, M0, N0, K0, accumulate=acc)
