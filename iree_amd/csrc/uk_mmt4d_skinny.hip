@@ -21,6 +21,8 @@
 #include "uk_common.h"
 #include "uk_mfma_cfg.h"
 
+#include <type_traits>
+
 namespace uk {
 namespace {
 
@@ -49,7 +51,9 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
   typedef typename Cfg::acc_t acc_t;
   typedef typename Cfg::out_t out_t;
   static_assert(SP % kDepth == 0, "the rolling buffer must divide the steps of a tile");
-  __shared__ out_t partial[2][kWaves][16][64];
+  // partial sums keep the accumulator's type (f32, or s32 for integer inputs)
+  typedef typename std::conditional<std::is_same<out_t, int32_t>::value, int32_t, float>::type sum_t;
+  __shared__ sum_t partial[2][kWaves][16][64];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int m0 = lane & 31, kh = lane >> 5;
@@ -59,14 +63,23 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
 
   // Right-hand side: lane offset inside a 1 KiB block, block of (j, step).
   const int lane_off = a.half_k0 ? lane * 16 : ((lane & 31) * 32 + (lane >> 5) * 16);
-  const char* rhs_lane = a.rhs + (int64_t)first * 1024 + lane_off;
-  // Steps past this wave's count read the wave's first block again (a valid
-  // address) and are multiplied by a zero left-hand side.
+  const char* rhs_lane = a.rhs + (int64_t)(count > 0 ? first : 0) * 1024 + lane_off;
+  // Steps past this wave's count still issue a load (of a valid block, so the
+  // number of loads in flight stays constant) but contribute zeros, whatever
+  // that block holds.
   auto load_block = [&](int j, int sp) -> frag_t {
     const int s = sp < count ? sp : 0;
     const int jj = j < a.N ? j : a.N - 1;
     union { int4v i; frag_t f; } u;
     u.i = *(const int4v*)(rhs_lane + (int64_t)jj * a.rhs_stride_bytes + (int64_t)s * 1024);
+    return u.f;
+  };
+  // (the zeroing happens when a block is consumed, not when it is requested:
+  // touching the loaded registers earlier would wait for the load)
+  auto live = [&](frag_t f, int sp) -> frag_t {
+    union { int4v i; frag_t f; } u;
+    u.f = f;
+    if (sp >= count) u.i = int4v{0, 0, 0, 0};
     return u.f;
   };
 
@@ -98,14 +111,14 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
     for (int v = 0; v < 16; ++v) acc[v] = 0;
 #pragma unroll
     for (int sp = 0; sp < SP; ++sp) {
-      acc = Cfg::mfma(ring[sp % kDepth], xf[sp], acc);
+      acc = Cfg::mfma(live(ring[sp % kDepth], sp), xf[sp], acc);
       // refill the slot: kDepth steps ahead, wrapping into the next tile
       __builtin_amdgcn_sched_barrier(0);
       ring[sp % kDepth] = sp + kDepth < SP ? load_block(j, sp + kDepth) : load_block(next, sp + kDepth - SP);
       __builtin_amdgcn_sched_barrier(0);
     }
     // ---- sum the 8 K slices in wave order and store -----------------------
-    out_t (*buf)[16][64] = partial[parity];
+    sum_t (*buf)[16][64] = partial[parity];
 #pragma unroll
     for (int v = 0; v < 16; ++v) buf[wave][v][lane] = acc[v];
     __syncthreads();
@@ -116,10 +129,10 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
       const int l = flat & 63, v = flat >> 6;
       const int mm = l & 31, nn = 8 * (v >> 2) + 4 * (l >> 5) + (v & 3);
       if (mm < a.M0) {
-        out_t sum = a.accumulate ? tile[mm * 32 + nn] : (out_t)0;
+        sum_t sum = a.accumulate ? (sum_t)tile[mm * 32 + nn] : (sum_t)0;
 #pragma unroll
         for (int w = 0; w < kWaves; ++w) sum += buf[w][v][l];
-        tile[mm * 32 + nn] = sum;
+        tile[mm * 32 + nn] = (out_t)sum;
       }
     }
     // The other half of `partial` serves the next tile; this half is rewritten
@@ -144,6 +157,12 @@ int mfma_k_of(uint32_t flags) {
   switch (flags & IREE_AMD_UK_FLAG_MMT4D_TYPE_MASK) {
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F32:
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16F32: return 16;
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F16:
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16BF16:
+      // one final rounding of an f32 sum: the reference's arithmetic only
+      // when intermediate roundings are skipped
+      return (flags & IREE_AMD_UK_FLAG_MMT4D_SKIP_INTERMEDIATE_ROUNDINGS) ? 16 : 0;
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F32F32F32: return 8;
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32: return 32;
     default: return 0;
   }
@@ -187,6 +206,9 @@ int launch_mmt4d_skinny(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) {
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F32: return launch_cfg<F16Cfg>(a, s);
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16F32: return launch_cfg<BF16Cfg>(a, s);
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32: return launch_cfg<S8Cfg>(a, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F32F32F32: return launch_cfg<F32Cfg>(a, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F16: return launch_cfg<F16F16Cfg>(a, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16BF16: return launch_cfg<BF16BF16Cfg>(a, s);
     default: return IREE_AMD_UK_STATUS_NOT_FOUND;
   }
 }
