@@ -312,3 +312,54 @@ def test_fused_gate_up_silu_invalid_arguments(uk, cuda):
         uk.mmt4d_silu_mul_f8e4m3(t[1:], t, t, 1, 2, 4, 16, mm, 1.0, 1.0, 1.0)    # misaligned operand
     assert e.value.status == F.STATUS_UNIMPLEMENTED
     uk.mmt4d_silu_mul_f8e4m3(t, t, t, 0, 2, 4, 16, mm, 1.0, 1.0, 1.0)             # M == 0: nothing to do
+
+
+def test_fp8_mlp_block_full_size_sampled_tokens(uk, cuda):
+    """The block at its real size (2048 tokens, hidden 4096, ffn 14336): for a
+    sample of token rows, h codes against the f64 formula on the same quantised
+    operands (within the fp8 MFMA's accumulation error), and y against f64
+    accumulation over the GPU's own h codes: |err| <= 1e-3 + 1e-2 |y|."""
+    import torch
+    M, H, Fn = 2048, 4096, 14336
+    g = torch.Generator(device="cuda")
+    g.manual_seed(99)
+    x = torch.randn(M * H, generator=g, device="cuda", dtype=torch.float16)
+    codes, scales = [], []
+    for n_el in (Fn * H, Fn * H, H * Fn):
+        w = torch.randn(n_el, generator=g, device="cuda", dtype=torch.float32) * 0.02
+        sc = float(w.abs().max()) / 448.0
+        q = torch.empty(n_el, dtype=torch.uint8, device="cuda")
+        uk.quantize_f16_to_f8e4m3(w.to(torch.float16), q, n_el, 1.0 / sc)
+        codes.append(q)
+        scales.append(sc)
+        del w
+    sg, su, sd = scales
+    sx = float(x.float().abs().max()) / 448.0
+    rows = np.array([0, 1, 31, 32, 777, 1024, 2047])
+    # reference gate/up for the sampled rows -> the scale of h
+    xq = quantize_np(x.cpu().numpy().astype(np.float32).reshape(M, H)[rows] * np.float32(1.0 / sx))
+    wg = TABLE[codes[0].cpu().numpy().reshape(Fn, H)]
+    wu = TABLE[codes[1].cpu().numpy().reshape(Fn, H)]
+    X = TABLE[xq]
+    gt = (X @ wg.T) * (sx * sg)
+    ut = (X @ wu.T) * (sx * su)
+    h = gt / (1.0 + np.exp(-gt)) * ut
+    sh = float(np.abs(h).max()) * 1.5 / 448.0          # head room for the rows not sampled
+    mlp = uk.Fp8Mlp(H, Fn, codes[0], codes[1], codes[2], sg, su, sd, sx, sh, max_tokens=M)
+    y = torch.zeros(M * H, dtype=torch.float32, device="cuda")
+    mlp(x, y, M)
+    torch.cuda.synchronize()
+    assert np.array_equal(mlp.xq.cpu().numpy().reshape(M, H)[rows], xq)
+    hq = mlp.h_tiles.cpu().numpy().reshape(M // 32, Fn // 16, 32, 16).transpose(0, 2, 1, 3).reshape(M, Fn)[rows]
+    eg = 4e-5 * (np.abs(X) @ np.abs(wg).T) * (sx * sg)
+    eu = 4e-5 * (np.abs(X) @ np.abs(wu).T) * (sx * su)
+    silu = lambda t: t / (1.0 + np.exp(-t))  # noqa: E731
+    corners = np.stack([silu(gt + a * eg) * (ut + b * eu) for a in (-1, 1) for b in (-1, 1)]) / sh
+    lo, hi = corners.min(axis=0), corners.max(axis=0)
+    pad = 1e-5 * np.maximum(np.abs(lo), np.abs(hi)) + 1e-12
+    _check_codes(hq, h / sh, lo - pad, hi + pad)
+    del wg, wu
+    wd = TABLE[codes[2].cpu().numpy().reshape(H, Fn)]
+    want = (TABLE[hq] @ wd.T) * (sh * sd)
+    got = y.cpu().numpy().reshape(M, H)[rows].astype(np.float64)
+    assert np.all(np.abs(got - want) <= ATOL + RTOL * np.abs(want)), float(np.abs(got - want).max())
