@@ -61,26 +61,39 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
   int count = a.ksteps - first;
   count = count < 0 ? 0 : (count > a.steps_per_wave ? a.steps_per_wave : count);
 
-  // Right-hand side: lane offset inside a 1 KiB block, block of (j, step).
-  const int lane_off = a.half_k0 ? lane * 16 : ((lane & 31) * 32 + (lane >> 5) * 16);
-  const char* rhs_lane = a.rhs + (int64_t)(count > 0 ? first : 0) * 1024 + lane_off;
+  // Right-hand side: lane offset inside an operand block (1 KiB; fp8: 2 KiB of
+  // four K0 = 16 tiles, of which lanes 0..31 take tiles 0, 1 and lanes 32..63
+  // tiles 2, 3 as two 16-byte pieces), block of (j, step).
+  constexpr int kSub = Cfg::kSub;
+  constexpr int kBlock = kSub * 1024;
+  const int lane_off = kSub == 2 ? ((lane >> 5) * 1024 + (lane & 31) * 16)
+                       : a.half_k0 ? lane * 16 : ((lane & 31) * 32 + (lane >> 5) * 16);
+  const char* rhs_lane = a.rhs + (int64_t)(count > 0 ? first : 0) * kBlock + lane_off;
+  auto make_frag = [](int4v lo, int4v hi) -> frag_t {
+    if constexpr (kSub == 2) {
+      return frag_t{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    } else {
+      union { int4v i; frag_t f; } u;
+      u.i = lo;
+      return u.f;
+    }
+  };
   // Steps past this wave's count still issue a load (of a valid block, so the
   // number of loads in flight stays constant) but contribute zeros, whatever
   // that block holds.
   auto load_block = [&](int j, int sp) -> frag_t {
     const int s = sp < count ? sp : 0;
     const int jj = j < a.N ? j : a.N - 1;
-    union { int4v i; frag_t f; } u;
-    u.i = *(const int4v*)(rhs_lane + (int64_t)jj * a.rhs_stride_bytes + (int64_t)s * 1024);
-    return u.f;
+    const char* p = rhs_lane + (int64_t)jj * a.rhs_stride_bytes + (int64_t)s * kBlock;
+    const int4v lo = *(const int4v*)p;
+    const int4v hi = kSub == 2 ? *(const int4v*)(p + 512) : lo;
+    return make_frag(lo, hi);
   };
   // (the zeroing happens when a block is consumed, not when it is requested:
   // touching the loaded registers earlier would wait for the load)
   auto live = [&](frag_t f, int sp) -> frag_t {
-    union { int4v i; frag_t f; } u;
-    u.f = f;
-    if (sp >= count) u.i = int4v{0, 0, 0, 0};
-    return u.f;
+    const int4v zero = {0, 0, 0, 0};
+    return sp >= count ? make_frag(zero, zero) : f;
   };
 
   // ---- first blocks of the first tile, then the left-hand side -------------
@@ -93,14 +106,21 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
 #pragma unroll
   for (int sp = 0; sp < SP; ++sp) {
     const int s = first + (sp < count ? sp : 0);
-    // K tile(s) of step s: two tiles of K0 = half the MFMA extent, or one.
-    const int64_t off = a.half_k0 ? ((int64_t)(2 * s + kh) * a.lhs_tile_bytes + m0 * 16)
-                                  : ((int64_t)s * a.lhs_tile_bytes + m0 * 32 + kh * 16);
-    int4v v = {0, 0, 0, 0};
-    if (m0 < a.M0 && sp < count) v = *(const int4v*)(a.lhs + off);
-    union { int4v i; frag_t f; } u;
-    u.i = v;
-    xf[sp] = u.f;
+    // K tile(s) of step s: two tiles of K0 = half the MFMA extent, or one;
+    // fp8: four tiles, two per lane half.
+    int4v lo = {0, 0, 0, 0}, hi = {0, 0, 0, 0};
+    if (m0 < a.M0 && sp < count) {
+      if constexpr (kSub == 2) {
+        const char* p = a.lhs + (int64_t)(4 * s + 2 * kh) * a.lhs_tile_bytes + m0 * 16;
+        lo = *(const int4v*)p;
+        hi = *(const int4v*)(p + a.lhs_tile_bytes);
+      } else {
+        const int64_t off = a.half_k0 ? ((int64_t)(2 * s + kh) * a.lhs_tile_bytes + m0 * 16)
+                                      : ((int64_t)s * a.lhs_tile_bytes + m0 * 32 + kh * 16);
+        lo = *(const int4v*)(a.lhs + off);
+      }
+    }
+    xf[sp] = make_frag(lo, hi);
   }
 
   int parity = 0;
@@ -146,10 +166,17 @@ int launch_cfg(SkinnyArgs a, hipStream_t s) {
   const int blocks = a.N < cus ? a.N : cus;
   const int per = (a.ksteps + kWaves - 1) / kWaves;
   a.steps_per_wave = per;
-  if (per <= 8) hipLaunchKernelGGL((mmt4d_skinny_kernel<Cfg, 8>), dim3(blocks), dim3(kThreads), 0, s, a);
-  else if (per <= 16) hipLaunchKernelGGL((mmt4d_skinny_kernel<Cfg, 16>), dim3(blocks), dim3(kThreads), 0, s, a);
-  else if (per <= 32) hipLaunchKernelGGL((mmt4d_skinny_kernel<Cfg, 32>), dim3(blocks), dim3(kThreads), 0, s, a);
-  else return IREE_AMD_UK_STATUS_NOT_FOUND;
+  if (per <= 8) {
+    hipLaunchKernelGGL((mmt4d_skinny_kernel<Cfg, 8>), dim3(blocks), dim3(kThreads), 0, s, a);
+  } else if (per <= 16) {
+    hipLaunchKernelGGL((mmt4d_skinny_kernel<Cfg, 16>), dim3(blocks), dim3(kThreads), 0, s, a);
+  } else if (per <= 32) {
+    // (32 fp8 steps of 8 registers each would not fit the register file)
+    if constexpr (Cfg::kSub == 2) return IREE_AMD_UK_STATUS_NOT_FOUND;
+    else hipLaunchKernelGGL((mmt4d_skinny_kernel<Cfg, 32>), dim3(blocks), dim3(kThreads), 0, s, a);
+  } else {
+    return IREE_AMD_UK_STATUS_NOT_FOUND;
+  }
   return check_hip(hipGetLastError(), "mmt4d_skinny launch");
 }
 
@@ -164,6 +191,7 @@ int mfma_k_of(uint32_t flags) {
       return (flags & IREE_AMD_UK_FLAG_MMT4D_SKIP_INTERMEDIATE_ROUNDINGS) ? 16 : 0;
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_F32F32F32: return 8;
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32: return 32;
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F8E4M3F8E4M3F32: return 64;
     default: return 0;
   }
 }
@@ -173,6 +201,7 @@ int mfma_k_of(uint32_t flags) {
 // Narrow tiles served: M0 < 32, N0 = 32, K0 = half or all of the MFMA's K extent.
 bool mmt4d_skinny_supported(uint32_t flags, int M0, int N0, int K0) {
   const int mk = mfma_k_of(flags);
+  if (mk == 64) return M0 >= 1 && M0 < 32 && N0 == 32 && K0 == 16;
   return mk && M0 >= 1 && M0 < 32 && N0 == 32 && (K0 == mk || K0 * 2 == mk);
 }
 
@@ -207,6 +236,7 @@ int launch_mmt4d_skinny(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) {
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16F32: return launch_cfg<BF16Cfg>(a, s);
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32: return launch_cfg<S8Cfg>(a, s);
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_F32F32F32: return launch_cfg<F32Cfg>(a, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F8E4M3F8E4M3F32: return launch_cfg<F8Cfg>(a, s);
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F16: return launch_cfg<F16F16Cfg>(a, s);
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16BF16: return launch_cfg<BF16BF16Cfg>(a, s);
     default: return IREE_AMD_UK_STATUS_NOT_FOUND;

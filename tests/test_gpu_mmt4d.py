@@ -103,7 +103,8 @@ def test_mfma_macro_tile_variants_bit_exact(uk, cuda, type_flag, K0, M, N):
 @pytest.mark.parametrize("type_flag,K0", [(F.MMT4D_TYPE_F16F16F32, 8), (F.MMT4D_TYPE_F16F16F32, 16),
                                           (F.MMT4D_TYPE_BF16BF16F32, 8), (F.MMT4D_TYPE_S8S8S32, 16),
                                           (F.MMT4D_TYPE_S8S8S32, 32), (F.MMT4D_TYPE_F32F32F32, 4),
-                                          (F.MMT4D_TYPE_F16F16F16, 8), (F.MMT4D_TYPE_BF16BF16BF16, 16)])
+                                          (F.MMT4D_TYPE_F16F16F16, 8), (F.MMT4D_TYPE_BF16BF16BF16, 16),
+                                          (F.MMT4D_TYPE_F8E4M3F8E4M3F32, 16)])
 def test_narrow_lhs_tiles_bit_exact(uk, cuda, type_flag, K0):
     """Narrow left-hand-side tiles (M0 < 32, one outer row: the decode shapes
     the tile-size query hands out for a static M below 32) run the streaming
@@ -113,7 +114,8 @@ def test_narrow_lhs_tiles_bit_exact(uk, cuda, type_flag, K0):
     count, a K beyond the register-resident range) must give the same bits
     through the element-wise kernel."""
     rng = np.random.default_rng(7000 + type_flag + K0)
-    mfma_k = {F.MMT4D_TYPE_S8S8S32: 32, F.MMT4D_TYPE_F32F32F32: 8}.get(type_flag, 16)
+    mfma_k = {F.MMT4D_TYPE_S8S8S32: 32, F.MMT4D_TYPE_F32F32F32: 8,
+              F.MMT4D_TYPE_F8E4M3F8E4M3F32: 64}.get(type_flag, 16)
     tps = mfma_k // K0                      # K tiles per MFMA step
     for M0 in (1, 2, 4, 8, 16):
         assert uk.mmt4d_info(M0, 32, K0, type_flag | F.MMT4D_SKIP_INTERMEDIATE_ROUNDINGS) == 1
