@@ -314,6 +314,19 @@ def extras(args, torch, iree_amd, F, synth, lhs, rhs, out):
     ex["matmul_f16_pack_mmt4d_unpack_tflops"] = round(flops / t / 1e12, 2)
     del a, b, c, ws
 
+    # the small i8 configuration, 1024^3 on row-major operands (2 packs, mmt4d,
+    # unpack = 4 launches): a latency figure, far too small for a roofline claim
+    n1k = 1024
+    a8 = torch.from_numpy(synth.uniform_int8(1, n1k * n1k)).cuda()
+    b8 = torch.from_numpy(synth.uniform_int8(2, n1k * n1k)).cuda()
+    c8 = torch.zeros(n1k * n1k, dtype=torch.int32, device="cuda")
+    ws8 = iree_amd.matmul_data_tiled(a8, b8, c8, n1k, n1k, n1k, F.MMT4D_TYPE_S8S8S32)
+    _, t = gpu_time(torch, lambda: iree_amd.matmul_data_tiled(a8, b8, c8, n1k, n1k, n1k,
+                                                              F.MMT4D_TYPE_S8S8S32, workspace=ws8),
+                    steps, warm)
+    ex["matmul_i8_1024_chain_us"] = round(t * 1e6, 1)
+    del a8, b8, c8, ws8
+
     # grouped int4 dequant matmul, decode shapes (K = 4096, N = 14336, groups of
     # 128, f16 scales, packed uint4 zero points, pre-tiled weights). Ten weight
     # sets (294 MB) rotate so that the weights come from HBM.
