@@ -208,3 +208,16 @@ def test_imports_run_pack_mmt4d_unpack_on_host_buffers(host, uk, cuda):
     assert mmt4d_fn(C.addressof(m), ctxs[1], None) != 0
     plugin.unload(self_ptr)
     assert host.live == 0
+
+
+@pytest.mark.gpu
+def test_plain_c_host_program_drives_the_plugin(cuda):
+    """plugin_host_check.c: the same protocol from a C program with no Python or
+    torch in the process (dlopen, query, load, resolve, three imports, unload)."""
+    import subprocess
+    exe = os.path.join(ROOT, "iree_amd", "plugin", "plugin_host_check")
+    if not os.path.exists(exe):
+        pytest.fail(f"{exe} is not built (run __graft_entry__.build())")
+    r = subprocess.run([exe, PLUGIN, _lib.library_path()], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "OK:" in r.stdout
