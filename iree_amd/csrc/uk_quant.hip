@@ -31,89 +31,13 @@
 //   * sums the 8 K-slices through LDS in a fixed order (deterministic).
 #include "uk_common.h"
 #include "uk_fp8.h"
+#include "uk_i4.h"
 
 #include <hip/hip_fp16.h>
 
 namespace uk {
+using namespace i4;
 namespace {
-
-typedef _Float16 half2v __attribute__((ext_vector_type(2)));
-typedef _Float16 half8 __attribute__((ext_vector_type(8)));
-typedef float floatx4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-
-constexpr int kWaves = 8;               // K-slices per workgroup
-constexpr int kThreads = kWaves * 64;
-
-struct I4Args {
-  const uint16_t* x;      // [M][K] f16
-  const uint8_t* w;       // u4, tiled or row-major
-  const uint16_t* scale;  // [N][G] f16
-  const void* zp;         // [N][G] f16 or packed u4
-  uint16_t* out;          // [M][N] f16
-  int M, N, K, G;
-  int log2_gs;            // group size = 1 << log2_gs
-  int zp_u4;
-  int tiled;
-  int n_tiles;            // ceil(N / 32)
-  int m_base;             // first activation row of this pass
-  // weight addressing of the fast kernel: byte offset of the 16 bytes that
-  // lane (nl, kc) reads for column c of tile nt in 128-k span s is
-  //   nt * K * 16 + s * span_stride + c * col_stride + kc * 16
-  uint32_t span_stride, col_stride;
-  uint32_t w_bytes;       // size of the weight buffer
-};
-
-// Position, in the tiled layout, of the byte that holds elements (n, k) and
-// (n, k+1), k even. A tile is 32 columns by 128 k (2 KiB): 64 bytes per column,
-// in which the 16 dwords of the row-major span are transposed as a 4 x 4
-// matrix, so that 16-byte chunk kc holds, as dword q, k = q*32 + kc*8 .. +8.
-__host__ __device__ inline size_t tiled_byte_index(int64_t n, int64_t k, int64_t K) {
-  const int64_t s = k >> 7, r = k & 127, q = r >> 5, kc = (r >> 3) & 3, j = r & 7;
-  return (size_t)((((n >> 5) * (K >> 7) + s) * 32 + (n & 31)) * 64 + kc * 16 + q * 4 + (j >> 1));
-}
-
-// 8 nibbles of one dword -> 8 small f16 integers (nibble - zero point), in the
-// k order [0,4,1,5,2,6,3,7] of the dword's nibbles (pairs (i, i+4) fall out of
-// one AND/OR); the activation operand is permuted the same way. `lo` is
-// 1024 + zp and `hi` 64 + zp as packed f16 pairs: 0x6400 | n is 1024 + n and
-// 0x6400 | (n << 4) is 1024 + 16 n, so (1024 + n) - lo and
-// (1024 + 16 n) / 16 - hi are both n - zp, every step exact for integer zp.
-__device__ __forceinline__ half8 dequant_dword(uint32_t w, half2v lo, half2v hi) {
-  union { uint32_t u; half2v h; } a, b, c, d;
-  const uint32_t w8 = w >> 8;
-  a.u = (w & 0x000F000Fu) | 0x64006400u;    // nibbles 0, 4
-  b.u = (w & 0x00F000F0u) | 0x64006400u;    // nibbles 1, 5 (x16)
-  c.u = (w8 & 0x000F000Fu) | 0x64006400u;   // nibbles 2, 6
-  d.u = (w8 & 0x00F000F0u) | 0x64006400u;   // nibbles 3, 7 (x16)
-  const half2v sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
-  const half2v r0 = a.h - lo, r1 = b.h * sixteenth - hi, r2 = c.h - lo, r3 = d.h * sixteenth - hi;
-  return half8{r0.x, r0.y, r1.x, r1.y, r2.x, r2.y, r3.x, r3.y};
-}
-
-// x[m][k .. k+8) (8 consecutive halves, 16 bytes) -> the same 8 halves in the
-// order [0,4,1,5,2,6,3,7].
-__device__ __forceinline__ half8 permute_x(u32x4 v) {
-  union { uint32_t u[4]; half8 h; } r;
-  // v.x = (h0,h1) v.y = (h2,h3) v.z = (h4,h5) v.w = (h6,h7)
-  r.u[0] = __builtin_amdgcn_perm(v.z, v.x, 0x05040100);  // (h0, h4)
-  r.u[1] = __builtin_amdgcn_perm(v.z, v.x, 0x07060302);  // (h1, h5)
-  r.u[2] = __builtin_amdgcn_perm(v.w, v.y, 0x05040100);  // (h2, h6)
-  r.u[3] = __builtin_amdgcn_perm(v.w, v.y, 0x07060302);  // (h3, h7)
-  return r.h;
-}
-
-// NB bytes (1 .. 16 naturally aligned, 32 aligned to 16) into NB/4 (at least 1) dwords.
-template <int NB>
-__device__ __forceinline__ void load_bits(const void* p, uint32_t* dst) {
-  if constexpr (NB == 1) dst[0] = *(const uint8_t*)p;
-  else if constexpr (NB == 2) dst[0] = *(const uint16_t*)p;
-  else if constexpr (NB == 4) dst[0] = *(const uint32_t*)p;
-  else if constexpr (NB == 8) { const u32x2 v = *(const u32x2*)p; dst[0] = v.x; dst[1] = v.y; }
-  else if constexpr (NB == 16) { const u32x4 v = *(const u32x4*)p; dst[0] = v.x; dst[1] = v.y; dst[2] = v.z; dst[3] = v.w; }
-  else { static_assert(NB == 32, "unsupported width"); load_bits<16>(p, dst); load_bits<16>((const uint8_t*)p + 16, dst + 4); }
-}
 
 // Work decomposition. A tile is 32 columns (n) of the output. Wave w of the
 // workgroup owns k in [w*KB*64, (w+1)*KB*64), walked in KB/2 spans of 128: in
@@ -259,9 +183,8 @@ __global__ __launch_bounds__(kThreads) void dequant_matmul_i4_kernel(I4Args a) {
             // such a sum would round away: they are subtracted in a second step.
             if (kZpU4) {
               const uint32_t zb = (mt.z[h][g >> 3] >> ((g & 7) * 4 + mt.zsh[h])) & 0xF;
-              lo.u = 0x64006400u | zb | (zb << 16);
-              const _Float16 c = (_Float16)(float)(64 + zb);
-              hi.h = half2v{c, c};
+              lo.u = offset_lo_bits(zb);
+              hi.u = offset_hi_bits(zb);
             } else {
               const uint32_t zb = (mt.z[h][g >> 1] >> ((g & 1) * 16)) & 0xFFFF;
               lo.u = 0x64006400u;
@@ -437,6 +360,14 @@ int launch_dequant_matmul_i4(const void* x, const void* w, const void* scale, co
   if (k_ok && gs_ok && size_ok && aligned) {
     a.w_bytes = (uint32_t)w_bytes;
     return kb == 4 ? launch_fast<4>(a, s) : launch_fast<8>(a, s);
+  }
+  if (gs_pow2 && size_ok && aligned && M <= 16) {
+    // Other K (whole 2048s that fit LDS with these rows): the per-wave-column
+    // kernel. It has a longer start-up (one wave walks all of K for its
+    // columns) but no limit on K beyond LDS capacity.
+    a.w_bytes = (uint32_t)w_bytes;
+    const int st = launch_dequant_gemv_i4(a, 0, (int)M, s);
+    if (st != IREE_AMD_UK_STATUS_NOT_FOUND) return st;
   }
   const int64_t total = M * N;
   int64_t blocks = ceil_div(total, 256);

@@ -73,6 +73,18 @@ def test_mfma_kernel_group_sizes_and_zero_point_forms(uk, cuda, K, gs, zp_u4):
         run_case(uk, M, N, K, gs, zp_u4, tiled, seed=K + gs)
 
 
+@pytest.mark.parametrize("K,gs", [(6144, 128), (8192, 64), (14336, 128), (14336, 256), (2048, 64)])
+@pytest.mark.parametrize("zp_u4", [False, True])
+def test_long_k_small_batches(uk, cuda, K, gs, zp_u4):
+    """K beyond 4096 (in whole 2048s) for the row counts whose activations fit
+    the 160 KiB of LDS, ragged N for row-major weights, and row counts that do
+    not fit (served by the element-wise kernel): all against the f64 oracle."""
+    for M, N, tiled in [(1, 64, True), (1, 50, False), (4, 96, True), (5, 47, False), (16, 32, True)]:
+        if gs < 128 and not tiled:
+            continue
+        run_case(uk, M, N, K, gs, zp_u4, tiled, seed=K + gs + M)
+
+
 def test_fractional_f16_zero_points(uk, cuda):
     run_case(uk, 5, 64, 2048, 128, False, False, seed=3, frac_zp=True)
     run_case(uk, 5, 64, 2048, 128, False, True, seed=4, frac_zp=True)
