@@ -29,17 +29,24 @@ def _check(status):
 
 
 def _ptr(t):
+    # (plain ints: the declared argtypes convert them, which is cheaper than
+    # building a c_void_p per argument)
     if t is None:
         return None
     if not t.is_cuda:
         raise ValueError("ukernel buffers must be CUDA (HIP) tensors")
-    return C.c_void_p(t.data_ptr())
+    return t.data_ptr()
+
+
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 
 
 def _stream(stream):
     if stream is None:
+        if _raw_stream is not None:
+            return _raw_stream(torch.cuda.current_device())
         stream = torch.cuda.current_stream()
-    return C.c_void_p(stream.cuda_stream)
+    return stream.cuda_stream
 
 
 def mmt4d(lhs_buffer, rhs_buffer, out_buffer, M, N, K, M0, N0, K0, flags, *,
