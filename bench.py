@@ -244,6 +244,22 @@ def extras(args, torch, iree_amd, F, synth, lhs, rhs, out):
     M1 = N1 = size // 32
     flops = 2.0 * size ** 3
 
+    # What the matrix cores sustain with NO data movement (operand fragments
+    # stay in registers), for the benchmark's own operand bits and for zeros.
+    # The rate depends on the data: the difference is the power limit, and the
+    # first figure is the practical ceiling for the mmt4d line above.
+    sink = torch.zeros(256, dtype=torch.float32, device="cuda")
+    zeros = torch.zeros(64 * 1024, dtype=torch.uint8, device="cuda")
+    rnd8 = torch.from_numpy(synth.uniform_int8(3, 64 * 1024)).cuda()
+    for name, flag, ops_buf in (("f16_bench_data", F.MMT4D_TYPE_F16F16F32, lhs),
+                                ("f16_zeros", F.MMT4D_TYPE_F16F16F32, zeros),
+                                ("i8_uniform", F.MMT4D_TYPE_S8S8S32, rnd8),
+                                ("i8_zeros", F.MMT4D_TYPE_S8S8S32, zeros)):
+        n_ops = iree_amd.mfma_probe(flag, ops_buf, 512, sink)
+        _, t = gpu_time(torch, lambda: iree_amd.mfma_probe(flag, ops_buf, 512, sink), steps, warm)
+        ex[f"mfma_register_only_{name}_tops"] = round(n_ops / t / 1e12, 1)
+    del sink, zeros, rnd8
+
     # f16 with accumulate (reads the 64 MiB accumulator as well)
     acc_flags = F.MMT4D_TYPE_F16F16F32 | F.MMT4D_ACCUMULATE | F.MMT4D_SKIP_INTERMEDIATE_ROUNDINGS
     _, t = gpu_time(torch, lambda: iree_amd.mmt4d(lhs, rhs, out, M1, N1, size // 8, 32, 32, 8, acc_flags),

@@ -13,6 +13,7 @@ from .ukernel import (  # noqa: F401
     UkError,
     dequant_matmul_i4,
     matmul_data_tiled,
+    mfma_probe,
     mmt4d,
     mmt4d_info,
     mmt4d_silu_mul_f8e4m3,

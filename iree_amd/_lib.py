@@ -113,6 +113,8 @@ def _declare(lib):
                                                        C.c_float, C.c_float, C.c_float, vp]
     lib.iree_amd_uk_scale_f32.restype = C.c_int
     lib.iree_amd_uk_scale_f32.argtypes = [vp, i64, C.c_float, vp]
+    lib.iree_amd_uk_mfma_probe.restype = C.c_int
+    lib.iree_amd_uk_mfma_probe.argtypes = [C.c_uint32, vp, i64, vp, C.POINTER(C.c_int64), vp]
     lib.iree_amd_uk_device_count.restype = C.c_int
     lib.iree_amd_uk_device_count.argtypes = [C.POINTER(C.c_int)]
     lib.iree_amd_uk_device_set.restype = C.c_int

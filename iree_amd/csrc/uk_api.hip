@@ -482,6 +482,17 @@ extern "C" int iree_amd_uk_scale_f32(void* buf_f32, iree_amd_uk_index_t n, float
   return launch_scale_f32(buf_f32, n, scale, (hipStream_t)stream);
 }
 
+extern "C" int iree_amd_uk_mfma_probe(uint32_t type_flag, const void* operands,
+                                      iree_amd_uk_index_t iters, void* sink,
+                                      int64_t* out_ops_per_launch, void* stream) {
+  if (!operands || !sink || (uintptr_t)operands % 16 || (uintptr_t)sink % 4)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "mfma_probe: null or misaligned buffer");
+  if (iters < 0 || iters > (1 << 24))
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "mfma_probe: iters out of range");
+  return launch_mfma_probe(type_flag, operands, iters, sink, out_ops_per_launch,
+                           (hipStream_t)stream);
+}
+
 //===----------------------------------------------------------------------===//
 // Thin device ABI
 //===----------------------------------------------------------------------===//

@@ -82,6 +82,8 @@ int launch_silu_mul_quantize_tiled(const void* acc, int64_t acc_stride0, int64_t
                                    int64_t N1, float gate_scale, float up_scale,
                                    float inv_out_scale, hipStream_t s);
 int launch_scale_f32(void* buf, int64_t n, float scale, hipStream_t s);
+int launch_mfma_probe(uint32_t type_flag, const void* operands, int64_t iters, void* sink,
+                      int64_t* out_ops_per_launch, hipStream_t s);
 
 // Number of compute units of the current device (cached per device).
 int device_cu_count();

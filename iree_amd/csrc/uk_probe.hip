@@ -1,0 +1,77 @@
+// Measurement aid: the MFMA issue pattern of the mmt4d kernel (a wave holds 4
+// A fragments and 4 B fragments and updates its 4 x 4 accumulator blocks once
+// per K-step) with ALL data movement removed: the fragments are loaded from a
+// small buffer once and stay in registers. What it sustains is the ceiling of
+// the matrix cores for operands with that bit pattern: on MI355X the rate
+// depends strongly on the data (constant operands reach the nominal peak,
+// random ones far less: the pipe is power-limited by operand toggling).
+#include "uk_common.h"
+#include "uk_mfma_cfg.h"
+
+namespace uk {
+namespace {
+
+template <typename Cfg>
+__global__ __launch_bounds__(256) void mfma_probe_kernel(const char* operands, int64_t iters, float* sink) {
+  typedef typename Cfg::frag_t frag_t;
+  typedef typename Cfg::acc_t acc_t;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  constexpr int kFragBytes = sizeof(frag_t);
+  // 8 fragments per wave: operands[(wave * 8 + f) * 64 + lane]
+  frag_t a[4], b[4];
+#pragma unroll
+  for (int f = 0; f < 4; ++f) {
+    a[f] = *(const frag_t*)(operands + ((size_t)(wave * 8 + f) * 64 + lane) * kFragBytes);
+    b[f] = *(const frag_t*)(operands + ((size_t)(wave * 8 + 4 + f) * 64 + lane) * kFragBytes);
+  }
+  acc_t acc[4][4];
+#pragma unroll
+  for (int x = 0; x < 4; ++x)
+#pragma unroll
+    for (int y = 0; y < 4; ++y)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[x][y][v] = 0;
+  for (int64_t it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int x = 0; x < 4; ++x)
+#pragma unroll
+      for (int y = 0; y < 4; ++y) acc[x][y] = Cfg::mfma(a[x], b[y], acc[x][y]);
+  }
+  // keep the result alive without storing it in the common case
+  float s = 0.f;
+#pragma unroll
+  for (int x = 0; x < 4; ++x)
+#pragma unroll
+    for (int y = 0; y < 4; ++y)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) s += (float)acc[x][y][v];
+  if (s == 12345.678f) sink[threadIdx.x] = s;
+}
+
+template <typename Cfg>
+int launch(const void* operands, int64_t iters, void* sink, int blocks, hipStream_t s) {
+  hipLaunchKernelGGL((mfma_probe_kernel<Cfg>), dim3(blocks), dim3(256), 0, s, (const char*)operands,
+                     iters, (float*)sink);
+  return check_hip(hipGetLastError(), "mfma_probe launch");
+}
+
+}  // namespace
+
+int launch_mfma_probe(uint32_t type_flag, const void* operands, int64_t iters, void* sink,
+                      int64_t* out_ops_per_launch, hipStream_t s) {
+  const int blocks = device_cu_count();   // one workgroup of 4 waves per compute unit, as the large tile
+  int st;
+  int64_t k;
+  switch (type_flag & IREE_AMD_UK_FLAG_MMT4D_TYPE_MASK) {
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F32: st = launch<F16Cfg>(operands, iters, sink, blocks, s); k = 16; break;
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16F32: st = launch<BF16Cfg>(operands, iters, sink, blocks, s); k = 16; break;
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32: st = launch<S8Cfg>(operands, iters, sink, blocks, s); k = 32; break;
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F8E4M3F8E4M3F32: st = launch<F8Cfg>(operands, iters, sink, blocks, s); k = 64; break;
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F32F32F32: st = launch<F32Cfg>(operands, iters, sink, blocks, s); k = 8; break;
+    default: return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "mfma_probe: type has no MFMA kernel");
+  }
+  if (out_ops_per_launch) *out_ops_per_launch = (int64_t)blocks * 4 * iters * 16 * 2 * 32 * 32 * k;
+  return st;
+}
+
+}  // namespace uk

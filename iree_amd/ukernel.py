@@ -175,6 +175,16 @@ def scale_f32(buf, n, scale, stream=None):
     _check(load_library().iree_amd_uk_scale_f32(_ptr(buf), n, scale, _stream(stream)))
 
 
+def mfma_probe(type_flag, operands, iters, sink, stream=None):
+    """Register-only matrix-core loop on the bit content of ``operands`` (at
+    least 64 KiB); returns the operation count (2 per multiply-add) of the
+    launch. A measurement aid, not part of the reference's interface."""
+    ops = C.c_int64(0)
+    _check(load_library().iree_amd_uk_mfma_probe(type_flag, _ptr(operands), iters, _ptr(sink),
+                                                 C.byref(ops), _stream(stream)))
+    return ops.value
+
+
 # ---------------------------------------------------------------------------
 # The reference's end-to-end chain: pack LHS, pack RHS (inner+outer transposed),
 # [pack accumulator], mmt4d, unpack

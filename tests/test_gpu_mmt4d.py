@@ -299,3 +299,25 @@ def test_host_pointer_variants(uk, cuda):
     p = ucase.params(ukref.ptr(ucase.inp).value, ukref.ptr(out).value)
     assert lib.iree_amd_uk_unpack_host(C.byref(p)) == 0
     assert np.array_equal(out, ucase.run_oracle())
+
+
+@pytest.mark.gpu
+def test_mfma_probe_runs_and_counts_operations(uk, cuda):
+    """The register-only matrix-core loop bench.py times: it launches for every
+    type with a matrix-core kernel, reports 2 operations per multiply-add of
+    one 4-wave workgroup per compute unit, leaves its sink alone, and refuses
+    types without such a kernel."""
+    import torch
+    ops = torch.zeros(64 * 1024, dtype=torch.uint8, device=cuda)
+    sink = torch.zeros(256, dtype=torch.float32, device=cuda)
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    for flag, k in ((F.MMT4D_TYPE_F16F16F32, 16), (F.MMT4D_TYPE_BF16BF16F32, 16), (F.MMT4D_TYPE_S8S8S32, 32),
+                    (F.MMT4D_TYPE_F8E4M3F8E4M3F32, 64), (F.MMT4D_TYPE_F32F32F32, 8)):
+        n = uk.mfma_probe(flag, ops, 7, sink)
+        assert n == cus * 4 * 7 * 16 * 2 * 32 * 32 * k
+    torch.cuda.synchronize()
+    assert float(sink.abs().sum()) == 0.0
+    with pytest.raises(uk.UkError):
+        uk.mfma_probe(F.MMT4D_TYPE_S16S16S32, ops, 7, sink)
+    with pytest.raises(uk.UkError):
+        uk.mfma_probe(F.MMT4D_TYPE_F16F16F32, ops, -1, sink)
