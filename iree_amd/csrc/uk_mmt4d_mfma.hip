@@ -42,6 +42,8 @@
 #include "uk_fp8.h"
 #include "uk_mfma_cfg.h"
 
+#include <type_traits>
+
 namespace uk {
 namespace {
 
@@ -77,20 +79,30 @@ __device__ __forceinline__ void wait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
-// Pins the issue order of one basic block: kSlots times {1 MFMA, a share of the
-// kVmem vector-memory loads, a share of the kDsr LDS reads}, then the remaining
-// MFMAs. Memory instructions issued right behind an MFMA run in its shadow.
-template <int kMfma, int kVmem, int kDsr, int kSlots, int I = 0>
-__device__ __forceinline__ void interleave_issue() {
-  if constexpr (I < kSlots) {
+// Share of `n` items that falls to slot `i` of `slots` when they are spread evenly.
+constexpr int share(int n, int slots, int i) { return (i + 1) * n / slots - i * n / slots; }
+
+// Pins the issue order of one basic block to kMfma times {1 MFMA, its share of
+// the kDsr LDS reads, its share of the kVmem vector-memory loads}. A memory
+// instruction issued right behind an MFMA runs in its shadow; spreading them
+// keeps a wave (which issues in order) from queueing behind a burst of loads
+// while the matrix pipe runs dry. The LDS reads go behind the first kDsrMfma
+// MFMAs only: the block that follows waits for the LAST read issued (LDS reads
+// retire in order and the compiler waits for all of them), so the reads must
+// be done while MFMAs of this block are still queued. The LDS reads and the
+// direct-to-LDS loads must appear in the source in this same order: the
+// compiler keeps their relative order (they may alias).
+template <int kMfma, int kDsrMfma, int kDsr, int kVmem, int kInstrPerDsr, int I = 0>
+__device__ __forceinline__ void spread_issue() {
+  if constexpr (I < kMfma) {
     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-    constexpr int v = (kVmem + kSlots - 1 - I) / kSlots;
+    if constexpr (I < kDsrMfma) {
+      constexpr int d = share(kDsr, kDsrMfma, I) * kInstrPerDsr;
+      if constexpr (d > 0) __builtin_amdgcn_sched_group_barrier(0x100, d, 0);
+    }
+    constexpr int v = share(kVmem, kMfma, I);
     if constexpr (v > 0) __builtin_amdgcn_sched_group_barrier(0x020, v, 0);
-    constexpr int d = (kDsr + kSlots - 1 - I) / kSlots;
-    if constexpr (d > 0) __builtin_amdgcn_sched_group_barrier(0x100, d, 0);
-    interleave_issue<kMfma, kVmem, kDsr, kSlots, I + 1>();
-  } else if constexpr (kMfma > kSlots) {
-    __builtin_amdgcn_sched_group_barrier(0x008, kMfma - kSlots, 0);
+    spread_issue<kMfma, kDsrMfma, kDsr, kVmem, kInstrPerDsr, I + 1>();
   }
 }
 
@@ -116,11 +128,13 @@ __device__ __forceinline__ void tile_coord(int bid, int tiles_m, int tiles_n,
 
 // K-loop organisation. LDS is a ring of kRing slots; slot (ks % kRing) holds
 // K-step ks: the TM blocks of A followed by the TN blocks of B, 1 KiB each, in
-// MFMA lane order. Waves synchronise once every kSync K-steps; right after
-// that barrier each wave issues its share of the direct-to-LDS loads for the
-// kSync K-steps that lie kAhead = kRing - kSync steps ahead, so up to kAhead
-// K-steps of loads are in flight behind the one being multiplied. Operand
-// fragments are read from LDS one K-step ahead of the MFMAs that use them.
+// MFMA lane order. Waves synchronise once every kSync K-steps, at the start of
+// the last K-step of a group: the barrier publishes the next group's data and
+// frees the slots of the group just read. EVERY K-step then has the same
+// memory work, spread evenly behind its MFMAs: the LDS reads of the next
+// K-step's fragments, and this wave's share of the direct-to-LDS loads of the
+// K-step that lies kRing - kSync + 1 ahead (into a slot the last barrier
+// freed). Loads therefore stay in flight for kRing - 2 kSync + 1 K-steps.
 // kOcc: waves per SIMD the register allocation must leave room for (2 = two
 // workgroups of 4 waves resident on one compute unit).
 // kSiluMul: instead of storing the accumulators, treat even outer columns as
@@ -140,8 +154,17 @@ __global__ __launch_bounds__(kThreads, kOcc) void mmt4d_mfma_kernel(MfmaArgs a) 
   constexpr int kARowsPerWave = TM / 4, kBRowsPerWave = TN / 4;
   constexpr int kLoadsPerStep = (kARowsPerWave + kBRowsPerWave) * kSub;  // per wave
   constexpr int kBody = (kSync % 2) ? 2 * kSync : kSync;        // K-steps per unrolled body
-  static_assert(kAhead >= kSync && kAhead % kSync == 0, "ring must hold whole sync groups");
-  static_assert((kAhead - kSync) * kLoadsPerStep < 64, "too many loads in flight for vmcnt");
+  constexpr int kFrags = WM + WN;               // operand fragments a wave reads per K-step
+  constexpr int kPro = kRing - kSync + 1;       // K-steps loaded before the loop starts
+  // MFMAs of a whole K-step / of the part behind a barrier, and how many of
+  // them (from the front) get fragment reads slipped in behind them: the last
+  // third or so stays free so that the reads have landed when the step ends.
+  constexpr int kMfmaAll = WM * WN, kMfmaRest = (WM - 1) * WN;
+  constexpr int kReadAll = kMfmaAll - (kMfmaAll >= 8 ? 6 : kMfmaAll / 2);
+  constexpr int kReadRest = kMfmaRest - (kMfmaRest >= 8 ? 4 : kMfmaRest / 2);
+  static_assert(kAhead >= kSync, "ring must hold two sync groups");
+  static_assert(kPro >= kBody - 1, "the loop's remainder must already be in the ring");
+  static_assert((kPro - kSync) * kLoadsPerStep < 64, "too many loads in flight for vmcnt");
   extern __shared__ __attribute__((aligned(1024))) char lds[];
 
   const int lane = threadIdx.x & 63;
@@ -198,21 +221,23 @@ __global__ __launch_bounds__(kThreads, kOcc) void mmt4d_mfma_kernel(MfmaArgs a) 
         for (int v = 0; v < 16; ++v) acc[x][y][v] = 0;
   }
 
-  // This wave's share of the loads of K-step `ks` into ring slot `slot`.
-  auto issue_step = [&](int ks, int slot) {
+  // Load `d` (of kLoadsPerStep) of this wave's share of K-step `ks` into ring
+  // slot `slot`: its rows of A first, then its rows of B, kSub pieces each.
+  auto issue_one = [&](int ks, int slot, int d) {
     char* base = lds + slot * kSlotBytes;
+    const int r = d / kSub, j = d % kSub;
+    if (r < kARowsPerWave) {
+      load_block_to_lds(a_src[r] + (int64_t)ks * kBlockBytes + j * kPieceStride,
+                        base + (wave * kARowsPerWave + r) * kBlockBytes + j * kPieceBytes);
+    } else {
+      const int rb = r - kARowsPerWave;
+      load_block_to_lds(b_src[rb] + (int64_t)ks * kBlockBytes + j * kPieceStride,
+                        base + kABytes + (wave * kBRowsPerWave + rb) * kBlockBytes + j * kPieceBytes);
+    }
+  };
+  auto issue_step = [&](int ks, int slot) {
 #pragma unroll
-    for (int r = 0; r < kARowsPerWave; ++r)
-#pragma unroll
-      for (int j = 0; j < kSub; ++j)
-        load_block_to_lds(a_src[r] + (int64_t)ks * kBlockBytes + j * kPieceStride,
-                          base + (wave * kARowsPerWave + r) * kBlockBytes + j * kPieceBytes);
-#pragma unroll
-    for (int r = 0; r < kBRowsPerWave; ++r)
-#pragma unroll
-      for (int j = 0; j < kSub; ++j)
-        load_block_to_lds(b_src[r] + (int64_t)ks * kBlockBytes + j * kPieceStride,
-                          base + kABytes + (wave * kBRowsPerWave + r) * kBlockBytes + j * kPieceBytes);
+    for (int d = 0; d < kLoadsPerStep; ++d) issue_one(ks, slot, d);
   };
   auto read_frag = [&](const char* p) -> frag_t {
     if constexpr (kSub == 1) {
@@ -222,13 +247,34 @@ __global__ __launch_bounds__(kThreads, kOcc) void mmt4d_mfma_kernel(MfmaArgs a) 
       return frag_t{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
     }
   };
+  // Fragment `r` (of kFrags) of this wave for the K-step in `slot`: its WN
+  // blocks of B, then its WM blocks of A. The MFMAs run over A blocks in the
+  // outer loop, so the fragments read last (A blocks 1..) are needed last.
+  auto read_one = [&](int slot, int r, frag_t (&fa)[WM], frag_t (&fb)[WN]) {
+    const char* s0 = lds + slot * kSlotBytes + lane * 16;
+    if (r < WN) fb[r] = read_frag(s0 + kABytes + (wn * WN + r) * kBlockBytes);
+    else fa[r - WN] = read_frag(s0 + (wm * WM + r - WN) * kBlockBytes);
+  };
   auto read_frags = [&](int slot, frag_t (&fa)[WM], frag_t (&fb)[WN]) {
-    const char* sa = lds + slot * kSlotBytes + (wm * WM) * kBlockBytes + lane * 16;
-    const char* sb = lds + slot * kSlotBytes + kABytes + (wn * WN) * kBlockBytes + lane * 16;
 #pragma unroll
-    for (int x = 0; x < WM; ++x) fa[x] = read_frag(sa + x * kBlockBytes);
+    for (int r = 0; r < kFrags; ++r) read_one(slot, r, fa, fb);
+  };
+  // The memory work of one K-step, in the order spread_issue<nM, nR, ...> pins
+  // it behind nM MFMAs: fragment reads of `read_slot` (behind the first nR
+  // MFMAs), loads of K-step `ks`.
+  auto memory_ops = [&](auto n_mfma, auto n_read_mfma, int ks, int load_slot, int read_slot,
+                        frag_t (&na)[WM], frag_t (&nb)[WN]) {
+    constexpr int nM = decltype(n_mfma)::value, nR = decltype(n_read_mfma)::value;
 #pragma unroll
-    for (int y = 0; y < WN; ++y) fb[y] = read_frag(sb + y * kBlockBytes);
+    for (int i = 0; i < nM; ++i) {
+      if (i < nR) {
+#pragma unroll
+        for (int r = i * kFrags / nR; r < (i + 1) * kFrags / nR; ++r) read_one(read_slot, r, na, nb);
+      }
+#pragma unroll
+      for (int d = i * kLoadsPerStep / nM; d < (i + 1) * kLoadsPerStep / nM; ++d)
+        issue_one(ks, load_slot, d);
+    }
   };
   // MFMAs of block rows [x0, x1) of this wave's WM x WN blocks.
   auto multiply_rows = [&](const frag_t (&fa)[WM], const frag_t (&fb)[WN], int x0, int x1) {
@@ -247,62 +293,55 @@ __global__ __launch_bounds__(kThreads, kOcc) void mmt4d_mfma_kernel(MfmaArgs a) 
   int done = 0;  // K-steps multiplied so far
   if (T > kRing) {
     // ---- pipelined path -------------------------------------------------
-    int issue_ks = 0, issue_slot = 0;   // next K-step to load and its slot
-    int read_slot = 0;                  // slot of K-step `done`
+    int issue_ks = kPro, issue_slot = kPro % kRing;   // next K-step to load and its slot
+    int read_slot = 0;                                // slot of K-step `done`
 #pragma unroll 1
-    for (; issue_ks < kRing; ++issue_ks) issue_step(issue_ks, issue_ks);
-    issue_slot = 0;  // kRing % kRing
-    wait_vmcnt<(kAhead) * kLoadsPerStep>();  // the first kSync K-steps have landed
+    for (int ks = 0; ks < kPro; ++ks) issue_step(ks, ks);
+    wait_vmcnt<(kPro - kSync) * kLoadsPerStep>();  // the first kSync K-steps have landed
     __syncthreads();
     read_frags(0, fa[0], fb[0]);
-    // Each body multiplies kBody K-steps; `base` is the first of them. The
-    // loop runs while another whole body remains AFTER this one needs no
-    // special casing; the last bodies and the remainder are handled below.
+    // Each body multiplies kBody K-steps (whole sync groups, and an even
+    // number so that the fragment double buffer returns to fa[0]/fb[0]).
     while (done + kBody <= T) {
 #pragma unroll
       for (int g = 0; g < kBody; ++g) {
         const int p = g & 1;
         const bool sync_point = (g % kSync) == kSync - 1;
         int next_slot = read_slot + 1; if (next_slot == kRing) next_slot = 0;
+        // Past the end of K the last K-step is loaded again (into a slot nobody
+        // reads any more): that keeps the number of loads in flight, and with
+        // it the vmcnt arithmetic, constant.
+        const int load_ks = issue_ks < T ? issue_ks : T - 1;
         if (!sync_point) {
-          read_frags(next_slot, fa[p ^ 1], fb[p ^ 1]);
+          memory_ops(std::integral_constant<int, kMfmaAll>(), std::integral_constant<int, kReadAll>(),
+                     load_ks, issue_slot, next_slot, fa[p ^ 1], fb[p ^ 1]);
           multiply(fa[p], fb[p]);
-          // Issue order: one LDS read slipped in behind each of the first
-          // MFMAs (an LDS read issues in the shadow of the running MFMA),
-          // then the rest of the MFMAs back to back.
-          constexpr int kReads = (WM + WN) * kSub;
-          interleave_issue<WM * WN, 0, kReads, (WM * WN < kReads ? WM * WN : kReads)>();
+          spread_issue<kMfmaAll, kReadAll, kFrags, kLoadsPerStep, kSub>();
         } else {
           // The first row of MFMAs goes ahead of the barrier so that the
-          // matrix pipe has work while the waves meet. All reads of K-steps
-          // <= done+g are complete once fa[p]/fb[p] have arrived; the barrier
-          // then frees the slots of this sync group and publishes the next
-          // group's data. The scheduling fences keep the compiler from moving
-          // MFMAs across the synchronisation sequence.
+          // matrix pipe has work while the waves meet. This wave's reads of
+          // K-steps <= done+g are complete once fa[p]/fb[p] have arrived, and
+          // its loads of the next sync group once vmcnt has dropped to what
+          // was issued since: the barrier then frees the slots of this group
+          // and publishes the next group's data. The scheduling fences keep
+          // the compiler from moving anything across the sequence.
           __builtin_amdgcn_sched_barrier(0);
           multiply_rows(fa[p], fb[p], 0, 1);
           __builtin_amdgcn_sched_barrier(0);
           asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-          wait_vmcnt<(kAhead - kSync) * kLoadsPerStep>();
-          __syncthreads();
+          wait_vmcnt<(kRing - 2 * kSync) * kLoadsPerStep>();
+          // A bare barrier: __syncthreads() carries a release fence for which
+          // the compiler drains every direct-to-LDS load still in flight.
+          __builtin_amdgcn_s_barrier();
           __builtin_amdgcn_sched_barrier(0);
-          // Loads for the K-steps kAhead beyond this sync group go into the
-          // slots it just vacated. Past the end of K the last K-step is loaded
-          // again (into a slot nobody reads any more): that keeps the number
-          // of loads in flight, and with it the vmcnt arithmetic, constant.
-#pragma unroll
-          for (int q = 0; q < kSync; ++q) {
-            issue_step(issue_ks < T ? issue_ks : T - 1, issue_slot);
-            ++issue_ks;
-            ++issue_slot; if (issue_slot == kRing) issue_slot = 0;
-          }
-          read_frags(next_slot, fa[p ^ 1], fb[p ^ 1]);
+          memory_ops(std::integral_constant<int, kMfmaRest>(), std::integral_constant<int, kReadRest>(),
+                     load_ks, issue_slot, next_slot, fa[p ^ 1], fb[p ^ 1]);
           multiply_rows(fa[p], fb[p], 1, WM);
-          constexpr int kDma = kSync * kLoadsPerStep, kMma = (WM - 1) * WN, kDsr = (WM + WN) * kSub;
-          constexpr int kSlots = kMma < kDsr ? kMma : kDsr;
-          interleave_issue<kMma, kDma, kDsr, kSlots>();
+          spread_issue<kMfmaRest, kReadRest, kFrags, kLoadsPerStep, kSub>();
           __builtin_amdgcn_sched_barrier(0);
         }
+        ++issue_ks;
+        ++issue_slot; if (issue_slot == kRing) issue_slot = 0;
         read_slot = next_slot;
       }
       done += kBody;
