@@ -47,7 +47,6 @@
 namespace uk {
 namespace {
 
-constexpr int kThreads = 256;
 constexpr int kPieceBytes = 1024;   // what one 64-lane 128-bit load moves
 
 struct MfmaArgs {
@@ -66,11 +65,19 @@ struct MfmaArgs {
   float gate_scale, up_scale, inv_out_scale;
 };
 
-__device__ __forceinline__ void load_block_to_lds(const char* gptr, char* lds) {
-  // 64 lanes x 16 bytes -> lds[0..1024) in lane order; gptr is per lane.
-  __builtin_amdgcn_global_load_lds(
-      (const __attribute__((address_space(1))) void*)gptr,
-      (__attribute__((address_space(3))) void*)lds, 16, 0, 0);
+__device__ __forceinline__ void load_block_to_lds(__amdgpu_buffer_rsrc_t row, uint32_t lane_off,
+                                                  uint32_t block_off, char* lds) {
+  // 64 lanes x 16 bytes -> lds[0..1024) in lane order, from byte
+  // block_off + lane_off of the operand row `row` describes. The row base and
+  // block_off live in scalar registers and lane_off never changes, so a load
+  // costs no per-lane address arithmetic.
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(row, (__attribute__((address_space(3))) void*)lds, 16,
+                                           lane_off, block_off, 0, 0);
+}
+
+// Buffer descriptor of one operand row (its length is checked on the host).
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t row_descriptor(const char* row) {
+  return __builtin_amdgcn_make_buffer_rsrc((void*)row, 0, 0x7FFFFFFF, 0x00020000);
 }
 
 template <int N>
@@ -140,18 +147,21 @@ __device__ __forceinline__ void tile_coord(int bid, int tiles_m, int tiles_n,
 // kSiluMul: instead of storing the accumulators, treat even outer columns as
 // gate and the following odd ones as up, and store e4m3(silu(gate) * up) as
 // left-hand-side tiles 32x16 of the next matmul (one byte per element).
-template <typename Cfg, int WM, int WN, int kRing, int kSync, int kOcc = 1, bool kSiluMul = false>
-__global__ __launch_bounds__(kThreads, kOcc) void mmt4d_mfma_kernel(MfmaArgs a) {
+template <typename Cfg, int WM, int WN, int kRing, int kSync, int kOcc = 1, bool kSiluMul = false,
+          int kWavesN = 2>
+__global__ __launch_bounds__(128 * kWavesN, kOcc) void mmt4d_mfma_kernel(MfmaArgs a) {
   typedef typename Cfg::frag_t frag_t;
   typedef typename Cfg::acc_t acc_t;
   typedef typename Cfg::out_t out_t;
-  constexpr int TM = 2 * WM, TN = 2 * WN;      // outer tiles per workgroup
+  constexpr int kWaves = 2 * kWavesN;                // a 2 x kWavesN grid of waves
+  constexpr int TM = 2 * WM, TN = kWavesN * WN;      // outer tiles per workgroup
+  static_assert(TM % kWaves == 0 && TN % kWaves == 0, "every wave loads whole operand rows");
   constexpr int kSub = Cfg::kSub;
   constexpr int kBlockBytes = kSub * kPieceBytes;   // one 32-row operand block of one K-step
   constexpr int kABytes = TM * kBlockBytes;
   constexpr int kSlotBytes = (TM + TN) * kBlockBytes;
   constexpr int kAhead = kRing - kSync;
-  constexpr int kARowsPerWave = TM / 4, kBRowsPerWave = TN / 4;
+  constexpr int kARowsPerWave = TM / kWaves, kBRowsPerWave = TN / kWaves;
   constexpr int kLoadsPerStep = (kARowsPerWave + kBRowsPerWave) * kSub;  // per wave
   constexpr int kBody = (kSync % 2) ? 2 * kSync : kSync;        // K-steps per unrolled body
   constexpr int kFrags = WM + WN;               // operand fragments a wave reads per K-step
@@ -169,7 +179,7 @@ __global__ __launch_bounds__(kThreads, kOcc) void mmt4d_mfma_kernel(MfmaArgs a) 
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / kWavesN, wn = wave % kWavesN;
   int tm, tn;
   tile_coord(blockIdx.x, a.tiles_m, a.tiles_n, &tm, &tn);
   const int i_base = tm * TM, j_base = tn * TN;
@@ -177,25 +187,24 @@ __global__ __launch_bounds__(kThreads, kOcc) void mmt4d_mfma_kernel(MfmaArgs a) 
 
   // Per-lane byte offset inside an operand block in global memory (of its
   // first piece; with two pieces the second lies one 512-byte tile further).
-  const int lane_off = kSub == 2 ? ((lane >> 5) * 1024 + (lane & 31) * 16)
+  const uint32_t lane_off = kSub == 2 ? ((lane >> 5) * 1024 + (lane & 31) * 16)
                        : a.half_k0 ? lane * 16 : ((lane & 31) * 32 + (lane >> 5) * 16);
   constexpr int kPieceStride = 512;
 
   // Rows this wave copies: TM/4 rows of A and TN/4 rows of B. Out-of-range
   // rows are clamped to the last valid one (loaded, never stored).
-  const char* a_src[kARowsPerWave];
-  const char* b_src[kBRowsPerWave];
+  __amdgpu_buffer_rsrc_t a_src[kARowsPerWave], b_src[kBRowsPerWave];
 #pragma unroll
   for (int r = 0; r < kARowsPerWave; ++r) {
     int i = i_base + wave * kARowsPerWave + r;
     i = i < a.M ? i : a.M - 1;
-    a_src[r] = a.lhs + (int64_t)i * a.lhs_stride_bytes + lane_off;
+    a_src[r] = row_descriptor(a.lhs + (int64_t)i * a.lhs_stride_bytes);
   }
 #pragma unroll
   for (int r = 0; r < kBRowsPerWave; ++r) {
     int j = j_base + wave * kBRowsPerWave + r;
     j = j < a.N ? j : a.N - 1;
-    b_src[r] = a.rhs + (int64_t)j * a.rhs_stride_bytes + lane_off;
+    b_src[r] = row_descriptor(a.rhs + (int64_t)j * a.rhs_stride_bytes);
   }
 
   acc_t acc[WM][WN];
@@ -227,11 +236,11 @@ __global__ __launch_bounds__(kThreads, kOcc) void mmt4d_mfma_kernel(MfmaArgs a) 
     char* base = lds + slot * kSlotBytes;
     const int r = d / kSub, j = d % kSub;
     if (r < kARowsPerWave) {
-      load_block_to_lds(a_src[r] + (int64_t)ks * kBlockBytes + j * kPieceStride,
+      load_block_to_lds(a_src[r], lane_off, (uint32_t)ks * kBlockBytes + j * kPieceStride,
                         base + (wave * kARowsPerWave + r) * kBlockBytes + j * kPieceBytes);
     } else {
       const int rb = r - kARowsPerWave;
-      load_block_to_lds(b_src[rb] + (int64_t)ks * kBlockBytes + j * kPieceStride,
+      load_block_to_lds(b_src[rb], lane_off, (uint32_t)ks * kBlockBytes + j * kPieceStride,
                         base + kABytes + (wave * kBRowsPerWave + rb) * kBlockBytes + j * kPieceBytes);
     }
   };
@@ -298,7 +307,7 @@ __global__ __launch_bounds__(kThreads, kOcc) void mmt4d_mfma_kernel(MfmaArgs a) 
 #pragma unroll 1
     for (int ks = 0; ks < kPro; ++ks) issue_step(ks, ks);
     wait_vmcnt<(kPro - kSync) * kLoadsPerStep>();  // the first kSync K-steps have landed
-    __syncthreads();
+    __builtin_amdgcn_s_barrier();                  // (bare, as in the loop below)
     read_frags(0, fa[0], fb[0]);
     // Each body multiplies kBody K-steps (whole sync groups, and an even
     // number so that the fragment double buffer returns to fa[0]/fb[0]).
@@ -452,24 +461,25 @@ __global__ __launch_bounds__(kThreads, kOcc) void mmt4d_mfma_kernel(MfmaArgs a) 
     }
 }
 
-template <typename Cfg, int WM, int WN, int kRing, int kSync, int kOcc = 1, bool kSiluMul = false>
+template <typename Cfg, int WM, int WN, int kRing, int kSync, int kOcc = 1, bool kSiluMul = false,
+          int kWavesN = 2>
 int launch_variant(const MfmaArgs& a0, hipStream_t s) {
   MfmaArgs a = a0;
-  constexpr int TM = 2 * WM, TN = 2 * WN;
+  constexpr int TM = 2 * WM, TN = kWavesN * WN;
   a.tiles_m = (a.M + TM - 1) / TM;
   a.tiles_n = (a.N + TN - 1) / TN;
   const int64_t blocks = (int64_t)a.tiles_m * a.tiles_n;
   if (blocks > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
   constexpr int lds_bytes = kRing * (TM + TN) * Cfg::kSub * kPieceBytes;
   static_assert(lds_bytes <= 160 * 1024, "LDS ring exceeds 160 KiB");
-  auto kernel = mmt4d_mfma_kernel<Cfg, WM, WN, kRing, kSync, kOcc, kSiluMul>;
+  auto kernel = mmt4d_mfma_kernel<Cfg, WM, WN, kRing, kSync, kOcc, kSiluMul, kWavesN>;
   static bool attr_set = false;  // benign race: the call is idempotent
   if (!attr_set) {
     UK_RETURN_IF_HIP(hipFuncSetAttribute((const void*)kernel,
                                          hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes));
     attr_set = true;
   }
-  hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(kThreads), lds_bytes, s, a);
+  hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(128 * kWavesN), lds_bytes, s, a);
   return check_hip(hipGetLastError(), "mmt4d_mfma launch");
 }
 
@@ -564,7 +574,8 @@ int make_args(const iree_amd_uk_mmt4d_params_t& p, int out_elem_bytes, MfmaArgs*
   const char* rhs = (const char*)p.rhs_buffer + p.rhs_offset * eb;
   if (((uintptr_t)lhs | (uintptr_t)rhs) % 16) return IREE_AMD_UK_STATUS_NOT_FOUND;
   if ((p.lhs_stride0 * eb) % 16 || (p.rhs_stride0 * eb) % 16) return IREE_AMD_UK_STATUS_NOT_FOUND;
-  if (k_elems / sv.mfma_k > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  // (the kernel addresses an operand row with 32-bit byte offsets)
+  if (k_elems * eb + 4096 > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
   MfmaArgs& a = *out_args;
   a.lhs = lhs; a.rhs = rhs;
   a.out = (char*)p.out_buffer + p.out_offset * out_elem_bytes;
