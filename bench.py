@@ -38,14 +38,24 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # by what the counters read for a copy kernel of known size (fetch x 2.0, write
 # x 1.0): 200.2 MiB read (each of the 8 XCD L2s fetches its own operand panels;
 # most of it is served by the 256 MiB memory-side cache) + 72.0 MiB written.
-MEASURED_TRAFFIC_BYTES = {"mmt4d_f16_4096": 285.4e6}
+MEASURED_TRAFFIC_BYTES = {"mmt4d_f16_4096": 277.0e6}
+
+
+# After an idle spell (or CPU-only work) the GPU's power management needs about
+# 10 ms of load before launches reach their sustained duration (a 4096^3 f16
+# mmt4d: 135-145 us during the ramp, 117 us from then on, flat over thousands
+# of launches). Every measurement keeps the device busy with the measured
+# kernel itself for this long before its warmup steps.
+RAMP_SECONDS = 0.03
 
 
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--ramp-ms", type=float, default=RAMP_SECONDS * 1e3,
+                    help="keep the GPU busy this long before each measurement's warmup steps")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary measurements")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--only", default="", help="run only the named kernel in a loop (for profilers): "
@@ -53,9 +63,17 @@ def parse_args():
     return ap.parse_args()
 
 
-def gpu_time(torch, fn, steps, warmup):
+def gpu_time(torch, fn, steps, warmup, ramp_seconds=None):
     """(seconds per step by wall clock, seconds per launch by HIP events on the
-    launch stream) for `steps` back-to-back calls after `warmup` untimed ones."""
+    launch stream) for `steps` back-to-back calls after a ramp phase (see
+    RAMP_SECONDS) and `warmup` untimed calls."""
+    if ramp_seconds is None:
+        ramp_seconds = RAMP_SECONDS
+    t_ramp = time.perf_counter()
+    while time.perf_counter() - t_ramp < ramp_seconds:
+        for _ in range(8):
+            fn()
+        torch.cuda.synchronize()
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -125,6 +143,8 @@ def cpu_baseline(F, synth, size):
 
 def main():
     args = parse_args()
+    global RAMP_SECONDS
+    RAMP_SECONDS = args.ramp_ms * 1e-3
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; the path has no multi-GPU part "
               "(--gpus must be 1).", file=sys.stderr)
