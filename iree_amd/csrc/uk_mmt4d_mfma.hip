@@ -24,20 +24,21 @@
 // lanes 0-31 fetch one whole tile and lanes 32-63 the tile two further on, so
 // each half is again in lane order in LDS. (OCP e4m3fn, unit block scales.)
 //
-// Kernel shape: a workgroup of 4 waves owns a macro tile of (2*WM) x (2*WN)
-// outer tiles; each wave accumulates WM x WN blocks of 32x32 in registers. The K
-// loop moves operand blocks global -> LDS with direct-to-LDS 128-bit loads
-// (no register staging) into a ring of K-step slots, several K-steps ahead of
-// the MFMAs; operand fragments are read from LDS one K-step ahead and every
-// memory instruction is issued in the shadow of an MFMA. Workgroup ids are
+// Kernel shape: a workgroup of 2 x kWavesN waves (4 by default) owns a macro
+// tile of (2*WM) x (kWavesN*WN) outer tiles; each wave accumulates WM x WN blocks
+// of 32x32 in registers. The K loop moves operand blocks global -> LDS with
+// direct-to-LDS 128-bit buffer loads (no register staging) into a ring of
+// K-step slots, several K-steps ahead of the MFMAs; operand fragments are read
+// from LDS one K-step ahead and every memory instruction is issued in the
+// shadow of an MFMA. Workgroup ids are
 // remapped so that the 8 XCDs (which receive consecutive workgroup ids
 // round-robin) each work on a compact block of macro tiles and reuse operand
 // panels in their own L2.
 //
 // Measured bound that matters more than the nominal peak: with N(0,1) f16
-// operands a register-only MFMA loop sustains about 1.3 PFLOP/s on MI355X
-// (2.1 with all-zero operands): the matrix pipe is power-limited by operand
-// toggling, so data movement that costs energy also costs MFMA rate.
+// operands a register-only MFMA loop sustains 1.45-1.7 PFLOP/s on MI355X
+// (2.2-2.4 with all-zero operands): the matrix pipe is power-limited by operand
+// toggling and the clock drops, so every stall cycle costs more time as well.
 #include "uk_common.h"
 #include "uk_fp8.h"
 #include "uk_mfma_cfg.h"
