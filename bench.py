@@ -348,6 +348,15 @@ def extras(args, torch, iree_amd, F, synth, lhs, rhs, out):
                                                               F.MMT4D_TYPE_F16F16F32, workspace=ws),
                     max(5, steps // 4), 2)
     ex["matmul_f16_pack_mmt4d_unpack_tflops"] = round(flops / t / 1e12, 2)
+    # the same with the unpack fused into the matmul's epilogue (3 launches)
+    c_two = c.clone()
+    _, t = gpu_time(torch, lambda: iree_amd.matmul_data_tiled(a, b, c, size, size, size,
+                                                              F.MMT4D_TYPE_F16F16F32, workspace=ws,
+                                                              fuse_unpack=True),
+                    max(5, steps // 4), 2)
+    ex["matmul_f16_pack_mmt4d_fused_unpack_tflops"] = round(flops / t / 1e12, 2)
+    assert torch.equal(c, c_two), "fused unpack differs from mmt4d + unpack"
+    del c_two
     del a, b, c, ws
 
     # the small i8 configuration, 1024^3 on row-major operands (2 packs, mmt4d,

@@ -405,6 +405,28 @@ IREE_AMD_UK_EXPORT int iree_amd_uk_mmt4d_silu_mul_f8e4m3(
     iree_amd_uk_index_t N, iree_amd_uk_index_t K, int32_t K0, uint32_t flags,
     float gate_scale, float up_scale, float inv_out_scale, void* stream);
 
+/* mmt4d fused with the unpack that would follow it (no counterpart ukernel in
+ * the reference; its dispatches are linalg.mmt4d followed by tensor.unpack,
+ * REF compiler/src/iree/compiler/Codegen/Common/CPU/CPULowerToUKernels.cpp:339-480):
+ * operands and meaning as iree_amd_uk_mmt4d with tiles M0 = N0 = 32, but the
+ * result is written (and, with the ACCUMULATE flag, first read) as the row-major
+ * out_size0 x out_size1 matrix that iree_amd_uk_unpack without transpose flags
+ * would produce from the tiled result: out_stride0 is the element pitch between
+ * matrix rows, out_offset in elements, (M-1)*32 < out_size0 <= M*32 and
+ * (N-1)*32 < out_size1 <= N*32. Bit-identical to the two-call sequence; saves
+ * writing and re-reading the tiled accumulator. Only tile shapes and types with
+ * a matrix-core kernel (see iree_amd_uk_mmt4d_info) and 16-byte aligned
+ * operands: IREE_AMD_UK_STATUS_UNIMPLEMENTED otherwise. */
+IREE_AMD_UK_EXPORT int iree_amd_uk_mmt4d_unpack(
+    const void* lhs_buffer, iree_amd_uk_index_t lhs_offset,
+    iree_amd_uk_index_t lhs_stride0, const void* rhs_buffer,
+    iree_amd_uk_index_t rhs_offset, iree_amd_uk_index_t rhs_stride0,
+    void* out_buffer, iree_amd_uk_index_t out_offset,
+    iree_amd_uk_index_t out_stride0, iree_amd_uk_index_t out_size0,
+    iree_amd_uk_index_t out_size1, iree_amd_uk_index_t M,
+    iree_amd_uk_index_t N, iree_amd_uk_index_t K, int32_t K0, uint32_t flags,
+    void* stream);
+
 /* buf[i] *= scale over n f32 elements, in place (applies the product of the
  * per-tensor scales to an fp8 matmul result). */
 IREE_AMD_UK_EXPORT int iree_amd_uk_scale_f32(void* buf_f32, iree_amd_uk_index_t n,

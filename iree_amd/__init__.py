@@ -17,6 +17,7 @@ from .ukernel import (  # noqa: F401
     mmt4d,
     mmt4d_info,
     mmt4d_silu_mul_f8e4m3,
+    mmt4d_unpack,
     pack,
     pack_i4_weights,
     quantize_f16_to_f8e4m3,

@@ -111,6 +111,9 @@ def _declare(lib):
     lib.iree_amd_uk_mmt4d_silu_mul_f8e4m3.argtypes = [vp, i64, i64, vp, i64, i64, vp, i64, i64,
                                                        i64, i64, i64, i32, u32,
                                                        C.c_float, C.c_float, C.c_float, vp]
+    lib.iree_amd_uk_mmt4d_unpack.restype = C.c_int
+    lib.iree_amd_uk_mmt4d_unpack.argtypes = [vp, i64, i64, vp, i64, i64, vp, i64, i64, i64, i64,
+                                             i64, i64, i64, C.c_int32, C.c_uint32, vp]
     lib.iree_amd_uk_scale_f32.restype = C.c_int
     lib.iree_amd_uk_scale_f32.argtypes = [vp, i64, C.c_float, vp]
     lib.iree_amd_uk_mfma_probe.restype = C.c_int

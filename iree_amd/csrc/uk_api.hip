@@ -473,6 +473,40 @@ extern "C" int iree_amd_uk_mmt4d_silu_mul_f8e4m3(
   return st;
 }
 
+extern "C" int iree_amd_uk_mmt4d_unpack(
+    const void* lhs_buffer, iree_amd_uk_index_t lhs_offset,
+    iree_amd_uk_index_t lhs_stride0, const void* rhs_buffer,
+    iree_amd_uk_index_t rhs_offset, iree_amd_uk_index_t rhs_stride0,
+    void* out_buffer, iree_amd_uk_index_t out_offset,
+    iree_amd_uk_index_t out_stride0, iree_amd_uk_index_t out_size0,
+    iree_amd_uk_index_t out_size1, iree_amd_uk_index_t M,
+    iree_amd_uk_index_t N, iree_amd_uk_index_t K, int32_t K0, uint32_t flags,
+    void* stream) {
+  iree_amd_uk_mmt4d_params_t p = {lhs_buffer, lhs_offset, lhs_stride0,
+                                  rhs_buffer, rhs_offset, rhs_stride0,
+                                  out_buffer, out_offset, out_stride0,
+                                  M, N, K, 32, 32, K0, flags, nullptr};
+  UK_RETURN_IF_ERROR(validate_mmt4d(p));
+  // the size conditions of unpack (unpack.c:31-80 of the reference) for 32x32 tiles
+  if (out_size0 < 0 || out_size1 < 0 || out_size0 > M * 32 || out_size1 > N * 32 ||
+      (M > 0 && out_size0 <= (M - 1) * 32) || (N > 0 && out_size1 <= (N - 1) * 32))
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT,
+                "mmt4d_unpack: matrix size does not match the outer tile counts");
+  if (out_stride0 < out_size1)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "mmt4d_unpack: out_stride0 smaller than a row");
+  if (M == 0 || N == 0) return 0;
+  if (!lhs_buffer || !rhs_buffer || !out_buffer)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "mmt4d_unpack: null buffer");
+  int st = IREE_AMD_UK_STATUS_NOT_FOUND;
+  if (mmt4d_mfma_supported(flags, 32, 32, K0))
+    st = launch_mmt4d_unpack_mfma(p, out_size0, out_size1, (hipStream_t)stream);
+  if (st == IREE_AMD_UK_STATUS_NOT_FOUND)
+    return fail(IREE_AMD_UK_STATUS_UNIMPLEMENTED,
+                "mmt4d_unpack: needs a type and K0 with a matrix-core kernel, K > 0 and "
+                "16-byte aligned operands");
+  return st;
+}
+
 extern "C" int iree_amd_uk_scale_f32(void* buf_f32, iree_amd_uk_index_t n, float scale,
                                      void* stream) {
   if (n < 0) return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "scale_f32: negative n");

@@ -60,6 +60,9 @@ struct MfmaArgs {
   int tail_tiles;    // K tiles left over after them (less than one MFMA's worth)
   int tiles_m, tiles_n;  // macro-tile grid
   int accumulate;
+  // row-major result (mmt4d fused with the unpack that would follow it): the
+  // matrix has out_rows x out_cols elements, out_stride_bytes is its row pitch
+  int row_major_out, out_rows, out_cols;
   int half_k0;       // K0 is half the MFMA's K extent (else the full extent)
   // fused SiLU * up epilogue only: scales of the gate and up accumulators and
   // the inverse scale of the e4m3 result
@@ -209,7 +212,24 @@ __global__ __launch_bounds__(128 * kWavesN, kOcc) void mmt4d_mfma_kernel(MfmaArg
   }
 
   acc_t acc[WM][WN];
-  if (a.accumulate) {
+  if (a.accumulate && a.row_major_out) {
+    // (rows and columns past the matrix edge are read from the last valid
+    // one: their accumulators are never stored)
+#pragma unroll
+    for (int x = 0; x < WM; ++x)
+#pragma unroll
+      for (int y = 0; y < WN; ++y) {
+        int col = (j_base + wn * WN + y) * 32 + (lane & 31);
+        col = col < a.out_cols ? col : a.out_cols - 1;
+        const int row0 = (i_base + wm * WM + x) * 32 + 4 * (lane >> 5);
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          int row = row0 + 8 * (v >> 2) + (v & 3);
+          row = row < a.out_rows ? row : a.out_rows - 1;
+          acc[x][y][v] = *((const out_t*)(a.out + (int64_t)row * a.out_stride_bytes) + col);
+        }
+      }
+  } else if (a.accumulate) {
 #pragma unroll
     for (int x = 0; x < WM; ++x)
 #pragma unroll
@@ -448,6 +468,26 @@ __global__ __launch_bounds__(128 * kWavesN, kOcc) void mmt4d_mfma_kernel(MfmaArg
       }
     return;
   }
+  if (a.row_major_out) {
+    // One store instruction writes 128 contiguous bytes of two matrix rows,
+    // exactly as it does for a tile; only the addresses differ.
+#pragma unroll
+    for (int x = 0; x < WM; ++x)
+#pragma unroll
+      for (int y = 0; y < WN; ++y) {
+        const int col = (j_base + wn * WN + y) * 32 + (lane & 31);
+        const int row0 = (i_base + wm * WM + x) * 32 + 4 * (lane >> 5);
+        if (col < a.out_cols) {
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            const int row = row0 + 8 * (v >> 2) + (v & 3);
+            if (row < a.out_rows)
+              *((out_t*)(a.out + (int64_t)row * a.out_stride_bytes) + col) = acc[x][y][v];
+          }
+        }
+      }
+    return;
+  }
 #pragma unroll
   for (int x = 0; x < WM; ++x)
 #pragma unroll
@@ -589,9 +629,14 @@ int make_args(const iree_amd_uk_mmt4d_params_t& p, int out_elem_bytes, MfmaArgs*
   a.tiles_m = a.tiles_n = 0;
   a.accumulate = (p.flags & IREE_AMD_UK_FLAG_MMT4D_ACCUMULATE) != 0;
   a.half_k0 = p.K0 * 2 == sv.mfma_k;
+  a.row_major_out = 0; a.out_rows = a.out_cols = 0;
   a.gate_scale = a.up_scale = a.inv_out_scale = 1.0f;
   return 0;
 }
+}  // namespace
+
+namespace {
+int launch_typed(const iree_amd_uk_mmt4d_params_t& p, const MfmaArgs& a, hipStream_t s);
 }  // namespace
 
 int launch_mmt4d_mfma(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) {
@@ -600,6 +645,28 @@ int launch_mmt4d_mfma(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) {
   MfmaArgs a;
   const int st = make_args(p, ti.out_bytes, &a);
   if (st) return st;
+  return launch_typed(p, a, s);
+}
+
+// mmt4d whose result goes to a row-major out_rows x out_cols matrix (element
+// pitch p.out_stride0 between rows) instead of tiles: what mmt4d followed by
+// an unpack without transposes writes, and reads when accumulating.
+int launch_mmt4d_unpack_mfma(const iree_amd_uk_mmt4d_params_t& p, int64_t out_rows,
+                             int64_t out_cols, hipStream_t s) {
+  Mmt4dTypeInfo ti;
+  mmt4d_type_info(p.flags, &ti);
+  MfmaArgs a;
+  const int st = make_args(p, ti.out_bytes, &a);
+  if (st) return st;
+  if (out_rows > 0x7FFFFFFF || out_cols > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  a.row_major_out = 1;
+  a.out_rows = (int)out_rows;
+  a.out_cols = (int)out_cols;
+  return launch_typed(p, a, s);
+}
+
+namespace {
+int launch_typed(const iree_amd_uk_mmt4d_params_t& p, const MfmaArgs& a, hipStream_t s) {
   switch (p.flags & IREE_AMD_UK_FLAG_MMT4D_TYPE_MASK) {
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F32: return launch_cfg<F16Cfg>(a, s);
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16F32: return launch_cfg<BF16Cfg>(a, s);
@@ -611,6 +678,7 @@ int launch_mmt4d_mfma(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) {
     default: return IREE_AMD_UK_STATUS_NOT_FOUND;
   }
 }
+}  // namespace
 
 // mmt4d whose epilogue is e4m3(silu(gate) * up): `p.N` counts gate AND up outer
 // columns (interleaved, so it is even); the output has N / 2 outer columns of

@@ -171,6 +171,23 @@ def mmt4d_silu_mul_f8e4m3(lhs_buffer, rhs_buffer, out_buffer, M, N, K, K0, flags
         gate_scale, up_scale, inv_out_scale, _stream(stream)))
 
 
+def mmt4d_unpack(lhs_buffer, rhs_buffer, out_buffer, out_size0, out_size1, M, N, K, K0, flags, *,
+                 lhs_offset=0, lhs_stride0=None, rhs_offset=0, rhs_stride0=None, out_offset=0,
+                 out_stride0=None, stream=None):
+    """mmt4d (tiles 32x32xK0) whose result is written / accumulated as the
+    row-major ``out_size0`` x ``out_size1`` matrix an unpack would produce."""
+    if lhs_stride0 is None:
+        lhs_stride0 = K * 32 * K0
+    if rhs_stride0 is None:
+        rhs_stride0 = K * 32 * K0
+    if out_stride0 is None:
+        out_stride0 = out_size1
+    _check(load_library().iree_amd_uk_mmt4d_unpack(
+        _ptr(lhs_buffer), lhs_offset, lhs_stride0, _ptr(rhs_buffer), rhs_offset, rhs_stride0,
+        _ptr(out_buffer), out_offset, out_stride0, out_size0, out_size1, M, N, K, K0, flags,
+        _stream(stream)))
+
+
 def scale_f32(buf, n, scale, stream=None):
     _check(load_library().iree_amd_uk_scale_f32(_ptr(buf), n, scale, _stream(stream)))
 
@@ -226,8 +243,10 @@ def _ceil_div(a, b):
 
 
 def matmul_data_tiled(a, b, c, M, N, K, mmt4d_type, *, accumulate=False,
-                      tile=None, workspace=None):
+                      tile=None, workspace=None, fuse_unpack=False):
     """Row-major C[M][N] (+)= A[M][K] * B[K][N] through pack -> mmt4d -> unpack.
+    With ``fuse_unpack`` the last two (and the pack of C when accumulating) are
+    the one kernel ``mmt4d_unpack``; it needs a tile with a matrix-core kernel.
 
     ``a``/``b``/``c`` are flat CUDA tensors holding the row-major matrices with
     the element types of ``mmt4d_type``. ``tile`` = (M0, N0, K0); by default the
@@ -249,13 +268,20 @@ def matmul_data_tiled(a, b, c, M, N, K, mmt4d_type, *, accumulate=False,
         ws["lhs"] = torch.empty(M1 * K1 * M0 * K0, dtype=a.dtype, device=a.device)
     if "rhs" not in ws:
         ws["rhs"] = torch.empty(N1 * K1 * N0 * K0, dtype=b.dtype, device=b.device)
-    if "out" not in ws:
+    if "out" not in ws and not fuse_unpack:
         ws["out"] = torch.empty(M1 * N1 * M0 * N0, dtype=c.dtype, device=c.device)
     pack(a, ws["lhs"], M, K, M1, K1, M0, K0, 0, in_type)
     pack(b, ws["rhs"], K, N, N1, K1, N0, K0, 0,
          in_type | F.PACK_TRANSPOSE_INNER | F.PACK_TRANSPOSE_OUTER)
     mm_flags = mmt4d_type | F.MMT4D_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION | \
         F.MMT4D_SKIP_INTERMEDIATE_ROUNDINGS
+    if fuse_unpack:
+        if (M0, N0) != (32, 32):
+            raise ValueError("fuse_unpack needs 32x32 tiles")
+        if accumulate:
+            mm_flags |= F.MMT4D_ACCUMULATE
+        mmt4d_unpack(ws["lhs"], ws["rhs"], c, M, N, M1, N1, K1, K0, mm_flags)
+        return ws
     if accumulate:
         pack(c, ws["out"], M, N, M1, N1, M0, N0, 0, out_type)
         mm_flags |= F.MMT4D_ACCUMULATE

@@ -321,3 +321,76 @@ def test_mfma_probe_runs_and_counts_operations(uk, cuda):
         uk.mfma_probe(F.MMT4D_TYPE_S16S16S32, ops, 7, sink)
     with pytest.raises(uk.UkError):
         uk.mfma_probe(F.MMT4D_TYPE_F16F16F32, ops, -1, sink)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,N,K", [(1024, 1024, 1024), (123, 456, 789), (81, 19, 41), (1, 1000, 1000),
+                                   (300, 257, 48)])
+@pytest.mark.parametrize("accumulate", [False, True])
+def test_i8_matmul_with_fused_unpack_is_bit_exact(uk, cuda, M, N, K, accumulate):
+    """mmt4d_unpack (mmt4d writing / accumulating the row-major matrix itself)
+    against the plain integer matmul of the oracle and against the two-call
+    sequence, on the 1024^3 configuration and ragged shapes; the row pitch of C
+    is wider than a row and the bytes between rows must stay untouched."""
+    import torch
+    A = synth.uniform_int8(1, M * K)
+    B = synth.uniform_int8(2, K * N)
+    ldc = N + 5
+    c0 = (synth.uniform_int8(3, M * ldc).astype(np.int32) * 1000)
+    c = torch.from_numpy(c0.copy()).cuda()
+    a_d, b_d = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda()
+    M1, N1, K1 = -(-M // 32), -(-N // 32), -(-K // 16)
+    lhs = torch.empty(M1 * K1 * 512, dtype=torch.int8, device=cuda)
+    rhs = torch.empty(N1 * K1 * 512, dtype=torch.int8, device=cuda)
+    uk.pack(a_d, lhs, M, K, M1, K1, 32, 16, 0, F.PACK_TYPE_I8I8)
+    uk.pack(b_d, rhs, K, N, N1, K1, 32, 16, 0,
+            F.PACK_TYPE_I8I8 | F.PACK_TRANSPOSE_INNER | F.PACK_TRANSPOSE_OUTER)
+    flags = F.MMT4D_TYPE_S8S8S32 | (F.MMT4D_ACCUMULATE if accumulate else 0)
+    uk.mmt4d_unpack(lhs, rhs, c, M, N, M1, N1, K1, 16, flags, out_stride0=ldc)
+    torch.cuda.synchronize()
+    got = c.cpu().numpy().reshape(M, ldc)
+    want = _pack_chain_oracle_i8(A, B, M, N, K)
+    before = c0.reshape(M, ldc)
+    if accumulate:
+        want = want + before[:, :N]
+    assert np.array_equal(got[:, :N], want)
+    assert np.array_equal(got[:, N:], before[:, N:])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("type_flag,K0,dt", [(F.MMT4D_TYPE_F16F16F32, 8, np.float16), (F.MMT4D_TYPE_F32F32F32, 4, np.float32)])
+def test_fused_unpack_equals_mmt4d_then_unpack_bitwise(uk, cuda, type_flag, K0, dt):
+    """Same kernel arithmetic, different store addresses: the fused form must
+    reproduce mmt4d + unpack bit for bit on float data too (ragged M and N, a K
+    with a partial last matrix-core step)."""
+    import torch
+    M, N, K = 200, 333, 8 * 37 + (4 if dt is np.float32 else 0)
+    M1, N1, K1 = -(-M // 32), -(-N // 32), -(-K // K0)
+    rng = np.random.default_rng(11)
+    lhs = torch.from_numpy(rng.standard_normal(M1 * K1 * 32 * K0).astype(dt)).cuda()
+    rhs = torch.from_numpy(rng.standard_normal(N1 * K1 * 32 * K0).astype(dt)).cuda()
+    tiled = torch.zeros(M1 * N1 * 1024, dtype=torch.float32, device=cuda)
+    two = torch.full((M * N,), -3.0, dtype=torch.float32, device=cuda)
+    one = torch.full((M * N,), -3.0, dtype=torch.float32, device=cuda)
+    uk.mmt4d(lhs, rhs, tiled, M1, N1, K1, 32, 32, K0, type_flag)
+    uk.unpack(tiled, two, M1, N1, 32, 32, M, N, F.UNPACK_TYPE_F32F32)
+    uk.mmt4d_unpack(lhs, rhs, one, M, N, M1, N1, K1, K0, type_flag)
+    torch.cuda.synchronize()
+    assert np.array_equal(one.cpu().numpy().view(np.uint32), two.cpu().numpy().view(np.uint32))
+
+
+@pytest.mark.gpu
+def test_fused_unpack_rejects_what_it_cannot_serve(uk, cuda):
+    import torch
+    lhs = torch.zeros(4 * 512, dtype=torch.int8, device=cuda)
+    out = torch.zeros(64 * 64, dtype=torch.int32, device=cuda)
+    ok = dict(out_size0=33, out_size1=64, M=2, N=2, K=2, K0=16, flags=F.MMT4D_TYPE_S8S8S32)
+    uk.mmt4d_unpack(lhs, lhs, out, **ok)
+    for bad in (dict(out_size0=32), dict(out_size0=65), dict(out_size1=0), dict(flags=0x0C),
+                dict(out_stride0=63)):
+        with pytest.raises(uk.UkError):
+            uk.mmt4d_unpack(lhs, lhs, out, **{**ok, **bad})
+    # a type without a matrix-core kernel: unimplemented, not a wrong result
+    with pytest.raises(uk.UkError) as e:
+        uk.mmt4d_unpack(lhs, lhs, out, **{**ok, "flags": F.MMT4D_TYPE_S16S16S32, "K0": 8})
+    assert e.value.status == 12
