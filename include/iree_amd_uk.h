@@ -413,8 +413,10 @@ IREE_AMD_UK_EXPORT int iree_amd_uk_mmt4d_silu_mul_f8e4m3(
  * out_size0 x out_size1 matrix that iree_amd_uk_unpack without transpose flags
  * would produce from the tiled result: out_stride0 is the element pitch between
  * matrix rows, out_offset in elements, (M-1)*32 < out_size0 <= M*32 and
- * (N-1)*32 < out_size1 <= N*32. Bit-identical to the two-call sequence; saves
- * writing and re-reading the tiled accumulator. Only tile shapes and types with
+ * (N-1)*32 < out_size1 <= N*32. Float results are multiplied by out_scale on
+ * the store (the product of the per-tensor scales of an fp8 matmul; must be 1
+ * for integer types and with ACCUMULATE). With out_scale = 1 bit-identical to
+ * the two-call sequence; saves writing and re-reading the tiled accumulator. Only tile shapes and types with
  * a matrix-core kernel (see iree_amd_uk_mmt4d_info) and 16-byte aligned
  * operands: IREE_AMD_UK_STATUS_UNIMPLEMENTED otherwise. */
 IREE_AMD_UK_EXPORT int iree_amd_uk_mmt4d_unpack(
@@ -425,7 +427,7 @@ IREE_AMD_UK_EXPORT int iree_amd_uk_mmt4d_unpack(
     iree_amd_uk_index_t out_stride0, iree_amd_uk_index_t out_size0,
     iree_amd_uk_index_t out_size1, iree_amd_uk_index_t M,
     iree_amd_uk_index_t N, iree_amd_uk_index_t K, int32_t K0, uint32_t flags,
-    void* stream);
+    float out_scale, void* stream);
 
 /* buf[i] *= scale over n f32 elements, in place (applies the product of the
  * per-tensor scales to an fp8 matmul result). */

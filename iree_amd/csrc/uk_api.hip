@@ -481,12 +481,23 @@ extern "C" int iree_amd_uk_mmt4d_unpack(
     iree_amd_uk_index_t out_stride0, iree_amd_uk_index_t out_size0,
     iree_amd_uk_index_t out_size1, iree_amd_uk_index_t M,
     iree_amd_uk_index_t N, iree_amd_uk_index_t K, int32_t K0, uint32_t flags,
-    void* stream) {
+    float out_scale, void* stream) {
   iree_amd_uk_mmt4d_params_t p = {lhs_buffer, lhs_offset, lhs_stride0,
                                   rhs_buffer, rhs_offset, rhs_stride0,
                                   out_buffer, out_offset, out_stride0,
                                   M, N, K, 32, 32, K0, flags, nullptr};
   UK_RETURN_IF_ERROR(validate_mmt4d(p));
+  if (out_scale != 1.0f) {
+    const uint32_t type = flags & IREE_AMD_UK_FLAG_MMT4D_TYPE_MASK;
+    const bool integer = type == IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32 ||
+                         type == IREE_AMD_UK_FLAG_MMT4D_TYPE_S16S16S32 ||
+                         type == IREE_AMD_UK_FLAG_MMT4D_TYPE_S16U4S32 ||
+                         type == IREE_AMD_UK_FLAG_MMT4D_TYPE_S16S8S32 ||
+                         type == IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S4S32;
+    if (integer || (flags & IREE_AMD_UK_FLAG_MMT4D_ACCUMULATE))
+      return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT,
+                  "mmt4d_unpack: out_scale other than 1 needs a float type and no accumulate flag");
+  }
   // the size conditions of unpack (unpack.c:31-80 of the reference) for 32x32 tiles
   if (out_size0 < 0 || out_size1 < 0 || out_size0 > M * 32 || out_size1 > N * 32 ||
       (M > 0 && out_size0 <= (M - 1) * 32) || (N > 0 && out_size1 <= (N - 1) * 32))
@@ -499,7 +510,7 @@ extern "C" int iree_amd_uk_mmt4d_unpack(
     return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "mmt4d_unpack: null buffer");
   int st = IREE_AMD_UK_STATUS_NOT_FOUND;
   if (mmt4d_mfma_supported(flags, 32, 32, K0))
-    st = launch_mmt4d_unpack_mfma(p, out_size0, out_size1, (hipStream_t)stream);
+    st = launch_mmt4d_unpack_mfma(p, out_size0, out_size1, out_scale, (hipStream_t)stream);
   if (st == IREE_AMD_UK_STATUS_NOT_FOUND)
     return fail(IREE_AMD_UK_STATUS_UNIMPLEMENTED,
                 "mmt4d_unpack: needs a type and K0 with a matrix-core kernel, K > 0 and "

@@ -67,6 +67,8 @@ struct MfmaArgs {
   // fused SiLU * up epilogue only: scales of the gate and up accumulators and
   // the inverse scale of the e4m3 result
   float gate_scale, up_scale, inv_out_scale;
+  // row-major result of a float type only: factor applied on the store
+  float out_scale;
 };
 
 __device__ __forceinline__ void load_block_to_lds(__amdgpu_buffer_rsrc_t row, uint32_t lane_off,
@@ -481,8 +483,13 @@ __global__ __launch_bounds__(128 * kWavesN, kOcc) void mmt4d_mfma_kernel(MfmaArg
 #pragma unroll
           for (int v = 0; v < 16; ++v) {
             const int row = row0 + 8 * (v >> 2) + (v & 3);
-            if (row < a.out_rows)
-              *((out_t*)(a.out + (int64_t)row * a.out_stride_bytes) + col) = acc[x][y][v];
+            if (row < a.out_rows) {
+              out_t* dst = (out_t*)(a.out + (int64_t)row * a.out_stride_bytes) + col;
+              if constexpr (std::is_floating_point<decltype(acc[x][y][v] + 0)>::value)
+                *dst = (out_t)(acc[x][y][v] * a.out_scale);   // (x 1.0f is exact)
+              else
+                *dst = acc[x][y][v];
+            }
           }
         }
       }
@@ -630,7 +637,7 @@ int make_args(const iree_amd_uk_mmt4d_params_t& p, int out_elem_bytes, MfmaArgs*
   a.accumulate = (p.flags & IREE_AMD_UK_FLAG_MMT4D_ACCUMULATE) != 0;
   a.half_k0 = p.K0 * 2 == sv.mfma_k;
   a.row_major_out = 0; a.out_rows = a.out_cols = 0;
-  a.gate_scale = a.up_scale = a.inv_out_scale = 1.0f;
+  a.gate_scale = a.up_scale = a.inv_out_scale = a.out_scale = 1.0f;
   return 0;
 }
 }  // namespace
@@ -650,9 +657,10 @@ int launch_mmt4d_mfma(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) {
 
 // mmt4d whose result goes to a row-major out_rows x out_cols matrix (element
 // pitch p.out_stride0 between rows) instead of tiles: what mmt4d followed by
-// an unpack without transposes writes, and reads when accumulating.
+// an unpack without transposes writes, and reads when accumulating; float
+// results are multiplied by out_scale on the store.
 int launch_mmt4d_unpack_mfma(const iree_amd_uk_mmt4d_params_t& p, int64_t out_rows,
-                             int64_t out_cols, hipStream_t s) {
+                             int64_t out_cols, float out_scale, hipStream_t s) {
   Mmt4dTypeInfo ti;
   mmt4d_type_info(p.flags, &ti);
   MfmaArgs a;
@@ -660,6 +668,7 @@ int launch_mmt4d_unpack_mfma(const iree_amd_uk_mmt4d_params_t& p, int64_t out_ro
   if (st) return st;
   if (out_rows > 0x7FFFFFFF || out_cols > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
   a.row_major_out = 1;
+  a.out_scale = out_scale;
   a.out_rows = (int)out_rows;
   a.out_cols = (int)out_cols;
   return launch_typed(p, a, s);

@@ -173,9 +173,10 @@ def mmt4d_silu_mul_f8e4m3(lhs_buffer, rhs_buffer, out_buffer, M, N, K, K0, flags
 
 def mmt4d_unpack(lhs_buffer, rhs_buffer, out_buffer, out_size0, out_size1, M, N, K, K0, flags, *,
                  lhs_offset=0, lhs_stride0=None, rhs_offset=0, rhs_stride0=None, out_offset=0,
-                 out_stride0=None, stream=None):
+                 out_stride0=None, out_scale=1.0, stream=None):
     """mmt4d (tiles 32x32xK0) whose result is written / accumulated as the
-    row-major ``out_size0`` x ``out_size1`` matrix an unpack would produce."""
+    row-major ``out_size0`` x ``out_size1`` matrix an unpack would produce,
+    float results times ``out_scale``."""
     if lhs_stride0 is None:
         lhs_stride0 = K * 32 * K0
     if rhs_stride0 is None:
@@ -185,7 +186,7 @@ def mmt4d_unpack(lhs_buffer, rhs_buffer, out_buffer, out_size0, out_size1, M, N,
     _check(load_library().iree_amd_uk_mmt4d_unpack(
         _ptr(lhs_buffer), lhs_offset, lhs_stride0, _ptr(rhs_buffer), rhs_offset, rhs_stride0,
         _ptr(out_buffer), out_offset, out_stride0, out_size0, out_size1, M, N, K, K0, flags,
-        _stream(stream)))
+        out_scale, _stream(stream)))
 
 
 def scale_f32(buf, n, scale, stream=None):
@@ -353,6 +354,10 @@ class Fp8Mlp:
             mmt4d(self.x_tiles, self.wgu, self.acc, M1, 2 * F1, hidden // 16, 32, 32, 16, mm)
             silu_mul_quantize_tiled(self.acc, 2 * F1 * 1024, 0, F1, self.h_tiles, ffn * 32, M1, F1,
                                     self.sx * self.sg, self.sx * self.su, 1.0 / self.sh)
-        mmt4d(self.h_tiles, self.wd, self.acc2, M1, H1, ffn // 16, 32, 32, 16, mm)
-        unpack(self.acc2, y_f32, M1, H1, 32, 32, M, hidden, F.UNPACK_TYPE_F32F32)
-        scale_f32(y_f32, M * hidden, self.sh * self.sd)
+        if self.fused:
+            mmt4d_unpack(self.h_tiles, self.wd, y_f32, M, hidden, M1, H1, ffn // 16, 16, mm,
+                         out_scale=self.sh * self.sd)
+        else:
+            mmt4d(self.h_tiles, self.wd, self.acc2, M1, H1, ffn // 16, 32, 32, 16, mm)
+            unpack(self.acc2, y_f32, M1, H1, 32, 32, M, hidden, F.UNPACK_TYPE_F32F32)
+            scale_f32(y_f32, M * hidden, self.sh * self.sd)

@@ -394,3 +394,33 @@ def test_fused_unpack_rejects_what_it_cannot_serve(uk, cuda):
     with pytest.raises(uk.UkError) as e:
         uk.mmt4d_unpack(lhs, lhs, out, **{**ok, "flags": F.MMT4D_TYPE_S16S16S32, "K0": 8})
     assert e.value.status == 12
+
+
+@pytest.mark.gpu
+def test_fused_unpack_applies_the_output_scale(uk, cuda):
+    """out_scale multiplies a float result once on the store: the same single
+    f32 multiplication as scale_f32 after mmt4d + unpack, so bit-identical.
+    Integer types and accumulation refuse a scale."""
+    import torch
+    M, N, K = 96, 160, 128
+    M1, N1, K1 = M // 32, N // 32, K // 16
+    src = torch.from_numpy(synth.normal_f16(5, (M + N) * K).view(np.int16)).cuda()
+    q = torch.empty((M + N) * K, dtype=torch.uint8, device=cuda)
+    uk.quantize_f16_to_f8e4m3(src, q, (M + N) * K, 1.0)
+    lhs, rhs = q[:M * K], q[M * K:]
+    flags = F.MMT4D_TYPE_F8E4M3F8E4M3F32
+    tiled = torch.zeros(M1 * N1 * 1024, dtype=torch.float32, device=cuda)
+    two = torch.zeros(M * N, dtype=torch.float32, device=cuda)
+    one = torch.zeros(M * N, dtype=torch.float32, device=cuda)
+    uk.mmt4d(lhs, rhs, tiled, M1, N1, K1, 32, 32, 16, flags)
+    uk.unpack(tiled, two, M1, N1, 32, 32, M, N, F.UNPACK_TYPE_F32F32)
+    uk.scale_f32(two, M * N, 0.37)
+    uk.mmt4d_unpack(lhs, rhs, one, M, N, M1, N1, K1, 16, flags, out_scale=0.37)
+    torch.cuda.synchronize()
+    assert float(two.abs().max()) > 0
+    assert np.array_equal(one.cpu().numpy().view(np.uint32), two.cpu().numpy().view(np.uint32))
+    with pytest.raises(uk.UkError):
+        uk.mmt4d_unpack(lhs, rhs, one, M, N, M1, N1, K1, 16, flags | F.MMT4D_ACCUMULATE, out_scale=0.37)
+    oi = torch.zeros(M * N, dtype=torch.int32, device=cuda)
+    with pytest.raises(uk.UkError):
+        uk.mmt4d_unpack(lhs, rhs, oi, M, N, M1, N1, K1, 16, F.MMT4D_TYPE_S8S8S32, out_scale=2.0)
