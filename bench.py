@@ -417,7 +417,20 @@ def extras(args, torch, iree_amd, F, synth, lhs, rhs, out):
         _, t = gpu_time(torch, do_n, steps, warm)
         ex[f"mmt4d_f16_narrow_m{M0}_gbs"] = round((Nn * Kn * 2 + M0 * Kn * 2 + M0 * Nn * 4) / t / 1e9, 1)
     ex["mmt4d_f16_narrow_m1_frac_of_hbm_peak"] = round(ex["mmt4d_f16_narrow_m1_gbs"] / PEAK_HBM_GBS, 4)
-    del rn
+    # the transposed shape (N 4096, K 14336: a K longer than one launch keeps in
+    # registers, run as four accumulating launches over K slices), same buffers
+    ll = torch.from_numpy(synth.normal_f16(61, 8 * Nn).view(np.int16)).cuda()
+    ol = torch.empty(8 * Kn, dtype=torch.float32, device="cuda")
+    state["i"] = 0
+
+    def do_long():
+        k = state["i"] % 6
+        state["i"] += 1
+        iree_amd.mmt4d(ll, rn[k], ol, 1, Kn // 32, Nn // 8, 8, 32, 8, F.MMT4D_TYPE_F16F16F32)
+
+    _, t = gpu_time(torch, do_long, steps, warm)
+    ex["mmt4d_f16_narrow_m8_k14336_gbs"] = round((Nn * Kn * 2 + 8 * Nn * 2 + 8 * Kn * 4) / t / 1e9, 1)
+    del rn, ll, ol
 
     # fp8 e4m3 x e4m3 -> f32 at 4096^3, tile 32x32x16 (codes of N(0,1) values)
     K1 = size // 16

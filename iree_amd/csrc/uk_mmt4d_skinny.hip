@@ -205,17 +205,56 @@ bool mmt4d_skinny_supported(uint32_t flags, int M0, int N0, int K0) {
   return mk && M0 >= 1 && M0 < 32 && N0 == 32 && (K0 == mk || K0 * 2 == mk);
 }
 
+namespace {
+// MFMA steps one launch can take: the left-hand side of a wave's K slice stays
+// in registers (32 steps per wave; 16 for fp8, whose step is twice as large).
+int max_steps_per_launch(int mfma_k) { return kWaves * (mfma_k == 64 ? 16 : 32); }
+
+int launch_chunk(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s);
+}  // namespace
+
 int launch_mmt4d_skinny(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) {
   if (!mmt4d_skinny_supported(p.flags, p.M0, p.N0, p.K0)) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  const int mk = mfma_k_of(p.flags);
+  const int64_t k_elems = p.K * p.K0;
+  if (p.M != 1 || p.K == 0 || k_elems % mk) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  const int64_t steps = k_elems / mk;
+  const int max_steps = max_steps_per_launch(mk);
+  if (steps <= max_steps) return launch_chunk(p, s);
+  // A longer K runs as several launches over equal K slices, each accumulating
+  // into the result of the one before: exact for integers; for f32 results the
+  // same sum in another order. Results narrower than the accumulator (f16,
+  // bf16) would be rounded between the slices, so those are not split.
+  Mmt4dTypeInfo ti;
+  mmt4d_type_info(p.flags, &ti);
+  if (ti.out_bytes != 4) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  const int64_t n_chunks = (steps + max_steps - 1) / max_steps;
+  const int64_t chunk_steps = (steps + n_chunks - 1) / n_chunks;
+  const int64_t tiles_per_step_num = mk, tiles_per_step_den = p.K0;   // K tiles per step = mk / K0 (1 or 2; fp8 4)
+  for (int64_t first = 0; first < steps; first += chunk_steps) {
+    const int64_t n = steps - first < chunk_steps ? steps - first : chunk_steps;
+    iree_amd_uk_mmt4d_params_t q = p;
+    const int64_t tile0 = first * tiles_per_step_num / tiles_per_step_den;
+    q.K = n * tiles_per_step_num / tiles_per_step_den;
+    q.lhs_offset += tile0 * p.M0 * p.K0;
+    q.rhs_offset += tile0 * p.N0 * p.K0;
+    if (first > 0) q.flags |= IREE_AMD_UK_FLAG_MMT4D_ACCUMULATE;
+    const int st = launch_chunk(q, s);
+    // (only the first slice can be refused: alignment and strides are the same for all)
+    if (st) return st;
+  }
+  return 0;
+}
+
+namespace {
+int launch_chunk(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) {
   const int mk = mfma_k_of(p.flags);
   Mmt4dTypeInfo ti;
   mmt4d_type_info(p.flags, &ti);
   const int eb = ti.lhs_bits / 8;
   const int64_t k_elems = p.K * p.K0;
-  // One outer row, whole MFMA steps, a K that fits the register-resident
-  // left-hand side (8 waves x 32 steps), 16-byte aligned operands.
-  if (p.M != 1 || p.K == 0 || k_elems % mk || k_elems / mk > kWaves * 32 || p.N > 0x7FFFFFFF)
-    return IREE_AMD_UK_STATUS_NOT_FOUND;
+  // 16-byte aligned operands
+  if (p.N > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
   const char* lhs = (const char*)p.lhs_buffer + p.lhs_offset * eb;
   const char* rhs = (const char*)p.rhs_buffer + p.rhs_offset * eb;
   if (((uintptr_t)lhs | (uintptr_t)rhs) % 16 || (p.rhs_stride0 * eb) % 16 || (p.M0 * p.K0 * eb) % 16)
@@ -242,5 +281,6 @@ int launch_mmt4d_skinny(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) {
     default: return IREE_AMD_UK_STATUS_NOT_FOUND;
   }
 }
+}  // namespace
 
 }  // namespace uk

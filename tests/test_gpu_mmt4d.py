@@ -110,9 +110,9 @@ def test_narrow_lhs_tiles_bit_exact(uk, cuda, type_flag, K0):
     the tile-size query hands out for a static M below 32) run the streaming
     MFMA kernel: K step counts that fill 8, 16 and 32 register slots per wave,
     ragged splits over the 8 waves, more outer columns than compute units,
-    accumulate. Calls that kernel does not take (two outer rows, an odd K tile
-    count, a K beyond the register-resident range) must give the same bits
-    through the element-wise kernel."""
+    accumulate, long K. Calls that kernel does not take (two outer rows, an odd
+    K tile count, unaligned operands) must give the same bits through the
+    element-wise kernel."""
     rng = np.random.default_rng(7000 + type_flag + K0)
     mfma_k = {F.MMT4D_TYPE_S8S8S32: 32, F.MMT4D_TYPE_F32F32F32: 8,
               F.MMT4D_TYPE_F8E4M3F8E4M3F32: 64}.get(type_flag, 16)
@@ -121,6 +121,14 @@ def test_narrow_lhs_tiles_bit_exact(uk, cuda, type_flag, K0):
         assert uk.mmt4d_info(M0, 32, K0, type_flag | F.MMT4D_SKIP_INTERMEDIATE_ROUNDINGS) == 1
         for N, steps, acc in ((1, 1, False), (5, 8, True), (300, 13, False), (3, 70, True),
                               (7, 128, False), (2, 255, True)):
+            case = ukref.Mmt4dCase(rng, type_flag, 1, N, steps * tps, M0, 32, K0, accumulate=acc)
+            got = gpucase.run_mmt4d(case, flags=case.flags & ~F.MMT4D_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION)
+            assert np.array_equal(got.view(np.uint8), case.run_oracle(ukref.F16_IEEE).view(np.uint8)), \
+                (hex(type_flag), M0, K0, N, steps, acc)
+    # a K beyond what one launch keeps in registers runs as several accumulating
+    # launches over K slices (results as wide as the accumulator only)
+    if type_flag not in (F.MMT4D_TYPE_F16F16F16, F.MMT4D_TYPE_BF16BF16BF16):
+        for M0, N, steps, acc in ((8, 40, 600, False), (1, 9, 896, True), (16, 3, 257, False)):
             case = ukref.Mmt4dCase(rng, type_flag, 1, N, steps * tps, M0, 32, K0, accumulate=acc)
             got = gpucase.run_mmt4d(case, flags=case.flags & ~F.MMT4D_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION)
             assert np.array_equal(got.view(np.uint8), case.run_oracle(ukref.F16_IEEE).view(np.uint8)), \
