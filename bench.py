@@ -113,18 +113,33 @@ def cpu_baseline(F, synth, size):
         cd = ukref.cpu_data(fs)
         out = np.zeros(M1 * N1 * M0 * N0, np.float32)
 
-        def run(rows):
-            lib.iree_uk_mmt4d(ukref.ptr(lhs), 0, K1 * M0 * K0, ukref.ptr(rhs), 0, K1 * N0 * K0,
-                              ukref.ptr(out), 0, N1 * M0 * N0, rows, N1, K1, M0, N0, K0, flags,
-                              C.cast(cd, C.c_void_p))
-        run(8)  # warm-up slice
+        def run(row0, rows):
+            # outer rows [row0, row0 + rows): offsets in elements
+            lib.iree_uk_mmt4d(ukref.ptr(lhs), row0 * K1 * M0 * K0, K1 * M0 * K0, ukref.ptr(rhs), 0,
+                              K1 * N0 * K0, ukref.ptr(out), row0 * N1 * M0 * N0, N1 * M0 * N0, rows, N1,
+                              K1, M0, N0, K0, flags, C.cast(cd, C.c_void_p))
+        run(0, 8)  # warm-up slice
         t0 = time.perf_counter()
-        run(M1)
-        dt = time.perf_counter() - t0
-        return {"value": round(2.0 * size ** 3 / dt / 1e12, 5), "unit": "TFLOP/s", "cores": 1,
+        run(0, M1)
+        dt1 = time.perf_counter() - t0
+        # all cores: outer rows split over threads, the way the reference's
+        # dispatch tiling distributes workgroups (one ukernel call per slice;
+        # the foreign call releases the interpreter lock)
+        import threading
+        threads = min(os.cpu_count() or 1, 16)
+        per = -(-M1 // threads)
+        workers = [threading.Thread(target=run, args=(r0, min(per, M1 - r0))) for r0 in range(0, M1, per)]
+        t0 = time.perf_counter()
+        for w in workers:
+            w.start()
+        for w in workers:
+            w.join()
+        dtn = time.perf_counter() - t0
+        return {"value": round(2.0 * size ** 3 / dtn / 1e12, 5), "unit": "TFLOP/s", "cores": len(workers),
                 "kind": "reference",
                 "sample": f"reference iree_uk_mmt4d f16f16f32, tile 16x16x1 ({fs or 'generic'} path), "
-                          f"full {size}^3 problem, 1 call on 1 thread, {dt:.2f} s"}
+                          f"full {size}^3 problem: {len(workers)} threads over outer rows {dtn:.2f} s; "
+                          f"one call on one thread {dt1:.2f} s = {2.0 * size ** 3 / dt1 / 1e12:.4f} TFLOP/s"}
     # Fallback: the repository's own scalar restatement on a bounded slice.
     from iree_amd._lib import Mmt4dParams
     rows = 4
