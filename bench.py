@@ -461,7 +461,13 @@ def extras(args, torch, iree_amd, F, synth, lhs, rhs, out):
                                                   F.MMT4D_TYPE_F8E4M3F8E4M3F32), steps, warm)
     ex["mmt4d_fp8_tflops"] = round(flops / t / 1e12, 2)
     ex["mmt4d_fp8_frac_of_peak"] = round(flops / t / 1e12 / PEAK_FP8_TFLOPS, 4)
-    del src, l8, r8, o8
+    # the matrix cores' own rate on these operand bits, no data movement
+    sink = torch.zeros(256, dtype=torch.float32, device="cuda")
+    n_ops = iree_amd.mfma_probe(F.MMT4D_TYPE_F8E4M3F8E4M3F32, l8, 256, sink)
+    _, t = gpu_time(torch, lambda: iree_amd.mfma_probe(F.MMT4D_TYPE_F8E4M3F8E4M3F32, l8, 256, sink),
+                    steps, warm)
+    ex["mfma_register_only_fp8_bench_data_tops"] = round(n_ops / t / 1e12, 1)
+    del src, l8, r8, o8, sink
 
     mlp, xm, ym, Mt, Hd, Ff = make_fp8_mlp(torch, iree_amd)
     _, t = gpu_time(torch, lambda: mlp(xm, ym, Mt), max(5, steps // 4), 2)

@@ -521,11 +521,15 @@ int launch_variant(const MfmaArgs& a0, hipStream_t s) {
   constexpr int lds_bytes = kRing * (TM + TN) * Cfg::kSub * kPieceBytes;
   static_assert(lds_bytes <= 160 * 1024, "LDS ring exceeds 160 KiB");
   auto kernel = mmt4d_mfma_kernel<Cfg, WM, WN, kRing, kSync, kOcc, kSiluMul, kWavesN>;
-  static bool attr_set = false;  // benign race: the call is idempotent
-  if (!attr_set) {
+  // The attribute belongs to the kernel on ONE device: set it once per device
+  // ordinal (a benign race: the call is idempotent).
+  static unsigned long long attr_set_on = 0;
+  int dev = 0;
+  UK_RETURN_IF_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= 64 || !((attr_set_on >> dev) & 1)) {
     UK_RETURN_IF_HIP(hipFuncSetAttribute((const void*)kernel,
                                          hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes));
-    attr_set = true;
+    if (dev >= 0 && dev < 64) attr_set_on |= 1ull << dev;
   }
   hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(128 * kWavesN), lds_bytes, s, a);
   return check_hip(hipGetLastError(), "mmt4d_mfma launch");
