@@ -295,6 +295,24 @@ def extras(args, torch, iree_amd, F, synth, lhs, rhs, out):
         ex[f"mfma_register_only_{name}_tops"] = round(n_ops / t / 1e12, 1)
     del sink, zeros, rnd8
 
+    # The same mmt4d through the host-pointer entry point the HAL plugin calls
+    # (pageable host buffers: 64 MiB staged in, 64 MiB staged out, per-call
+    # device allocation, synchronous): the PCIe-inclusive rate, never `value`.
+    import ctypes as C
+    from iree_amd._lib import Mmt4dParams
+    lh, rh = lhs.cpu().numpy(), rhs.cpu().numpy()
+    oh = np.zeros(M1 * N1 * 1024, np.float32)
+    hp = Mmt4dParams(lh.ctypes.data, 0, size * 32, rh.ctypes.data, 0, size * 32, oh.ctypes.data, 0,
+                     N1 * 1024, M1, N1, size // 8, 32, 32, 8, F.MMT4D_TYPE_F16F16F32, None)
+    lib = iree_amd.load_library()
+    assert lib.iree_amd_uk_mmt4d_host(C.byref(hp)) == 0
+    t0 = time.perf_counter()
+    for _ in range(3):
+        assert lib.iree_amd_uk_mmt4d_host(C.byref(hp)) == 0
+    ex["mmt4d_f16_host_pointers_tflops"] = round(flops / ((time.perf_counter() - t0) / 3) / 1e12, 2)
+    assert np.array_equal(oh, out.cpu().numpy()), "host-pointer mmt4d differs from the device entry point"
+    del lh, rh, oh
+
     # f16 with accumulate (reads the 64 MiB accumulator as well)
     acc_flags = F.MMT4D_TYPE_F16F16F32 | F.MMT4D_ACCUMULATE | F.MMT4D_SKIP_INTERMEDIATE_ROUNDINGS
     _, t = gpu_time(torch, lambda: iree_amd.mmt4d(lhs, rhs, out, M1, N1, size // 8, 32, 32, 8, acc_flags),
