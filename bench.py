@@ -430,6 +430,21 @@ def extras(args, torch, iree_amd, F, synth, lhs, rhs, out):
         ex[f"dequant_matmul_i4_m{Mq}_gbs"] = round(qbytes / t / 1e9, 1)
         ex[f"dequant_matmul_i4_m{Mq}_us"] = round(t * 1e6, 2)
     ex["dequant_matmul_i4_m1_frac_of_hbm_peak"] = round(ex["dequant_matmul_i4_m1_gbs"] / PEAK_HBM_GBS, 4)
+    # the transposed shape (N 4096, K 14336, the same byte counts and buffers):
+    # a K the register-resident kernel cannot take; the activations go through
+    # LDS, 1 row in one pass, 8 rows in two passes over the weights
+    for Mq in (1, 8):
+        xq = torch.from_numpy(synth.normal_f16(45 + Mq, Mq * Nq).view(np.int16)).cuda()
+        oq = torch.empty(Mq * Kq, dtype=torch.int16, device="cuda")
+        state["i"] = 0
+
+        def do_ql():
+            k = state["i"] % nrot
+            state["i"] += 1
+            iree_amd.dequant_matmul_i4(xq, wq[k], sq, zq, oq, Mq, Kq, Nq, gs, qflags)
+
+        _, t = gpu_time(torch, do_ql, steps, warm)
+        ex[f"dequant_matmul_i4_m{Mq}_n4096_k14336_us"] = round(t * 1e6, 2)
     del wq, sq, zq
 
     # f16 mmt4d with a narrow left-hand side (decode shape: one outer row of

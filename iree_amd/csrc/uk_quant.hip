@@ -361,13 +361,26 @@ int launch_dequant_matmul_i4(const void* x, const void* w, const void* scale, co
     a.w_bytes = (uint32_t)w_bytes;
     return kb == 4 ? launch_fast<4>(a, s) : launch_fast<8>(a, s);
   }
-  if (gs_pow2 && size_ok && aligned && M <= 16) {
-    // Other K (whole 2048s that fit LDS with these rows): the per-wave-column
-    // kernel. It has a longer start-up (one wave walks all of K for its
-    // columns) but no limit on K beyond LDS capacity.
+  if (gs_pow2 && size_ok && aligned && K > 0) {
+    // Other K (whole 2048s): the per-wave-column kernel. It has a longer
+    // start-up (one wave walks all of K for its columns) but no limit on K as
+    // long as one row of activations fits LDS. Rows go in passes of as many
+    // as fit (at most 16), each pass streaming the weights again: up to 8
+    // passes are still far cheaper than the element-wise kernel.
     a.w_bytes = (uint32_t)w_bytes;
-    const int st = launch_dequant_gemv_i4(a, 0, (int)M, s);
-    if (st != IREE_AMD_UK_STATUS_NOT_FOUND) return st;
+    int64_t rows_per_pass = (144 * 1024) / (K * 2);
+    if (rows_per_pass > 16) rows_per_pass = 16;
+    if (rows_per_pass >= 1 && ceil_div(M, rows_per_pass) <= 8) {
+      // equal passes (8 rows at 5 per pass: 4 + 4 rather than 5 + 3)
+      const int64_t passes = ceil_div(M, rows_per_pass);
+      const int64_t rows = ceil_div(M, passes);
+      int st = 0;
+      for (int64_t m0 = 0; m0 < M; m0 += rows) {
+        st = launch_dequant_gemv_i4(a, (int)m0, (int)(M - m0 < rows ? M - m0 : rows), s);
+        if (st) break;     // NOT_FOUND can only come from the first pass: nothing has run yet
+      }
+      if (st != IREE_AMD_UK_STATUS_NOT_FOUND) return st;
+    }
   }
   const int64_t total = M * N;
   int64_t blocks = ceil_div(total, 256);

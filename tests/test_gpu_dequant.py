@@ -76,10 +76,12 @@ def test_mfma_kernel_group_sizes_and_zero_point_forms(uk, cuda, K, gs, zp_u4):
 @pytest.mark.parametrize("K,gs", [(6144, 128), (8192, 64), (14336, 128), (14336, 256), (2048, 64)])
 @pytest.mark.parametrize("zp_u4", [False, True])
 def test_long_k_small_batches(uk, cuda, K, gs, zp_u4):
-    """K beyond 4096 (in whole 2048s) for the row counts whose activations fit
-    the 160 KiB of LDS, ragged N for row-major weights, and row counts that do
-    not fit (served by the element-wise kernel): all against the f64 oracle."""
-    for M, N, tiled in [(1, 64, True), (1, 50, False), (4, 96, True), (5, 47, False), (16, 32, True)]:
+    """K beyond 4096 (in whole 2048s): rows go through LDS in passes of as many
+    as fit (one pass, several, and more than the 8 passes allowed, which the
+    element-wise kernel serves), ragged N for row-major weights: all against
+    the f64 oracle."""
+    for M, N, tiled in [(1, 64, True), (1, 50, False), (4, 96, True), (5, 47, False), (16, 32, True),
+                        (33, 64, True), (41, 40, False)]:
         if gs < 128 and not tiled:
             continue
         run_case(uk, M, N, K, gs, zp_u4, tiled, seed=K + gs + M)
