@@ -15,6 +15,11 @@
 //     K is a whole number of chunks) with the group scales and zero points of
 //     a chunk fetched one chunk ahead.
 //
+// When N is small (fewer units than waves on the device) the chunks of a unit
+// are dealt to 2, 4 or 8 waves of the workgroup, which add their partial sums
+// through LDS in a fixed order: a unit of K = 14336 then streams through 7
+// waves at once instead of one.
+//
 // Measured against the K-split kernel where both apply (K = 4096, N = 14336,
 // one row): 10.2 us against 10.1 us, and worse for small N, because one wave
 // walks all of K for its columns alone (about 8 us of dependent latency and
@@ -48,6 +53,9 @@ struct GemvArgs {
   int units;              // ceil(N / 16)
   int spans;              // K / 128
   int chunks;             // spans / 16
+  int ksplit;             // waves that share one unit (1, 2, 4 or 8), each a range of chunks
+  int chunks_per_part;    // chunks of one such wave (the last part may have fewer)
+  int x_bytes;            // size of the staged activations in LDS (the partial sums follow)
   uint32_t w_bytes, scale_bytes, zp_bytes;
 };
 
@@ -68,10 +76,21 @@ __global__ __launch_bounds__(kThreads) void dequant_gemv_i4_kernel(GemvArgs a) {
   // ---- flat sequence of (unit, chunk) pairs of this wave --------------------
   // Units go to workgroups first, then to waves, so that a small N still
   // spreads over all compute units.
-  const int unit0 = blockIdx.x + wave * gridDim.x;
-  const int unit_step = gridDim.x * kWaves;
+  // With ksplit > 1, wave w is part w % ksplit of unit lane w / ksplit.
+  const int kp = wave % a.ksplit, ulane = wave / a.ksplit;
+  const int unit_lanes = kWaves / a.ksplit;
+  const int unit0 = blockIdx.x + ulane * gridDim.x;
+  const int unit_step = gridDim.x * unit_lanes;
   const int n_units = unit0 < a.units ? (a.units - unit0 + unit_step - 1) / unit_step : 0;
-  const int n_pairs = n_units * a.chunks;
+  int c0 = kp * a.chunks_per_part;
+  c0 = c0 < a.chunks ? c0 : a.chunks;
+  int c1 = c0 + a.chunks_per_part;
+  c1 = c1 < a.chunks ? c1 : a.chunks;
+  const int n_pairs = n_units * (c1 - c0);
+  // parts that own chunks, and the unit rounds of the workgroup (unit lane 0
+  // has the most): every wave meets that many barriers when ksplit > 1
+  const int parts_used = (a.chunks + a.chunks_per_part - 1) / a.chunks_per_part;
+  const int rounds = ((int)blockIdx.x < a.units) ? (a.units - (int)blockIdx.x + unit_step - 1) / unit_step : 0;
 
   const uint32_t span_stride = a.tiled ? 2048u : 64u;
   const uint32_t col_stride = a.tiled ? 64u : (uint32_t)(a.K >> 1);
@@ -132,9 +151,9 @@ __global__ __launch_bounds__(kThreads) void dequant_gemv_i4_kernel(GemvArgs a) {
   Meta meta_next;
   {
     const __amdgpu_buffer_rsrc_t r0 = unit_rsrc(n_pairs > 0 ? unit0 : a.units);
-    if (n_pairs > 0) load_meta(unit0, 0, meta_next);
+    if (n_pairs > 0) load_meta(unit0, c0, meta_next);
 #pragma unroll
-    for (int d = 0; d < kRingDepth; ++d) ring[d] = load_slab(r0, d);
+    for (int d = 0; d < kRingDepth; ++d) ring[d] = load_slab(r0, c0 * kChunkSpans + d);
   }
   __builtin_amdgcn_sched_barrier(0);
   // x -> LDS in MFMA A-operand order: the 16 bytes that lane (row m, kc) feeds
@@ -165,11 +184,12 @@ __global__ __launch_bounds__(kThreads) void dequant_gemv_i4_kernel(GemvArgs a) {
   float run_scale = 0.f;                       // kRuntimeGroups: scale of the open group
   union { uint32_t u; half2v h; } run_lo, run_hi, run_zf;
   run_lo.u = 0x64006400u; run_hi.u = 0x54005400u; run_zf.u = 0;
-  int unit = unit0, chunk = 0;
+  floatx4* partial = (floatx4*)(x_lds + a.x_bytes);   // [2][kWaves][64], ksplit > 1 only
+  int unit = unit0, chunk = c0, parity = 0;
   for (int pair = 0; pair < n_pairs; ++pair) {
     // the pair after this one (for the refills and the parameter prefetch)
     int next_unit = unit, next_chunk = chunk + 1;
-    if (next_chunk == a.chunks) { next_chunk = 0; next_unit = unit + unit_step; }
+    if (next_chunk == c1) { next_chunk = c0; next_unit = unit + unit_step; }
     const bool have_next = pair + 1 < n_pairs;
     const __amdgpu_buffer_rsrc_t rsrc_next = unit_rsrc(have_next ? next_unit : a.units);
     const Meta mt = meta_next;
@@ -257,19 +277,45 @@ __global__ __launch_bounds__(kThreads) void dequant_gemv_i4_kernel(GemvArgs a) {
       ring[s % kRingDepth] = load_slab(rsrc_next, next_chunk * kChunkSpans + s);
       __builtin_amdgcn_sched_barrier(0);
     }
-    if (chunk + 1 == a.chunks) {
-      // the unit is complete: rows 4*kc + r of column n
-      const int ncol = unit * 16 + nl;
+    if (chunk + 1 == c1) {
+      // this wave's part of the unit is complete
+      if (a.ksplit > 1) {
+        // Sum the parts in part order (deterministic) in the wave of part 0.
+        // The buffer alternates between units: a wave can only be one barrier
+        // ahead of the reader of the previous unit's half.
+        floatx4* buf = partial + parity * (kWaves * 64);
+        buf[wave * 64 + lane] = acc;
+        __syncthreads();
+        if (kp == 0) {
+          acc = buf[wave * 64 + lane];
+          for (int p = 1; p < parts_used; ++p) {
+            const floatx4 v = buf[(wave + p) * 64 + lane];
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int m = 4 * kc + r;
-        if (m < a.m_eff && ncol < a.N)
-          a.out[(size_t)(a.m_base + m) * a.N + ncol] = __half_as_ushort(__float2half_rn(acc[r]));
+            for (int r = 0; r < 4; ++r) acc[r] += v[r];
+          }
+        }
+        parity ^= 1;
+      }
+      if (kp == 0) {
+        // rows 4*kc + r of column n
+        const int ncol = unit * 16 + nl;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int m = 4 * kc + r;
+          if (m < a.m_eff && ncol < a.N)
+            a.out[(size_t)(a.m_base + m) * a.N + ncol] = __half_as_ushort(__float2half_rn(acc[r]));
+        }
       }
       acc = floatx4{0.f, 0.f, 0.f, 0.f};
     }
     unit = next_unit;
     chunk = next_chunk;
+  }
+  if (a.ksplit > 1) {
+    // waves with fewer units than unit lane 0 (or without chunks) still meet
+    // the barriers of the remaining rounds
+    const int met = c1 > c0 ? n_units : 0;
+    for (int r = met; r < rounds; ++r) __syncthreads();
   }
 }
 
@@ -318,7 +364,7 @@ int launch_dequant_gemv_i4(const I4Args& p, int m_base, int m_eff, hipStream_t s
   // that fit LDS.
   if (K % 2048 || m_eff < 1 || m_eff > 16) return IREE_AMD_UK_STATUS_NOT_FOUND;
   if (gs < (p.tiled ? 64 : 128) || gs > 256) return IREE_AMD_UK_STATUS_NOT_FOUND;
-  const size_t lds = (size_t)m_eff * K * 2;
+  size_t lds = (size_t)m_eff * K * 2;
   if (lds > 144 * 1024) return IREE_AMD_UK_STATUS_NOT_FOUND;
   const int64_t g_total = N * p.G;
   if (N * K / 2 + K * 16 >= (1ll << 32) || g_total * 2 >= (1ll << 32)) return IREE_AMD_UK_STATUS_NOT_FOUND;
@@ -333,7 +379,17 @@ int launch_dequant_gemv_i4(const I4Args& p, int m_base, int m_eff, hipStream_t s
   a.w_bytes = (uint32_t)(N * K / 2);
   a.scale_bytes = (uint32_t)(g_total * 2);
   a.zp_bytes = (uint32_t)(p.zp_u4 ? (g_total + 1) / 2 : g_total * 2);
+  // Few units (small N): deal the chunks of a unit to several waves, as many
+  // as still leave every wave of the device at most one part of one unit.
   const int cus = device_cu_count();
+  a.ksplit = 1;
+  while (a.ksplit < kWaves && (int64_t)a.units * a.ksplit * 2 <= (int64_t)cus * kWaves &&
+         a.ksplit < a.chunks)
+    a.ksplit *= 2;
+  a.chunks_per_part = (a.chunks + a.ksplit - 1) / a.ksplit;
+  a.x_bytes = (int)lds;
+  if (a.ksplit > 1) lds += 2 * kWaves * 64 * sizeof(floatx4);   // 16 KiB of partial sums
+  // (units go to workgroups first, then to the unit lanes of a workgroup)
   const int blocks = a.units < cus ? a.units : cus;
   return p.zp_u4 ? launch_zp<true>(a, blocks, lds, s) : launch_zp<false>(a, blocks, lds, s);
 }

@@ -87,6 +87,15 @@ def test_long_k_small_batches(uk, cuda, K, gs, zp_u4):
         run_case(uk, M, N, K, gs, zp_u4, tiled, seed=K + gs + M)
 
 
+@pytest.mark.parametrize("M,N,K,tiled", [(2, 4800, 6144, True), (1, 4112, 8192, False), (3, 1024, 14336, True),
+                                        (1, 8192, 6144, True)])
+def test_long_k_medium_n_splits_k_over_waves(uk, cuda, M, N, K, tiled):
+    """Column counts between one and eight units per compute unit: the chunks of
+    a unit are shared by 2, 4 or 8 waves (one part may be shorter or empty, some
+    unit lanes of a workgroup have no unit) and summed through LDS."""
+    run_case(uk, M, N, K, 128, True, tiled, seed=N + K)
+
+
 def test_fractional_f16_zero_points(uk, cuda):
     run_case(uk, 5, 64, 2048, 128, False, False, seed=3, frac_zp=True)
     run_case(uk, 5, 64, 2048, 128, False, True, seed=4, frac_zp=True)
