@@ -197,7 +197,7 @@ __global__ __launch_bounds__(128 * kWavesN, kOcc) void mmt4d_mfma_kernel(MfmaArg
                        : a.half_k0 ? lane * 16 : ((lane & 31) * 32 + (lane >> 5) * 16);
   constexpr int kPieceStride = 512;
 
-  // Rows this wave copies: TM/4 rows of A and TN/4 rows of B. Out-of-range
+  // Rows this wave copies: its share of the TM rows of A and TN of B. Out-of-range
   // rows are clamped to the last valid one (loaded, never stored).
   __amdgpu_buffer_rsrc_t a_src[kARowsPerWave], b_src[kBRowsPerWave];
 #pragma unroll
