@@ -390,6 +390,13 @@ def extras(args, torch, iree_amd, F, synth, lhs, rhs, out):
                     max(5, steps // 4), 2)
     ex["matmul_f16_pack_mmt4d_fused_unpack_tflops"] = round(flops / t / 1e12, 2)
     assert torch.equal(c, c_two), "fused unpack differs from mmt4d + unpack"
+    # and with the right-hand side packed ahead of time (weights) and the
+    # left-hand side read row-major by the matmul itself: one launch
+    c.fill_(0)
+    _, t = gpu_time(torch, lambda: iree_amd.matmul_packed_rhs(a, ws["rhs"], c, size, size, size, 8,
+                                                              F.MMT4D_TYPE_F16F16F32), steps, warm)
+    ex["matmul_f16_rowmajor_lhs_packed_rhs_tflops"] = round(flops / t / 1e12, 2)
+    assert torch.equal(c, c_two), "one-kernel matmul differs from pack + mmt4d + unpack"
     del c_two
     del a, b, c, ws
 

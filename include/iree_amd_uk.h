@@ -429,6 +429,32 @@ IREE_AMD_UK_EXPORT int iree_amd_uk_mmt4d_unpack(
     iree_amd_uk_index_t N, iree_amd_uk_index_t K, int32_t K0, uint32_t flags,
     float out_scale, void* stream);
 
+/* A whole matmul with a pre-packed right-hand side in one kernel: what the
+ * reference runs as pack(LHS) -> mmt4d -> unpack
+ * (REF compiler/src/iree/compiler/Codegen/Common/CPU/CPULowerToUKernels.cpp:339-480)
+ * when the right-hand side (the weights) was packed ahead of time.
+ *   out[m][n] (+)= sum_k lhs[m][k] * rhs_packed[n / 32][k / K0][n % 32][k % K0]
+ * lhs is the row-major M x K matrix (lhs_stride0 = element pitch between
+ * rows), rhs the packed buffer of ceil(N / 32) outer rows of K / K0 tiles
+ * 32 x K0 (rhs_stride0 = element pitch between outer rows; columns past N must
+ * be padded, with any values), out the row-major M x N result (out_stride0 =
+ * element pitch). Offsets in elements. M, N, K count ELEMENTS here. flags: an
+ * IREE_AMD_UK_FLAG_MMT4D_TYPE_* with a matrix-core kernel, optionally
+ * ACCUMULATE / SKIP_INTERMEDIATE_ROUNDINGS. out_scale as for
+ * iree_amd_uk_mmt4d_unpack. Requirements (IREE_AMD_UK_STATUS_UNIMPLEMENTED
+ * otherwise; use the three-call sequence then): K a multiple of the
+ * matrix-core K extent (16 for f16/bf16, 32 for i8, 8 for f32, 64 for fp8),
+ * K0 as served by iree_amd_uk_mmt4d, 16-byte aligned lhs rows and rhs tiles.
+ * Bit-identical to pack + mmt4d + unpack. */
+IREE_AMD_UK_EXPORT int iree_amd_uk_matmul_packed_rhs(
+    const void* lhs_buffer, iree_amd_uk_index_t lhs_offset,
+    iree_amd_uk_index_t lhs_stride0, const void* rhs_buffer,
+    iree_amd_uk_index_t rhs_offset, iree_amd_uk_index_t rhs_stride0,
+    void* out_buffer, iree_amd_uk_index_t out_offset,
+    iree_amd_uk_index_t out_stride0, iree_amd_uk_index_t M,
+    iree_amd_uk_index_t N, iree_amd_uk_index_t K, int32_t K0, uint32_t flags,
+    float out_scale, void* stream);
+
 /* buf[i] *= scale over n f32 elements, in place (applies the product of the
  * per-tensor scales to an fp8 matmul result). */
 IREE_AMD_UK_EXPORT int iree_amd_uk_scale_f32(void* buf_f32, iree_amd_uk_index_t n,

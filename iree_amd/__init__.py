@@ -13,6 +13,7 @@ from .ukernel import (  # noqa: F401
     UkError,
     dequant_matmul_i4,
     matmul_data_tiled,
+    matmul_packed_rhs,
     mfma_probe,
     mmt4d,
     mmt4d_info,

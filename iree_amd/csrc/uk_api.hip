@@ -518,6 +518,50 @@ extern "C" int iree_amd_uk_mmt4d_unpack(
   return st;
 }
 
+extern "C" int iree_amd_uk_matmul_packed_rhs(
+    const void* lhs_buffer, iree_amd_uk_index_t lhs_offset,
+    iree_amd_uk_index_t lhs_stride0, const void* rhs_buffer,
+    iree_amd_uk_index_t rhs_offset, iree_amd_uk_index_t rhs_stride0,
+    void* out_buffer, iree_amd_uk_index_t out_offset,
+    iree_amd_uk_index_t out_stride0, iree_amd_uk_index_t M,
+    iree_amd_uk_index_t N, iree_amd_uk_index_t K, int32_t K0, uint32_t flags,
+    float out_scale, void* stream) {
+  if (M < 0 || N < 0 || K < 0 || K0 <= 0)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "matmul_packed_rhs: negative size or K0 <= 0");
+  if (K % K0)
+    return fail(IREE_AMD_UK_STATUS_UNIMPLEMENTED, "matmul_packed_rhs: K must be whole K0 tiles");
+  // the equivalent mmt4d: outer counts and K tiles
+  iree_amd_uk_mmt4d_params_t p = {lhs_buffer, lhs_offset, lhs_stride0,
+                                  rhs_buffer, rhs_offset, rhs_stride0,
+                                  out_buffer, out_offset, out_stride0,
+                                  (M + 31) / 32, (N + 31) / 32, K / K0, 32, 32, K0, flags, nullptr};
+  UK_RETURN_IF_ERROR(validate_mmt4d(p));
+  if (out_scale != 1.0f) {
+    const uint32_t type = flags & IREE_AMD_UK_FLAG_MMT4D_TYPE_MASK;
+    const bool integer = type == IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32 ||
+                         type == IREE_AMD_UK_FLAG_MMT4D_TYPE_S16S16S32 ||
+                         type == IREE_AMD_UK_FLAG_MMT4D_TYPE_S16U4S32 ||
+                         type == IREE_AMD_UK_FLAG_MMT4D_TYPE_S16S8S32 ||
+                         type == IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S4S32;
+    if (integer || (flags & IREE_AMD_UK_FLAG_MMT4D_ACCUMULATE))
+      return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT,
+                  "matmul_packed_rhs: out_scale other than 1 needs a float type and no accumulate flag");
+  }
+  if (lhs_stride0 < K || out_stride0 < N)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "matmul_packed_rhs: a row pitch smaller than a row");
+  if (M == 0 || N == 0) return 0;
+  if (!lhs_buffer || !rhs_buffer || !out_buffer)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "matmul_packed_rhs: null buffer");
+  int st = IREE_AMD_UK_STATUS_NOT_FOUND;
+  if (mmt4d_mfma_supported(flags, 32, 32, K0))
+    st = launch_matmul_packed_rhs_mfma(p, M, N, out_scale, (hipStream_t)stream);
+  if (st == IREE_AMD_UK_STATUS_NOT_FOUND)
+    return fail(IREE_AMD_UK_STATUS_UNIMPLEMENTED,
+                "matmul_packed_rhs: needs a type and K0 with a matrix-core kernel, K > 0 in whole "
+                "matrix-core steps and 16-byte aligned rows and tiles");
+  return st;
+}
+
 extern "C" int iree_amd_uk_scale_f32(void* buf_f32, iree_amd_uk_index_t n, float scale,
                                      void* stream) {
   if (n < 0) return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "scale_f32: negative n");

@@ -62,6 +62,8 @@ int launch_mmt4d_skinny(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s);
 int launch_mmt4d_mfma(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s);
 int launch_mmt4d_unpack_mfma(const iree_amd_uk_mmt4d_params_t& p, int64_t out_rows,
                              int64_t out_cols, float out_scale, hipStream_t s);
+int launch_matmul_packed_rhs_mfma(const iree_amd_uk_mmt4d_params_t& p, int64_t out_rows,
+                                  int64_t out_cols, float out_scale, hipStream_t s);
 int launch_mmt4d_silu_mul_mfma(const iree_amd_uk_mmt4d_params_t& p, float gate_scale,
                                float up_scale, float inv_out_scale, hipStream_t s);
 

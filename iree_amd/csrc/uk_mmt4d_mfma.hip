@@ -63,6 +63,11 @@ struct MfmaArgs {
   // row-major result (mmt4d fused with the unpack that would follow it): the
   // matrix has out_rows x out_cols elements, out_stride_bytes is its row pitch
   int row_major_out, out_rows, out_cols;
+  // row-major left-hand side (the pack of the LHS fused into the loads): lhs is
+  // the out_rows x K matrix itself, lhs_stride_bytes its row pitch; the block
+  // of (outer row i, K-step ks) is rows 32 i .. 32 i + 31, bytes
+  // lhs_step_bytes * ks .. of each row
+  int lhs_row_major;
   int half_k0;       // K0 is half the MFMA's K extent (else the full extent)
   // fused SiLU * up epilogue only: scales of the gate and up accumulators and
   // the inverse scale of the e4m3 result
@@ -200,11 +205,27 @@ __global__ __launch_bounds__(128 * kWavesN, kOcc) void mmt4d_mfma_kernel(MfmaArg
   // Rows this wave copies: its share of the TM rows of A and TN of B. Out-of-range
   // rows are clamped to the last valid one (loaded, never stored).
   __amdgpu_buffer_rsrc_t a_src[kARowsPerWave], b_src[kBRowsPerWave];
+  // Left-hand side: per-lane offset inside a row block, bytes between K-steps
+  // and between the two pieces of a wide block. Packed: as the right-hand side.
+  // Row-major: lane l reads row l % 32 (clamped to the last matrix row), the
+  // 16 * kSub bytes of half l / 32 of the K-step: the same bytes in the same
+  // lane order, so LDS and everything behind it are unchanged.
+  uint32_t a_lane_off[kARowsPerWave];
+  const uint32_t a_step_bytes = a.lhs_row_major ? 32 * kSub : kBlockBytes;
+  const uint32_t a_piece_stride = a.lhs_row_major ? 16 : kPieceStride;
 #pragma unroll
   for (int r = 0; r < kARowsPerWave; ++r) {
     int i = i_base + wave * kARowsPerWave + r;
     i = i < a.M ? i : a.M - 1;
-    a_src[r] = row_descriptor(a.lhs + (int64_t)i * a.lhs_stride_bytes);
+    if (a.lhs_row_major) {
+      int row = i * 32 + (lane & 31);
+      row = row < a.out_rows ? row : a.out_rows - 1;
+      a_src[r] = row_descriptor(a.lhs);
+      a_lane_off[r] = (uint32_t)row * (uint32_t)a.lhs_stride_bytes + (lane >> 5) * 16 * kSub;
+    } else {
+      a_src[r] = row_descriptor(a.lhs + (int64_t)i * a.lhs_stride_bytes);
+      a_lane_off[r] = lane_off;
+    }
   }
 #pragma unroll
   for (int r = 0; r < kBRowsPerWave; ++r) {
@@ -259,7 +280,7 @@ __global__ __launch_bounds__(128 * kWavesN, kOcc) void mmt4d_mfma_kernel(MfmaArg
     char* base = lds + slot * kSlotBytes;
     const int r = d / kSub, j = d % kSub;
     if (r < kARowsPerWave) {
-      load_block_to_lds(a_src[r], lane_off, (uint32_t)ks * kBlockBytes + j * kPieceStride,
+      load_block_to_lds(a_src[r], a_lane_off[r], (uint32_t)ks * a_step_bytes + j * a_piece_stride,
                         base + (wave * kARowsPerWave + r) * kBlockBytes + j * kPieceBytes);
     } else {
       const int rb = r - kARowsPerWave;
@@ -649,6 +670,7 @@ int make_args(const iree_amd_uk_mmt4d_params_t& p, int out_elem_bytes, MfmaArgs*
   a.accumulate = (p.flags & IREE_AMD_UK_FLAG_MMT4D_ACCUMULATE) != 0;
   a.half_k0 = p.K0 * 2 == sv.mfma_k;
   a.row_major_out = 0; a.out_rows = a.out_cols = 0;
+  a.lhs_row_major = 0;
   a.gate_scale = a.up_scale = a.inv_out_scale = a.out_scale = 1.0f;
   return 0;
 }
@@ -683,6 +705,30 @@ int launch_mmt4d_unpack_mfma(const iree_amd_uk_mmt4d_params_t& p, int64_t out_ro
   a.out_scale = out_scale;
   a.out_rows = (int)out_rows;
   a.out_cols = (int)out_cols;
+  return launch_typed(p, a, s);
+}
+
+// The same with a row-major left-hand side as well: `p` describes the
+// equivalent mmt4d (outer counts, K tiles, packed right-hand side), except that
+// p.lhs_buffer / lhs_offset / lhs_stride0 are the out_rows x (K * K0) matrix,
+// its first element and its row pitch in elements.
+int launch_matmul_packed_rhs_mfma(const iree_amd_uk_mmt4d_params_t& p, int64_t out_rows,
+                                  int64_t out_cols, float out_scale, hipStream_t s) {
+  Mmt4dTypeInfo ti;
+  mmt4d_type_info(p.flags, &ti);
+  MfmaArgs a;
+  const int st = make_args(p, ti.out_bytes, &a);
+  if (st) return st;
+  // whole matrix-core K-steps only (a partial one would read past the row end),
+  // and a matrix that 32-bit byte offsets can address
+  if (a.tail_tiles != 0 || out_rows > 0x7FFFFFFF || out_cols > 0x7FFFFFFF ||
+      out_rows * a.lhs_stride_bytes + 4096 > 0x7FFFFFFF)
+    return IREE_AMD_UK_STATUS_NOT_FOUND;
+  a.row_major_out = 1;
+  a.lhs_row_major = 1;
+  a.out_rows = (int)out_rows;
+  a.out_cols = (int)out_cols;
+  a.out_scale = out_scale;
   return launch_typed(p, a, s);
 }
 

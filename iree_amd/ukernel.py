@@ -189,6 +189,23 @@ def mmt4d_unpack(lhs_buffer, rhs_buffer, out_buffer, out_size0, out_size1, M, N,
         out_scale, _stream(stream)))
 
 
+def matmul_packed_rhs(lhs, rhs_packed, out, M, N, K, K0, flags, *, lhs_offset=0, lhs_stride0=None,
+                      rhs_offset=0, rhs_stride0=None, out_offset=0, out_stride0=None, out_scale=1.0,
+                      stream=None):
+    """Row-major ``out[M][N] (+)= lhs[M][K] * rhs`` with ``rhs`` already packed
+    into 32 x K0 tiles: pack(LHS), mmt4d and unpack in one kernel. M, N, K are
+    element counts."""
+    if lhs_stride0 is None:
+        lhs_stride0 = K
+    if rhs_stride0 is None:
+        rhs_stride0 = K * 32
+    if out_stride0 is None:
+        out_stride0 = N
+    _check(load_library().iree_amd_uk_matmul_packed_rhs(
+        _ptr(lhs), lhs_offset, lhs_stride0, _ptr(rhs_packed), rhs_offset, rhs_stride0,
+        _ptr(out), out_offset, out_stride0, M, N, K, K0, flags, out_scale, _stream(stream)))
+
+
 def scale_f32(buf, n, scale, stream=None):
     _check(load_library().iree_amd_uk_scale_f32(_ptr(buf), n, scale, _stream(stream)))
 

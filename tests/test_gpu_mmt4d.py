@@ -432,3 +432,86 @@ def test_fused_unpack_applies_the_output_scale(uk, cuda):
     oi = torch.zeros(M * N, dtype=torch.int32, device=cuda)
     with pytest.raises(uk.UkError):
         uk.mmt4d_unpack(lhs, rhs, oi, M, N, M1, N1, K1, 16, F.MMT4D_TYPE_S8S8S32, out_scale=2.0)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,N,K", [(1024, 1024, 1024), (123, 456, 800), (81, 19, 64), (1, 1000, 992),
+                                   (300, 257, 32)])
+@pytest.mark.parametrize("accumulate", [False, True])
+def test_i8_matmul_with_packed_rhs_in_one_kernel_is_bit_exact(uk, cuda, M, N, K, accumulate):
+    """matmul_packed_rhs: row-major LHS read by the matmul itself, pre-packed
+    RHS, row-major result. Against the plain integer matmul of the oracle; row
+    pitches of A and C wider than a row (the bytes between rows of C must stay
+    untouched), ragged M and N, K in whole matrix-core steps of 32."""
+    import torch
+    lda, ldc = K + 16, N + 5
+    A = synth.uniform_int8(1, M * K).reshape(M, K)
+    B = synth.uniform_int8(2, K * N)
+    a_pad = synth.uniform_int8(9, M * lda).reshape(M, lda).copy()
+    a_pad[:, :K] = A
+    c0 = (synth.uniform_int8(3, M * ldc).astype(np.int32) * 1000)
+    c = torch.from_numpy(c0.copy()).cuda()
+    N1, K1 = -(-N // 32), K // 16
+    rhs = torch.empty(N1 * K1 * 512, dtype=torch.int8, device=cuda)
+    uk.pack(torch.from_numpy(B).cuda(), rhs, K, N, N1, K1, 32, 16, 0,
+            F.PACK_TYPE_I8I8 | F.PACK_TRANSPOSE_INNER | F.PACK_TRANSPOSE_OUTER)
+    flags = F.MMT4D_TYPE_S8S8S32 | (F.MMT4D_ACCUMULATE if accumulate else 0)
+    uk.matmul_packed_rhs(torch.from_numpy(a_pad).cuda(), rhs, c, M, N, K, 16, flags,
+                         lhs_stride0=lda, out_stride0=ldc)
+    torch.cuda.synchronize()
+    got = c.cpu().numpy().reshape(M, ldc)
+    want = _pack_chain_oracle_i8(A.reshape(-1), B, M, N, K)
+    before = c0.reshape(M, ldc)
+    if accumulate:
+        want = want + before[:, :N]
+    assert np.array_equal(got[:, :N], want)
+    assert np.array_equal(got[:, N:], before[:, N:])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("type_flag,K0,dt,K", [(F.MMT4D_TYPE_F16F16F32, 8, np.float16, 16 * 19),
+                                               (F.MMT4D_TYPE_F16F16F32, 16, np.float16, 16 * 19),
+                                               (F.MMT4D_TYPE_F32F32F32, 4, np.float32, 8 * 21),
+                                               (F.MMT4D_TYPE_F8E4M3F8E4M3F32, 16, np.uint8, 64 * 5)])
+def test_matmul_packed_rhs_equals_pack_mmt4d_unpack_bitwise(uk, cuda, type_flag, K0, dt, K):
+    """The one-kernel form against the three-call sequence on float data: same
+    bytes reach the same lanes, so the results are bit-identical."""
+    import torch
+    M, N = 200, 333
+    M1, N1, K1 = -(-M // 32), -(-N // 32), K // K0
+    rng = np.random.default_rng(17)
+    if dt is np.uint8:
+        a = rng.integers(0, 0x78, size=M * K).astype(np.uint8)       # finite e4m3 codes
+        rhs_h = rng.integers(0, 0x78, size=N1 * K1 * 32 * K0).astype(np.uint8)
+        pack_type = F.PACK_TYPE_I8I8
+    else:
+        a = rng.standard_normal(M * K).astype(dt)
+        rhs_h = rng.standard_normal(N1 * K1 * 32 * K0).astype(dt)
+        pack_type = F.PACK_TYPE_F16F16 if dt is np.float16 else F.PACK_TYPE_F32F32
+    a_d, rhs = torch.from_numpy(a).cuda(), torch.from_numpy(rhs_h).cuda()
+    lhs = torch.empty(M1 * K1 * 32 * K0, dtype=a_d.dtype, device=cuda)
+    uk.pack(a_d, lhs, M, K, M1, K1, 32, K0, 0, pack_type)
+    tiled = torch.zeros(M1 * N1 * 1024, dtype=torch.float32, device=cuda)
+    three = torch.full((M * N,), -3.0, dtype=torch.float32, device=cuda)
+    one = torch.full((M * N,), -3.0, dtype=torch.float32, device=cuda)
+    uk.mmt4d(lhs, rhs, tiled, M1, N1, K1, 32, 32, K0, type_flag)
+    uk.unpack(tiled, three, M1, N1, 32, 32, M, N, F.UNPACK_TYPE_F32F32)
+    uk.matmul_packed_rhs(a_d, rhs, one, M, N, K, K0, type_flag)
+    torch.cuda.synchronize()
+    assert float(three.abs().max()) > 0
+    assert np.array_equal(one.cpu().numpy().view(np.uint32), three.cpu().numpy().view(np.uint32))
+
+
+@pytest.mark.gpu
+def test_matmul_packed_rhs_rejects_what_it_cannot_serve(uk, cuda):
+    import torch
+    a = torch.zeros(64 * 64, dtype=torch.int8, device=cuda)
+    out = torch.zeros(64 * 64, dtype=torch.int32, device=cuda)
+    ok = dict(M=33, N=64, K=64, K0=16, flags=F.MMT4D_TYPE_S8S8S32)
+    uk.matmul_packed_rhs(a, a, out, **ok)
+    for bad, status in ((dict(K=48), 12), (dict(K=40), 12), (dict(lhs_stride0=63), 3), (dict(out_stride0=63), 3),
+                        (dict(flags=0x0C), 3), (dict(flags=F.MMT4D_TYPE_S16S16S32, K0=8), 12),
+                        (dict(lhs_offset=1), 12), (dict(out_scale=2.0), 3)):
+        with pytest.raises(uk.UkError) as e:
+            uk.matmul_packed_rhs(a, a, out, **{**ok, **bad})
+        assert e.value.status == status, (bad, e.value.status)
