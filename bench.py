@@ -220,11 +220,31 @@ def main():
                      "unit": "TFLOP/s", "frac": round(achieved / PEAK_F16_TFLOPS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES["mmt4d_f16_4096"]},
     }
+    # The headline line must not be lost to a failure in a secondary
+    # measurement: what was measured up to there is kept, the error is reported
+    # in the line and on stderr, and the exit status says so.
+    failed = False
     if not args.no_extra:
-        result["extra"] = extras(args, torch, iree_amd, F, synth, lhs, rhs, out)
+        result["extra"] = {}
+        try:
+            extras(args, torch, iree_amd, F, synth, lhs, rhs, out, result["extra"])
+        except Exception as e:  # noqa: BLE001
+            import traceback
+            traceback.print_exc()
+            result["extra_error"] = f"{type(e).__name__}: {e}"
+            failed = True
     if not args.no_cpu:
-        result["cpu_baseline"] = cpu_baseline(F, synth, size)
+        try:
+            result["cpu_baseline"] = cpu_baseline(F, synth, size)
+        except Exception as e:  # noqa: BLE001
+            import traceback
+            traceback.print_exc()
+            result["cpu_baseline"] = {"value": None, "unit": "TFLOP/s", "cores": 0, "kind": "port",
+                                      "sample": f"failed: {type(e).__name__}: {e}"}
+            failed = True
     print(json.dumps(result))
+    if failed:
+        sys.exit(1)
 
 
 def verify_tiles(torch, iree_amd, F, lhs, rhs, out, M1, N1, K1, M0, N0, K0):
@@ -273,8 +293,7 @@ def make_fp8_mlp(torch, iree_amd):
     return mlp, xm, ym, Mt, Hd, Ff
 
 
-def extras(args, torch, iree_amd, F, synth, lhs, rhs, out):
-    ex = {}
+def extras(args, torch, iree_amd, F, synth, lhs, rhs, out, ex):
     size = 4096
     steps, warm = args.steps, args.warmup
     M1 = N1 = size // 32
