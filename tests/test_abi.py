@@ -163,4 +163,17 @@ def test_validation_happens_before_any_device_work():
     assert lib.iree_amd_uk_unpack(one, 0, 8, 4, one, 0, 4, 1, 1, 2, 2, 2, 2, 4, 2, None, None) == 3
     assert lib.iree_amd_uk_unpack(None, 0, 8, 4, None, 0, 4, 1, 1, 2, 2, 2, 0, 4, 1, None, None) == 0
     assert lib.iree_amd_uk_dequant_matmul_i4(one, one, one, one, one, 1, 8, 100, 32, 0, None) == 3
+    # the fused forms: size conditions of unpack for 32x32 tiles, row pitches, scale rules, empty calls
+    f1 = C.c_float(1.0)
+    mu = lib.iree_amd_uk_mmt4d_unpack
+    assert mu(one, 0, 512, one, 0, 512, one, 0, 64, 32, 64, 2, 2, 2, 16, 2, f1, None) == 3    # 32 rows cannot need 2 outer rows
+    assert mu(one, 0, 512, one, 0, 512, one, 0, 63, 33, 64, 2, 2, 2, 16, 2, f1, None) == 3    # pitch below a row
+    assert mu(one, 0, 512, one, 0, 512, one, 0, 64, 33, 64, 2, 2, 2, 16, 2, C.c_float(2.0), None) == 3   # scale on integers
+    assert mu(None, 0, 512, None, 0, 512, None, 0, 64, 0, 64, 0, 2, 2, 16, 2, f1, None) == 0
+    mp = lib.iree_amd_uk_matmul_packed_rhs
+    assert mp(one, 0, 64, one, 0, 2048, one, 0, 64, 33, 64, 64, 0, 2, f1, None) == 3        # K0 = 0
+    assert mp(one, 0, 63, one, 0, 2048, one, 0, 64, 33, 64, 64, 16, 2, f1, None) == 3       # lhs pitch below a row
+    assert mp(one, 0, 64, one, 0, 2048, one, 0, 64, 33, 64, 40, 16, 2, f1, None) == 12      # K not whole tiles
+    assert mp(None, 0, 64, None, 0, 2048, None, 0, 64, 0, 64, 64, 16, 2, f1, None) == 0
+    assert lib.iree_amd_uk_mfma_probe(2, None, 1, None, None, None) == 3
     assert lib.iree_amd_uk_version() >= 1
