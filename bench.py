@@ -430,7 +430,14 @@ def extras(args, torch, iree_amd, F, synth, lhs, rhs, out, ex):
                                                               F.MMT4D_TYPE_S8S8S32, workspace=ws8),
                     steps, warm)
     ex["matmul_i8_1024_chain_us"] = round(t * 1e6, 1)
-    del a8, b8, c8, ws8
+    # the same product as one launch: right-hand side packed ahead of time,
+    # left-hand side read row-major, row-major result
+    c8_chain = c8.clone()
+    _, t = gpu_time(torch, lambda: iree_amd.matmul_packed_rhs(a8, ws8["rhs"], c8, n1k, n1k, n1k, 16,
+                                                              F.MMT4D_TYPE_S8S8S32), steps, warm)
+    ex["matmul_i8_1024_one_kernel_us"] = round(t * 1e6, 1)
+    assert torch.equal(c8, c8_chain), "one-kernel i8 matmul differs from the chain"
+    del a8, b8, c8, ws8, c8_chain
 
     # grouped int4 dequant matmul, decode shapes (K = 4096, N = 14336, groups of
     # 128, f16 scales, packed uint4 zero points, pre-tiled weights). Ten weight
