@@ -1,6 +1,7 @@
 // MFMA instruction wrappers shared by the matmul kernels: one struct per
-// element-type tuple giving the operand fragment type of one lane, the
-// accumulator type of a 32x32 block and the instruction.
+// element-type tuple and instruction shape giving the operand fragment type of
+// one lane (16 bytes per 1 KiB operand block), the accumulator type of one
+// kRows x kRows block and the instruction.
 #ifndef IREE_AMD_UK_MFMA_CFG_H_
 #define IREE_AMD_UK_MFMA_CFG_H_
 
@@ -18,6 +19,7 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef int intx16 __attribute__((ext_vector_type(16)));
 
 struct F16Cfg {
+  static constexpr int kRows = 32;     // the instruction's block is kRows x kRows
   typedef half8 frag_t;
   typedef floatx16 acc_t;
   typedef float out_t;
@@ -29,6 +31,7 @@ struct F16Cfg {
   }
 };
 struct BF16Cfg {
+  static constexpr int kRows = 32;     // the instruction's block is kRows x kRows
   typedef bf16x8 frag_t;
   typedef floatx16 acc_t;
   typedef float out_t;
@@ -38,6 +41,43 @@ struct BF16Cfg {
   __device__ static acc_t mfma(frag_t a, frag_t b, acc_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
+};
+// The 16x16x32 shapes of the same types: half the rows, twice the K per
+// instruction, the same 1 KiB operand block per fragment (lane l: row l % 16,
+// k = 8 (l / 16) .. + 8). Measured on MI355X with N(0,1) data and no memory
+// traffic at all, v_mfma_f32_16x16x32_f16 sustains 1.80-1.85 PFLOP/s where
+// v_mfma_f32_32x32x16_f16 sustains 1.60: the matrix pipe is power-limited and
+// the smaller block costs less energy per flop (with all-zero operands both
+// run at 2.3-2.4).
+struct F16Cfg16 {
+  static constexpr int kRows = 16;
+  typedef half8 frag_t;
+  typedef floatx4 acc_t;
+  typedef float out_t;
+  static constexpr int kElemBytes = 2;
+  static constexpr int kMfmaK = 32;
+  static constexpr int kSub = 1;
+  __device__ static acc_t mfma(frag_t a, frag_t b, acc_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  }
+};
+struct BF16Cfg16 {
+  static constexpr int kRows = 16;
+  typedef bf16x8 frag_t;
+  typedef floatx4 acc_t;
+  typedef float out_t;
+  static constexpr int kElemBytes = 2;
+  static constexpr int kMfmaK = 32;
+  static constexpr int kSub = 1;
+  __device__ static acc_t mfma(frag_t a, frag_t b, acc_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+};
+struct F16F16Cfg16 : F16Cfg16 {
+  typedef _Float16 out_t;
+};
+struct BF16BF16Cfg16 : BF16Cfg16 {
+  typedef __bf16 out_t;
 };
 // f16 / bf16 results: f32 accumulation, one rounding (to nearest even) when the
 // accumulators are stored, which is the reference's arithmetic when
@@ -54,6 +94,7 @@ struct BF16BF16Cfg : BF16Cfg {
 // and element e of lanes 32..63 form the k pair of the e-th of four
 // instructions; both operands pair the same way, so every k meets its partner.
 struct F32Cfg {
+  static constexpr int kRows = 32;     // the instruction's block is kRows x kRows
   typedef floatx4 frag_t;
   typedef floatx16 acc_t;
   typedef float out_t;
@@ -67,6 +108,7 @@ struct F32Cfg {
   }
 };
 struct S8Cfg {
+  static constexpr int kRows = 32;     // the instruction's block is kRows x kRows
   typedef int4v frag_t;
   typedef intx16 acc_t;
   typedef int32_t out_t;
@@ -78,6 +120,7 @@ struct S8Cfg {
   }
 };
 struct F8Cfg {
+  static constexpr int kRows = 32;     // the instruction's block is kRows x kRows
   typedef int8v frag_t;
   typedef floatx16 acc_t;
   typedef float out_t;

@@ -68,7 +68,7 @@ struct MfmaArgs {
   // of (outer row i, K-step ks) is rows 32 i .. 32 i + 31, bytes
   // lhs_step_bytes * ks .. of each row
   int lhs_row_major;
-  int half_k0;       // K0 is half the MFMA's K extent (else the full extent)
+  int k0_div;        // the instruction's K extent / K0: 1, 2 (or 4 for the 16-row shapes)
   // fused SiLU * up epilogue only: scales of the gate and up accumulators and
   // the inverse scale of the e4m3 result
   float gate_scale, up_scale, inv_out_scale;
@@ -165,10 +165,16 @@ __global__ __launch_bounds__(128 * kWavesN, kOcc) void mmt4d_mfma_kernel(MfmaArg
   typedef typename Cfg::acc_t acc_t;
   typedef typename Cfg::out_t out_t;
   constexpr int kWaves = 2 * kWavesN;                // a 2 x kWavesN grid of waves
-  constexpr int TM = 2 * WM, TN = kWavesN * WN;      // outer tiles per workgroup
+  // WM, WN, TM, TN count BLOCKS of R rows (R = 32 or 16: the instruction's
+  // block); an outer tile of 32 rows is kPerTile of them.
+  constexpr int R = Cfg::kRows, kPerTile = 32 / R;
+  constexpr int kAccRegs = R * R / 64;               // accumulator registers of one block
+  constexpr int kChunks = 64 / R;                    // 16-byte K chunks of a fragment row
+  constexpr int TM = 2 * WM, TN = kWavesN * WN;      // blocks per workgroup
+  static_assert(R == 32 || (R == 16 && Cfg::kSub == 1 && !kSiluMul), "unsupported block shape");
   static_assert(TM % kWaves == 0 && TN % kWaves == 0, "every wave loads whole operand rows");
   constexpr int kSub = Cfg::kSub;
-  constexpr int kBlockBytes = kSub * kPieceBytes;   // one 32-row operand block of one K-step
+  constexpr int kBlockBytes = kSub * kPieceBytes;   // one R-row operand block of one K-step
   constexpr int kABytes = TM * kBlockBytes;
   constexpr int kSlotBytes = (TM + TN) * kBlockBytes;
   constexpr int kAhead = kRing - kSync;
@@ -181,8 +187,9 @@ __global__ __launch_bounds__(128 * kWavesN, kOcc) void mmt4d_mfma_kernel(MfmaArg
   // them (from the front) get fragment reads slipped in behind them: the last
   // third or so stays free so that the reads have landed when the step ends.
   constexpr int kMfmaAll = WM * WN, kMfmaRest = (WM - 1) * WN;
-  constexpr int kReadAll = kMfmaAll - (kMfmaAll >= 8 ? 6 : kMfmaAll / 2);
-  constexpr int kReadRest = kMfmaRest - (kMfmaRest >= 8 ? 4 : kMfmaRest / 2);
+  constexpr int kTail = kPerTile * kPerTile;    // (a 16x16 MFMA is half as long)
+  constexpr int kReadAll = kMfmaAll - (kMfmaAll >= 8 * kTail ? 6 * kTail : kMfmaAll / 2);
+  constexpr int kReadRest = kMfmaRest - (kMfmaRest >= 8 * kTail ? 4 * kTail : kMfmaRest / 2);
   static_assert(kAhead >= kSync, "ring must hold two sync groups");
   static_assert(kPro >= kBody - 1, "the loop's remainder must already be in the ring");
   static_assert((kPro - kSync) * kLoadsPerStep < 64, "too many loads in flight for vmcnt");
@@ -196,11 +203,21 @@ __global__ __launch_bounds__(128 * kWavesN, kOcc) void mmt4d_mfma_kernel(MfmaArg
   const int i_base = tm * TM, j_base = tn * TN;
   const int T = a.ksteps;
 
-  // Per-lane byte offset inside an operand block in global memory (of its
-  // first piece; with two pieces the second lies one 512-byte tile further).
-  const uint32_t lane_off = kSub == 2 ? ((lane >> 5) * 1024 + (lane & 31) * 16)
-                       : a.half_k0 ? lane * 16 : ((lane & 31) * 32 + (lane >> 5) * 16);
+  // Per-lane byte offset of a fragment inside the K-step of its outer row in
+  // global memory. A lane feeds the instruction row l % R, 16-byte K chunk
+  // l / R; a packed tile holds `cpt` chunks per row (K0 = the instruction's K
+  // extent / k0_div), so chunk c lies in tile c / cpt at row pitch 16 cpt.
+  // `sub` selects the block of R rows inside the 32-row tile. (fp8: two pieces
+  // per lane, the second one 512-byte tile further.)
+  const int frag_row = lane % R, frag_chunk = lane / R;
+  const int cpt = kChunks / a.k0_div;
+  auto packed_lane_off = [&](int sub) -> uint32_t {
+    if constexpr (kSub == 2) return (lane >> 5) * 1024 + (lane & 31) * 16;
+    return (uint32_t)((frag_chunk / cpt) * 512 * cpt + (sub * R + frag_row) * 16 * cpt +
+                      (frag_chunk % cpt) * 16);
+  };
   constexpr int kPieceStride = 512;
+  constexpr int kStepBytes = kPerTile * kBlockBytes;   // of one outer row of packed tiles
 
   // Rows this wave copies: its share of the TM rows of A and TN of B. Out-of-range
   // rows are clamped to the last valid one (loaded, never stored).
@@ -210,29 +227,40 @@ __global__ __launch_bounds__(128 * kWavesN, kOcc) void mmt4d_mfma_kernel(MfmaArg
   // Row-major: lane l reads row l % 32 (clamped to the last matrix row), the
   // 16 * kSub bytes of half l / 32 of the K-step: the same bytes in the same
   // lane order, so LDS and everything behind it are unchanged.
-  uint32_t a_lane_off[kARowsPerWave];
-  const uint32_t a_step_bytes = a.lhs_row_major ? 32 * kSub : kBlockBytes;
+  uint32_t a_lane_off[kARowsPerWave], b_lane_off[kBRowsPerWave];
+  const uint32_t a_step_bytes = a.lhs_row_major ? kChunks * 16 * kSub : kStepBytes;
   const uint32_t a_piece_stride = a.lhs_row_major ? 16 : kPieceStride;
 #pragma unroll
   for (int r = 0; r < kARowsPerWave; ++r) {
-    int i = i_base + wave * kARowsPerWave + r;
+    const int blk = i_base + wave * kARowsPerWave + r;
+    int i = blk / kPerTile;
+    const int sub = blk % kPerTile;
     i = i < a.M ? i : a.M - 1;
     if (a.lhs_row_major) {
-      int row = i * 32 + (lane & 31);
+      int row = i * 32 + sub * R + frag_row;
       row = row < a.out_rows ? row : a.out_rows - 1;
       a_src[r] = row_descriptor(a.lhs);
-      a_lane_off[r] = (uint32_t)row * (uint32_t)a.lhs_stride_bytes + (lane >> 5) * 16 * kSub;
+      a_lane_off[r] = (uint32_t)row * (uint32_t)a.lhs_stride_bytes + frag_chunk * 16 * kSub;
     } else {
       a_src[r] = row_descriptor(a.lhs + (int64_t)i * a.lhs_stride_bytes);
-      a_lane_off[r] = lane_off;
+      a_lane_off[r] = packed_lane_off(sub);
     }
   }
 #pragma unroll
   for (int r = 0; r < kBRowsPerWave; ++r) {
-    int j = j_base + wave * kBRowsPerWave + r;
+    const int blk = j_base + wave * kBRowsPerWave + r;
+    int j = blk / kPerTile;
     j = j < a.N ? j : a.N - 1;
     b_src[r] = row_descriptor(a.rhs + (int64_t)j * a.rhs_stride_bytes);
+    b_lane_off[r] = packed_lane_off(blk % kPerTile);
   }
+  // Accumulator element v of this lane: row and column inside its block
+  // (32x32: register v of lane l is row 8 (v / 4) + 4 (l / 32) + v % 4, column
+  // l % 32; 16x16: row 4 (l / 16) + v, column l % 16).
+  auto acc_row = [&](int v) -> int {
+    return R == 32 ? 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3) : 4 * (lane >> 4) + v;
+  };
+  const int acc_col = lane % R;
 
   acc_t acc[WM][WN];
   if (a.accumulate && a.row_major_out) {
@@ -242,12 +270,12 @@ __global__ __launch_bounds__(128 * kWavesN, kOcc) void mmt4d_mfma_kernel(MfmaArg
     for (int x = 0; x < WM; ++x)
 #pragma unroll
       for (int y = 0; y < WN; ++y) {
-        int col = (j_base + wn * WN + y) * 32 + (lane & 31);
+        int col = (j_base + wn * WN + y) * R + acc_col;
         col = col < a.out_cols ? col : a.out_cols - 1;
-        const int row0 = (i_base + wm * WM + x) * 32 + 4 * (lane >> 5);
+        const int row0 = (i_base + wm * WM + x) * R;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          int row = row0 + 8 * (v >> 2) + (v & 3);
+        for (int v = 0; v < kAccRegs; ++v) {
+          int row = row0 + acc_row(v);
           row = row < a.out_rows ? row : a.out_rows - 1;
           acc[x][y][v] = *((const out_t*)(a.out + (int64_t)row * a.out_stride_bytes) + col);
         }
@@ -257,13 +285,14 @@ __global__ __launch_bounds__(128 * kWavesN, kOcc) void mmt4d_mfma_kernel(MfmaArg
     for (int x = 0; x < WM; ++x)
 #pragma unroll
       for (int y = 0; y < WN; ++y) {
-        int i = i_base + wm * WM + x, j = j_base + wn * WN + y;
+        const int bi = i_base + wm * WM + x, bj = j_base + wn * WN + y;
+        int i = bi / kPerTile, j = bj / kPerTile;
         i = i < a.M ? i : a.M - 1;
         j = j < a.N ? j : a.N - 1;
-        const out_t* t = (const out_t*)(a.out + (int64_t)i * a.out_stride_bytes) + (int64_t)j * 1024;
+        const out_t* t = (const out_t*)(a.out + (int64_t)i * a.out_stride_bytes) + (int64_t)j * 1024 +
+                         (bi % kPerTile) * R * 32 + (bj % kPerTile) * R;
 #pragma unroll
-        for (int v = 0; v < 16; ++v)
-          acc[x][y][v] = t[(8 * (v >> 2) + 4 * (lane >> 5) + (v & 3)) * 32 + (lane & 31)];
+        for (int v = 0; v < kAccRegs; ++v) acc[x][y][v] = t[acc_row(v) * 32 + acc_col];
       }
   } else {
 #pragma unroll
@@ -271,7 +300,7 @@ __global__ __launch_bounds__(128 * kWavesN, kOcc) void mmt4d_mfma_kernel(MfmaArg
 #pragma unroll
       for (int y = 0; y < WN; ++y)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) acc[x][y][v] = 0;
+        for (int v = 0; v < kAccRegs; ++v) acc[x][y][v] = 0;
   }
 
   // Load `d` (of kLoadsPerStep) of this wave's share of K-step `ks` into ring
@@ -284,7 +313,7 @@ __global__ __launch_bounds__(128 * kWavesN, kOcc) void mmt4d_mfma_kernel(MfmaArg
                         base + (wave * kARowsPerWave + r) * kBlockBytes + j * kPieceBytes);
     } else {
       const int rb = r - kARowsPerWave;
-      load_block_to_lds(b_src[rb], lane_off, (uint32_t)ks * kBlockBytes + j * kPieceStride,
+      load_block_to_lds(b_src[rb], b_lane_off[rb], (uint32_t)ks * kStepBytes + j * kPieceStride,
                         base + kABytes + (wave * kBRowsPerWave + rb) * kBlockBytes + j * kPieceBytes);
     }
   };
@@ -426,12 +455,13 @@ __global__ __launch_bounds__(128 * kWavesN, kOcc) void mmt4d_mfma_kernel(MfmaArg
   // come straight from global memory, with zeros in the lanes (or lane halves)
   // that stand for the missing tiles.
   if (a.tail_tiles > 0) {
-    const int64_t tail_off = (int64_t)T * kBlockBytes;
-    auto tail_frag = [&](const char* block) -> frag_t {
+    const int64_t tail_off = (int64_t)T * kStepBytes;
+    auto tail_frag = [&](const char* block, int sub) -> frag_t {
       const int4v zero = {0, 0, 0, 0};
       if constexpr (kSub == 1) {
-        // (reached with K0 = half the MFMA extent only: lanes 32..63 hold the second tile)
-        const int4v v = (lane >> 5) < a.tail_tiles ? *(const int4v*)(block + lane * 16) : zero;
+        // (reached with a K0 below the instruction's K extent only: the lane's
+        // chunk belongs to K tile chunk / cpt of the step)
+        const int4v v = (frag_chunk / cpt) < a.tail_tiles ? *(const int4v*)(block + packed_lane_off(sub)) : zero;
         union { int4v i; frag_t f; } u;
         u.i = v;
         return u.f;
@@ -445,22 +475,24 @@ __global__ __launch_bounds__(128 * kWavesN, kOcc) void mmt4d_mfma_kernel(MfmaArg
     };
 #pragma unroll
     for (int x = 0; x < WM; ++x) {
-      int i = i_base + wm * WM + x;
+      const int blk = i_base + wm * WM + x;
+      int i = blk / kPerTile;
       i = i < a.M ? i : a.M - 1;
-      fa[0][x] = tail_frag(a.lhs + (int64_t)i * a.lhs_stride_bytes + tail_off);
+      fa[0][x] = tail_frag(a.lhs + (int64_t)i * a.lhs_stride_bytes + tail_off, blk % kPerTile);
     }
 #pragma unroll
     for (int y = 0; y < WN; ++y) {
-      int j = j_base + wn * WN + y;
+      const int blk = j_base + wn * WN + y;
+      int j = blk / kPerTile;
       j = j < a.N ? j : a.N - 1;
-      fb[0][y] = tail_frag(a.rhs + (int64_t)j * a.rhs_stride_bytes + tail_off);
+      fb[0][y] = tail_frag(a.rhs + (int64_t)j * a.rhs_stride_bytes + tail_off, blk % kPerTile);
     }
     multiply(fa[0], fb[0]);
   }
 
-  // Epilogue. MFMA 32x32 accumulator layout: register v of lane l holds
-  // row 8*(v/4) + 4*(l/32) + v%4, column l%32 of the block; one store
-  // instruction therefore writes two full 128-byte rows of the tile.
+  // Epilogue (accumulator layout: acc_row / acc_col above). With 32x32 blocks
+  // one store instruction writes two full 128-byte rows of the tile, with
+  // 16x16 blocks four 64-byte row pieces.
   if constexpr (kSiluMul) {
     static_assert(WN % 2 == 0, "gate/up pairs must not straddle waves");
     // Block pair (y, y+1) -> 32x32 bytes, stored as the two 32x16 tiles
@@ -498,12 +530,12 @@ __global__ __launch_bounds__(128 * kWavesN, kOcc) void mmt4d_mfma_kernel(MfmaArg
     for (int x = 0; x < WM; ++x)
 #pragma unroll
       for (int y = 0; y < WN; ++y) {
-        const int col = (j_base + wn * WN + y) * 32 + (lane & 31);
-        const int row0 = (i_base + wm * WM + x) * 32 + 4 * (lane >> 5);
+        const int col = (j_base + wn * WN + y) * R + acc_col;
+        const int row0 = (i_base + wm * WM + x) * R;
         if (col < a.out_cols) {
 #pragma unroll
-          for (int v = 0; v < 16; ++v) {
-            const int row = row0 + 8 * (v >> 2) + (v & 3);
+          for (int v = 0; v < kAccRegs; ++v) {
+            const int row = row0 + acc_row(v);
             if (row < a.out_rows) {
               out_t* dst = (out_t*)(a.out + (int64_t)row * a.out_stride_bytes) + col;
               if constexpr (std::is_floating_point<decltype(acc[x][y][v] + 0)>::value)
@@ -520,12 +552,13 @@ __global__ __launch_bounds__(128 * kWavesN, kOcc) void mmt4d_mfma_kernel(MfmaArg
   for (int x = 0; x < WM; ++x)
 #pragma unroll
     for (int y = 0; y < WN; ++y) {
-      const int i = i_base + wm * WM + x, j = j_base + wn * WN + y;
+      const int bi = i_base + wm * WM + x, bj = j_base + wn * WN + y;
+      const int i = bi / kPerTile, j = bj / kPerTile;
       if (i < a.M && j < a.N) {
-        out_t* t = (out_t*)(a.out + (int64_t)i * a.out_stride_bytes) + (int64_t)j * 1024;
+        out_t* t = (out_t*)(a.out + (int64_t)i * a.out_stride_bytes) + (int64_t)j * 1024 +
+                   (bi % kPerTile) * R * 32 + (bj % kPerTile) * R;
 #pragma unroll
-        for (int v = 0; v < 16; ++v)
-          t[(8 * (v >> 2) + 4 * (lane >> 5) + (v & 3)) * 32 + (lane & 31)] = acc[x][y][v];
+        for (int v = 0; v < kAccRegs; ++v) t[acc_row(v) * 32 + acc_col] = acc[x][y][v];
       }
     }
 }
@@ -534,9 +567,11 @@ template <typename Cfg, int WM, int WN, int kRing, int kSync, int kOcc = 1, bool
           int kWavesN = 2>
 int launch_variant(const MfmaArgs& a0, hipStream_t s) {
   MfmaArgs a = a0;
-  constexpr int TM = 2 * WM, TN = kWavesN * WN;
-  a.tiles_m = (a.M + TM - 1) / TM;
-  a.tiles_n = (a.N + TN - 1) / TN;
+  constexpr int kPerTile = 32 / Cfg::kRows;
+  constexpr int TM = 2 * WM, TN = kWavesN * WN;   // blocks of Cfg::kRows rows
+  static_assert(TM % kPerTile == 0 && TN % kPerTile == 0, "a workgroup covers whole outer tiles");
+  a.tiles_m = (a.M * kPerTile + TM - 1) / TM;
+  a.tiles_n = (a.N * kPerTile + TN - 1) / TN;
   const int64_t blocks = (int64_t)a.tiles_m * a.tiles_n;
   if (blocks > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
   constexpr int lds_bytes = kRing * (TM + TN) * Cfg::kSub * kPieceBytes;
@@ -575,8 +610,11 @@ int launch_cfg(const MfmaArgs& a, hipStream_t s) {
   // With the SiLU epilogue, whose arithmetic the second workgroup hides and
   // whose output is an eighth of the bytes, it is the other way round: 218
   // against 198 us.)
-  constexpr bool kWide = Cfg::kSub == 2;
-  constexpr bool kShallow = kWide && !kSiluMul;
+  // S: blocks per 32 rows. The 16-row shapes and fp8 have K-steps of twice the
+  // bytes ("wide"), hence the shorter rings.
+  constexpr int S = 32 / Cfg::kRows;
+  constexpr bool kWide = Cfg::kSub == 2 || S == 2;
+  constexpr bool kShallow = Cfg::kSub == 2 && !kSiluMul;
   struct Variant { int wm, wn, occ; double eff_alone, eff_full; };
   static const Variant variants[4] = {{4, 4, 1, 1.0, 1.0},
                                       {4, 2, 2, kShallow ? 0.85 : 0.9, kShallow ? 0.82 : 0.94},
@@ -598,25 +636,29 @@ int launch_cfg(const MfmaArgs& a, hipStream_t s) {
     if (v == 0 || cost < best_cost * 0.999) { best = v; best_cost = cost; }
   }
   switch (best) {
-    case 0: return launch_variant<Cfg, 4, 4, kWide ? 5 : 8, kWide ? 1 : 2, 1, kSiluMul>(a, s);
-    case 1: return launch_variant<Cfg, 4, 2, kWide ? 3 : 6, kWide ? 1 : 2, 2, kSiluMul>(a, s);
-    case 2: return launch_variant<Cfg, 2, 4, kWide ? 3 : 6, kWide ? 1 : 2, 2, kSiluMul>(a, s);
-    default: return launch_variant<Cfg, 2, 2, 8, 2, 1, kSiluMul>(a, s);
+    case 0: return launch_variant<Cfg, 4 * S, 4 * S, kWide ? 5 : 8, kWide ? 1 : 2, 1, kSiluMul>(a, s);
+    case 1: return launch_variant<Cfg, 4 * S, 2 * S, kWide ? 3 : 6, kWide ? 1 : 2, 2, kSiluMul>(a, s);
+    case 2: return launch_variant<Cfg, 2 * S, 4 * S, kWide ? 3 : 6, kWide ? 1 : 2, 2, kSiluMul>(a, s);
+    default: return launch_variant<Cfg, 2 * S, 2 * S, S == 2 ? 4 : 8, S == 2 ? 1 : 2, 1, kSiluMul>(a, s);
   }
 }
 
+// mfma_k: K extent of the instruction the call runs on. f16 / bf16 use the
+// 16x16x32 shapes, except with the fused SiLU epilogue (32x32x16).
 struct Served { int mfma_k; };
-bool served(uint32_t flags, int M0, int N0, int K0, Served* out) {
+bool served(uint32_t flags, int M0, int N0, int K0, bool silu, Served* out) {
   int mfma_k = 0;
+  bool half_type = false;
   switch (flags & IREE_AMD_UK_FLAG_MMT4D_TYPE_MASK) {
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F32:
-    case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16F32: mfma_k = 16; break;
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16F32: mfma_k = silu ? 16 : 32; half_type = true; break;
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F16:
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16BF16:
       // f32 accumulation with one final rounding is only the reference's
       // arithmetic when intermediate roundings are skipped
       if (!(flags & IREE_AMD_UK_FLAG_MMT4D_SKIP_INTERMEDIATE_ROUNDINGS)) return false;
-      mfma_k = 16;
+      mfma_k = silu ? 16 : 32;
+      half_type = true;
       break;
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_F32F32F32: mfma_k = 8; break;
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32: mfma_k = 32; break;
@@ -626,6 +668,8 @@ bool served(uint32_t flags, int M0, int N0, int K0, Served* out) {
   if (M0 != 32 || N0 != 32) return false;
   if (mfma_k == 64) {
     if (K0 != 16) return false;
+  } else if (half_type) {
+    if (K0 != 8 && K0 != 16) return false;   // a quarter / half (or half / all) of the K extent
   } else if (K0 != mfma_k && K0 * 2 != mfma_k) {
     return false;
   }
@@ -636,14 +680,14 @@ bool served(uint32_t flags, int M0, int N0, int K0, Served* out) {
 }  // namespace
 
 bool mmt4d_mfma_supported(uint32_t flags, int M0, int N0, int K0) {
-  return served(flags, M0, N0, K0, nullptr);
+  return served(flags, M0, N0, K0, false, nullptr);
 }
 
 namespace {
 // Fills `a` from the parameters; NOT_FOUND when the MFMA kernels cannot take the call.
-int make_args(const iree_amd_uk_mmt4d_params_t& p, int out_elem_bytes, MfmaArgs* out_args) {
+int make_args(const iree_amd_uk_mmt4d_params_t& p, int out_elem_bytes, bool silu, MfmaArgs* out_args) {
   Served sv;
-  if (!served(p.flags, p.M0, p.N0, p.K0, &sv)) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  if (!served(p.flags, p.M0, p.N0, p.K0, silu, &sv)) return IREE_AMD_UK_STATUS_NOT_FOUND;
   Mmt4dTypeInfo ti;
   mmt4d_type_info(p.flags, &ti);
   const int eb = ti.lhs_bits / 8;
@@ -668,7 +712,7 @@ int make_args(const iree_amd_uk_mmt4d_params_t& p, int out_elem_bytes, MfmaArgs*
   a.tail_tiles = (int)((k_elems % sv.mfma_k) / p.K0);
   a.tiles_m = a.tiles_n = 0;
   a.accumulate = (p.flags & IREE_AMD_UK_FLAG_MMT4D_ACCUMULATE) != 0;
-  a.half_k0 = p.K0 * 2 == sv.mfma_k;
+  a.k0_div = sv.mfma_k / p.K0;
   a.row_major_out = 0; a.out_rows = a.out_cols = 0;
   a.lhs_row_major = 0;
   a.gate_scale = a.up_scale = a.inv_out_scale = a.out_scale = 1.0f;
@@ -684,7 +728,7 @@ int launch_mmt4d_mfma(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) {
   Mmt4dTypeInfo ti;
   mmt4d_type_info(p.flags, &ti);
   MfmaArgs a;
-  const int st = make_args(p, ti.out_bytes, &a);
+  const int st = make_args(p, ti.out_bytes, false, &a);
   if (st) return st;
   return launch_typed(p, a, s);
 }
@@ -698,7 +742,7 @@ int launch_mmt4d_unpack_mfma(const iree_amd_uk_mmt4d_params_t& p, int64_t out_ro
   Mmt4dTypeInfo ti;
   mmt4d_type_info(p.flags, &ti);
   MfmaArgs a;
-  const int st = make_args(p, ti.out_bytes, &a);
+  const int st = make_args(p, ti.out_bytes, false, &a);
   if (st) return st;
   if (out_rows > 0x7FFFFFFF || out_cols > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
   a.row_major_out = 1;
@@ -717,7 +761,7 @@ int launch_matmul_packed_rhs_mfma(const iree_amd_uk_mmt4d_params_t& p, int64_t o
   Mmt4dTypeInfo ti;
   mmt4d_type_info(p.flags, &ti);
   MfmaArgs a;
-  const int st = make_args(p, ti.out_bytes, &a);
+  const int st = make_args(p, ti.out_bytes, false, &a);
   if (st) return st;
   // whole matrix-core K-steps only (a partial one would read past the row end),
   // and a matrix that 32-bit byte offsets can address
@@ -735,13 +779,13 @@ int launch_matmul_packed_rhs_mfma(const iree_amd_uk_mmt4d_params_t& p, int64_t o
 namespace {
 int launch_typed(const iree_amd_uk_mmt4d_params_t& p, const MfmaArgs& a, hipStream_t s) {
   switch (p.flags & IREE_AMD_UK_FLAG_MMT4D_TYPE_MASK) {
-    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F32: return launch_cfg<F16Cfg>(a, s);
-    case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16F32: return launch_cfg<BF16Cfg>(a, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F32: return launch_cfg<F16Cfg16>(a, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16F32: return launch_cfg<BF16Cfg16>(a, s);
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32: return launch_cfg<S8Cfg>(a, s);
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_F8E4M3F8E4M3F32: return launch_cfg<F8Cfg>(a, s);
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_F32F32F32: return launch_cfg<F32Cfg>(a, s);
-    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F16: return launch_cfg<F16F16Cfg>(a, s);
-    case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16BF16: return launch_cfg<BF16BF16Cfg>(a, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F16: return launch_cfg<F16F16Cfg16>(a, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16BF16: return launch_cfg<BF16BF16Cfg16>(a, s);
     default: return IREE_AMD_UK_STATUS_NOT_FOUND;
   }
 }
@@ -753,7 +797,7 @@ int launch_typed(const iree_amd_uk_mmt4d_params_t& p, const MfmaArgs& a, hipStre
 int launch_mmt4d_silu_mul_mfma(const iree_amd_uk_mmt4d_params_t& p, float gate_scale,
                                float up_scale, float inv_out_scale, hipStream_t s) {
   MfmaArgs a;
-  const int st = make_args(p, 1, &a);
+  const int st = make_args(p, 1, true, &a);
   if (st) return st;
   a.gate_scale = gate_scale; a.up_scale = up_scale; a.inv_out_scale = inv_out_scale;
   a.accumulate = 0;

@@ -469,8 +469,8 @@ def test_i8_matmul_with_packed_rhs_in_one_kernel_is_bit_exact(uk, cuda, M, N, K,
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("type_flag,K0,dt,K", [(F.MMT4D_TYPE_F16F16F32, 8, np.float16, 16 * 19),
-                                               (F.MMT4D_TYPE_F16F16F32, 16, np.float16, 16 * 19),
+@pytest.mark.parametrize("type_flag,K0,dt,K", [(F.MMT4D_TYPE_F16F16F32, 8, np.float16, 32 * 9),
+                                               (F.MMT4D_TYPE_F16F16F32, 16, np.float16, 32 * 9),
                                                (F.MMT4D_TYPE_F32F32F32, 4, np.float32, 8 * 21),
                                                (F.MMT4D_TYPE_F8E4M3F8E4M3F32, 16, np.uint8, 64 * 5)])
 def test_matmul_packed_rhs_equals_pack_mmt4d_unpack_bitwise(uk, cuda, type_flag, K0, dt, K):
