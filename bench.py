@@ -310,8 +310,8 @@ def extras(args, torch, iree_amd, F, synth, lhs, rhs, out, ex):
                                 ("f16_zeros", F.MMT4D_TYPE_F16F16F32, zeros),
                                 ("i8_uniform", F.MMT4D_TYPE_S8S8S32, rnd8),
                                 ("i8_zeros", F.MMT4D_TYPE_S8S8S32, zeros)):
-        n_ops = iree_amd.mfma_probe(flag, ops_buf, 512, sink)
-        _, t = gpu_time(torch, lambda: iree_amd.mfma_probe(flag, ops_buf, 512, sink), steps, warm)
+        n_ops = iree_amd.mfma_probe(flag, ops_buf, 256, sink)
+        _, t = gpu_time(torch, lambda: iree_amd.mfma_probe(flag, ops_buf, 256, sink), steps, warm)
         ex[f"mfma_register_only_{name}_tops"] = round(n_ops / t / 1e12, 1)
     del sink, zeros, rnd8
 

@@ -461,16 +461,16 @@ IREE_AMD_UK_EXPORT int iree_amd_uk_scale_f32(void* buf_f32, iree_amd_uk_index_t 
                                              float scale, void* stream);
 
 /* Measurement aid with no counterpart in the reference: runs the mmt4d
- * kernel's matrix-core instruction pattern (4 x 4 accumulator blocks per wave,
- * one workgroup of 4 waves per compute unit) for `iters` K-steps on operand
+ * kernel's matrix-core instruction pattern (every accumulator block of a wave's
+ * 128 x 128 tile once per K-step, with the instruction shape the kernel uses for
+ * the type; one workgroup of 4 waves per compute unit) for `iters` K-steps on operand
  * fragments that are read ONCE from `operands` and then stay in registers, so
  * the launch does no memory traffic. Timing it gives the rate the matrix cores
  * sustain for operands with that bit content, which on this part depends on
  * the data (the pipe is power-limited). `type_flag` is an
  * IREE_AMD_UK_FLAG_MMT4D_TYPE_* value with a matrix-core kernel; `operands`
- * holds at least 64 KiB (4 waves x 8 fragments x 64 lanes x up to 32 bytes);
- * `sink`
- * is at least 1 KiB and is normally left untouched; `*out_ops_per_launch`
+ * holds at least 64 KiB (4 waves x up to 16 fragments x 64 lanes x 16 bytes, or
+ * 8 fragments of 32 bytes for fp8); `sink` is at least 1 KiB and is normally left untouched; `*out_ops_per_launch`
  * receives the multiply-add operation count (2 per MAC) of one launch. */
 IREE_AMD_UK_EXPORT int iree_amd_uk_mfma_probe(uint32_t type_flag,
                                               const void* operands,

@@ -1,6 +1,7 @@
-// Measurement aid: the MFMA issue pattern of the mmt4d kernel (a wave holds 4
-// A fragments and 4 B fragments and updates its 4 x 4 accumulator blocks once
-// per K-step) with ALL data movement removed: the fragments are loaded from a
+// Measurement aid: the MFMA issue pattern of the mmt4d kernel (a wave holds the
+// A and B fragments of its 128 x 128 tile and updates all accumulator blocks
+// once per K-step, with the instruction shape the kernel uses for the type)
+// with ALL data movement removed: the fragments are loaded from a
 // small buffer once and stay in registers. What it sustains is the ceiling of
 // the matrix cores for operands with that bit pattern: on MI355X the rate
 // depends strongly on the data (constant operands reach the nominal peak,
@@ -17,34 +18,36 @@ __global__ __launch_bounds__(256) void mfma_probe_kernel(const char* operands, i
   typedef typename Cfg::acc_t acc_t;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   constexpr int kFragBytes = sizeof(frag_t);
-  // 8 fragments per wave: operands[(wave * 8 + f) * 64 + lane]
-  frag_t a[4], b[4];
+  // a wave's tile is 128 x 128: W x W blocks of the instruction's shape
+  constexpr int W = 128 / Cfg::kRows, kAccRegs = Cfg::kRows * Cfg::kRows / 64;
+  // 2 W fragments per wave: operands[(wave * 2 W + f) * 64 + lane]
+  frag_t a[W], b[W];
 #pragma unroll
-  for (int f = 0; f < 4; ++f) {
-    a[f] = *(const frag_t*)(operands + ((size_t)(wave * 8 + f) * 64 + lane) * kFragBytes);
-    b[f] = *(const frag_t*)(operands + ((size_t)(wave * 8 + 4 + f) * 64 + lane) * kFragBytes);
+  for (int f = 0; f < W; ++f) {
+    a[f] = *(const frag_t*)(operands + ((size_t)(wave * 2 * W + f) * 64 + lane) * kFragBytes);
+    b[f] = *(const frag_t*)(operands + ((size_t)(wave * 2 * W + W + f) * 64 + lane) * kFragBytes);
   }
-  acc_t acc[4][4];
+  acc_t acc[W][W];
 #pragma unroll
-  for (int x = 0; x < 4; ++x)
+  for (int x = 0; x < W; ++x)
 #pragma unroll
-    for (int y = 0; y < 4; ++y)
+    for (int y = 0; y < W; ++y)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) acc[x][y][v] = 0;
+      for (int v = 0; v < kAccRegs; ++v) acc[x][y][v] = 0;
   for (int64_t it = 0; it < iters; ++it) {
 #pragma unroll
-    for (int x = 0; x < 4; ++x)
+    for (int x = 0; x < W; ++x)
 #pragma unroll
-      for (int y = 0; y < 4; ++y) acc[x][y] = Cfg::mfma(a[x], b[y], acc[x][y]);
+      for (int y = 0; y < W; ++y) acc[x][y] = Cfg::mfma(a[x], b[y], acc[x][y]);
   }
   // keep the result alive without storing it in the common case
   float s = 0.f;
 #pragma unroll
-  for (int x = 0; x < 4; ++x)
+  for (int x = 0; x < W; ++x)
 #pragma unroll
-    for (int y = 0; y < 4; ++y)
+    for (int y = 0; y < W; ++y)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) s += (float)acc[x][y][v];
+      for (int v = 0; v < kAccRegs; ++v) s += (float)acc[x][y][v];
   if (s == 12345.678f) sink[threadIdx.x] = s;
 }
 
@@ -63,14 +66,16 @@ int launch_mfma_probe(uint32_t type_flag, const void* operands, int64_t iters, v
   int st;
   int64_t k;
   switch (type_flag & IREE_AMD_UK_FLAG_MMT4D_TYPE_MASK) {
-    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F32: st = launch<F16Cfg>(operands, iters, sink, blocks, s); k = 16; break;
-    case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16F32: st = launch<BF16Cfg>(operands, iters, sink, blocks, s); k = 16; break;
+    // (the shapes the mmt4d kernel uses for each type)
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F32: st = launch<F16Cfg16>(operands, iters, sink, blocks, s); k = 32; break;
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16F32: st = launch<BF16Cfg16>(operands, iters, sink, blocks, s); k = 32; break;
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32: st = launch<S8Cfg>(operands, iters, sink, blocks, s); k = 32; break;
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_F8E4M3F8E4M3F32: st = launch<F8Cfg>(operands, iters, sink, blocks, s); k = 64; break;
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_F32F32F32: st = launch<F32Cfg>(operands, iters, sink, blocks, s); k = 8; break;
     default: return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "mfma_probe: type has no MFMA kernel");
   }
-  if (out_ops_per_launch) *out_ops_per_launch = (int64_t)blocks * 4 * iters * 16 * 2 * 32 * 32 * k;
+  // per wave and iteration: a 128 x 128 x k update
+  if (out_ops_per_launch) *out_ops_per_launch = (int64_t)blocks * 4 * iters * 2 * 128 * 128 * k;
   return st;
 }
 
