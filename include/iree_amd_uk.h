@@ -443,7 +443,7 @@ IREE_AMD_UK_EXPORT int iree_amd_uk_mmt4d_unpack(
  * ACCUMULATE / SKIP_INTERMEDIATE_ROUNDINGS. out_scale as for
  * iree_amd_uk_mmt4d_unpack. Requirements (IREE_AMD_UK_STATUS_UNIMPLEMENTED
  * otherwise; use the three-call sequence then): K a multiple of the
- * matrix-core K extent (16 for f16/bf16, 32 for i8, 8 for f32, 64 for fp8),
+ * matrix-core K extent (32 for f16/bf16 and i8, 8 for f32, 64 for fp8),
  * K0 as served by iree_amd_uk_mmt4d, 16-byte aligned lhs rows and rhs tiles.
  * Bit-identical to pack + mmt4d + unpack. */
 IREE_AMD_UK_EXPORT int iree_amd_uk_matmul_packed_rhs(

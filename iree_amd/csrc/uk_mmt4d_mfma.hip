@@ -7,38 +7,45 @@
 // tile row:
 //
 //   type            MFMA                         K per MFMA   K0 served
-//   f16 x f16 -> f32  v_mfma_f32_32x32x16_f16        16         8, 16
-//   bf16 x bf16 -> f32 v_mfma_f32_32x32x16_bf16      16         8, 16
+//   f16 x f16 -> f32  v_mfma_f32_16x16x32_f16        32         8, 16
+//   bf16 x bf16 -> f32 v_mfma_f32_16x16x32_bf16      32         8, 16
 //   s8 x s8 -> s32    v_mfma_i32_32x32x32_i8         32         16, 32
 //   f32 x f32 -> f32  4 x v_mfma_f32_32x32x2_f32      8          4, 8
 //   f16 -> f16, bf16 -> bf16 (intermediate roundings skipped): as -> f32, rounded on store
 //   e4m3 x e4m3 -> f32 v_mfma_scale_f32_32x32x64_f8f6f4  64         16
+//   (f16 / bf16 with the fused SiLU epilogue: v_mfma_f32_32x32x16_*, K 16)
 //
-// With K0 = half the MFMA's K extent, two consecutive K tiles of one outer row
-// ARE one MFMA operand in register order (lane l <-> bytes [16 l, 16 l + 16)),
-// so a 64-lane 128-bit load moves a 1 KiB operand block with perfectly linear
-// addressing. With K0 = the full extent the same 1 KiB holds one tile and the
-// lane <-> address map is (l % 32) * 32 + (l / 32) * 16. The fp8 instruction
-// takes 32 bytes per lane (k = 32 (l / 32) .. + 32 of row l % 32): four K0 = 16
-// tiles make one operand block of 2 KiB, moved as two 1 KiB halves in which
-// lanes 0-31 fetch one whole tile and lanes 32-63 the tile two further on, so
-// each half is again in lane order in LDS. (OCP e4m3fn, unit block scales.)
+// An operand fragment is always 1 KiB: R rows (the instruction's block, 32 or
+// 16) of 64 / R chunks of 16 bytes; lane l feeds row l % R, chunk l / R. A
+// packed tile row holds K0 elements, i.e. one, two or four of those chunks'
+// worth is spread over as many consecutive K tiles of the outer row, and the
+// per-lane global offset follows from that (packed_lane_off below); the 64-lane
+// 128-bit load then lands the fragment in LDS in lane order, so LDS reads are
+// linear whatever K0 is. With K0 = the 16 bytes of one chunk (what the
+// tile-size query answers for the 32-row shapes) the global addresses are
+// linear too. The fp8 instruction takes 32 bytes per lane (k = 32 (l / 32) ..
+// + 32 of row l % 32): four K0 = 16 tiles make one operand block of 2 KiB,
+// moved as two 1 KiB halves in which lanes 0-31 fetch one whole tile and lanes
+// 32-63 the tile two further on. (OCP e4m3fn, unit block scales.)
 //
 // Kernel shape: a workgroup of 2 x kWavesN waves (4 by default) owns a macro
-// tile of (2*WM) x (kWavesN*WN) outer tiles; each wave accumulates WM x WN blocks
-// of 32x32 in registers. The K loop moves operand blocks global -> LDS with
-// direct-to-LDS 128-bit buffer loads (no register staging) into a ring of
-// K-step slots, several K-steps ahead of the MFMAs; operand fragments are read
-// from LDS one K-step ahead and every memory instruction is issued in the
-// shadow of an MFMA. Workgroup ids are
-// remapped so that the 8 XCDs (which receive consecutive workgroup ids
-// round-robin) each work on a compact block of macro tiles and reuse operand
-// panels in their own L2.
+// tile of (2*WM) x (kWavesN*WN) blocks of R x R; each wave accumulates WM x WN
+// blocks in registers (a 128 x 128 tile for the large variant). The K loop
+// moves operand fragments global -> LDS with direct-to-LDS 128-bit buffer loads
+// (no register staging) into a ring of K-step slots, several K-steps ahead of
+// the MFMAs; fragments are read from LDS one K-step ahead and every memory
+// instruction is issued in the shadow of an MFMA. Workgroup ids are remapped so
+// that the 8 XCDs (which receive consecutive workgroup ids round-robin) each
+// work on a compact block of macro tiles and reuse operand panels in their own
+// L2.
 //
-// Measured bound that matters more than the nominal peak: with N(0,1) f16
-// operands a register-only MFMA loop sustains 1.45-1.7 PFLOP/s on MI355X
-// (2.2-2.4 with all-zero operands): the matrix pipe is power-limited by operand
-// toggling and the clock drops, so every stall cycle costs more time as well.
+// Measured bound that matters more than the nominal peak: the matrix pipe is
+// power-limited by operand toggling. With N(0,1) f16 operands a register-only
+// loop of v_mfma_f32_32x32x16_f16 sustains 1.45-1.7 PFLOP/s on MI355X and one
+// of v_mfma_f32_16x16x32_f16 1.8-1.9 (both 2.3-2.4 with all-zero operands),
+// which is why f16 / bf16 run on the 16-row shape; for i8 and fp8 the 32-row
+// shapes are the faster ones. The clock drops under that limit, so every stall
+// cycle costs more time as well.
 #include "uk_common.h"
 #include "uk_fp8.h"
 #include "uk_mfma_cfg.h"
