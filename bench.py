@@ -39,7 +39,7 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # x 1.0): 212 MiB read (each of the 8 XCD L2s fetches its own operand panels;
 # most of it is served by the 256 MiB memory-side cache; 196-212 MiB from run
 # to run) + 68 MiB written.
-MEASURED_TRAFFIC_BYTES = {"mmt4d_f16_4096": 293.8e6}
+MEASURED_TRAFFIC_BYTES = {"mmt4d_f16_4096": 281.9e6}
 
 
 # After an idle spell (or CPU-only work) the GPU's power management needs about
