@@ -624,17 +624,16 @@ int launch_cfg(const MfmaArgs& a, hipStream_t s) {
   constexpr bool kShallow = Cfg::kSub == 2 && !kSiluMul;
   struct Variant { int wm, wn, occ; double eff_alone, eff_full; };
   // (16-row shapes: 256x128 measured 115 us against 104 for 256x256 at 4096^3)
-  constexpr double kEffAlone = kShallow ? 0.85 : S == 2 ? 0.86 : 0.9;
-  constexpr double kEffFull = kShallow ? 0.82 : S == 2 ? 0.9 : 0.94;
+  constexpr double kEffAlone = kSiluMul ? 1.0 : kShallow ? 0.85 : S == 2 ? 0.86 : 0.9;
+  constexpr double kEffFull = kSiluMul ? 1.05 : kShallow ? 0.82 : S == 2 ? 0.9 : 0.94;
   static const Variant variants[4] = {{4, 4, 1, 1.0, 1.0},
                                       {4, 2, 2, kEffAlone, kEffFull},
                                       {2, 4, 2, kEffAlone, kEffFull},
                                       {2, 2, 2, 0.7, 0.75}};
-  int best = 0;
-  double best_cost = 0;
-  for (int v = 0; v < 4; ++v) {
+  // cost of variant v on an M x N (outer tiles) problem
+  auto cost_of = [&](int v, int64_t M, int64_t N) -> double {
     const Variant& t = variants[v];
-    const int64_t tiles = (int64_t)ceil_div(a.M, 2 * t.wm) * ceil_div(a.N, 2 * t.wn);
+    const int64_t tiles = ceil_div(M, (int64_t)2 * t.wm) * ceil_div(N, (int64_t)2 * t.wn);
     const int64_t slots = (int64_t)t.occ * cus;
     const double work = t.wm * t.wn;
     double cost = (double)(tiles / slots) * t.occ * work / t.eff_full;
@@ -643,14 +642,65 @@ int launch_cfg(const MfmaArgs& a, hipStream_t s) {
       const int resident = (int)ceil_div(rest, (int64_t)cus);   // workgroups sharing a compute unit
       cost += resident * work / (resident == t.occ ? t.eff_full : t.eff_alone);
     }
-    if (v == 0 || cost < best_cost * 0.999) { best = v; best_cost = cost; }
+    return cost;
+  };
+  auto pick = [&](int64_t M, int64_t N, double* out_cost) -> int {
+    int best = 0;
+    double best_cost = 0;
+    for (int v = 0; v < 4; ++v) {
+      const double cost = cost_of(v, M, N);
+      if (v == 0 || cost < best_cost * 0.999) { best = v; best_cost = cost; }
+    }
+    *out_cost = best_cost;
+    return best;
+  };
+  auto launch = [&](int v, const MfmaArgs& b) -> int {
+    switch (v) {
+      case 0: return launch_variant<Cfg, 4 * S, 4 * S, kWide ? 5 : 8, kWide ? 1 : 2, 1, kSiluMul>(b, s);
+      case 1: return launch_variant<Cfg, 4 * S, 2 * S, kWide ? 3 : 6, kWide ? 1 : 2, 2, kSiluMul>(b, s);
+      case 2: return launch_variant<Cfg, 2 * S, 4 * S, kWide ? 3 : 6, kWide ? 1 : 2, 2, kSiluMul>(b, s);
+      default: return launch_variant<Cfg, 2 * S, 2 * S, S == 2 ? 4 : 8, S == 2 ? 1 : 2, 1, kSiluMul>(b, s);
+    }
+  };
+  double best_cost = 0;
+  const int best = pick(a.M, a.N, &best_cost);
+  // A last round that fills only part of the device costs a whole round. When
+  // the large tile leaves such a round, the outer columns can be split: whole
+  // rounds of 256x256 tiles first, the remaining columns as a second launch
+  // with whatever suits them (usually tiles of half the size, one per compute
+  // unit). Taken when the model predicts at least 5 % (a launch costs a few
+  // microseconds, so only for long K).
+  const int64_t rows0 = ceil_div((int64_t)a.M, (int64_t)8);   // macro-tile rows of the large tile
+  const int64_t cols0 = ceil_div((int64_t)a.N, (int64_t)8);
+  const int64_t rounds0 = rows0 * cols0 / cus;
+  if (rounds0 >= 1 && (int64_t)a.ksteps * Cfg::kMfmaK * Cfg::kElemBytes >= 2048) {
+    const int64_t cols_first = rounds0 * cus / rows0;            // macro columns in whole rounds
+    const int64_t n_first = cols_first * 8;                       // outer tile columns
+    if (cols_first >= 1 && n_first < a.N) {
+      double rest_cost = 0;
+      const int rest_v = pick(a.M, a.N - n_first, &rest_cost);
+      const double split_cost = cost_of(0, a.M, n_first) + rest_cost;
+      if (split_cost < best_cost * 0.95) {
+        MfmaArgs first = a, rest = a;
+        first.N = (int)n_first;
+        rest.N = a.N - (int)n_first;
+        rest.rhs = a.rhs + n_first * a.rhs_stride_bytes;
+        if (kSiluMul) {
+          rest.out = a.out + (n_first / 2) * 1024;               // bytes: one e4m3 tile pair per two columns
+        } else if (a.row_major_out) {
+          rest.out = a.out + n_first * 32 * (int64_t)sizeof(typename Cfg::out_t);
+          first.out_cols = a.out_cols < n_first * 32 ? a.out_cols : (int)(n_first * 32);
+          rest.out_cols = a.out_cols - (int)(n_first * 32);
+        } else {
+          rest.out = a.out + n_first * 1024 * (int64_t)sizeof(typename Cfg::out_t);
+        }
+        const int st = launch(0, first);
+        if (st) return st;
+        return launch(rest_v, rest);
+      }
+    }
   }
-  switch (best) {
-    case 0: return launch_variant<Cfg, 4 * S, 4 * S, kWide ? 5 : 8, kWide ? 1 : 2, 1, kSiluMul>(a, s);
-    case 1: return launch_variant<Cfg, 4 * S, 2 * S, kWide ? 3 : 6, kWide ? 1 : 2, 2, kSiluMul>(a, s);
-    case 2: return launch_variant<Cfg, 2 * S, 4 * S, kWide ? 3 : 6, kWide ? 1 : 2, 2, kSiluMul>(a, s);
-    default: return launch_variant<Cfg, 2 * S, 2 * S, S == 2 ? 4 : 8, S == 2 ? 1 : 2, 1, kSiluMul>(a, s);
-  }
+  return launch(best, a);
 }
 
 // mfma_k: K extent of the instruction the call runs on. f16 / bf16 use the
