@@ -665,34 +665,52 @@ int launch_cfg(const MfmaArgs& a, hipStream_t s) {
   double best_cost = 0;
   const int best = pick(a.M, a.N, &best_cost);
   // A last round that fills only part of the device costs a whole round. When
-  // the large tile leaves such a round, the outer columns can be split: whole
-  // rounds of 256x256 tiles first, the remaining columns as a second launch
-  // with whatever suits them (usually tiles of half the size, one per compute
-  // unit). Taken when the model predicts at least 5 % (a launch costs a few
+  // the large tile leaves such a round, the longer outer dimension is split:
+  // whole rounds of 256x256 tiles first, the remaining rows or columns as a
+  // second launch with whatever suits them (usually tiles of half the size, one
+  // per compute unit). Taken when the model predicts at least 5 % (a launch costs a few
   // microseconds, so only for long K).
   const int64_t rows0 = ceil_div((int64_t)a.M, (int64_t)8);   // macro-tile rows of the large tile
   const int64_t cols0 = ceil_div((int64_t)a.N, (int64_t)8);
   const int64_t rounds0 = rows0 * cols0 / cus;
   if (rounds0 >= 1 && (int64_t)a.ksteps * Cfg::kMfmaK * Cfg::kElemBytes >= 2048) {
-    const int64_t cols_first = rounds0 * cus / rows0;            // macro columns in whole rounds
-    const int64_t n_first = cols_first * 8;                       // outer tile columns
-    if (cols_first >= 1 && n_first < a.N) {
+    // split the longer dimension: `across` macro tiles lie across it
+    const bool by_cols = cols0 >= rows0;
+    const int64_t across = by_cols ? rows0 : cols0;
+    const int64_t along_first = rounds0 * cus / across;          // macro tiles along it in whole rounds
+    const int64_t t_first = along_first * 8;                      // outer tiles
+    const int64_t t_all = by_cols ? a.N : a.M;
+    if (along_first >= 1 && t_first < t_all) {
       double rest_cost = 0;
-      const int rest_v = pick(a.M, a.N - n_first, &rest_cost);
-      const double split_cost = cost_of(0, a.M, n_first) + rest_cost;
+      const int rest_v = by_cols ? pick(a.M, a.N - t_first, &rest_cost) : pick(a.M - t_first, a.N, &rest_cost);
+      const double split_cost = (by_cols ? cost_of(0, a.M, t_first) : cost_of(0, t_first, a.N)) + rest_cost;
       if (split_cost < best_cost * 0.95) {
         MfmaArgs first = a, rest = a;
-        first.N = (int)n_first;
-        rest.N = a.N - (int)n_first;
-        rest.rhs = a.rhs + n_first * a.rhs_stride_bytes;
-        if (kSiluMul) {
-          rest.out = a.out + (n_first / 2) * 1024;               // bytes: one e4m3 tile pair per two columns
-        } else if (a.row_major_out) {
-          rest.out = a.out + n_first * 32 * (int64_t)sizeof(typename Cfg::out_t);
-          first.out_cols = a.out_cols < n_first * 32 ? a.out_cols : (int)(n_first * 32);
-          rest.out_cols = a.out_cols - (int)(n_first * 32);
+        const int64_t out_elem = kSiluMul ? 1 : (int64_t)sizeof(typename Cfg::out_t);
+        if (by_cols) {
+          first.N = (int)t_first;
+          rest.N = a.N - (int)t_first;
+          rest.rhs = a.rhs + t_first * a.rhs_stride_bytes;
+          if (kSiluMul) {
+            rest.out = a.out + (t_first / 2) * 1024;             // one e4m3 tile pair per two columns
+          } else if (a.row_major_out) {
+            rest.out = a.out + t_first * 32 * out_elem;
+            first.out_cols = (int)(t_first * 32);                 // (out_cols > 32 (N - 1) >= 32 t_first)
+            rest.out_cols = a.out_cols - (int)(t_first * 32);
+          } else {
+            rest.out = a.out + t_first * 1024 * out_elem;
+          }
         } else {
-          rest.out = a.out + n_first * 1024 * (int64_t)sizeof(typename Cfg::out_t);
+          first.M = (int)t_first;
+          rest.M = a.M - (int)t_first;
+          // (tiled results and the SiLU form: out_stride_bytes is the pitch of an
+          // outer row; row-major ones: of a matrix row)
+          rest.out = a.out + t_first * (a.row_major_out ? 32 : 1) * a.out_stride_bytes;
+          rest.lhs = a.lhs + t_first * (a.lhs_row_major ? 32 : 1) * a.lhs_stride_bytes;
+          if (a.row_major_out) {
+            first.out_rows = (int)(t_first * 32);
+            rest.out_rows = a.out_rows - (int)(t_first * 32);
+          }
         }
         const int st = launch(0, first);
         if (st) return st;

@@ -516,3 +516,33 @@ def test_matmul_packed_rhs_rejects_what_it_cannot_serve(uk, cuda):
         with pytest.raises(uk.UkError) as e:
             uk.matmul_packed_rhs(a, a, out, **{**ok, **bad})
         assert e.value.status == status, (bad, e.value.status)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,N", [(9216, 2048), (2048, 9216)])
+def test_i8_shapes_that_split_into_two_launches(uk, cuda, M, N):
+    """288 large tiles on 256 compute units: the launcher runs one whole round of
+    256x256 tiles and a second launch for the remaining rows (or columns).
+    Tiled and row-major results, and the row-major left-hand side, against an
+    exact float64 product (|sum| < 2^53)."""
+    import torch
+    K = 2048
+    A = synth.uniform_int8(1, M * K).reshape(M, K)
+    B = synth.uniform_int8(2, N * K).reshape(N, K)          # B^T, row-major [N][K]
+    want = (A.astype(np.float64) @ B.astype(np.float64).T).astype(np.int64)
+    a_d, b_d = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda()
+    M1, N1, K1 = M // 32, N // 32, K // 16
+    lhs = torch.empty(M * K, dtype=torch.int8, device=cuda)
+    rhs = torch.empty(N * K, dtype=torch.int8, device=cuda)
+    uk.pack(a_d, lhs, M, K, M1, K1, 32, 16, 0, F.PACK_TYPE_I8I8)
+    uk.pack(b_d, rhs, N, K, N1, K1, 32, 16, 0, F.PACK_TYPE_I8I8)
+    tiled = torch.empty(M * N, dtype=torch.int32, device=cuda)
+    uk.mmt4d(lhs, rhs, tiled, M1, N1, K1, 32, 32, 16, F.MMT4D_TYPE_S8S8S32)
+    got = tiled.cpu().numpy().reshape(M1, N1, 32, 32).transpose(0, 2, 1, 3).reshape(M, N)
+    assert np.array_equal(got, want)
+    for fn in (lambda c: uk.mmt4d_unpack(lhs, rhs, c, M, N, M1, N1, K1, 16, F.MMT4D_TYPE_S8S8S32),
+               lambda c: uk.matmul_packed_rhs(a_d, rhs, c, M, N, K, 16, F.MMT4D_TYPE_S8S8S32)):
+        c = torch.full((M * N,), -1, dtype=torch.int32, device=cuda)
+        fn(c)
+        torch.cuda.synchronize()
+        assert np.array_equal(c.cpu().numpy().reshape(M, N), want)
