@@ -194,7 +194,7 @@ __global__ __launch_bounds__(128 * kWavesN, kOcc) void mmt4d_mfma_kernel(MfmaArg
   // them (from the front) get fragment reads slipped in behind them: the last
   // third or so stays free so that the reads have landed when the step ends.
   constexpr int kMfmaAll = WM * WN, kMfmaRest = (WM - 1) * WN;
-  constexpr int kTail = kPerTile * kPerTile;    // (a 16x16 MFMA is half as long)
+  constexpr int kTail = kPerTile * kPerTile;    // (16-row shapes: 4x the MFMAs per K-step, each half as long)
   constexpr int kReadAll = kMfmaAll - (kMfmaAll >= 8 * kTail ? 6 * kTail : kMfmaAll / 2);
   constexpr int kReadRest = kMfmaRest - (kMfmaRest >= 8 * kTail ? 4 * kTail : kMfmaRest / 2);
   static_assert(kAhead >= kSync, "ring must hold two sync groups");
