@@ -301,14 +301,17 @@ __global__ __launch_bounds__(128 * kWavesN, kOcc) void mmt4d_mfma_kernel(MfmaArg
 #pragma unroll
         for (int v = 0; v < kAccRegs; ++v) acc[x][y][v] = t[acc_row(v) * 32 + acc_col];
       }
-  } else {
+  }
+  // (without the accumulate flag the accumulators are cleared after the first
+  // loads have been issued, in the shadow of their latency)
+  auto clear_acc = [&]() {
 #pragma unroll
     for (int x = 0; x < WM; ++x)
 #pragma unroll
       for (int y = 0; y < WN; ++y)
 #pragma unroll
         for (int v = 0; v < kAccRegs; ++v) acc[x][y][v] = 0;
-  }
+  };
 
   // Load `d` (of kLoadsPerStep) of this wave's share of K-step `ks` into ring
   // slot `slot`: its rows of A first, then its rows of B, kSub pieces each.
@@ -386,6 +389,7 @@ __global__ __launch_bounds__(128 * kWavesN, kOcc) void mmt4d_mfma_kernel(MfmaArg
     int read_slot = 0;                                // slot of K-step `done`
 #pragma unroll 1
     for (int ks = 0; ks < kPro; ++ks) issue_step(ks, ks);
+    if (!a.accumulate) clear_acc();
     wait_vmcnt<(kPro - kSync) * kLoadsPerStep>();  // the first kSync K-steps have landed
     __builtin_amdgcn_s_barrier();                  // (bare, as in the loop below)
     read_frags(0, fa[0], fb[0]);
@@ -449,6 +453,7 @@ __global__ __launch_bounds__(128 * kWavesN, kOcc) void mmt4d_mfma_kernel(MfmaArg
     // ---- short-K path: everything fits in the ring ------------------------
 #pragma unroll 1
     for (int ks = 0; ks < T; ++ks) issue_step(ks, ks);
+    if (!a.accumulate) clear_acc();
     wait_vmcnt<0>();
     __syncthreads();
 #pragma unroll 1
