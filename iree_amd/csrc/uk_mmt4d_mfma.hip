@@ -1,578 +1,21 @@
-// mmt4d on the gfx950 matrix cores.
+// mmt4d on the gfx950 matrix cores: the host side. Picks the macro tile for a
+// call, launches the kernel of uk_mmt4d_mfma_kernel.h and serves the fused
+// forms (row-major result, row-major left-hand side, SiLU epilogue).
 //
 // Contract: include/iree_amd_uk.h (mirrors iree_uk_mmt4d,
-// runtime/src/iree/builtins/ukernel/mmt4d.h:14-21 of the reference). This file
-// serves the tile shapes the gfx950 tile-size query hands out: M0 = N0 = 32 and
-// a K0 such that one lane's MFMA operand (16 bytes) is one contiguous piece of a
-// tile row:
-//
-//   type            MFMA                         K per MFMA   K0 served
-//   f16 x f16 -> f32  v_mfma_f32_16x16x32_f16        32         8, 16
-//   bf16 x bf16 -> f32 v_mfma_f32_16x16x32_bf16      32         8, 16
-//   s8 x s8 -> s32    v_mfma_i32_32x32x32_i8         32         16, 32
-//   f32 x f32 -> f32  4 x v_mfma_f32_32x32x2_f32      8          4, 8
-//   f16 -> f16, bf16 -> bf16 (intermediate roundings skipped): as -> f32, rounded on store
-//   e4m3 x e4m3 -> f32 v_mfma_scale_f32_32x32x64_f8f6f4  64         16
-//   (f16 / bf16 with the fused SiLU epilogue: v_mfma_f32_32x32x16_*, K 16)
-//
-// An operand fragment is always 1 KiB: R rows (the instruction's block, 32 or
-// 16) of 64 / R chunks of 16 bytes; lane l feeds row l % R, chunk l / R. A
-// packed tile row holds K0 elements, i.e. one, two or four of those chunks'
-// worth is spread over as many consecutive K tiles of the outer row, and the
-// per-lane global offset follows from that (packed_lane_off below); the 64-lane
-// 128-bit load then lands the fragment in LDS in lane order, so LDS reads are
-// linear whatever K0 is. With K0 = the 16 bytes of one chunk (what the
-// tile-size query answers for the 32-row shapes) the global addresses are
-// linear too. The fp8 instruction takes 32 bytes per lane (k = 32 (l / 32) ..
-// + 32 of row l % 32): four K0 = 16 tiles make one operand block of 2 KiB,
-// moved as two 1 KiB halves in which lanes 0-31 fetch one whole tile and lanes
-// 32-63 the tile two further on. (OCP e4m3fn, unit block scales.)
-//
-// Kernel shape: a workgroup of 2 x kWavesN waves (4 by default) owns a macro
-// tile of (2*WM) x (kWavesN*WN) blocks of R x R; each wave accumulates WM x WN
-// blocks in registers (a 128 x 128 tile for the large variant). The K loop
-// moves operand fragments global -> LDS with direct-to-LDS 128-bit buffer loads
-// (no register staging) into a ring of K-step slots, several K-steps ahead of
-// the MFMAs; fragments are read from LDS one K-step ahead and every memory
-// instruction is issued in the shadow of an MFMA. Workgroup ids are remapped so
-// that the 8 XCDs (which receive consecutive workgroup ids round-robin) each
-// work on a compact block of macro tiles and reuse operand panels in their own
-// L2.
-//
-// Measured bound that matters more than the nominal peak: the matrix pipe is
-// power-limited by operand toggling. With N(0,1) f16 operands a register-only
-// loop of v_mfma_f32_32x32x16_f16 sustains 1.45-1.7 PFLOP/s on MI355X and one
-// of v_mfma_f32_16x16x32_f16 1.8-1.9 (both 2.3-2.4 with all-zero operands),
-// which is why f16 / bf16 run on the 16-row shape; for i8 and fp8 the 32-row
-// shapes are the faster ones. The clock drops under that limit, so every stall
-// cycle costs more time as well.
+// runtime/src/iree/builtins/ukernel/mmt4d.h:14-21 of the reference).
 #include "uk_common.h"
-#include "uk_fp8.h"
-#include "uk_mfma_cfg.h"
-
-#include <type_traits>
+#include "uk_mmt4d_mfma_kernel.h"
 
 namespace uk {
 namespace {
 
-constexpr int kPieceBytes = 1024;   // what one 64-lane 128-bit load moves
-
-struct MfmaArgs {
-  const char* lhs;  // offset applied
-  const char* rhs;
-  char* out;
-  int64_t lhs_stride_bytes, rhs_stride_bytes, out_stride_bytes;
-  int M, N;          // outer tile counts
-  int ksteps;        // whole MFMA K-steps = K * K0 / kMfmaK
-  int tail_tiles;    // K tiles left over after them (less than one MFMA's worth)
-  int tiles_m, tiles_n;  // macro-tile grid
-  int accumulate;
-  // row-major result (mmt4d fused with the unpack that would follow it): the
-  // matrix has out_rows x out_cols elements, out_stride_bytes is its row pitch
-  int row_major_out, out_rows, out_cols;
-  // row-major left-hand side (the pack of the LHS fused into the loads): lhs is
-  // the out_rows x K matrix itself, lhs_stride_bytes its row pitch; the block
-  // of (outer row i, K-step ks) is rows 32 i .. 32 i + 31, bytes
-  // lhs_step_bytes * ks .. of each row
-  int lhs_row_major;
-  int k0_div;        // the instruction's K extent / K0: 1, 2 (or 4 for the 16-row shapes)
-  // fused SiLU * up epilogue only: scales of the gate and up accumulators and
-  // the inverse scale of the e4m3 result
-  float gate_scale, up_scale, inv_out_scale;
-  // row-major result of a float type only: factor applied on the store
-  float out_scale;
-};
-
-__device__ __forceinline__ void load_block_to_lds(__amdgpu_buffer_rsrc_t row, uint32_t lane_off,
-                                                  uint32_t block_off, char* lds) {
-  // 64 lanes x 16 bytes -> lds[0..1024) in lane order, from byte
-  // block_off + lane_off of the operand row `row` describes. The row base and
-  // block_off live in scalar registers and lane_off never changes, so a load
-  // costs no per-lane address arithmetic.
-  __builtin_amdgcn_raw_ptr_buffer_load_lds(row, (__attribute__((address_space(3))) void*)lds, 16,
-                                           lane_off, block_off, 0, 0);
-}
-
-// Buffer descriptor of one operand row (its length is checked on the host).
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t row_descriptor(const char* row) {
-  return __builtin_amdgcn_make_buffer_rsrc((void*)row, 0, 0x7FFFFFFF, 0x00020000);
-}
-
-template <int N>
-__device__ __forceinline__ void wait_vmcnt() {
-  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-}
-
-// Share of `n` items that falls to slot `i` of `slots` when they are spread evenly.
-constexpr int share(int n, int slots, int i) { return (i + 1) * n / slots - i * n / slots; }
-
-// Pins the issue order of one basic block to kMfma times {1 MFMA, its share of
-// the kDsr LDS reads, its share of the kVmem vector-memory loads}. A memory
-// instruction issued right behind an MFMA runs in its shadow; spreading them
-// keeps a wave (which issues in order) from queueing behind a burst of loads
-// while the matrix pipe runs dry. The LDS reads go behind the first kDsrMfma
-// MFMAs only: the block that follows waits for the LAST read issued (LDS reads
-// retire in order and the compiler waits for all of them), so the reads must
-// be done while MFMAs of this block are still queued. The LDS reads and the
-// direct-to-LDS loads must appear in the source in this same order: the
-// compiler keeps their relative order (they may alias).
-template <int kMfma, int kDsrMfma, int kDsr, int kVmem, int kInstrPerDsr, int I = 0>
-__device__ __forceinline__ void spread_issue() {
-  if constexpr (I < kMfma) {
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-    if constexpr (I < kDsrMfma) {
-      constexpr int d = share(kDsr, kDsrMfma, I) * kInstrPerDsr;
-      if constexpr (d > 0) __builtin_amdgcn_sched_group_barrier(0x100, d, 0);
-    }
-    constexpr int v = share(kVmem, kMfma, I);
-    if constexpr (v > 0) __builtin_amdgcn_sched_group_barrier(0x020, v, 0);
-    spread_issue<kMfma, kDsrMfma, kDsr, kVmem, kInstrPerDsr, I + 1>();
-  }
-}
-
-// Maps the hardware workgroup id to a macro-tile coordinate. Workgroup ids go
-// round-robin over the 8 XCDs; give XCD x the x-th contiguous slice of the
-// logical tile sequence, and order that sequence in column-panels of `kGroup`
-// macro-tile rows so that a slice is a compact 2-D block.
-__device__ __forceinline__ void tile_coord(int bid, int tiles_m, int tiles_n,
-                                           int* tm, int* tn) {
-  constexpr int kXcds = 8, kGroup = 4;
-  const int total = tiles_m * tiles_n;
-  const int per = total / kXcds, rem = total % kXcds;
-  const int xcd = bid % kXcds, idx = bid / kXcds;
-  const int logical = xcd * per + (xcd < rem ? xcd : rem) + idx;
-  const int group_size = kGroup * tiles_n;
-  const int g = logical / group_size;
-  const int first_m = g * kGroup;
-  const int rows = (tiles_m - first_m) < kGroup ? (tiles_m - first_m) : kGroup;
-  const int in_group = logical - g * group_size;
-  *tm = first_m + in_group % rows;
-  *tn = in_group / rows;
-}
-
-// K-loop organisation. LDS is a ring of kRing slots; slot (ks % kRing) holds
-// K-step ks: the TM blocks of A followed by the TN blocks of B, 1 KiB each, in
-// MFMA lane order. Waves synchronise once every kSync K-steps, at the start of
-// the last K-step of a group: the barrier publishes the next group's data and
-// frees the slots of the group just read. EVERY K-step then has the same
-// memory work, spread evenly behind its MFMAs: the LDS reads of the next
-// K-step's fragments, and this wave's share of the direct-to-LDS loads of the
-// K-step that lies kRing - kSync + 1 ahead (into a slot the last barrier
-// freed). Loads therefore stay in flight for kRing - 2 kSync + 1 K-steps.
 // kOcc: waves per SIMD the register allocation must leave room for (2 = two
 // workgroups of 4 waves resident on one compute unit).
-// kSiluMul: instead of storing the accumulators, treat even outer columns as
-// gate and the following odd ones as up, and store e4m3(silu(gate) * up) as
-// left-hand-side tiles 32x16 of the next matmul (one byte per element).
 template <typename Cfg, int WM, int WN, int kRing, int kSync, int kOcc = 1, bool kSiluMul = false,
           int kWavesN = 2>
 __global__ __launch_bounds__(128 * kWavesN, kOcc) void mmt4d_mfma_kernel(MfmaArgs a) {
-  typedef typename Cfg::frag_t frag_t;
-  typedef typename Cfg::acc_t acc_t;
-  typedef typename Cfg::out_t out_t;
-  constexpr int kWaves = 2 * kWavesN;                // a 2 x kWavesN grid of waves
-  // WM, WN, TM, TN count BLOCKS of R rows (R = 32 or 16: the instruction's
-  // block); an outer tile of 32 rows is kPerTile of them.
-  constexpr int R = Cfg::kRows, kPerTile = 32 / R;
-  constexpr int kAccRegs = R * R / 64;               // accumulator registers of one block
-  constexpr int kChunks = 64 / R;                    // 16-byte K chunks of a fragment row
-  constexpr int TM = 2 * WM, TN = kWavesN * WN;      // blocks per workgroup
-  static_assert(R == 32 || (R == 16 && Cfg::kSub == 1 && !kSiluMul), "unsupported block shape");
-  static_assert(TM % kWaves == 0 && TN % kWaves == 0, "every wave loads whole operand rows");
-  constexpr int kSub = Cfg::kSub;
-  constexpr int kBlockBytes = kSub * kPieceBytes;   // one R-row operand block of one K-step
-  constexpr int kABytes = TM * kBlockBytes;
-  constexpr int kSlotBytes = (TM + TN) * kBlockBytes;
-  constexpr int kAhead = kRing - kSync;
-  constexpr int kARowsPerWave = TM / kWaves, kBRowsPerWave = TN / kWaves;
-  constexpr int kLoadsPerStep = (kARowsPerWave + kBRowsPerWave) * kSub;  // per wave
-  constexpr int kBody = (kSync % 2) ? 2 * kSync : kSync;        // K-steps per unrolled body
-  constexpr int kFrags = WM + WN;               // operand fragments a wave reads per K-step
-  constexpr int kPro = kRing - kSync + 1;       // K-steps loaded before the loop starts
-  // MFMAs of a whole K-step / of the part behind a barrier, and how many of
-  // them (from the front) get fragment reads slipped in behind them: the last
-  // third or so stays free so that the reads have landed when the step ends.
-  constexpr int kMfmaAll = WM * WN, kMfmaRest = (WM - 1) * WN;
-  constexpr int kTail = kPerTile * kPerTile;    // (16-row shapes: 4x the MFMAs per K-step, each half as long)
-  constexpr int kReadAll = kMfmaAll - (kMfmaAll >= 8 * kTail ? 6 * kTail : kMfmaAll / 2);
-  constexpr int kReadRest = kMfmaRest - (kMfmaRest >= 8 * kTail ? 4 * kTail : kMfmaRest / 2);
-  static_assert(kAhead >= kSync, "ring must hold two sync groups");
-  static_assert(kPro >= kBody - 1, "the loop's remainder must already be in the ring");
-  static_assert((kPro - kSync) * kLoadsPerStep < 64, "too many loads in flight for vmcnt");
-  extern __shared__ __attribute__((aligned(1024))) char lds[];
-
-  const int lane = threadIdx.x & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int wm = wave / kWavesN, wn = wave % kWavesN;
-  int tm, tn;
-  tile_coord(blockIdx.x, a.tiles_m, a.tiles_n, &tm, &tn);
-  const int i_base = tm * TM, j_base = tn * TN;
-  const int T = a.ksteps;
-
-  // Per-lane byte offset of a fragment inside the K-step of its outer row in
-  // global memory. A lane feeds the instruction row l % R, 16-byte K chunk
-  // l / R; a packed tile holds `cpt` chunks per row (K0 = the instruction's K
-  // extent / k0_div), so chunk c lies in tile c / cpt at row pitch 16 cpt.
-  // `sub` selects the block of R rows inside the 32-row tile. (fp8: two pieces
-  // per lane, the second one 512-byte tile further.)
-  const int frag_row = lane % R, frag_chunk = lane / R;
-  const int cpt = kChunks / a.k0_div;
-  auto packed_lane_off = [&](int sub) -> uint32_t {
-    if constexpr (kSub == 2) return (lane >> 5) * 1024 + (lane & 31) * 16;
-    return (uint32_t)((frag_chunk / cpt) * 512 * cpt + (sub * R + frag_row) * 16 * cpt +
-                      (frag_chunk % cpt) * 16);
-  };
-  constexpr int kPieceStride = 512;
-  constexpr int kStepBytes = kPerTile * kBlockBytes;   // of one outer row of packed tiles
-
-  // Rows this wave copies: its share of the TM rows of A and TN of B. Out-of-range
-  // rows are clamped to the last valid one (loaded, never stored).
-  __amdgpu_buffer_rsrc_t a_src[kARowsPerWave], b_src[kBRowsPerWave];
-  // Left-hand side: per-lane offset inside a row block, bytes between K-steps
-  // and between the two pieces of a wide block. Packed: as the right-hand side.
-  // Row-major: lane l reads row l % 32 (clamped to the last matrix row), the
-  // 16 * kSub bytes of half l / 32 of the K-step: the same bytes in the same
-  // lane order, so LDS and everything behind it are unchanged.
-  uint32_t a_lane_off[kARowsPerWave], b_lane_off[kBRowsPerWave];
-  const uint32_t a_step_bytes = a.lhs_row_major ? kChunks * 16 * kSub : kStepBytes;
-  const uint32_t a_piece_stride = a.lhs_row_major ? 16 : kPieceStride;
-#pragma unroll
-  for (int r = 0; r < kARowsPerWave; ++r) {
-    const int blk = i_base + wave * kARowsPerWave + r;
-    int i = blk / kPerTile;
-    const int sub = blk % kPerTile;
-    i = i < a.M ? i : a.M - 1;
-    if (a.lhs_row_major) {
-      int row = i * 32 + sub * R + frag_row;
-      row = row < a.out_rows ? row : a.out_rows - 1;
-      a_src[r] = row_descriptor(a.lhs);
-      a_lane_off[r] = (uint32_t)row * (uint32_t)a.lhs_stride_bytes + frag_chunk * 16 * kSub;
-    } else {
-      a_src[r] = row_descriptor(a.lhs + (int64_t)i * a.lhs_stride_bytes);
-      a_lane_off[r] = packed_lane_off(sub);
-    }
-  }
-#pragma unroll
-  for (int r = 0; r < kBRowsPerWave; ++r) {
-    const int blk = j_base + wave * kBRowsPerWave + r;
-    int j = blk / kPerTile;
-    j = j < a.N ? j : a.N - 1;
-    b_src[r] = row_descriptor(a.rhs + (int64_t)j * a.rhs_stride_bytes);
-    b_lane_off[r] = packed_lane_off(blk % kPerTile);
-  }
-  // Accumulator element v of this lane: row and column inside its block
-  // (32x32: register v of lane l is row 8 (v / 4) + 4 (l / 32) + v % 4, column
-  // l % 32; 16x16: row 4 (l / 16) + v, column l % 16).
-  auto acc_row = [&](int v) -> int {
-    return R == 32 ? 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3) : 4 * (lane >> 4) + v;
-  };
-  const int acc_col = lane % R;
-
-  acc_t acc[WM][WN];
-  if (a.accumulate && a.row_major_out) {
-    // (rows and columns past the matrix edge are read from the last valid
-    // one: their accumulators are never stored)
-#pragma unroll
-    for (int x = 0; x < WM; ++x)
-#pragma unroll
-      for (int y = 0; y < WN; ++y) {
-        int col = (j_base + wn * WN + y) * R + acc_col;
-        col = col < a.out_cols ? col : a.out_cols - 1;
-        const int row0 = (i_base + wm * WM + x) * R;
-#pragma unroll
-        for (int v = 0; v < kAccRegs; ++v) {
-          int row = row0 + acc_row(v);
-          row = row < a.out_rows ? row : a.out_rows - 1;
-          acc[x][y][v] = *((const out_t*)(a.out + (int64_t)row * a.out_stride_bytes) + col);
-        }
-      }
-  } else if (a.accumulate) {
-#pragma unroll
-    for (int x = 0; x < WM; ++x)
-#pragma unroll
-      for (int y = 0; y < WN; ++y) {
-        const int bi = i_base + wm * WM + x, bj = j_base + wn * WN + y;
-        int i = bi / kPerTile, j = bj / kPerTile;
-        i = i < a.M ? i : a.M - 1;
-        j = j < a.N ? j : a.N - 1;
-        const out_t* t = (const out_t*)(a.out + (int64_t)i * a.out_stride_bytes) + (int64_t)j * 1024 +
-                         (bi % kPerTile) * R * 32 + (bj % kPerTile) * R;
-#pragma unroll
-        for (int v = 0; v < kAccRegs; ++v) acc[x][y][v] = t[acc_row(v) * 32 + acc_col];
-      }
-  }
-  // (without the accumulate flag the accumulators are cleared after the first
-  // loads have been issued, in the shadow of their latency)
-  auto clear_acc = [&]() {
-#pragma unroll
-    for (int x = 0; x < WM; ++x)
-#pragma unroll
-      for (int y = 0; y < WN; ++y)
-#pragma unroll
-        for (int v = 0; v < kAccRegs; ++v) acc[x][y][v] = 0;
-  };
-
-  // Load `d` (of kLoadsPerStep) of this wave's share of K-step `ks` into ring
-  // slot `slot`: its rows of A first, then its rows of B, kSub pieces each.
-  auto issue_one = [&](int ks, int slot, int d) {
-    char* base = lds + slot * kSlotBytes;
-    const int r = d / kSub, j = d % kSub;
-    if (r < kARowsPerWave) {
-      load_block_to_lds(a_src[r], a_lane_off[r], (uint32_t)ks * a_step_bytes + j * a_piece_stride,
-                        base + (wave * kARowsPerWave + r) * kBlockBytes + j * kPieceBytes);
-    } else {
-      const int rb = r - kARowsPerWave;
-      load_block_to_lds(b_src[rb], b_lane_off[rb], (uint32_t)ks * kStepBytes + j * kPieceStride,
-                        base + kABytes + (wave * kBRowsPerWave + rb) * kBlockBytes + j * kPieceBytes);
-    }
-  };
-  auto issue_step = [&](int ks, int slot) {
-#pragma unroll
-    for (int d = 0; d < kLoadsPerStep; ++d) issue_one(ks, slot, d);
-  };
-  auto read_frag = [&](const char* p) -> frag_t {
-    if constexpr (kSub == 1) {
-      return *(const frag_t*)p;
-    } else {
-      const int4v lo = *(const int4v*)p, hi = *(const int4v*)(p + kPieceBytes);
-      return frag_t{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-    }
-  };
-  // Fragment `r` (of kFrags) of this wave for the K-step in `slot`: its WN
-  // blocks of B, then its WM blocks of A. The MFMAs run over A blocks in the
-  // outer loop, so the fragments read last (A blocks 1..) are needed last.
-  auto read_one = [&](int slot, int r, frag_t (&fa)[WM], frag_t (&fb)[WN]) {
-    const char* s0 = lds + slot * kSlotBytes + lane * 16;
-    if (r < WN) fb[r] = read_frag(s0 + kABytes + (wn * WN + r) * kBlockBytes);
-    else fa[r - WN] = read_frag(s0 + (wm * WM + r - WN) * kBlockBytes);
-  };
-  auto read_frags = [&](int slot, frag_t (&fa)[WM], frag_t (&fb)[WN]) {
-#pragma unroll
-    for (int r = 0; r < kFrags; ++r) read_one(slot, r, fa, fb);
-  };
-  // The memory work of one K-step, in the order spread_issue<nM, nR, ...> pins
-  // it behind nM MFMAs: fragment reads of `read_slot` (behind the first nR
-  // MFMAs), loads of K-step `ks`.
-  auto memory_ops = [&](auto n_mfma, auto n_read_mfma, int ks, int load_slot, int read_slot,
-                        frag_t (&na)[WM], frag_t (&nb)[WN]) {
-    constexpr int nM = decltype(n_mfma)::value, nR = decltype(n_read_mfma)::value;
-#pragma unroll
-    for (int i = 0; i < nM; ++i) {
-      if (i < nR) {
-#pragma unroll
-        for (int r = i * kFrags / nR; r < (i + 1) * kFrags / nR; ++r) read_one(read_slot, r, na, nb);
-      }
-#pragma unroll
-      for (int d = i * kLoadsPerStep / nM; d < (i + 1) * kLoadsPerStep / nM; ++d)
-        issue_one(ks, load_slot, d);
-    }
-  };
-  // MFMAs of block rows [x0, x1) of this wave's WM x WN blocks.
-  auto multiply_rows = [&](const frag_t (&fa)[WM], const frag_t (&fb)[WN], int x0, int x1) {
-#pragma unroll
-    for (int x = 0; x < WM; ++x)
-      if (x >= x0 && x < x1) {
-#pragma unroll
-        for (int y = 0; y < WN; ++y) acc[x][y] = Cfg::mfma(fa[x], fb[y], acc[x][y]);
-      }
-  };
-  auto multiply = [&](const frag_t (&fa)[WM], const frag_t (&fb)[WN]) {
-    multiply_rows(fa, fb, 0, WM);
-  };
-
-  frag_t fa[2][WM], fb[2][WN];
-  int done = 0;  // K-steps multiplied so far
-  if (T > kRing) {
-    // ---- pipelined path -------------------------------------------------
-    int issue_ks = kPro, issue_slot = kPro % kRing;   // next K-step to load and its slot
-    int read_slot = 0;                                // slot of K-step `done`
-#pragma unroll 1
-    for (int ks = 0; ks < kPro; ++ks) issue_step(ks, ks);
-    if (!a.accumulate) clear_acc();
-    wait_vmcnt<(kPro - kSync) * kLoadsPerStep>();  // the first kSync K-steps have landed
-    __builtin_amdgcn_s_barrier();                  // (bare, as in the loop below)
-    read_frags(0, fa[0], fb[0]);
-    // Each body multiplies kBody K-steps (whole sync groups, and an even
-    // number so that the fragment double buffer returns to fa[0]/fb[0]).
-    while (done + kBody <= T) {
-#pragma unroll
-      for (int g = 0; g < kBody; ++g) {
-        const int p = g & 1;
-        const bool sync_point = (g % kSync) == kSync - 1;
-        int next_slot = read_slot + 1; if (next_slot == kRing) next_slot = 0;
-        // Past the end of K the last K-step is loaded again (into a slot nobody
-        // reads any more): that keeps the number of loads in flight, and with
-        // it the vmcnt arithmetic, constant.
-        const int load_ks = issue_ks < T ? issue_ks : T - 1;
-        if (!sync_point) {
-          memory_ops(std::integral_constant<int, kMfmaAll>(), std::integral_constant<int, kReadAll>(),
-                     load_ks, issue_slot, next_slot, fa[p ^ 1], fb[p ^ 1]);
-          multiply(fa[p], fb[p]);
-          spread_issue<kMfmaAll, kReadAll, kFrags, kLoadsPerStep, kSub>();
-        } else {
-          // The first row of MFMAs goes ahead of the barrier so that the
-          // matrix pipe has work while the waves meet. This wave's reads of
-          // K-steps <= done+g are complete once fa[p]/fb[p] have arrived, and
-          // its loads of the next sync group once vmcnt has dropped to what
-          // was issued since: the barrier then frees the slots of this group
-          // and publishes the next group's data. The scheduling fences keep
-          // the compiler from moving anything across the sequence.
-          __builtin_amdgcn_sched_barrier(0);
-          multiply_rows(fa[p], fb[p], 0, 1);
-          __builtin_amdgcn_sched_barrier(0);
-          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-          wait_vmcnt<(kRing - 2 * kSync) * kLoadsPerStep>();
-          // A bare barrier: __syncthreads() carries a release fence for which
-          // the compiler drains every direct-to-LDS load still in flight.
-          __builtin_amdgcn_s_barrier();
-          __builtin_amdgcn_sched_barrier(0);
-          memory_ops(std::integral_constant<int, kMfmaRest>(), std::integral_constant<int, kReadRest>(),
-                     load_ks, issue_slot, next_slot, fa[p ^ 1], fb[p ^ 1]);
-          multiply_rows(fa[p], fb[p], 1, WM);
-          spread_issue<kMfmaRest, kReadRest, kFrags, kLoadsPerStep, kSub>();
-          __builtin_amdgcn_sched_barrier(0);
-        }
-        ++issue_ks;
-        ++issue_slot; if (issue_slot == kRing) issue_slot = 0;
-        read_slot = next_slot;
-      }
-      done += kBody;
-    }
-    // Remainder (< kBody K-steps): everything has been issued; wait for all
-    // of it and multiply straight out of the ring.
-    wait_vmcnt<0>();
-    __syncthreads();
-#pragma unroll 1
-    for (; done < T; ++done) {
-      read_frags(read_slot, fa[0], fb[0]);
-      multiply(fa[0], fb[0]);
-      ++read_slot; if (read_slot == kRing) read_slot = 0;
-    }
-  } else {
-    // ---- short-K path: everything fits in the ring ------------------------
-#pragma unroll 1
-    for (int ks = 0; ks < T; ++ks) issue_step(ks, ks);
-    if (!a.accumulate) clear_acc();
-    wait_vmcnt<0>();
-    __syncthreads();
-#pragma unroll 1
-    for (; done < T; ++done) {
-      read_frags(done, fa[0], fb[0]);
-      multiply(fa[0], fb[0]);
-    }
-  }
-
-  // K tail: fewer K tiles than one MFMA consumes are left. Their fragments
-  // come straight from global memory, with zeros in the lanes (or lane halves)
-  // that stand for the missing tiles.
-  if (a.tail_tiles > 0) {
-    const int64_t tail_off = (int64_t)T * kStepBytes;
-    auto tail_frag = [&](const char* block, int sub) -> frag_t {
-      const int4v zero = {0, 0, 0, 0};
-      if constexpr (kSub == 1) {
-        // (reached with a K0 below the instruction's K extent only: the lane's
-        // chunk belongs to K tile chunk / cpt of the step)
-        const int4v v = (frag_chunk / cpt) < a.tail_tiles ? *(const int4v*)(block + packed_lane_off(sub)) : zero;
-        union { int4v i; frag_t f; } u;
-        u.i = v;
-        return u.f;
-      } else {
-        const int t0 = 2 * (lane >> 5);
-        const char* p = block + (lane >> 5) * 1024 + (lane & 31) * 16;
-        const int4v lo = t0 < a.tail_tiles ? *(const int4v*)p : zero;
-        const int4v hi = t0 + 1 < a.tail_tiles ? *(const int4v*)(p + kPieceStride) : zero;
-        return frag_t{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-      }
-    };
-#pragma unroll
-    for (int x = 0; x < WM; ++x) {
-      const int blk = i_base + wm * WM + x;
-      int i = blk / kPerTile;
-      i = i < a.M ? i : a.M - 1;
-      fa[0][x] = tail_frag(a.lhs + (int64_t)i * a.lhs_stride_bytes + tail_off, blk % kPerTile);
-    }
-#pragma unroll
-    for (int y = 0; y < WN; ++y) {
-      const int blk = j_base + wn * WN + y;
-      int j = blk / kPerTile;
-      j = j < a.N ? j : a.N - 1;
-      fb[0][y] = tail_frag(a.rhs + (int64_t)j * a.rhs_stride_bytes + tail_off, blk % kPerTile);
-    }
-    multiply(fa[0], fb[0]);
-  }
-
-  // Epilogue (accumulator layout: acc_row / acc_col above). With 32x32 blocks
-  // one store instruction writes two full 128-byte rows of the tile, with
-  // 16x16 blocks four 64-byte row pieces.
-  if constexpr (kSiluMul) {
-    static_assert(WN % 2 == 0, "gate/up pairs must not straddle waves");
-    // Block pair (y, y+1) -> 32x32 bytes, stored as the two 32x16 tiles
-    // (rows of 16 bytes) that the next matmul reads as left-hand side: column
-    // c of row r lies at (c / 16) * 512 + r * 16 + c % 16.
-    const int col = lane & 31;
-    const int col_off = (col >> 4) * 512 + (col & 15);
-#pragma unroll
-    for (int x = 0; x < WM; ++x)
-#pragma unroll
-      for (int y = 0; y < WN; y += 2) {
-        const int i = i_base + wm * WM + x, j = j_base + wn * WN + y;
-        if (i < a.M && j + 1 < a.N) {
-          uint8_t* t = (uint8_t*)a.out + (int64_t)i * a.out_stride_bytes + (int64_t)(j >> 1) * 1024 + col_off;
-#pragma unroll
-          for (int v = 0; v < 16; v += 4) {
-            float h[4];
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-              h[e] = silu_mul((float)acc[x][y][v + e] * a.gate_scale,
-                              (float)acc[x][y + 1][v + e] * a.up_scale) * a.inv_out_scale;
-            const uint32_t packed = pack4_e4m3(h[0], h[1], h[2], h[3]);
-            const int row = 8 * (v >> 2) + 4 * (lane >> 5);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) t[(row + e) * 16] = (uint8_t)(packed >> (8 * e));
-          }
-        }
-      }
-    return;
-  }
-  if (a.row_major_out) {
-    // One store instruction writes 128 contiguous bytes of two matrix rows,
-    // exactly as it does for a tile; only the addresses differ.
-#pragma unroll
-    for (int x = 0; x < WM; ++x)
-#pragma unroll
-      for (int y = 0; y < WN; ++y) {
-        const int col = (j_base + wn * WN + y) * R + acc_col;
-        const int row0 = (i_base + wm * WM + x) * R;
-        if (col < a.out_cols) {
-#pragma unroll
-          for (int v = 0; v < kAccRegs; ++v) {
-            const int row = row0 + acc_row(v);
-            if (row < a.out_rows) {
-              out_t* dst = (out_t*)(a.out + (int64_t)row * a.out_stride_bytes) + col;
-              if constexpr (std::is_floating_point<decltype(acc[x][y][v] + 0)>::value)
-                *dst = (out_t)(acc[x][y][v] * a.out_scale);   // (x 1.0f is exact)
-              else
-                *dst = acc[x][y][v];
-            }
-          }
-        }
-      }
-    return;
-  }
-#pragma unroll
-  for (int x = 0; x < WM; ++x)
-#pragma unroll
-    for (int y = 0; y < WN; ++y) {
-      const int bi = i_base + wm * WM + x, bj = j_base + wn * WN + y;
-      const int i = bi / kPerTile, j = bj / kPerTile;
-      if (i < a.M && j < a.N) {
-        out_t* t = (out_t*)(a.out + (int64_t)i * a.out_stride_bytes) + (int64_t)j * 1024 +
-                   (bi % kPerTile) * R * 32 + (bj % kPerTile) * R;
-#pragma unroll
-        for (int v = 0; v < kAccRegs; ++v) t[acc_row(v) * 32 + acc_col] = acc[x][y][v];
-      }
-    }
+  mmt4d_mfma_body<Cfg, WM, WN, kRing, kSync, kSiluMul, kWavesN>(a);
 }
 
 template <typename Cfg, int WM, int WN, int kRing, int kSync, int kOcc = 1, bool kSiluMul = false,
@@ -586,7 +29,7 @@ int launch_variant(const MfmaArgs& a0, hipStream_t s) {
   a.tiles_n = (a.N * kPerTile + TN - 1) / TN;
   const int64_t blocks = (int64_t)a.tiles_m * a.tiles_n;
   if (blocks > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
-  constexpr int lds_bytes = kRing * (TM + TN) * Cfg::kSub * kPieceBytes;
+  constexpr int lds_bytes = mmt4d_mfma_lds_bytes<Cfg, WM, WN, kRing, kWavesN>();
   static_assert(lds_bytes <= 160 * 1024, "LDS ring exceeds 160 KiB");
   auto kernel = mmt4d_mfma_kernel<Cfg, WM, WN, kRing, kSync, kOcc, kSiluMul, kWavesN>;
   // The attribute belongs to the kernel on ONE device: set it once per device
