@@ -339,6 +339,21 @@ def extras(args, torch, iree_amd, F, synth, lhs, rhs, out, ex):
                     steps, warm)
     ex["mmt4d_f16_accumulate_tflops"] = round(flops / t / 1e12, 2)
 
+    # The same f16 mmt4d dispatched from the code object a HAL executable on a
+    # HIP device links (hipModuleLaunchKernel, bindings + 32-bit push constants)
+    from iree_amd import hal_executable
+    exe = hal_executable.HalExecutable()
+    hal_out = torch.empty_like(out)
+    name = "mi355x_mmt4d_f16f16f32_t8"
+    hal_step = lambda: exe.mmt4d(name, lhs, rhs, hal_out, M1, N1, size // 8, 8, F.MMT4D_TYPE_F16F16F32)
+    _, t = gpu_time(torch, hal_step, steps, warm)
+    iree_amd.mmt4d(lhs, rhs, out, M1, N1, size // 8, 32, 32, 8, F.MMT4D_TYPE_F16F16F32)
+    torch.cuda.synchronize()
+    assert torch.equal(hal_out.view(torch.int32), out.view(torch.int32)), "HAL export differs from the library"
+    ex["hal_executable_mmt4d_f16_tflops"] = round(flops / t / 1e12, 2)
+    exe.close()
+    del hal_out
+
     # i8 x i8 -> i32 at 4096^3, tile 32x32x16
     K1 = size // 16
     li = torch.from_numpy(synth.uniform_int8(1, M1 * K1 * 32 * 16)).cuda()

@@ -1,0 +1,67 @@
+/*
+ * iree_amd_hal_executable.h - loads a gfx950 code object of hand-written kernels
+ * and dispatches its exports the way IREE's HIP HAL driver does, so that the
+ * kernels linked into a `hal.executable.source`
+ * (REF samples/custom_dispatch/hip/kernels/example.mlir:36-118) can be run and
+ * tested without the IREE runtime.
+ *
+ * What each call stands for in the reference:
+ *   load      iree_hal_hip_native_executable_create: hipModuleLoadDataEx on the
+ *             code object bytes        REF runtime/src/iree/hal/drivers/hip/native_executable.c:180-200
+ *   add_export  per entry point: hipModuleGetFunction, the check of the shared
+ *             memory size against the device limit, hipFuncSetAttribute(
+ *             MAX_DYNAMIC_SHARED_SIZE_BYTES), block size kept for the launches
+ *                                      REF native_executable.c:213-253
+ *   dispatch  iree_hal_hip_stream_command_buffer_dispatch: kernel parameters =
+ *             the binding device pointers in order, then every push constant as
+ *             a 32-bit value in a parameter slot of its own; hipModuleLaunchKernel
+ *             with the export's block size and shared memory size
+ *                                      REF runtime/src/iree/hal/drivers/hip/stream_command_buffer.c:519-581
+ * Status codes are those of iree_amd_uk.h (0 = OK); the message of a failure is
+ * read with iree_amd_uk_last_error().
+ */
+#ifndef IREE_AMD_HAL_EXECUTABLE_H_
+#define IREE_AMD_HAL_EXECUTABLE_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#if defined(_WIN32)
+#define IREE_AMD_HAL_EXPORT
+#else
+#define IREE_AMD_HAL_EXPORT __attribute__((visibility("default")))
+#endif
+
+typedef struct iree_amd_hal_executable_t iree_amd_hal_executable_t;
+
+/* Loads the code object `data[0..size)` on the current device. */
+IREE_AMD_HAL_EXPORT int iree_amd_hal_executable_load(const void* data, size_t size,
+                                 iree_amd_hal_executable_t** out_executable);
+
+/* Registers the export `name` with the block size and dynamic shared memory
+ * size its hal.executable.export declares (workgroup_size,
+ * workgroup_local_memory); *out_ordinal is its index for dispatch. */
+IREE_AMD_HAL_EXPORT int iree_amd_hal_executable_add_export(iree_amd_hal_executable_t* executable, const char* name,
+                                       uint32_t block_x, uint32_t block_y, uint32_t block_z,
+                                       uint32_t shared_memory_size, int32_t* out_ordinal);
+
+/* Launches export `ordinal` over workgroup_x * _y * _z workgroups on `stream`
+ * (a hipStream_t; NULL = the default stream). `bindings` are device pointers. */
+IREE_AMD_HAL_EXPORT int iree_amd_hal_executable_dispatch(iree_amd_hal_executable_t* executable, int32_t ordinal,
+                                     uint32_t workgroup_x, uint32_t workgroup_y,
+                                     uint32_t workgroup_z, const void* const* bindings,
+                                     size_t binding_count, const uint32_t* push_constants,
+                                     size_t push_constant_count, void* stream);
+
+/* Unloads the module and frees the handle (NULL is accepted). */
+IREE_AMD_HAL_EXPORT void iree_amd_hal_executable_release(iree_amd_hal_executable_t* executable);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* IREE_AMD_HAL_EXECUTABLE_H_ */

@@ -149,6 +149,17 @@ def _declare(lib):
     lib.iree_amd_uk_pack_host.argtypes = [C.POINTER(PackParams)]
     lib.iree_amd_uk_unpack_host.restype = C.c_int
     lib.iree_amd_uk_unpack_host.argtypes = [C.POINTER(UnpackParams)]
+    # include/iree_amd_hal_executable.h
+    lib.iree_amd_hal_executable_load.restype = C.c_int
+    lib.iree_amd_hal_executable_load.argtypes = [vp, C.c_size_t, C.POINTER(vp)]
+    lib.iree_amd_hal_executable_add_export.restype = C.c_int
+    lib.iree_amd_hal_executable_add_export.argtypes = [vp, C.c_char_p, u32, u32, u32, u32,
+                                                       C.POINTER(i32)]
+    lib.iree_amd_hal_executable_dispatch.restype = C.c_int
+    lib.iree_amd_hal_executable_dispatch.argtypes = [vp, i32, u32, u32, u32, C.POINTER(vp),
+                                                     C.c_size_t, C.POINTER(u32), C.c_size_t, vp]
+    lib.iree_amd_hal_executable_release.restype = None
+    lib.iree_amd_hal_executable_release.argtypes = [vp]
 
 
 def load_library():

@@ -1,4 +1,6 @@
-"""Builds the C-ABI library (iree_amd/csrc/libiree_amd_uk.so) for gfx950.
+"""Builds the C-ABI library (iree_amd/csrc/libiree_amd_uk.so) and the code
+object of the mmt4d kernels for a HAL executable
+(iree_amd/hal/mi355x_kernels_gfx950.co) for gfx950.
 
     python -m iree_amd.build            # incremental
     python -m iree_amd.build --force    # recompile everything
@@ -22,6 +24,8 @@ def build(force=False, jobs=8, quiet=False):
     lib = os.path.join(CSRC, "libiree_amd_uk.so")
     if not os.path.exists(lib):
         raise RuntimeError("build finished but libiree_amd_uk.so is missing")
+    if not os.path.exists(os.path.join(HERE, "hal", "mi355x_kernels_gfx950.co")):
+        raise RuntimeError("build finished but hal/mi355x_kernels_gfx950.co is missing")
     return lib
 
 

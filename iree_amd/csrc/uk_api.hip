@@ -28,6 +28,9 @@ int check_hip(hipError_t err, const char* what) {
   } else if (err == hipErrorOutOfMemory) {
     status = 8;  // RESOURCE_EXHAUSTED
   }
+  // The error is reported here: take it off the runtime's "last error", or the
+  // caller's next HIP call (torch's, say) reports it a second time.
+  (void)hipGetLastError();
   return fail(status, "%s: %s", what, hipGetErrorString(err));
 }
 

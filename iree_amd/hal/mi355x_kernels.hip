@@ -1,0 +1,108 @@
+// The mmt4d kernels as a gfx950 code object for a HAL executable on a HIP
+// device: the device-resident route of the reference, where hand-written
+// kernels are linked into a `hal.executable.source` through
+// `#hal.executable.object<{path = "...co"}>`
+// (samples/custom_dispatch/hip/kernels/example.mlir:36-118) and launched by the
+// HIP HAL driver (runtime/src/iree/hal/drivers/hip/stream_command_buffer.c:519-581).
+//
+// ABI of every kernel here, as that driver packs it (kernels.cu:16-23 of the
+// same sample): C name, the binding device pointers in order, then one 32-bit
+// push constant per kernel parameter:
+//
+//   bindings        0 lhs (read only), 1 rhs (read only), 2 out
+//   push constants  M, N, K   outer tile counts, as iree_uk_mmt4d takes them
+//                             (runtime/src/iree/builtins/ukernel/mmt4d.h:14-21)
+//                   K0        elements per tile row (M0 = N0 = 32)
+//                   flags     the ukernel's flag word; IREE_UK_FLAG_MMT4D_ACCUMULATE
+//                             (0x100, exported_bits.h:43) is the one bit read here,
+//                             the type is fixed by the kernel's name
+//   (mi355x_mmt4d_unpack_*: two more, out_rows and out_cols)
+//
+// Operands are dense: lhs is [M][K][32][K0], rhs [N][K][32][K0], out
+// [M][N][32][32] (mi355x_mmt4d_unpack_*: the row-major out_rows x out_cols matrix
+// an unpack of it would give; accumulates from there as well). K >= 1, every
+// binding 16-byte aligned.
+//
+// Launch shape, fixed per export (workgroup_size and workgroup_local_memory of
+// the hal.executable.export): 256 threads; the dynamic LDS size and the macro
+// tile T (outer tiles of 32 rows per workgroup, both ways) are those of the
+// table at the end of this file. The grid is one-dimensional:
+// ceildiv(M, T) * ceildiv(N, T) workgroups.
+#include "../csrc/uk_mmt4d_mfma_kernel.h"
+
+namespace {
+
+using namespace uk;
+
+template <typename Cfg, int WM, int WN, int kRing, int kSync>
+__device__ __forceinline__ void hal_mmt4d(const void* lhs, const void* rhs, void* out, int M, int N,
+                                          int K, int K0, uint32_t flags, bool row_major,
+                                          int out_rows, int out_cols) {
+  constexpr int kPerTile = 32 / Cfg::kRows;
+  constexpr int TM = 2 * WM, TN = 2 * WN;
+  static_assert(TM == TN && TM % kPerTile == 0, "square macro tile of whole outer tiles");
+  typedef typename Cfg::out_t out_t;
+  MfmaArgs a;
+  const int64_t k_elems = (int64_t)K * K0;
+  a.lhs = (const char*)lhs;
+  a.rhs = (const char*)rhs;
+  a.out = (char*)out;
+  a.lhs_stride_bytes = a.rhs_stride_bytes = k_elems * 32 * Cfg::kElemBytes;
+  a.out_stride_bytes = row_major ? (int64_t)out_cols * (int64_t)sizeof(out_t)
+                                 : (int64_t)N * 1024 * (int64_t)sizeof(out_t);
+  a.M = M;
+  a.N = N;
+  a.ksteps = (int)(k_elems / Cfg::kMfmaK);
+  a.tail_tiles = (int)((k_elems % Cfg::kMfmaK) / K0);
+  a.tiles_m = (M * kPerTile + TM - 1) / TM;
+  a.tiles_n = (N * kPerTile + TN - 1) / TN;
+  a.accumulate = (flags & 0x100u) != 0;
+  a.row_major_out = row_major;
+  a.out_rows = out_rows;
+  a.out_cols = out_cols;
+  a.lhs_row_major = 0;
+  a.k0_div = Cfg::kMfmaK / K0;
+  a.gate_scale = a.up_scale = a.inv_out_scale = a.out_scale = 1.0f;
+  // a grid larger than the tile count (a count region that rounds up) is harmless
+  if (K < 1 || (int)blockIdx.x >= a.tiles_m * a.tiles_n) return;
+  mmt4d_mfma_body<Cfg, WM, WN, kRing, kSync>(a);
+}
+
+}  // namespace
+
+// One export per element-type tuple and macro tile, in the tiled and the
+// row-major-result form.
+#define MI355X_MMT4D_EXPORTS(NAME, CFG, WM, WN, RING, SYNC, OCC, LDS)                              \
+  static_assert(uk::mmt4d_mfma_lds_bytes<uk::CFG, WM, WN, RING>() == LDS, "LDS size of the table"); \
+  extern "C" __global__ __launch_bounds__(256, OCC) void mi355x_mmt4d_##NAME(                      \
+      const void* __restrict__ lhs, const void* __restrict__ rhs, void* __restrict__ out, int M,   \
+      int N, int K, int K0, unsigned flags) {                                                      \
+    hal_mmt4d<uk::CFG, WM, WN, RING, SYNC>(lhs, rhs, out, M, N, K, K0, flags, false, 0, 0);       \
+  }                                                                                                \
+  extern "C" __global__ __launch_bounds__(256, OCC) void mi355x_mmt4d_unpack_##NAME(               \
+      const void* __restrict__ lhs, const void* __restrict__ rhs, void* __restrict__ out, int M,   \
+      int N, int K, int K0, unsigned flags, int out_rows, int out_cols) {                          \
+    hal_mmt4d<uk::CFG, WM, WN, RING, SYNC>(lhs, rhs, out, M, N, K, K0, flags, true, out_rows,     \
+                                           out_cols);                                              \
+  }
+
+// name                      config      blocks/wave  ring sync occ    T   LDS bytes   K0 served
+// f16f16f32_t8   (256x256)  F16Cfg16      8 x 8        5    1   1     8   163840      8, 16
+// f16f16f32_t4   (128x128)  F16Cfg16      4 x 4        4    1   1     4    65536      8, 16
+// bf16bf16f32_t8 / _t4      BF16Cfg16     as f16
+// s8s8s32_t8     (256x256)  S8Cfg         4 x 4        8    2   1     8   131072      16, 32
+// s8s8s32_t4     (128x128)  S8Cfg         2 x 2        8    2   1     4    65536      16, 32
+// f8e4m3f8e4m3f32_t8        F8Cfg         4 x 4        5    1   1     8   163840      16
+// f8e4m3f8e4m3f32_t4        F8Cfg         2 x 2        8    2   1     4   131072      16
+// f32f32f32_t8              F32Cfg        4 x 4        8    2   1     8   131072      4, 8
+// f32f32f32_t4              F32Cfg        2 x 2        8    2   1     4    65536      4, 8
+MI355X_MMT4D_EXPORTS(f16f16f32_t8, F16Cfg16, 8, 8, 5, 1, 1, 163840)
+MI355X_MMT4D_EXPORTS(f16f16f32_t4, F16Cfg16, 4, 4, 4, 1, 1, 65536)
+MI355X_MMT4D_EXPORTS(bf16bf16f32_t8, BF16Cfg16, 8, 8, 5, 1, 1, 163840)
+MI355X_MMT4D_EXPORTS(bf16bf16f32_t4, BF16Cfg16, 4, 4, 4, 1, 1, 65536)
+MI355X_MMT4D_EXPORTS(s8s8s32_t8, S8Cfg, 4, 4, 8, 2, 1, 131072)
+MI355X_MMT4D_EXPORTS(s8s8s32_t4, S8Cfg, 2, 2, 8, 2, 1, 65536)
+MI355X_MMT4D_EXPORTS(f8e4m3f8e4m3f32_t8, F8Cfg, 4, 4, 5, 1, 1, 163840)
+MI355X_MMT4D_EXPORTS(f8e4m3f8e4m3f32_t4, F8Cfg, 2, 2, 8, 2, 1, 131072)
+MI355X_MMT4D_EXPORTS(f32f32f32_t8, F32Cfg, 4, 4, 8, 2, 1, 131072)
+MI355X_MMT4D_EXPORTS(f32f32f32_t4, F32Cfg, 2, 2, 8, 2, 1, 65536)

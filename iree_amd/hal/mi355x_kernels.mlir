@@ -1,0 +1,351 @@
+// hal.executable.source for iree_amd/hal/mi355x_kernels_gfx950.co: the gfx950
+// mmt4d kernels as hand-written dispatches on a HIP device, after the
+// reference's samples/custom_dispatch/hip/kernels/example.mlir:16-118.
+// Written by iree_amd.hal_executable.mlir_source(); NOT compiled here (this
+// build has no iree-compile).
+//
+// Every export: bindings lhs (read only), rhs (read only), out; push constants
+// M, N, K (outer tile counts), K0, flags (0x100 = accumulate), and for
+// mi355x_mmt4d_unpack_* also out_rows, out_cols. The workload of a dispatch is
+// (M, N).
+
+#rocm_gfx950_target = #hal.executable.target<"rocm", "rocm-hsaco-fb", {
+  target_arch = "gfx950"
+}>
+
+hal.executable.source public @mi355x_mmt4d attributes {
+  objects = #hal.executable.objects<{
+    #rocm_gfx950_target = [
+      #hal.executable.object<{path = "iree_amd/hal/mi355x_kernels_gfx950.co"}>
+    ]
+  }>
+} {
+  hal.executable.export public @mi355x_mmt4d_f16f16f32_t8 ordinal(0)
+      layout(#hal.pipeline.layout<push_constants = 5, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer, ReadOnly>,
+            <2, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index],
+    workgroup_local_memory = 163840 : index
+  } {
+  ^bb0(%device: !hal.device, %m: index, %n: index):
+    %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 8) * (s1 ceildiv 8))>()[%m, %n]
+    %c1 = arith.constant 1 : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  hal.executable.export public @mi355x_mmt4d_unpack_f16f16f32_t8 ordinal(1)
+      layout(#hal.pipeline.layout<push_constants = 7, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer, ReadOnly>,
+            <2, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index],
+    workgroup_local_memory = 163840 : index
+  } {
+  ^bb0(%device: !hal.device, %m: index, %n: index):
+    %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 8) * (s1 ceildiv 8))>()[%m, %n]
+    %c1 = arith.constant 1 : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  hal.executable.export public @mi355x_mmt4d_f16f16f32_t4 ordinal(2)
+      layout(#hal.pipeline.layout<push_constants = 5, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer, ReadOnly>,
+            <2, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index],
+    workgroup_local_memory = 65536 : index
+  } {
+  ^bb0(%device: !hal.device, %m: index, %n: index):
+    %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 4) * (s1 ceildiv 4))>()[%m, %n]
+    %c1 = arith.constant 1 : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  hal.executable.export public @mi355x_mmt4d_unpack_f16f16f32_t4 ordinal(3)
+      layout(#hal.pipeline.layout<push_constants = 7, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer, ReadOnly>,
+            <2, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index],
+    workgroup_local_memory = 65536 : index
+  } {
+  ^bb0(%device: !hal.device, %m: index, %n: index):
+    %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 4) * (s1 ceildiv 4))>()[%m, %n]
+    %c1 = arith.constant 1 : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  hal.executable.export public @mi355x_mmt4d_bf16bf16f32_t8 ordinal(4)
+      layout(#hal.pipeline.layout<push_constants = 5, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer, ReadOnly>,
+            <2, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index],
+    workgroup_local_memory = 163840 : index
+  } {
+  ^bb0(%device: !hal.device, %m: index, %n: index):
+    %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 8) * (s1 ceildiv 8))>()[%m, %n]
+    %c1 = arith.constant 1 : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  hal.executable.export public @mi355x_mmt4d_unpack_bf16bf16f32_t8 ordinal(5)
+      layout(#hal.pipeline.layout<push_constants = 7, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer, ReadOnly>,
+            <2, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index],
+    workgroup_local_memory = 163840 : index
+  } {
+  ^bb0(%device: !hal.device, %m: index, %n: index):
+    %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 8) * (s1 ceildiv 8))>()[%m, %n]
+    %c1 = arith.constant 1 : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  hal.executable.export public @mi355x_mmt4d_bf16bf16f32_t4 ordinal(6)
+      layout(#hal.pipeline.layout<push_constants = 5, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer, ReadOnly>,
+            <2, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index],
+    workgroup_local_memory = 65536 : index
+  } {
+  ^bb0(%device: !hal.device, %m: index, %n: index):
+    %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 4) * (s1 ceildiv 4))>()[%m, %n]
+    %c1 = arith.constant 1 : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  hal.executable.export public @mi355x_mmt4d_unpack_bf16bf16f32_t4 ordinal(7)
+      layout(#hal.pipeline.layout<push_constants = 7, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer, ReadOnly>,
+            <2, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index],
+    workgroup_local_memory = 65536 : index
+  } {
+  ^bb0(%device: !hal.device, %m: index, %n: index):
+    %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 4) * (s1 ceildiv 4))>()[%m, %n]
+    %c1 = arith.constant 1 : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  hal.executable.export public @mi355x_mmt4d_s8s8s32_t8 ordinal(8)
+      layout(#hal.pipeline.layout<push_constants = 5, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer, ReadOnly>,
+            <2, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index],
+    workgroup_local_memory = 131072 : index
+  } {
+  ^bb0(%device: !hal.device, %m: index, %n: index):
+    %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 8) * (s1 ceildiv 8))>()[%m, %n]
+    %c1 = arith.constant 1 : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  hal.executable.export public @mi355x_mmt4d_unpack_s8s8s32_t8 ordinal(9)
+      layout(#hal.pipeline.layout<push_constants = 7, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer, ReadOnly>,
+            <2, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index],
+    workgroup_local_memory = 131072 : index
+  } {
+  ^bb0(%device: !hal.device, %m: index, %n: index):
+    %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 8) * (s1 ceildiv 8))>()[%m, %n]
+    %c1 = arith.constant 1 : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  hal.executable.export public @mi355x_mmt4d_s8s8s32_t4 ordinal(10)
+      layout(#hal.pipeline.layout<push_constants = 5, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer, ReadOnly>,
+            <2, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index],
+    workgroup_local_memory = 65536 : index
+  } {
+  ^bb0(%device: !hal.device, %m: index, %n: index):
+    %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 4) * (s1 ceildiv 4))>()[%m, %n]
+    %c1 = arith.constant 1 : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  hal.executable.export public @mi355x_mmt4d_unpack_s8s8s32_t4 ordinal(11)
+      layout(#hal.pipeline.layout<push_constants = 7, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer, ReadOnly>,
+            <2, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index],
+    workgroup_local_memory = 65536 : index
+  } {
+  ^bb0(%device: !hal.device, %m: index, %n: index):
+    %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 4) * (s1 ceildiv 4))>()[%m, %n]
+    %c1 = arith.constant 1 : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  hal.executable.export public @mi355x_mmt4d_f8e4m3f8e4m3f32_t8 ordinal(12)
+      layout(#hal.pipeline.layout<push_constants = 5, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer, ReadOnly>,
+            <2, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index],
+    workgroup_local_memory = 163840 : index
+  } {
+  ^bb0(%device: !hal.device, %m: index, %n: index):
+    %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 8) * (s1 ceildiv 8))>()[%m, %n]
+    %c1 = arith.constant 1 : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  hal.executable.export public @mi355x_mmt4d_unpack_f8e4m3f8e4m3f32_t8 ordinal(13)
+      layout(#hal.pipeline.layout<push_constants = 7, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer, ReadOnly>,
+            <2, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index],
+    workgroup_local_memory = 163840 : index
+  } {
+  ^bb0(%device: !hal.device, %m: index, %n: index):
+    %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 8) * (s1 ceildiv 8))>()[%m, %n]
+    %c1 = arith.constant 1 : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  hal.executable.export public @mi355x_mmt4d_f8e4m3f8e4m3f32_t4 ordinal(14)
+      layout(#hal.pipeline.layout<push_constants = 5, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer, ReadOnly>,
+            <2, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index],
+    workgroup_local_memory = 131072 : index
+  } {
+  ^bb0(%device: !hal.device, %m: index, %n: index):
+    %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 4) * (s1 ceildiv 4))>()[%m, %n]
+    %c1 = arith.constant 1 : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  hal.executable.export public @mi355x_mmt4d_unpack_f8e4m3f8e4m3f32_t4 ordinal(15)
+      layout(#hal.pipeline.layout<push_constants = 7, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer, ReadOnly>,
+            <2, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index],
+    workgroup_local_memory = 131072 : index
+  } {
+  ^bb0(%device: !hal.device, %m: index, %n: index):
+    %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 4) * (s1 ceildiv 4))>()[%m, %n]
+    %c1 = arith.constant 1 : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  hal.executable.export public @mi355x_mmt4d_f32f32f32_t8 ordinal(16)
+      layout(#hal.pipeline.layout<push_constants = 5, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer, ReadOnly>,
+            <2, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index],
+    workgroup_local_memory = 131072 : index
+  } {
+  ^bb0(%device: !hal.device, %m: index, %n: index):
+    %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 8) * (s1 ceildiv 8))>()[%m, %n]
+    %c1 = arith.constant 1 : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  hal.executable.export public @mi355x_mmt4d_unpack_f32f32f32_t8 ordinal(17)
+      layout(#hal.pipeline.layout<push_constants = 7, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer, ReadOnly>,
+            <2, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index],
+    workgroup_local_memory = 131072 : index
+  } {
+  ^bb0(%device: !hal.device, %m: index, %n: index):
+    %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 8) * (s1 ceildiv 8))>()[%m, %n]
+    %c1 = arith.constant 1 : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  hal.executable.export public @mi355x_mmt4d_f32f32f32_t4 ordinal(18)
+      layout(#hal.pipeline.layout<push_constants = 5, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer, ReadOnly>,
+            <2, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index],
+    workgroup_local_memory = 65536 : index
+  } {
+  ^bb0(%device: !hal.device, %m: index, %n: index):
+    %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 4) * (s1 ceildiv 4))>()[%m, %n]
+    %c1 = arith.constant 1 : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  hal.executable.export public @mi355x_mmt4d_unpack_f32f32f32_t4 ordinal(19)
+      layout(#hal.pipeline.layout<push_constants = 7, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer, ReadOnly>,
+            <2, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index],
+    workgroup_local_memory = 65536 : index
+  } {
+  ^bb0(%device: !hal.device, %m: index, %n: index):
+    %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 4) * (s1 ceildiv 4))>()[%m, %n]
+    %c1 = arith.constant 1 : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+}
+
+// A dispatch site (f16, 4096^3: M = N = 128 outer tiles, K = 512 tiles of K0 = 8):
+//   %out = flow.dispatch @mi355x_mmt4d::@mi355x_mmt4d_f16f16f32_t8[%c128, %c128](
+//       %c128_i32, %c128_i32, %c512_i32, %c8_i32, %c0_i32, %lhs, %rhs)
+//     : (i32, i32, i32, i32, i32, tensor<128x512x32x8xf16>, tensor<128x512x32x8xf16>)
+//       -> tensor<128x128x32x32xf32>
+// (primitive operands come first and must be i32, example.mlir:128-140; with
+// the accumulate flag the result is tied to a third tensor operand: `-> %acc`.)

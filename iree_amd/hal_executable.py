@@ -1,0 +1,185 @@
+"""The mmt4d kernels as a HAL executable object for a HIP device.
+
+``iree_amd/hal/mi355x_kernels.hip`` builds into ``mi355x_kernels_gfx950.co``: a
+code object of ``extern "C"`` kernels that IREE links into a
+``hal.executable.source`` (reference
+samples/custom_dispatch/hip/kernels/example.mlir:36-118). This module holds the
+table of its exports (what the ``hal.executable.export`` ops must declare),
+writes that MLIR, and loads and dispatches the object the way the HIP HAL
+driver does (runtime/src/iree/hal/drivers/hip/native_executable.c:180-253,
+stream_command_buffer.c:519-581) through the C-ABI of
+``include/iree_amd_hal_executable.h`` - which is how the tests run it without
+an IREE runtime.
+"""
+import ctypes as C
+import os
+from collections import namedtuple
+
+from . import flags as F
+from ._lib import load_library
+from .ukernel import _check, _ptr, _stream
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CODE_OBJECT = os.path.join(HERE, "hal", "mi355x_kernels_gfx950.co")
+WORKGROUP_SIZE = 256
+
+# name: element-type tuple of the reference's flag enum; tile: outer tiles (of
+# 32 rows) per workgroup in both directions; lds: workgroup_local_memory in
+# bytes; k0: the K0 values served (the first is what the tile-size query answers).
+Export = namedtuple("Export", "name type_flag tile lds k0 lhs_bytes out_bytes")
+
+
+def _exports():
+    kib = 1024
+    rows = [
+        ("f16f16f32", F.MMT4D_TYPE_F16F16F32, 160 * kib, 64 * kib, (8, 16), 2, 4),
+        ("bf16bf16f32", F.MMT4D_TYPE_BF16BF16F32, 160 * kib, 64 * kib, (8, 16), 2, 4),
+        ("s8s8s32", F.MMT4D_TYPE_S8S8S32, 128 * kib, 64 * kib, (16, 32), 1, 4),
+        ("f8e4m3f8e4m3f32", F.MMT4D_TYPE_F8E4M3F8E4M3F32, 160 * kib, 128 * kib, (16,), 1, 4),
+        ("f32f32f32", F.MMT4D_TYPE_F32F32F32, 128 * kib, 64 * kib, (4, 8), 4, 4),
+    ]
+    out = {}
+    for name, flag, lds8, lds4, k0, lb, ob in rows:
+        for tile, lds in ((8, lds8), (4, lds4)):
+            for prefix in ("mi355x_mmt4d_", "mi355x_mmt4d_unpack_"):
+                full = f"{prefix}{name}_t{tile}"
+                out[full] = Export(full, flag, tile, lds, k0, lb, ob)
+    return out
+
+
+EXPORTS = _exports()
+
+
+def workgroup_count(export, M, N):
+    """Grid of an export for M x N outer tiles: what its count region returns."""
+    t = EXPORTS[export].tile if isinstance(export, str) else export.tile
+    return -(-M // t) * -(-N // t)
+
+
+class HalExecutable:
+    """A loaded code object; `dispatch` launches one export."""
+
+    def __init__(self, path=CODE_OBJECT):
+        if not os.path.exists(path):
+            raise RuntimeError(f"{path} is missing: build it with `python -m iree_amd.build`")
+        with open(path, "rb") as f:
+            self._image = f.read()
+        self._lib = load_library()
+        handle = C.c_void_p()
+        _check(self._lib.iree_amd_hal_executable_load(self._image, len(self._image), C.byref(handle)))
+        self._handle = handle
+        self._ordinals = {}
+
+    def add_export(self, name, block=(WORKGROUP_SIZE, 1, 1), shared_memory_size=None):
+        if shared_memory_size is None:
+            shared_memory_size = EXPORTS[name].lds
+        ordinal = C.c_int32(-1)
+        _check(self._lib.iree_amd_hal_executable_add_export(
+            self._handle, name.encode(), block[0], block[1], block[2], shared_memory_size,
+            C.byref(ordinal)))
+        self._ordinals[name] = ordinal.value
+        return ordinal.value
+
+    def dispatch(self, name, workgroups, bindings, push_constants, stream=None):
+        """bindings: CUDA tensors (or raw device addresses); push_constants: ints,
+        each passed as one 32-bit value."""
+        if name not in self._ordinals:
+            self.add_export(name)
+        if isinstance(workgroups, int):
+            workgroups = (workgroups, 1, 1)
+        ptrs = (C.c_void_p * max(len(bindings), 1))(
+            *[b if isinstance(b, int) else _ptr(b) for b in bindings])
+        consts = (C.c_uint32 * max(len(push_constants), 1))(
+            *[int(c) & 0xFFFFFFFF for c in push_constants])
+        _check(self._lib.iree_amd_hal_executable_dispatch(
+            self._handle, self._ordinals[name], workgroups[0], workgroups[1], workgroups[2],
+            ptrs, len(bindings), consts, len(push_constants), _stream(stream)))
+
+    def mmt4d(self, name, lhs, rhs, out, M, N, K, K0, flags, out_rows=None, out_cols=None,
+              stream=None):
+        """One mmt4d export over dense operands (see the table in
+        iree_amd/hal/mi355x_kernels.hip for the layouts)."""
+        e = EXPORTS[name]
+        consts = [M, N, K, K0, flags]
+        if "_unpack_" in name:
+            consts += [out_rows, out_cols]
+        self.dispatch(name, workgroup_count(e, M, N), [lhs, rhs, out], consts, stream)
+
+    def close(self):
+        if self._handle:
+            self._lib.iree_amd_hal_executable_release(self._handle)
+            self._handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+_MLIR_HEADER = """\
+// hal.executable.source for iree_amd/hal/mi355x_kernels_gfx950.co: the gfx950
+// mmt4d kernels as hand-written dispatches on a HIP device, after the
+// reference's samples/custom_dispatch/hip/kernels/example.mlir:16-118.
+// Written by iree_amd.hal_executable.mlir_source(); NOT compiled here (this
+// build has no iree-compile).
+//
+// Every export: bindings lhs (read only), rhs (read only), out; push constants
+// M, N, K (outer tile counts), K0, flags (0x100 = accumulate), and for
+// mi355x_mmt4d_unpack_* also out_rows, out_cols. The workload of a dispatch is
+// (M, N).
+
+#rocm_gfx950_target = #hal.executable.target<"rocm", "rocm-hsaco-fb", {
+  target_arch = "gfx950"
+}>
+
+hal.executable.source public @mi355x_mmt4d attributes {
+  objects = #hal.executable.objects<{
+    #rocm_gfx950_target = [
+      #hal.executable.object<{path = "iree_amd/hal/mi355x_kernels_gfx950.co"}>
+    ]
+  }>
+} {
+"""
+
+_MLIR_EXPORT = """\
+  hal.executable.export public @{name} ordinal({ordinal})
+      layout(#hal.pipeline.layout<push_constants = {constants}, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer, ReadOnly>,
+            <2, storage_buffer>
+        ]>
+      ]>) attributes {{
+    workgroup_size = [{wg} : index, 1 : index, 1 : index],
+    workgroup_local_memory = {lds} : index
+  }} {{
+  ^bb0(%device: !hal.device, %m: index, %n: index):
+    %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv {tile}) * (s1 ceildiv {tile}))>()[%m, %n]
+    %c1 = arith.constant 1 : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }}
+"""
+
+_MLIR_FOOTER = """\
+}
+
+// A dispatch site (f16, 4096^3: M = N = 128 outer tiles, K = 512 tiles of K0 = 8):
+//   %out = flow.dispatch @mi355x_mmt4d::@mi355x_mmt4d_f16f16f32_t8[%c128, %c128](
+//       %c128_i32, %c128_i32, %c512_i32, %c8_i32, %c0_i32, %lhs, %rhs)
+//     : (i32, i32, i32, i32, i32, tensor<128x512x32x8xf16>, tensor<128x512x32x8xf16>)
+//       -> tensor<128x128x32x32xf32>
+// (primitive operands come first and must be i32, example.mlir:128-140; with
+// the accumulate flag the result is tied to a third tensor operand: `-> %acc`.)
+"""
+
+
+def mlir_source():
+    """Text of the hal.executable.source that declares every export."""
+    parts = [_MLIR_HEADER]
+    for ordinal, e in enumerate(EXPORTS.values()):
+        parts.append(_MLIR_EXPORT.format(
+            name=e.name, ordinal=ordinal, constants=7 if "_unpack_" in e.name else 5,
+            wg=WORKGROUP_SIZE, lds=e.lds, tile=e.tile))
+    parts.append(_MLIR_FOOTER)
+    return "".join(parts)

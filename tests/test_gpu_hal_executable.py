@@ -1,0 +1,169 @@
+"""The code object of the mmt4d kernels for a HAL executable on a HIP device
+(iree_amd/hal/mi355x_kernels.hip), loaded and dispatched the way the reference's
+HIP HAL driver does (runtime/src/iree/hal/drivers/hip/native_executable.c:180-253,
+stream_command_buffer.c:519-581) through include/iree_amd_hal_executable.h.
+Every export is checked against the oracle bit for bit on the reference's
+small-integer inputs (tools/mmt4d_test.c:430-436), and the row-major-result
+exports against the library's own fused entry point on N(0,1) data."""
+import itertools
+import os
+import re
+import zlib
+
+import numpy as np
+import pytest
+
+import ukref
+from iree_amd import flags as F
+from iree_amd import hal_executable as H
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+TILED = [n for n in H.EXPORTS if "_unpack_" not in n]
+UNPACK = [n for n in H.EXPORTS if "_unpack_" in n]
+# outer shapes: one tile, ragged macro tiles both ways, more workgroups than
+# XCDs, K tile counts with and without a partial last matrix-core step
+SHAPES = [(1, 1, 1), (1, 1, 8), (3, 2, 6), (5, 7, 10), (9, 4, 19), (17, 9, 4), (4, 33, 2), (2, 3, 44)]
+
+
+def test_export_table_matches_the_sources():
+    """The Python table, the kernel source and the committed MLIR agree."""
+    with open(os.path.join(ROOT, "iree_amd", "hal", "mi355x_kernels.hip")) as f:
+        src = f.read()
+    rows = re.findall(r"^MI355X_MMT4D_EXPORTS\((\w+), \w+, \d+, \d+, \d+, \d+, \d+, (\d+)\)", src, re.M)
+    assert len(rows) * 2 == len(H.EXPORTS)
+    for name, lds in rows:
+        for prefix in ("mi355x_mmt4d_", "mi355x_mmt4d_unpack_"):
+            e = H.EXPORTS[prefix + name]
+            assert e.lds == int(lds) and e.tile == int(name[-1])
+    with open(os.path.join(ROOT, "iree_amd", "hal", "mi355x_kernels.mlir")) as f:
+        assert f.read() == H.mlir_source()
+    assert H.workgroup_count("mi355x_mmt4d_s8s8s32_t8", 9, 17) == 2 * 3
+    assert H.workgroup_count("mi355x_mmt4d_s8s8s32_t4", 9, 17) == 3 * 5
+
+
+def test_code_object_is_built_and_names_every_export():
+    with open(H.CODE_OBJECT, "rb") as f:
+        image = f.read()
+    for name in H.EXPORTS:
+        assert name.encode() + b"\0" in image, name
+
+
+def test_library_exports_the_declared_entry_points(uk):
+    with open(os.path.join(ROOT, "include", "iree_amd_hal_executable.h")) as f:
+        text = re.sub(r"/\*.*?\*/", "", f.read(), flags=re.S)
+    names = re.findall(r"IREE_AMD_HAL_EXPORT\s+\w+\s+(iree_amd_hal_executable_\w+)\s*\(", text)
+    assert sorted(names) == ["iree_amd_hal_executable_add_export", "iree_amd_hal_executable_dispatch",
+                             "iree_amd_hal_executable_load", "iree_amd_hal_executable_release"]
+    lib = uk.load_library()
+    for n in names:
+        assert hasattr(lib, n)
+
+
+@pytest.fixture(scope="module")
+def exe(uk, cuda):
+    e = H.HalExecutable()
+    yield e
+    e.close()
+
+
+def _dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a).view(np.uint8).reshape(-1).copy()).cuda()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", TILED)
+def test_tiled_exports_bit_exact_against_the_oracle(exe, name):
+    import torch
+    e = H.EXPORTS[name]
+    rng = np.random.default_rng(zlib.crc32(name.encode()))
+    for K0 in e.k0:
+        for (M, N, K), acc in itertools.product(SHAPES, (False, True)):
+            case = ukref.Mmt4dCase(rng, e.type_flag, M, N, K, 32, 32, K0, accumulate=acc)
+            lhs, rhs, out = _dev(case.lhs), _dev(case.rhs), _dev(case.out_init)
+            exe.mmt4d(name, lhs, rhs, out, M, N, K, K0, case.flags)
+            torch.cuda.synchronize()
+            got = out.cpu().numpy().view(case.out_init.dtype)
+            want = case.run_oracle(ukref.F16_IEEE)
+            assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), (name, K0, (M, N, K), acc)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", UNPACK)
+def test_row_major_exports_equal_the_library_entry_point(uk, cuda, exe, name):
+    """Same kernel body as iree_amd_uk_mmt4d_unpack: identical bits on float data,
+    with ragged M and N, a partial last K step, with and without accumulation;
+    elements outside the matrix stay untouched (the buffers are exactly M x N)."""
+    import torch
+    e = H.EXPORTS[name]
+    K0 = e.k0[0]
+    M, N = 200, 333
+    K1 = 37
+    M1, N1 = -(-M // 32), -(-N // 32)
+    rng = np.random.default_rng(21)
+
+    def operand(n):
+        if e.type_flag == F.MMT4D_TYPE_S8S8S32:
+            return torch.from_numpy(rng.integers(-128, 128, n, dtype=np.int8)).cuda()
+        if e.type_flag == F.MMT4D_TYPE_F8E4M3F8E4M3F32:
+            # every byte but the two NaN encodings
+            b = rng.integers(0, 256, n, dtype=np.uint8)
+            b[(b & 0x7F) == 0x7F] = 0x38
+            return torch.from_numpy(b).cuda()
+        x = torch.from_numpy(rng.standard_normal(n).astype(np.float32)).cuda()
+        return {F.MMT4D_TYPE_F16F16F32: x.half(), F.MMT4D_TYPE_BF16BF16F32: x.bfloat16(),
+                F.MMT4D_TYPE_F32F32F32: x}[e.type_flag]
+
+    lhs, rhs = operand(M1 * K1 * 32 * K0), operand(N1 * K1 * 32 * K0)
+    odt = torch.int32 if e.type_flag == F.MMT4D_TYPE_S8S8S32 else torch.float32
+    for acc in (0, F.MMT4D_ACCUMULATE):
+        init = torch.from_numpy(rng.integers(-50, 50, M * N).astype(np.int32)).cuda().to(odt)
+        one, two = init.clone(), init.clone()
+        exe.mmt4d(name, lhs, rhs, one, M1, N1, K1, K0, e.type_flag | acc, out_rows=M, out_cols=N)
+        uk.mmt4d_unpack(lhs, rhs, two, M, N, M1, N1, K1, K0, e.type_flag | acc)
+        torch.cuda.synchronize()
+        assert np.array_equal(one.cpu().numpy().view(np.uint32), two.cpu().numpy().view(np.uint32)), (name, acc)
+        assert not torch.equal(one, init)
+
+
+@pytest.mark.gpu
+def test_full_size_f16_dispatch_equals_the_library(uk, cuda, exe):
+    """4096^3 f16 through the 256x256 export: the bits of iree_amd_uk_mmt4d."""
+    import torch
+    from iree_amd import synth
+    M1 = N1 = 128
+    K0, K1 = 8, 512
+    lhs = torch.from_numpy(synth.normal_f16(1, 4096 * 4096, scale=1 / 64).view(np.int16)).cuda()
+    rhs = torch.from_numpy(synth.normal_f16(2, 4096 * 4096, scale=1 / 64).view(np.int16)).cuda()
+    one = torch.empty(4096 * 4096, dtype=torch.float32, device=cuda)
+    two = torch.empty(4096 * 4096, dtype=torch.float32, device=cuda)
+    exe.mmt4d("mi355x_mmt4d_f16f16f32_t8", lhs, rhs, one, M1, N1, K1, K0, F.MMT4D_TYPE_F16F16F32)
+    uk.mmt4d(lhs, rhs, two, M1, N1, K1, 32, 32, K0, F.MMT4D_TYPE_F16F16F32)
+    torch.cuda.synchronize()
+    assert float(two.abs().max()) > 0
+    assert torch.equal(one.view(torch.int32), two.view(torch.int32))
+
+
+@pytest.mark.gpu
+def test_loader_rejects_what_the_driver_rejects(uk, cuda, exe):
+    with pytest.raises(uk.UkError) as err:
+        exe.add_export("mi355x_no_such_kernel", shared_memory_size=0)
+    assert err.value.status == 5 and "not found" in str(err.value)
+    with pytest.raises(uk.UkError) as err:
+        exe.add_export("mi355x_mmt4d_s8s8s32_t8", shared_memory_size=1 << 20)
+    assert err.value.status == 3 and "shared memory" in str(err.value)
+    with pytest.raises(uk.UkError):
+        exe.add_export("mi355x_mmt4d_s8s8s32_t8", block=(2048, 1, 1))
+    import ctypes as C
+    lib = uk.load_library()
+    handle = C.c_void_p()
+    assert lib.iree_amd_hal_executable_load(None, 0, C.byref(handle)) == 3
+    junk = b"not a code object" * 16
+    assert lib.iree_amd_hal_executable_load(junk, len(junk), C.byref(handle)) != 0
+    assert not handle.value
+    # an empty grid is a no-op
+    import torch
+    out = torch.full((1024,), 7, dtype=torch.int32, device=cuda)
+    exe.dispatch("mi355x_mmt4d_s8s8s32_t4", 0, [out, out, out], [0, 0, 1, 16, 0])
+    torch.cuda.synchronize()
+    assert int(out.min()) == 7
