@@ -12,10 +12,30 @@ namespace {
 
 // kOcc: waves per SIMD the register allocation must leave room for (2 = two
 // workgroups of 4 waves resident on one compute unit).
-template <typename Cfg, int WM, int WN, int kRing, int kSync, int kOcc = 1, bool kSiluMul = false,
-          int kWavesN = 2>
+template <typename Cfg, int WM, int WN, int kRing, int kSync, int kOcc, bool kSiluMul, int kWavesN,
+          int kForm>
 __global__ __launch_bounds__(128 * kWavesN, kOcc) void mmt4d_mfma_kernel(MfmaArgs a) {
-  mmt4d_mfma_body<Cfg, WM, WN, kRing, kSync, kSiluMul, kWavesN>(a);
+  mmt4d_mfma_body<Cfg, WM, WN, kRing, kSync, kSiluMul, kWavesN, kForm>(a);
+}
+
+template <typename Cfg, int WM, int WN, int kRing, int kSync, int kOcc, bool kSiluMul, int kWavesN,
+          int kForm>
+int launch_form(const MfmaArgs& a, unsigned blocks, hipStream_t s) {
+  constexpr int lds_bytes = mmt4d_mfma_lds_bytes<Cfg, WM, WN, kRing, kWavesN>();
+  static_assert(lds_bytes <= 160 * 1024, "LDS ring exceeds 160 KiB");
+  auto kernel = mmt4d_mfma_kernel<Cfg, WM, WN, kRing, kSync, kOcc, kSiluMul, kWavesN, kForm>;
+  // The attribute belongs to the kernel on ONE device: set it once per device
+  // ordinal (a benign race: the call is idempotent).
+  static unsigned long long attr_set_on = 0;
+  int dev = 0;
+  UK_RETURN_IF_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= 64 || !((attr_set_on >> dev) & 1)) {
+    UK_RETURN_IF_HIP(hipFuncSetAttribute((const void*)kernel,
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes));
+    if (dev >= 0 && dev < 64) attr_set_on |= 1ull << dev;
+  }
+  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(128 * kWavesN), lds_bytes, s, a);
+  return check_hip(hipGetLastError(), "mmt4d_mfma launch");
 }
 
 template <typename Cfg, int WM, int WN, int kRing, int kSync, int kOcc = 1, bool kSiluMul = false,
@@ -29,21 +49,15 @@ int launch_variant(const MfmaArgs& a0, hipStream_t s) {
   a.tiles_n = (a.N * kPerTile + TN - 1) / TN;
   const int64_t blocks = (int64_t)a.tiles_m * a.tiles_n;
   if (blocks > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
-  constexpr int lds_bytes = mmt4d_mfma_lds_bytes<Cfg, WM, WN, kRing, kWavesN>();
-  static_assert(lds_bytes <= 160 * 1024, "LDS ring exceeds 160 KiB");
-  auto kernel = mmt4d_mfma_kernel<Cfg, WM, WN, kRing, kSync, kOcc, kSiluMul, kWavesN>;
-  // The attribute belongs to the kernel on ONE device: set it once per device
-  // ordinal (a benign race: the call is idempotent).
-  static unsigned long long attr_set_on = 0;
-  int dev = 0;
-  UK_RETURN_IF_HIP(hipGetDevice(&dev));
-  if (dev < 0 || dev >= 64 || !((attr_set_on >> dev) & 1)) {
-    UK_RETURN_IF_HIP(hipFuncSetAttribute((const void*)kernel,
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes));
-    if (dev >= 0 && dev < 64) attr_set_on |= 1ull << dev;
+  // one kernel instance per operand form (the forms the entry points produce)
+  if constexpr (!kSiluMul) {
+    if (a.lhs_row_major && a.row_major_out)
+      return launch_form<Cfg, WM, WN, kRing, kSync, kOcc, kSiluMul, kWavesN, 2>(a, (unsigned)blocks, s);
+    if (a.row_major_out)
+      return launch_form<Cfg, WM, WN, kRing, kSync, kOcc, kSiluMul, kWavesN, 1>(a, (unsigned)blocks, s);
   }
-  hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(128 * kWavesN), lds_bytes, s, a);
-  return check_hip(hipGetLastError(), "mmt4d_mfma launch");
+  if (a.lhs_row_major || a.row_major_out) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  return launch_form<Cfg, WM, WN, kRing, kSync, kOcc, kSiluMul, kWavesN, 0>(a, (unsigned)blocks, s);
 }
 
 template <typename Cfg, bool kSiluMul = false>

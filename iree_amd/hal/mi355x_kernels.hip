@@ -34,10 +34,9 @@ namespace {
 
 using namespace uk;
 
-template <typename Cfg, int WM, int WN, int kRing, int kSync>
+template <typename Cfg, int WM, int WN, int kRing, int kSync, bool row_major>
 __device__ __forceinline__ void hal_mmt4d(const void* lhs, const void* rhs, void* out, int M, int N,
-                                          int K, int K0, uint32_t flags, bool row_major,
-                                          int out_rows, int out_cols) {
+                                          int K, int K0, uint32_t flags, int out_rows, int out_cols) {
   constexpr int kPerTile = 32 / Cfg::kRows;
   constexpr int TM = 2 * WM, TN = 2 * WN;
   static_assert(TM == TN && TM % kPerTile == 0, "square macro tile of whole outer tiles");
@@ -65,7 +64,7 @@ __device__ __forceinline__ void hal_mmt4d(const void* lhs, const void* rhs, void
   a.gate_scale = a.up_scale = a.inv_out_scale = a.out_scale = 1.0f;
   // a grid larger than the tile count (a count region that rounds up) is harmless
   if (K < 1 || (int)blockIdx.x >= a.tiles_m * a.tiles_n) return;
-  mmt4d_mfma_body<Cfg, WM, WN, kRing, kSync>(a);
+  mmt4d_mfma_body<Cfg, WM, WN, kRing, kSync, false, 2, row_major ? 1 : 0>(a);
 }
 
 }  // namespace
@@ -77,13 +76,13 @@ __device__ __forceinline__ void hal_mmt4d(const void* lhs, const void* rhs, void
   extern "C" __global__ __launch_bounds__(256, OCC) void mi355x_mmt4d_##NAME(                      \
       const void* __restrict__ lhs, const void* __restrict__ rhs, void* __restrict__ out, int M,   \
       int N, int K, int K0, unsigned flags) {                                                      \
-    hal_mmt4d<uk::CFG, WM, WN, RING, SYNC>(lhs, rhs, out, M, N, K, K0, flags, false, 0, 0);       \
+    hal_mmt4d<uk::CFG, WM, WN, RING, SYNC, false>(lhs, rhs, out, M, N, K, K0, flags, 0, 0);       \
   }                                                                                                \
   extern "C" __global__ __launch_bounds__(256, OCC) void mi355x_mmt4d_unpack_##NAME(               \
       const void* __restrict__ lhs, const void* __restrict__ rhs, void* __restrict__ out, int M,   \
       int N, int K, int K0, unsigned flags, int out_rows, int out_cols) {                          \
-    hal_mmt4d<uk::CFG, WM, WN, RING, SYNC>(lhs, rhs, out, M, N, K, K0, flags, true, out_rows,     \
-                                           out_cols);                                              \
+    hal_mmt4d<uk::CFG, WM, WN, RING, SYNC, true>(lhs, rhs, out, M, N, K, K0, flags, out_rows,     \
+                                                 out_cols);                                        \
   }
 
 // name                      config      blocks/wave  ring sync occ    T   LDS bytes   K0 served
