@@ -62,9 +62,6 @@
 #include "uk_mfma_cfg.h"
 
 namespace uk {
-namespace {
-
-constexpr int kPieceBytes = 1024;   // what one 64-lane 128-bit load moves
 
 struct MfmaArgs {
   const char* lhs;  // offset applied
@@ -91,6 +88,11 @@ struct MfmaArgs {
   // row-major result of a float type only: factor applied on the store
   float out_scale;
 };
+
+namespace {
+
+constexpr int kPieceBytes = 1024;   // what one 64-lane 128-bit load moves
+
 
 __device__ __forceinline__ void load_block_to_lds(__amdgpu_buffer_rsrc_t row, uint32_t lane_off,
                                                   uint32_t block_off, char* lds) {
