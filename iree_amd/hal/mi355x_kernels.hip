@@ -1,5 +1,5 @@
-// The mmt4d kernels as a gfx950 code object for a HAL executable on a HIP
-// device: the device-resident route of the reference, where hand-written
+// The mmt4d, pack and unpack kernels as a gfx950 code object for a HAL
+// executable on a HIP device: the device-resident route of the reference, where hand-written
 // kernels are linked into a `hal.executable.source` through
 // `#hal.executable.object<{path = "...co"}>`
 // (samples/custom_dispatch/hip/kernels/example.mlir:36-118) and launched by the
@@ -28,7 +28,25 @@
 // tile T (outer tiles of 32 rows per workgroup, both ways) are those of the
 // table at the end of this file. The grid is one-dimensional:
 // ceildiv(M, T) * ceildiv(N, T) workgroups.
+//
+// mi355x_pack_{8,16,32}bit / mi355x_unpack_{16,32}bit: iree_uk_pack / iree_uk_unpack
+// without transposes (runtime/src/iree/builtins/ukernel/pack.h:26-34,
+// unpack.h:17-25) on dense operands, for power-of-two tiles whose rows are whole
+// 16-byte chunks:
+//
+//   pack    bindings 0 in: the size0 x size1 matrix (read only), 1 out: tiles
+//           [ceildiv(size0, tile0)][ceildiv(size1, tile1)][tile0][tile1]
+//           push constants size0, size1, tile0, tile1, padding (the element's bits)
+//   unpack  bindings 0 in: the tiles (read only), 1 out: the size0 x size1 matrix
+//           push constants size0, size1, tile0, tile1
+//
+// 256 threads, no LDS; grid = ceildiv(C, 32) * ceildiv(R, 16) with, for pack,
+// C = ceildiv(size1, tile1) * tile1 * bytes / 16 and R = ceildiv(size0, tile0) *
+// tile0 (the padded extent), for unpack C = ceildiv(size1 * bytes, 16) and
+// R = size0. Limits (32-bit offsets inside a block of 16 rows): a matrix row
+// and one outer row of tiles below 2^26 bytes each.
 #include "../csrc/uk_mmt4d_mfma_kernel.h"
+#include "../csrc/uk_pack_stream_kernel.h"
 
 namespace {
 
@@ -67,7 +85,55 @@ __device__ __forceinline__ void hal_mmt4d(const void* lhs, const void* rhs, void
   mmt4d_mfma_body<Cfg, WM, WN, kRing, kSync, false, 2, row_major ? 1 : 0>(a);
 }
 
+template <int ES, bool kPack>
+__device__ __forceinline__ void hal_pack(const void* mat, void* tiled, int size0, int size1,
+                                         int tile0, int tile1, uint32_t padding) {
+  constexpr int CE = 16 / ES;
+  if (size0 < 1 || size1 < 1 || tile0 < 1 || tile1 < CE) return;
+  Pow2Args a;
+  a.log2_tile_rows = __builtin_ctz((unsigned)tile0);
+  const int cpr = tile1 / CE;
+  a.log2_cpr = __builtin_ctz((unsigned)cpr);
+  const int64_t outer0 = ((int64_t)size0 + tile0 - 1) >> a.log2_tile_rows;
+  const int64_t outer1 = ((int64_t)size1 + tile1 - 1) / tile1;
+  a.mat = (const char*)mat;
+  a.tiled = (char*)tiled;
+  a.m_size0 = size0;
+  a.m_size1 = size1;
+  a.m_pitch_bytes = (int64_t)size1 * ES;
+  a.t_stride_col_bytes = (int64_t)tile0 * tile1 * ES;
+  a.t_stride_row_bytes = outer1 * a.t_stride_col_bytes;
+  a.padded_rows = outer0 << a.log2_tile_rows;
+  a.chunks_per_row = (uint32_t)(((int64_t)size1 + CE - 1) / CE);
+  a.padded_chunks_per_row = (uint32_t)(outer1 * cpr);
+  const int64_t cols = kPack ? a.padded_chunks_per_row : a.chunks_per_row;
+  const int64_t rows = kPack ? a.padded_rows : (int64_t)size0;
+  a.blocks_x = (uint32_t)((cols + 4 * kBlockChunks - 1) / (4 * kBlockChunks));
+  a.blocks_y = (uint32_t)((rows + kBlockRows * kStreamUnroll - 1) / (kBlockRows * kStreamUnroll));
+  a.padding = padding;
+  if (blockIdx.x >= a.blocks_x * a.blocks_y) return;
+  stream_pow2_body<ES, kPack>(a);
+}
+
 }  // namespace
+
+#define MI355X_PACK_EXPORTS(BITS, ES)                                                              \
+  extern "C" __global__ __launch_bounds__(256) void mi355x_pack_##BITS##bit(                      \
+      const void* __restrict__ in, void* __restrict__ out, int size0, int size1, int tile0,       \
+      int tile1, unsigned padding) {                                                               \
+    hal_pack<ES, true>(in, out, size0, size1, tile0, tile1, padding);                             \
+  }
+#define MI355X_UNPACK_EXPORTS(BITS, ES)                                                            \
+  extern "C" __global__ __launch_bounds__(256) void mi355x_unpack_##BITS##bit(                    \
+      const void* __restrict__ in, void* __restrict__ out, int size0, int size1, int tile0,       \
+      int tile1) {                                                                                 \
+    hal_pack<ES, false>(out, const_cast<void*>(in), size0, size1, tile0, tile1, 0);               \
+  }
+MI355X_PACK_EXPORTS(8, 1)
+MI355X_PACK_EXPORTS(16, 2)
+MI355X_PACK_EXPORTS(32, 4)
+MI355X_UNPACK_EXPORTS(16, 2)
+MI355X_UNPACK_EXPORTS(32, 4)
 
 // One export per element-type tuple and macro tile, in the tiled and the
 // row-major-result form.

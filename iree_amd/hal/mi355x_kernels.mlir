@@ -1,10 +1,10 @@
 // hal.executable.source for iree_amd/hal/mi355x_kernels_gfx950.co: the gfx950
-// mmt4d kernels as hand-written dispatches on a HIP device, after the
+// mmt4d, pack and unpack kernels as hand-written dispatches on a HIP device, after the
 // reference's samples/custom_dispatch/hip/kernels/example.mlir:16-118.
 // Written by iree_amd.hal_executable.mlir_source(); NOT compiled here (this
 // build has no iree-compile).
 //
-// Every export: bindings lhs (read only), rhs (read only), out; push constants
+// Every mmt4d export: bindings lhs (read only), rhs (read only), out; push constants
 // M, N, K (outer tile counts), K0, flags (0x100 = accumulate), and for
 // mi355x_mmt4d_unpack_* also out_rows, out_cols. The workload of a dispatch is
 // (M, N).
@@ -338,6 +338,128 @@ hal.executable.source public @mi355x_mmt4d attributes {
   ^bb0(%device: !hal.device, %m: index, %n: index):
     %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 4) * (s1 ceildiv 4))>()[%m, %n]
     %c1 = arith.constant 1 : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  // pack: in = matrix, out = tiles; push constants size0, size1, tile0, tile1, padding; workload (size0, size1, tile0, tile1)
+  hal.executable.export public @mi355x_pack_8bit ordinal(20)
+      layout(#hal.pipeline.layout<push_constants = 5, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index]
+  } {
+  ^bb0(%device: !hal.device, %size0: index, %size1: index, %tile0: index, %tile1: index):
+    %c1 = arith.constant 1 : index
+    %c16 = arith.constant 16 : index
+    %c32 = arith.constant 32 : index
+    %bytes = arith.constant 1 : index
+    %o0 = arith.ceildivui %size0, %tile0 : index
+    %rows = arith.muli %o0, %tile0 : index
+    %o1 = arith.ceildivui %size1, %tile1 : index
+    %cols = arith.muli %o1, %tile1 : index
+    %row_bytes = arith.muli %cols, %bytes : index
+    %chunks = arith.ceildivui %row_bytes, %c16 : index
+    %bx = arith.ceildivui %chunks, %c32 : index
+    %by = arith.ceildivui %rows, %c16 : index
+    %x = arith.muli %bx, %by : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  // pack: in = matrix, out = tiles; push constants size0, size1, tile0, tile1, padding; workload (size0, size1, tile0, tile1)
+  hal.executable.export public @mi355x_pack_16bit ordinal(21)
+      layout(#hal.pipeline.layout<push_constants = 5, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index]
+  } {
+  ^bb0(%device: !hal.device, %size0: index, %size1: index, %tile0: index, %tile1: index):
+    %c1 = arith.constant 1 : index
+    %c16 = arith.constant 16 : index
+    %c32 = arith.constant 32 : index
+    %bytes = arith.constant 2 : index
+    %o0 = arith.ceildivui %size0, %tile0 : index
+    %rows = arith.muli %o0, %tile0 : index
+    %o1 = arith.ceildivui %size1, %tile1 : index
+    %cols = arith.muli %o1, %tile1 : index
+    %row_bytes = arith.muli %cols, %bytes : index
+    %chunks = arith.ceildivui %row_bytes, %c16 : index
+    %bx = arith.ceildivui %chunks, %c32 : index
+    %by = arith.ceildivui %rows, %c16 : index
+    %x = arith.muli %bx, %by : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  // pack: in = matrix, out = tiles; push constants size0, size1, tile0, tile1, padding; workload (size0, size1, tile0, tile1)
+  hal.executable.export public @mi355x_pack_32bit ordinal(22)
+      layout(#hal.pipeline.layout<push_constants = 5, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index]
+  } {
+  ^bb0(%device: !hal.device, %size0: index, %size1: index, %tile0: index, %tile1: index):
+    %c1 = arith.constant 1 : index
+    %c16 = arith.constant 16 : index
+    %c32 = arith.constant 32 : index
+    %bytes = arith.constant 4 : index
+    %o0 = arith.ceildivui %size0, %tile0 : index
+    %rows = arith.muli %o0, %tile0 : index
+    %o1 = arith.ceildivui %size1, %tile1 : index
+    %cols = arith.muli %o1, %tile1 : index
+    %row_bytes = arith.muli %cols, %bytes : index
+    %chunks = arith.ceildivui %row_bytes, %c16 : index
+    %bx = arith.ceildivui %chunks, %c32 : index
+    %by = arith.ceildivui %rows, %c16 : index
+    %x = arith.muli %bx, %by : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  // unpack: in = tiles, out = matrix; push constants size0, size1, tile0, tile1; workload (size0, size1, tile0, tile1)
+  hal.executable.export public @mi355x_unpack_16bit ordinal(23)
+      layout(#hal.pipeline.layout<push_constants = 4, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index]
+  } {
+  ^bb0(%device: !hal.device, %size0: index, %size1: index, %tile0: index, %tile1: index):
+    %c1 = arith.constant 1 : index
+    %c16 = arith.constant 16 : index
+    %c32 = arith.constant 32 : index
+    %bytes = arith.constant 2 : index
+    %row_bytes = arith.muli %size1, %bytes : index
+    %chunks = arith.ceildivui %row_bytes, %c16 : index
+    %bx = arith.ceildivui %chunks, %c32 : index
+    %by = arith.ceildivui %size0, %c16 : index
+    %x = arith.muli %bx, %by : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  // unpack: in = tiles, out = matrix; push constants size0, size1, tile0, tile1; workload (size0, size1, tile0, tile1)
+  hal.executable.export public @mi355x_unpack_32bit ordinal(24)
+      layout(#hal.pipeline.layout<push_constants = 4, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index]
+  } {
+  ^bb0(%device: !hal.device, %size0: index, %size1: index, %tile0: index, %tile1: index):
+    %c1 = arith.constant 1 : index
+    %c16 = arith.constant 16 : index
+    %c32 = arith.constant 32 : index
+    %bytes = arith.constant 4 : index
+    %row_bytes = arith.muli %size1, %bytes : index
+    %chunks = arith.ceildivui %row_bytes, %c16 : index
+    %bx = arith.ceildivui %chunks, %c32 : index
+    %by = arith.ceildivui %size0, %c16 : index
+    %x = arith.muli %bx, %by : index
     hal.return %x, %c1, %c1 : index, index, index
   }
 }

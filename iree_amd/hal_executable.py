@@ -1,4 +1,4 @@
-"""The mmt4d kernels as a HAL executable object for a HIP device.
+"""The mmt4d, pack and unpack kernels as a HAL executable object for a HIP device.
 
 ``iree_amd/hal/mi355x_kernels.hip`` builds into ``mi355x_kernels_gfx950.co``: a
 code object of ``extern "C"`` kernels that IREE links into a
@@ -49,6 +49,25 @@ def _exports():
 
 EXPORTS = _exports()
 
+# pack / unpack without transposes, by element size: name -> (bytes per element,
+# True for pack). Power-of-two tiles whose rows are whole 16-byte chunks.
+PACK_EXPORTS = {"mi355x_pack_8bit": (1, True), "mi355x_pack_16bit": (2, True),
+                "mi355x_pack_32bit": (4, True), "mi355x_unpack_16bit": (2, False),
+                "mi355x_unpack_32bit": (4, False)}
+
+
+def pack_workgroup_count(name, size0, size1, tile0, tile1):
+    """Grid of a pack / unpack export: blocks of 16 rows x 32 chunks of 16 bytes
+    over the padded extent (pack) or the matrix itself (unpack)."""
+    es, is_pack = PACK_EXPORTS[name]
+    if is_pack:
+        cols = -(-size1 // tile1) * tile1 * es // 16
+        rows = -(-size0 // tile0) * tile0
+    else:
+        cols = -(-size1 * es // 16)
+        rows = size0
+    return -(-cols // 32) * -(-rows // 16)
+
 
 def workgroup_count(export, M, N):
     """Grid of an export for M x N outer tiles: what its count region returns."""
@@ -72,7 +91,7 @@ class HalExecutable:
 
     def add_export(self, name, block=(WORKGROUP_SIZE, 1, 1), shared_memory_size=None):
         if shared_memory_size is None:
-            shared_memory_size = EXPORTS[name].lds
+            shared_memory_size = 0 if name in PACK_EXPORTS else EXPORTS[name].lds
         ordinal = C.c_int32(-1)
         _check(self._lib.iree_amd_hal_executable_add_export(
             self._handle, name.encode(), block[0], block[1], block[2], shared_memory_size,
@@ -105,6 +124,19 @@ class HalExecutable:
             consts += [out_rows, out_cols]
         self.dispatch(name, workgroup_count(e, M, N), [lhs, rhs, out], consts, stream)
 
+    def pack(self, name, matrix, tiles, size0, size1, tile0, tile1, padding=0, stream=None):
+        """mi355x_pack_*: matrix (size0 x size1, dense) -> tiles; `padding` is the
+        bit pattern of the padding element."""
+        assert PACK_EXPORTS[name][1]
+        self.dispatch(name, pack_workgroup_count(name, size0, size1, tile0, tile1), [matrix, tiles],
+                      [size0, size1, tile0, tile1, padding], stream)
+
+    def unpack(self, name, tiles, matrix, size0, size1, tile0, tile1, stream=None):
+        """mi355x_unpack_*: tiles -> matrix (size0 x size1, dense)."""
+        assert not PACK_EXPORTS[name][1]
+        self.dispatch(name, pack_workgroup_count(name, size0, size1, tile0, tile1), [tiles, matrix],
+                      [size0, size1, tile0, tile1], stream)
+
     def close(self):
         if self._handle:
             self._lib.iree_amd_hal_executable_release(self._handle)
@@ -119,12 +151,12 @@ class HalExecutable:
 
 _MLIR_HEADER = """\
 // hal.executable.source for iree_amd/hal/mi355x_kernels_gfx950.co: the gfx950
-// mmt4d kernels as hand-written dispatches on a HIP device, after the
+// mmt4d, pack and unpack kernels as hand-written dispatches on a HIP device, after the
 // reference's samples/custom_dispatch/hip/kernels/example.mlir:16-118.
 // Written by iree_amd.hal_executable.mlir_source(); NOT compiled here (this
 // build has no iree-compile).
 //
-// Every export: bindings lhs (read only), rhs (read only), out; push constants
+// Every mmt4d export: bindings lhs (read only), rhs (read only), out; push constants
 // M, N, K (outer tile counts), K0, flags (0x100 = accumulate), and for
 // mi355x_mmt4d_unpack_* also out_rows, out_cols. The workload of a dispatch is
 // (M, N).
@@ -161,6 +193,41 @@ _MLIR_EXPORT = """\
   }}
 """
 
+_MLIR_PACK_EXPORT = """\
+  // {what}; push constants size0, size1, tile0, tile1{extra}; workload (size0, size1, tile0, tile1)
+  hal.executable.export public @{name} ordinal({ordinal})
+      layout(#hal.pipeline.layout<push_constants = {constants}, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer>
+        ]>
+      ]>) attributes {{
+    workgroup_size = [{wg} : index, 1 : index, 1 : index]
+  }} {{
+  ^bb0(%device: !hal.device, %size0: index, %size1: index, %tile0: index, %tile1: index):
+    %c1 = arith.constant 1 : index
+    %c16 = arith.constant 16 : index
+    %c32 = arith.constant 32 : index
+    %bytes = arith.constant {es} : index
+{extent}
+    %chunks = arith.ceildivui %row_bytes, %c16 : index
+    %bx = arith.ceildivui %chunks, %c32 : index
+    %by = arith.ceildivui {rows}, %c16 : index
+    %x = arith.muli %bx, %by : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }}
+"""
+
+_MLIR_PACK_EXTENT = """\
+    %o0 = arith.ceildivui %size0, %tile0 : index
+    %rows = arith.muli %o0, %tile0 : index
+    %o1 = arith.ceildivui %size1, %tile1 : index
+    %cols = arith.muli %o1, %tile1 : index
+    %row_bytes = arith.muli %cols, %bytes : index"""
+
+_MLIR_UNPACK_EXTENT = """\
+    %row_bytes = arith.muli %size1, %bytes : index"""
+
 _MLIR_FOOTER = """\
 }
 
@@ -181,5 +248,14 @@ def mlir_source():
         parts.append(_MLIR_EXPORT.format(
             name=e.name, ordinal=ordinal, constants=7 if "_unpack_" in e.name else 5,
             wg=WORKGROUP_SIZE, lds=e.lds, tile=e.tile))
+    ordinal = len(EXPORTS)
+    for name, (es, is_pack) in PACK_EXPORTS.items():
+        parts.append(_MLIR_PACK_EXPORT.format(
+            name=name, ordinal=ordinal, es=es, wg=WORKGROUP_SIZE, constants=5 if is_pack else 4,
+            what=("pack: in = matrix, out = tiles" if is_pack else "unpack: in = tiles, out = matrix"),
+            extra=", padding" if is_pack else "",
+            extent=_MLIR_PACK_EXTENT if is_pack else _MLIR_UNPACK_EXTENT,
+            rows="%rows" if is_pack else "%size0"))
+        ordinal += 1
     parts.append(_MLIR_FOOTER)
     return "".join(parts)

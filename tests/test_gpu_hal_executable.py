@@ -39,12 +39,16 @@ def test_export_table_matches_the_sources():
         assert f.read() == H.mlir_source()
     assert H.workgroup_count("mi355x_mmt4d_s8s8s32_t8", 9, 17) == 2 * 3
     assert H.workgroup_count("mi355x_mmt4d_s8s8s32_t4", 9, 17) == 3 * 5
+    # f16 8191 x 5001 -> 32 x 16 tiles: 256 x 313 tiles = 8192 rows of 626 chunks
+    assert H.pack_workgroup_count("mi355x_pack_16bit", 8191, 5001, 32, 16) == 20 * 512
+    assert H.pack_workgroup_count("mi355x_unpack_16bit", 8191, 5001, 32, 16) == 20 * 512
+    assert H.pack_workgroup_count("mi355x_unpack_32bit", 17, 9, 8, 4) == 1 * 2
 
 
 def test_code_object_is_built_and_names_every_export():
     with open(H.CODE_OBJECT, "rb") as f:
         image = f.read()
-    for name in H.EXPORTS:
+    for name in list(H.EXPORTS) + list(H.PACK_EXPORTS):
         assert name.encode() + b"\0" in image, name
 
 
@@ -124,6 +128,72 @@ def test_row_major_exports_equal_the_library_entry_point(uk, cuda, exe, name):
         torch.cuda.synchronize()
         assert np.array_equal(one.cpu().numpy().view(np.uint32), two.cpu().numpy().view(np.uint32)), (name, acc)
         assert not torch.equal(one, init)
+
+
+PACK_CASES = [  # size0, size1, tile0, tile1 (elements)
+    (1, 1, 1, 16), (33, 70, 32, 16), (100, 257, 8, 32), (64, 64, 32, 32), (17, 500, 16, 64),
+    (300, 33, 1, 16), (129, 1000, 32, 16)]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", sorted(H.PACK_EXPORTS))
+def test_pack_and_unpack_exports_match_the_closed_form(uk, cuda, exe, name):
+    """pack: out[o0][o1][t0][t1] = in[o0 t0 + i0][o1 t1 + i1] or the padding element
+    (the reference's own statement of it, tools/pack_test.c:36-70); unpack: the
+    inverse, elements outside the matrix untouched (tools/unpack_test.c:13-58).
+    Also bit-identical to the library's iree_amd_uk_pack / _unpack."""
+    import torch
+    es, is_pack = H.PACK_EXPORTS[name]
+    dt = {1: np.uint8, 2: np.uint16, 4: np.uint32}[es]
+    lib_type = {1: F.PACK_TYPE_I8I8, 2: F.PACK_TYPE_F16F16, 4: F.PACK_TYPE_F32F32}[es]
+    rng = np.random.default_rng(zlib.crc32(name.encode()))
+    for size0, size1, tile0, tile1 in PACK_CASES:
+        if tile1 * es % 16:
+            continue
+        o0, o1 = -(-size0 // tile0), -(-size1 // tile1)
+        pad = int(rng.integers(1, 1 << (8 * es)))
+        mat = rng.integers(0, 1 << (8 * es), (size0, size1), dtype=np.uint64).astype(dt)
+        padded = np.full((o0 * tile0, o1 * tile1), pad, dtype=dt)
+        padded[:size0, :size1] = mat
+        tiles = np.ascontiguousarray(padded.reshape(o0, tile0, o1, tile1).transpose(0, 2, 1, 3))
+        if is_pack:
+            src = torch.from_numpy(mat.view(np.uint8).reshape(-1).copy()).cuda()
+            got = torch.full((tiles.size * es,), 0xA5, dtype=torch.uint8, device=cuda)
+            ref = torch.full((tiles.size * es,), 0x5A, dtype=torch.uint8, device=cuda)
+            exe.pack(name, src, got, size0, size1, tile0, tile1, pad)
+            uk.pack(src, ref, size0, size1, o0, o1, tile0, tile1, pad, lib_type)
+            torch.cuda.synchronize()
+            assert np.array_equal(got.cpu().numpy(), tiles.view(np.uint8).reshape(-1)), (name, size0, size1, tile0, tile1)
+            assert torch.equal(got, ref)
+        else:
+            src = torch.from_numpy(tiles.view(np.uint8).reshape(-1).copy()).cuda()
+            # a destination with a guard row behind the matrix: it must stay as it was
+            got = torch.full(((size0 + 1) * size1 * es,), 0xA5, dtype=torch.uint8, device=cuda)
+            exe.unpack(name, src, got, size0, size1, tile0, tile1)
+            torch.cuda.synchronize()
+            out = got.cpu().numpy()
+            assert np.array_equal(out[:size0 * size1 * es], mat.view(np.uint8).reshape(-1)), (name, size0, size1, tile0, tile1)
+            assert (out[size0 * size1 * es:] == 0xA5).all()
+
+
+@pytest.mark.gpu
+def test_pack_export_round_trip_at_full_size(uk, cuda, exe):
+    """f16 8191 x 5001 <-> 32 x 16 tiles: the library's packed bytes, and the
+    round trip returns the source."""
+    import torch
+    from iree_amd import synth
+    R, Cc = 8191, 5001
+    o0, o1 = 256, 313
+    x = torch.from_numpy(synth.uniform_pm1_f16(1, R * Cc).view(np.int16)).cuda()
+    p1 = torch.empty(o0 * o1 * 512, dtype=torch.int16, device=cuda)
+    p2 = torch.empty_like(p1)
+    back = torch.zeros_like(x)
+    exe.pack("mi355x_pack_16bit", x, p1, R, Cc, 32, 16, 0)
+    uk.pack(x, p2, R, Cc, o0, o1, 32, 16, 0, F.PACK_TYPE_F16F16)
+    exe.unpack("mi355x_unpack_16bit", p1, back, R, Cc, 32, 16)
+    torch.cuda.synchronize()
+    assert torch.equal(p1, p2)
+    assert torch.equal(back, x)
 
 
 @pytest.mark.gpu
