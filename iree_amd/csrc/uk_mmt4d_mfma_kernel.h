@@ -305,51 +305,53 @@ __device__ __forceinline__ void mmt4d_mfma_body(const MfmaArgs a) {
   typedef out_t out4_t __attribute__((ext_vector_type(4), aligned(sizeof(out_t))));
 
   acc_t acc[WM][WN];
-  if constexpr (row_major_out) {
-   if (a.accumulate) {
-    // (rows and columns past the matrix edge are read from the last valid
-    // one: their accumulators are never stored)
+  // Initial accumulator values. Both variants run AFTER the first K-steps of
+  // operand loads have been issued, in the shadow of their latency: reading the
+  // result tile (accumulate flag) ...
+  auto load_acc = [&]() {
+    if constexpr (row_major_out) {
+      // (rows and columns past the matrix edge are read from the last valid
+      // one: their accumulators are never stored)
 #pragma unroll
-    for (int x = 0; x < WM; ++x) {
-      int row = (i_base + wm * WM + x) * R + acc_r;
-      row = row < a.out_rows ? row : a.out_rows - 1;
-      const out_t* src = (const out_t*)(a.out + (int64_t)row * a.out_stride_bytes);
+      for (int x = 0; x < WM; ++x) {
+        int row = (i_base + wm * WM + x) * R + acc_r;
+        row = row < a.out_rows ? row : a.out_rows - 1;
+        const out_t* src = (const out_t*)(a.out + (int64_t)row * a.out_stride_bytes);
 #pragma unroll
-      for (int y = 0; y < WN; ++y)
+        for (int y = 0; y < WN; ++y)
 #pragma unroll
-        for (int g = 0; g < kGroups; ++g) {
-          const int col = (j_base + wn * WN + y) * R + acc_c0(g);
-          if (col + 4 <= a.out_cols) {
-            const out4_t v4 = *(const out4_t*)(src + col);
+          for (int g = 0; g < kGroups; ++g) {
+            const int col = (j_base + wn * WN + y) * R + acc_c0(g);
+            if (col + 4 <= a.out_cols) {
+              const out4_t v4 = *(const out4_t*)(src + col);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) acc[x][y][4 * g + e] = v4[e];
-          } else {
+              for (int e = 0; e < 4; ++e) acc[x][y][4 * g + e] = v4[e];
+            } else {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              const int c = col + e < a.out_cols ? col + e : a.out_cols - 1;
-              acc[x][y][4 * g + e] = src[c];
+              for (int e = 0; e < 4; ++e) {
+                const int c = col + e < a.out_cols ? col + e : a.out_cols - 1;
+                acc[x][y][4 * g + e] = src[c];
+              }
             }
           }
+      }
+    } else {
+#pragma unroll
+      for (int x = 0; x < WM; ++x)
+#pragma unroll
+        for (int y = 0; y < WN; ++y) {
+          const int bi = i_base + wm * WM + x, bj = j_base + wn * WN + y;
+          int i = bi / kPerTile, j = bj / kPerTile;
+          i = i < a.M ? i : a.M - 1;
+          j = j < a.N ? j : a.N - 1;
+          const out_t* t = (const out_t*)(a.out + (int64_t)i * a.out_stride_bytes) + (int64_t)j * 1024 +
+                           (bi % kPerTile) * R * 32 + (bj % kPerTile) * R;
+#pragma unroll
+          for (int v = 0; v < kAccRegs; ++v) acc[x][y][v] = t[acc_row(v) * 32 + acc_col];
         }
     }
-   }
-  } else if (a.accumulate) {
-#pragma unroll
-    for (int x = 0; x < WM; ++x)
-#pragma unroll
-      for (int y = 0; y < WN; ++y) {
-        const int bi = i_base + wm * WM + x, bj = j_base + wn * WN + y;
-        int i = bi / kPerTile, j = bj / kPerTile;
-        i = i < a.M ? i : a.M - 1;
-        j = j < a.N ? j : a.N - 1;
-        const out_t* t = (const out_t*)(a.out + (int64_t)i * a.out_stride_bytes) + (int64_t)j * 1024 +
-                         (bi % kPerTile) * R * 32 + (bj % kPerTile) * R;
-#pragma unroll
-        for (int v = 0; v < kAccRegs; ++v) acc[x][y][v] = t[acc_row(v) * 32 + acc_col];
-      }
-  }
-  // (without the accumulate flag the accumulators are cleared after the first
-  // loads have been issued, in the shadow of their latency)
+  };
+  // ... or clearing them.
   auto clear_acc = [&]() {
 #pragma unroll
     for (int x = 0; x < WM; ++x)
@@ -436,7 +438,7 @@ __device__ __forceinline__ void mmt4d_mfma_body(const MfmaArgs a) {
     int read_slot = 0;                                // slot of K-step `done`
 #pragma unroll 1
     for (int ks = 0; ks < kPro; ++ks) issue_step(ks, ks);
-    if (!a.accumulate) clear_acc();
+    if (a.accumulate) load_acc(); else clear_acc();
     wait_vmcnt<(kPro - kSync) * kLoadsPerStep>();  // the first kSync K-steps have landed
     __builtin_amdgcn_s_barrier();                  // (bare, as in the loop below)
     read_frags(0, fa[0], fb[0]);
@@ -500,7 +502,7 @@ __device__ __forceinline__ void mmt4d_mfma_body(const MfmaArgs a) {
     // ---- short-K path: everything fits in the ring ------------------------
 #pragma unroll 1
     for (int ks = 0; ks < T; ++ks) issue_step(ks, ks);
-    if (!a.accumulate) clear_acc();
+    if (a.accumulate) load_acc(); else clear_acc();
     wait_vmcnt<0>();
     __syncthreads();
 #pragma unroll 1
