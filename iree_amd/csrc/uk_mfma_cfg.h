@@ -18,7 +18,11 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef int intx16 __attribute__((ext_vector_type(16)));
 
+// kStepUs: measured time in microseconds of one K-step (the instruction's K
+// extent) of a 256x256 macro tile with all compute units busy on MI355X; the
+// launcher's estimates of absolute time start from it.
 struct F16Cfg {
+  static constexpr float kStepUs = 0.40f;
   static constexpr int kRows = 32;     // the instruction's block is kRows x kRows
   typedef half8 frag_t;
   typedef floatx16 acc_t;
@@ -31,6 +35,7 @@ struct F16Cfg {
   }
 };
 struct BF16Cfg {
+  static constexpr float kStepUs = 0.40f;
   static constexpr int kRows = 32;     // the instruction's block is kRows x kRows
   typedef bf16x8 frag_t;
   typedef floatx16 acc_t;
@@ -50,6 +55,7 @@ struct BF16Cfg {
 // the smaller block costs less energy per flop (with all-zero operands both
 // run at 2.3-2.4).
 struct F16Cfg16 {
+  static constexpr float kStepUs = 0.69f;
   static constexpr int kRows = 16;
   typedef half8 frag_t;
   typedef floatx4 acc_t;
@@ -62,6 +68,7 @@ struct F16Cfg16 {
   }
 };
 struct BF16Cfg16 {
+  static constexpr float kStepUs = 0.69f;
   static constexpr int kRows = 16;
   typedef bf16x8 frag_t;
   typedef floatx4 acc_t;
@@ -94,6 +101,7 @@ struct BF16BF16Cfg : BF16Cfg {
 // and element e of lanes 32..63 form the k pair of the e-th of four
 // instructions; both operands pair the same way, so every k meets its partner.
 struct F32Cfg {
+  static constexpr float kStepUs = 1.75f;
   static constexpr int kRows = 32;     // the instruction's block is kRows x kRows
   typedef floatx4 frag_t;
   typedef floatx16 acc_t;
@@ -108,6 +116,7 @@ struct F32Cfg {
   }
 };
 struct S8Cfg {
+  static constexpr float kStepUs = 0.38f;
   static constexpr int kRows = 32;     // the instruction's block is kRows x kRows
   typedef int4v frag_t;
   typedef intx16 acc_t;
@@ -120,6 +129,7 @@ struct S8Cfg {
   }
 };
 struct F8Cfg {
+  static constexpr float kStepUs = 0.86f;
   static constexpr int kRows = 32;     // the instruction's block is kRows x kRows
   typedef int8v frag_t;
   typedef floatx16 acc_t;
@@ -132,6 +142,14 @@ struct F8Cfg {
     return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
   }
 };
+
+// The configuration that computes the same products with the accumulator type
+// as result type (partial sums of a K split are kept in it).
+template <typename Cfg> struct PartialSumCfg { typedef Cfg type; };
+template <> struct PartialSumCfg<F16F16Cfg16> { typedef F16Cfg16 type; };
+template <> struct PartialSumCfg<BF16BF16Cfg16> { typedef BF16Cfg16 type; };
+template <> struct PartialSumCfg<F16F16Cfg> { typedef F16Cfg type; };
+template <> struct PartialSumCfg<BF16BF16Cfg> { typedef BF16Cfg type; };
 
 }  // namespace uk
 

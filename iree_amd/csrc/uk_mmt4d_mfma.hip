@@ -8,7 +8,117 @@
 #include "uk_mmt4d_mfma_kernel.h"
 #include "uk_mmt4d_mfma_launch.h"
 
+#include <mutex>
+#include <vector>
+
 namespace uk {
+namespace {
+
+// Sum of the partial results of a K split. One thread owns 4 consecutive
+// columns of one tile row: it adds the slices in order (after the old result,
+// when accumulating) and writes what the matmul kernel's epilogue would have.
+template <typename AccT, typename OutT>
+__global__ __launch_bounds__(256) void ksplit_reduce_kernel(KSplitReduceArgs r) {
+  typedef AccT acc4_t __attribute__((ext_vector_type(4)));
+  typedef OutT out4_t __attribute__((ext_vector_type(4), aligned(sizeof(OutT))));
+  const int64_t groups = (int64_t)r.M * r.N * 256;
+  const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (g >= groups) return;
+  const int64_t tile = g >> 8;
+  const int in_tile = (int)(g & 255);
+  const int row_in_tile = in_tile >> 3, col_in_tile = (in_tile & 7) * 4;
+  const int i = (int)(tile / r.N), j = (int)(tile % r.N);
+  OutT* dst;
+  int valid = 4;   // leading elements of the group that exist in the result
+  if (r.row_major_out) {
+    const int row = i * 32 + row_in_tile, col = j * 32 + col_in_tile;
+    if (row >= r.out_rows || col >= r.out_cols) return;
+    valid = r.out_cols - col < 4 ? r.out_cols - col : 4;
+    dst = (OutT*)((char*)r.out + (int64_t)row * r.out_stride_bytes) + col;
+  } else {
+    dst = (OutT*)((char*)r.out + (int64_t)i * r.out_stride_bytes) + (int64_t)j * 1024 + in_tile * 4;
+  }
+  acc4_t sum = {0, 0, 0, 0};
+  if (r.accumulate) {
+    if (valid == 4) {
+      const out4_t old = *(const out4_t*)dst;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) sum[e] = (AccT)old[e];
+    } else {
+      for (int e = 0; e < valid; ++e) sum[e] = (AccT)dst[e];
+    }
+  }
+  const acc4_t* p = (const acc4_t*)r.partials + g;
+  for (int sl = 0; sl < r.slices; ++sl) sum += p[(int64_t)sl * groups];
+  out4_t v;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    if constexpr (std::is_floating_point<AccT>::value)
+      v[e] = r.row_major_out ? (OutT)(sum[e] * r.out_scale) : (OutT)sum[e];
+    else
+      v[e] = (OutT)sum[e];
+  }
+  if (valid == 4) {
+    *(out4_t*)dst = v;
+  } else {
+    for (int e = 0; e < valid; ++e) dst[e] = v[e];
+  }
+}
+
+}  // namespace
+
+void* ksplit_scratch(hipStream_t s, size_t bytes) {
+  struct Entry { int device; hipStream_t stream; void* ptr; size_t bytes; };
+  static std::mutex mutex;
+  static std::vector<Entry> entries;
+  constexpr size_t kMaxBytes = (size_t)512 << 20;   // larger problems run unsplit
+  constexpr size_t kMaxEntries = 64;
+  if (bytes == 0 || bytes > kMaxBytes) return nullptr;
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+  std::lock_guard<std::mutex> lock(mutex);
+  for (Entry& e : entries) {
+    if (e.device != device || e.stream != s) continue;
+    if (e.bytes >= bytes) return e.ptr;
+    // Too small: earlier work on the stream may still use it, so it is freed
+    // in stream order; the replacement is twice what is asked for.
+    void* bigger = nullptr;
+    const size_t want = bytes * 2 < kMaxBytes ? bytes * 2 : kMaxBytes;
+    if (hipMalloc(&bigger, want) != hipSuccess || !bigger) { (void)hipGetLastError(); return nullptr; }
+    if (hipFreeAsync(e.ptr, s) != hipSuccess) { (void)hipGetLastError(); (void)hipFree(e.ptr); }
+    e.ptr = bigger;
+    e.bytes = want;
+    return e.ptr;
+  }
+  if (entries.size() >= kMaxEntries) {
+    // (streams come and go: drop the oldest buffer; hipFree waits for the device)
+    (void)hipFree(entries.front().ptr);
+    entries.erase(entries.begin());
+  }
+  void* ptr = nullptr;
+  const size_t want = bytes < ((size_t)16 << 20) ? (size_t)16 << 20 : bytes;
+  if (hipMalloc(&ptr, want) != hipSuccess || !ptr) { (void)hipGetLastError(); return nullptr; }
+  entries.push_back({device, s, ptr, want});
+  return ptr;
+}
+
+int launch_ksplit_reduce(const KSplitReduceArgs& r, hipStream_t s) {
+  const int64_t groups = (int64_t)r.M * r.N * 256;
+  const int64_t blocks = (groups + 255) / 256;
+  if (blocks < 1 || blocks > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  const dim3 grid((unsigned)blocks), block(256);
+  if (!r.acc_is_float) {
+    hipLaunchKernelGGL((ksplit_reduce_kernel<int32_t, int32_t>), grid, block, 0, s, r);
+  } else if (r.out_kind == 1) {
+    hipLaunchKernelGGL((ksplit_reduce_kernel<float, _Float16>), grid, block, 0, s, r);
+  } else if (r.out_kind == 2) {
+    hipLaunchKernelGGL((ksplit_reduce_kernel<float, __bf16>), grid, block, 0, s, r);
+  } else {
+    hipLaunchKernelGGL((ksplit_reduce_kernel<float, float>), grid, block, 0, s, r);
+  }
+  return check_hip(hipGetLastError(), "ksplit_reduce launch");
+}
+
 namespace {
 
 // mfma_k: K extent of the instruction the call runs on. f16 / bf16 use the
@@ -79,6 +189,7 @@ int make_args(const iree_amd_uk_mmt4d_params_t& p, int out_elem_bytes, bool silu
   a.ksteps = (int)(k_elems / sv.mfma_k);
   a.tail_tiles = (int)((k_elems % sv.mfma_k) / p.K0);
   a.tiles_m = a.tiles_n = 0;
+  a.k_slices = 0; a.slice_ksteps = 0; a.slice_out_bytes = 0;
   a.accumulate = (p.flags & IREE_AMD_UK_FLAG_MMT4D_ACCUMULATE) != 0;
   a.k0_div = sv.mfma_k / p.K0;
   a.row_major_out = 0; a.out_rows = a.out_cols = 0;

@@ -87,6 +87,11 @@ struct MfmaArgs {
   float gate_scale, up_scale, inv_out_scale;
   // row-major result of a float type only: factor applied on the store
   float out_scale;
+  // K split (launch side): k_slices > 1 = workgroup row blockIdx.y computes
+  // K-steps [y * slice_ksteps, ...) into the tiled partial result
+  // out + y * slice_out_bytes
+  int k_slices, slice_ksteps;
+  int64_t slice_out_bytes;
 };
 
 namespace {
@@ -176,15 +181,16 @@ __device__ __forceinline__ void tile_coord(int bid, int tiles_m, int tiles_n,
 // left-hand-side tiles 32x16 of the next matmul (one byte per element).
 // kForm: which of the operand forms the instance is compiled for: 0 = packed
 // left-hand side, tiled result; 1 = row-major result; 2 = row-major left-hand
-// side and result. (An instance compiled for one form has constant step sizes
+// side and result; 3 = row-major left-hand side, tiled result (the partial
+// sums of a K split). (An instance compiled for one form has constant step sizes
 // in its loop and one epilogue: measured 2 % (f16) to 6 % (i8) faster at 4096^3
 // than one that reads the form from its arguments.)
 template <typename Cfg, int WM, int WN, int kRing, int kSync, bool kSiluMul = false, int kWavesN = 2,
           int kForm = 0>
 __device__ __forceinline__ void mmt4d_mfma_body(const MfmaArgs a) {
-  static_assert(kForm >= 0 && kForm <= 2 && (!kSiluMul || kForm == 0), "unknown operand form");
-  constexpr bool lhs_row_major = kForm == 2;
-  constexpr bool row_major_out = kForm >= 1;
+  static_assert(kForm >= 0 && kForm <= 3 && (!kSiluMul || kForm == 0), "unknown operand form");
+  constexpr bool lhs_row_major = kForm >= 2;
+  constexpr bool row_major_out = kForm == 1 || kForm == 2;
   // kSwap: the MFMAs are issued with the operands exchanged (B fragment first),
   // so that a block's accumulator holds the TRANSPOSE in the instruction's
   // layout and a lane owns 4 consecutive COLUMNS of one row per register group

@@ -24,6 +24,27 @@ int launch_mfma_silu_f16(const MfmaArgs& a, hipStream_t s);
 int launch_mfma_silu_bf16(const MfmaArgs& a, hipStream_t s);
 int launch_mfma_silu_f8(const MfmaArgs& a, hipStream_t s);
 
+// Sums the partial results of a K split (tiled, accumulator type) in slice
+// order into the result, tiled or row-major: what the kernel's own epilogue
+// would have written (defined in uk_mmt4d_mfma.hip).
+struct KSplitReduceArgs {
+  const void* partials;      // slices x M x N tiles of 32x32 accumulator elements
+  int slices;
+  int M, N;                  // outer tile counts
+  void* out;                 // offset applied
+  int64_t out_stride_bytes;
+  int accumulate, row_major_out, out_rows, out_cols;
+  float out_scale;
+  int acc_is_float;          // else int32
+  int out_kind;              // 0 = accumulator type, 1 = f16, 2 = bf16
+};
+int launch_ksplit_reduce(const KSplitReduceArgs& r, hipStream_t s);
+// Device memory for the partial sums of a K split on stream `s` of the current
+// device: one buffer per stream, kept and reused by later calls (work on one
+// stream is ordered, so they cannot overlap), grown when a call needs more.
+// nullptr when it cannot be had (the call then runs unsplit).
+void* ksplit_scratch(hipStream_t s, size_t bytes);
+
 namespace {
 
 // kOcc: waves per SIMD the register allocation must leave room for (2 = two
@@ -34,23 +55,60 @@ __global__ __launch_bounds__(128 * kWavesN, kOcc) void mmt4d_mfma_kernel(MfmaArg
   mmt4d_mfma_body<Cfg, WM, WN, kRing, kSync, kSiluMul, kWavesN, kForm>(a);
 }
 
+// K split: workgroup row blockIdx.y multiplies its slice of K into its own
+// tiled partial result.
+template <typename Cfg, int WM, int WN, int kRing, int kSync, int kOcc, int kWavesN, int kForm>
+__global__ __launch_bounds__(128 * kWavesN, kOcc) void mmt4d_mfma_ksplit_kernel(MfmaArgs a) {
+  static_assert(kForm == 0 || kForm == 3, "partial results are tiled");
+  // bytes of one K-step in an outer row of packed tiles / in a row of a row-major matrix
+  constexpr int64_t kPackedStep = (32 / Cfg::kRows) * Cfg::kSub * 1024;
+  constexpr int64_t kRowStep = (64 / Cfg::kRows) * 16 * Cfg::kSub;
+  const int slice = blockIdx.y;
+  const int first = slice * a.slice_ksteps;
+  a.lhs += first * (kForm == 3 ? kRowStep : kPackedStep);
+  a.rhs += first * kPackedStep;
+  a.out += slice * a.slice_out_bytes;
+  if (slice == a.k_slices - 1) {
+    a.ksteps -= first;
+  } else {
+    a.ksteps = a.slice_ksteps;
+    a.tail_tiles = 0;
+  }
+  mmt4d_mfma_body<Cfg, WM, WN, kRing, kSync, false, kWavesN, kForm>(a);
+}
+
 template <typename Cfg, int WM, int WN, int kRing, int kSync, int kOcc, bool kSiluMul, int kWavesN,
           int kForm>
 int launch_form(const MfmaArgs& a, unsigned blocks, hipStream_t s) {
   constexpr int lds_bytes = mmt4d_mfma_lds_bytes<Cfg, WM, WN, kRing, kWavesN>();
   static_assert(lds_bytes <= 160 * 1024, "LDS ring exceeds 160 KiB");
-  auto kernel = mmt4d_mfma_kernel<Cfg, WM, WN, kRing, kSync, kOcc, kSiluMul, kWavesN, kForm>;
+  // (form 3 exists only as the K-split kernel, and partial sums only in the
+  // accumulator type)
+  constexpr bool kCanSplit = !kSiluMul && (kForm == 0 || kForm == 3) &&
+                             std::is_same<typename PartialSumCfg<Cfg>::type, Cfg>::value;
+  void (*kernel)(MfmaArgs) = nullptr;
+  unsigned slices = 1;
+  if (a.k_slices > 1) {
+    if constexpr (kCanSplit) {
+      kernel = mmt4d_mfma_ksplit_kernel<Cfg, WM, WN, kRing, kSync, kOcc, kWavesN, kForm>;
+      slices = (unsigned)a.k_slices;
+    }
+  } else {
+    if constexpr (kForm != 3) kernel = mmt4d_mfma_kernel<Cfg, WM, WN, kRing, kSync, kOcc, kSiluMul, kWavesN, kForm>;
+  }
+  if (!kernel) return IREE_AMD_UK_STATUS_NOT_FOUND;
   // The attribute belongs to the kernel on ONE device: set it once per device
   // ordinal (a benign race: the call is idempotent).
-  static unsigned long long attr_set_on = 0;
+  static unsigned long long attr_set_on[2] = {0, 0};
+  unsigned long long& set_on = attr_set_on[slices > 1];
   int dev = 0;
   UK_RETURN_IF_HIP(hipGetDevice(&dev));
-  if (dev < 0 || dev >= 64 || !((attr_set_on >> dev) & 1)) {
+  if (dev < 0 || dev >= 64 || !((set_on >> dev) & 1)) {
     UK_RETURN_IF_HIP(hipFuncSetAttribute((const void*)kernel,
                                          hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes));
-    if (dev >= 0 && dev < 64) attr_set_on |= 1ull << dev;
+    if (dev >= 0 && dev < 64) set_on |= 1ull << dev;
   }
-  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(128 * kWavesN), lds_bytes, s, a);
+  hipLaunchKernelGGL(kernel, dim3(blocks, slices), dim3(128 * kWavesN), lds_bytes, s, a);
   return check_hip(hipGetLastError(), "mmt4d_mfma launch");
 }
 
@@ -67,13 +125,79 @@ int launch_variant(const MfmaArgs& a0, hipStream_t s) {
   if (blocks > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
   // one kernel instance per operand form (the forms the entry points produce)
   if constexpr (!kSiluMul) {
+    if (a.k_slices > 1 && a.row_major_out) return IREE_AMD_UK_STATUS_NOT_FOUND;
     if (a.lhs_row_major && a.row_major_out)
       return launch_form<Cfg, WM, WN, kRing, kSync, kOcc, kSiluMul, kWavesN, 2>(a, (unsigned)blocks, s);
     if (a.row_major_out)
       return launch_form<Cfg, WM, WN, kRing, kSync, kOcc, kSiluMul, kWavesN, 1>(a, (unsigned)blocks, s);
   }
+  if constexpr (!kSiluMul) {
+    if (a.lhs_row_major)   // (tiled result: the partial sums of a K split)
+      return launch_form<Cfg, WM, WN, kRing, kSync, kOcc, kSiluMul, kWavesN, 3>(a, (unsigned)blocks, s);
+  }
   if (a.lhs_row_major || a.row_major_out) return IREE_AMD_UK_STATUS_NOT_FOUND;
   return launch_form<Cfg, WM, WN, kRing, kSync, kOcc, kSiluMul, kWavesN, 0>(a, (unsigned)blocks, s);
+}
+
+// The four macro tiles (in outer tiles of 32 rows: 8x8, 8x4, 4x8, 4x4) with
+// their LDS rings: 8 K-steps and a barrier every 2 for the single-occupancy
+// tiles (fp8 and the 16-row shapes, whose K-step is twice as large: 5 and every
+// step), 6 (wide: 3) for the double-occupancy ones.
+template <typename Cfg, bool kSiluMul>
+int launch_by_index(int v, const MfmaArgs& b, hipStream_t s) {
+  constexpr int S = 32 / Cfg::kRows;
+  constexpr bool kWide = Cfg::kSub == 2 || S == 2;
+  switch (v) {
+    case 0: return launch_variant<Cfg, 4 * S, 4 * S, kWide ? 5 : 8, kWide ? 1 : 2, 1, kSiluMul>(b, s);
+    case 1: return launch_variant<Cfg, 4 * S, 2 * S, kWide ? 3 : 6, kWide ? 1 : 2, 2, kSiluMul>(b, s);
+    case 2: return launch_variant<Cfg, 2 * S, 4 * S, kWide ? 3 : 6, kWide ? 1 : 2, 2, kSiluMul>(b, s);
+    default: return launch_variant<Cfg, 2 * S, 2 * S, S == 2 ? 4 : 8, S == 2 ? 1 : 2, 1, kSiluMul>(b, s);
+  }
+}
+
+// K split: `slices` workgroup rows multiply one slice of K each into tiled
+// partial results in the stream's scratch buffer, which a second kernel
+// sums in slice order into the result (deterministic; integer results are
+// those of the unsplit kernel, float results differ from it in the order of
+// the additions only). Returns NOT_FOUND when the scratch memory cannot be had
+// (the caller then runs unsplit).
+template <typename Cfg>
+int launch_k_split(const MfmaArgs& a, int v, int slices, hipStream_t s) {
+  typedef typename PartialSumCfg<Cfg>::type PCfg;
+  typedef typename PCfg::out_t acc_elem_t;
+  const int slice_ksteps = (a.ksteps + slices - 1) / slices;
+  slices = (a.ksteps + slice_ksteps - 1) / slice_ksteps;      // (no empty last slice)
+  if (slices < 2) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  const int64_t slice_bytes = (int64_t)a.M * a.N * 1024 * (int64_t)sizeof(acc_elem_t);
+  void* scratch = ksplit_scratch(s, (size_t)(slice_bytes * slices));
+  if (!scratch) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  MfmaArgs p = a;
+  p.out = (char*)scratch;
+  p.out_stride_bytes = (int64_t)a.N * 1024 * (int64_t)sizeof(acc_elem_t);
+  p.row_major_out = 0;
+  p.accumulate = 0;
+  p.out_scale = 1.0f;
+  p.k_slices = slices;
+  p.slice_ksteps = slice_ksteps;
+  p.slice_out_bytes = slice_bytes;
+  int st = launch_by_index<PCfg, false>(v, p, s);
+  if (!st) {
+    KSplitReduceArgs r;
+    r.partials = scratch;
+    r.slices = slices;
+    r.M = a.M; r.N = a.N;
+    r.out = a.out;
+    r.out_stride_bytes = a.out_stride_bytes;
+    r.accumulate = a.accumulate;
+    r.row_major_out = a.row_major_out;
+    r.out_rows = a.out_rows; r.out_cols = a.out_cols;
+    r.out_scale = a.out_scale;
+    r.acc_is_float = std::is_floating_point<acc_elem_t>::value;
+    r.out_kind = std::is_same<typename Cfg::out_t, acc_elem_t>::value ? 0
+                 : std::is_same<typename Cfg::out_t, _Float16>::value ? 1 : 2;
+    st = launch_ksplit_reduce(r, s);
+  }
+  return st;
 }
 
 template <typename Cfg, bool kSiluMul = false>
@@ -109,9 +233,9 @@ int launch_cfg(const MfmaArgs& a, hipStream_t s) {
                                       {2, 4, 2, kEffAlone, kEffFull},
                                       {2, 2, 2, 0.7, 0.75}};
   // cost of variant v on an M x N (outer tiles) problem
-  auto cost_of = [&](int v, int64_t M, int64_t N) -> double {
+  auto cost_of = [&](int v, int64_t M, int64_t N, int64_t k_slices = 1) -> double {
     const Variant& t = variants[v];
-    const int64_t tiles = ceil_div(M, (int64_t)2 * t.wm) * ceil_div(N, (int64_t)2 * t.wn);
+    const int64_t tiles = ceil_div(M, (int64_t)2 * t.wm) * ceil_div(N, (int64_t)2 * t.wn) * k_slices;
     const int64_t slots = (int64_t)t.occ * cus;
     const double work = t.wm * t.wn;
     double cost = (double)(tiles / slots) * t.occ * work / t.eff_full;
@@ -132,16 +256,39 @@ int launch_cfg(const MfmaArgs& a, hipStream_t s) {
     *out_cost = best_cost;
     return best;
   };
-  auto launch = [&](int v, const MfmaArgs& b) -> int {
-    switch (v) {
-      case 0: return launch_variant<Cfg, 4 * S, 4 * S, kWide ? 5 : 8, kWide ? 1 : 2, 1, kSiluMul>(b, s);
-      case 1: return launch_variant<Cfg, 4 * S, 2 * S, kWide ? 3 : 6, kWide ? 1 : 2, 2, kSiluMul>(b, s);
-      case 2: return launch_variant<Cfg, 2 * S, 4 * S, kWide ? 3 : 6, kWide ? 1 : 2, 2, kSiluMul>(b, s);
-      default: return launch_variant<Cfg, 2 * S, 2 * S, S == 2 ? 4 : 8, S == 2 ? 1 : 2, 1, kSiluMul>(b, s);
-    }
-  };
+  auto launch = [&](int v, const MfmaArgs& b) -> int { return launch_by_index<Cfg, kSiluMul>(v, b, s); };
   double best_cost = 0;
   const int best = pick(a.M, a.N, &best_cost);
+  // Few macro tiles and a long K (a few hundred rows against a wide K, as in the
+  // down projection of an MLP at small batch) leave most compute units idle:
+  // K is then split over workgroup rows. Estimated times in microseconds: cost
+  // units (block rows of MFMAs per K-step) x K-steps x the measured time of a
+  // unit, plus, for a split, the second launch and the traffic of the partial
+  // sums (written once, read once, at about 3 TB/s).
+  if constexpr (!kSiluMul) {
+    const Variant& bv = variants[best];
+    const int64_t best_tiles = ceil_div((int64_t)a.M, (int64_t)2 * bv.wm) * ceil_div((int64_t)a.N, (int64_t)2 * bv.wn);
+    if (a.k_slices == 0 && a.ksteps >= 64 && best_tiles * 2 <= (int64_t)bv.occ * cus) {
+      const double unit_us = Cfg::kStepUs / 16.0;
+      const double out_mb = (double)a.M * a.N * 4096.0 / 1e6;
+      double best_us = best_cost * a.ksteps * unit_us * 0.9;    // a split must win by 10 %
+      int split_v = -1, split_n = 0;
+      for (int v = 0; v < 4; ++v)
+        for (int n = 2; n <= 8; ++n) {
+          if (a.ksteps / n < 24) break;
+          const int64_t tiles = ceil_div((int64_t)a.M, (int64_t)2 * variants[v].wm) *
+                                ceil_div((int64_t)a.N, (int64_t)2 * variants[v].wn) * n;
+          if (tiles > (int64_t)variants[v].occ * cus) break;     // at most one round
+          const double us = cost_of(v, a.M, a.N, n) * ceil_div((int64_t)a.ksteps, (int64_t)n) * unit_us + 6.0 +
+                            (n + 1 + (a.accumulate ? 1 : 0)) * out_mb / 3.0;
+          if (us < best_us) { best_us = us; split_v = v; split_n = n; }
+        }
+      if (split_n > 1) {
+        const int st = launch_k_split<Cfg>(a, split_v, split_n, s);
+        if (st != IREE_AMD_UK_STATUS_NOT_FOUND) return st;
+      }
+    }
+  }
   // A last round that fills only part of the device costs a whole round. When
   // the large tile leaves such a round, the longer outer dimension is split:
   // whole rounds of 256x256 tiles first, the remaining rows or columns as a

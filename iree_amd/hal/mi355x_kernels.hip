@@ -78,6 +78,9 @@ __device__ __forceinline__ void hal_mmt4d(const void* lhs, const void* rhs, void
   a.out_rows = out_rows;
   a.out_cols = out_cols;
   a.lhs_row_major = 0;
+  a.k_slices = 0;
+  a.slice_ksteps = 0;
+  a.slice_out_bytes = 0;
   a.k0_div = Cfg::kMfmaK / K0;
   a.gate_scale = a.up_scale = a.inv_out_scale = a.out_scale = 1.0f;
   // a grid larger than the tile count (a count region that rounds up) is harmless

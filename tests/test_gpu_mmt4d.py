@@ -546,3 +546,80 @@ def test_i8_shapes_that_split_into_two_launches(uk, cuda, M, N):
         fn(c)
         torch.cuda.synchronize()
         assert np.array_equal(c.cpu().numpy().reshape(M, N), want)
+
+
+# Few macro tiles and a long K: the launcher splits K over workgroup rows and
+# sums the partial results in slice order.
+KSPLIT_TYPES = [(F.MMT4D_TYPE_S8S8S32, 16, 32), (F.MMT4D_TYPE_F16F16F32, 8, 32),
+                (F.MMT4D_TYPE_F16F16F16, 16, 32), (F.MMT4D_TYPE_BF16BF16F32, 8, 32),
+                (F.MMT4D_TYPE_F8E4M3F8E4M3F32, 16, 64), (F.MMT4D_TYPE_F32F32F32, 4, 8)]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("type_flag,K0,mfma_k", KSPLIT_TYPES)
+def test_k_split_shapes_bit_exact(uk, cuda, type_flag, K0, mfma_k):
+    """Outer shapes of a few tiles with 70 to 200 matrix-core K-steps (plus a
+    partial last one where K0 allows it), tiled result, with and without
+    accumulate: the bits of the oracle (every partial sum is exact)."""
+    rng = np.random.default_rng(9100 + type_flag + K0)
+    tps = mfma_k // K0
+    for (M, N, steps), acc in itertools.product([(8, 16, 128), (3, 5, 70), (1, 40, 200)], (False, True)):
+        K = steps * tps + (1 if tps > 1 else 0)
+        case = ukref.Mmt4dCase(rng, type_flag, M, N, K, 32, 32, K0, accumulate=acc)
+        got = gpucase.run_mmt4d(case)
+        want = case.run_oracle(ukref.F16_IEEE)
+        assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), (hex(type_flag), (M, N, K), acc)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("type_flag,K0,mfma_k,dt", [(F.MMT4D_TYPE_S8S8S32, 16, 32, np.int8),
+                                                    (F.MMT4D_TYPE_F16F16F32, 8, 32, np.float16),
+                                                    (F.MMT4D_TYPE_F32F32F32, 4, 8, np.float32)])
+@pytest.mark.parametrize("accumulate", [False, True])
+def test_k_split_row_major_forms_equal_the_three_call_chain(uk, cuda, type_flag, K0, mfma_k, dt, accumulate):
+    """The fused forms on a K-split shape (200 x 333, 96 K-steps) with random
+    data: mmt4d_unpack and matmul_packed_rhs give the bits of pack + mmt4d +
+    unpack (all three split alike and add the slices in the same order), and
+    within the stated tolerance of a float64 matmul."""
+    import torch
+    M, N, K = 200, 333, 96 * mfma_k
+    M1, N1, K1 = -(-M // 32), -(-N // 32), K // K0
+    rng = np.random.default_rng(77)
+    if dt is np.int8:
+        A = rng.integers(-128, 128, (M, K), dtype=np.int8)
+        B = rng.integers(-128, 128, (N, K), dtype=np.int8)
+        odt, ptype = torch.int32, F.PACK_TYPE_I8I8
+    else:
+        A = (rng.standard_normal((M, K)) / 8).astype(dt)
+        B = (rng.standard_normal((N, K)) / 8).astype(dt)
+        odt, ptype = torch.float32, (F.PACK_TYPE_F16F16 if dt is np.float16 else F.PACK_TYPE_F32F32)
+    a_dev, b_dev = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda()
+    lhs = torch.empty(M1 * K1 * 32 * K0, dtype=a_dev.dtype, device=cuda)
+    rhs = torch.empty(N1 * K1 * 32 * K0, dtype=a_dev.dtype, device=cuda)
+    uk.pack(a_dev, lhs, M, K, M1, K1, 32, K0, 0, ptype)
+    uk.pack(b_dev, rhs, N, K, N1, K1, 32, K0, 0, ptype)
+    init = torch.from_numpy(rng.integers(-40, 40, M * N).astype(np.int32)).cuda().to(odt)
+    flags = type_flag | (F.MMT4D_ACCUMULATE if accumulate else 0)
+    utype = F.UNPACK_TYPE_I32I32 if odt == torch.int32 else F.UNPACK_TYPE_F32F32
+    # three calls (the tiled accumulator starts from the packed initial result)
+    tiled = torch.zeros(M1 * N1 * 1024, dtype=odt, device=cuda)
+    uk.pack(init, tiled, M, N, M1, N1, 32, 32, 0, F.PACK_TYPE_I32I32 if odt == torch.int32 else F.PACK_TYPE_F32F32)
+    uk.mmt4d(lhs, rhs, tiled, M1, N1, K1, 32, 32, K0, flags)
+    three = init.clone()
+    uk.unpack(tiled, three, M1, N1, 32, 32, M, N, utype)
+    fused = init.clone()
+    uk.mmt4d_unpack(lhs, rhs, fused, M, N, M1, N1, K1, K0, flags)
+    one = init.clone()
+    uk.matmul_packed_rhs(a_dev, rhs, one, M, N, K, K0, flags)
+    torch.cuda.synchronize()
+    t3, tf, t1 = (x.cpu().numpy().view(np.uint32) for x in (three, fused, one))
+    assert np.array_equal(tf, t3)
+    assert np.array_equal(t1, t3)
+    want = A.astype(np.float64) @ B.astype(np.float64).T
+    if accumulate:
+        want = want + init.cpu().numpy().reshape(M, N).astype(np.float64)
+    got = three.cpu().numpy().reshape(M, N).astype(np.float64)
+    if dt is np.int8:
+        assert np.array_equal(got, want)
+    else:
+        assert np.all(np.abs(got - want) <= ATOL + RTOL * np.abs(want))
