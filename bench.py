@@ -339,6 +339,18 @@ def extras(args, torch, iree_amd, F, synth, lhs, rhs, out, ex):
                     steps, warm)
     ex["mmt4d_f16_accumulate_tflops"] = round(flops / t / 1e12, 2)
 
+    # A shape of few macro tiles and a long K (256 rows of activations against a
+    # 4096 x 14336 down projection): K is split over workgroup rows.
+    Ms, Ns, Ks = 256, 4096, 14336
+    ls = torch.from_numpy(synth.normal_f16(7, Ms * Ks, scale=1 / 64).view(np.int16)).cuda()
+    rs = torch.from_numpy(synth.normal_f16(8, Ns * Ks, scale=1 / 64).view(np.int16)).cuda()
+    os_ = torch.empty(Ms * Ns, dtype=torch.float32, device="cuda")
+    _, t = gpu_time(torch, lambda: iree_amd.mmt4d(ls, rs, os_, Ms // 32, Ns // 32, Ks // 8, 32, 32, 8,
+                                                  F.MMT4D_TYPE_F16F16F32), steps, warm)
+    ex["mmt4d_f16_m256_n4096_k14336_us"] = round(t * 1e6, 1)
+    ex["mmt4d_f16_m256_n4096_k14336_tflops"] = round(2.0 * Ms * Ns * Ks / t / 1e12, 1)
+    del ls, rs, os_
+
     # The same f16 mmt4d dispatched from the code object a HAL executable on a
     # HIP device links (hipModuleLaunchKernel, bindings + 32-bit push constants)
     from iree_amd import hal_executable

@@ -158,7 +158,10 @@ typedef struct iree_amd_uk_mmt4d_params_t {
   const uint64_t* cpu_data; /* accepted, ignored */
 } iree_amd_uk_mmt4d_params_t;
 
-/* Replaces REF mmt4d.h:14-21 / mmt4d.c:151-177 (iree_uk_mmt4d). */
+/* Replaces REF mmt4d.h:14-21 / mmt4d.c:151-177 (iree_uk_mmt4d).
+ * A matrix-core call of few macro tiles and a long K splits K and keeps the
+ * partial sums in a scratch buffer the library allocates once per stream
+ * (16 to 512 MiB, never freed); every other call allocates nothing. */
 IREE_AMD_UK_EXPORT int iree_amd_uk_mmt4d(
     const void* lhs_buffer, iree_amd_uk_index_t lhs_offset,
     iree_amd_uk_index_t lhs_stride0, const void* rhs_buffer,

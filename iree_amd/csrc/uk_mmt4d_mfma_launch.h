@@ -1,5 +1,6 @@
 // Launch side of the matrix-core mmt4d kernels: the __global__ wrapper, the
-// choice of the macro tile for a problem and the split of a partial last round.
+// choice of the macro tile for a problem, the split of a partial last round
+// and the split of K for problems of few macro tiles.
 // Included by the translation units that instantiate the kernels of one
 // element-type tuple each (uk_mmt4d_mfma_inst_*.hip), so that they compile in
 // parallel; uk_mmt4d_mfma.hip calls them through the functions declared here.
