@@ -21,7 +21,7 @@ template <typename AccT, typename OutT>
 __global__ __launch_bounds__(256) void ksplit_reduce_kernel(KSplitReduceArgs r) {
   typedef AccT acc4_t __attribute__((ext_vector_type(4)));
   typedef OutT out4_t __attribute__((ext_vector_type(4), aligned(sizeof(OutT))));
-  const int64_t groups = (int64_t)r.M * r.N * 256;
+  const int64_t groups = r.flat_elems > 0 ? r.flat_elems / 4 : (int64_t)r.M * r.N * 256;
   const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (g >= groups) return;
   const int64_t tile = g >> 8;
@@ -30,7 +30,9 @@ __global__ __launch_bounds__(256) void ksplit_reduce_kernel(KSplitReduceArgs r) 
   const int i = (int)(tile / r.N), j = (int)(tile % r.N);
   OutT* dst;
   int valid = 4;   // leading elements of the group that exist in the result
-  if (r.row_major_out) {
+  if (r.flat_elems > 0) {
+    dst = (OutT*)r.out + g * 4;
+  } else if (r.row_major_out) {
     const int row = i * 32 + row_in_tile, col = j * 32 + col_in_tile;
     if (row >= r.out_rows || col >= r.out_cols) return;
     valid = r.out_cols - col < 4 ? r.out_cols - col : 4;
@@ -103,7 +105,7 @@ void* ksplit_scratch(hipStream_t s, size_t bytes) {
 }
 
 int launch_ksplit_reduce(const KSplitReduceArgs& r, hipStream_t s) {
-  const int64_t groups = (int64_t)r.M * r.N * 256;
+  const int64_t groups = r.flat_elems > 0 ? r.flat_elems / 4 : (int64_t)r.M * r.N * 256;
   const int64_t blocks = (groups + 255) / 256;
   if (blocks < 1 || blocks > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
   const dim3 grid((unsigned)blocks), block(256);

@@ -32,6 +32,7 @@ struct KSplitReduceArgs {
   const void* partials;      // slices x M x N tiles of 32x32 accumulator elements
   int slices;
   int M, N;                  // outer tile counts
+  int64_t flat_elems;        // > 0: partials and result are dense arrays of so many elements (a multiple of 4) instead
   void* out;                 // offset applied
   int64_t out_stride_bytes;
   int accumulate, row_major_out, out_rows, out_cols;
@@ -187,6 +188,7 @@ int launch_k_split(const MfmaArgs& a, int v, int slices, hipStream_t s) {
     r.partials = scratch;
     r.slices = slices;
     r.M = a.M; r.N = a.N;
+    r.flat_elems = 0;
     r.out = a.out;
     r.out_stride_bytes = a.out_stride_bytes;
     r.accumulate = a.accumulate;

@@ -20,6 +20,7 @@
 // and rows m0 < M0 are stored.
 #include "uk_common.h"
 #include "uk_mfma_cfg.h"
+#include "uk_mmt4d_mfma_launch.h"
 
 #include <type_traits>
 
@@ -42,10 +43,17 @@ struct SkinnyArgs {
   int lhs_tile_bytes;  // M0 * K0 * element size
   int half_k0;
   int accumulate;
+  // K split over workgroup rows: row blockIdx.y takes steps [y * chunk_steps,
+  // ...) and writes its sums, in the accumulator's type, chunk_out_elems
+  // further on (one launch row and chunk_steps = ksteps when K is not split)
+  int chunk_steps;
+  int64_t chunk_out_elems;
 };
 
 // SP: K steps per wave held in registers (compile-time bound; a.steps_per_wave <= SP).
-template <typename Cfg, int SP>
+// kPartialOut: the result is stored in the accumulator's type (the partial sums
+// of a K split whose final result is narrower: f16, bf16).
+template <typename Cfg, int SP, bool kPartialOut = false>
 __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
   typedef typename Cfg::frag_t frag_t;
   typedef typename Cfg::acc_t acc_t;
@@ -53,12 +61,15 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
   static_assert(SP % kDepth == 0, "the rolling buffer must divide the steps of a tile");
   // partial sums keep the accumulator's type (f32, or s32 for integer inputs)
   typedef typename std::conditional<std::is_same<out_t, int32_t>::value, int32_t, float>::type sum_t;
+  typedef typename std::conditional<kPartialOut, sum_t, out_t>::type store_t;
   __shared__ sum_t partial[2][kWaves][16][64];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int m0 = lane & 31, kh = lane >> 5;
-  const int first = wave * a.steps_per_wave;
-  int count = a.ksteps - first;
+  const int chunk_first = blockIdx.y * a.chunk_steps;
+  const int chunk_end = chunk_first + a.chunk_steps < a.ksteps ? chunk_first + a.chunk_steps : a.ksteps;
+  const int first = chunk_first + wave * a.steps_per_wave;
+  int count = chunk_end - first;
   count = count < 0 ? 0 : (count > a.steps_per_wave ? a.steps_per_wave : count);
 
   // Right-hand side: lane offset inside an operand block (1 KiB; fp8: 2 KiB of
@@ -142,7 +153,7 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
 #pragma unroll
     for (int v = 0; v < 16; ++v) buf[wave][v][lane] = acc[v];
     __syncthreads();
-    out_t* tile = (out_t*)a.out + (int64_t)j * a.out_stride_elems;
+    store_t* tile = (store_t*)a.out + blockIdx.y * a.chunk_out_elems + (int64_t)j * a.out_stride_elems;
 #pragma unroll
     for (int rep = 0; rep < 2; ++rep) {
       const int flat = rep * kThreads + threadIdx.x;   // v * 64 + lane
@@ -152,7 +163,7 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
         sum_t sum = a.accumulate ? (sum_t)tile[mm * 32 + nn] : (sum_t)0;
 #pragma unroll
         for (int w = 0; w < kWaves; ++w) sum += buf[w][v][l];
-        tile[mm * 32 + nn] = (out_t)sum;
+        tile[mm * 32 + nn] = (store_t)sum;
       }
     }
     // The other half of `partial` serves the next tile; this half is rewritten
@@ -160,20 +171,31 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
   }
 }
 
+// chunks: workgroup rows, each taking a.chunk_steps K steps; with more than one
+// the results are partial sums in the accumulator's type.
 template <typename Cfg>
-int launch_cfg(SkinnyArgs a, hipStream_t s) {
+int launch_cfg(SkinnyArgs a, int chunks, hipStream_t s) {
   const int cus = device_cu_count();
   const int blocks = a.N < cus ? a.N : cus;
-  const int per = (a.ksteps + kWaves - 1) / kWaves;
+  const int per = (a.chunk_steps + kWaves - 1) / kWaves;
   a.steps_per_wave = per;
-  if (per <= 8) {
-    hipLaunchKernelGGL((mmt4d_skinny_kernel<Cfg, 8>), dim3(blocks), dim3(kThreads), 0, s, a);
+  constexpr bool kNarrowOut = sizeof(typename Cfg::out_t) < 4;
+  const dim3 grid(blocks, chunks), block(kThreads);
+  if (chunks > 1 && kNarrowOut) {
+    if constexpr (kNarrowOut) {
+      if (per <= 8) hipLaunchKernelGGL((mmt4d_skinny_kernel<Cfg, 8, true>), grid, block, 0, s, a);
+      else if (per <= 16) hipLaunchKernelGGL((mmt4d_skinny_kernel<Cfg, 16, true>), grid, block, 0, s, a);
+      else if (per <= 32) hipLaunchKernelGGL((mmt4d_skinny_kernel<Cfg, 32, true>), grid, block, 0, s, a);
+      else return IREE_AMD_UK_STATUS_NOT_FOUND;
+    }
+  } else if (per <= 8) {
+    hipLaunchKernelGGL((mmt4d_skinny_kernel<Cfg, 8>), grid, block, 0, s, a);
   } else if (per <= 16) {
-    hipLaunchKernelGGL((mmt4d_skinny_kernel<Cfg, 16>), dim3(blocks), dim3(kThreads), 0, s, a);
+    hipLaunchKernelGGL((mmt4d_skinny_kernel<Cfg, 16>), grid, block, 0, s, a);
   } else if (per <= 32) {
     // (32 fp8 steps of 8 registers each would not fit the register file)
     if constexpr (Cfg::kSub == 2) return IREE_AMD_UK_STATUS_NOT_FOUND;
-    else hipLaunchKernelGGL((mmt4d_skinny_kernel<Cfg, 32>), dim3(blocks), dim3(kThreads), 0, s, a);
+    else hipLaunchKernelGGL((mmt4d_skinny_kernel<Cfg, 32>), grid, block, 0, s, a);
   } else {
     return IREE_AMD_UK_STATUS_NOT_FOUND;
   }
@@ -210,23 +232,68 @@ namespace {
 // in registers (32 steps per wave; 16 for fp8, whose step is twice as large).
 int max_steps_per_launch(int mfma_k) { return kWaves * (mfma_k == 64 ? 16 : 32); }
 
-int launch_chunk(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s);
+// One launch over the K of `p`: `chunks` workgroup rows of `chunk_steps` K steps
+// each; with more than one, the results are partial sums written to `scratch`.
+int launch_chunk(const iree_amd_uk_mmt4d_params_t& p, int chunks, int chunk_steps, void* scratch,
+                 hipStream_t s);
 }  // namespace
 
 int launch_mmt4d_skinny(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) {
   if (!mmt4d_skinny_supported(p.flags, p.M0, p.N0, p.K0)) return IREE_AMD_UK_STATUS_NOT_FOUND;
   const int mk = mfma_k_of(p.flags);
   const int64_t k_elems = p.K * p.K0;
-  if (p.M != 1 || p.K == 0 || k_elems % mk) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  if (p.M != 1 || p.K == 0 || k_elems % mk || p.N > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
   const int64_t steps = k_elems / mk;
+  if (steps > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
   const int max_steps = max_steps_per_launch(mk);
-  if (steps <= max_steps) return launch_chunk(p, s);
-  // A longer K runs as several launches over equal K slices, each accumulating
-  // into the result of the one before: exact for integers; for f32 results the
-  // same sum in another order. Results narrower than the accumulator (f16,
-  // bf16) would be rounded between the slices, so those are not split.
   Mmt4dTypeInfo ti;
   mmt4d_type_info(p.flags, &ti);
+  // K is split over workgroup rows when one launch row cannot hold it in
+  // registers, and when the outer columns alone leave half of the compute units
+  // or more idle: every row writes its sums (in the accumulator's type) to the
+  // stream's scratch buffer, and a second kernel adds them in row order, after
+  // the old result when accumulating. Deterministic; exact for integers, for
+  // floats the same sum in another order.
+  const int cus = device_cu_count();
+  int64_t chunks = (steps + max_steps - 1) / max_steps;
+  if (p.N * chunks * 2 <= cus && steps >= 64) {
+    int64_t more = cus / p.N;
+    if (more > steps / 32) more = steps / 32;
+    if (more > 8) more = 8;
+    if (more > chunks) chunks = more;
+  }
+  if (chunks > 1) {
+    const int64_t chunk_steps = (steps + chunks - 1) / chunks;
+    chunks = (steps + chunk_steps - 1) / chunk_steps;
+    const int64_t elems = p.N * p.M0 * 32;
+    // (the tiles of the single outer row are consecutive: partial sums and
+    // result are dense arrays)
+    void* scratch = ksplit_scratch(s, (size_t)(chunks * elems * 4));
+    if (scratch && chunks > 1) {
+      int st = launch_chunk(p, (int)chunks, (int)chunk_steps, scratch, s);
+      if (st) return st;
+      KSplitReduceArgs r;
+      r.partials = scratch;
+      r.slices = (int)chunks;
+      r.M = 1; r.N = 1;
+      r.flat_elems = elems;
+      r.out = (char*)p.out_buffer + p.out_offset * ti.out_bytes;
+      r.out_stride_bytes = 0;
+      r.accumulate = (p.flags & IREE_AMD_UK_FLAG_MMT4D_ACCUMULATE) != 0;
+      r.row_major_out = 0; r.out_rows = r.out_cols = 0;
+      r.out_scale = 1.0f;
+      r.acc_is_float = (p.flags & IREE_AMD_UK_FLAG_MMT4D_TYPE_MASK) != IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32;
+      const uint32_t type = p.flags & IREE_AMD_UK_FLAG_MMT4D_TYPE_MASK;
+      r.out_kind = type == IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F16 ? 1
+                   : type == IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16BF16 ? 2 : 0;
+      return launch_ksplit_reduce(r, s);
+    }
+  }
+  if (steps <= max_steps) return launch_chunk(p, 1, (int)steps, nullptr, s);
+  // Without scratch memory a longer K runs as several launches over equal K
+  // slices, each accumulating into the result of the one before. Results
+  // narrower than the accumulator (f16, bf16) would be rounded between the
+  // slices, so those are refused.
   if (ti.out_bytes != 4) return IREE_AMD_UK_STATUS_NOT_FOUND;
   const int64_t n_chunks = (steps + max_steps - 1) / max_steps;
   const int64_t chunk_steps = (steps + n_chunks - 1) / n_chunks;
@@ -239,7 +306,7 @@ int launch_mmt4d_skinny(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) {
     q.lhs_offset += tile0 * p.M0 * p.K0;
     q.rhs_offset += tile0 * p.N0 * p.K0;
     if (first > 0) q.flags |= IREE_AMD_UK_FLAG_MMT4D_ACCUMULATE;
-    const int st = launch_chunk(q, s);
+    const int st = launch_chunk(q, 1, (int)n, nullptr, s);
     // (only the first slice can be refused: alignment and strides are the same for all)
     if (st) return st;
   }
@@ -247,7 +314,8 @@ int launch_mmt4d_skinny(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) {
 }
 
 namespace {
-int launch_chunk(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) {
+int launch_chunk(const iree_amd_uk_mmt4d_params_t& p, int chunks, int chunk_steps, void* scratch,
+                 hipStream_t s) {
   const int mk = mfma_k_of(p.flags);
   Mmt4dTypeInfo ti;
   mmt4d_type_info(p.flags, &ti);
@@ -270,14 +338,21 @@ int launch_chunk(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) {
   a.lhs_tile_bytes = p.M0 * p.K0 * eb;
   a.half_k0 = p.K0 * 2 == mk;
   a.accumulate = (p.flags & IREE_AMD_UK_FLAG_MMT4D_ACCUMULATE) != 0;
+  a.chunk_steps = chunk_steps;
+  a.chunk_out_elems = 0;
+  if (chunks > 1) {
+    a.out = (char*)scratch;
+    a.accumulate = 0;
+    a.chunk_out_elems = (int64_t)p.N * p.M0 * 32;
+  }
   switch (p.flags & IREE_AMD_UK_FLAG_MMT4D_TYPE_MASK) {
-    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F32: return launch_cfg<F16Cfg>(a, s);
-    case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16F32: return launch_cfg<BF16Cfg>(a, s);
-    case IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32: return launch_cfg<S8Cfg>(a, s);
-    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F32F32F32: return launch_cfg<F32Cfg>(a, s);
-    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F8E4M3F8E4M3F32: return launch_cfg<F8Cfg>(a, s);
-    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F16: return launch_cfg<F16F16Cfg>(a, s);
-    case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16BF16: return launch_cfg<BF16BF16Cfg>(a, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F32: return launch_cfg<F16Cfg>(a, chunks, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16F32: return launch_cfg<BF16Cfg>(a, chunks, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32: return launch_cfg<S8Cfg>(a, chunks, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F32F32F32: return launch_cfg<F32Cfg>(a, chunks, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F8E4M3F8E4M3F32: return launch_cfg<F8Cfg>(a, chunks, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F16: return launch_cfg<F16F16Cfg>(a, chunks, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16BF16: return launch_cfg<BF16BF16Cfg>(a, chunks, s);
     default: return IREE_AMD_UK_STATUS_NOT_FOUND;
   }
 }

@@ -125,10 +125,12 @@ def test_narrow_lhs_tiles_bit_exact(uk, cuda, type_flag, K0):
             got = gpucase.run_mmt4d(case, flags=case.flags & ~F.MMT4D_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION)
             assert np.array_equal(got.view(np.uint8), case.run_oracle(ukref.F16_IEEE).view(np.uint8)), \
                 (hex(type_flag), M0, K0, N, steps, acc)
-    # a K beyond what one launch keeps in registers runs as several accumulating
-    # launches over K slices (results as wide as the accumulator only)
-    if type_flag not in (F.MMT4D_TYPE_F16F16F16, F.MMT4D_TYPE_BF16BF16BF16):
-        for M0, N, steps, acc in ((8, 40, 600, False), (1, 9, 896, True), (16, 3, 257, False)):
+    # a K beyond what one launch row keeps in registers (and a K of 64 steps or
+    # more with few outer columns) is split over workgroup rows whose partial
+    # sums a second kernel adds
+    if True:
+        for M0, N, steps, acc in ((8, 40, 600, False), (1, 9, 896, True), (16, 3, 257, False),
+                                  (4, 100, 300, True), (2, 128, 64, False)):
             case = ukref.Mmt4dCase(rng, type_flag, 1, N, steps * tps, M0, 32, K0, accumulate=acc)
             got = gpucase.run_mmt4d(case, flags=case.flags & ~F.MMT4D_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION)
             assert np.array_equal(got.view(np.uint8), case.run_oracle(ukref.F16_IEEE).view(np.uint8)), \
