@@ -76,6 +76,9 @@ void* ksplit_scratch(hipStream_t s, size_t bytes) {
   constexpr size_t kMaxBytes = (size_t)512 << 20;   // larger problems run unsplit
   constexpr size_t kMaxEntries = 64;
   if (bytes == 0 || bytes > kMaxBytes) return nullptr;
+  // (the per-thread default stream is one handle for a different stream in
+  // every host thread: a buffer keyed by it would be shared by unordered work)
+  if (s == hipStreamPerThread) return nullptr;
   int device = 0;
   if (hipGetDevice(&device) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
   std::lock_guard<std::mutex> lock(mutex);
