@@ -625,3 +625,37 @@ def test_k_split_row_major_forms_equal_the_three_call_chain(uk, cuda, type_flag,
         assert np.array_equal(got, want)
     else:
         assert np.all(np.abs(got - want) <= ATOL + RTOL * np.abs(want))
+
+
+@pytest.mark.gpu
+def test_k_split_scratch_grows_and_is_kept_per_stream(uk, cuda):
+    """K-split calls of growing size on two streams, interleaved: the scratch
+    buffer of a stream is replaced by a larger one while earlier work may still
+    be queued, and the two streams never share one. Every result equals the
+    exact integer product."""
+    import torch
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    rng = np.random.default_rng(5)
+    jobs = []
+    # 16 MiB is the smallest buffer: 4 slices of 40 x 40 tiles need 26 MiB, 4 of 64 x 48 need 50
+    for idx, (M1, N1, K1) in enumerate([(2, 3, 256), (40, 40, 256), (1, 2, 512), (64, 48, 256), (40, 40, 256)]):
+        A = rng.integers(-128, 128, (M1 * 32, K1 * 16), dtype=np.int8)
+        B = rng.integers(-128, 128, (N1 * 32, K1 * 16), dtype=np.int8)
+        a_dev, b_dev = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda()
+        N1b, K1b = N1, K1
+        rhs = torch.empty(N1 * K1 * 512, dtype=torch.int8, device=cuda)
+        uk.pack(b_dev, rhs, N1 * 32, K1 * 16, N1b, K1b, 32, 16, 0, F.PACK_TYPE_I8I8)
+        outs = []
+        for st in streams:
+            out = torch.zeros(M1 * 32 * N1 * 32, dtype=torch.int32, device=cuda)
+            torch.cuda.synchronize()
+            with torch.cuda.stream(st):
+                uk.matmul_packed_rhs(a_dev, rhs, out, M1 * 32, N1 * 32, K1 * 16, 16, F.MMT4D_TYPE_S8S8S32,
+                                     stream=st)
+            outs.append(out)
+        jobs.append((A, B, outs, a_dev, rhs))
+    torch.cuda.synchronize()
+    for A, B, outs, _, _ in jobs:
+        want = A.astype(np.int32) @ B.astype(np.int32).T
+        for out in outs:
+            assert np.array_equal(out.cpu().numpy().reshape(want.shape), want)
