@@ -659,3 +659,34 @@ def test_k_split_scratch_grows_and_is_kept_per_stream(uk, cuda):
         want = A.astype(np.int32) @ B.astype(np.int32).T
         for out in outs:
             assert np.array_equal(out.cpu().numpy().reshape(want.shape), want)
+
+
+@pytest.mark.gpu
+def test_random_outer_shapes_i8_exact(uk, cuda):
+    """Seeded random outer shapes (1 to 70 tiles each way, 2 to 1100 K tiles of
+    16) through every launch decision - the four macro tiles, the split of a
+    partial last round into two launches, the K split - with and without
+    accumulate, against the exact integer product (computed in float64, where
+    every sum below 2^53 is exact)."""
+    import torch
+    rng = np.random.default_rng(20240)
+    for case in range(24):
+        M1, N1 = (int(v) for v in rng.integers(1, 71, 2))
+        K1 = int(rng.choice([2, 7, 33, 128, 129, 260, 512, 900, 1100]))
+        if case % 6 == 0:
+            M1, N1, K1 = int(rng.integers(60, 100)), int(rng.integers(60, 100)), int(rng.choice([64, 128, 300]))
+        acc = bool(case % 2)
+        lhs = rng.integers(-128, 128, (M1, K1, 32, 16), dtype=np.int8)
+        rhs = rng.integers(-128, 128, (N1, K1, 32, 16), dtype=np.int8)
+        init = rng.integers(-1000, 1000, (M1, N1, 32, 32)).astype(np.int32)
+        out = torch.from_numpy(init.copy()).cuda()
+        uk.mmt4d(torch.from_numpy(lhs).cuda(), torch.from_numpy(rhs).cuda(), out, M1, N1, K1, 32, 32, 16,
+                 F.MMT4D_TYPE_S8S8S32 | (F.MMT4D_ACCUMULATE if acc else 0))
+        torch.cuda.synchronize()
+        A = lhs.transpose(0, 2, 1, 3).reshape(M1 * 32, K1 * 16).astype(np.float64)
+        B = rhs.transpose(0, 2, 1, 3).reshape(N1 * 32, K1 * 16).astype(np.float64)
+        want = (A @ B.T).reshape(M1, 32, N1, 32).transpose(0, 2, 1, 3)
+        if acc:
+            want = want + init
+        got = out.cpu().numpy().reshape(M1, N1, 32, 32)
+        assert np.array_equal(got.astype(np.float64), want), (case, M1, N1, K1, acc)
