@@ -368,9 +368,13 @@ int launch_dequant_matmul_i4(const void* x, const void* w, const void* scale, co
     // as fit (at most 16), each pass streaming the weights again: up to 8
     // passes are still far cheaper than the element-wise kernel.
     a.w_bytes = (uint32_t)w_bytes;
-    int64_t rows_per_pass = (144 * 1024) / (K * 2);
-    if (rows_per_pass > 16) rows_per_pass = 16;
-    if (rows_per_pass >= 1 && ceil_div(M, rows_per_pass) <= 8) {
+    // First with 16 rows per pass whatever K is (the kernel splits a K whose
+    // activations do not fit LDS over workgroup rows, which needs scratch
+    // memory), then with as many rows as fit without that.
+    for (int attempt = 0; attempt < 2; ++attempt) {
+      int64_t rows_per_pass = attempt == 0 ? 16 : (144 * 1024) / (K * 2);
+      if (rows_per_pass > 16) rows_per_pass = 16;
+      if (rows_per_pass < 1 || ceil_div(M, rows_per_pass) > 8) continue;
       // equal passes (8 rows at 5 per pass: 4 + 4 rather than 5 + 3)
       const int64_t passes = ceil_div(M, rows_per_pass);
       const int64_t rows = ceil_div(M, passes);

@@ -31,6 +31,7 @@
 // integers, and per-group f32 partial sums are scaled by the group's scale (the
 // lane owns output column n, so the scale is a per-lane scalar).
 #include "uk_common.h"
+#include "uk_mmt4d_mfma_launch.h"
 #include "uk_i4.h"
 
 namespace uk {
@@ -57,6 +58,11 @@ struct GemvArgs {
   int chunks_per_part;    // chunks of one such wave (the last part may have fewer)
   int x_bytes;            // size of the staged activations in LDS (the partial sums follow)
   uint32_t w_bytes, scale_bytes, zp_bytes;
+  // K split over workgroup rows (activations of all of K do not fit LDS):
+  // row blockIdx.y owns chunks [y * row_chunks, ...) and writes f32 partial
+  // sums [y][m][n] to partial_out; k_rows == 1: all chunks, f16 result
+  int k_rows, row_chunks;
+  float* partial_out;
 };
 
 // kLog2Gs: log2 of the group size for 6..8; 9 stands for "512 or more" (group
@@ -82,14 +88,17 @@ __global__ __launch_bounds__(kThreads) void dequant_gemv_i4_kernel(GemvArgs a) {
   const int unit0 = blockIdx.x + ulane * gridDim.x;
   const int unit_step = gridDim.x * unit_lanes;
   const int n_units = unit0 < a.units ? (a.units - unit0 + unit_step - 1) / unit_step : 0;
+  // (chunk indices below are local to this workgroup row's K range)
+  const int chunk_base = blockIdx.y * a.row_chunks;
+  const int my_chunks = a.chunks - chunk_base < a.row_chunks ? a.chunks - chunk_base : a.row_chunks;
   int c0 = kp * a.chunks_per_part;
-  c0 = c0 < a.chunks ? c0 : a.chunks;
+  c0 = c0 < my_chunks ? c0 : my_chunks;
   int c1 = c0 + a.chunks_per_part;
-  c1 = c1 < a.chunks ? c1 : a.chunks;
+  c1 = c1 < my_chunks ? c1 : my_chunks;
   const int n_pairs = n_units * (c1 - c0);
   // parts that own chunks, and the unit rounds of the workgroup (unit lane 0
   // has the most): every wave meets that many barriers when ksplit > 1
-  const int parts_used = (a.chunks + a.chunks_per_part - 1) / a.chunks_per_part;
+  const int parts_used = (my_chunks + a.chunks_per_part - 1) / a.chunks_per_part;
   const int rounds = ((int)blockIdx.x < a.units) ? (a.units - (int)blockIdx.x + unit_step - 1) / unit_step : 0;
 
   const uint32_t span_stride = a.tiled ? 2048u : 64u;
@@ -124,7 +133,7 @@ __global__ __launch_bounds__(kThreads) void dequant_gemv_i4_kernel(GemvArgs a) {
     if constexpr (!kRuntimeGroups) {
       int n = unit * 16 + nl;
       n = n < a.N ? n : a.N - 1;
-      const uint32_t g0 = (uint32_t)n * a.G + (uint32_t)chunk * GC;     // first group of the chunk
+      const uint32_t g0 = (uint32_t)n * a.G + (uint32_t)(chunk_base + chunk) * GC;     // first group of the chunk
 #pragma unroll
       for (int i = 0; i < SW; ++i)
         m.s[i] = __builtin_amdgcn_raw_buffer_load_b128(scale_rsrc, g0 * 2 + i * 16, 0, 0);
@@ -153,7 +162,7 @@ __global__ __launch_bounds__(kThreads) void dequant_gemv_i4_kernel(GemvArgs a) {
     const __amdgpu_buffer_rsrc_t r0 = unit_rsrc(n_pairs > 0 ? unit0 : a.units);
     if (n_pairs > 0) load_meta(unit0, c0, meta_next);
 #pragma unroll
-    for (int d = 0; d < kRingDepth; ++d) ring[d] = load_slab(r0, c0 * kChunkSpans + d);
+    for (int d = 0; d < kRingDepth; ++d) ring[d] = load_slab(r0, (chunk_base + c0) * kChunkSpans + d);
   }
   __builtin_amdgcn_sched_barrier(0);
   // x -> LDS in MFMA A-operand order: the 16 bytes that lane (row m, kc) feeds
@@ -162,13 +171,13 @@ __global__ __launch_bounds__(kThreads) void dequant_gemv_i4_kernel(GemvArgs a) {
   // on the weight layout (see the other kernel): chunk q*4+kc of the span for
   // tiled weights, kc*4+q for row-major ones.
   {
-    const int chunks_per_row = a.K >> 3;
+    const int chunks_per_row = my_chunks * 256;        // 8-element pieces of this row's K range
     const int total = a.m_eff * chunks_per_row;
     for (int c = threadIdx.x; c < total; c += kThreads) {
       const int m = c / chunks_per_row, kchunk = c - m * chunks_per_row;
       const int span = kchunk >> 4, r = kchunk & 15;
       const int q = a.tiled ? (r >> 2) : (r & 3), kcc = a.tiled ? (r & 3) : (r >> 2);
-      const u32x4 v = *(const u32x4*)(a.x + (size_t)(a.m_base + m) * a.K + kchunk * 8);
+      const u32x4 v = *(const u32x4*)(a.x + (size_t)(a.m_base + m) * a.K + (size_t)chunk_base * 2048 + kchunk * 8);
       union { half8 h; u32x4 u; } p;
       p.h = permute_x(v);
       *(u32x4*)(x_lds + (((span * 4 + q) * 4 + kcc) * a.m_eff + m) * 16) = p.u;
@@ -210,7 +219,7 @@ __global__ __launch_bounds__(kThreads) void dequant_gemv_i4_kernel(GemvArgs a) {
         const int k_in_chunk = s * 128 + q * 32;
         bool group_start, group_end;
         if constexpr (kRuntimeGroups) {
-          const int k_abs = span0 * 128 + k_in_chunk;
+          const int k_abs = (chunk_base * kChunkSpans + span0) * 128 + k_in_chunk;
           group_start = (k_abs & (gs - 1)) == 0;
           group_end = ((k_abs + 32) & (gs - 1)) == 0;
           if (group_start) {
@@ -274,7 +283,7 @@ __global__ __launch_bounds__(kThreads) void dequant_gemv_i4_kernel(GemvArgs a) {
       // for the oldest outstanding load.
       __builtin_amdgcn_sched_barrier(0);
       static_assert(kRingDepth == kChunkSpans, "a refill always lands in the next chunk");
-      ring[s % kRingDepth] = load_slab(rsrc_next, next_chunk * kChunkSpans + s);
+      ring[s % kRingDepth] = load_slab(rsrc_next, (chunk_base + next_chunk) * kChunkSpans + s);
       __builtin_amdgcn_sched_barrier(0);
     }
     if (chunk + 1 == c1) {
@@ -302,8 +311,12 @@ __global__ __launch_bounds__(kThreads) void dequant_gemv_i4_kernel(GemvArgs a) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const int m = 4 * kc + r;
-          if (m < a.m_eff && ncol < a.N)
-            a.out[(size_t)(a.m_base + m) * a.N + ncol] = __half_as_ushort(__float2half_rn(acc[r]));
+          if (m < a.m_eff && ncol < a.N) {
+            if (a.k_rows > 1)
+              a.partial_out[((size_t)blockIdx.y * a.m_eff + m) * a.N + ncol] = acc[r];
+            else
+              a.out[(size_t)(a.m_base + m) * a.N + ncol] = __half_as_ushort(__float2half_rn(acc[r]));
+          }
         }
       }
       acc = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -321,7 +334,7 @@ __global__ __launch_bounds__(kThreads) void dequant_gemv_i4_kernel(GemvArgs a) {
 
 template <bool kZpU4>
 int launch_zp(const GemvArgs& a, int blocks, size_t lds, hipStream_t s) {
-  const dim3 g(blocks), b(kThreads);
+  const dim3 g(blocks, a.k_rows), b(kThreads);
   // (once per kernel would do; the call is cheap and idempotent)
   auto set_lds = [&](const void* fn) {
     return hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
@@ -364,8 +377,6 @@ int launch_dequant_gemv_i4(const I4Args& p, int m_base, int m_eff, hipStream_t s
   // that fit LDS.
   if (K % 2048 || m_eff < 1 || m_eff > 16) return IREE_AMD_UK_STATUS_NOT_FOUND;
   if (gs < (p.tiled ? 64 : 128) || gs > 256) return IREE_AMD_UK_STATUS_NOT_FOUND;
-  size_t lds = (size_t)m_eff * K * 2;
-  if (lds > 144 * 1024) return IREE_AMD_UK_STATUS_NOT_FOUND;
   const int64_t g_total = N * p.G;
   if (N * K / 2 + K * 16 >= (1ll << 32) || g_total * 2 >= (1ll << 32)) return IREE_AMD_UK_STATUS_NOT_FOUND;
   GemvArgs a;
@@ -379,19 +390,54 @@ int launch_dequant_gemv_i4(const I4Args& p, int m_base, int m_eff, hipStream_t s
   a.w_bytes = (uint32_t)(N * K / 2);
   a.scale_bytes = (uint32_t)(g_total * 2);
   a.zp_bytes = (uint32_t)(p.zp_u4 ? (g_total + 1) / 2 : g_total * 2);
+  // The activations of a workgroup's K range live in LDS (144 KiB of it). When
+  // those of all of K do not fit, K is split over workgroup rows: every row
+  // writes f32 partial sums to the stream's scratch buffer and the K-split
+  // reduction kernel adds them in row order and rounds to f16 once.
+  const int64_t chunk_x_bytes = (int64_t)m_eff * 2048 * 2;
+  a.row_chunks = a.chunks;
+  a.k_rows = 1;
+  a.partial_out = nullptr;
+  if (a.chunks * chunk_x_bytes > 144 * 1024) {
+    a.row_chunks = (int)((144 * 1024) / chunk_x_bytes);
+    if (a.row_chunks < 1 || N % 4) return IREE_AMD_UK_STATUS_NOT_FOUND;
+    a.k_rows = (a.chunks + a.row_chunks - 1) / a.row_chunks;
+    a.row_chunks = (a.chunks + a.k_rows - 1) / a.k_rows;      // equal rows
+    a.k_rows = (a.chunks + a.row_chunks - 1) / a.row_chunks;
+    a.partial_out = (float*)ksplit_scratch(s, (size_t)a.k_rows * m_eff * N * 4);
+    if (!a.partial_out) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  }
+  size_t lds = (size_t)(a.row_chunks * chunk_x_bytes);
   // Few units (small N): deal the chunks of a unit to several waves, as many
   // as still leave every wave of the device at most one part of one unit.
   const int cus = device_cu_count();
   a.ksplit = 1;
-  while (a.ksplit < kWaves && (int64_t)a.units * a.ksplit * 2 <= (int64_t)cus * kWaves &&
-         a.ksplit < a.chunks)
+  while (a.ksplit < kWaves && (int64_t)a.units * a.k_rows * a.ksplit * 2 <= (int64_t)cus * kWaves &&
+         a.ksplit < a.row_chunks)
     a.ksplit *= 2;
-  a.chunks_per_part = (a.chunks + a.ksplit - 1) / a.ksplit;
+  a.chunks_per_part = (a.row_chunks + a.ksplit - 1) / a.ksplit;
   a.x_bytes = (int)lds;
   if (a.ksplit > 1) lds += 2 * kWaves * 64 * sizeof(floatx4);   // 16 KiB of partial sums
-  // (units go to workgroups first, then to the unit lanes of a workgroup)
-  const int blocks = a.units < cus ? a.units : cus;
-  return p.zp_u4 ? launch_zp<true>(a, blocks, lds, s) : launch_zp<false>(a, blocks, lds, s);
+  // (units go to workgroups first, then to the unit lanes of a workgroup; with
+  // K rows, a row gets its share of the compute units)
+  int blocks = cus / a.k_rows;
+  if (blocks < 1) blocks = 1;
+  if (blocks > a.units) blocks = a.units;
+  int st = p.zp_u4 ? launch_zp<true>(a, blocks, lds, s) : launch_zp<false>(a, blocks, lds, s);
+  if (st || a.k_rows == 1) return st;
+  KSplitReduceArgs r;
+  r.partials = a.partial_out;
+  r.slices = a.k_rows;
+  r.M = 1; r.N = 1;
+  r.flat_elems = (int64_t)m_eff * N;
+  r.out = p.out + (size_t)m_base * N;
+  r.out_stride_bytes = 0;
+  r.accumulate = 0;
+  r.row_major_out = 0; r.out_rows = r.out_cols = 0;
+  r.out_scale = 1.0f;
+  r.acc_is_float = 1;
+  r.out_kind = 1;   // f16
+  return launch_ksplit_reduce(r, s);
 }
 
 }  // namespace uk

@@ -96,6 +96,15 @@ def test_long_k_medium_n_splits_k_over_waves(uk, cuda, M, N, K, tiled):
     run_case(uk, M, N, K, 128, True, tiled, seed=N + K)
 
 
+@pytest.mark.parametrize("M,N,K,tiled", [(8, 4096, 14336, True), (16, 1024, 14336, False), (12, 4096, 8192, True),
+                                        (32, 2048, 14336, True), (6, 36, 10240, False)])
+def test_long_k_batches_split_k_over_workgroup_rows(uk, cuda, M, N, K, tiled):
+    """More rows than fit LDS over all of K: K is split over workgroup rows whose
+    f32 partial sums a second kernel adds (2 to 4 rows of K, one or two passes
+    of 16 rows, few and many units per row)."""
+    run_case(uk, M, N, K, 128, True, tiled, seed=M + N + K)
+
+
 def test_fractional_f16_zero_points(uk, cuda):
     run_case(uk, 5, 64, 2048, 128, False, False, seed=3, frac_zp=True)
     run_case(uk, 5, 64, 2048, 128, False, True, seed=4, frac_zp=True)
