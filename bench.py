@@ -36,10 +36,10 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE
 # and WRITE_SIZE runs of this same command (summaries under profiles/), scaled
 # by what the counters read for a copy kernel of known size (fetch x 2.0, write
-# x 1.0): 199 MiB read (each of the 8 XCD L2s fetches its own operand panels;
-# most of it is served by the 256 MiB memory-side cache; 196-212 MiB from run
-# to run) + 64 MiB written.
-MEASURED_TRAFFIC_BYTES = {"mmt4d_f16_4096": 276.1e6}
+# x 1.0): 192 MiB read (each of the 8 XCD L2s fetches its own operand panels,
+# 12 panels of 2 MiB each: most of it is served by the 256 MiB memory-side
+# cache; 192-212 MiB from run to run) + 64 MiB written.
+MEASURED_TRAFFIC_BYTES = {"mmt4d_f16_4096": 268.7e6}
 
 
 # After an idle spell (or CPU-only work) the GPU's power management needs about
