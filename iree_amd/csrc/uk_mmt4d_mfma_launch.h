@@ -247,6 +247,17 @@ int launch_cfg(const MfmaArgs& a, hipStream_t s) {
       const int resident = (int)ceil_div(rest, (int64_t)cus);   // workgroups sharing a compute unit
       cost += resident * work / (resident == t.occ ? t.eff_full : t.eff_alone);
     }
+    // A row-major left-hand side is the dearer operand to fetch (half or
+    // quarter cache lines per row and K-step): tiles with more rows than
+    // columns pay most. Measured at 2048 x 4096 x 4096 against the packed
+    // operand: 256x256 1.10 (f16) and 1.22 (i8), 256x128 1.27 and 1.36,
+    // 128x256 1.07 and 1.06, 128x128 1.30 and 1.28.
+    if (a.lhs_row_major) {
+      // (a K-step is 64 bytes of a row for f16 / bf16 / fp8, 32 for i8 and f32)
+      constexpr bool kHalfLines = Cfg::kRows == 16 || Cfg::kSub == 2;
+      static const double penalty[2][4] = {{1.22, 1.36, 1.06, 1.28}, {1.09, 1.27, 1.07, 1.30}};
+      cost *= penalty[kHalfLines][v];
+    }
     return cost;
   };
   auto pick = [&](int64_t M, int64_t N, double* out_cost) -> int {

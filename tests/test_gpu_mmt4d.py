@@ -690,3 +690,32 @@ def test_random_outer_shapes_i8_exact(uk, cuda):
             want = want + init
         got = out.cpu().numpy().reshape(M1, N1, 32, 32)
         assert np.array_equal(got.astype(np.float64), want), (case, M1, N1, K1, acc)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("accumulate", [False, True])
+def test_matmul_packed_rhs_wide_result_packs_the_lhs_first(uk, cuda, accumulate):
+    """8192 result columns and more (and 512 rows): matmul_packed_rhs packs its
+    left-hand side into the stream's scratch buffer and runs the packed-operand
+    kernel. Ragged M and N, a row pitch wider than the row, exact integers."""
+    import torch
+    M, N, K = 530, 8200, 160
+    lda, ldc = K + 16, N + 8
+    rng = np.random.default_rng(31)
+    a_pad = rng.integers(-128, 128, (M, lda), dtype=np.int8)
+    B = rng.integers(-128, 128, (N, K), dtype=np.int8)
+    N1, K1 = -(-N // 32), K // 16
+    rhs = torch.empty(N1 * K1 * 512, dtype=torch.int8, device=cuda)
+    uk.pack(torch.from_numpy(B).cuda(), rhs, N, K, N1, K1, 32, 16, 0, F.PACK_TYPE_I8I8)
+    c0 = rng.integers(-1000, 1000, (M, ldc)).astype(np.int32)
+    c = torch.from_numpy(c0.copy()).cuda()
+    uk.matmul_packed_rhs(torch.from_numpy(a_pad).cuda(), rhs, c, M, N, K, 16,
+                         F.MMT4D_TYPE_S8S8S32 | (F.MMT4D_ACCUMULATE if accumulate else 0),
+                         lhs_stride0=lda, out_stride0=ldc)
+    torch.cuda.synchronize()
+    got = c.cpu().numpy()
+    want = a_pad[:, :K].astype(np.int32) @ B.astype(np.int32).T
+    if accumulate:
+        want = want + c0[:, :N]
+    assert np.array_equal(got[:, :N], want)
+    assert np.array_equal(got[:, N:], c0[:, N:])
