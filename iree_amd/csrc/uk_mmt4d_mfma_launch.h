@@ -25,28 +25,6 @@ int launch_mfma_silu_f16(const MfmaArgs& a, hipStream_t s);
 int launch_mfma_silu_bf16(const MfmaArgs& a, hipStream_t s);
 int launch_mfma_silu_f8(const MfmaArgs& a, hipStream_t s);
 
-// Sums the partial results of a K split (tiled, accumulator type) in slice
-// order into the result, tiled or row-major: what the kernel's own epilogue
-// would have written (defined in uk_mmt4d_mfma.hip).
-struct KSplitReduceArgs {
-  const void* partials;      // slices x M x N tiles of 32x32 accumulator elements
-  int slices;
-  int M, N;                  // outer tile counts
-  int64_t flat_elems;        // > 0: partials and result are dense arrays of so many elements (a multiple of 4) instead
-  void* out;                 // offset applied
-  int64_t out_stride_bytes;
-  int accumulate, row_major_out, out_rows, out_cols;
-  float out_scale;
-  int acc_is_float;          // else int32
-  int out_kind;              // 0 = accumulator type, 1 = f16, 2 = bf16
-};
-int launch_ksplit_reduce(const KSplitReduceArgs& r, hipStream_t s);
-// Device memory for the partial sums of a K split on stream `s` of the current
-// device: one buffer per stream, kept and reused by later calls (work on one
-// stream is ordered, so they cannot overlap), grown when a call needs more.
-// nullptr when it cannot be had (the call then runs unsplit).
-void* ksplit_scratch(hipStream_t s, size_t bytes);
-
 namespace {
 
 // kOcc: waves per SIMD the register allocation must leave room for (2 = two

@@ -20,7 +20,6 @@
 // and rows m0 < M0 are stored.
 #include "uk_common.h"
 #include "uk_mfma_cfg.h"
-#include "uk_mmt4d_mfma_launch.h"
 
 #include <type_traits>
 

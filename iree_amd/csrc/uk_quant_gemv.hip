@@ -31,7 +31,6 @@
 // integers, and per-group f32 partial sums are scaled by the group's scale (the
 // lane owns output column n, so the scale is a per-lane scalar).
 #include "uk_common.h"
-#include "uk_mmt4d_mfma_launch.h"
 #include "uk_i4.h"
 
 namespace uk {
