@@ -29,6 +29,16 @@
 // table at the end of this file. The grid is one-dimensional:
 // ceildiv(M, T) * ceildiv(N, T) workgroups.
 //
+// mi355x_matmul_packed_rhs_*: the whole linear layer out[M][N] (+)= lhs[M][K] *
+// rhs in one dispatch: bindings 0 lhs, the dense row-major M x K matrix (read
+// only), 1 rhs, packed [ceildiv(N, 32)][K / K0][32][K0] (read only: weights
+// packed ahead of time), 2 out, the dense row-major M x N matrix; push
+// constants M, N, K (ELEMENTS; K a whole number of matrix-core K-steps: 32 for
+// f16 / bf16 / i8, 8 for f32, 64 for fp8), K0, flags. Macro tiles of 128 x 256
+// (_t4x8: the cheaper one for a row-major left-hand side, two workgroups per
+// compute unit) or 256 x 256 (_t8x8); grid = ceildiv(ceildiv(M, 32), 4 or 8) *
+// ceildiv(ceildiv(N, 32), 8).
+//
 // mi355x_pack_{8,16,32}bit / mi355x_unpack_{16,32}bit: iree_uk_pack / iree_uk_unpack
 // without transposes (runtime/src/iree/builtins/ukernel/pack.h:26-34,
 // unpack.h:17-25) on dense operands, for power-of-two tiles whose rows are whole
@@ -88,6 +98,41 @@ __device__ __forceinline__ void hal_mmt4d(const void* lhs, const void* rhs, void
   mmt4d_mfma_body<Cfg, WM, WN, kRing, kSync, false, 2, row_major ? 1 : 0>(a);
 }
 
+template <typename Cfg, int WM, int WN, int kRing, int kSync>
+__device__ __forceinline__ void hal_matmul_packed_rhs(const void* lhs, const void* rhs, void* out,
+                                                      int M, int N, int K, int K0, uint32_t flags) {
+  constexpr int kPerTile = 32 / Cfg::kRows;
+  constexpr int TM = 2 * WM, TN = 2 * WN;
+  static_assert(TM % kPerTile == 0 && TN % kPerTile == 0, "macro tile of whole outer tiles");
+  typedef typename Cfg::out_t out_t;
+  if (M < 1 || N < 1 || K < Cfg::kMfmaK || K % Cfg::kMfmaK) return;
+  MfmaArgs a;
+  a.lhs = (const char*)lhs;
+  a.rhs = (const char*)rhs;
+  a.out = (char*)out;
+  a.lhs_stride_bytes = (int64_t)K * Cfg::kElemBytes;            // row pitch of the matrix
+  a.rhs_stride_bytes = (int64_t)K * 32 * Cfg::kElemBytes;       // one outer row of packed tiles
+  a.out_stride_bytes = (int64_t)N * (int64_t)sizeof(out_t);
+  a.M = (M + 31) / 32;
+  a.N = (N + 31) / 32;
+  a.ksteps = K / Cfg::kMfmaK;
+  a.tail_tiles = 0;
+  a.tiles_m = (a.M * kPerTile + TM - 1) / TM;
+  a.tiles_n = (a.N * kPerTile + TN - 1) / TN;
+  a.accumulate = (flags & 0x100u) != 0;
+  a.row_major_out = 1;
+  a.out_rows = M;
+  a.out_cols = N;
+  a.lhs_row_major = 1;
+  a.k_slices = 0;
+  a.slice_ksteps = 0;
+  a.slice_out_bytes = 0;
+  a.k0_div = Cfg::kMfmaK / K0;
+  a.gate_scale = a.up_scale = a.inv_out_scale = a.out_scale = 1.0f;
+  if ((int)blockIdx.x >= a.tiles_m * a.tiles_n) return;
+  mmt4d_mfma_body<Cfg, WM, WN, kRing, kSync, false, 2, 2>(a);
+}
+
 template <int ES, bool kPack>
 __device__ __forceinline__ void hal_pack(const void* mat, void* tiled, int size0, int size1,
                                          int tile0, int tile1, uint32_t padding) {
@@ -137,6 +182,25 @@ MI355X_PACK_EXPORTS(16, 2)
 MI355X_PACK_EXPORTS(32, 4)
 MI355X_UNPACK_EXPORTS(16, 2)
 MI355X_UNPACK_EXPORTS(32, 4)
+
+#define MI355X_MATMUL_EXPORT(NAME, CFG, WM, WN, RING, SYNC, OCC, LDS)                              \
+  static_assert(uk::mmt4d_mfma_lds_bytes<uk::CFG, WM, WN, RING>() == LDS, "LDS size of the table"); \
+  extern "C" __global__ __launch_bounds__(256, OCC) void mi355x_matmul_packed_rhs_##NAME(          \
+      const void* __restrict__ lhs, const void* __restrict__ rhs, void* __restrict__ out, int M,   \
+      int N, int K, int K0, unsigned flags) {                                                      \
+    hal_matmul_packed_rhs<uk::CFG, WM, WN, RING, SYNC>(lhs, rhs, out, M, N, K, K0, flags);        \
+  }
+// name            config    blocks/wave ring sync occ  LDS bytes
+MI355X_MATMUL_EXPORT(f16f16f32_t4x8, F16Cfg16, 4, 8, 3, 1, 2, 73728)
+MI355X_MATMUL_EXPORT(f16f16f32_t8x8, F16Cfg16, 8, 8, 5, 1, 1, 163840)
+MI355X_MATMUL_EXPORT(bf16bf16f32_t4x8, BF16Cfg16, 4, 8, 3, 1, 2, 73728)
+MI355X_MATMUL_EXPORT(bf16bf16f32_t8x8, BF16Cfg16, 8, 8, 5, 1, 1, 163840)
+MI355X_MATMUL_EXPORT(s8s8s32_t4x8, S8Cfg, 2, 4, 6, 2, 2, 73728)
+MI355X_MATMUL_EXPORT(s8s8s32_t8x8, S8Cfg, 4, 4, 8, 2, 1, 131072)
+MI355X_MATMUL_EXPORT(f8e4m3f8e4m3f32_t4x8, F8Cfg, 2, 4, 3, 1, 2, 73728)
+MI355X_MATMUL_EXPORT(f8e4m3f8e4m3f32_t8x8, F8Cfg, 4, 4, 5, 1, 1, 163840)
+MI355X_MATMUL_EXPORT(f32f32f32_t4x8, F32Cfg, 2, 4, 6, 2, 2, 73728)
+MI355X_MATMUL_EXPORT(f32f32f32_t8x8, F32Cfg, 4, 4, 8, 2, 1, 131072)
 
 // One export per element-type tuple and macro tile, in the tiled and the
 // row-major-result form.

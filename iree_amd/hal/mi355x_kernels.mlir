@@ -340,8 +340,178 @@ hal.executable.source public @mi355x_mmt4d attributes {
     %c1 = arith.constant 1 : index
     hal.return %x, %c1, %c1 : index, index, index
   }
+  // out[M][N] (+)= lhs[M][K] * rhs (packed); push constants M, N, K (elements), K0, flags; workload (M, N)
+  hal.executable.export public @mi355x_matmul_packed_rhs_f16f16f32_t4x8 ordinal(20)
+      layout(#hal.pipeline.layout<push_constants = 5, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer, ReadOnly>,
+            <2, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index],
+    workgroup_local_memory = 73728 : index
+  } {
+  ^bb0(%device: !hal.device, %m: index, %n: index):
+    %x = affine.apply affine_map<()[s0, s1] -> (((s0 ceildiv 32) ceildiv 4) * ((s1 ceildiv 32) ceildiv 8))>()[%m, %n]
+    %c1 = arith.constant 1 : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  // out[M][N] (+)= lhs[M][K] * rhs (packed); push constants M, N, K (elements), K0, flags; workload (M, N)
+  hal.executable.export public @mi355x_matmul_packed_rhs_f16f16f32_t8x8 ordinal(21)
+      layout(#hal.pipeline.layout<push_constants = 5, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer, ReadOnly>,
+            <2, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index],
+    workgroup_local_memory = 163840 : index
+  } {
+  ^bb0(%device: !hal.device, %m: index, %n: index):
+    %x = affine.apply affine_map<()[s0, s1] -> (((s0 ceildiv 32) ceildiv 8) * ((s1 ceildiv 32) ceildiv 8))>()[%m, %n]
+    %c1 = arith.constant 1 : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  // out[M][N] (+)= lhs[M][K] * rhs (packed); push constants M, N, K (elements), K0, flags; workload (M, N)
+  hal.executable.export public @mi355x_matmul_packed_rhs_bf16bf16f32_t4x8 ordinal(22)
+      layout(#hal.pipeline.layout<push_constants = 5, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer, ReadOnly>,
+            <2, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index],
+    workgroup_local_memory = 73728 : index
+  } {
+  ^bb0(%device: !hal.device, %m: index, %n: index):
+    %x = affine.apply affine_map<()[s0, s1] -> (((s0 ceildiv 32) ceildiv 4) * ((s1 ceildiv 32) ceildiv 8))>()[%m, %n]
+    %c1 = arith.constant 1 : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  // out[M][N] (+)= lhs[M][K] * rhs (packed); push constants M, N, K (elements), K0, flags; workload (M, N)
+  hal.executable.export public @mi355x_matmul_packed_rhs_bf16bf16f32_t8x8 ordinal(23)
+      layout(#hal.pipeline.layout<push_constants = 5, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer, ReadOnly>,
+            <2, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index],
+    workgroup_local_memory = 163840 : index
+  } {
+  ^bb0(%device: !hal.device, %m: index, %n: index):
+    %x = affine.apply affine_map<()[s0, s1] -> (((s0 ceildiv 32) ceildiv 8) * ((s1 ceildiv 32) ceildiv 8))>()[%m, %n]
+    %c1 = arith.constant 1 : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  // out[M][N] (+)= lhs[M][K] * rhs (packed); push constants M, N, K (elements), K0, flags; workload (M, N)
+  hal.executable.export public @mi355x_matmul_packed_rhs_s8s8s32_t4x8 ordinal(24)
+      layout(#hal.pipeline.layout<push_constants = 5, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer, ReadOnly>,
+            <2, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index],
+    workgroup_local_memory = 73728 : index
+  } {
+  ^bb0(%device: !hal.device, %m: index, %n: index):
+    %x = affine.apply affine_map<()[s0, s1] -> (((s0 ceildiv 32) ceildiv 4) * ((s1 ceildiv 32) ceildiv 8))>()[%m, %n]
+    %c1 = arith.constant 1 : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  // out[M][N] (+)= lhs[M][K] * rhs (packed); push constants M, N, K (elements), K0, flags; workload (M, N)
+  hal.executable.export public @mi355x_matmul_packed_rhs_s8s8s32_t8x8 ordinal(25)
+      layout(#hal.pipeline.layout<push_constants = 5, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer, ReadOnly>,
+            <2, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index],
+    workgroup_local_memory = 131072 : index
+  } {
+  ^bb0(%device: !hal.device, %m: index, %n: index):
+    %x = affine.apply affine_map<()[s0, s1] -> (((s0 ceildiv 32) ceildiv 8) * ((s1 ceildiv 32) ceildiv 8))>()[%m, %n]
+    %c1 = arith.constant 1 : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  // out[M][N] (+)= lhs[M][K] * rhs (packed); push constants M, N, K (elements), K0, flags; workload (M, N)
+  hal.executable.export public @mi355x_matmul_packed_rhs_f8e4m3f8e4m3f32_t4x8 ordinal(26)
+      layout(#hal.pipeline.layout<push_constants = 5, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer, ReadOnly>,
+            <2, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index],
+    workgroup_local_memory = 73728 : index
+  } {
+  ^bb0(%device: !hal.device, %m: index, %n: index):
+    %x = affine.apply affine_map<()[s0, s1] -> (((s0 ceildiv 32) ceildiv 4) * ((s1 ceildiv 32) ceildiv 8))>()[%m, %n]
+    %c1 = arith.constant 1 : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  // out[M][N] (+)= lhs[M][K] * rhs (packed); push constants M, N, K (elements), K0, flags; workload (M, N)
+  hal.executable.export public @mi355x_matmul_packed_rhs_f8e4m3f8e4m3f32_t8x8 ordinal(27)
+      layout(#hal.pipeline.layout<push_constants = 5, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer, ReadOnly>,
+            <2, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index],
+    workgroup_local_memory = 163840 : index
+  } {
+  ^bb0(%device: !hal.device, %m: index, %n: index):
+    %x = affine.apply affine_map<()[s0, s1] -> (((s0 ceildiv 32) ceildiv 8) * ((s1 ceildiv 32) ceildiv 8))>()[%m, %n]
+    %c1 = arith.constant 1 : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  // out[M][N] (+)= lhs[M][K] * rhs (packed); push constants M, N, K (elements), K0, flags; workload (M, N)
+  hal.executable.export public @mi355x_matmul_packed_rhs_f32f32f32_t4x8 ordinal(28)
+      layout(#hal.pipeline.layout<push_constants = 5, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer, ReadOnly>,
+            <2, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index],
+    workgroup_local_memory = 73728 : index
+  } {
+  ^bb0(%device: !hal.device, %m: index, %n: index):
+    %x = affine.apply affine_map<()[s0, s1] -> (((s0 ceildiv 32) ceildiv 4) * ((s1 ceildiv 32) ceildiv 8))>()[%m, %n]
+    %c1 = arith.constant 1 : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  // out[M][N] (+)= lhs[M][K] * rhs (packed); push constants M, N, K (elements), K0, flags; workload (M, N)
+  hal.executable.export public @mi355x_matmul_packed_rhs_f32f32f32_t8x8 ordinal(29)
+      layout(#hal.pipeline.layout<push_constants = 5, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer, ReadOnly>,
+            <2, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index],
+    workgroup_local_memory = 131072 : index
+  } {
+  ^bb0(%device: !hal.device, %m: index, %n: index):
+    %x = affine.apply affine_map<()[s0, s1] -> (((s0 ceildiv 32) ceildiv 8) * ((s1 ceildiv 32) ceildiv 8))>()[%m, %n]
+    %c1 = arith.constant 1 : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
   // pack: in = matrix, out = tiles; push constants size0, size1, tile0, tile1, padding; workload (size0, size1, tile0, tile1)
-  hal.executable.export public @mi355x_pack_8bit ordinal(20)
+  hal.executable.export public @mi355x_pack_8bit ordinal(30)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
         <0, bindings = [
             <0, storage_buffer, ReadOnly>,
@@ -367,7 +537,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
     hal.return %x, %c1, %c1 : index, index, index
   }
   // pack: in = matrix, out = tiles; push constants size0, size1, tile0, tile1, padding; workload (size0, size1, tile0, tile1)
-  hal.executable.export public @mi355x_pack_16bit ordinal(21)
+  hal.executable.export public @mi355x_pack_16bit ordinal(31)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
         <0, bindings = [
             <0, storage_buffer, ReadOnly>,
@@ -393,7 +563,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
     hal.return %x, %c1, %c1 : index, index, index
   }
   // pack: in = matrix, out = tiles; push constants size0, size1, tile0, tile1, padding; workload (size0, size1, tile0, tile1)
-  hal.executable.export public @mi355x_pack_32bit ordinal(22)
+  hal.executable.export public @mi355x_pack_32bit ordinal(32)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
         <0, bindings = [
             <0, storage_buffer, ReadOnly>,
@@ -419,7 +589,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
     hal.return %x, %c1, %c1 : index, index, index
   }
   // unpack: in = tiles, out = matrix; push constants size0, size1, tile0, tile1; workload (size0, size1, tile0, tile1)
-  hal.executable.export public @mi355x_unpack_16bit ordinal(23)
+  hal.executable.export public @mi355x_unpack_16bit ordinal(33)
       layout(#hal.pipeline.layout<push_constants = 4, sets = [
         <0, bindings = [
             <0, storage_buffer, ReadOnly>,
@@ -441,7 +611,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
     hal.return %x, %c1, %c1 : index, index, index
   }
   // unpack: in = tiles, out = matrix; push constants size0, size1, tile0, tile1; workload (size0, size1, tile0, tile1)
-  hal.executable.export public @mi355x_unpack_32bit ordinal(24)
+  hal.executable.export public @mi355x_unpack_32bit ordinal(34)
       layout(#hal.pipeline.layout<push_constants = 4, sets = [
         <0, bindings = [
             <0, storage_buffer, ReadOnly>,

@@ -49,6 +49,36 @@ def _exports():
 
 EXPORTS = _exports()
 
+# The whole linear layer on a row-major left-hand side and pre-packed weights:
+# name -> (type flag, macro tile in outer tiles (rows, columns), LDS bytes, K0
+# served, elements of K per matrix-core step).
+MatmulExport = namedtuple("MatmulExport", "name type_flag tile_m tile_n lds k0 mfma_k")
+
+
+def _matmul_exports():
+    kib = 1024
+    rows = [("f16f16f32", F.MMT4D_TYPE_F16F16F32, 160 * kib, (8, 16), 32),
+            ("bf16bf16f32", F.MMT4D_TYPE_BF16BF16F32, 160 * kib, (8, 16), 32),
+            ("s8s8s32", F.MMT4D_TYPE_S8S8S32, 128 * kib, (16, 32), 32),
+            ("f8e4m3f8e4m3f32", F.MMT4D_TYPE_F8E4M3F8E4M3F32, 160 * kib, (16,), 64),
+            ("f32f32f32", F.MMT4D_TYPE_F32F32F32, 128 * kib, (4, 8), 8)]
+    out = {}
+    for name, flag, lds8, k0, mk in rows:
+        for tm, lds in ((4, 72 * kib), (8, lds8)):
+            full = f"mi355x_matmul_packed_rhs_{name}_t{tm}x8"
+            out[full] = MatmulExport(full, flag, tm, 8, lds, k0, mk)
+    return out
+
+
+MATMUL_EXPORTS = _matmul_exports()
+
+
+def matmul_workgroup_count(name, M, N):
+    """Grid of a matmul export for an M x N result (elements)."""
+    e = MATMUL_EXPORTS[name]
+    return -(-(-(-M // 32)) // e.tile_m) * -(-(-(-N // 32)) // e.tile_n)
+
+
 # pack / unpack without transposes, by element size: name -> (bytes per element,
 # True for pack). Power-of-two tiles whose rows are whole 16-byte chunks.
 PACK_EXPORTS = {"mi355x_pack_8bit": (1, True), "mi355x_pack_16bit": (2, True),
@@ -91,7 +121,8 @@ class HalExecutable:
 
     def add_export(self, name, block=(WORKGROUP_SIZE, 1, 1), shared_memory_size=None):
         if shared_memory_size is None:
-            shared_memory_size = 0 if name in PACK_EXPORTS else EXPORTS[name].lds
+            shared_memory_size = (0 if name in PACK_EXPORTS else
+                                  MATMUL_EXPORTS[name].lds if name in MATMUL_EXPORTS else EXPORTS[name].lds)
         ordinal = C.c_int32(-1)
         _check(self._lib.iree_amd_hal_executable_add_export(
             self._handle, name.encode(), block[0], block[1], block[2], shared_memory_size,
@@ -123,6 +154,12 @@ class HalExecutable:
         if "_unpack_" in name:
             consts += [out_rows, out_cols]
         self.dispatch(name, workgroup_count(e, M, N), [lhs, rhs, out], consts, stream)
+
+    def matmul_packed_rhs(self, name, lhs, rhs_packed, out, M, N, K, K0, flags, stream=None):
+        """mi355x_matmul_packed_rhs_*: out[M][N] (+)= lhs[M][K] * rhs, all dense,
+        M, N, K in elements."""
+        self.dispatch(name, matmul_workgroup_count(name, M, N), [lhs, rhs_packed, out],
+                      [M, N, K, K0, flags], stream)
 
     def pack(self, name, matrix, tiles, size0, size1, tile0, tile1, padding=0, stream=None):
         """mi355x_pack_*: matrix (size0 x size1, dense) -> tiles; `padding` is the
@@ -193,6 +230,26 @@ _MLIR_EXPORT = """\
   }}
 """
 
+_MLIR_MATMUL_EXPORT = """\
+  // out[M][N] (+)= lhs[M][K] * rhs (packed); push constants M, N, K (elements), K0, flags; workload (M, N)
+  hal.executable.export public @{name} ordinal({ordinal})
+      layout(#hal.pipeline.layout<push_constants = 5, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer, ReadOnly>,
+            <2, storage_buffer>
+        ]>
+      ]>) attributes {{
+    workgroup_size = [{wg} : index, 1 : index, 1 : index],
+    workgroup_local_memory = {lds} : index
+  }} {{
+  ^bb0(%device: !hal.device, %m: index, %n: index):
+    %x = affine.apply affine_map<()[s0, s1] -> (((s0 ceildiv 32) ceildiv {tile_m}) * ((s1 ceildiv 32) ceildiv {tile_n}))>()[%m, %n]
+    %c1 = arith.constant 1 : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }}
+"""
+
 _MLIR_PACK_EXPORT = """\
   // {what}; push constants size0, size1, tile0, tile1{extra}; workload (size0, size1, tile0, tile1)
   hal.executable.export public @{name} ordinal({ordinal})
@@ -249,6 +306,10 @@ def mlir_source():
             name=e.name, ordinal=ordinal, constants=7 if "_unpack_" in e.name else 5,
             wg=WORKGROUP_SIZE, lds=e.lds, tile=e.tile))
     ordinal = len(EXPORTS)
+    for e in MATMUL_EXPORTS.values():
+        parts.append(_MLIR_MATMUL_EXPORT.format(name=e.name, ordinal=ordinal, wg=WORKGROUP_SIZE,
+                                                lds=e.lds, tile_m=e.tile_m, tile_n=e.tile_n))
+        ordinal += 1
     for name, (es, is_pack) in PACK_EXPORTS.items():
         parts.append(_MLIR_PACK_EXPORT.format(
             name=name, ordinal=ordinal, es=es, wg=WORKGROUP_SIZE, constants=5 if is_pack else 4,

@@ -43,12 +43,18 @@ def test_export_table_matches_the_sources():
     assert H.pack_workgroup_count("mi355x_pack_16bit", 8191, 5001, 32, 16) == 20 * 512
     assert H.pack_workgroup_count("mi355x_unpack_16bit", 8191, 5001, 32, 16) == 20 * 512
     assert H.pack_workgroup_count("mi355x_unpack_32bit", 17, 9, 8, 4) == 1 * 2
+    mm = re.findall(r"^MI355X_MATMUL_EXPORT\((\w+), \w+, \d+, \d+, \d+, \d+, \d+, (\d+)\)", src, re.M)
+    assert len(mm) == len(H.MATMUL_EXPORTS)
+    for name, lds in mm:
+        assert H.MATMUL_EXPORTS["mi355x_matmul_packed_rhs_" + name].lds == int(lds)
+    assert H.matmul_workgroup_count("mi355x_matmul_packed_rhs_s8s8s32_t4x8", 200, 333) == 2 * 2
+    assert H.matmul_workgroup_count("mi355x_matmul_packed_rhs_s8s8s32_t8x8", 4096, 4096) == 16 * 16
 
 
 def test_code_object_is_built_and_names_every_export():
     with open(H.CODE_OBJECT, "rb") as f:
         image = f.read()
-    for name in list(H.EXPORTS) + list(H.PACK_EXPORTS):
+    for name in list(H.EXPORTS) + list(H.PACK_EXPORTS) + list(H.MATMUL_EXPORTS):
         assert name.encode() + b"\0" in image, name
 
 
@@ -128,6 +134,51 @@ def test_row_major_exports_equal_the_library_entry_point(uk, cuda, exe, name):
         torch.cuda.synchronize()
         assert np.array_equal(one.cpu().numpy().view(np.uint32), two.cpu().numpy().view(np.uint32)), (name, acc)
         assert not torch.equal(one, init)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", sorted(H.MATMUL_EXPORTS))
+def test_matmul_exports_equal_the_library_entry_point(uk, cuda, exe, name):
+    """mi355x_matmul_packed_rhs_*: the bits of iree_amd_uk_matmul_packed_rhs (same
+    kernel body) on random data, ragged M and N, with and without accumulation;
+    for i8 also the exact integer product."""
+    import torch
+    e = H.MATMUL_EXPORTS[name]
+    K0 = e.k0[0]
+    M, N, K = 200, 333, 9 * e.mfma_k
+    N1, K1 = -(-N // 32), K // K0
+    rng = np.random.default_rng(zlib.crc32(name.encode()))
+    if e.type_flag == F.MMT4D_TYPE_S8S8S32:
+        A = rng.integers(-128, 128, (M, K), dtype=np.int8)
+        B = rng.integers(-128, 128, (N, K), dtype=np.int8)
+        a_dev, b_dev, ptype = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda(), F.PACK_TYPE_I8I8
+    elif e.type_flag == F.MMT4D_TYPE_F8E4M3F8E4M3F32:
+        A = rng.integers(0, 256, (M, K), dtype=np.uint8)
+        B = rng.integers(0, 256, (N, K), dtype=np.uint8)
+        A[(A & 0x7F) == 0x7F] = 0x38
+        B[(B & 0x7F) == 0x7F] = 0x38
+        a_dev, b_dev, ptype = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda(), F.PACK_TYPE_I8I8
+    else:
+        tdt = {F.MMT4D_TYPE_F16F16F32: torch.float16, F.MMT4D_TYPE_BF16BF16F32: torch.bfloat16,
+               F.MMT4D_TYPE_F32F32F32: torch.float32}[e.type_flag]
+        a_dev = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).cuda().to(tdt)
+        b_dev = torch.from_numpy(rng.standard_normal((N, K)).astype(np.float32)).cuda().to(tdt)
+        ptype = F.PACK_TYPE_F32F32 if tdt == torch.float32 else F.PACK_TYPE_F16F16
+    rhs = torch.empty(N1 * K1 * 32 * K0, dtype=b_dev.dtype, device=cuda)
+    uk.pack(b_dev, rhs, N, K, N1, K1, 32, K0, 0, ptype)
+    odt = torch.int32 if e.type_flag == F.MMT4D_TYPE_S8S8S32 else torch.float32
+    for acc in (0, F.MMT4D_ACCUMULATE):
+        init = torch.from_numpy(rng.integers(-50, 50, M * N).astype(np.int32)).cuda().to(odt)
+        one, two = init.clone(), init.clone()
+        exe.matmul_packed_rhs(name, a_dev, rhs, one, M, N, K, K0, e.type_flag | acc)
+        uk.matmul_packed_rhs(a_dev, rhs, two, M, N, K, K0, e.type_flag | acc)
+        torch.cuda.synchronize()
+        assert np.array_equal(one.cpu().numpy().view(np.uint32), two.cpu().numpy().view(np.uint32)), (name, acc)
+        if e.type_flag == F.MMT4D_TYPE_S8S8S32:
+            want = A.astype(np.int32) @ B.astype(np.int32).T
+            if acc:
+                want = want + init.cpu().numpy().reshape(M, N)
+            assert np.array_equal(one.cpu().numpy().reshape(M, N), want)
 
 
 PACK_CASES = [  # size0, size1, tile0, tile1 (elements)
