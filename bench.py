@@ -60,7 +60,8 @@ def parse_args():
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary measurements")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--only", default="", help="run only the named kernel in a loop (for profilers): "
-                    "mmt4d_f16 | mmt4d_i8 | mmt4d_fp8 | mlp_fp8 | pack | unpack | dequant_i4 | copy")
+                    "mmt4d_f16 | mmt4d_i8 | mmt4d_fp8 | mmt4d_f16_ksplit | mlp_fp8 | pack | unpack | "
+                    "dequant_i4 | copy")
     return ap.parse_args()
 
 
@@ -637,6 +638,14 @@ def run_only(args, torch, iree_amd, F, synth, mm_step):
         n = 64 * 1024 * 1024
         buf = torch.ones(n, dtype=torch.float32, device="cuda")
         fn = lambda: iree_amd.scale_f32(buf, n, 1.0)  # noqa: E731
+    elif args.only == "mmt4d_f16_ksplit":
+        # 256 x 4096 x 14336: few macro tiles, long K (the launcher splits K)
+        Ms, Ns, Ks = 256, 4096, 14336
+        ls = torch.from_numpy(synth.normal_f16(7, Ms * Ks, scale=1 / 64).view(np.int16)).cuda()
+        rs = torch.from_numpy(synth.normal_f16(8, Ns * Ks, scale=1 / 64).view(np.int16)).cuda()
+        os_ = torch.empty(Ms * Ns, dtype=torch.float32, device="cuda")
+        fn = lambda: iree_amd.mmt4d(ls, rs, os_, Ms // 32, Ns // 32, Ks // 8, 32, 32, 8,  # noqa: E731
+                                    F.MMT4D_TYPE_F16F16F32)
     else:
         raise SystemExit(f"unknown --only {args.only}")
     wall, per_launch = gpu_time(torch, fn, args.steps, args.warmup)
