@@ -226,7 +226,13 @@ __device__ __forceinline__ void mmt4d_mfma_body(const MfmaArgs a) {
   // MFMAs of a whole K-step / of the part behind a barrier, and how many of
   // them (from the front) get fragment reads slipped in behind them: the last
   // third or so stays free so that the reads have landed when the step ends.
-  constexpr int kMfmaAll = WM * WN, kMfmaRest = (WM - 1) * WN;
+  // kOuterB: with exchanged operands the MFMAs run over B blocks in the outer
+  // loop, so that the instruction's first operand is the one that stays (and
+  // the A fragments are the ones every first MFMA needs: they are read first).
+  // Measured 2 % on the MLP block, 0.1-0.3 % on square problems.
+  constexpr bool kOuterB = kSwap;
+  constexpr int kOuter = kOuterB ? WN : WM, kInner = kOuterB ? WM : WN;
+  constexpr int kMfmaAll = WM * WN, kMfmaRest = (kOuter - 1) * kInner;
   constexpr int kTail = kPerTile * kPerTile;    // (16-row shapes: 4x the MFMAs per K-step, each half as long)
   constexpr int kReadAll = kMfmaAll - (kMfmaAll >= 8 * kTail ? 6 * kTail : kMfmaAll / 2);
   constexpr int kReadRest = kMfmaRest - (kMfmaRest >= 8 * kTail ? 4 * kTail : kMfmaRest / 2);
@@ -398,8 +404,11 @@ __device__ __forceinline__ void mmt4d_mfma_body(const MfmaArgs a) {
   // outer loop, so the fragments read last (A blocks 1..) are needed last.
   auto read_one = [&](int slot, int r, frag_t (&fa)[WM], frag_t (&fb)[WN]) {
     const char* s0 = lds + slot * kSlotBytes + lane * 16;
-    if (r < WN) fb[r] = read_frag(s0 + kABytes + (wn * WN + r) * kBlockBytes);
-    else fa[r - WN] = read_frag(s0 + (wm * WM + r - WN) * kBlockBytes);
+    // (the inner loop's operand first: all of it is needed by the first MFMAs)
+    const bool is_b = kOuterB ? r >= WM : r < WN;
+    const int idx = kOuterB ? (r < WM ? r : r - WM) : (r < WN ? r : r - WN);
+    if (is_b) fb[idx] = read_frag(s0 + kABytes + (wn * WN + idx) * kBlockBytes);
+    else fa[idx] = read_frag(s0 + (wm * WM + idx) * kBlockBytes);
   };
   auto read_frags = [&](int slot, frag_t (&fa)[WM], frag_t (&fb)[WN]) {
 #pragma unroll
@@ -423,17 +432,27 @@ __device__ __forceinline__ void mmt4d_mfma_body(const MfmaArgs a) {
     }
   };
   // MFMAs of block rows [x0, x1) of this wave's WM x WN blocks.
-  auto multiply_rows = [&](const frag_t (&fa)[WM], const frag_t (&fb)[WN], int x0, int x1) {
+  auto multiply_rows = [&](const frag_t (&fa)[WM], const frag_t (&fb)[WN], int o0, int o1) {
+    if constexpr (kOuterB) {
+      // exchanged operands: the B fragment is the instruction's first operand
+      // and stays the same over the inner loop
 #pragma unroll
-    for (int x = 0; x < WM; ++x)
-      if (x >= x0 && x < x1) {
+      for (int y = 0; y < WN; ++y)
+        if (y >= o0 && y < o1) {
 #pragma unroll
-        for (int y = 0; y < WN; ++y)
-          acc[x][y] = kSwap ? Cfg::mfma(fb[y], fa[x], acc[x][y]) : Cfg::mfma(fa[x], fb[y], acc[x][y]);
-      }
+          for (int x = 0; x < WM; ++x) acc[x][y] = Cfg::mfma(fb[y], fa[x], acc[x][y]);
+        }
+    } else {
+#pragma unroll
+      for (int x = 0; x < WM; ++x)
+        if (x >= o0 && x < o1) {
+#pragma unroll
+          for (int y = 0; y < WN; ++y) acc[x][y] = Cfg::mfma(fa[x], fb[y], acc[x][y]);
+        }
+    }
   };
   auto multiply = [&](const frag_t (&fa)[WM], const frag_t (&fb)[WN]) {
-    multiply_rows(fa, fb, 0, WM);
+    multiply_rows(fa, fb, 0, kOuter);
   };
 
   frag_t fa[2][WM], fb[2][WN];
@@ -484,7 +503,7 @@ __device__ __forceinline__ void mmt4d_mfma_body(const MfmaArgs a) {
           __builtin_amdgcn_sched_barrier(0);
           memory_ops(std::integral_constant<int, kMfmaRest>(), std::integral_constant<int, kReadRest>(),
                      load_ks, issue_slot, next_slot, fa[p ^ 1], fb[p ^ 1]);
-          multiply_rows(fa[p], fb[p], 1, WM);
+          multiply_rows(fa[p], fb[p], 1, kOuter);
           spread_issue<kMfmaRest, kReadRest, kFrags, kLoadsPerStep, kSub>();
           __builtin_amdgcn_sched_barrier(0);
         }
