@@ -352,6 +352,27 @@ def extras(args, torch, iree_amd, F, synth, lhs, rhs, out, ex):
     ex["mmt4d_f16_m256_n4096_k14336_tflops"] = round(2.0 * Ms * Ns * Ks / t / 1e12, 1)
     del ls, rs, os_
 
+    # batch_mmt4d: 16 problems of 1024^3 in one launch (batch entries are planes
+    # of the grid), against the same entries run one call each.
+    Bn, Bs = 16, 1024
+    lb = torch.from_numpy(synth.normal_f16(9, Bn * Bs * Bs, scale=1 / 64).view(np.int16)).cuda()
+    rb = torch.from_numpy(synth.normal_f16(10, Bn * Bs * Bs, scale=1 / 64).view(np.int16)).cuda()
+    ob = torch.empty(Bn * Bs * Bs, dtype=torch.float32, device="cuda")
+    o1 = torch.empty(Bn * Bs * Bs, dtype=torch.float32, device="cuda")
+    bt, bk = Bs // 32, Bs // 8
+    _, t = gpu_time(torch, lambda: iree_amd.batch_mmt4d(lb, rb, ob, Bn, bt, bt, bk, 32, 32, 8,
+                                                        F.MMT4D_TYPE_F16F16F32), steps, warm)
+
+    def one_by_one():
+        for b in range(Bn):
+            iree_amd.mmt4d(lb, rb, o1, bt, bt, bk, 32, 32, 8, F.MMT4D_TYPE_F16F16F32,
+                           lhs_offset=b * Bs * Bs, rhs_offset=b * Bs * Bs, out_offset=b * Bs * Bs)
+    _, t1 = gpu_time(torch, one_by_one, max(steps // 4, 2), 1)
+    assert torch.equal(ob.view(torch.int32), o1.view(torch.int32)), "batch_mmt4d differs from per-entry mmt4d"
+    ex["batch_mmt4d_f16_16x1024_tflops"] = round(2.0 * Bn * Bs ** 3 / t / 1e12, 1)
+    ex["batch_mmt4d_f16_16x1024_entry_by_entry_tflops"] = round(2.0 * Bn * Bs ** 3 / t1 / 1e12, 1)
+    del lb, rb, ob, o1
+
     # The same f16 mmt4d dispatched from the code object a HAL executable on a
     # HIP device links (hipModuleLaunchKernel, bindings + 32-bit push constants)
     from iree_amd import hal_executable

@@ -175,6 +175,23 @@ IREE_AMD_UK_EXPORT int iree_amd_uk_mmt4d(
 IREE_AMD_UK_EXPORT int iree_amd_uk_mmt4d_p(
     const iree_amd_uk_mmt4d_params_t* params, void* stream);
 
+/* linalg.batch_mmt4d: `batch` mmt4d problems of the shape `params` gives, entry
+ * b on operands lying b * {lhs,rhs,out}_batch_stride elements after those of
+ * entry 0 (offsets added to params->*_offset). Replaces the loop the reference
+ * generates around its mmt4d ukernel: it tiles the batch dimension to 1 and
+ * rank-reduces each entry to mmt4d (REF compiler/src/iree/compiler/Codegen/
+ * Common/CPU/CPUPrepareUkernels.cpp:23-43 tileBatchDimsForBatchMmt4dOp,
+ * :165-245 ConvertBatchMmt4DtoMmt4DPattern), so every entry has exactly the
+ * result of iree_amd_uk_mmt4d_p on it. Matrix-core tiles whose batch strides
+ * are whole 16 bytes run as ONE launch (batch entries are planes of the grid;
+ * K is not split in it, so it allocates nothing); everything else runs as
+ * iree_amd_uk_mmt4d_p entry by entry. Entries must not overlap in `out`.
+ * batch == 0 does nothing. */
+IREE_AMD_UK_EXPORT int iree_amd_uk_batch_mmt4d(
+    const iree_amd_uk_mmt4d_params_t* params, iree_amd_uk_index_t batch,
+    iree_amd_uk_index_t lhs_batch_stride, iree_amd_uk_index_t rhs_batch_stride,
+    iree_amd_uk_index_t out_batch_stride, void* stream);
+
 /* Replaces REF mmt4d.h:23-25 / mmt4d.c:179-185 (iree_uk_mmt4d_info): bit 0 set
  * when a gfx950 MFMA kernel (not the generic one) serves this type and tile. */
 IREE_AMD_UK_EXPORT uint32_t iree_amd_uk_mmt4d_info(int32_t M0, int32_t N0,

@@ -254,6 +254,39 @@ extern "C" int iree_amd_uk_mmt4d(
   return iree_amd_uk_mmt4d_p(&p, stream);
 }
 
+extern "C" int iree_amd_uk_batch_mmt4d(const iree_amd_uk_mmt4d_params_t* params,
+                                       iree_amd_uk_index_t batch,
+                                       iree_amd_uk_index_t lhs_batch_stride,
+                                       iree_amd_uk_index_t rhs_batch_stride,
+                                       iree_amd_uk_index_t out_batch_stride, void* stream) {
+  if (!params) return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "batch_mmt4d: null params");
+  if (batch < 0) return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "batch_mmt4d: negative batch");
+  const iree_amd_uk_mmt4d_params_t& p = *params;
+  UK_RETURN_IF_ERROR(validate_mmt4d(p));
+  if (batch == 0) return 0;
+  if (batch == 1) return iree_amd_uk_mmt4d_p(params, stream);
+  // One launch over all batch entries where the matrix-core kernel takes the
+  // problem; the same early returns as a single mmt4d come first.
+  const bool nothing_to_do = p.M == 0 || p.N == 0 || p.M0 == 0 || p.N0 == 0 ||
+                             (p.K == 0 && (p.flags & IREE_AMD_UK_FLAG_MMT4D_ACCUMULATE));
+  if (nothing_to_do) return 0;
+  if (p.lhs_buffer && p.rhs_buffer && p.out_buffer && mmt4d_mfma_supported(p.flags, p.M0, p.N0, p.K0)) {
+    const int st = launch_batch_mmt4d_mfma(p, batch, lhs_batch_stride, rhs_batch_stride,
+                                           out_batch_stride, (hipStream_t)stream);
+    if (st != IREE_AMD_UK_STATUS_NOT_FOUND) return st;
+  }
+  // Otherwise entry by entry, the way the reference lowers the op (batch tiled
+  // to 1, then rank-reduced to mmt4d: CPUPrepareUkernels.cpp:23-43,165-245).
+  for (iree_amd_uk_index_t b = 0; b < batch; ++b) {
+    iree_amd_uk_mmt4d_params_t q = p;
+    q.lhs_offset += b * lhs_batch_stride;
+    q.rhs_offset += b * rhs_batch_stride;
+    q.out_offset += b * out_batch_stride;
+    UK_RETURN_IF_ERROR(iree_amd_uk_mmt4d_p(&q, stream));
+  }
+  return 0;
+}
+
 extern "C" uint32_t iree_amd_uk_mmt4d_info(int32_t M0, int32_t N0, int32_t K0,
                                            uint32_t flags,
                                            const uint64_t* cpu_data) {

@@ -195,6 +195,7 @@ int make_args(const iree_amd_uk_mmt4d_params_t& p, int out_elem_bytes, bool silu
   a.tail_tiles = (int)((k_elems % sv.mfma_k) / p.K0);
   a.tiles_m = a.tiles_n = 0;
   a.k_slices = 0; a.slice_ksteps = 0; a.slice_out_bytes = 0;
+  a.batch = 1; a.lhs_batch_bytes = a.rhs_batch_bytes = a.out_batch_bytes = 0;
   a.accumulate = (p.flags & IREE_AMD_UK_FLAG_MMT4D_ACCUMULATE) != 0;
   a.k0_div = sv.mfma_k / p.K0;
   a.row_major_out = 0; a.out_rows = a.out_cols = 0;
@@ -215,6 +216,34 @@ int launch_mmt4d_mfma(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) {
   const int st = make_args(p, ti.out_bytes, false, &a);
   if (st) return st;
   return launch_typed(p, a, s);
+}
+
+// `batch` mmt4d problems of one shape, operands `*_batch_stride` elements
+// apart: one launch whose workgroup planes are the batch entries (at most
+// 65535 planes a launch).
+int launch_batch_mmt4d_mfma(const iree_amd_uk_mmt4d_params_t& p, int64_t batch, int64_t lhs_batch_stride,
+                            int64_t rhs_batch_stride, int64_t out_batch_stride, hipStream_t s) {
+  Mmt4dTypeInfo ti;
+  mmt4d_type_info(p.flags, &ti);
+  MfmaArgs a;
+  const int st = make_args(p, ti.out_bytes, false, &a);
+  if (st) return st;
+  const int eb = ti.lhs_bits / 8;
+  a.lhs_batch_bytes = lhs_batch_stride * eb;
+  a.rhs_batch_bytes = rhs_batch_stride * eb;
+  a.out_batch_bytes = out_batch_stride * ti.out_bytes;
+  if (a.lhs_batch_bytes % 16 || a.rhs_batch_bytes % 16) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  const int64_t kPlanes = 65535;
+  for (int64_t b0 = 0; b0 < batch; b0 += kPlanes) {
+    MfmaArgs c = a;
+    c.batch = (int)(batch - b0 < kPlanes ? batch - b0 : kPlanes);
+    c.lhs = a.lhs + b0 * a.lhs_batch_bytes;
+    c.rhs = a.rhs + b0 * a.rhs_batch_bytes;
+    c.out = a.out + b0 * a.out_batch_bytes;
+    const int lst = launch_typed(p, c, s);
+    if (lst) return lst;      // (NOT_FOUND can only come from the first launch)
+  }
+  return 0;
 }
 
 // mmt4d whose result goes to a row-major out_rows x out_cols matrix (element

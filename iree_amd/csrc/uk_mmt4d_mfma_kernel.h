@@ -92,6 +92,10 @@ struct MfmaArgs {
   // out + y * slice_out_bytes
   int k_slices, slice_ksteps;
   int64_t slice_out_bytes;
+  // batch (launch side): workgroup plane blockIdx.z multiplies the operands
+  // that lie z * {lhs,rhs,out}_batch_bytes further on
+  int batch;
+  int64_t lhs_batch_bytes, rhs_batch_bytes, out_batch_bytes;
 };
 
 namespace {

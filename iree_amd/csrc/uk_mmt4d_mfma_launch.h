@@ -32,6 +32,10 @@ namespace {
 template <typename Cfg, int WM, int WN, int kRing, int kSync, int kOcc, bool kSiluMul, int kWavesN,
           int kForm>
 __global__ __launch_bounds__(128 * kWavesN, kOcc) void mmt4d_mfma_kernel(MfmaArgs a) {
+  // (plane blockIdx.z of a batch; the strides are 0 without one)
+  a.lhs += blockIdx.z * a.lhs_batch_bytes;
+  a.rhs += blockIdx.z * a.rhs_batch_bytes;
+  a.out += blockIdx.z * a.out_batch_bytes;
   mmt4d_mfma_body<Cfg, WM, WN, kRing, kSync, kSiluMul, kWavesN, kForm>(a);
 }
 
@@ -69,6 +73,7 @@ int launch_form(const MfmaArgs& a, unsigned blocks, hipStream_t s) {
   void (*kernel)(MfmaArgs) = nullptr;
   unsigned slices = 1;
   if (a.k_slices > 1) {
+    if (a.batch > 1) return IREE_AMD_UK_STATUS_NOT_FOUND;
     if constexpr (kCanSplit) {
       kernel = mmt4d_mfma_ksplit_kernel<Cfg, WM, WN, kRing, kSync, kOcc, kWavesN, kForm>;
       slices = (unsigned)a.k_slices;
@@ -88,7 +93,8 @@ int launch_form(const MfmaArgs& a, unsigned blocks, hipStream_t s) {
                                          hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes));
     if (dev >= 0 && dev < 64) set_on |= 1ull << dev;
   }
-  hipLaunchKernelGGL(kernel, dim3(blocks, slices), dim3(128 * kWavesN), lds_bytes, s, a);
+  hipLaunchKernelGGL(kernel, dim3(blocks, slices, a.batch > 1 ? (unsigned)a.batch : 1u), dim3(128 * kWavesN),
+                     lds_bytes, s, a);
   return check_hip(hipGetLastError(), "mmt4d_mfma launch");
 }
 
@@ -216,7 +222,8 @@ int launch_cfg(const MfmaArgs& a, hipStream_t s) {
   // cost of variant v on an M x N (outer tiles) problem
   auto cost_of = [&](int v, int64_t M, int64_t N, int64_t k_slices = 1) -> double {
     const Variant& t = variants[v];
-    const int64_t tiles = ceil_div(M, (int64_t)2 * t.wm) * ceil_div(N, (int64_t)2 * t.wn) * k_slices;
+    const int64_t tiles = ceil_div(M, (int64_t)2 * t.wm) * ceil_div(N, (int64_t)2 * t.wn) * k_slices *
+                          (a.batch > 1 ? a.batch : 1);
     const int64_t slots = (int64_t)t.occ * cus;
     const double work = t.wm * t.wn;
     double cost = (double)(tiles / slots) * t.occ * work / t.eff_full;
@@ -260,7 +267,7 @@ int launch_cfg(const MfmaArgs& a, hipStream_t s) {
   if constexpr (!kSiluMul) {
     const Variant& bv = variants[best];
     const int64_t best_tiles = ceil_div((int64_t)a.M, (int64_t)2 * bv.wm) * ceil_div((int64_t)a.N, (int64_t)2 * bv.wn);
-    if (a.k_slices == 0 && a.ksteps >= 64 && best_tiles * 2 <= (int64_t)bv.occ * cus) {
+    if (a.k_slices == 0 && a.batch <= 1 && a.ksteps >= 64 && best_tiles * 2 <= (int64_t)bv.occ * cus) {
       const double unit_us = Cfg::kStepUs / 16.0;
       const double out_mb = (double)a.M * a.N * 4096.0 / 1e6;
       double best_us = best_cost * a.ksteps * unit_us * 0.9;    // a split must win by 10 %
@@ -290,7 +297,7 @@ int launch_cfg(const MfmaArgs& a, hipStream_t s) {
   const int64_t rows0 = ceil_div((int64_t)a.M, (int64_t)8);   // macro-tile rows of the large tile
   const int64_t cols0 = ceil_div((int64_t)a.N, (int64_t)8);
   const int64_t rounds0 = rows0 * cols0 / cus;
-  if (rounds0 >= 1 && (int64_t)a.ksteps * Cfg::kMfmaK * Cfg::kElemBytes >= 2048) {
+  if (rounds0 >= 1 && a.batch <= 1 && (int64_t)a.ksteps * Cfg::kMfmaK * Cfg::kElemBytes >= 2048) {
     // split the longer dimension: `across` macro tiles lie across it
     const bool by_cols = cols0 >= rows0;
     const int64_t across = by_cols ? rows0 : cols0;

@@ -66,6 +66,32 @@ def mmt4d(lhs_buffer, rhs_buffer, out_buffer, M, N, K, M0, N0, K0, flags, *,
         K0, flags, None, _stream(stream)))
 
 
+def batch_mmt4d(lhs_buffer, rhs_buffer, out_buffer, batch, M, N, K, M0, N0, K0, flags, *,
+                lhs_offset=0, lhs_stride0=None, rhs_offset=0, rhs_stride0=None,
+                out_offset=0, out_stride0=None, lhs_batch_stride=None,
+                rhs_batch_stride=None, out_batch_stride=None, stream=None):
+    """linalg.batch_mmt4d: `batch` mmt4d problems of one shape, which the
+    reference runs as one mmt4d ukernel call per entry (reference
+    CPUPrepareUkernels.cpp:23-43,165-245). Strides default to tight."""
+    if lhs_stride0 is None:
+        lhs_stride0 = K * M0 * K0
+    if rhs_stride0 is None:
+        rhs_stride0 = K * N0 * K0
+    if out_stride0 is None:
+        out_stride0 = N * M0 * N0
+    if lhs_batch_stride is None:
+        lhs_batch_stride = M * lhs_stride0
+    if rhs_batch_stride is None:
+        rhs_batch_stride = N * rhs_stride0
+    if out_batch_stride is None:
+        out_batch_stride = M * out_stride0
+    p = Mmt4dParams(_ptr(lhs_buffer), lhs_offset, lhs_stride0, _ptr(rhs_buffer), rhs_offset,
+                    rhs_stride0, _ptr(out_buffer), out_offset, out_stride0, M, N, K, M0, N0,
+                    K0, flags, None)
+    _check(load_library().iree_amd_uk_batch_mmt4d(
+        C.byref(p), batch, lhs_batch_stride, rhs_batch_stride, out_batch_stride, _stream(stream)))
+
+
 def mmt4d_info(M0, N0, K0, flags):
     """iree_uk_mmt4d_info (reference mmt4d.h:23-25)."""
     return load_library().iree_amd_uk_mmt4d_info(M0, N0, K0, flags, None)

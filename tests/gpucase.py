@@ -31,6 +31,16 @@ def run_mmt4d(case, flags=None):
     return out.cpu().numpy().view(case.out_init.dtype)
 
 
+def run_batch_mmt4d(case):
+    lib = iree_amd.load_library()
+    lhs, rhs, out = _to_dev(case.lhs), _to_dev(case.rhs), _to_dev(case.out_init)
+    p = case.params(lhs.data_ptr(), rhs.data_ptr(), out.data_ptr())
+    _check(lib.iree_amd_uk_batch_mmt4d(C.byref(p), case.batch, case.lhs_batch_stride,
+                                       case.rhs_batch_stride, case.out_batch_stride, _stream()))
+    torch.cuda.synchronize()
+    return out.cpu().numpy().view(case.out_init.dtype)
+
+
 def run_pack(case):
     lib = iree_amd.load_library()
     inp, out = _to_dev(case.inp), _to_dev(case.out_init)

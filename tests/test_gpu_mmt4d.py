@@ -719,3 +719,80 @@ def test_matmul_packed_rhs_wide_result_packs_the_lhs_first(uk, cuda, accumulate)
         want = want + c0[:, :N]
     assert np.array_equal(got[:, :N], want)
     assert np.array_equal(got[:, N:], c0[:, N:])
+
+
+BATCH_CASES = [
+    # type, tile, batch, (M, N, K), gap (lhs, rhs, out) in elements
+    (F.MMT4D_TYPE_S8S8S32, (32, 32, 16), 3, (2, 3, 4), (0, 0, 0)),
+    (F.MMT4D_TYPE_S8S8S32, (32, 32, 16), 5, (9, 4, 19), (64, 32, 16)),
+    (F.MMT4D_TYPE_F16F16F32, (32, 32, 8), 4, (5, 7, 10), (16, 8, 4)),
+    (F.MMT4D_TYPE_F16F16F32, (32, 32, 8), 7, (1, 1, 2), (0, 0, 0)),
+    (F.MMT4D_TYPE_BF16BF16F32, (32, 32, 16), 2, (17, 9, 4), (0, 0, 0)),
+    (F.MMT4D_TYPE_F8E4M3F8E4M3F32, (32, 32, 16), 6, (3, 2, 6), (0, 0, 0)),
+    (F.MMT4D_TYPE_F32F32F32, (32, 32, 4), 3, (4, 5, 21), (0, 0, 0)),
+    (F.MMT4D_TYPE_F16F16F16, (32, 32, 8), 3, (2, 3, 3), (0, 0, 0)),
+    # long K and few macro tiles per entry (a single mmt4d would split K)
+    (F.MMT4D_TYPE_F16F16F32, (32, 32, 8), 2, (2, 2, 512), (0, 0, 0)),
+    # batch strides the matrix-core kernel cannot address (odd byte alignment):
+    # entry by entry
+    (F.MMT4D_TYPE_S8S8S32, (32, 32, 16), 3, (2, 3, 4), (3, 5, 1)),
+    # tiles of the element-wise kernel and of the narrow left-hand-side kernel
+    (F.MMT4D_TYPE_S8S8S32, (4, 6, 2), 3, (2, 3, 4), (1, 2, 3)),
+    (F.MMT4D_TYPE_F16F16F32, (8, 32, 8), 3, (1, 5, 12), (0, 0, 0)),
+    (F.MMT4D_TYPE_S16U4S32, (3, 5, 8), 2, (2, 3, 4), (0, 0, 0)),
+]
+
+
+@pytest.mark.parametrize("type_flag,tile,batch,shape,gap", BATCH_CASES)
+@pytest.mark.parametrize("acc", [False, True])
+def test_batch_mmt4d_bit_exact(uk, cuda, type_flag, tile, batch, shape, gap, acc):
+    """Every entry of a batch has the bits of the reference's per-entry mmt4d
+    call, and nothing between the entries is written."""
+    rng = np.random.default_rng(8100 + type_flag + batch + shape[2])
+    case = ukref.BatchMmt4dCase(rng, type_flag, batch, *shape, *tile, accumulate=acc, gap=gap)
+    got = gpucase.run_batch_mmt4d(case)
+    want = case.run_oracle(ukref.F16_IEEE)
+    assert np.array_equal(got.view(np.uint8), want.view(np.uint8))
+
+
+def test_batch_mmt4d_degenerate_and_large_batch(uk, cuda):
+    rng = np.random.default_rng(8200)
+    # batch == 0: nothing is touched
+    case = ukref.BatchMmt4dCase(rng, F.MMT4D_TYPE_S8S8S32, 0, 2, 2, 2, 32, 32, 16)
+    assert np.array_equal(gpucase.run_batch_mmt4d(case), case.out_init)
+    # K == 0 zero-fills every entry (accumulate: leaves them)
+    for acc in (False, True):
+        case = ukref.BatchMmt4dCase(rng, F.MMT4D_TYPE_S8S8S32, 3, 2, 2, 0, 32, 32, 16, accumulate=acc,
+                                    gap=(0, 0, 9))
+        assert np.array_equal(gpucase.run_batch_mmt4d(case), case.run_oracle())
+    # more entries than one launch has planes, shared right-hand side (batch stride 0)
+    M0 = N0 = 32
+    K0 = 16
+    batch = 65535 + 300
+    lhs = rng.integers(-128, 128, size=batch * M0 * K0, dtype=np.int8)
+    rhs = rng.integers(-128, 128, size=N0 * K0, dtype=np.int8)
+    import torch
+    from iree_amd import ukernel
+    d_lhs, d_rhs = torch.from_numpy(lhs).cuda(), torch.from_numpy(rhs).cuda()
+    d_out = torch.full((batch, M0, N0), 7, dtype=torch.int32, device="cuda")
+    ukernel.batch_mmt4d(d_lhs, d_rhs, d_out, batch, 1, 1, 1, M0, N0, K0, F.MMT4D_TYPE_S8S8S32,
+                        rhs_batch_stride=0)
+    want = lhs.reshape(batch, M0, K0).astype(np.int32) @ rhs.reshape(N0, K0).astype(np.int32).T
+    assert np.array_equal(d_out.cpu().numpy(), want)
+
+
+def test_batch_mmt4d_large_entries_match_single_calls(uk, cuda):
+    """At a size the oracle does not reach: a batch equals its entries run one
+    by one through iree_amd_uk_mmt4d (itself checked against the oracle)."""
+    import torch
+    from iree_amd import ukernel
+    g = torch.Generator(device="cuda").manual_seed(5)
+    batch, M, N, K, K0 = 6, 24, 20, 48, 8
+    lhs = torch.randn(batch, M, K, 32, K0, device="cuda", generator=g).half()
+    rhs = torch.randn(batch, N, K, 32, K0, device="cuda", generator=g).half()
+    out = torch.zeros(batch, M, N, 32, 32, device="cuda")
+    ukernel.batch_mmt4d(lhs, rhs, out, batch, M, N, K, 32, 32, K0, F.MMT4D_TYPE_F16F16F32)
+    for b in range(batch):
+        one = torch.zeros(M, N, 32, 32, device="cuda")
+        ukernel.mmt4d(lhs[b], rhs[b], one, M, N, K, 32, 32, K0, F.MMT4D_TYPE_F16F16F32)
+        assert torch.equal(out[b], one), b

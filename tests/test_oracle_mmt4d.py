@@ -1,6 +1,7 @@
 """Pins oracle_mmt4d: against the compiled reference library (bit-exact, the
 reference's own shape/tile/flag matrix of tools/mmt4d_test.c:459-608), against
 an independent numpy einsum, and through tile-shape invariance."""
+import ctypes as C
 import itertools
 
 import numpy as np
@@ -211,3 +212,41 @@ def test_oracle_rejects_what_the_reference_asserts_on():
                  flags=F.MMT4D_TYPE_S8S4S32)
     p.K0 = 3  # 3 x 4 bits is not a whole number of bytes
     assert ukref.oracle().oracle_mmt4d(C.byref(p), 0) == F.STATUS_INVALID_ARGUMENT
+
+
+def test_batch_oracle_is_one_mmt4d_per_entry_and_matches_numpy():
+    """linalg.batch_mmt4d restated as the loop the reference lowers it to; the
+    einsum over the batch pins the entry offsets (a wrong batch stride or a
+    dropped entry changes the sums) and untouched gaps pin the extents."""
+    rng = np.random.default_rng(77)
+    for tf, tile in ((F.MMT4D_TYPE_S8S8S32, (4, 6, 2)), (F.MMT4D_TYPE_F16F16F32, (32, 32, 8)),
+                     (F.MMT4D_TYPE_S8S8S32, (32, 32, 16))):
+        for acc in (False, True):
+            case = ukref.BatchMmt4dCase(rng, tf, 3, 2, 3, 4, *tile, accumulate=acc,
+                                        gap=(5, 3, 7), offsets=True)
+            out = case.run_oracle()
+            got = case.written_regions(out).astype(np.float64)
+            want = case.run_numpy().astype(np.float64)
+            if acc:
+                want = want + case.written_regions(case.out_init).astype(np.float64)
+            assert np.array_equal(got, want)
+            # nothing outside the batch entries is written
+            mask = np.ones(out.size, bool)
+            M, N, K, M0, N0, K0 = case.dims
+            for b in range(case.batch):
+                for i in range(M):
+                    o = case.out_offset + b * case.out_batch_stride + i * case.out_stride0
+                    mask[o:o + N * M0 * N0] = False
+            assert np.array_equal(out[mask], case.out_init[mask])
+            # and against the real reference library, entry by entry
+            lib = ukref.reflib()
+            if lib is not None:
+                ref = case.out_init.copy()
+                for b in range(case.batch):
+                    p = case.entry_params(b, 0, 0, 0)
+                    lib.iree_uk_mmt4d(ukref.ptr(case.lhs), p.lhs_offset, p.lhs_stride0,
+                                      ukref.ptr(case.rhs), p.rhs_offset, p.rhs_stride0,
+                                      ukref.ptr(ref), p.out_offset, p.out_stride0,
+                                      M, N, K, M0, N0, K0, case.flags,
+                                      C.cast(ukref.cpu_data(""), C.c_void_p))
+                assert np.array_equal(ref, out)

@@ -358,6 +358,65 @@ class Mmt4dCase:
         return np.stack(rows).reshape(M, N, M0, N0) if M else np.zeros((0, N, M0, N0), out.dtype)
 
 
+class BatchMmt4dCase(Mmt4dCase):
+    """`batch` mmt4d problems of one shape (linalg.batch_mmt4d). The oracle runs
+    them the way the reference lowers the op: one mmt4d call per batch entry on
+    rank-reduced slices (compiler/src/iree/compiler/Codegen/Common/CPU/
+    CPUPrepareUkernels.cpp:23-43,165-245). `gap`: elements between the end of
+    one entry and the start of the next, per operand (lhs, rhs, out)."""
+
+    def __init__(self, rng, type_flag, batch, M, N, K, M0, N0, K0, accumulate=False,
+                 gap=(0, 0, 0), offsets=False, generator=random_operand):
+        super().__init__(rng, type_flag, M, N, K, M0, N0, K0, accumulate=accumulate,
+                         offsets=offsets, generator=generator)
+        self.batch = batch
+        self.lhs_batch_stride = M * self.lhs_stride0 + gap[0]
+        self.rhs_batch_stride = N * self.rhs_stride0 + gap[1]
+        self.out_batch_stride = M * self.out_stride0 + gap[2]
+        nb = max(batch, 1)
+        self.lhs = generator(rng, type_flag, 0, self.lhs_offset + nb * self.lhs_batch_stride + 1)
+        self.rhs = generator(rng, type_flag, 1, self.rhs_offset + nb * self.rhs_batch_stride + 2)
+        self.out_init = generator(rng, type_flag, 2, self.out_offset + nb * self.out_batch_stride + 1)
+
+    def entry_params(self, b, lhs_ptr, rhs_ptr, out_ptr):
+        p = self.params(lhs_ptr, rhs_ptr, out_ptr)
+        p.lhs_offset += b * self.lhs_batch_stride
+        p.rhs_offset += b * self.rhs_batch_stride
+        p.out_offset += b * self.out_batch_stride
+        return p
+
+    def run_oracle(self, f16_mode=F16_IEEE, f64=False):
+        out = self.out_init.copy()
+        for b in range(self.batch):
+            p = self.entry_params(b, ptr(self.lhs).value, ptr(self.rhs).value, ptr(out).value)
+            st = oracle().oracle_mmt4d_f64(C.byref(p)) if f64 else \
+                oracle().oracle_mmt4d(C.byref(p), f16_mode)
+            assert st == 0, f"oracle_mmt4d status {st}"
+        return out
+
+    def run_numpy(self):
+        """(batch, M, N, M0, N0) products by einsum in int64 / float64."""
+        M, N, K, M0, N0, K0 = self.dims
+        lhs_all = decode_operand(self.type_flag, 0, self.lhs, self.lhs.size)
+        rhs_all = decode_operand(self.type_flag, 1, self.rhs, self.rhs.size)
+        res = []
+        for b in range(self.batch):
+            lo = self.lhs_offset + b * self.lhs_batch_stride
+            ro = self.rhs_offset + b * self.rhs_batch_stride
+            lhs = np.stack([lhs_all[lo + i * self.lhs_stride0:][:K * M0 * K0]
+                            for i in range(M)]).reshape(M, K, M0, K0)
+            rhs = np.stack([rhs_all[ro + j * self.rhs_stride0:][:K * N0 * K0]
+                            for j in range(N)]).reshape(N, K, N0, K0)
+            res.append(np.einsum("ikac,jkbc->ijab", lhs, rhs))
+        return np.stack(res)
+
+    def written_regions(self, out):
+        M, N, K, M0, N0, K0 = self.dims
+        return np.stack([
+            np.stack([out[self.out_offset + b * self.out_batch_stride + i * self.out_stride0:][:N * M0 * N0]
+                      for i in range(M)]).reshape(M, N, M0, N0) for b in range(self.batch)])
+
+
 PACK_NP_DTYPE = {F.PACK_TYPE_F32F32: np.uint32, F.PACK_TYPE_I8I8: np.uint8,
                  F.PACK_TYPE_I32I32: np.uint32, F.PACK_TYPE_F16F16: np.uint16,
                  F.PACK_TYPE_BF16BF16: np.uint16}
