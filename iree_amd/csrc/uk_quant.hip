@@ -101,55 +101,49 @@ __global__ __launch_bounds__(kThreads) void dequant_matmul_i4_kernel(I4Args a) {
     return __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, soff_wave + sp * a.span_stride + h * half_stride, 0);
   };
 
-  // ---- request x, then the first tile's parameters and weights ------------
-  // Loads return in order: with the (small) activations first, their
-  // permutation runs while the weights are still in flight and the first
-  // MFMA can start as soon as the first slab lands.
+  // ---- request the first tile's parameters, then x and the weights span by
+  // span -------------------------------------------------------------------
+  // Loads return in order. Every workgroup reads all of x (from L2: 256 KiB at
+  // 32 rows, which takes several microseconds with all workgroups at it) but
+  // only a tile or two of weights, so the order of the requests decides how
+  // much of the weight stream overlaps the fetch of x: span 0 of x, span 0 of
+  // the weights, span 1 of x, ... The first tile permutes and multiplies span
+  // sp as soon as it has landed, and as it frees the span's weight registers
+  // it requests the same span of the NEXT tile, which so streams from HBM
+  // while the later spans of x still arrive.
   // activations: rows m_base + mh*16 + nl, this wave's K slice; rows past M
   // are read from the last row and zeroed.
-  u32x4 xraw[MH][SP][4];
-  {
-    const int cq = a.tiled ? 32 : 8, ckc = a.tiled ? 8 : 32;   // chunk strides in k
-#pragma unroll
-    for (int mh = 0; mh < MH; ++mh) {
-      const int m = a.m_base + mh * 16 + nl;
-      const int mr = m < a.M ? m : a.M - 1;
-      const uint16_t* row = a.x + (size_t)mr * a.K + k_slice + kc * ckc;
-#pragma unroll
-      for (int sp = 0; sp < SP; ++sp)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) xraw[mh][sp][q] = *(const u32x4*)(row + sp * 128 + q * cq);
-    }
-  }
-  __builtin_amdgcn_sched_barrier(0);
   int nt = blockIdx.x;
   Meta meta_next;
-  u32x4 wreg[SP][2];
   load_meta(nt < a.n_tiles ? nt : a.n_tiles - 1, meta_next);
+  u32x4 xraw[MH][SP][4];
+  u32x4 wreg[SP][2];
   {
+    const int cq = a.tiled ? 32 : 8, ckc = a.tiled ? 8 : 32;   // chunk strides in k
     const __amdgpu_buffer_rsrc_t rsrc = tile_rsrc(nt);
 #pragma unroll
-    for (int sp = 0; sp < SP; ++sp)
+    for (int sp = 0; sp < SP; ++sp) {
+#pragma unroll
+      for (int mh = 0; mh < MH; ++mh) {
+        const int m = a.m_base + mh * 16 + nl;
+        const int mr = m < a.M ? m : a.M - 1;
+        const uint16_t* row = a.x + (size_t)mr * a.K + k_slice + kc * ckc;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) xraw[mh][sp][q] = *(const u32x4*)(row + sp * 128 + q * cq);
+      }
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int h = 0; h < 2; ++h) wreg[sp][h] = load_slab(rsrc, sp, h);
+      __builtin_amdgcn_sched_barrier(0);
+    }
   }
-  __builtin_amdgcn_sched_barrier(0);
   half8 xf[MH][SP][4];
-#pragma unroll
-  for (int mh = 0; mh < MH; ++mh) {
-    const uint32_t keep = a.m_base + mh * 16 + nl < a.M ? 0xFFFFFFFFu : 0u;
-#pragma unroll
-    for (int sp = 0; sp < SP; ++sp)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        u32x4 v = xraw[mh][sp][q];
-        v.x &= keep; v.y &= keep; v.z &= keep; v.w &= keep;
-        xf[mh][sp][q] = permute_x(v);
-      }
-  }
 
   int parity = 0;
-  for (; nt < a.n_tiles; nt += gridDim.x, parity ^= 1) {
+  // One tile; `first`: the workgroup's first, which turns each span of x into
+  // MFMA operands when it gets to it.
+  auto tile = [&](auto first) {
+    constexpr bool kFirst = decltype(first)::value;
     const int next = nt + gridDim.x;
     const Meta mt = meta_next;
     load_meta(next < a.n_tiles ? next : a.n_tiles - 1, meta_next);
@@ -162,6 +156,18 @@ __global__ __launch_bounds__(kThreads) void dequant_matmul_i4_kernel(I4Args a) {
       for (int mh = 0; mh < MH; ++mh) acc[h][mh] = part[h][mh] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int sp = 0; sp < SP; ++sp) {
+      if constexpr (kFirst) {
+#pragma unroll
+        for (int mh = 0; mh < MH; ++mh) {
+          const uint32_t keep = a.m_base + mh * 16 + nl < a.M ? 0xFFFFFFFFu : 0u;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            u32x4 v = xraw[mh][sp][q];
+            v.x &= keep; v.y &= keep; v.z &= keep; v.w &= keep;
+            xf[mh][sp][q] = permute_x(v);
+          }
+        }
+      }
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
         const u32x4 wv = wreg[sp][h];
@@ -242,7 +248,13 @@ __global__ __launch_bounds__(kThreads) void dequant_matmul_i4_kernel(I4Args a) {
     }
     // The other half of `partial` is used by the next tile; this half is
     // rewritten only two tiles later, after the next tile's barrier.
+  };
+  if (nt < a.n_tiles) {
+    tile(std::true_type{});
+    nt += gridDim.x;
+    parity ^= 1;
   }
+  for (; nt < a.n_tiles; nt += gridDim.x, parity ^= 1) tile(std::false_type{});
 }
 
 // Row-major [N][K/2] bytes -> the tiled layout (one thread per dword).
