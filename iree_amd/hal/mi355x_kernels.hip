@@ -26,8 +26,11 @@
 // Launch shape, fixed per export (workgroup_size and workgroup_local_memory of
 // the hal.executable.export): 256 threads; the dynamic LDS size and the macro
 // tile T (outer tiles of 32 rows per workgroup, both ways) are those of the
-// table at the end of this file. The grid is one-dimensional:
-// ceildiv(M, T) * ceildiv(N, T) workgroups.
+// table at the end of this file. The grid is ceildiv(M, T) * ceildiv(N, T)
+// workgroups in x; in y it is 1, or the batch count of a linalg.batch_mmt4d:
+// workgroup plane y works on the y-th of `batch` dense problems laid one after
+// the other in each binding ([batch][M][K][32][K0] and so on; the row-major
+// result of mi355x_mmt4d_unpack_* is [batch][out_rows][out_cols]).
 //
 // mi355x_matmul_packed_rhs_*: the whole linear layer out[M][N] (+)= lhs[M][K] *
 // rhs in one dispatch: bindings 0 lhs, the dense row-major M x K matrix (read
@@ -95,6 +98,11 @@ __device__ __forceinline__ void hal_mmt4d(const void* lhs, const void* rhs, void
   a.gate_scale = a.up_scale = a.inv_out_scale = a.out_scale = 1.0f;
   // a grid larger than the tile count (a count region that rounds up) is harmless
   if (K < 1 || (int)blockIdx.x >= a.tiles_m * a.tiles_n) return;
+  // batch entry blockIdx.y of dense operands
+  const int64_t plane = blockIdx.y;
+  a.lhs += plane * M * a.lhs_stride_bytes;
+  a.rhs += plane * N * a.rhs_stride_bytes;
+  a.out += plane * (row_major ? out_rows : M) * a.out_stride_bytes;
   mmt4d_mfma_body<Cfg, WM, WN, kRing, kSync, false, 2, row_major ? 1 : 0>(a);
 }
 

@@ -7,7 +7,8 @@
 // Every mmt4d export: bindings lhs (read only), rhs (read only), out; push constants
 // M, N, K (outer tile counts), K0, flags (0x100 = accumulate), and for
 // mi355x_mmt4d_unpack_* also out_rows, out_cols. The workload of a dispatch is
-// (M, N).
+// (M, N, batch): batch = 1 for linalg.mmt4d, the batch size of a
+// linalg.batch_mmt4d on dense operands (workgroup planes in y).
 
 #rocm_gfx950_target = #hal.executable.target<"rocm", "rocm-hsaco-fb", {
   target_arch = "gfx950"
@@ -31,10 +32,10 @@ hal.executable.source public @mi355x_mmt4d attributes {
     workgroup_size = [256 : index, 1 : index, 1 : index],
     workgroup_local_memory = 163840 : index
   } {
-  ^bb0(%device: !hal.device, %m: index, %n: index):
+  ^bb0(%device: !hal.device, %m: index, %n: index, %batch: index):
     %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 8) * (s1 ceildiv 8))>()[%m, %n]
     %c1 = arith.constant 1 : index
-    hal.return %x, %c1, %c1 : index, index, index
+    hal.return %x, %batch, %c1 : index, index, index
   }
   hal.executable.export public @mi355x_mmt4d_unpack_f16f16f32_t8 ordinal(1)
       layout(#hal.pipeline.layout<push_constants = 7, sets = [
@@ -47,10 +48,10 @@ hal.executable.source public @mi355x_mmt4d attributes {
     workgroup_size = [256 : index, 1 : index, 1 : index],
     workgroup_local_memory = 163840 : index
   } {
-  ^bb0(%device: !hal.device, %m: index, %n: index):
+  ^bb0(%device: !hal.device, %m: index, %n: index, %batch: index):
     %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 8) * (s1 ceildiv 8))>()[%m, %n]
     %c1 = arith.constant 1 : index
-    hal.return %x, %c1, %c1 : index, index, index
+    hal.return %x, %batch, %c1 : index, index, index
   }
   hal.executable.export public @mi355x_mmt4d_f16f16f32_t4 ordinal(2)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
@@ -63,10 +64,10 @@ hal.executable.source public @mi355x_mmt4d attributes {
     workgroup_size = [256 : index, 1 : index, 1 : index],
     workgroup_local_memory = 65536 : index
   } {
-  ^bb0(%device: !hal.device, %m: index, %n: index):
+  ^bb0(%device: !hal.device, %m: index, %n: index, %batch: index):
     %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 4) * (s1 ceildiv 4))>()[%m, %n]
     %c1 = arith.constant 1 : index
-    hal.return %x, %c1, %c1 : index, index, index
+    hal.return %x, %batch, %c1 : index, index, index
   }
   hal.executable.export public @mi355x_mmt4d_unpack_f16f16f32_t4 ordinal(3)
       layout(#hal.pipeline.layout<push_constants = 7, sets = [
@@ -79,10 +80,10 @@ hal.executable.source public @mi355x_mmt4d attributes {
     workgroup_size = [256 : index, 1 : index, 1 : index],
     workgroup_local_memory = 65536 : index
   } {
-  ^bb0(%device: !hal.device, %m: index, %n: index):
+  ^bb0(%device: !hal.device, %m: index, %n: index, %batch: index):
     %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 4) * (s1 ceildiv 4))>()[%m, %n]
     %c1 = arith.constant 1 : index
-    hal.return %x, %c1, %c1 : index, index, index
+    hal.return %x, %batch, %c1 : index, index, index
   }
   hal.executable.export public @mi355x_mmt4d_bf16bf16f32_t8 ordinal(4)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
@@ -95,10 +96,10 @@ hal.executable.source public @mi355x_mmt4d attributes {
     workgroup_size = [256 : index, 1 : index, 1 : index],
     workgroup_local_memory = 163840 : index
   } {
-  ^bb0(%device: !hal.device, %m: index, %n: index):
+  ^bb0(%device: !hal.device, %m: index, %n: index, %batch: index):
     %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 8) * (s1 ceildiv 8))>()[%m, %n]
     %c1 = arith.constant 1 : index
-    hal.return %x, %c1, %c1 : index, index, index
+    hal.return %x, %batch, %c1 : index, index, index
   }
   hal.executable.export public @mi355x_mmt4d_unpack_bf16bf16f32_t8 ordinal(5)
       layout(#hal.pipeline.layout<push_constants = 7, sets = [
@@ -111,10 +112,10 @@ hal.executable.source public @mi355x_mmt4d attributes {
     workgroup_size = [256 : index, 1 : index, 1 : index],
     workgroup_local_memory = 163840 : index
   } {
-  ^bb0(%device: !hal.device, %m: index, %n: index):
+  ^bb0(%device: !hal.device, %m: index, %n: index, %batch: index):
     %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 8) * (s1 ceildiv 8))>()[%m, %n]
     %c1 = arith.constant 1 : index
-    hal.return %x, %c1, %c1 : index, index, index
+    hal.return %x, %batch, %c1 : index, index, index
   }
   hal.executable.export public @mi355x_mmt4d_bf16bf16f32_t4 ordinal(6)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
@@ -127,10 +128,10 @@ hal.executable.source public @mi355x_mmt4d attributes {
     workgroup_size = [256 : index, 1 : index, 1 : index],
     workgroup_local_memory = 65536 : index
   } {
-  ^bb0(%device: !hal.device, %m: index, %n: index):
+  ^bb0(%device: !hal.device, %m: index, %n: index, %batch: index):
     %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 4) * (s1 ceildiv 4))>()[%m, %n]
     %c1 = arith.constant 1 : index
-    hal.return %x, %c1, %c1 : index, index, index
+    hal.return %x, %batch, %c1 : index, index, index
   }
   hal.executable.export public @mi355x_mmt4d_unpack_bf16bf16f32_t4 ordinal(7)
       layout(#hal.pipeline.layout<push_constants = 7, sets = [
@@ -143,10 +144,10 @@ hal.executable.source public @mi355x_mmt4d attributes {
     workgroup_size = [256 : index, 1 : index, 1 : index],
     workgroup_local_memory = 65536 : index
   } {
-  ^bb0(%device: !hal.device, %m: index, %n: index):
+  ^bb0(%device: !hal.device, %m: index, %n: index, %batch: index):
     %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 4) * (s1 ceildiv 4))>()[%m, %n]
     %c1 = arith.constant 1 : index
-    hal.return %x, %c1, %c1 : index, index, index
+    hal.return %x, %batch, %c1 : index, index, index
   }
   hal.executable.export public @mi355x_mmt4d_s8s8s32_t8 ordinal(8)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
@@ -159,10 +160,10 @@ hal.executable.source public @mi355x_mmt4d attributes {
     workgroup_size = [256 : index, 1 : index, 1 : index],
     workgroup_local_memory = 131072 : index
   } {
-  ^bb0(%device: !hal.device, %m: index, %n: index):
+  ^bb0(%device: !hal.device, %m: index, %n: index, %batch: index):
     %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 8) * (s1 ceildiv 8))>()[%m, %n]
     %c1 = arith.constant 1 : index
-    hal.return %x, %c1, %c1 : index, index, index
+    hal.return %x, %batch, %c1 : index, index, index
   }
   hal.executable.export public @mi355x_mmt4d_unpack_s8s8s32_t8 ordinal(9)
       layout(#hal.pipeline.layout<push_constants = 7, sets = [
@@ -175,10 +176,10 @@ hal.executable.source public @mi355x_mmt4d attributes {
     workgroup_size = [256 : index, 1 : index, 1 : index],
     workgroup_local_memory = 131072 : index
   } {
-  ^bb0(%device: !hal.device, %m: index, %n: index):
+  ^bb0(%device: !hal.device, %m: index, %n: index, %batch: index):
     %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 8) * (s1 ceildiv 8))>()[%m, %n]
     %c1 = arith.constant 1 : index
-    hal.return %x, %c1, %c1 : index, index, index
+    hal.return %x, %batch, %c1 : index, index, index
   }
   hal.executable.export public @mi355x_mmt4d_s8s8s32_t4 ordinal(10)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
@@ -191,10 +192,10 @@ hal.executable.source public @mi355x_mmt4d attributes {
     workgroup_size = [256 : index, 1 : index, 1 : index],
     workgroup_local_memory = 65536 : index
   } {
-  ^bb0(%device: !hal.device, %m: index, %n: index):
+  ^bb0(%device: !hal.device, %m: index, %n: index, %batch: index):
     %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 4) * (s1 ceildiv 4))>()[%m, %n]
     %c1 = arith.constant 1 : index
-    hal.return %x, %c1, %c1 : index, index, index
+    hal.return %x, %batch, %c1 : index, index, index
   }
   hal.executable.export public @mi355x_mmt4d_unpack_s8s8s32_t4 ordinal(11)
       layout(#hal.pipeline.layout<push_constants = 7, sets = [
@@ -207,10 +208,10 @@ hal.executable.source public @mi355x_mmt4d attributes {
     workgroup_size = [256 : index, 1 : index, 1 : index],
     workgroup_local_memory = 65536 : index
   } {
-  ^bb0(%device: !hal.device, %m: index, %n: index):
+  ^bb0(%device: !hal.device, %m: index, %n: index, %batch: index):
     %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 4) * (s1 ceildiv 4))>()[%m, %n]
     %c1 = arith.constant 1 : index
-    hal.return %x, %c1, %c1 : index, index, index
+    hal.return %x, %batch, %c1 : index, index, index
   }
   hal.executable.export public @mi355x_mmt4d_f8e4m3f8e4m3f32_t8 ordinal(12)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
@@ -223,10 +224,10 @@ hal.executable.source public @mi355x_mmt4d attributes {
     workgroup_size = [256 : index, 1 : index, 1 : index],
     workgroup_local_memory = 163840 : index
   } {
-  ^bb0(%device: !hal.device, %m: index, %n: index):
+  ^bb0(%device: !hal.device, %m: index, %n: index, %batch: index):
     %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 8) * (s1 ceildiv 8))>()[%m, %n]
     %c1 = arith.constant 1 : index
-    hal.return %x, %c1, %c1 : index, index, index
+    hal.return %x, %batch, %c1 : index, index, index
   }
   hal.executable.export public @mi355x_mmt4d_unpack_f8e4m3f8e4m3f32_t8 ordinal(13)
       layout(#hal.pipeline.layout<push_constants = 7, sets = [
@@ -239,10 +240,10 @@ hal.executable.source public @mi355x_mmt4d attributes {
     workgroup_size = [256 : index, 1 : index, 1 : index],
     workgroup_local_memory = 163840 : index
   } {
-  ^bb0(%device: !hal.device, %m: index, %n: index):
+  ^bb0(%device: !hal.device, %m: index, %n: index, %batch: index):
     %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 8) * (s1 ceildiv 8))>()[%m, %n]
     %c1 = arith.constant 1 : index
-    hal.return %x, %c1, %c1 : index, index, index
+    hal.return %x, %batch, %c1 : index, index, index
   }
   hal.executable.export public @mi355x_mmt4d_f8e4m3f8e4m3f32_t4 ordinal(14)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
@@ -255,10 +256,10 @@ hal.executable.source public @mi355x_mmt4d attributes {
     workgroup_size = [256 : index, 1 : index, 1 : index],
     workgroup_local_memory = 131072 : index
   } {
-  ^bb0(%device: !hal.device, %m: index, %n: index):
+  ^bb0(%device: !hal.device, %m: index, %n: index, %batch: index):
     %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 4) * (s1 ceildiv 4))>()[%m, %n]
     %c1 = arith.constant 1 : index
-    hal.return %x, %c1, %c1 : index, index, index
+    hal.return %x, %batch, %c1 : index, index, index
   }
   hal.executable.export public @mi355x_mmt4d_unpack_f8e4m3f8e4m3f32_t4 ordinal(15)
       layout(#hal.pipeline.layout<push_constants = 7, sets = [
@@ -271,10 +272,10 @@ hal.executable.source public @mi355x_mmt4d attributes {
     workgroup_size = [256 : index, 1 : index, 1 : index],
     workgroup_local_memory = 131072 : index
   } {
-  ^bb0(%device: !hal.device, %m: index, %n: index):
+  ^bb0(%device: !hal.device, %m: index, %n: index, %batch: index):
     %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 4) * (s1 ceildiv 4))>()[%m, %n]
     %c1 = arith.constant 1 : index
-    hal.return %x, %c1, %c1 : index, index, index
+    hal.return %x, %batch, %c1 : index, index, index
   }
   hal.executable.export public @mi355x_mmt4d_f32f32f32_t8 ordinal(16)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
@@ -287,10 +288,10 @@ hal.executable.source public @mi355x_mmt4d attributes {
     workgroup_size = [256 : index, 1 : index, 1 : index],
     workgroup_local_memory = 131072 : index
   } {
-  ^bb0(%device: !hal.device, %m: index, %n: index):
+  ^bb0(%device: !hal.device, %m: index, %n: index, %batch: index):
     %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 8) * (s1 ceildiv 8))>()[%m, %n]
     %c1 = arith.constant 1 : index
-    hal.return %x, %c1, %c1 : index, index, index
+    hal.return %x, %batch, %c1 : index, index, index
   }
   hal.executable.export public @mi355x_mmt4d_unpack_f32f32f32_t8 ordinal(17)
       layout(#hal.pipeline.layout<push_constants = 7, sets = [
@@ -303,10 +304,10 @@ hal.executable.source public @mi355x_mmt4d attributes {
     workgroup_size = [256 : index, 1 : index, 1 : index],
     workgroup_local_memory = 131072 : index
   } {
-  ^bb0(%device: !hal.device, %m: index, %n: index):
+  ^bb0(%device: !hal.device, %m: index, %n: index, %batch: index):
     %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 8) * (s1 ceildiv 8))>()[%m, %n]
     %c1 = arith.constant 1 : index
-    hal.return %x, %c1, %c1 : index, index, index
+    hal.return %x, %batch, %c1 : index, index, index
   }
   hal.executable.export public @mi355x_mmt4d_f32f32f32_t4 ordinal(18)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
@@ -319,10 +320,10 @@ hal.executable.source public @mi355x_mmt4d attributes {
     workgroup_size = [256 : index, 1 : index, 1 : index],
     workgroup_local_memory = 65536 : index
   } {
-  ^bb0(%device: !hal.device, %m: index, %n: index):
+  ^bb0(%device: !hal.device, %m: index, %n: index, %batch: index):
     %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 4) * (s1 ceildiv 4))>()[%m, %n]
     %c1 = arith.constant 1 : index
-    hal.return %x, %c1, %c1 : index, index, index
+    hal.return %x, %batch, %c1 : index, index, index
   }
   hal.executable.export public @mi355x_mmt4d_unpack_f32f32f32_t4 ordinal(19)
       layout(#hal.pipeline.layout<push_constants = 7, sets = [
@@ -335,10 +336,10 @@ hal.executable.source public @mi355x_mmt4d attributes {
     workgroup_size = [256 : index, 1 : index, 1 : index],
     workgroup_local_memory = 65536 : index
   } {
-  ^bb0(%device: !hal.device, %m: index, %n: index):
+  ^bb0(%device: !hal.device, %m: index, %n: index, %batch: index):
     %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 4) * (s1 ceildiv 4))>()[%m, %n]
     %c1 = arith.constant 1 : index
-    hal.return %x, %c1, %c1 : index, index, index
+    hal.return %x, %batch, %c1 : index, index, index
   }
   // out[M][N] (+)= lhs[M][K] * rhs (packed); push constants M, N, K (elements), K0, flags; workload (M, N)
   hal.executable.export public @mi355x_matmul_packed_rhs_f16f16f32_t4x8 ordinal(20)
@@ -635,7 +636,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
 }
 
 // A dispatch site (f16, 4096^3: M = N = 128 outer tiles, K = 512 tiles of K0 = 8):
-//   %out = flow.dispatch @mi355x_mmt4d::@mi355x_mmt4d_f16f16f32_t8[%c128, %c128](
+//   %out = flow.dispatch @mi355x_mmt4d::@mi355x_mmt4d_f16f16f32_t8[%c128, %c128, %c1](
 //       %c128_i32, %c128_i32, %c512_i32, %c8_i32, %c0_i32, %lhs, %rhs)
 //     : (i32, i32, i32, i32, i32, tensor<128x512x32x8xf16>, tensor<128x512x32x8xf16>)
 //       -> tensor<128x128x32x32xf32>

@@ -146,14 +146,15 @@ class HalExecutable:
             ptrs, len(bindings), consts, len(push_constants), _stream(stream)))
 
     def mmt4d(self, name, lhs, rhs, out, M, N, K, K0, flags, out_rows=None, out_cols=None,
-              stream=None):
+              batch=1, stream=None):
         """One mmt4d export over dense operands (see the table in
-        iree_amd/hal/mi355x_kernels.hip for the layouts)."""
+        iree_amd/hal/mi355x_kernels.hip for the layouts); `batch` problems laid
+        one after the other in each binding run as workgroup planes in y."""
         e = EXPORTS[name]
         consts = [M, N, K, K0, flags]
         if "_unpack_" in name:
             consts += [out_rows, out_cols]
-        self.dispatch(name, workgroup_count(e, M, N), [lhs, rhs, out], consts, stream)
+        self.dispatch(name, (workgroup_count(e, M, N), batch, 1), [lhs, rhs, out], consts, stream)
 
     def matmul_packed_rhs(self, name, lhs, rhs_packed, out, M, N, K, K0, flags, stream=None):
         """mi355x_matmul_packed_rhs_*: out[M][N] (+)= lhs[M][K] * rhs, all dense,
@@ -196,7 +197,8 @@ _MLIR_HEADER = """\
 // Every mmt4d export: bindings lhs (read only), rhs (read only), out; push constants
 // M, N, K (outer tile counts), K0, flags (0x100 = accumulate), and for
 // mi355x_mmt4d_unpack_* also out_rows, out_cols. The workload of a dispatch is
-// (M, N).
+// (M, N, batch): batch = 1 for linalg.mmt4d, the batch size of a
+// linalg.batch_mmt4d on dense operands (workgroup planes in y).
 
 #rocm_gfx950_target = #hal.executable.target<"rocm", "rocm-hsaco-fb", {
   target_arch = "gfx950"
@@ -223,10 +225,10 @@ _MLIR_EXPORT = """\
     workgroup_size = [{wg} : index, 1 : index, 1 : index],
     workgroup_local_memory = {lds} : index
   }} {{
-  ^bb0(%device: !hal.device, %m: index, %n: index):
+  ^bb0(%device: !hal.device, %m: index, %n: index, %batch: index):
     %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv {tile}) * (s1 ceildiv {tile}))>()[%m, %n]
     %c1 = arith.constant 1 : index
-    hal.return %x, %c1, %c1 : index, index, index
+    hal.return %x, %batch, %c1 : index, index, index
   }}
 """
 
@@ -289,7 +291,7 @@ _MLIR_FOOTER = """\
 }
 
 // A dispatch site (f16, 4096^3: M = N = 128 outer tiles, K = 512 tiles of K0 = 8):
-//   %out = flow.dispatch @mi355x_mmt4d::@mi355x_mmt4d_f16f16f32_t8[%c128, %c128](
+//   %out = flow.dispatch @mi355x_mmt4d::@mi355x_mmt4d_f16f16f32_t8[%c128, %c128, %c1](
 //       %c128_i32, %c128_i32, %c512_i32, %c8_i32, %c0_i32, %lhs, %rhs)
 //     : (i32, i32, i32, i32, i32, tensor<128x512x32x8xf16>, tensor<128x512x32x8xf16>)
 //       -> tensor<128x128x32x32xf32>

@@ -137,6 +137,43 @@ def test_row_major_exports_equal_the_library_entry_point(uk, cuda, exe, name):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("name", ["mi355x_mmt4d_s8s8s32_t8", "mi355x_mmt4d_f16f16f32_t4",
+                                  "mi355x_mmt4d_f8e4m3f8e4m3f32_t8"])
+def test_tiled_exports_batch_planes_bit_exact_against_the_oracle(exe, name):
+    """A grid of `batch` planes in y: every plane has the bits of the
+    reference's per-entry mmt4d call on dense operands."""
+    import torch
+    e = H.EXPORTS[name]
+    rng = np.random.default_rng(zlib.crc32(name.encode()) + 1)
+    for (batch, M, N, K), acc in itertools.product([(3, 2, 3, 5), (5, 9, 4, 2)], (False, True)):
+        case = ukref.BatchMmt4dCase(rng, e.type_flag, batch, M, N, K, 32, 32, e.k0[0], accumulate=acc)
+        lhs, rhs, out = _dev(case.lhs), _dev(case.rhs), _dev(case.out_init)
+        exe.mmt4d(name, lhs, rhs, out, M, N, K, e.k0[0], case.flags, batch=batch)
+        torch.cuda.synchronize()
+        got = out.cpu().numpy().view(case.out_init.dtype)
+        want = case.run_oracle(ukref.F16_IEEE)
+        assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), (name, batch, (M, N, K), acc)
+
+
+@pytest.mark.gpu
+def test_row_major_export_batch_planes_equal_single_dispatches(uk, cuda, exe):
+    import torch
+    name = "mi355x_mmt4d_unpack_f16f16f32_t4"
+    batch, M, N, K1, K0 = 3, 100, 77, 9, 8
+    M1, N1 = -(-M // 32), -(-N // 32)
+    g = torch.Generator(device="cuda").manual_seed(11)
+    lhs = torch.randn(batch, M1 * K1 * 32 * K0, device="cuda", generator=g).half()
+    rhs = torch.randn(batch, N1 * K1 * 32 * K0, device="cuda", generator=g).half()
+    out = torch.full((batch, M, N), 3.0, device="cuda")
+    exe.mmt4d(name, lhs, rhs, out, M1, N1, K1, K0, F.MMT4D_TYPE_F16F16F32, out_rows=M, out_cols=N,
+              batch=batch)
+    for b in range(batch):
+        one = torch.full((M, N), 3.0, device="cuda")
+        exe.mmt4d(name, lhs[b], rhs[b], one, M1, N1, K1, K0, F.MMT4D_TYPE_F16F16F32, out_rows=M, out_cols=N)
+        assert torch.equal(out[b], one), b
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("name", sorted(H.MATMUL_EXPORTS))
 def test_matmul_exports_equal_the_library_entry_point(uk, cuda, exe, name):
     """mi355x_matmul_packed_rhs_*: the bits of iree_amd_uk_matmul_packed_rhs (same
