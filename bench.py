@@ -61,7 +61,7 @@ def parse_args():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--only", default="", help="run only the named kernel in a loop (for profilers): "
                     "mmt4d_f16 | mmt4d_i8 | mmt4d_fp8 | mmt4d_f16_ksplit | mlp_fp8 | pack | unpack | "
-                    "dequant_i4 | copy")
+                    "dequant_i4 | batch_mmt4d_f16 | copy")
     return ap.parse_args()
 
 
@@ -667,6 +667,14 @@ def run_only(args, torch, iree_amd, F, synth, mm_step):
         os_ = torch.empty(Ms * Ns, dtype=torch.float32, device="cuda")
         fn = lambda: iree_amd.mmt4d(ls, rs, os_, Ms // 32, Ns // 32, Ks // 8, 32, 32, 8,  # noqa: E731
                                     F.MMT4D_TYPE_F16F16F32)
+    elif args.only == "batch_mmt4d_f16":
+        # 16 problems of 1024^3 as one launch (batch entries = grid planes)
+        Bn, Bs = 16, 1024
+        lb = torch.from_numpy(synth.normal_f16(9, Bn * Bs * Bs, scale=1 / 64).view(np.int16)).cuda()
+        rb = torch.from_numpy(synth.normal_f16(10, Bn * Bs * Bs, scale=1 / 64).view(np.int16)).cuda()
+        ob = torch.empty(Bn * Bs * Bs, dtype=torch.float32, device="cuda")
+        fn = lambda: iree_amd.batch_mmt4d(lb, rb, ob, Bn, Bs // 32, Bs // 32, Bs // 8, 32, 32, 8,  # noqa: E731
+                                          F.MMT4D_TYPE_F16F16F32)
     else:
         raise SystemExit(f"unknown --only {args.only}")
     wall, per_launch = gpu_time(torch, fn, args.steps, args.warmup)
