@@ -196,6 +196,7 @@ int make_args(const iree_amd_uk_mmt4d_params_t& p, int out_elem_bytes, bool silu
   a.tiles_m = a.tiles_n = 0;
   a.k_slices = 0; a.slice_ksteps = 0; a.slice_out_bytes = 0;
   a.batch = 1; a.lhs_batch_bytes = a.rhs_batch_bytes = a.out_batch_bytes = 0;
+  a.batch_by_xcd = 0;
   a.accumulate = (p.flags & IREE_AMD_UK_FLAG_MMT4D_ACCUMULATE) != 0;
   a.k0_div = sv.mfma_k / p.K0;
   a.row_major_out = 0; a.out_rows = a.out_cols = 0;

@@ -96,6 +96,8 @@ struct MfmaArgs {
   // that lie z * {lhs,rhs,out}_batch_bytes further on
   int batch;
   int64_t lhs_batch_bytes, rhs_batch_bytes, out_batch_bytes;
+  // this many leading planes are dealt to the XCDs whole (see the __global__ wrapper)
+  int batch_by_xcd;
 };
 
 namespace {
@@ -191,7 +193,7 @@ __device__ __forceinline__ void tile_coord(int bid, int tiles_m, int tiles_n,
 // than one that reads the form from its arguments.)
 template <typename Cfg, int WM, int WN, int kRing, int kSync, bool kSiluMul = false, int kWavesN = 2,
           int kForm = 0>
-__device__ __forceinline__ void mmt4d_mfma_body(const MfmaArgs a) {
+__device__ __forceinline__ void mmt4d_mfma_body(const MfmaArgs a, const int bid = blockIdx.x) {
   static_assert(kForm >= 0 && kForm <= 3 && (!kSiluMul || kForm == 0), "unknown operand form");
   constexpr bool lhs_row_major = kForm >= 2;
   constexpr bool row_major_out = kForm == 1 || kForm == 2;
@@ -249,7 +251,7 @@ __device__ __forceinline__ void mmt4d_mfma_body(const MfmaArgs a) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wm = wave / kWavesN, wn = wave % kWavesN;
   int tm, tn;
-  tile_coord(blockIdx.x, a.tiles_m, a.tiles_n, &tm, &tn);
+  tile_coord(bid, a.tiles_m, a.tiles_n, &tm, &tn);
   const int i_base = tm * TM, j_base = tn * TN;
   const int T = a.ksteps;
 

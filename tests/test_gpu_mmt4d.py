@@ -731,6 +731,10 @@ BATCH_CASES = [
     (F.MMT4D_TYPE_F8E4M3F8E4M3F32, (32, 32, 16), 6, (3, 2, 6), (0, 0, 0)),
     (F.MMT4D_TYPE_F32F32F32, (32, 32, 4), 3, (4, 5, 21), (0, 0, 0)),
     (F.MMT4D_TYPE_F16F16F16, (32, 32, 8), 3, (2, 3, 3), (0, 0, 0)),
+    # 8 and more entries of few macro tiles: whole entries are dealt to the XCDs
+    (F.MMT4D_TYPE_S8S8S32, (32, 32, 16), 16, (9, 4, 19), (0, 0, 0)),
+    (F.MMT4D_TYPE_F16F16F32, (32, 32, 8), 9, (5, 7, 10), (16, 8, 4)),
+    (F.MMT4D_TYPE_BF16BF16F32, (32, 32, 8), 23, (17, 20, 4), (0, 0, 0)),
     # long K and few macro tiles per entry (a single mmt4d would split K)
     (F.MMT4D_TYPE_F16F16F32, (32, 32, 8), 2, (2, 2, 512), (0, 0, 0)),
     # batch strides the matrix-core kernel cannot address (odd byte alignment):
