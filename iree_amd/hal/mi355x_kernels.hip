@@ -96,14 +96,26 @@ __device__ __forceinline__ void hal_mmt4d(const void* lhs, const void* rhs, void
   a.slice_out_bytes = 0;
   a.k0_div = Cfg::kMfmaK / K0;
   a.gate_scale = a.up_scale = a.inv_out_scale = a.out_scale = 1.0f;
+  if (K < 1) return;
+  // Batch entry blockIdx.y of dense operands. Workgroups go to the 8 XCDs
+  // round-robin in launch order; entries of at most 64 macro tiles are dealt to
+  // the XCDs whole (the leading multiple of 8 planes: workgroup L takes tile
+  // (L / 8) % tiles of plane L % 8 + 8 * (L / 8 / tiles)), so that the tiles of
+  // an entry share their operands in one L2.
+  unsigned plane_y = blockIdx.y, bid = blockIdx.x;
+  if (gridDim.x <= 64 && blockIdx.y < gridDim.y / 8 * 8) {
+    const unsigned linear = blockIdx.y * gridDim.x + blockIdx.x;
+    const unsigned j = linear / 8;
+    plane_y = linear % 8 + 8 * (j / gridDim.x);
+    bid = j % gridDim.x;
+  }
   // a grid larger than the tile count (a count region that rounds up) is harmless
-  if (K < 1 || (int)blockIdx.x >= a.tiles_m * a.tiles_n) return;
-  // batch entry blockIdx.y of dense operands
-  const int64_t plane = blockIdx.y;
+  if ((int)bid >= a.tiles_m * a.tiles_n) return;
+  const int64_t plane = plane_y;
   a.lhs += plane * M * a.lhs_stride_bytes;
   a.rhs += plane * N * a.rhs_stride_bytes;
   a.out += plane * (row_major ? out_rows : M) * a.out_stride_bytes;
-  mmt4d_mfma_body<Cfg, WM, WN, kRing, kSync, false, 2, row_major ? 1 : 0>(a);
+  mmt4d_mfma_body<Cfg, WM, WN, kRing, kSync, false, 2, row_major ? 1 : 0>(a, (int)bid);
 }
 
 template <typename Cfg, int WM, int WN, int kRing, int kSync>

@@ -145,7 +145,7 @@ def test_tiled_exports_batch_planes_bit_exact_against_the_oracle(exe, name):
     import torch
     e = H.EXPORTS[name]
     rng = np.random.default_rng(zlib.crc32(name.encode()) + 1)
-    for (batch, M, N, K), acc in itertools.product([(3, 2, 3, 5), (5, 9, 4, 2)], (False, True)):
+    for (batch, M, N, K), acc in itertools.product([(3, 2, 3, 5), (5, 9, 4, 2), (19, 9, 10, 3)], (False, True)):
         case = ukref.BatchMmt4dCase(rng, e.type_flag, batch, M, N, K, 32, 32, e.k0[0], accumulate=acc)
         lhs, rhs, out = _dev(case.lhs), _dev(case.rhs), _dev(case.out_init)
         exe.mmt4d(name, lhs, rhs, out, M, N, K, e.k0[0], case.flags, batch=batch)
