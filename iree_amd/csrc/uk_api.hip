@@ -270,7 +270,12 @@ extern "C" int iree_amd_uk_batch_mmt4d(const iree_amd_uk_mmt4d_params_t* params,
   const bool nothing_to_do = p.M == 0 || p.N == 0 || p.M0 == 0 || p.N0 == 0 ||
                              (p.K == 0 && (p.flags & IREE_AMD_UK_FLAG_MMT4D_ACCUMULATE));
   if (nothing_to_do) return 0;
-  if (p.lhs_buffer && p.rhs_buffer && p.out_buffer && mmt4d_mfma_supported(p.flags, p.M0, p.N0, p.K0)) {
+  if (p.lhs_buffer && p.rhs_buffer && p.out_buffer && mmt4d_skinny_supported(p.flags, p.M0, p.N0, p.K0)) {
+    // (narrow left-hand sides: the entries of a decode step)
+    const int st = launch_batch_mmt4d_skinny(p, batch, lhs_batch_stride, rhs_batch_stride,
+                                             out_batch_stride, (hipStream_t)stream);
+    if (st != IREE_AMD_UK_STATUS_NOT_FOUND) return st;
+  } else if (p.lhs_buffer && p.rhs_buffer && p.out_buffer && mmt4d_mfma_supported(p.flags, p.M0, p.N0, p.K0)) {
     const int st = launch_batch_mmt4d_mfma(p, batch, lhs_batch_stride, rhs_batch_stride,
                                            out_batch_stride, (hipStream_t)stream);
     if (st != IREE_AMD_UK_STATUS_NOT_FOUND) return st;

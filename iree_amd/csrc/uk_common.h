@@ -60,6 +60,8 @@ int launch_mmt4d_skinny(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s);
 // NOT_FOUND (without recording an error) when the call must take the generic
 // kernel instead.
 int launch_mmt4d_mfma(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s);
+int launch_batch_mmt4d_skinny(const iree_amd_uk_mmt4d_params_t& p, int64_t batch, int64_t lhs_batch_stride,
+                              int64_t rhs_batch_stride, int64_t out_batch_stride, hipStream_t s);
 int launch_batch_mmt4d_mfma(const iree_amd_uk_mmt4d_params_t& p, int64_t batch, int64_t lhs_batch_stride,
                             int64_t rhs_batch_stride, int64_t out_batch_stride, hipStream_t s);
 int launch_mmt4d_unpack_mfma(const iree_amd_uk_mmt4d_params_t& p, int64_t out_rows,

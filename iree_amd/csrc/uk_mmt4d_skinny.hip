@@ -47,12 +47,20 @@ struct SkinnyArgs {
   // further on (one launch row and chunk_steps = ksteps when K is not split)
   int chunk_steps;
   int64_t chunk_out_elems;
+  // batch: workgroup plane blockIdx.z works on the operands that lie
+  // z * {lhs,rhs,out}_batch_bytes further on (one plane and zeros without one)
+  int batch;
+  int64_t lhs_batch_bytes, rhs_batch_bytes, out_batch_bytes;
 };
 
 // SP: K steps per wave held in registers (compile-time bound; a.steps_per_wave <= SP).
 // kPartialOut: the result is stored in the accumulator's type (the partial sums
 // of a K split whose final result is narrower: f16, bf16).
-template <typename Cfg, int SP, bool kPartialOut = false>
+// kPerWave: a K of at most SP steps (the head size of an attention step, say)
+// is not worth splitting over the waves: every wave takes all of K for an
+// outer column of its own, 8 columns per workgroup at a time, and stores its
+// block itself (no sum through LDS, no barrier).
+template <typename Cfg, int SP, bool kPartialOut = false, bool kPerWave = false>
 __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
   typedef typename Cfg::frag_t frag_t;
   typedef typename Cfg::acc_t acc_t;
@@ -62,12 +70,15 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
   typedef typename std::conditional<std::is_same<out_t, int32_t>::value, int32_t, float>::type sum_t;
   typedef typename std::conditional<kPartialOut, sum_t, out_t>::type store_t;
   __shared__ sum_t partial[2][kWaves][16][64];
+  a.lhs += blockIdx.z * a.lhs_batch_bytes;
+  a.rhs += blockIdx.z * a.rhs_batch_bytes;
+  a.out += blockIdx.z * a.out_batch_bytes;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int m0 = lane & 31, kh = lane >> 5;
   const int chunk_first = blockIdx.y * a.chunk_steps;
   const int chunk_end = chunk_first + a.chunk_steps < a.ksteps ? chunk_first + a.chunk_steps : a.ksteps;
-  const int first = chunk_first + wave * a.steps_per_wave;
+  const int first = chunk_first + (kPerWave ? 0 : wave * a.steps_per_wave);
   int count = chunk_end - first;
   count = count < 0 ? 0 : (count > a.steps_per_wave ? a.steps_per_wave : count);
 
@@ -107,7 +118,8 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
   };
 
   // ---- first blocks of the first tile, then the left-hand side -------------
-  int j = blockIdx.x;
+  int j = kPerWave ? blockIdx.x * kWaves + wave : blockIdx.x;
+  const int j_step = kPerWave ? gridDim.x * kWaves : gridDim.x;
   frag_t ring[kDepth];
 #pragma unroll
   for (int d = 0; d < kDepth; ++d) ring[d] = load_block(j, d);
@@ -134,8 +146,8 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
   }
 
   int parity = 0;
-  for (; j < a.N; j += gridDim.x, parity ^= 1) {
-    const int next = j + gridDim.x;
+  for (; j < a.N; j += j_step, parity ^= 1) {
+    const int next = j + j_step;
     acc_t acc;
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc[v] = 0;
@@ -146,6 +158,19 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
       __builtin_amdgcn_sched_barrier(0);
       ring[sp % kDepth] = sp + kDepth < SP ? load_block(j, sp + kDepth) : load_block(next, sp + kDepth - SP);
       __builtin_amdgcn_sched_barrier(0);
+    }
+    if constexpr (kPerWave) {
+      store_t* tile = (store_t*)a.out + (int64_t)j * a.out_stride_elems;
+      const int mm = lane & 31;
+      if (mm < a.M0) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int nn = 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+          const sum_t sum = (a.accumulate ? (sum_t)tile[mm * 32 + nn] : (sum_t)0) + (sum_t)acc[v];
+          tile[mm * 32 + nn] = (store_t)sum;
+        }
+      }
+      continue;
     }
     // ---- sum the 8 K slices in wave order and store -----------------------
     sum_t (*buf)[16][64] = partial[parity];
@@ -175,11 +200,25 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
 template <typename Cfg>
 int launch_cfg(SkinnyArgs a, int chunks, hipStream_t s) {
   const int cus = device_cu_count();
-  const int blocks = a.N < cus ? a.N : cus;
+  // (a batch: about two workgroups per compute unit over all planes)
+  int per_plane = a.batch > 1 ? (2 * cus + a.batch - 1) / a.batch : cus;
+  per_plane = per_plane > cus ? cus : per_plane;
+  constexpr bool kNarrowOut = sizeof(typename Cfg::out_t) < 4;
+  // (Not for fp8: its instance of the per-wave form returned wrong values in
+  // the result columns n0 >= M0 and the cause has not been found; fp8 keeps
+  // the split over the waves.)
+  if (chunks == 1 && a.chunk_steps <= 8 && Cfg::kSub != 2) {
+    // a short K: one outer column per wave
+    const int groups = (a.N + kWaves - 1) / kWaves;
+    a.steps_per_wave = a.chunk_steps;
+    const dim3 grid(groups < per_plane ? groups : per_plane, 1, a.batch > 1 ? a.batch : 1);
+    hipLaunchKernelGGL((mmt4d_skinny_kernel<Cfg, 8, false, true>), grid, dim3(kThreads), 0, s, a);
+    return check_hip(hipGetLastError(), "mmt4d_skinny launch");
+  }
+  const int blocks = a.N < per_plane ? a.N : per_plane;
   const int per = (a.chunk_steps + kWaves - 1) / kWaves;
   a.steps_per_wave = per;
-  constexpr bool kNarrowOut = sizeof(typename Cfg::out_t) < 4;
-  const dim3 grid(blocks, chunks), block(kThreads);
+  const dim3 grid(blocks, chunks, a.batch > 1 ? a.batch : 1), block(kThreads);
   if (chunks > 1 && kNarrowOut) {
     if constexpr (kNarrowOut) {
       if (per <= 8) hipLaunchKernelGGL((mmt4d_skinny_kernel<Cfg, 8, true>), grid, block, 0, s, a);
@@ -233,9 +272,26 @@ int max_steps_per_launch(int mfma_k) { return kWaves * (mfma_k == 64 ? 16 : 32);
 
 // One launch over the K of `p`: `chunks` workgroup rows of `chunk_steps` K steps
 // each; with more than one, the results are partial sums written to `scratch`.
+struct BatchStrides { int64_t batch, lhs, rhs, out; };   // strides in elements
 int launch_chunk(const iree_amd_uk_mmt4d_params_t& p, int chunks, int chunk_steps, void* scratch,
-                 hipStream_t s);
+                 hipStream_t s, const BatchStrides* batch = nullptr);
 }  // namespace
+
+// `batch` problems of one narrow shape as the planes of one launch; only what a
+// single launch row takes (K short enough to stay in registers), at most 65535
+// entries and batch strides of whole 16 bytes.
+int launch_batch_mmt4d_skinny(const iree_amd_uk_mmt4d_params_t& p, int64_t batch, int64_t lhs_batch_stride,
+                              int64_t rhs_batch_stride, int64_t out_batch_stride, hipStream_t s) {
+  if (!mmt4d_skinny_supported(p.flags, p.M0, p.N0, p.K0)) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  const int mk = mfma_k_of(p.flags);
+  const int64_t k_elems = p.K * p.K0;
+  if (p.M != 1 || p.K == 0 || k_elems % mk || p.N > 0x7FFFFFFF || batch > 65535)
+    return IREE_AMD_UK_STATUS_NOT_FOUND;
+  const int64_t steps = k_elems / mk;
+  if (steps > max_steps_per_launch(mk)) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  const BatchStrides bs = {batch, lhs_batch_stride, rhs_batch_stride, out_batch_stride};
+  return launch_chunk(p, 1, (int)steps, nullptr, s, &bs);
+}
 
 int launch_mmt4d_skinny(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) {
   if (!mmt4d_skinny_supported(p.flags, p.M0, p.N0, p.K0)) return IREE_AMD_UK_STATUS_NOT_FOUND;
@@ -314,7 +370,7 @@ int launch_mmt4d_skinny(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) {
 
 namespace {
 int launch_chunk(const iree_amd_uk_mmt4d_params_t& p, int chunks, int chunk_steps, void* scratch,
-                 hipStream_t s) {
+                 hipStream_t s, const BatchStrides* batch) {
   const int mk = mfma_k_of(p.flags);
   Mmt4dTypeInfo ti;
   mmt4d_type_info(p.flags, &ti);
@@ -339,6 +395,15 @@ int launch_chunk(const iree_amd_uk_mmt4d_params_t& p, int chunks, int chunk_step
   a.accumulate = (p.flags & IREE_AMD_UK_FLAG_MMT4D_ACCUMULATE) != 0;
   a.chunk_steps = chunk_steps;
   a.chunk_out_elems = 0;
+  a.batch = 1;
+  a.lhs_batch_bytes = a.rhs_batch_bytes = a.out_batch_bytes = 0;
+  if (batch) {
+    a.batch = (int)batch->batch;
+    a.lhs_batch_bytes = batch->lhs * eb;
+    a.rhs_batch_bytes = batch->rhs * eb;
+    a.out_batch_bytes = batch->out * ti.out_bytes;
+    if (a.lhs_batch_bytes % 16 || a.rhs_batch_bytes % 16) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  }
   if (chunks > 1) {
     a.out = (char*)scratch;
     a.accumulate = 0;

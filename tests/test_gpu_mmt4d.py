@@ -744,6 +744,14 @@ BATCH_CASES = [
     (F.MMT4D_TYPE_S8S8S32, (4, 6, 2), 3, (2, 3, 4), (1, 2, 3)),
     (F.MMT4D_TYPE_F16F16F32, (8, 32, 8), 3, (1, 5, 12), (0, 0, 0)),
     (F.MMT4D_TYPE_S16U4S32, (3, 5, 8), 2, (2, 3, 4), (0, 0, 0)),
+    # narrow left-hand sides (one outer row): the entries are planes of one
+    # launch of the streaming kernel; odd gaps run entry by entry
+    (F.MMT4D_TYPE_S8S8S32, (4, 32, 32), 9, (1, 7, 8), (0, 0, 0)),
+    (F.MMT4D_TYPE_F8E4M3F8E4M3F32, (16, 32, 16), 5, (1, 3, 4), (0, 0, 0)),
+    (F.MMT4D_TYPE_BF16BF16BF16, (2, 32, 16), 4, (1, 9, 6), (0, 0, 0)),
+    (F.MMT4D_TYPE_F16F16F32, (1, 32, 16), 40, (1, 33, 8), (8, 16, 3)),
+    (F.MMT4D_TYPE_F16F16F32, (1, 32, 8), 300, (1, 2, 16), (0, 0, 0)),
+    (F.MMT4D_TYPE_F32F32F32, (8, 32, 8), 3, (1, 5, 3), (3, 1, 0)),
 ]
 
 
