@@ -373,6 +373,25 @@ def extras(args, torch, iree_amd, F, synth, lhs, rhs, out, ex):
     ex["batch_mmt4d_f16_16x1024_entry_by_entry_tflops"] = round(2.0 * Bn * Bs ** 3 / t1 / 1e12, 1)
     del lb, rb, ob, o1
 
+    # batch_mmt4d with narrow left-hand sides: 32 entries of one row against
+    # 32768 x 128 (the scores of one decode step of attention: heads x cached
+    # positions x head size), 9 rotating right-hand sides (2.4 GB > the 256 MiB cache)
+    Hn, Sn, Dn = 32, 32768, 128
+    qn = torch.from_numpy(synth.normal_f16(11, Hn * Dn).view(np.int16)).cuda()
+    kn = [torch.from_numpy(synth.normal_f16(12 + i, Hn * Sn * Dn).view(np.int16)).cuda() for i in range(3)]
+    kn = kn * 3
+    on = torch.empty(Hn * Sn, dtype=torch.float32, device="cuda")
+    stn = {"i": 0}
+
+    def narrow_batch():
+        kx = kn[stn["i"] % len(kn)]
+        stn["i"] += 1
+        iree_amd.batch_mmt4d(qn, kx, on, Hn, 1, Sn // 32, Dn // 16, 1, 32, 16, F.MMT4D_TYPE_F16F16F32)
+    _, t = gpu_time(torch, narrow_batch, steps, warm)
+    ex["batch_mmt4d_f16_narrow_32x1x32768x128_us"] = round(t * 1e6, 1)
+    ex["batch_mmt4d_f16_narrow_32x1x32768x128_gbs"] = round((Hn * Sn * Dn * 2 + Hn * Sn * 4) / t / 1e9, 1)
+    del qn, kn, on
+
     # The same f16 mmt4d dispatched from the code object a HAL executable on a
     # HIP device links (hipModuleLaunchKernel, bindings + 32-bit push constants)
     from iree_amd import hal_executable

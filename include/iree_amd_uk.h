@@ -182,10 +182,11 @@ IREE_AMD_UK_EXPORT int iree_amd_uk_mmt4d_p(
  * rank-reduces each entry to mmt4d (REF compiler/src/iree/compiler/Codegen/
  * Common/CPU/CPUPrepareUkernels.cpp:23-43 tileBatchDimsForBatchMmt4dOp,
  * :165-245 ConvertBatchMmt4DtoMmt4DPattern), so every entry has exactly the
- * result of iree_amd_uk_mmt4d_p on it. Matrix-core tiles whose batch strides
- * are whole 16 bytes run as ONE launch (batch entries are planes of the grid;
- * K is not split in it, so it allocates nothing); everything else runs as
- * iree_amd_uk_mmt4d_p entry by entry. Entries must not overlap in `out`.
+ * result of iree_amd_uk_mmt4d_p on it. Matrix-core tiles (M0 = 32, and the
+ * narrow ones, M = 1 and M0 < 32, whose K one launch row holds) whose batch
+ * strides are whole 16 bytes run as ONE launch (batch entries are planes of
+ * the grid; K is not split in it, so it allocates nothing); everything else
+ * runs as iree_amd_uk_mmt4d_p entry by entry. Entries must not overlap in `out`.
  * batch == 0 does nothing. */
 IREE_AMD_UK_EXPORT int iree_amd_uk_batch_mmt4d(
     const iree_amd_uk_mmt4d_params_t* params, iree_amd_uk_index_t batch,

@@ -56,7 +56,7 @@ struct SkinnyArgs {
 // SP: K steps per wave held in registers (compile-time bound; a.steps_per_wave <= SP).
 // kPartialOut: the result is stored in the accumulator's type (the partial sums
 // of a K split whose final result is narrower: f16, bf16).
-// kPerWave: a K of at most SP steps (the head size of an attention step, say)
+// kPerWave: a K of at most SP (8 or 16) steps (the head size of an attention step, say)
 // is not worth splitting over the waves: every wave takes all of K for an
 // outer column of its own, 8 columns per workgroup at a time, and stores its
 // block itself (no sum through LDS, no barrier).
@@ -207,12 +207,15 @@ int launch_cfg(SkinnyArgs a, int chunks, hipStream_t s) {
   // (Not for fp8: its instance of the per-wave form returned wrong values in
   // the result columns n0 >= M0 and the cause has not been found; fp8 keeps
   // the split over the waves.)
-  if (chunks == 1 && a.chunk_steps <= 8 && Cfg::kSub != 2) {
-    // a short K: one outer column per wave
-    const int groups = (a.N + kWaves - 1) / kWaves;
+  const int groups = (a.N + kWaves - 1) / kWaves;
+  if (chunks == 1 && a.chunk_steps <= 16 && Cfg::kSub != 2 &&
+      (int64_t)groups * (a.batch > 1 ? a.batch : 1) >= cus) {
+    // a short K and enough outer columns to give every compute unit 8 of
+    // them: one outer column per wave
     a.steps_per_wave = a.chunk_steps;
     const dim3 grid(groups < per_plane ? groups : per_plane, 1, a.batch > 1 ? a.batch : 1);
-    hipLaunchKernelGGL((mmt4d_skinny_kernel<Cfg, 8, false, true>), grid, dim3(kThreads), 0, s, a);
+    if (a.chunk_steps <= 8) hipLaunchKernelGGL((mmt4d_skinny_kernel<Cfg, 8, false, true>), grid, dim3(kThreads), 0, s, a);
+    else hipLaunchKernelGGL((mmt4d_skinny_kernel<Cfg, 16, false, true>), grid, dim3(kThreads), 0, s, a);
     return check_hip(hipGetLastError(), "mmt4d_skinny launch");
   }
   const int blocks = a.N < per_plane ? a.N : per_plane;

@@ -119,8 +119,10 @@ def test_narrow_lhs_tiles_bit_exact(uk, cuda, type_flag, K0):
     tps = mfma_k // K0                      # K tiles per MFMA step
     for M0 in (1, 2, 4, 8, 16):
         assert uk.mmt4d_info(M0, 32, K0, type_flag | F.MMT4D_SKIP_INTERMEDIATE_ROUNDINGS) == 1
+        # (2100 and more outer columns of at most 16 steps: one column per wave)
         for N, steps, acc in ((1, 1, False), (5, 8, True), (300, 13, False), (3, 70, True),
-                              (7, 128, False), (2, 255, True)):
+                              (7, 128, False), (2, 255, True), (2100, 8, True), (2051, 13, False),
+                              (2300, 3, False)):
             case = ukref.Mmt4dCase(rng, type_flag, 1, N, steps * tps, M0, 32, K0, accumulate=acc)
             got = gpucase.run_mmt4d(case, flags=case.flags & ~F.MMT4D_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION)
             assert np.array_equal(got.view(np.uint8), case.run_oracle(ukref.F16_IEEE).view(np.uint8)), \
@@ -751,6 +753,8 @@ BATCH_CASES = [
     (F.MMT4D_TYPE_BF16BF16BF16, (2, 32, 16), 4, (1, 9, 6), (0, 0, 0)),
     (F.MMT4D_TYPE_F16F16F32, (1, 32, 16), 40, (1, 33, 8), (8, 16, 3)),
     (F.MMT4D_TYPE_F16F16F32, (1, 32, 8), 300, (1, 2, 16), (0, 0, 0)),
+    (F.MMT4D_TYPE_S8S8S32, (8, 32, 16), 70, (1, 37, 26), (16, 0, 32)),
+    (F.MMT4D_TYPE_BF16BF16BF16, (2, 32, 16), 33, (1, 70, 9), (0, 0, 0)),
     (F.MMT4D_TYPE_F32F32F32, (8, 32, 8), 3, (1, 5, 3), (3, 1, 0)),
 ]
 
