@@ -137,9 +137,19 @@ struct F8Cfg {
   static constexpr int kElemBytes = 1;
   static constexpr int kMfmaK = 64;
   static constexpr int kSub = 2;
-  __device__ static acc_t mfma(frag_t a, frag_t b, acc_t c) {
-    // formats 0 / 0: both operands e4m3; block scales 0x7F = 2^0.
-    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+  // formats 0 / 0: both operands e4m3; block scales 0x7F = 2^0. The scales are
+  // per-lane register operands, and the instruction reads them from ALL lanes
+  // whatever the execution mask: a kernel with divergent regions passes
+  // `scales` from unit_scales(), called where every lane is active, because
+  // the compiler is free to materialise the constant inside such a region,
+  // where it reaches the active lanes only.
+  __device__ static acc_t mfma(frag_t a, frag_t b, acc_t c, int scales = 0x7F7F7F7F) {
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, scales, 0, scales);
+  }
+  __device__ static int unit_scales() {
+    int v;
+    asm volatile("v_mov_b32 %0, 0x7f7f7f7f" : "=v"(v));
+    return v;
   }
 };
 

@@ -248,6 +248,16 @@ __device__ __forceinline__ void mmt4d_mfma_body(const MfmaArgs a, const int bid 
   extern __shared__ __attribute__((aligned(1024))) char lds[];
 
   const int lane = threadIdx.x & 63;
+  // fp8: the MFMA's block scales are register operands read from all lanes
+  // whatever the execution mask; they are set here, where every lane is active
+  // (a constant the compiler materialises inside a divergent region would
+  // reach the active lanes only).
+  int unit_scales = 0;
+  if constexpr (Cfg::kSub == 2) unit_scales = Cfg::unit_scales();
+  auto mfma = [&](const frag_t& x, const frag_t& y, const auto& c) {
+    if constexpr (Cfg::kSub == 2) return Cfg::mfma(x, y, c, unit_scales);
+    else return Cfg::mfma(x, y, c);
+  };
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wm = wave / kWavesN, wn = wave % kWavesN;
   int tm, tn;
@@ -446,14 +456,14 @@ __device__ __forceinline__ void mmt4d_mfma_body(const MfmaArgs a, const int bid 
       for (int y = 0; y < WN; ++y)
         if (y >= o0 && y < o1) {
 #pragma unroll
-          for (int x = 0; x < WM; ++x) acc[x][y] = Cfg::mfma(fb[y], fa[x], acc[x][y]);
+          for (int x = 0; x < WM; ++x) acc[x][y] = mfma(fb[y], fa[x], acc[x][y]);
         }
     } else {
 #pragma unroll
       for (int x = 0; x < WM; ++x)
         if (x >= o0 && x < o1) {
 #pragma unroll
-          for (int y = 0; y < WN; ++y) acc[x][y] = Cfg::mfma(fa[x], fb[y], acc[x][y]);
+          for (int y = 0; y < WN; ++y) acc[x][y] = mfma(fa[x], fb[y], acc[x][y]);
         }
     }
   };

@@ -70,6 +70,9 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
   typedef typename std::conditional<std::is_same<out_t, int32_t>::value, int32_t, float>::type sum_t;
   typedef typename std::conditional<kPartialOut, sum_t, out_t>::type store_t;
   __shared__ sum_t partial[2][kWaves][16][64];
+  // (fp8: the block scales of the MFMA, set while every lane is active)
+  int unit_scales = 0;
+  if constexpr (Cfg::kSub == 2) unit_scales = Cfg::unit_scales();
   a.lhs += blockIdx.z * a.lhs_batch_bytes;
   a.rhs += blockIdx.z * a.rhs_batch_bytes;
   a.out += blockIdx.z * a.out_batch_bytes;
@@ -153,7 +156,8 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
     for (int v = 0; v < 16; ++v) acc[v] = 0;
 #pragma unroll
     for (int sp = 0; sp < SP; ++sp) {
-      acc = Cfg::mfma(live(ring[sp % kDepth], sp), xf[sp], acc);
+      if constexpr (Cfg::kSub == 2) acc = Cfg::mfma(live(ring[sp % kDepth], sp), xf[sp], acc, unit_scales);
+      else acc = Cfg::mfma(live(ring[sp % kDepth], sp), xf[sp], acc);
       // refill the slot: kDepth steps ahead, wrapping into the next tile
       __builtin_amdgcn_sched_barrier(0);
       ring[sp % kDepth] = sp + kDepth < SP ? load_block(j, sp + kDepth) : load_block(next, sp + kDepth - SP);
