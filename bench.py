@@ -61,7 +61,7 @@ def parse_args():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--only", default="", help="run only the named kernel in a loop (for profilers): "
                     "mmt4d_f16 | mmt4d_i8 | mmt4d_fp8 | mmt4d_f16_ksplit | mlp_fp8 | pack | unpack | "
-                    "dequant_i4 | batch_mmt4d_f16 | copy")
+                    "dequant_i4 | batch_mmt4d_f16 | batch_mmt4d_f16_narrow | copy")
     return ap.parse_args()
 
 
@@ -694,6 +694,18 @@ def run_only(args, torch, iree_amd, F, synth, mm_step):
         ob = torch.empty(Bn * Bs * Bs, dtype=torch.float32, device="cuda")
         fn = lambda: iree_amd.batch_mmt4d(lb, rb, ob, Bn, Bs // 32, Bs // 32, Bs // 8, 32, 32, 8,  # noqa: E731
                                           F.MMT4D_TYPE_F16F16F32)
+    elif args.only == "batch_mmt4d_f16_narrow":
+        # 32 entries of one row against 32768 x 128, 9 rotating right-hand sides
+        Hn, Sn, Dn = 32, 32768, 128
+        qn = torch.from_numpy(synth.normal_f16(11, Hn * Dn).view(np.int16)).cuda()
+        kn = [torch.from_numpy(synth.normal_f16(12 + i, Hn * Sn * Dn).view(np.int16)).cuda() for i in range(3)] * 3
+        on = torch.empty(Hn * Sn, dtype=torch.float32, device="cuda")
+        st = {"i": 0}
+
+        def fn():
+            kx = kn[st["i"] % len(kn)]
+            st["i"] += 1
+            iree_amd.batch_mmt4d(qn, kx, on, Hn, 1, Sn // 32, Dn // 16, 1, 32, 16, F.MMT4D_TYPE_F16F16F32)
     else:
         raise SystemExit(f"unknown --only {args.only}")
     wall, per_launch = gpu_time(torch, fn, args.steps, args.warmup)
