@@ -161,7 +161,9 @@ typedef struct iree_amd_uk_mmt4d_params_t {
 /* Replaces REF mmt4d.h:14-21 / mmt4d.c:151-177 (iree_uk_mmt4d).
  * A matrix-core call of few macro tiles and a long K splits K and keeps the
  * partial sums in a scratch buffer the library allocates once per stream
- * (16 to 512 MiB, never freed); every other call allocates nothing. */
+ * (16 to 512 MiB; kept until iree_amd_uk_release_scratch or, with more than 64
+ * streams in use, until it is the least recently used one); every other call
+ * allocates nothing. */
 IREE_AMD_UK_EXPORT int iree_amd_uk_mmt4d(
     const void* lhs_buffer, iree_amd_uk_index_t lhs_offset,
     iree_amd_uk_index_t lhs_stride0, const void* rhs_buffer,
@@ -295,12 +297,20 @@ IREE_AMD_UK_EXPORT int iree_amd_uk_unpack_p(
 /*===------------------------------------------------------------------------===
  * query_tile_sizes_2d: (operation, operand role) -> (tile_size0, tile_size1).
  * LHS -> (M0,K0), RHS -> (N0,K0), RESULT -> (M0,N0) of the matmul tile chosen
- * for gfx950 (REF query_tile_sizes.c:43-63 for the role mapping). `size0` /
- * `size1` are the operand's own dimensions (INT64_MIN = dynamic): a static M
- * (LHS/RESULT size0) or N (RHS size0, RESULT size1) below 32 narrows that tile
- * dimension to the next power of two >= the size, as the reference's
+ * for gfx950 (REF query_tile_sizes.c:43-63 for the role mapping).
+ * `size0` / `size1` are the operand's own dimensions (INT64_MIN = dynamic): a
+ * static M (LHS / RESULT size0) or N (RHS size0, RESULT size1) below 32 narrows
+ * that tile dimension to the next power of two >= the size, as the reference's
  * compile-time chooser does for narrow matmuls
  * (REF compiler/src/iree/compiler/Codegen/Common/CPU/CPUMaterializeEncodingPass.cpp:284-377).
+ * Like that chooser (its lines 296-303) the library narrows at most ONE of M0
+ * and N0 per matmul, the one of the smaller static size, and a narrow N0 is
+ * served as the narrow-M0 problem with the operands exchanged
+ * (REF compiler/src/iree/compiler/Codegen/Common/EncodingUtils.cpp:23-92): the
+ * RESULT role, which sees both sizes, applies the rule itself; a caller whose M
+ * AND N are both static and below 32 passes the LHS / RHS query of the wider of
+ * the two a dynamic size0. Every tile this function returns has a matrix-core
+ * kernel (iree_amd_uk_mmt4d_info).
  *===------------------------------------------------------------------------===*/
 
 /* REF query_tile_sizes.h:18-23 */
@@ -483,7 +493,8 @@ IREE_AMD_UK_EXPORT int iree_amd_uk_matmul_packed_rhs(
 IREE_AMD_UK_EXPORT int iree_amd_uk_scale_f32(void* buf_f32, iree_amd_uk_index_t n,
                                              float scale, void* stream);
 
-/* Measurement aid with no counterpart in the reference: runs the mmt4d
+/* NOT part of the reference interface (no iree_uk_* counterpart, nothing a
+ * runtime binds to): a measurement aid for bench.py. It runs the mmt4d
  * kernel's matrix-core instruction pattern (every accumulator block of a wave's
  * 128 x 128 tile once per K-step, with the instruction shape the kernel uses for
  * the type; one workgroup of 4 waves per compute unit) for `iters` K-steps on operand
@@ -519,6 +530,10 @@ IREE_AMD_UK_EXPORT int iree_amd_uk_memcpy_d2h(void* dst, const void* src,
 IREE_AMD_UK_EXPORT int iree_amd_uk_stream_create(void** out_stream);
 IREE_AMD_UK_EXPORT int iree_amd_uk_stream_destroy(void* stream);
 IREE_AMD_UK_EXPORT int iree_amd_uk_stream_synchronize(void* stream);
+/* Frees the scratch buffers the library has cached per stream (see
+ * iree_amd_uk_mmt4d) that no call is using at the moment; they come back on
+ * demand. What a plugin calls from its unload. Waits for the device. */
+IREE_AMD_UK_EXPORT int iree_amd_uk_release_scratch(void);
 /* Human-readable text of the calling thread's last non-OK status ("" if none). */
 IREE_AMD_UK_EXPORT const char* iree_amd_uk_last_error(void);
 /* Library version: (major << 16) | minor. */
@@ -530,8 +545,28 @@ IREE_AMD_UK_EXPORT uint32_t iree_amd_uk_version(void);
  * REF samples/custom_dispatch/cpu/plugin/README.md:90-97). Each call stages the
  * touched byte ranges to device memory, runs the device entry point above,
  * copies the destination range back and synchronises before returning.
- * Reentrant; safe to call concurrently from several threads.
+ * Reentrant; safe to call concurrently from several threads
+ * (REF samples/custom_dispatch/cpu/plugin/system_plugin.c:21-25).
+ *
+ * The *_pooled forms take a pool that keeps the staging resources between
+ * calls: up to 8 slots per device, each one stream and three device buffers
+ * that grow on demand. A call owns a slot for its duration (calls beyond the
+ * slots wait for one), so concurrent calls share nothing. A pool is what a
+ * plugin instance owns: created in its load (touches no device), destroyed in
+ * its unload once no call is running; there is no global state
+ * (REF runtime/src/iree/hal/local/executable_plugin.h:415-418). The forms
+ * without a pool build one for the single call (stream and buffers created and
+ * freed per call). None of them splits K, so none uses the scratch cache.
  *===------------------------------------------------------------------------===*/
+typedef struct iree_amd_uk_host_pool_t iree_amd_uk_host_pool_t;
+IREE_AMD_UK_EXPORT int iree_amd_uk_host_pool_create(iree_amd_uk_host_pool_t** out_pool);
+IREE_AMD_UK_EXPORT void iree_amd_uk_host_pool_destroy(iree_amd_uk_host_pool_t* pool);
+IREE_AMD_UK_EXPORT int iree_amd_uk_mmt4d_host_pooled(
+    iree_amd_uk_host_pool_t* pool, const iree_amd_uk_mmt4d_params_t* params);
+IREE_AMD_UK_EXPORT int iree_amd_uk_pack_host_pooled(
+    iree_amd_uk_host_pool_t* pool, const iree_amd_uk_pack_params_t* params);
+IREE_AMD_UK_EXPORT int iree_amd_uk_unpack_host_pooled(
+    iree_amd_uk_host_pool_t* pool, const iree_amd_uk_unpack_params_t* params);
 IREE_AMD_UK_EXPORT int iree_amd_uk_mmt4d_host(
     const iree_amd_uk_mmt4d_params_t* params);
 IREE_AMD_UK_EXPORT int iree_amd_uk_pack_host(

@@ -141,10 +141,22 @@ def _declare(lib):
     lib.iree_amd_uk_stream_destroy.argtypes = [vp]
     lib.iree_amd_uk_stream_synchronize.restype = C.c_int
     lib.iree_amd_uk_stream_synchronize.argtypes = [vp]
+    lib.iree_amd_uk_release_scratch.restype = C.c_int
+    lib.iree_amd_uk_release_scratch.argtypes = []
     lib.iree_amd_uk_last_error.restype = C.c_char_p
     lib.iree_amd_uk_last_error.argtypes = []
     lib.iree_amd_uk_version.restype = u32
     lib.iree_amd_uk_version.argtypes = []
+    lib.iree_amd_uk_host_pool_create.restype = C.c_int
+    lib.iree_amd_uk_host_pool_create.argtypes = [C.POINTER(vp)]
+    lib.iree_amd_uk_host_pool_destroy.restype = None
+    lib.iree_amd_uk_host_pool_destroy.argtypes = [vp]
+    lib.iree_amd_uk_mmt4d_host_pooled.restype = C.c_int
+    lib.iree_amd_uk_mmt4d_host_pooled.argtypes = [vp, C.POINTER(Mmt4dParams)]
+    lib.iree_amd_uk_pack_host_pooled.restype = C.c_int
+    lib.iree_amd_uk_pack_host_pooled.argtypes = [vp, C.POINTER(PackParams)]
+    lib.iree_amd_uk_unpack_host_pooled.restype = C.c_int
+    lib.iree_amd_uk_unpack_host_pooled.argtypes = [vp, C.POINTER(UnpackParams)]
     lib.iree_amd_uk_mmt4d_host.restype = C.c_int
     lib.iree_amd_uk_mmt4d_host.argtypes = [C.POINTER(Mmt4dParams)]
     lib.iree_amd_uk_pack_host.restype = C.c_int

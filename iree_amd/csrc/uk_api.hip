@@ -388,10 +388,18 @@ extern "C" int iree_amd_uk_query_tile_sizes_2d(
       out_params->tile_size0 = narrow(t.N0, params->size0);
       out_params->tile_size1 = t.K0;
       return 0;
-    case IREE_AMD_UK_FLAG_QUERY_TILE_SIZES_OPERAND_ROLE_RESULT:
-      out_params->tile_size0 = narrow(t.M0, params->size0);
-      out_params->tile_size1 = narrow(t.N0, params->size1);
+    case IREE_AMD_UK_FLAG_QUERY_TILE_SIZES_OPERAND_ROLE_RESULT: {
+      // Both dimensions are known here. At most ONE is narrowed, the smaller
+      // one (the reference's chooser reduces narrow-N to narrow-M by
+      // transposition only when N is the narrower of the two and keeps the
+      // other dimension's full tile: CPUMaterializeEncodingPass.cpp:296-303).
+      const int m0 = narrow(t.M0, params->size0), n0 = narrow(t.N0, params->size1);
+      const bool m_narrow = m0 < t.M0, n_narrow = n0 < t.N0;
+      const bool pick_n = n_narrow && (!m_narrow || params->size1 < params->size0);
+      out_params->tile_size0 = pick_n ? t.M0 : m0;
+      out_params->tile_size1 = pick_n ? n0 : t.N0;
       return 0;
+    }
     default:
       return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "query_tile_sizes: unknown operand role 0x%x",
                   params->flags & IREE_AMD_UK_FLAG_QUERY_TILE_SIZES_OPERAND_ROLE_MASK);
@@ -670,121 +678,9 @@ extern "C" int iree_amd_uk_stream_destroy(void* stream) {
 extern "C" int iree_amd_uk_stream_synchronize(void* stream) {
   return check_hip(hipStreamSynchronize((hipStream_t)stream), "hipStreamSynchronize");
 }
+extern "C" int iree_amd_uk_release_scratch(void) {
+  (void)scratch_release_idle();
+  return 0;
+}
 extern "C" const char* iree_amd_uk_last_error(void) { return g_last_error; }
 extern "C" uint32_t iree_amd_uk_version(void) { return (0u << 16) | 1u; }
-
-//===----------------------------------------------------------------------===//
-// Host-pointer variants: stage the touched element ranges through device
-// memory. Each call owns its device buffers and one stream, so concurrent
-// calls from several host threads do not share state.
-//===----------------------------------------------------------------------===//
-
-namespace {
-
-struct Staging {
-  hipStream_t stream = nullptr;
-  void* dev[3] = {nullptr, nullptr, nullptr};
-  ~Staging() {
-    for (void* d : dev)
-      if (d) (void)hipFree(d);
-    if (stream) (void)hipStreamDestroy(stream);
-  }
-  int init() { return check_hip(hipStreamCreateWithFlags(&stream, hipStreamNonBlocking), "hipStreamCreate"); }
-  // Uploads [host + byte_off, +bytes) into a fresh device buffer `slot`.
-  int upload(int slot, const void* host, int64_t byte_off, int64_t bytes, bool copy) {
-    if (bytes <= 0) return 0;
-    UK_RETURN_IF_HIP(hipMalloc(&dev[slot], (size_t)bytes));
-    if (copy)
-      UK_RETURN_IF_HIP(hipMemcpyAsync(dev[slot], (const char*)host + byte_off, (size_t)bytes,
-                                      hipMemcpyHostToDevice, stream));
-    return 0;
-  }
-  int download(int slot, void* host, int64_t byte_off, int64_t bytes) {
-    if (bytes <= 0) return 0;
-    UK_RETURN_IF_HIP(hipMemcpyAsync((char*)host + byte_off, dev[slot], (size_t)bytes,
-                                    hipMemcpyDeviceToHost, stream));
-    return check_hip(hipStreamSynchronize(stream), "hipStreamSynchronize");
-  }
-};
-
-// Bytes spanned by `rows` rows of `row_elems` contiguous elements, `stride`
-// elements apart, for an element of `bits` bits.
-int64_t span_bytes(int64_t rows, int64_t stride, int64_t row_elems, int bits) {
-  if (rows <= 0 || row_elems <= 0) return 0;
-  return (((rows - 1) * stride + row_elems) * bits + 7) / 8;
-}
-
-}  // namespace
-
-extern "C" int iree_amd_uk_mmt4d_host(const iree_amd_uk_mmt4d_params_t* params) {
-  if (!params) return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "mmt4d_host: null params");
-  iree_amd_uk_mmt4d_params_t p = *params;
-  UK_RETURN_IF_ERROR(validate_mmt4d(p));
-  if (p.M == 0 || p.N == 0 || (p.K == 0 && (p.flags & IREE_AMD_UK_FLAG_MMT4D_ACCUMULATE))) return 0;
-  if (p.M0 == 0 || p.N0 == 0) return 0;
-  Mmt4dTypeInfo ti;
-  mmt4d_type_info(p.flags, &ti);
-  const int64_t lhs_bytes = span_bytes(p.M, p.lhs_stride0, p.K * p.M0 * p.K0, ti.lhs_bits);
-  const int64_t rhs_bytes = span_bytes(p.N, p.rhs_stride0, p.K * p.N0 * p.K0, ti.rhs_bits);
-  const int64_t out_bytes = span_bytes(p.M, p.out_stride0, p.N * p.M0 * p.N0, ti.out_bytes * 8);
-  const bool out_tight = p.out_stride0 == p.N * p.M0 * p.N0;
-  const bool need_out_in = (p.flags & IREE_AMD_UK_FLAG_MMT4D_ACCUMULATE) || !out_tight;
-  Staging st;
-  UK_RETURN_IF_ERROR(st.init());
-  UK_RETURN_IF_ERROR(st.upload(0, p.lhs_buffer, p.lhs_offset * ti.lhs_bits / 8, lhs_bytes, true));
-  UK_RETURN_IF_ERROR(st.upload(1, p.rhs_buffer, p.rhs_offset * ti.rhs_bits / 8, rhs_bytes, true));
-  UK_RETURN_IF_ERROR(st.upload(2, p.out_buffer, p.out_offset * ti.out_bytes, out_bytes, need_out_in));
-  void* host_out = p.out_buffer;
-  const int64_t host_out_off = p.out_offset * ti.out_bytes;
-  p.lhs_buffer = st.dev[0]; p.lhs_offset = 0;
-  p.rhs_buffer = st.dev[1]; p.rhs_offset = 0;
-  p.out_buffer = st.dev[2]; p.out_offset = 0;
-  UK_RETURN_IF_ERROR(iree_amd_uk_mmt4d_p(&p, st.stream));
-  return st.download(2, host_out, host_out_off, out_bytes);
-}
-
-extern "C" int iree_amd_uk_pack_host(const iree_amd_uk_pack_params_t* params) {
-  if (!params) return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "pack_host: null params");
-  iree_amd_uk_pack_params_t p = *params;
-  UK_RETURN_IF_ERROR(validate_pack(p));
-  if (p.out_size0 == 0 || p.out_size1 == 0 || p.out_size2 == 0 || p.out_size3 == 0) return 0;
-  const int es = pack_elem_bytes(p.flags);
-  const int64_t in_row = p.in_size1 > 0 ? (p.in_size1 - 1) * p.in_stride1 + 1 : 0;
-  const int64_t in_bytes = span_bytes(p.in_size0, p.in_stride0, in_row, es * 8);
-  const int64_t out_bytes = span_bytes(p.out_size0, p.out_stride0, p.out_size1 * p.out_stride1, es * 8);
-  const bool out_tight = p.out_stride0 == p.out_size1 * p.out_stride1;
-  Staging st;
-  UK_RETURN_IF_ERROR(st.init());
-  UK_RETURN_IF_ERROR(st.upload(0, p.in_buffer, p.in_offset * es, in_bytes, true));
-  UK_RETURN_IF_ERROR(st.upload(2, p.out_buffer, p.out_offset * es, out_bytes, !out_tight));
-  void* host_out = p.out_buffer;
-  const int64_t host_out_off = p.out_offset * es;
-  p.in_buffer = st.dev[0]; p.in_offset = 0;
-  p.out_buffer = st.dev[2]; p.out_offset = 0;
-  UK_RETURN_IF_ERROR(iree_amd_uk_pack_p(&p, st.stream));
-  return st.download(2, host_out, host_out_off, out_bytes);
-}
-
-extern "C" int iree_amd_uk_unpack_host(const iree_amd_uk_unpack_params_t* params) {
-  if (!params) return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "unpack_host: null params");
-  iree_amd_uk_unpack_params_t p = *params;
-  UK_RETURN_IF_ERROR(validate_unpack(p));
-  if (p.out_size0 == 0 || p.out_size1 == 0) return 0;
-  const int es = unpack_elem_bytes(p.flags);
-  const int64_t in_bytes = span_bytes(p.in_size0, p.in_stride0, p.in_size1 * p.in_stride1, es * 8);
-  const int64_t out_row = (p.out_size1 - 1) * p.out_stride1 + 1;
-  const int64_t out_bytes = span_bytes(p.out_size0, p.out_stride0, out_row, es * 8);
-  // The destination may have gaps (strides) the kernel must not disturb: start
-  // from the caller's bytes unless the destination is dense.
-  const bool out_dense = p.out_stride1 == 1 && p.out_stride0 == p.out_size1;
-  Staging st;
-  UK_RETURN_IF_ERROR(st.init());
-  UK_RETURN_IF_ERROR(st.upload(0, p.in_buffer, p.in_offset * es, in_bytes, true));
-  UK_RETURN_IF_ERROR(st.upload(2, p.out_buffer, p.out_offset * es, out_bytes, !out_dense));
-  void* host_out = p.out_buffer;
-  const int64_t host_out_off = p.out_offset * es;
-  p.in_buffer = st.dev[0]; p.in_offset = 0;
-  p.out_buffer = st.dev[2]; p.out_offset = 0;
-  UK_RETURN_IF_ERROR(iree_amd_uk_unpack_p(&p, st.stream));
-  return st.download(2, host_out, host_out_off, out_bytes);
-}

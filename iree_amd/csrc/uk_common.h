@@ -87,11 +87,52 @@ struct KSplitReduceArgs {
   int out_kind;              // 0 = accumulator type, 1 = f16, 2 = bf16
 };
 int launch_ksplit_reduce(const KSplitReduceArgs& r, hipStream_t s);
-// Device memory for the partial sums of a K split on stream `s` of the current
+// Device memory beyond a call's operands (the partial sums of a K split, a
+// packed copy of a row-major left-hand side) on stream `s` of the current
 // device: one buffer per stream, kept and reused by later calls (work on one
 // stream is ordered, so they cannot overlap), grown when a call needs more.
-// nullptr when it cannot be had (the call then runs unsplit).
-void* ksplit_scratch(hipStream_t s, size_t bytes);
+// The object must stay alive until the last launch that uses the memory has
+// been queued: until then the buffer is neither evicted nor replaced. ptr() is
+// nullptr when the memory cannot be had (the call then takes its fallback).
+//
+// A ScratchOverride on the calling thread replaces the cache for the calls made
+// under it: they get `ptr` when they need at most `bytes` and nothing
+// otherwise. With `strict`, a call that needs more does not fall back but fails
+// (overflowed() below): that is the entry point that allocates nothing.
+class ScratchLease {
+ public:
+  ScratchLease(hipStream_t s, size_t bytes);
+  ~ScratchLease();
+  ScratchLease(const ScratchLease&) = delete;
+  ScratchLease& operator=(const ScratchLease&) = delete;
+  void* ptr() const { return ptr_; }
+  // The calling thread runs under a strict override that is too small for
+  // this request: the caller returns scratch_overflow_status() instead of
+  // falling back.
+  bool overflowed() const { return overflowed_; }
+
+ private:
+  void* ptr_ = nullptr;
+  uint64_t id_ = 0;
+  bool overflowed_ = false;
+};
+class ScratchOverride {
+ public:
+  ScratchOverride(void* ptr, size_t bytes, bool strict);
+  ~ScratchOverride();
+  ScratchOverride(const ScratchOverride&) = delete;
+  ScratchOverride& operator=(const ScratchOverride&) = delete;
+
+ private:
+  void* prev_ptr_;
+  size_t prev_bytes_;
+  bool prev_strict_, prev_active_;
+};
+// Records the error of a request of `bytes` that a strict override cannot
+// serve and returns its status (RESOURCE_EXHAUSTED).
+int scratch_overflow_status(const char* what, size_t bytes);
+// Frees the cached buffers that no call is using; returns how many.
+size_t scratch_release_idle();
 
 int launch_pack(const iree_amd_uk_pack_params_t& p, hipStream_t s);
 int launch_unpack(const iree_amd_uk_unpack_params_t& p, hipStream_t s);

@@ -7,9 +7,9 @@
 #include "uk_common.h"
 #include "uk_mmt4d_mfma_kernel.h"
 #include "uk_mmt4d_mfma_launch.h"
+#include "uk_scratch_cache.h"
 
 #include <mutex>
-#include <vector>
 
 namespace uk {
 namespace {
@@ -69,43 +69,74 @@ __global__ __launch_bounds__(256) void ksplit_reduce_kernel(KSplitReduceArgs r) 
 
 }  // namespace
 
-void* ksplit_scratch(hipStream_t s, size_t bytes) {
-  struct Entry { int device; hipStream_t stream; void* ptr; size_t bytes; };
-  static std::mutex mutex;
-  static std::vector<Entry> entries;
-  constexpr size_t kMaxBytes = (size_t)512 << 20;   // larger problems run unsplit
-  constexpr size_t kMaxEntries = 64;
-  if (bytes == 0 || bytes > kMaxBytes) return nullptr;
+namespace {
+
+// The cache's allocator: plain hipMalloc / hipFree (which waits for the
+// device) / hipFreeAsync in stream order.
+void* scratch_alloc(size_t bytes, void*) {
+  void* p = nullptr;
+  if (hipMalloc(&p, bytes) != hipSuccess || !p) { (void)hipGetLastError(); return nullptr; }
+  return p;
+}
+void scratch_free_now(void* p, void*) {
+  if (hipFree(p) != hipSuccess) (void)hipGetLastError();
+}
+void scratch_free_ordered(void* p, void* stream, void*) {
+  if (hipFreeAsync(p, (hipStream_t)stream) != hipSuccess) { (void)hipGetLastError(); (void)hipFree(p); }
+}
+
+// 16 MiB at least per buffer, 512 MiB at most (larger problems run unsplit),
+// 64 (device, stream) pairs.
+ScratchCache& scratch_cache() {
+  static ScratchCache cache(ScratchAllocator{scratch_alloc, scratch_free_now, scratch_free_ordered, nullptr},
+                            (size_t)16 << 20, (size_t)512 << 20, 64);
+  return cache;
+}
+
+struct OverrideState { void* ptr; size_t bytes; bool strict, active; };
+thread_local OverrideState g_override = {nullptr, 0, false, false};
+
+}  // namespace
+
+ScratchLease::ScratchLease(hipStream_t s, size_t bytes) {
+  if (g_override.active) {
+    if (bytes != 0 && bytes <= g_override.bytes) ptr_ = g_override.ptr;
+    else overflowed_ = g_override.strict && bytes > g_override.bytes;
+    return;
+  }
   // (the per-thread default stream is one handle for a different stream in
   // every host thread: a buffer keyed by it would be shared by unordered work)
-  if (s == hipStreamPerThread) return nullptr;
+  if (s == hipStreamPerThread) return;
   int device = 0;
-  if (hipGetDevice(&device) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
-  std::lock_guard<std::mutex> lock(mutex);
-  for (Entry& e : entries) {
-    if (e.device != device || e.stream != s) continue;
-    if (e.bytes >= bytes) return e.ptr;
-    // Too small: earlier work on the stream may still use it, so it is freed
-    // in stream order; the replacement is twice what is asked for.
-    void* bigger = nullptr;
-    const size_t want = bytes * 2 < kMaxBytes ? bytes * 2 : kMaxBytes;
-    if (hipMalloc(&bigger, want) != hipSuccess || !bigger) { (void)hipGetLastError(); return nullptr; }
-    if (hipFreeAsync(e.ptr, s) != hipSuccess) { (void)hipGetLastError(); (void)hipFree(e.ptr); }
-    e.ptr = bigger;
-    e.bytes = want;
-    return e.ptr;
-  }
-  if (entries.size() >= kMaxEntries) {
-    // (streams come and go: drop the oldest buffer; hipFree waits for the device)
-    (void)hipFree(entries.front().ptr);
-    entries.erase(entries.begin());
-  }
-  void* ptr = nullptr;
-  const size_t want = bytes < ((size_t)16 << 20) ? (size_t)16 << 20 : bytes;
-  if (hipMalloc(&ptr, want) != hipSuccess || !ptr) { (void)hipGetLastError(); return nullptr; }
-  entries.push_back({device, s, ptr, want});
-  return ptr;
+  if (hipGetDevice(&device) != hipSuccess) { (void)hipGetLastError(); return; }
+  const ScratchCache::Lease lease = scratch_cache().acquire(device, (void*)s, bytes);
+  ptr_ = lease.ptr;
+  id_ = lease.id;
 }
+
+ScratchLease::~ScratchLease() {
+  if (id_) {
+    ScratchCache::Lease lease;
+    lease.ptr = ptr_;
+    lease.id = id_;
+    scratch_cache().release(lease);
+  }
+}
+
+ScratchOverride::ScratchOverride(void* ptr, size_t bytes, bool strict)
+    : prev_ptr_(g_override.ptr), prev_bytes_(g_override.bytes), prev_strict_(g_override.strict),
+      prev_active_(g_override.active) {
+  g_override = {ptr, bytes, strict, true};
+}
+ScratchOverride::~ScratchOverride() { g_override = {prev_ptr_, prev_bytes_, prev_strict_, prev_active_}; }
+
+int scratch_overflow_status(const char* what, size_t bytes) {
+  return fail(8 /* RESOURCE_EXHAUSTED */,
+              "%s needs %zu bytes of scratch memory; this entry point allocates nothing and has %zu",
+              what, bytes, g_override.bytes);
+}
+
+size_t scratch_release_idle() { return scratch_cache().release_idle(); }
 
 int launch_ksplit_reduce(const KSplitReduceArgs& r, hipStream_t s) {
   const int64_t groups = r.flat_elems > 0 ? r.flat_elems / 4 : (int64_t)r.M * r.N * 256;
@@ -297,7 +328,9 @@ int launch_matmul_packed_rhs_mfma(const iree_amd_uk_mmt4d_params_t& p, int64_t o
   const int eb = ti.lhs_bits / 8;
   const int64_t packed_bytes = p.M * p.K * 32 * p.K0 * eb;
   if (out_cols >= 8192 && out_rows >= 512) {
-    void* packed = ksplit_scratch(s, (size_t)packed_bytes);
+    // (held until the matmul that reads the packed copy has been queued)
+    ScratchLease lease(s, (size_t)packed_bytes);
+    void* packed = lease.ptr();
     if (packed) {
       iree_amd_uk_pack_params_t pp;
       pp.in_buffer = p.lhs_buffer; pp.in_offset = p.lhs_offset;

@@ -171,7 +171,10 @@ int launch_k_split(const MfmaArgs& a, int v, int slices, hipStream_t s) {
   slices = (a.ksteps + slice_ksteps - 1) / slice_ksteps;      // (no empty last slice)
   if (slices < 2) return IREE_AMD_UK_STATUS_NOT_FOUND;
   const int64_t slice_bytes = (int64_t)a.M * a.N * 1024 * (int64_t)sizeof(acc_elem_t);
-  void* scratch = ksplit_scratch(s, (size_t)(slice_bytes * slices));
+  // (held until the reduction kernel has been queued)
+  ScratchLease lease(s, (size_t)(slice_bytes * slices));
+  if (lease.overflowed()) return scratch_overflow_status("mmt4d: the K split", (size_t)(slice_bytes * slices));
+  void* scratch = lease.ptr();
   if (!scratch) return IREE_AMD_UK_STATUS_NOT_FOUND;
   MfmaArgs p = a;
   p.out = (char*)scratch;

@@ -18,6 +18,15 @@
 // q is consumed, across tile boundaries, so the stream never drains. The 8
 // partial 32x32 blocks are summed through LDS in wave order (deterministic)
 // and rows m0 < M0 are stored.
+//
+// A narrow RIGHT-hand side (N0 < 32, M0 = 32, one outer column: a result with
+// few columns, or the matrix-vector product) is the same problem with the
+// operands exchanged: the reference turns a narrow-N result into a narrow-M one
+// by transposition (compiler/src/iree/compiler/Codegen/Common/EncodingUtils.cpp:23-92
+// and chooseMatmulTile, .../Common/CPU/CPUMaterializeEncodingPass.cpp:296-303).
+// Here the kernel runs with the left-hand side streaming and the right-hand
+// side in registers and stores every block transposed, as the 32 x N0 tile the
+// caller asked for.
 #include "uk_common.h"
 #include "uk_mfma_cfg.h"
 
@@ -42,6 +51,9 @@ struct SkinnyArgs {
   int lhs_tile_bytes;  // M0 * K0 * element size
   int half_k0;
   int accumulate;
+  // the block is stored transposed: element (m0, n0) of the kernel's M0 x 32
+  // block at n0 * M0 + m0 (a 32 x M0 tile: the narrow right-hand side form)
+  int transpose_out;
   // K split over workgroup rows: row blockIdx.y takes steps [y * chunk_steps,
   // ...) and writes its sums, in the accumulator's type, chunk_out_elems
   // further on (one launch row and chunk_steps = ksteps when K is not split)
@@ -170,8 +182,9 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           const int nn = 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-          const sum_t sum = (a.accumulate ? (sum_t)tile[mm * 32 + nn] : (sum_t)0) + (sum_t)acc[v];
-          tile[mm * 32 + nn] = (store_t)sum;
+          const int at = a.transpose_out ? nn * a.M0 + mm : mm * 32 + nn;
+          const sum_t sum = (a.accumulate ? (sum_t)tile[at] : (sum_t)0) + (sum_t)acc[v];
+          tile[at] = (store_t)sum;
         }
       }
       continue;
@@ -188,10 +201,11 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
       const int l = flat & 63, v = flat >> 6;
       const int mm = l & 31, nn = 8 * (v >> 2) + 4 * (l >> 5) + (v & 3);
       if (mm < a.M0) {
-        sum_t sum = a.accumulate ? (sum_t)tile[mm * 32 + nn] : (sum_t)0;
+        const int at = a.transpose_out ? nn * a.M0 + mm : mm * 32 + nn;
+        sum_t sum = a.accumulate ? (sum_t)tile[at] : (sum_t)0;
 #pragma unroll
         for (int w = 0; w < kWaves; ++w) sum += buf[w][v][l];
-        tile[mm * 32 + nn] = (store_t)sum;
+        tile[at] = (store_t)sum;
       }
     }
     // The other half of `partial` serves the next tile; this half is rewritten
@@ -208,18 +222,22 @@ int launch_cfg(SkinnyArgs a, int chunks, hipStream_t s) {
   int per_plane = a.batch > 1 ? (2 * cus + a.batch - 1) / a.batch : cus;
   per_plane = per_plane > cus ? cus : per_plane;
   constexpr bool kNarrowOut = sizeof(typename Cfg::out_t) < 4;
-  // (Not for fp8: its instance of the per-wave form returned wrong values in
-  // the result columns n0 >= M0 and the cause has not been found; fp8 keeps
-  // the split over the waves.)
+  // (fp8: up to 8 steps; 16 of its 8-register fragments would not fit beside
+  // the rolling buffer)
+  constexpr int kPerWaveSteps = Cfg::kSub == 2 ? 8 : 16;
   const int groups = (a.N + kWaves - 1) / kWaves;
-  if (chunks == 1 && a.chunk_steps <= 16 && Cfg::kSub != 2 &&
+  if (chunks == 1 && a.chunk_steps <= kPerWaveSteps &&
       (int64_t)groups * (a.batch > 1 ? a.batch : 1) >= cus) {
     // a short K and enough outer columns to give every compute unit 8 of
     // them: one outer column per wave
     a.steps_per_wave = a.chunk_steps;
     const dim3 grid(groups < per_plane ? groups : per_plane, 1, a.batch > 1 ? a.batch : 1);
-    if (a.chunk_steps <= 8) hipLaunchKernelGGL((mmt4d_skinny_kernel<Cfg, 8, false, true>), grid, dim3(kThreads), 0, s, a);
-    else hipLaunchKernelGGL((mmt4d_skinny_kernel<Cfg, 16, false, true>), grid, dim3(kThreads), 0, s, a);
+    if (a.chunk_steps <= 8) {
+      hipLaunchKernelGGL((mmt4d_skinny_kernel<Cfg, 8, false, true>), grid, dim3(kThreads), 0, s, a);
+    } else {
+      if constexpr (kPerWaveSteps >= 16)
+        hipLaunchKernelGGL((mmt4d_skinny_kernel<Cfg, 16, false, true>), grid, dim3(kThreads), 0, s, a);
+    }
     return check_hip(hipGetLastError(), "mmt4d_skinny launch");
   }
   const int blocks = a.N < per_plane ? a.N : per_plane;
@@ -265,11 +283,13 @@ int mfma_k_of(uint32_t flags) {
 
 }  // namespace
 
-// Narrow tiles served: M0 < 32, N0 = 32, K0 = half or all of the MFMA's K extent.
+// Narrow tiles served: M0 < 32 with N0 = 32, or N0 < 32 with M0 = 32 (run with
+// the operands exchanged); K0 = half or all of the MFMA's K extent.
 bool mmt4d_skinny_supported(uint32_t flags, int M0, int N0, int K0) {
   const int mk = mfma_k_of(flags);
-  if (mk == 64) return M0 >= 1 && M0 < 32 && N0 == 32 && K0 == 16;
-  return mk && M0 >= 1 && M0 < 32 && N0 == 32 && (K0 == mk || K0 * 2 == mk);
+  const bool narrow = (M0 >= 1 && M0 < 32 && N0 == 32) || (N0 >= 1 && N0 < 32 && M0 == 32);
+  if (mk == 64) return narrow && K0 == 16;
+  return mk && narrow && (K0 == mk || K0 * 2 == mk);
 }
 
 namespace {
@@ -282,14 +302,37 @@ int max_steps_per_launch(int mfma_k) { return kWaves * (mfma_k == 64 ? 16 : 32);
 struct BatchStrides { int64_t batch, lhs, rhs, out; };   // strides in elements
 int launch_chunk(const iree_amd_uk_mmt4d_params_t& p, int chunks, int chunk_steps, void* scratch,
                  hipStream_t s, const BatchStrides* batch = nullptr);
+
+// The narrow right-hand side form as the narrow left-hand side problem the
+// kernel solves: operands exchanged, the 32 x N0 result tiles (one per outer
+// row, out_stride0 apart) written transposed. The marker travels in a flag
+// bit that no public flag uses.
+constexpr uint32_t kTransposedOut = 0x80000000u;
+bool narrow_rhs_form(const iree_amd_uk_mmt4d_params_t& p) { return p.N0 < 32 && p.M0 == 32; }
+iree_amd_uk_mmt4d_params_t exchanged(const iree_amd_uk_mmt4d_params_t& p) {
+  iree_amd_uk_mmt4d_params_t q = p;
+  q.lhs_buffer = p.rhs_buffer; q.lhs_offset = p.rhs_offset; q.lhs_stride0 = p.rhs_stride0;
+  q.rhs_buffer = p.lhs_buffer; q.rhs_offset = p.lhs_offset; q.rhs_stride0 = p.lhs_stride0;
+  q.M = p.N; q.N = p.M;
+  q.M0 = p.N0; q.N0 = p.M0;
+  q.flags = p.flags | kTransposedOut;
+  return q;
+}
 }  // namespace
 
 // `batch` problems of one narrow shape as the planes of one launch; only what a
 // single launch row takes (K short enough to stay in registers), at most 65535
 // entries and batch strides of whole 16 bytes.
-int launch_batch_mmt4d_skinny(const iree_amd_uk_mmt4d_params_t& p, int64_t batch, int64_t lhs_batch_stride,
+int launch_batch_mmt4d_skinny(const iree_amd_uk_mmt4d_params_t& p0, int64_t batch, int64_t lhs_batch_stride,
                               int64_t rhs_batch_stride, int64_t out_batch_stride, hipStream_t s) {
-  if (!mmt4d_skinny_supported(p.flags, p.M0, p.N0, p.K0)) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  if (!mmt4d_skinny_supported(p0.flags, p0.M0, p0.N0, p0.K0)) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  iree_amd_uk_mmt4d_params_t p = p0;
+  if (narrow_rhs_form(p0)) {
+    p = exchanged(p0);
+    const int64_t t = lhs_batch_stride;
+    lhs_batch_stride = rhs_batch_stride;
+    rhs_batch_stride = t;
+  }
   const int mk = mfma_k_of(p.flags);
   const int64_t k_elems = p.K * p.K0;
   if (p.M != 1 || p.K == 0 || k_elems % mk || p.N > 0x7FFFFFFF || batch > 65535)
@@ -300,8 +343,10 @@ int launch_batch_mmt4d_skinny(const iree_amd_uk_mmt4d_params_t& p, int64_t batch
   return launch_chunk(p, 1, (int)steps, nullptr, s, &bs);
 }
 
-int launch_mmt4d_skinny(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) {
-  if (!mmt4d_skinny_supported(p.flags, p.M0, p.N0, p.K0)) return IREE_AMD_UK_STATUS_NOT_FOUND;
+int launch_mmt4d_skinny(const iree_amd_uk_mmt4d_params_t& p0, hipStream_t s) {
+  if (!mmt4d_skinny_supported(p0.flags, p0.M0, p0.N0, p0.K0)) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  const iree_amd_uk_mmt4d_params_t p = narrow_rhs_form(p0) ? exchanged(p0) : p0;
+  const bool transposed = (p.flags & kTransposedOut) != 0;
   const int mk = mfma_k_of(p.flags);
   const int64_t k_elems = p.K * p.K0;
   if (p.M != 1 || p.K == 0 || k_elems % mk || p.N > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
@@ -318,19 +363,24 @@ int launch_mmt4d_skinny(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) {
   // floats the same sum in another order.
   const int cus = device_cu_count();
   int64_t chunks = (steps + max_steps - 1) / max_steps;
-  if (p.N * chunks * 2 <= cus && steps >= 64) {
+  // (partial sums and result are dense arrays there: transposed tiles must
+  // follow each other without gaps)
+  const bool dense_out = !transposed || p.N == 1 || p.out_stride0 == (int64_t)p.M0 * 32;
+  if (dense_out && p.N * chunks * 2 <= cus && steps >= 64) {
     int64_t more = cus / p.N;
     if (more > steps / 32) more = steps / 32;
     if (more > 8) more = 8;
     if (more > chunks) chunks = more;
   }
-  if (chunks > 1) {
+  if (chunks > 1 && dense_out) {
     const int64_t chunk_steps = (steps + chunks - 1) / chunks;
     chunks = (steps + chunk_steps - 1) / chunk_steps;
     const int64_t elems = p.N * p.M0 * 32;
     // (the tiles of the single outer row are consecutive: partial sums and
     // result are dense arrays)
-    void* scratch = ksplit_scratch(s, (size_t)(chunks * elems * 4));
+    ScratchLease lease(s, (size_t)(chunks * elems * 4));
+    if (lease.overflowed()) return scratch_overflow_status("mmt4d: the K split of a narrow tile", (size_t)(chunks * elems * 4));
+    void* scratch = lease.ptr();
     if (scratch && chunks > 1) {
       int st = launch_chunk(p, (int)chunks, (int)chunk_steps, scratch, s);
       if (st) return st;
@@ -393,7 +443,10 @@ int launch_chunk(const iree_amd_uk_mmt4d_params_t& p, int chunks, int chunk_step
   a.lhs = lhs; a.rhs = rhs;
   a.out = (char*)p.out_buffer + p.out_offset * ti.out_bytes;
   a.rhs_stride_bytes = p.rhs_stride0 * eb;
-  a.out_stride_elems = (int64_t)p.M0 * 32;   // consecutive outer columns of the single outer row
+  // consecutive outer columns of the single outer row; exchanged operands: the
+  // tiles of the caller's outer rows, out_stride0 apart
+  a.transpose_out = (p.flags & kTransposedOut) != 0;
+  a.out_stride_elems = a.transpose_out ? p.out_stride0 : (int64_t)p.M0 * 32;
   a.N = (int)p.N; a.M0 = p.M0;
   a.ksteps = (int)(k_elems / mk);
   a.steps_per_wave = 0;
@@ -415,6 +468,7 @@ int launch_chunk(const iree_amd_uk_mmt4d_params_t& p, int chunks, int chunk_step
     a.out = (char*)scratch;
     a.accumulate = 0;
     a.chunk_out_elems = (int64_t)p.N * p.M0 * 32;
+    a.out_stride_elems = (int64_t)p.M0 * 32;     // (partial sums are dense)
   }
   switch (p.flags & IREE_AMD_UK_FLAG_MMT4D_TYPE_MASK) {
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F32: return launch_cfg<F16Cfg>(a, chunks, s);

@@ -33,6 +33,8 @@
 #include "uk_common.h"
 #include "uk_i4.h"
 
+#include <memory>
+
 namespace uk {
 using namespace i4;
 namespace {
@@ -397,13 +399,15 @@ int launch_dequant_gemv_i4(const I4Args& p, int m_base, int m_eff, hipStream_t s
   a.row_chunks = a.chunks;
   a.k_rows = 1;
   a.partial_out = nullptr;
+  std::unique_ptr<ScratchLease> lease;   // held until the reduction has been queued
   if (a.chunks * chunk_x_bytes > 144 * 1024) {
     a.row_chunks = (int)((144 * 1024) / chunk_x_bytes);
     if (a.row_chunks < 1 || N % 4) return IREE_AMD_UK_STATUS_NOT_FOUND;
     a.k_rows = (a.chunks + a.row_chunks - 1) / a.row_chunks;
     a.row_chunks = (a.chunks + a.k_rows - 1) / a.k_rows;      // equal rows
     a.k_rows = (a.chunks + a.row_chunks - 1) / a.row_chunks;
-    a.partial_out = (float*)ksplit_scratch(s, (size_t)a.k_rows * m_eff * N * 4);
+    lease.reset(new ScratchLease(s, (size_t)a.k_rows * m_eff * N * 4));
+    a.partial_out = (float*)lease->ptr();
     if (!a.partial_out) return IREE_AMD_UK_STATUS_NOT_FOUND;
   }
   size_t lds = (size_t)(a.row_chunks * chunk_x_bytes);

@@ -46,17 +46,29 @@
 #include "iree_amd_hal_plugin_abi.h"
 #include "iree_amd_uk.h"
 
-typedef int (*mmt4d_host_fn_t)(const iree_amd_uk_mmt4d_params_t*);
-typedef int (*pack_host_fn_t)(const iree_amd_uk_pack_params_t*);
-typedef int (*unpack_host_fn_t)(const iree_amd_uk_unpack_params_t*);
+typedef int (*pool_create_fn_t)(iree_amd_uk_host_pool_t**);
+typedef void (*pool_destroy_fn_t)(iree_amd_uk_host_pool_t*);
+typedef int (*mmt4d_host_fn_t)(iree_amd_uk_host_pool_t*, const iree_amd_uk_mmt4d_params_t*);
+typedef int (*pack_host_fn_t)(iree_amd_uk_host_pool_t*, const iree_amd_uk_pack_params_t*);
+typedef int (*unpack_host_fn_t)(iree_amd_uk_host_pool_t*, const iree_amd_uk_unpack_params_t*);
+typedef int (*release_scratch_fn_t)(void);
 typedef const char* (*last_error_fn_t)(void);
 
+/* One per load(): several instances may live in one process
+ * (REF runtime/src/iree/hal/local/executable_plugin.h:415-418), so everything a
+ * call needs hangs off this struct - the staging pool included - and nothing is
+ * global. The imports are called from arbitrary threads concurrently
+ * (REF samples/custom_dispatch/cpu/plugin/system_plugin.c:21-25): the struct is
+ * read-only after load and the pool hands every call a slot of its own. */
 typedef struct mi355x_plugin_t {
   iree_amd_hal_plugin_allocator_t host_allocator;
   void* library;
+  iree_amd_uk_host_pool_t* pool;
+  pool_destroy_fn_t pool_destroy;
   mmt4d_host_fn_t mmt4d;
   pack_host_fn_t pack;
   unpack_host_fn_t unpack;
+  release_scratch_fn_t release_scratch;
   last_error_fn_t last_error;
 } mi355x_plugin_t;
 
@@ -72,17 +84,17 @@ static int report(mi355x_plugin_t* plugin, const char* what, int status) {
 static int import_mmt4d(void* params, void* context, void* reserved) {
   (void)reserved;
   mi355x_plugin_t* plugin = (mi355x_plugin_t*)context;
-  return report(plugin, "mmt4d", plugin->mmt4d((const iree_amd_uk_mmt4d_params_t*)params));
+  return report(plugin, "mmt4d", plugin->mmt4d(plugin->pool, (const iree_amd_uk_mmt4d_params_t*)params));
 }
 static int import_pack(void* params, void* context, void* reserved) {
   (void)reserved;
   mi355x_plugin_t* plugin = (mi355x_plugin_t*)context;
-  return report(plugin, "pack", plugin->pack((const iree_amd_uk_pack_params_t*)params));
+  return report(plugin, "pack", plugin->pack(plugin->pool, (const iree_amd_uk_pack_params_t*)params));
 }
 static int import_unpack(void* params, void* context, void* reserved) {
   (void)reserved;
   mi355x_plugin_t* plugin = (mi355x_plugin_t*)context;
-  return report(plugin, "unpack", plugin->unpack((const iree_amd_uk_unpack_params_t*)params));
+  return report(plugin, "unpack", plugin->unpack(plugin->pool, (const iree_amd_uk_unpack_params_t*)params));
 }
 
 /* The llvm-cpu form: a leading i32 result, then the parameters at the next
@@ -155,15 +167,22 @@ static iree_amd_hal_plugin_status_t plugin_load(
     }
   }
   plugin->library = open_uk_library(path);
+  pool_create_fn_t pool_create = NULL;
   if (plugin->library) {
-    plugin->mmt4d = (mmt4d_host_fn_t)dlsym(plugin->library, "iree_amd_uk_mmt4d_host");
-    plugin->pack = (pack_host_fn_t)dlsym(plugin->library, "iree_amd_uk_pack_host");
-    plugin->unpack = (unpack_host_fn_t)dlsym(plugin->library, "iree_amd_uk_unpack_host");
+    pool_create = (pool_create_fn_t)dlsym(plugin->library, "iree_amd_uk_host_pool_create");
+    plugin->pool_destroy = (pool_destroy_fn_t)dlsym(plugin->library, "iree_amd_uk_host_pool_destroy");
+    plugin->mmt4d = (mmt4d_host_fn_t)dlsym(plugin->library, "iree_amd_uk_mmt4d_host_pooled");
+    plugin->pack = (pack_host_fn_t)dlsym(plugin->library, "iree_amd_uk_pack_host_pooled");
+    plugin->unpack = (unpack_host_fn_t)dlsym(plugin->library, "iree_amd_uk_unpack_host_pooled");
+    plugin->release_scratch = (release_scratch_fn_t)dlsym(plugin->library, "iree_amd_uk_release_scratch");
     plugin->last_error = (last_error_fn_t)dlsym(plugin->library, "iree_amd_uk_last_error");
   }
-  if (!plugin->library || !plugin->mmt4d || !plugin->pack || !plugin->unpack) {
+  const int have_entry_points = plugin->library && pool_create && plugin->pool_destroy && plugin->mmt4d &&
+                                plugin->pack && plugin->unpack;
+  /* (creating the pool touches no device: its streams and buffers come with the first call) */
+  if (!have_entry_points || pool_create(&plugin->pool) != 0 || !plugin->pool) {
     fprintf(stderr, "mi355x_uk plugin: cannot load the microkernel library: %s\n",
-            plugin->library ? "missing entry points" : dlerror());
+            !plugin->library ? dlerror() : !have_entry_points ? "missing entry points" : "no staging pool");
     if (plugin->library) dlclose(plugin->library);
     void* p = plugin;
     environment->host_allocator.ctl(environment->host_allocator.self,
@@ -178,6 +197,10 @@ static void plugin_unload(void* self) {
   mi355x_plugin_t* plugin = (mi355x_plugin_t*)self;
   if (!plugin) return;
   iree_amd_hal_plugin_allocator_t allocator = plugin->host_allocator;
+  /* Everything is freed here: the library may be closed right after
+   * (REF executable_plugin.h:424-427). No import is running any more. */
+  if (plugin->pool) plugin->pool_destroy(plugin->pool);
+  if (plugin->release_scratch) plugin->release_scratch();
   if (plugin->library) dlclose(plugin->library);
   void* p = plugin;
   allocator.ctl(allocator.self, IREE_AMD_HAL_PLUGIN_ALLOCATOR_FREE, NULL, &p);

@@ -123,8 +123,16 @@ def test_query_tile_sizes_roles_and_narrowing():
     assert q(op | F.QUERY_ROLE_LHS, 1, 4096) == (1, 8)
     assert q(op | F.QUERY_ROLE_LHS, 7, 4096) == (8, 8)
     assert q(op | F.QUERY_ROLE_LHS, 17, 4096) == (32, 8)
-    assert q(op | F.QUERY_ROLE_RESULT, 8, 3) == (8, 4)
     assert q(op | F.QUERY_ROLE_RHS, 4096, 4096) == (32, 8)
+    assert q(op | F.QUERY_ROLE_RHS, 5, 4096) == (8, 8)
+    # the result role sees both sizes and narrows only the smaller one, N by
+    # transposition only when it is the narrower of the two
+    # (CPUMaterializeEncodingPass.cpp:296-303 of the reference)
+    assert q(op | F.QUERY_ROLE_RESULT, 8, 3) == (32, 4)
+    assert q(op | F.QUERY_ROLE_RESULT, 3, 8) == (4, 32)
+    assert q(op | F.QUERY_ROLE_RESULT, 8, 8) == (8, 32)
+    assert q(op | F.QUERY_ROLE_RESULT, 4096, 1) == (32, 1)
+    assert q(op | F.QUERY_ROLE_RESULT, 16, 4096) == (16, 32)
     with pytest.raises(iree_amd.UkError) as e:
         q(0x0700 | F.QUERY_ROLE_LHS)
     assert e.value.status == F.STATUS_INVALID_ARGUMENT
@@ -140,6 +148,46 @@ def test_mmt4d_info_reports_mfma_tiles():
     assert iree_amd.mmt4d_info(32, 32, 32, F.MMT4D_TYPE_S8S8S32) == have
     assert iree_amd.mmt4d_info(16, 16, 1, F.MMT4D_TYPE_F16F16F32) == 0
     assert iree_amd.mmt4d_info(32, 32, 8, F.MMT4D_TYPE_S16S16S32) == 0
+
+
+def test_every_tile_the_query_returns_has_an_architecture_kernel():
+    """mmt4d_info reports a matrix-core kernel for each tile
+    query_tile_sizes_2d can hand out: full tiles, narrow M0 (static M < 32) and
+    narrow N0 (static N < 32, served with the operands exchanged)."""
+    have = F.MMT4D_INFO_HAVE_ARCHITECTURE_SPECIFIC_TILE_FUNCTION
+    q = iree_amd.query_tile_sizes_2d
+    dyn = -2 ** 63
+    sizes = [dyn, 1, 2, 3, 4, 5, 7, 8, 9, 15, 16, 17, 31, 32, 33, 4096]
+    for op, type_flag in [(F.QUERY_OP_MATMUL_I8I8I32, F.MMT4D_TYPE_S8S8S32),
+                          (F.QUERY_OP_MATMUL_F16F16F32, F.MMT4D_TYPE_F16F16F32),
+                          (F.QUERY_OP_MATMUL_F16F16F16, F.MMT4D_TYPE_F16F16F16),
+                          (F.QUERY_OP_MATMUL_BF16BF16F32, F.MMT4D_TYPE_BF16BF16F32),
+                          (F.QUERY_OP_MATMUL_BF16BF16BF16, F.MMT4D_TYPE_BF16BF16BF16),
+                          (F.QUERY_OP_MATMUL_F32F32F32, F.MMT4D_TYPE_F32F32F32),
+                          (F.QUERY_OP_MATMUL_F8E4M3F8E4M3F32, F.MMT4D_TYPE_F8E4M3F8E4M3F32)]:
+        flags = type_flag | F.MMT4D_SKIP_INTERMEDIATE_ROUNDINGS
+        for m in sizes:
+            for n in sizes:
+                m0, n0 = q(op | F.QUERY_ROLE_RESULT, m, n)
+                assert m0 == 32 or n0 == 32, (m, n, m0, n0)
+                # the operand queries a caller makes for this matmul: the wider
+                # of two narrow dimensions is passed as dynamic
+                m_arg = m if m0 < 32 or n0 == 32 else dyn
+                n_arg = n if n0 < 32 or m0 == 32 else dyn
+                if m0 < 32:
+                    n_arg = dyn if 0 < n < 32 else n
+                if n0 < 32:
+                    m_arg = dyn if 0 < m < 32 else m
+                lm0, k0 = q(op | F.QUERY_ROLE_LHS, m_arg, 4096)
+                rn0, rk0 = q(op | F.QUERY_ROLE_RHS, n_arg, 4096)
+                assert (lm0, rn0, rk0) == (m0, n0, k0), (m, n)
+                assert iree_amd.mmt4d_info(m0, n0, k0, flags) == have, (hex(type_flag), m0, n0, k0)
+        # each operand query on its own also only yields served tiles
+        for sz in sizes:
+            lm0, k0 = q(op | F.QUERY_ROLE_LHS, sz, 4096)
+            assert iree_amd.mmt4d_info(lm0, 32, k0, flags) == have
+            rn0, k0 = q(op | F.QUERY_ROLE_RHS, sz, 4096)
+            assert iree_amd.mmt4d_info(32, rn0, k0, flags) == have
 
 
 def test_validation_happens_before_any_device_work():

@@ -143,6 +143,57 @@ def test_narrow_lhs_tiles_bit_exact(uk, cuda, type_flag, K0):
         assert np.array_equal(gpucase.run_mmt4d(case), case.run_oracle(ukref.F16_IEEE)), (M, N, K)
 
 
+@pytest.mark.parametrize("type_flag,K0", [(F.MMT4D_TYPE_F16F16F32, 8), (F.MMT4D_TYPE_F16F16F32, 16),
+                                          (F.MMT4D_TYPE_BF16BF16F32, 8), (F.MMT4D_TYPE_S8S8S32, 16),
+                                          (F.MMT4D_TYPE_S8S8S32, 32), (F.MMT4D_TYPE_F32F32F32, 4),
+                                          (F.MMT4D_TYPE_F16F16F16, 8), (F.MMT4D_TYPE_BF16BF16BF16, 16),
+                                          (F.MMT4D_TYPE_F8E4M3F8E4M3F32, 16)])
+def test_narrow_rhs_tiles_bit_exact(uk, cuda, type_flag, K0):
+    """Narrow right-hand-side tiles (N0 < 32, M0 = 32, one outer column: what
+    the tile-size query hands out for a static N below 32, and the
+    matrix-vector product at N0 = 1). The library runs them as the narrow
+    left-hand-side problem with the operands exchanged and stores the tiles
+    transposed (the reference does the transposition in the compiler,
+    EncodingUtils.cpp:23-92). Same shape list as the narrow left-hand-side
+    test, generic fallback NOT allowed, bits of the oracle; loose strides of
+    the result (tiles not back to back), and what the kernel does not take
+    (two outer columns, unaligned operands) through the element-wise kernel."""
+    rng = np.random.default_rng(7100 + type_flag + K0)
+    mfma_k = {F.MMT4D_TYPE_S8S8S32: 32, F.MMT4D_TYPE_F32F32F32: 8,
+              F.MMT4D_TYPE_F8E4M3F8E4M3F32: 64}.get(type_flag, 16)
+    tps = mfma_k // K0
+    for N0 in (1, 2, 4, 8, 16):
+        assert uk.mmt4d_info(32, N0, K0, type_flag | F.MMT4D_SKIP_INTERMEDIATE_ROUNDINGS) == 1
+        for M, steps, acc in ((1, 1, False), (5, 8, True), (300, 13, False), (3, 70, True),
+                              (7, 128, False), (2, 255, True), (2100, 8, True), (2051, 13, False),
+                              (2300, 3, False)):
+            case = ukref.Mmt4dCase(rng, type_flag, M, 1, steps * tps, 32, N0, K0, accumulate=acc)
+            got = gpucase.run_mmt4d(case, flags=case.flags & ~F.MMT4D_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION)
+            assert np.array_equal(got.view(np.uint8), case.run_oracle(ukref.F16_IEEE).view(np.uint8)), \
+                (hex(type_flag), N0, K0, M, steps, acc)
+    for N0, M, steps, acc in ((8, 40, 600, False), (1, 9, 896, True), (16, 3, 257, False),
+                              (4, 100, 300, True), (2, 128, 64, False)):
+        case = ukref.Mmt4dCase(rng, type_flag, M, 1, steps * tps, 32, N0, K0, accumulate=acc)
+        got = gpucase.run_mmt4d(case, flags=case.flags & ~F.MMT4D_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION)
+        assert np.array_equal(got.view(np.uint8), case.run_oracle(ukref.F16_IEEE).view(np.uint8)), \
+            (hex(type_flag), N0, K0, M, steps, acc)
+    # result tiles with gaps between them (16-byte aligned operand strides keep
+    # the call on the matrix-core kernel): short K, long K in one launch row,
+    # and a long K with few outer rows, which cannot be split through the
+    # dense scratch buffer
+    for M, steps, acc in ((6, 8, True), (300, 40, False), (3, 200, True)):
+        case = ukref.Mmt4dCase(rng, type_flag, M, 1, steps * tps, 32, 4, K0, accumulate=acc)
+        case.out_stride0 += 24
+        case.out_init = np.resize(case.out_init, case.out_init.size + M * 24)
+        got = gpucase.run_mmt4d(case, flags=case.flags & ~F.MMT4D_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION)
+        assert np.array_equal(got.view(np.uint8), case.run_oracle(ukref.F16_IEEE).view(np.uint8)), \
+            (hex(type_flag), M, steps, acc)
+    for M, N, K in ((3, 2, 4 * tps), (3, 1, 2 * tps + (1 if tps > 1 else 0)), (2, 1, 260 * tps)):
+        case = ukref.Mmt4dCase(rng, type_flag, M, N, K, 32, 8, K0, accumulate=True,
+                               loose_strides=True, offsets=True)
+        assert np.array_equal(gpucase.run_mmt4d(case), case.run_oracle(ukref.F16_IEEE)), (M, N, K)
+
+
 def test_without_fallback_permission_unserved_tiles_are_refused(uk, cuda):
     rng = np.random.default_rng(1)
     case = ukref.Mmt4dCase(rng, F.MMT4D_TYPE_S8S8S32, 2, 2, 2, 9, 6, 3)
@@ -650,7 +701,10 @@ def test_k_split_scratch_grows_and_is_kept_per_stream(uk, cuda):
         outs = []
         for st in streams:
             out = torch.zeros(M1 * 32 * N1 * 32, dtype=torch.int32, device=cuda)
-            torch.cuda.synchronize()
+            # (no device synchronisation between the calls: earlier work of the
+            # stream is still queued when its buffer is replaced; the stream
+            # only waits for the operands prepared on the current one)
+            st.wait_stream(torch.cuda.current_stream())
             with torch.cuda.stream(st):
                 uk.matmul_packed_rhs(a_dev, rhs, out, M1 * 32, N1 * 32, K1 * 16, 16, F.MMT4D_TYPE_S8S8S32,
                                      stream=st)
@@ -661,6 +715,17 @@ def test_k_split_scratch_grows_and_is_kept_per_stream(uk, cuda):
         want = A.astype(np.int32) @ B.astype(np.int32).T
         for out in outs:
             assert np.array_equal(out.cpu().numpy().reshape(want.shape), want)
+    # the cached buffers can be given back (what a plugin's unload does) and
+    # come back on demand
+    lib = uk.load_library()
+    free0 = torch.cuda.mem_get_info()[0]
+    assert lib.iree_amd_uk_release_scratch() == 0
+    assert torch.cuda.mem_get_info()[0] >= free0 + (16 << 20)
+    A, B, outs, a_dev, rhs = jobs[1]
+    again = torch.zeros_like(outs[0])
+    uk.matmul_packed_rhs(a_dev, rhs, again, A.shape[0], B.shape[0], A.shape[1], 16, F.MMT4D_TYPE_S8S8S32)
+    torch.cuda.synchronize()
+    assert torch.equal(again, outs[0])
 
 
 @pytest.mark.gpu

@@ -221,3 +221,63 @@ def test_plain_c_host_program_drives_the_plugin(cuda):
     r = subprocess.run([exe, PLUGIN, _lib.library_path()], capture_output=True, text=True, timeout=120)
     assert r.returncode == 0, r.stdout + r.stderr
     assert "OK:" in r.stdout
+
+
+@pytest.mark.gpu
+def test_imports_called_from_many_host_threads_at_once(host, uk, cuda):
+    """The contract of an import: "called from arbitrary threads concurrently"
+    (samples/custom_dispatch/cpu/plugin/system_plugin.c:21-25 of the reference).
+    12 host threads (more than the pool has slots, so some calls wait for one)
+    each run pack, pack, mmt4d, unpack on buffers of their own, several times,
+    with shapes that make the pool's buffers grow; every result is the exact
+    integer product."""
+    import threading
+    plugin = host.query().contents
+    status, self_ptr = host.load(plugin, [(b"uk_library", _lib.library_path().encode())])
+    assert status == 0
+    status, _, fns, ctxs = host.resolve(plugin, self_ptr,
+                                        [b"mi355x_uk_pack", b"mi355x_uk_mmt4d", b"mi355x_uk_unpack"])
+    assert status == 0
+    pack_fn, mmt4d_fn, unpack_fn = (IMPORT(f) for f in fns)
+    ptr = lambda x: x.ctypes.data_as(C.c_void_p)  # noqa: E731
+    M0, N0, K0 = 32, 32, 16
+    errors = []
+
+    def worker(t):
+        try:
+            rng = np.random.default_rng(100 + t)
+            for rep in range(3):
+                M, N, K = 40 + 37 * t + 5 * rep, 200 - 11 * t + rep, 64 + 48 * ((t + rep) % 5)
+                M1, N1, K1 = -(-M // M0), -(-N // N0), -(-K // K0)
+                a = rng.integers(-128, 128, size=(M, K)).astype(np.int8)
+                b = rng.integers(-128, 128, size=(K, N)).astype(np.int8)
+                lhs = np.full(M1 * K1 * M0 * K0, 0x55, np.int8)
+                rhs = np.full(N1 * K1 * N0 * K0, 0x55, np.int8)
+                acc = np.full(M1 * N1 * M0 * N0, -1, np.int32)
+                c = np.full((M, N), -7, np.int32)
+                p = _lib.PackParams(ptr(a), 0, K, 1, ptr(lhs), 0, K1 * M0 * K0, M0 * K0, M, K, M1, K1, M0, K0,
+                                    0, F.PACK_TYPE_I8I8, None)
+                assert pack_fn(C.addressof(p), ctxs[0], None) == 0
+                p = _lib.PackParams(ptr(b), 0, N, 1, ptr(rhs), 0, K1 * N0 * K0, N0 * K0, K, N, N1, K1, N0, K0,
+                                    0, F.PACK_TYPE_I8I8 | F.PACK_TRANSPOSE_INNER | F.PACK_TRANSPOSE_OUTER, None)
+                assert pack_fn(C.addressof(p), ctxs[0], None) == 0
+                m = _lib.Mmt4dParams(ptr(lhs), 0, K1 * M0 * K0, ptr(rhs), 0, K1 * N0 * K0, ptr(acc), 0,
+                                     N1 * M0 * N0, M1, N1, K1, M0, N0, K0, F.MMT4D_TYPE_S8S8S32, None)
+                assert mmt4d_fn(C.addressof(m), ctxs[1], None) == 0
+                u = _lib.UnpackParams(ptr(acc), 0, N1 * M0 * N0, M0 * N0, ptr(c), 0, N, 1, M1, N1, M0, N0,
+                                      M, N, F.UNPACK_TYPE_I32I32, None)
+                assert unpack_fn(C.addressof(u), ctxs[2], None) == 0
+                want = a.astype(np.int32) @ b.astype(np.int32)
+                assert np.array_equal(c, want), (t, rep, M, N, K)
+        except BaseException as e:  # noqa: BLE001
+            errors.append((t, repr(e)))
+
+    threads = [threading.Thread(target=worker, args=(t,)) for t in range(12)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join(timeout=300)
+    assert not any(th.is_alive() for th in threads), "a worker thread did not finish"
+    assert not errors, errors
+    plugin.unload(self_ptr)
+    assert host.live == 0
