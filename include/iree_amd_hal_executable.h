@@ -19,6 +19,16 @@
  *                                      REF runtime/src/iree/hal/drivers/hip/stream_command_buffer.c:519-581
  * Status codes are those of iree_amd_uk.h (0 = OK); the message of a failure is
  * read with iree_amd_uk_last_error().
+ *
+ * Limits of the exports in mi355x_kernels_gfx950.co (a kernel cannot report an
+ * error: a dispatch outside them returns without writing anything):
+ *   mi355x_mmt4d_*, mi355x_mmt4d_unpack_*   one outer row of an operand
+ *       (32 x K elements) below 2 GiB; K whole K0 tiles; dense operands.
+ *   mi355x_matmul_packed_rhs_*              the row-major left-hand side
+ *       (M x K elements) below 2 GiB: its rows are addressed with 32-bit byte
+ *       offsets; K a multiple of the matrix-core K extent.
+ *   mi355x_pack_*, mi355x_unpack_*          power-of-two tile sizes whose rows
+ *       are whole 16-byte chunks, no transposes.
  */
 #ifndef IREE_AMD_HAL_EXECUTABLE_H_
 #define IREE_AMD_HAL_EXECUTABLE_H_

@@ -153,6 +153,24 @@ struct F8Cfg {
   }
 };
 
+// Matrix-core instructions take their operands from all 64 lanes whatever the
+// execution mask, but the compiler treats the fp8 one
+// (v_mfma_scale_f32_32x32x64_f8f6f4) like per-lane arithmetic: when its result
+// is only consumed inside a divergent region (stores of the lanes m0 < M0,
+// say) it moves the instruction, and the per-lane selects and copies that
+// prepare its operands, into that region, where those run for the active lanes
+// only and the instruction then reads stale registers in all the others. This
+// pins a result to the point where it is called, with every lane active: the
+// empty volatile statement cannot move into a conditional block, and what
+// produced its operand has to come before it. One element is enough, the
+// instruction writes the whole block at once.
+template <typename Acc>
+__device__ __forceinline__ void keep_result_in_all_lanes(Acc& acc) {
+  auto first = acc[0];
+  asm volatile("" : "+v"(first));
+  acc[0] = first;
+}
+
 // The configuration that computes the same products with the accumulator type
 // as result type (partial sums of a K split are kept in it).
 template <typename Cfg> struct PartialSumCfg { typedef Cfg type; };

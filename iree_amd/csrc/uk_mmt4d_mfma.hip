@@ -213,8 +213,8 @@ int make_args(const iree_amd_uk_mmt4d_params_t& p, int out_elem_bytes, bool silu
   const char* rhs = (const char*)p.rhs_buffer + p.rhs_offset * eb;
   if (((uintptr_t)lhs | (uintptr_t)rhs) % 16) return IREE_AMD_UK_STATUS_NOT_FOUND;
   if ((p.lhs_stride0 * eb) % 16 || (p.rhs_stride0 * eb) % 16) return IREE_AMD_UK_STATUS_NOT_FOUND;
-  // (the kernel addresses an operand row with 32-bit byte offsets)
-  if (k_elems * eb + 4096 > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  // (the kernel addresses an outer row of 32 x K elements with 32-bit byte offsets)
+  if (k_elems * 32 * eb + 4096 > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
   MfmaArgs& a = *out_args;
   a.lhs = lhs; a.rhs = rhs;
   a.out = (char*)p.out_buffer + p.out_offset * out_elem_bytes;

@@ -590,6 +590,14 @@ __device__ __forceinline__ void mmt4d_mfma_body(const MfmaArgs a, const int bid 
       fb[0][y] = tail_frag(a.rhs + (int64_t)j * a.rhs_stride_bytes + tail_off, blk % kPerTile);
     }
     multiply(fa[0], fb[0]);
+    // (straight-line code whose results a row-major epilogue consumes under
+    // per-lane row conditions)
+    if constexpr (kSub == 2) {
+#pragma unroll
+      for (int x = 0; x < WM; ++x)
+#pragma unroll
+        for (int y = 0; y < WN; ++y) keep_result_in_all_lanes(acc[x][y]);
+    }
   }
 
   // Epilogue. Tiled result (instruction layout): with 32x32 blocks one store

@@ -176,6 +176,8 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
       __builtin_amdgcn_sched_barrier(0);
     }
     if constexpr (kPerWave) {
+      // (the stores below are divergent and the block's only consumer)
+      keep_result_in_all_lanes(acc);
       store_t* tile = (store_t*)a.out + (int64_t)j * a.out_stride_elems;
       const int mm = lane & 31;
       if (mm < a.M0) {

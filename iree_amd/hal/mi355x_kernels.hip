@@ -126,6 +126,9 @@ __device__ __forceinline__ void hal_matmul_packed_rhs(const void* lhs, const voi
   static_assert(TM % kPerTile == 0 && TN % kPerTile == 0, "macro tile of whole outer tiles");
   typedef typename Cfg::out_t out_t;
   if (M < 1 || N < 1 || K < Cfg::kMfmaK || K % Cfg::kMfmaK) return;
+  // The left-hand side is addressed with 32-bit byte offsets: a matrix of 2 GiB
+  // or more (the library's entry point refuses it as well) does nothing here.
+  if ((int64_t)M * K * Cfg::kElemBytes + 4096 > 0x7FFFFFFFll) return;
   MfmaArgs a;
   a.lhs = (const char*)lhs;
   a.rhs = (const char*)rhs;
@@ -158,6 +161,10 @@ __device__ __forceinline__ void hal_pack(const void* mat, void* tiled, int size0
                                          int tile0, int tile1, uint32_t padding) {
   constexpr int CE = 16 / ES;
   if (size0 < 1 || size1 < 1 || tile0 < 1 || tile1 < CE) return;
+  // power-of-two tiles whose rows are whole 16-byte chunks only (the geometry
+  // below is shifts); anything else does nothing
+  const int chunks = tile1 / CE;
+  if ((tile0 & (tile0 - 1)) || tile1 % CE || (chunks & (chunks - 1))) return;
   Pow2Args a;
   a.log2_tile_rows = __builtin_ctz((unsigned)tile0);
   const int cpr = tile1 / CE;

@@ -342,6 +342,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
     hal.return %x, %batch, %c1 : index, index, index
   }
   // out[M][N] (+)= lhs[M][K] * rhs (packed); push constants M, N, K (elements), K0, flags; workload (M, N)
+  // limits: M * K elements of lhs below 2 GiB, K a multiple of the matrix-core K extent (else nothing is written)
   hal.executable.export public @mi355x_matmul_packed_rhs_f16f16f32_t4x8 ordinal(20)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
         <0, bindings = [
@@ -359,6 +360,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
     hal.return %x, %c1, %c1 : index, index, index
   }
   // out[M][N] (+)= lhs[M][K] * rhs (packed); push constants M, N, K (elements), K0, flags; workload (M, N)
+  // limits: M * K elements of lhs below 2 GiB, K a multiple of the matrix-core K extent (else nothing is written)
   hal.executable.export public @mi355x_matmul_packed_rhs_f16f16f32_t8x8 ordinal(21)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
         <0, bindings = [
@@ -376,6 +378,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
     hal.return %x, %c1, %c1 : index, index, index
   }
   // out[M][N] (+)= lhs[M][K] * rhs (packed); push constants M, N, K (elements), K0, flags; workload (M, N)
+  // limits: M * K elements of lhs below 2 GiB, K a multiple of the matrix-core K extent (else nothing is written)
   hal.executable.export public @mi355x_matmul_packed_rhs_bf16bf16f32_t4x8 ordinal(22)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
         <0, bindings = [
@@ -393,6 +396,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
     hal.return %x, %c1, %c1 : index, index, index
   }
   // out[M][N] (+)= lhs[M][K] * rhs (packed); push constants M, N, K (elements), K0, flags; workload (M, N)
+  // limits: M * K elements of lhs below 2 GiB, K a multiple of the matrix-core K extent (else nothing is written)
   hal.executable.export public @mi355x_matmul_packed_rhs_bf16bf16f32_t8x8 ordinal(23)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
         <0, bindings = [
@@ -410,6 +414,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
     hal.return %x, %c1, %c1 : index, index, index
   }
   // out[M][N] (+)= lhs[M][K] * rhs (packed); push constants M, N, K (elements), K0, flags; workload (M, N)
+  // limits: M * K elements of lhs below 2 GiB, K a multiple of the matrix-core K extent (else nothing is written)
   hal.executable.export public @mi355x_matmul_packed_rhs_s8s8s32_t4x8 ordinal(24)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
         <0, bindings = [
@@ -427,6 +432,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
     hal.return %x, %c1, %c1 : index, index, index
   }
   // out[M][N] (+)= lhs[M][K] * rhs (packed); push constants M, N, K (elements), K0, flags; workload (M, N)
+  // limits: M * K elements of lhs below 2 GiB, K a multiple of the matrix-core K extent (else nothing is written)
   hal.executable.export public @mi355x_matmul_packed_rhs_s8s8s32_t8x8 ordinal(25)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
         <0, bindings = [
@@ -444,6 +450,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
     hal.return %x, %c1, %c1 : index, index, index
   }
   // out[M][N] (+)= lhs[M][K] * rhs (packed); push constants M, N, K (elements), K0, flags; workload (M, N)
+  // limits: M * K elements of lhs below 2 GiB, K a multiple of the matrix-core K extent (else nothing is written)
   hal.executable.export public @mi355x_matmul_packed_rhs_f8e4m3f8e4m3f32_t4x8 ordinal(26)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
         <0, bindings = [
@@ -461,6 +468,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
     hal.return %x, %c1, %c1 : index, index, index
   }
   // out[M][N] (+)= lhs[M][K] * rhs (packed); push constants M, N, K (elements), K0, flags; workload (M, N)
+  // limits: M * K elements of lhs below 2 GiB, K a multiple of the matrix-core K extent (else nothing is written)
   hal.executable.export public @mi355x_matmul_packed_rhs_f8e4m3f8e4m3f32_t8x8 ordinal(27)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
         <0, bindings = [
@@ -478,6 +486,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
     hal.return %x, %c1, %c1 : index, index, index
   }
   // out[M][N] (+)= lhs[M][K] * rhs (packed); push constants M, N, K (elements), K0, flags; workload (M, N)
+  // limits: M * K elements of lhs below 2 GiB, K a multiple of the matrix-core K extent (else nothing is written)
   hal.executable.export public @mi355x_matmul_packed_rhs_f32f32f32_t4x8 ordinal(28)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
         <0, bindings = [
@@ -495,6 +504,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
     hal.return %x, %c1, %c1 : index, index, index
   }
   // out[M][N] (+)= lhs[M][K] * rhs (packed); push constants M, N, K (elements), K0, flags; workload (M, N)
+  // limits: M * K elements of lhs below 2 GiB, K a multiple of the matrix-core K extent (else nothing is written)
   hal.executable.export public @mi355x_matmul_packed_rhs_f32f32f32_t8x8 ordinal(29)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
         <0, bindings = [
@@ -512,6 +522,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
     hal.return %x, %c1, %c1 : index, index, index
   }
   // pack: in = matrix, out = tiles; push constants size0, size1, tile0, tile1, padding; workload (size0, size1, tile0, tile1)
+  // limits: power-of-two tiles whose rows are whole 16-byte chunks, no transposes (else nothing is written)
   hal.executable.export public @mi355x_pack_8bit ordinal(30)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
         <0, bindings = [
@@ -538,6 +549,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
     hal.return %x, %c1, %c1 : index, index, index
   }
   // pack: in = matrix, out = tiles; push constants size0, size1, tile0, tile1, padding; workload (size0, size1, tile0, tile1)
+  // limits: power-of-two tiles whose rows are whole 16-byte chunks, no transposes (else nothing is written)
   hal.executable.export public @mi355x_pack_16bit ordinal(31)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
         <0, bindings = [
@@ -564,6 +576,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
     hal.return %x, %c1, %c1 : index, index, index
   }
   // pack: in = matrix, out = tiles; push constants size0, size1, tile0, tile1, padding; workload (size0, size1, tile0, tile1)
+  // limits: power-of-two tiles whose rows are whole 16-byte chunks, no transposes (else nothing is written)
   hal.executable.export public @mi355x_pack_32bit ordinal(32)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
         <0, bindings = [
@@ -590,6 +603,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
     hal.return %x, %c1, %c1 : index, index, index
   }
   // unpack: in = tiles, out = matrix; push constants size0, size1, tile0, tile1; workload (size0, size1, tile0, tile1)
+  // limits: power-of-two tiles whose rows are whole 16-byte chunks, no transposes (else nothing is written)
   hal.executable.export public @mi355x_unpack_16bit ordinal(33)
       layout(#hal.pipeline.layout<push_constants = 4, sets = [
         <0, bindings = [
@@ -612,6 +626,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
     hal.return %x, %c1, %c1 : index, index, index
   }
   // unpack: in = tiles, out = matrix; push constants size0, size1, tile0, tile1; workload (size0, size1, tile0, tile1)
+  // limits: power-of-two tiles whose rows are whole 16-byte chunks, no transposes (else nothing is written)
   hal.executable.export public @mi355x_unpack_32bit ordinal(34)
       layout(#hal.pipeline.layout<push_constants = 4, sets = [
         <0, bindings = [

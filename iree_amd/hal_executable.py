@@ -234,6 +234,7 @@ _MLIR_EXPORT = """\
 
 _MLIR_MATMUL_EXPORT = """\
   // out[M][N] (+)= lhs[M][K] * rhs (packed); push constants M, N, K (elements), K0, flags; workload (M, N)
+  // limits: M * K elements of lhs below 2 GiB, K a multiple of the matrix-core K extent (else nothing is written)
   hal.executable.export public @{name} ordinal({ordinal})
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
         <0, bindings = [
@@ -254,6 +255,7 @@ _MLIR_MATMUL_EXPORT = """\
 
 _MLIR_PACK_EXPORT = """\
   // {what}; push constants size0, size1, tile0, tile1{extra}; workload (size0, size1, tile0, tile1)
+  // limits: power-of-two tiles whose rows are whole 16-byte chunks, no transposes (else nothing is written)
   hal.executable.export public @{name} ordinal({ordinal})
       layout(#hal.pipeline.layout<push_constants = {constants}, sets = [
         <0, bindings = [

@@ -25,7 +25,7 @@
  *       numpy.float16 / bit-shift bf16, encode against numpy RNE.
  *   f8e4m3 conversions                 - the known answers of
  *       runtime/src/iree/base/internal/math_test.cc:420-525 (committed as data
- *       in tests/golden/f8e4m3_kat.json) and the closed form over all 256 codes.
+ *       in tests/golden/conversion_kat.json) and the closed form over all 256 codes.
  *   oracle_dequant_matmul_i4           - closed form in numpy float64; nibble
  *       order against tests/e2e/linalg/subbyte_to_fp.mlir's vectors.
  *   oracle_silu_mul                    - libm identity x*sigmoid(x)*u.
