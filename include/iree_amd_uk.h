@@ -177,6 +177,28 @@ IREE_AMD_UK_EXPORT int iree_amd_uk_mmt4d(
 IREE_AMD_UK_EXPORT int iree_amd_uk_mmt4d_p(
     const iree_amd_uk_mmt4d_params_t* params, void* stream);
 
+/* iree_amd_uk_mmt4d_p for callers that cannot allocate. It has no counterpart
+ * in the reference (whose ukernels never allocate, REF
+ * runtime/src/iree/builtins/ukernel/README.md:17-26); it is for callers that
+ * cannot call hipMalloc: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid it. Same parameters, kernels and results as
+ * iree_amd_uk_mmt4d_p, but the partial sums of a K split go to a device array
+ * of IREE_AMD_UK_NOALLOC_SCRATCH_BYTES that is part of the library's code
+ * object (every GPU the library runs on holds its own copy until the process
+ * ends) instead of the per-stream buffer iree_amd_uk_mmt4d_p allocates. The
+ * call makes no hipMalloc, hipFree or other allocating call. A call whose K
+ * split needs more than the array holds fails with status 8
+ * (RESOURCE_EXHAUSTED) and has launched nothing; iree_amd_uk_last_error says how
+ * many bytes it needed. Calls that do not split K (most) use no scratch at all.
+ * All calls on one GPU share that GPU's array and nothing in it needs to start
+ * at zero (every partial sum is written before it is read), but calls whose
+ * kernels overlap on one GPU - two streams, two host threads - race on it:
+ * keep them on one stream. The first call on a device looks up the array's
+ * address (hipGetSymbolAddress); make one call before starting a graph capture. */
+#define IREE_AMD_UK_NOALLOC_SCRATCH_BYTES (32u << 20)
+IREE_AMD_UK_EXPORT int iree_amd_uk_mmt4d_noalloc_p(
+    const iree_amd_uk_mmt4d_params_t* params, void* stream);
+
 /* linalg.batch_mmt4d: `batch` mmt4d problems of the shape `params` gives, entry
  * b on operands lying b * {lhs,rhs,out}_batch_stride elements after those of
  * entry 0 (offsets added to params->*_offset). Replaces the loop the reference

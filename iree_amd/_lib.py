@@ -79,6 +79,8 @@ def _declare(lib):
                                        i64, i64, i64, i32, i32, i32, u32, vp, vp]
     lib.iree_amd_uk_mmt4d_p.restype = C.c_int
     lib.iree_amd_uk_mmt4d_p.argtypes = [C.POINTER(Mmt4dParams), vp]
+    lib.iree_amd_uk_mmt4d_noalloc_p.restype = C.c_int
+    lib.iree_amd_uk_mmt4d_noalloc_p.argtypes = [C.POINTER(Mmt4dParams), vp]
     lib.iree_amd_uk_batch_mmt4d.restype = C.c_int
     lib.iree_amd_uk_batch_mmt4d.argtypes = [C.POINTER(Mmt4dParams), i64, i64, i64, i64, vp]
     lib.iree_amd_uk_mmt4d_info.restype = u32
