@@ -535,6 +535,17 @@ IREE_AMD_UK_EXPORT int iree_amd_uk_mfma_probe(uint32_t type_flag,
                                               int64_t* out_ops_per_launch,
                                               void* stream);
 
+/* NOT part of the reference interface either: the yardstick for the pack /
+ * unpack streams, a plain out-of-place copy of `bytes` (a multiple of 8 KiB,
+ * buffers 16-byte aligned and not overlapping) with 16-byte accesses, as the
+ * reference's benchmarks measure memcpy next to pack
+ * (REF runtime/src/iree/builtins/ukernel/tools/memcpy_benchmark.c:24-52).
+ * mode 0 = plain accesses, 1 = non-temporal ones; blocks_per_cu = workgroups
+ * per compute unit (0 = one workgroup per 8 KiB). */
+IREE_AMD_UK_EXPORT int iree_amd_uk_copy_probe(const void* src, void* dst,
+                                              iree_amd_uk_index_t bytes, int32_t mode,
+                                              int32_t blocks_per_cu, void* stream);
+
 /*===------------------------------------------------------------------------===
  * Thin device ABI, so that a pure-C host (the HAL executable plugin) needs no
  * HIP headers. Mirrors the handful of driver calls the reference's own HIP HAL

@@ -69,7 +69,9 @@ class QueryOutParams(C.Structure):
 
 
 def library_path():
-    return os.path.join(_HERE, "csrc", _LIB_NAME)
+    """The built library; IREE_AMD_UK_LIBRARY (the variable the HAL plugin reads
+    as well) names another build of it."""
+    return os.environ.get("IREE_AMD_UK_LIBRARY") or os.path.join(_HERE, "csrc", _LIB_NAME)
 
 
 def _declare(lib):
@@ -125,6 +127,8 @@ def _declare(lib):
     lib.iree_amd_uk_scale_f32.argtypes = [vp, i64, C.c_float, vp]
     lib.iree_amd_uk_mfma_probe.restype = C.c_int
     lib.iree_amd_uk_mfma_probe.argtypes = [C.c_uint32, vp, i64, vp, C.POINTER(C.c_int64), vp]
+    lib.iree_amd_uk_copy_probe.restype = C.c_int
+    lib.iree_amd_uk_copy_probe.argtypes = [vp, vp, i64, i32, i32, vp]
     lib.iree_amd_uk_device_count.restype = C.c_int
     lib.iree_amd_uk_device_count.argtypes = [C.POINTER(C.c_int)]
     lib.iree_amd_uk_device_set.restype = C.c_int

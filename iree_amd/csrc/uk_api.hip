@@ -631,6 +631,12 @@ extern "C" int iree_amd_uk_mfma_probe(uint32_t type_flag, const void* operands,
                            (hipStream_t)stream);
 }
 
+extern "C" int iree_amd_uk_copy_probe(const void* src, void* dst, iree_amd_uk_index_t bytes, int32_t mode,
+                                      int32_t blocks_per_cu, void* stream) {
+  if (!src || !dst) return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "copy_probe: null buffer");
+  return launch_copy_probe(src, dst, bytes, mode, blocks_per_cu, (hipStream_t)stream);
+}
+
 //===----------------------------------------------------------------------===//
 // Thin device ABI
 //===----------------------------------------------------------------------===//

@@ -156,6 +156,8 @@ int launch_scale_f32(void* buf, int64_t n, float scale, hipStream_t s);
 int launch_mfma_probe(uint32_t type_flag, const void* operands, int64_t iters, void* sink,
                       int64_t* out_ops_per_launch, hipStream_t s);
 
+int launch_copy_probe(const void* src, void* dst, int64_t bytes, int mode, int blocks_per_cu, hipStream_t s);
+
 // Number of compute units of the current device (cached per device).
 int device_cu_count();
 

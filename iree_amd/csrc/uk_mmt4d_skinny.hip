@@ -121,8 +121,9 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
     const int s = sp < count ? sp : 0;
     const int jj = j < a.N ? j : a.N - 1;
     const char* p = rhs_lane + (int64_t)jj * a.rhs_stride_bytes + (int64_t)s * kBlock;
-    const int4v lo = *(const int4v*)p;
-    const int4v hi = kSub == 2 ? *(const int4v*)(p + 512) : lo;
+    // (non-temporal: the right-hand side is read once)
+    const int4v lo = __builtin_nontemporal_load((const int4v*)p);
+    const int4v hi = kSub == 2 ? __builtin_nontemporal_load((const int4v*)(p + 512)) : lo;
     return make_frag(lo, hi);
   };
   // (the zeroing happens when a block is consumed, not when it is requested:

@@ -47,7 +47,16 @@ struct Pow2Args {
   uint64_t padding;
 };
 
-template <int ES, bool kPack>
+// Non-temporal accesses on the TILED side only (measured on MI355X, f16
+// 8191 x 5001 <-> 32x16 tiles): its pieces are whole 256-byte runs that nobody
+// else touches, and streaming them past the caches gives pack 5.25 instead of
+// 4.95 TB/s and unpack 4.76 instead of 4.69. On the matrix side they lose:
+// its 128-byte row segments share cache lines with the neighbouring waves
+// (non-temporal loads: pack 4.5 TB/s) and are pieces of DRAM pages that
+// non-temporal stores no longer merge (unpack 3.0 TB/s). A plain copy with
+// 8 KiB runs on both sides reaches 5.3-5.5 TB/s with ordinary and 6.0-6.2 with
+// non-temporal accesses on the same machine.
+template <int ES, bool kPack, bool kNtLoad = !kPack, bool kNtStore = kPack>
 __device__ __forceinline__ void stream_pow2_body(const Pow2Args a) {
   constexpr int CE = 16 / ES;
   constexpr int kRows = kBlockRows * kStreamUnroll;
@@ -95,12 +104,24 @@ __device__ __forceinline__ void stream_pow2_body(const Pow2Args a) {
   if (interior) {
     u32x4 v[kStreamUnroll];
 #pragma unroll
-    for (int u = 0; u < kStreamUnroll; ++u)
-      v[u] = kPack ? *(const mat_vec_t*)(mat_base + mat_off[u]) : *(const u32x4*)(tiled_base + tiled_off[u]);
+    for (int u = 0; u < kStreamUnroll; ++u) {
+      if (kPack) {
+        const mat_vec_t* p = (const mat_vec_t*)(mat_base + mat_off[u]);
+        v[u] = kNtLoad ? __builtin_nontemporal_load(p) : *p;
+      } else {
+        const u32x4* p = (const u32x4*)(tiled_base + tiled_off[u]);
+        v[u] = kNtLoad ? __builtin_nontemporal_load(p) : *p;
+      }
+    }
 #pragma unroll
     for (int u = 0; u < kStreamUnroll; ++u) {
-      if (kPack) *(u32x4*)(tiled_base + tiled_off[u]) = v[u];
-      else *(mat_vec_t*)((char*)mat_base + mat_off[u]) = v[u];
+      if (kPack) {
+        u32x4* p = (u32x4*)(tiled_base + tiled_off[u]);
+        if (kNtStore) __builtin_nontemporal_store(v[u], p); else *p = v[u];
+      } else {
+        mat_vec_t* p = (mat_vec_t*)((char*)mat_base + mat_off[u]);
+        if (kNtStore) __builtin_nontemporal_store((mat_vec_t)v[u], p); else *p = v[u];
+      }
     }
     return;
   }

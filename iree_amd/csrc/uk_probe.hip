@@ -12,6 +12,8 @@
 namespace uk {
 namespace {
 
+typedef uint32_t u32x4p __attribute__((ext_vector_type(4)));
+
 template <typename Cfg>
 __global__ __launch_bounds__(256) void mfma_probe_kernel(const char* operands, int64_t iters, float* sink) {
   typedef typename Cfg::frag_t frag_t;
@@ -51,6 +53,29 @@ __global__ __launch_bounds__(256) void mfma_probe_kernel(const char* operands, i
   if (s == 12345.678f) sink[threadIdx.x] = s;
 }
 
+// Second measurement aid: a plain out-of-place copy, the yardstick for the pack
+// / unpack streams (what the reference's own benchmarks do with memcpy,
+// runtime/src/iree/builtins/ukernel/tools/memcpy_benchmark.c:24-52). Every lane
+// moves 16 bytes per access; a wave keeps kCopyUnroll accesses of 1 KiB in
+// flight; workgroups walk contiguous chunks, XCD by XCD, like the pack kernel.
+constexpr int kCopyUnroll = 2;
+template <bool kNonTemporal>
+__global__ __launch_bounds__(256) void copy_probe_kernel(const u32x4p* src, u32x4p* dst, int64_t chunks) {
+  // chunk = kCopyUnroll * 256 lanes * 16 bytes
+  for (int64_t c = blockIdx.x; c < chunks; c += gridDim.x) {
+    const int64_t base = c * (kCopyUnroll * 256) + threadIdx.x;
+    u32x4p v[kCopyUnroll];
+#pragma unroll
+    for (int u = 0; u < kCopyUnroll; ++u)
+      v[u] = kNonTemporal ? __builtin_nontemporal_load(src + base + u * 256) : src[base + u * 256];
+#pragma unroll
+    for (int u = 0; u < kCopyUnroll; ++u) {
+      if (kNonTemporal) __builtin_nontemporal_store(v[u], dst + base + u * 256);
+      else dst[base + u * 256] = v[u];
+    }
+  }
+}
+
 template <typename Cfg>
 int launch(const void* operands, int64_t iters, void* sink, int blocks, hipStream_t s) {
   hipLaunchKernelGGL((mfma_probe_kernel<Cfg>), dim3(blocks), dim3(256), 0, s, (const char*)operands,
@@ -77,6 +102,24 @@ int launch_mfma_probe(uint32_t type_flag, const void* operands, int64_t iters, v
   // per wave and iteration: a 128 x 128 x k update
   if (out_ops_per_launch) *out_ops_per_launch = (int64_t)blocks * 4 * iters * 2 * 128 * 128 * k;
   return st;
+}
+
+// bytes: a multiple of 8 KiB; mode 0 = plain accesses, 1 = non-temporal;
+// blocks_per_cu workgroups per compute unit (0 = one workgroup per chunk).
+int launch_copy_probe(const void* src, void* dst, int64_t bytes, int mode, int blocks_per_cu, hipStream_t s) {
+  const int64_t chunk_bytes = (int64_t)kCopyUnroll * 256 * 16;
+  if (bytes <= 0 || bytes % chunk_bytes || ((uintptr_t)src | (uintptr_t)dst) % 16)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "copy_probe: bytes must be whole chunks of %lld and buffers 16-byte aligned",
+                (long long)chunk_bytes);
+  const int64_t chunks = bytes / chunk_bytes;
+  int64_t blocks = blocks_per_cu > 0 ? (int64_t)device_cu_count() * blocks_per_cu : chunks;
+  if (blocks > chunks) blocks = chunks;
+  if (blocks > 0x7FFFFFFF) blocks = 0x7FFFFFFF;
+  if (mode == 1)
+    hipLaunchKernelGGL(copy_probe_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, s, (const u32x4p*)src, (u32x4p*)dst, chunks);
+  else
+    hipLaunchKernelGGL(copy_probe_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, s, (const u32x4p*)src, (u32x4p*)dst, chunks);
+  return check_hip(hipGetLastError(), "copy_probe launch");
 }
 
 }  // namespace uk

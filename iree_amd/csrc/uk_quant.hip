@@ -98,7 +98,8 @@ __global__ __launch_bounds__(kThreads) void dequant_matmul_i4_kernel(I4Args a) {
     return __builtin_amdgcn_make_buffer_rsrc((void*)(a.w + off), 0, left, 0x00020000);
   };
   auto load_slab = [&](__amdgpu_buffer_rsrc_t rsrc, int sp, int h) -> u32x4 {
-    return __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, soff_wave + sp * a.span_stride + h * half_stride, 0);
+    // (non-temporal: the weights are read once; measured 9.2 -> 8.8 us at one row)
+    return __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, soff_wave + sp * a.span_stride + h * half_stride, 2);
   };
 
   // ---- request the first tile's parameters, then x and the weights span by

@@ -122,7 +122,7 @@ __global__ __launch_bounds__(kThreads) void dequant_gemv_i4_kernel(GemvArgs a) {
   // (the whole offset goes into the vector operand: that is the part the
   // hardware's range check is documented to cover)
   auto load_slab = [&](__amdgpu_buffer_rsrc_t rsrc, int span) -> u32x4 {
-    return __builtin_amdgcn_raw_buffer_load_b128(rsrc, w_voff + (uint32_t)span * span_stride, 0, 0);
+    return __builtin_amdgcn_raw_buffer_load_b128(rsrc, w_voff + (uint32_t)span * span_stride, 0, 2);   // (non-temporal: read once)
   };
   const __amdgpu_buffer_rsrc_t scale_rsrc =
       __builtin_amdgcn_make_buffer_rsrc((void*)a.scale, 0, a.scale_bytes, 0x00020000);
