@@ -60,8 +60,10 @@ def parse_args():
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary measurements")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--only", default="", help="run only the named kernel in a loop (for profilers): "
-                    "mmt4d_f16 | mmt4d_i8 | mmt4d_fp8 | mmt4d_f16_ksplit | mlp_fp8 | pack | unpack | "
-                    "dequant_i4 | batch_mmt4d_f16 | batch_mmt4d_f16_narrow | copy")
+                    "mmt4d_f16 | mmt4d_f16_acc | mmt4d_i8 | mmt4d_fp8 | mmt4d_f16_ksplit | mlp_fp8 | pack | unpack | "
+                    "pack_transpose | dequant_i4[_m8|_m32] | dequant_i4_reassoc[_m8|_m32] | batch_mmt4d_f16 | "
+                    "batch_mmt4d_f16_narrow | mmt4d_f16_narrow_m1 | mmt4d_f16_narrow_m8 | mmt4d_f16_narrow_n8 | "
+                    "chain_i8_1024 | copy | copy_rotating | copy_rotating_nt")
     return ap.parse_args()
 
 
@@ -219,7 +221,9 @@ def main():
                    "tile": [M0, N0, K0], "accumulate": False},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_F16_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(achieved / PEAK_F16_TFLOPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES["mmt4d_f16_4096"]},
+                     "traffic": MEASURED_TRAFFIC_BYTES["mmt4d_f16_4096"],
+                     "traffic_source": "profiles/mmt4d_f16_4096x4096x4096.txt (rocprofv3 --pmc FETCH_SIZE / "
+                                       "WRITE_SIZE of this command, committed; not re-measured in this run)"},
     }
     # The headline line must not be lost to a failure in a secondary
     # measurement: what was measured up to there is kept, the error is reported
@@ -257,6 +261,21 @@ def verify_tiles(torch, iree_amd, F, lhs, rhs, out, M1, N1, K1, M0, N0, K0):
         got = out[(i * N1 + j) * M0 * N0:(i * N1 + j + 1) * M0 * N0].cpu().numpy()
         if not np.all(np.abs(got - want) <= 1e-3 + 1e-2 * np.abs(want)):
             raise SystemExit("bench.py: mmt4d result is outside tolerance; refusing to time it")
+
+
+def make_copy_rotating(torch, iree_amd, mode):
+    """(fn, bytes per copy): out-of-place copies of 81.9 MB (about what pack
+    moves each way), rotating over four buffer pairs."""
+    nb, nrot = 81920000, 4
+    srcs = [torch.full((nb,), 3 + i, dtype=torch.uint8, device="cuda") for i in range(nrot)]
+    dsts = [torch.empty(nb, dtype=torch.uint8, device="cuda") for _ in range(nrot)]
+    st = {"i": 0}
+
+    def fn():
+        k = st["i"] % nrot
+        st["i"] += 1
+        iree_amd.copy_probe(srcs[k], dsts[k], nb, mode, 32)
+    return fn, nb
 
 
 def make_fp8_mlp(torch, iree_amd):
@@ -316,9 +335,11 @@ def extras(args, torch, iree_amd, F, synth, lhs, rhs, out, ex):
         ex[f"mfma_register_only_{name}_tops"] = round(n_ops / t / 1e12, 1)
     del sink, zeros, rnd8
 
-    # The same mmt4d through the host-pointer entry point the HAL plugin calls
-    # (pageable host buffers: 64 MiB staged in, 64 MiB staged out, per-call
-    # device allocation, synchronous): the PCIe-inclusive rate, never `value`.
+    # The same mmt4d through the host-pointer entry points (pageable host
+    # buffers: 64 MiB staged in, 64 MiB staged out, synchronous): the
+    # PCIe-inclusive rate, never `value`. First the form the HAL plugin calls,
+    # which stages through a pool its instance owns (stream and device buffers
+    # kept between calls), then the form that builds everything per call.
     import ctypes as C
     from iree_amd._lib import Mmt4dParams
     lh, rh = lhs.cpu().numpy(), rhs.cpu().numpy()
@@ -326,11 +347,21 @@ def extras(args, torch, iree_amd, F, synth, lhs, rhs, out, ex):
     hp = Mmt4dParams(lh.ctypes.data, 0, size * 32, rh.ctypes.data, 0, size * 32, oh.ctypes.data, 0,
                      N1 * 1024, M1, N1, size // 8, 32, 32, 8, F.MMT4D_TYPE_F16F16F32, None)
     lib = iree_amd.load_library()
+    pool = C.c_void_p()
+    assert lib.iree_amd_uk_host_pool_create(C.byref(pool)) == 0
+    assert lib.iree_amd_uk_mmt4d_host_pooled(pool, C.byref(hp)) == 0
+    t0 = time.perf_counter()
+    for _ in range(5):
+        assert lib.iree_amd_uk_mmt4d_host_pooled(pool, C.byref(hp)) == 0
+    ex["mmt4d_f16_host_pointers_tflops"] = round(flops / ((time.perf_counter() - t0) / 5) / 1e12, 2)
+    assert np.array_equal(oh, out.cpu().numpy()), "host-pointer mmt4d differs from the device entry point"
+    lib.iree_amd_uk_host_pool_destroy(pool)
+    oh[:] = 0
     assert lib.iree_amd_uk_mmt4d_host(C.byref(hp)) == 0
     t0 = time.perf_counter()
     for _ in range(3):
         assert lib.iree_amd_uk_mmt4d_host(C.byref(hp)) == 0
-    ex["mmt4d_f16_host_pointers_tflops"] = round(flops / ((time.perf_counter() - t0) / 3) / 1e12, 2)
+    ex["mmt4d_f16_host_pointers_per_call_resources_tflops"] = round(flops / ((time.perf_counter() - t0) / 3) / 1e12, 2)
     assert np.array_equal(oh, out.cpu().numpy()), "host-pointer mmt4d differs from the device entry point"
     del lh, rh, oh
 
@@ -459,6 +490,15 @@ def extras(args, torch, iree_amd, F, synth, lhs, rhs, out, ex):
     torch.cuda.synchronize()
     assert np.array_equal(xs[0].cpu().numpy(), x_host), "pack/unpack round trip is not bit-exact"
     del xs, ps
+    # The yardstick for these streams (the reference benchmarks memcpy next to
+    # pack): a plain out-of-place copy of the same size, four rotating buffer
+    # pairs (656 MB), with ordinary and with non-temporal accesses.
+    for mode, name in ((0, "copy_rotating"), (1, "copy_rotating_nontemporal")):
+        fn, nb = make_copy_rotating(torch, iree_amd, mode)
+        _, t = gpu_time(torch, fn, steps, warm)
+        ex[f"{name}_gbs"] = round(2 * nb / t / 1e9, 1)
+    ex["pack_frac_of_copy_yardstick"] = round(ex["pack_f16_8191x5001_gbs"] / ex["copy_rotating_nontemporal_gbs"], 4)
+    ex["unpack_frac_of_copy_yardstick"] = round(ex["unpack_f16_8191x5001_gbs"] / ex["copy_rotating_nontemporal_gbs"], 4)
 
     # whole chain on row-major operands: pack LHS, pack RHS (transposing), mmt4d, unpack
     a = torch.from_numpy(synth.normal_f16(1, size * size, 1 / 64).view(np.int16)).cuda().view(torch.float16)
@@ -531,7 +571,22 @@ def extras(args, torch, iree_amd, F, synth, lhs, rhs, out, ex):
         _, t = gpu_time(torch, do_q, steps, warm)
         ex[f"dequant_matmul_i4_m{Mq}_gbs"] = round(qbytes / t / 1e9, 1)
         ex[f"dequant_matmul_i4_m{Mq}_us"] = round(t * 1e6, 2)
-    ex["dequant_matmul_i4_m1_frac_of_hbm_peak"] = round(ex["dequant_matmul_i4_m1_gbs"] / PEAK_HBM_GBS, 4)
+        ex[f"dequant_matmul_i4_m{Mq}_frac_of_hbm_peak"] = round(qbytes / t / 1e9 / PEAK_HBM_GBS, 4)
+        # the reassociated form (16-bit activations, integer products): the
+        # quantisation kernel and the matmul, two launches
+        oq2 = torch.empty_like(oq)
+
+        def do_qr():
+            k = state["i"] % nrot
+            state["i"] += 1
+            iree_amd.dequant_matmul_i4(xq, wq[k], sq, zq, oq2, Mq, Nq, Kq, gs, qflags | F.DEQUANT_MATMUL_REASSOCIATE)
+
+        _, t = gpu_time(torch, do_qr, steps, warm)
+        ex[f"dequant_matmul_i4_reassociated_m{Mq}_us"] = round(t * 1e6, 2)
+        ex[f"dequant_matmul_i4_reassociated_m{Mq}_gbs"] = round(qbytes / t / 1e9, 1)
+        a16, b16 = oq.view(torch.float16).float(), oq2.view(torch.float16).float()
+        # (the rewrite loses precision by design: twice the absolute part of the stated bound)
+        assert bool(((a16 - b16).abs() <= 2e-3 + 1e-2 * a16.abs()).all()), "reassociated int4 result out of tolerance"
     # the transposed shape (N 4096, K 14336, the same byte counts and buffers):
     # a K the register-resident kernel cannot take; the activations go through
     # LDS, 1 row in one pass, 8 rows in two passes over the weights
@@ -567,6 +622,20 @@ def extras(args, torch, iree_amd, F, synth, lhs, rhs, out, ex):
         _, t = gpu_time(torch, do_n, steps, warm)
         ex[f"mmt4d_f16_narrow_m{M0}_gbs"] = round((Nn * Kn * 2 + M0 * Kn * 2 + M0 * Nn * 4) / t / 1e9, 1)
     ex["mmt4d_f16_narrow_m1_frac_of_hbm_peak"] = round(ex["mmt4d_f16_narrow_m1_gbs"] / PEAK_HBM_GBS, 4)
+    # the same problem as a narrow RESULT: 14336 rows x 8 columns (32 x 8 result
+    # tiles, the wide operand on the left), which the library runs with the
+    # operands exchanged and the tiles stored transposed
+    ln = torch.from_numpy(synth.normal_f16(60, 8 * Kn).view(np.int16)).cuda()
+    on = torch.empty(8 * Nn, dtype=torch.float32, device="cuda")
+    state["i"] = 0
+
+    def do_nn():
+        k = state["i"] % 6
+        state["i"] += 1
+        iree_amd.mmt4d(rn[k], ln, on, Nn // 32, 1, Kn // 8, 32, 8, 8, F.MMT4D_TYPE_F16F16F32)
+
+    _, t = gpu_time(torch, do_nn, steps, warm)
+    ex["mmt4d_f16_narrow_n8_gbs"] = round((Nn * Kn * 2 + 8 * Kn * 2 + 8 * Nn * 4) / t / 1e9, 1)
     # the transposed shape (N 4096, K 14336: a K longer than one launch keeps in
     # registers, run as four accumulating launches over K slices), same buffers
     ll = torch.from_numpy(synth.normal_f16(61, 8 * Nn).view(np.int16)).cuda()
@@ -654,21 +723,70 @@ def run_only(args, torch, iree_amd, F, synth, mm_step):
         iree_amd.quantize_f16_to_f8e4m3(src.flip(0), r8, size * size, 0.5)
         o8 = torch.empty(M1 * N1 * 1024, dtype=torch.float32, device="cuda")
         fn = lambda: iree_amd.mmt4d(l8, r8, o8, M1, N1, K1, 32, 32, 16, F.MMT4D_TYPE_F8E4M3F8E4M3F32)  # noqa: E731
-    elif args.only == "dequant_i4":
+    elif args.only.startswith("dequant_i4"):
         Nq, Kq, gs = 14336, 4096, 128
         G = Kq // gs
+        Mq = 32 if args.only.endswith("_m32") else 8 if args.only.endswith("_m8") else 1
+        qflags = F.DEQUANT_MATMUL_ZP_U4 | F.DEQUANT_MATMUL_W_TILED
+        if "reassoc" in args.only:
+            qflags |= F.DEQUANT_MATMUL_REASSOCIATE
         wq = [torch.from_numpy(synth.uniform_u4_packed(10 + i, Nq * Kq)).cuda() for i in range(10)]
         sq = torch.from_numpy(synth.uniform_f16(30, Nq * G, 0.005, 0.02).view(np.int16)).cuda()
         zq = torch.from_numpy(synth.uniform_u4_packed(31, Nq * G)).cuda()
-        xq = torch.from_numpy(synth.normal_f16(41, Kq).view(np.int16)).cuda()
-        oq = torch.empty(Nq, dtype=torch.int16, device="cuda")
+        xq = torch.from_numpy(synth.normal_f16(40 + Mq, Mq * Kq).view(np.int16)).cuda()
+        oq = torch.empty(Mq * Nq, dtype=torch.int16, device="cuda")
         st = {"i": 0}
 
         def fn():
             k = st["i"] % 10
             st["i"] += 1
-            iree_amd.dequant_matmul_i4(xq, wq[k], sq, zq, oq, 1, Nq, Kq, gs,
-                                       F.DEQUANT_MATMUL_ZP_U4 | F.DEQUANT_MATMUL_W_TILED)
+            iree_amd.dequant_matmul_i4(xq, wq[k], sq, zq, oq, Mq, Nq, Kq, gs, qflags)
+    elif args.only in ("copy_rotating", "copy_rotating_nt"):
+        fn, _ = make_copy_rotating(torch, iree_amd, 1 if args.only.endswith("_nt") else 0)
+    elif args.only == "mmt4d_f16_acc":
+        size = 4096
+        lhs, rhs = packed_operands_f16(torch, synth, size // 32, size // 32, size // 8, 32, 32, 8, size)
+        oa = torch.zeros(size * size, dtype=torch.float32, device="cuda")
+        fn = lambda: iree_amd.mmt4d(lhs, rhs, oa, size // 32, size // 32, size // 8, 32, 32, 8,  # noqa: E731
+                                    F.MMT4D_TYPE_F16F16F32 | F.MMT4D_ACCUMULATE)
+    elif args.only in ("mmt4d_f16_narrow_m1", "mmt4d_f16_narrow_m8", "mmt4d_f16_narrow_n8"):
+        # one outer row of M0 x 8 tiles against N 14336, K 4096 (six rotating
+        # right-hand sides, 705 MB); _n8: the same problem as a narrow RESULT
+        # (32 x 8 tiles, the wide operand on the left), which runs exchanged
+        Nn, Kn = 14336, 4096
+        m0 = 1 if args.only.endswith("_m1") else 8
+        rn = [torch.from_numpy(synth.normal_f16(50 + i, Nn * Kn, 1 / 64).view(np.int16)).cuda() for i in range(6)]
+        ln = torch.from_numpy(synth.normal_f16(60, m0 * Kn).view(np.int16)).cuda()
+        on = torch.empty(m0 * Nn, dtype=torch.float32, device="cuda")
+        st = {"i": 0}
+
+        def fn():
+            k = st["i"] % 6
+            st["i"] += 1
+            if args.only.endswith("_n8"):
+                iree_amd.mmt4d(rn[k], ln, on, Nn // 32, 1, Kn // 8, 32, 8, 8, F.MMT4D_TYPE_F16F16F32)
+            else:
+                iree_amd.mmt4d(ln, rn[k], on, 1, Nn // 32, Kn // 8, m0, 32, 8, F.MMT4D_TYPE_F16F16F32)
+    elif args.only == "chain_i8_1024":
+        n1k = 1024
+        a8 = torch.from_numpy(synth.uniform_int8(1, n1k * n1k)).cuda()
+        b8 = torch.from_numpy(synth.uniform_int8(2, n1k * n1k)).cuda()
+        c8 = torch.zeros(n1k * n1k, dtype=torch.int32, device="cuda")
+        ws8 = iree_amd.matmul_data_tiled(a8, b8, c8, n1k, n1k, n1k, F.MMT4D_TYPE_S8S8S32)
+        fn = lambda: iree_amd.matmul_data_tiled(a8, b8, c8, n1k, n1k, n1k, F.MMT4D_TYPE_S8S8S32,  # noqa: E731
+                                                workspace=ws8)
+    elif args.only == "pack_transpose":
+        # the right-hand side of the 4096^3 f16 matmul given as B[K][N]: 32x8 tiles, inner and outer transposed
+        size = 4096
+        b = torch.from_numpy(synth.normal_f16(2, size * size, 1 / 64).view(np.int16)).cuda()
+        pb = [torch.empty(size * size, dtype=torch.int16, device="cuda") for _ in range(4)]
+        st = {"i": 0}
+
+        def fn():
+            k = st["i"] % 4
+            st["i"] += 1
+            iree_amd.pack(b, pb[k], size, size, size // 32, size // 8, 32, 8, 0,
+                          F.PACK_TYPE_F16F16 | F.PACK_TRANSPOSE_INNER | F.PACK_TRANSPOSE_OUTER)
     elif args.only == "mlp_fp8":
         mlp, xm, ym, Mt, _, _ = make_fp8_mlp(torch, iree_amd)
         fn = lambda: mlp(xm, ym, Mt)  # noqa: E731

@@ -384,12 +384,34 @@ IREE_AMD_UK_EXPORT int iree_amd_uk_query_tile_sizes_2d(
  * Needs N % 32 == 0 and K % 128 == 0. Without the flag the weights are
  * row-major [N][K/2]; groups smaller than 128 are fast only from tiled weights. */
 #define IREE_AMD_UK_FLAG_DEQUANT_MATMUL_W_TILED 0x2
+/* The reassociated form, opt-in as in the reference ("introduces precision
+ * loss", REF compiler/src/iree/compiler/GlobalOptimization/FuseDequantizationMatmul.cpp:746-767;
+ * rewrite :398-645): the activations are quantised per group to 16 bits
+ * (scale_x = max |x| / 32767, q = fptosi(x / scale_x)), the products are
+ * integer (i16 x u4 -> i32 per group: the reference's S16U4S32 mmt4d,
+ * REF runtime/src/iree/builtins/ukernel/arch/x86_64/mmt4d_x86_64_avx512_vnni.c:210-294)
+ * and out = sum_g float(acc) * scale_x * s - (zp * s) * sum_k x, all float steps
+ * in f32, rounded to f16 once. The quantised activations live in the stream's
+ * scratch buffer (see iree_amd_uk_mmt4d). On the matrix cores from tiled
+ * weights with K = 2048 or 4096 and power-of-two groups of 128 to K / 8;
+ * everything else runs an element-wise kernel. */
+#define IREE_AMD_UK_FLAG_DEQUANT_MATMUL_REASSOCIATE 0x4
 
 IREE_AMD_UK_EXPORT int iree_amd_uk_dequant_matmul_i4(
     const void* x_buffer, const void* w_buffer, const void* scale_buffer,
     const void* zp_buffer, void* out_buffer, iree_amd_uk_index_t M,
     iree_amd_uk_index_t N, iree_amd_uk_index_t K,
     iree_amd_uk_index_t group_size, uint32_t flags, void* stream);
+
+/* The quantisation step of the reassociated form by itself (the first three
+ * dispatches of the rewrite, REF FuseDequantizationMatmul.cpp:398-492):
+ * x f16 [M][K] -> q i16 [M][K], scale_x f32 [M][K/gs] = max |x| / 32767 per
+ * group, group_sum f32 [M][K/gs] (lane-strided partial sums combined by a
+ * butterfly; the reference adds in k order). A group of zeros gives zeros. */
+IREE_AMD_UK_EXPORT int iree_amd_uk_quantize_groups_i16(
+    const void* x_f16, void* q_i16, void* scale_x_f32, void* group_sum_f32,
+    iree_amd_uk_index_t M, iree_amd_uk_index_t K, iree_amd_uk_index_t group_size,
+    void* stream);
 
 /* Row-major [N][K/2] 4-bit weights -> the ..._W_TILED layout above (done once
  * per weight matrix, like the reference's pack of a constant right-hand side

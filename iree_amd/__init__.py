@@ -15,6 +15,7 @@ from .ukernel import (  # noqa: F401
     matmul_data_tiled,
     matmul_packed_rhs,
     mfma_probe,
+    quantize_groups_i16,
     copy_probe,
     batch_mmt4d,
     mmt4d,

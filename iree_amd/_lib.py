@@ -103,6 +103,8 @@ def _declare(lib):
     lib.iree_amd_uk_dequant_matmul_i4.restype = C.c_int
     lib.iree_amd_uk_dequant_matmul_i4.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64,
                                                    i64, u32, vp]
+    lib.iree_amd_uk_quantize_groups_i16.restype = C.c_int
+    lib.iree_amd_uk_quantize_groups_i16.argtypes = [vp, vp, vp, vp, i64, i64, i64, vp]
     lib.iree_amd_uk_pack_i4_weights.restype = C.c_int
     lib.iree_amd_uk_pack_i4_weights.argtypes = [vp, vp, i64, i64, vp]
     lib.iree_amd_uk_quantize_f16_to_f8e4m3.restype = C.c_int

@@ -415,7 +415,7 @@ extern "C" int iree_amd_uk_dequant_matmul_i4(
     const void* zp_buffer, void* out_buffer, iree_amd_uk_index_t M,
     iree_amd_uk_index_t N, iree_amd_uk_index_t K,
     iree_amd_uk_index_t group_size, uint32_t flags, void* stream) {
-  if (flags & ~3u) return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "dequant_matmul_i4: unknown flag bits");
+  if (flags & ~7u) return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "dequant_matmul_i4: unknown flag bits");
   if (M < 0 || N < 0 || K < 0 || group_size <= 0)
     return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "dequant_matmul_i4: bad sizes");
   if (K % group_size || group_size % 32)
@@ -424,9 +424,26 @@ extern "C" int iree_amd_uk_dequant_matmul_i4(
   if (M == 0 || N == 0) return 0;
   if (!x_buffer || !w_buffer || !scale_buffer || !zp_buffer || !out_buffer)
     return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "dequant_matmul_i4: null buffer");
+  if (flags & IREE_AMD_UK_FLAG_DEQUANT_MATMUL_REASSOCIATE)
+    return launch_dequant_matmul_i4_reassoc(x_buffer, w_buffer, scale_buffer, zp_buffer,
+                                            out_buffer, M, N, K, group_size, flags,
+                                            (hipStream_t)stream);
   return launch_dequant_matmul_i4(x_buffer, w_buffer, scale_buffer, zp_buffer,
                                   out_buffer, M, N, K, group_size, flags,
                                   (hipStream_t)stream);
+}
+
+extern "C" int iree_amd_uk_quantize_groups_i16(const void* x_f16, void* q_i16, void* scale_x_f32,
+                                               void* group_sum_f32, iree_amd_uk_index_t M,
+                                               iree_amd_uk_index_t K, iree_amd_uk_index_t group_size,
+                                               void* stream) {
+  if (M < 0 || K < 0 || group_size <= 0 || K % group_size)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "quantize_groups_i16: need K %% group_size == 0");
+  if (M == 0 || K == 0) return 0;
+  if (!x_f16 || !q_i16 || !scale_x_f32 || !group_sum_f32)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "quantize_groups_i16: null buffer");
+  return launch_quantize_groups_i16(x_f16, q_i16, scale_x_f32, group_sum_f32, M, K, group_size,
+                                    (hipStream_t)stream);
 }
 
 extern "C" int iree_amd_uk_pack_i4_weights(const void* w_rowmajor, void* w_tiled,

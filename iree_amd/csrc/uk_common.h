@@ -141,6 +141,12 @@ int launch_dequant_matmul_i4(const void* x, const void* w, const void* scale,
                              const void* zp, void* out, int64_t M, int64_t N,
                              int64_t K, int64_t group_size, uint32_t flags,
                              hipStream_t s);
+int launch_dequant_matmul_i4_reassoc(const void* x, const void* w, const void* scale,
+                                     const void* zp, void* out, int64_t M, int64_t N,
+                                     int64_t K, int64_t group_size, uint32_t flags,
+                                     hipStream_t s);
+int launch_quantize_groups_i16(const void* x, void* q, void* scale_x, void* group_sum, int64_t M,
+                               int64_t K, int64_t gs, hipStream_t s);
 int launch_pack_i4_weights(const void* src, void* dst, int64_t N, int64_t K, hipStream_t s);
 int launch_quantize_f16_to_f8e4m3(const void* in, void* out, int64_t n,
                                   float inv_scale, hipStream_t s);

@@ -154,6 +154,13 @@ def dequant_matmul_i4(x, w, scale, zp, out, M, N, K, group_size, flags=0,
         flags, _stream(stream)))
 
 
+def quantize_groups_i16(x, q, scale_x, group_sum, M, K, group_size, stream=None):
+    """Per-group 16-bit quantisation of f16 activations: the first step of the
+    reassociated dequantising matmul (see include/iree_amd_uk.h)."""
+    _check(load_library().iree_amd_uk_quantize_groups_i16(
+        _ptr(x), _ptr(q), _ptr(scale_x), _ptr(group_sum), M, K, group_size, _stream(stream)))
+
+
 def pack_i4_weights(w_rowmajor, w_tiled, N, K, stream=None):
     """Row-major [N][K/2] 4-bit weights -> the DEQUANT_MATMUL_W_TILED layout."""
     _check(load_library().iree_amd_uk_pack_i4_weights(

@@ -28,12 +28,20 @@
  *       in tests/golden/conversion_kat.json) and the closed form over all 256 codes.
  *   oracle_dequant_matmul_i4           - closed form in numpy float64; nibble
  *       order against tests/e2e/linalg/subbyte_to_fp.mlir's vectors.
+ *   oracle_quantize_groups_i16 / oracle_dequant_matmul_i4_reassoc - no
+ *       reference implementation can be run (the pattern is compiler IR): the
+ *       quantisation against numpy float32 arithmetic, the integer core against
+ *       oracle/_ref's iree_uk_mmt4d S16U4S32 on the 1x32x8 tile and a numpy
+ *       integer product, the epilogue against the closed form in float64, and
+ *       the whole against oracle_dequant_matmul_i4 on inputs the 16-bit
+ *       quantisation represents exactly.
  *   oracle_silu_mul                    - libm identity x*sigmoid(x)*u.
  */
 #include "oracle.h"
 
 #include <math.h>
 #include <stddef.h>
+#include <stdlib.h>
 #include <string.h>
 
 /*---------------------------------------------------------------------------*
@@ -644,6 +652,92 @@ int oracle_dequant_matmul_i4(const uint16_t* x, const uint8_t* w,
       out[m * N + n] = f32_to_f16_ieee((float)acc);
     }
   }
+  return 0;
+}
+
+/* The reassociated form of the same dispatch
+ * (REF compiler/src/iree/compiler/GlobalOptimization/FuseDequantizationMatmul.cpp:
+ * generateGroupMaxGeneric :398-415, generateScalesGeneric :419-441 with
+ * (1 << (16 - 1)) - 1 = 32767, generateGroupSumsGeneric :445-461, the quantize
+ * generic :483-492 (divf then fptosi), the integer matmul :539-562 (sext i16,
+ * zext i4, i32 multiply-accumulate per group), and the final generic :622-633
+ * (sitofp; * new scale; * scale; zp * scale; * group sum; subf; addf over the
+ * groups in order)), in f32 as the pattern's float type: the activations are
+ * widened from f16 first. "Introduces precision loss ... opt-in only"
+ * (:746-748). fptosi truncates toward zero. A group of zeros has scale 0 and
+ * 0/0 in the quantize step; the reference leaves that undefined, here the
+ * group's quantised values are 0. */
+int oracle_quantize_groups_i16(const uint16_t* x, int64_t M, int64_t K, int64_t gs,
+                               int16_t* q, float* scale_x, float* group_sum) {
+  if (gs <= 0 || K % gs) return IREE_AMD_UK_STATUS_INVALID_ARGUMENT;
+  const int64_t G = K / gs;
+  for (int64_t m = 0; m < M; ++m)
+    for (int64_t g = 0; g < G; ++g) {
+      const uint16_t* xs = x + m * K + g * gs;
+      float mx = 0.0f, sum = 0.0f;
+      for (int64_t k = 0; k < gs; ++k) {
+        const float v = oracle_f16_to_f32(xs[k], ORACLE_F16_IEEE);
+        const float a = fabsf(v);
+        mx = a > mx ? a : mx;
+        sum = sum + v;
+      }
+      const float sc = mx / 32767.0f;
+      scale_x[m * G + g] = sc;
+      group_sum[m * G + g] = sum;
+      for (int64_t k = 0; k < gs; ++k) {
+        const float v = oracle_f16_to_f32(xs[k], ORACLE_F16_IEEE);
+        q[m * K + g * gs + k] = sc > 0.0f ? (int16_t)(v / sc) : (int16_t)0;
+      }
+    }
+  return 0;
+}
+
+int oracle_dequant_matmul_i4_reassoc(const uint16_t* x, const uint8_t* w,
+                                     const uint16_t* scale, const void* zp,
+                                     uint16_t* out, int64_t M, int64_t N, int64_t K,
+                                     int64_t gs, int zp_is_u4, int32_t* int_core) {
+  if (gs <= 0 || K % gs || (K & 1)) return IREE_AMD_UK_STATUS_INVALID_ARGUMENT;
+  const int64_t G = K / gs;
+  int16_t* q = (int16_t*)malloc((size_t)(M * K > 0 ? M * K : 1) * sizeof(int16_t));
+  float* sx = (float*)malloc((size_t)(M * G > 0 ? M * G : 1) * sizeof(float));
+  float* gsum = (float*)malloc((size_t)(M * G > 0 ? M * G : 1) * sizeof(float));
+  if (!q || !sx || !gsum) { free(q); free(sx); free(gsum); return 8; }
+  const int st = oracle_quantize_groups_i16(x, M, K, gs, q, sx, gsum);
+  if (st) { free(q); free(sx); free(gsum); return st; }
+#pragma omp parallel for
+  for (int64_t n = 0; n < N; ++n) {
+    for (int64_t m = 0; m < M; ++m) {
+      float acc_out = 0.0f;
+      for (int64_t g = 0; g < G; ++g) {
+        const int64_t sg = n * G + g;
+        const float s = oracle_f16_to_f32(scale[sg], ORACLE_F16_IEEE);
+        float z;
+        if (zp_is_u4) {
+          uint8_t b = ((const uint8_t*)zp)[sg >> 1];
+          z = (float)((sg & 1) ? (b >> 4) : (b & 0xF));
+        } else {
+          z = oracle_f16_to_f32(((const uint16_t*)zp)[sg], ORACLE_F16_IEEE);
+        }
+        int32_t acc = 0;
+        for (int64_t k = 0; k < gs; ++k) {
+          const int64_t e = n * K + g * gs + k;
+          const uint8_t b = w[e >> 1];
+          const int32_t wv = (e & 1) ? (b >> 4) : (b & 0xF);
+          acc += (int32_t)q[m * K + g * gs + k] * wv;
+        }
+        if (int_core) int_core[(m * N + n) * G + g] = acc;
+        const float dq = (float)acc;
+        const float r0 = dq * sx[m * G + g];
+        const float r1 = r0 * s;
+        const float z0 = z * s;
+        const float z1 = z0 * gsum[m * G + g];
+        const float res = r1 - z1;
+        acc_out = res + acc_out;
+      }
+      out[m * N + n] = f32_to_f16_ieee(acc_out);
+    }
+  }
+  free(q); free(sx); free(gsum);
   return 0;
 }
 

@@ -76,6 +76,19 @@ int oracle_dequant_matmul_i4(const uint16_t* x, const uint8_t* w,
                              uint16_t* out, int64_t M, int64_t N, int64_t K,
                              int64_t group_size, int zp_is_u4);
 
+/* The opt-in reassociated form (REF FuseDequantizationMatmul.cpp:398-645,
+ * 749-767): activations quantised per group to i16 (scale = absmax / 32767,
+ * fptosi(x / scale)), i16 x u4 -> i32 products summed per group, then
+ * sum_g (float(acc) * scale_x * scale - zp * scale * group_sum), all float
+ * steps in f32 in the reference's order. q: [M][K], scale_x / group_sum:
+ * [M][K/gs]. int_core (may be NULL) receives the integer sums [M][N][K/gs]. */
+int oracle_quantize_groups_i16(const uint16_t* x, int64_t M, int64_t K, int64_t gs,
+                               int16_t* q, float* scale_x, float* group_sum);
+int oracle_dequant_matmul_i4_reassoc(const uint16_t* x, const uint8_t* w,
+                                     const uint16_t* scale, const void* zp,
+                                     uint16_t* out, int64_t M, int64_t N, int64_t K,
+                                     int64_t gs, int zp_is_u4, int32_t* int_core);
+
 /* REF compiler/src/iree/compiler/GlobalOptimization/FuseSiluHorizontalMatmul.cpp:32-82:
  * (g / (1 + exp(-g))) * u, in double. */
 double oracle_silu_mul(double g, double u);

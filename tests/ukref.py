@@ -69,6 +69,14 @@ def oracle():
         lib.oracle_dequant_matmul_i4.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p,
                                                  C.c_void_p, C.c_void_p, C.c_int64,
                                                  C.c_int64, C.c_int64, C.c_int64, C.c_int]
+        lib.oracle_quantize_groups_i16.restype = C.c_int
+        lib.oracle_quantize_groups_i16.argtypes = [C.c_void_p, C.c_int64, C.c_int64, C.c_int64,
+                                                   C.c_void_p, C.c_void_p, C.c_void_p]
+        lib.oracle_dequant_matmul_i4_reassoc.restype = C.c_int
+        lib.oracle_dequant_matmul_i4_reassoc.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p,
+                                                         C.c_void_p, C.c_void_p, C.c_int64,
+                                                         C.c_int64, C.c_int64, C.c_int64, C.c_int,
+                                                         C.c_void_p]
         lib.oracle_silu_mul.restype = C.c_double
         lib.oracle_silu_mul.argtypes = [C.c_double, C.c_double]
         _oracle = lib
