@@ -364,6 +364,40 @@ def test_host_pointer_variants(uk, cuda):
     assert np.array_equal(out, ucase.run_oracle())
 
 
+@pytest.mark.parametrize("accumulate", [False, True])
+def test_host_pointer_mmt4d_in_row_blocks(uk, cuda, accumulate):
+    """A host-pointer mmt4d large enough to be pipelined over blocks of outer
+    rows (uploads of the next block overlapping the download of the finished
+    one): bit-equal to the device-pointer entry point on the same operands,
+    with a row count that the blocks do not divide, an offset left-hand side and
+    a loose left-hand-side stride; twice through one pool."""
+    import torch
+    lib = uk.load_library()
+    from iree_amd._lib import Mmt4dParams
+    M1, N1, K1, M0, N0, K0 = 77, 96, 16, 32, 32, 16
+    lhs_stride = K1 * M0 * K0 + 64
+    lhs = synth.uniform_int8(31, 128 + M1 * lhs_stride)
+    rhs = synth.uniform_int8(32, N1 * K1 * N0 * K0)
+    init = np.arange(M1 * N1 * M0 * N0, dtype=np.int32) % 1000 - 500
+    flags = F.MMT4D_TYPE_S8S8S32 | (F.MMT4D_ACCUMULATE if accumulate else 0)
+    want = torch.from_numpy(init.copy()).cuda()
+    uk.mmt4d(torch.from_numpy(lhs).cuda(), torch.from_numpy(rhs).cuda(), want, M1, N1, K1, M0, N0, K0, flags,
+             lhs_offset=128, lhs_stride0=lhs_stride)
+    torch.cuda.synchronize()
+    want = want.cpu().numpy()
+    pool = C.c_void_p()
+    assert lib.iree_amd_uk_host_pool_create(C.byref(pool)) == 0
+    try:
+        for _ in range(2):
+            out = init.copy()
+            p = Mmt4dParams(ukref.ptr(lhs).value, 128, lhs_stride, ukref.ptr(rhs).value, 0, K1 * N0 * K0,
+                            ukref.ptr(out).value, 0, N1 * M0 * N0, M1, N1, K1, M0, N0, K0, flags, None)
+            assert lib.iree_amd_uk_mmt4d_host_pooled(pool, C.byref(p)) == 0, lib.iree_amd_uk_last_error()
+            assert np.array_equal(out, want)
+    finally:
+        lib.iree_amd_uk_host_pool_destroy(pool)
+
+
 @pytest.mark.gpu
 def test_mfma_probe_runs_and_counts_operations(uk, cuda):
     """The register-only matrix-core loop bench.py times: it launches for every
