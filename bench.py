@@ -63,7 +63,7 @@ def parse_args():
                     "mmt4d_f16 | mmt4d_f16_acc | mmt4d_i8 | mmt4d_fp8 | mmt4d_f16_ksplit | mlp_fp8 | pack | unpack | "
                     "pack_transpose | dequant_i4[_m8|_m32] | dequant_i4_reassoc[_m8|_m32] | batch_mmt4d_f16 | "
                     "batch_mmt4d_f16_narrow | mmt4d_f16_narrow_m1 | mmt4d_f16_narrow_m8 | mmt4d_f16_narrow_n8 | "
-                    "chain_i8_1024 | copy | copy_rotating | copy_rotating_nt")
+                    "chain_i8_1024 | copy | copy_rotating | copy_rotating_nt | read_only_29mb")
     return ap.parse_args()
 
 
@@ -594,6 +594,33 @@ def extras(args, torch, iree_amd, F, synth, lhs, rhs, out, ex):
         diff = (a16 - b16).abs()
         assert float((diff > 1e-3 + 1e-2 * a16.abs()).float().mean()) <= 1e-3 and \
             bool((diff <= 4e-3 + 2e-2 * a16.abs()).all()), "reassociated int4 result out of tolerance"
+    # The yardstick for these weight streams: the same 29.4 MB buffers read by a
+    # kernel that does nothing else (16-byte loads, plain and non-temporal, one
+    # workgroup per 8 KiB and a few resident ones per compute unit), rotating
+    # like the kernels above. A 29 MB pass is short enough that launch, ramp and
+    # drain are a good part of it, for the kernels as for the yardstick.
+    wbytes = Nq * Kq // 2
+    rsink = torch.zeros(64, dtype=torch.int32, device="cuda")
+    best = None
+    for mode, tag in ((2, "plain"), (3, "nontemporal")):
+        for bpc in (0, 4, 8):
+            state["i"] = 0
+
+            def do_r():
+                k = state["i"] % nrot
+                state["i"] += 1
+                iree_amd.copy_probe(wq[k], rsink, wbytes, mode, bpc)
+
+            _, t = gpu_time(torch, do_r, steps, warm)
+            if best is None or t < best:
+                best = t
+            key = f"read_only_29mb_{tag}_us"
+            ex[key] = min(ex.get(key, 1e9), round(t * 1e6, 2))
+    ex["read_only_29mb_best_gbs"] = round(wbytes / best / 1e9, 1)
+    for Mq in (1, 8, 32):
+        ex[f"dequant_matmul_i4_m{Mq}_frac_of_read_yardstick"] = round(best * 1e6 / ex[f"dequant_matmul_i4_m{Mq}_us"], 4)
+    assert int(rsink.abs().sum()) == 0
+    del rsink
     # the transposed shape (N 4096, K 14336, the same byte counts and buffers):
     # a K the register-resident kernel cannot take; the activations go through
     # LDS, 1 row in one pass, 8 rows in two passes over the weights
@@ -748,6 +775,16 @@ def run_only(args, torch, iree_amd, F, synth, mm_step):
             k = st["i"] % 10
             st["i"] += 1
             iree_amd.dequant_matmul_i4(xq, wq[k], sq, zq, oq, Mq, Nq, Kq, gs, qflags)
+    elif args.only == "read_only_29mb":
+        # the read-only yardstick of the int4 weight stream: ten rotating 29.4 MB buffers
+        wq = [torch.from_numpy(synth.uniform_u4_packed(10 + i, 14336 * 4096)).cuda() for i in range(10)]
+        rsink = torch.zeros(64, dtype=torch.int32, device="cuda")
+        st = {"i": 0}
+
+        def fn():
+            k = st["i"] % 10
+            st["i"] += 1
+            iree_amd.copy_probe(wq[k], rsink, 14336 * 4096 // 2, 3, 0)
     elif args.only in ("copy_rotating", "copy_rotating_nt"):
         fn, _ = make_copy_rotating(torch, iree_amd, 1 if args.only.endswith("_nt") else 0)
     elif args.only == "mmt4d_f16_acc":

@@ -562,8 +562,10 @@ IREE_AMD_UK_EXPORT int iree_amd_uk_mfma_probe(uint32_t type_flag,
  * buffers 16-byte aligned and not overlapping) with 16-byte accesses, as the
  * reference's benchmarks measure memcpy next to pack
  * (REF runtime/src/iree/builtins/ukernel/tools/memcpy_benchmark.c:24-52).
- * mode 0 = plain accesses, 1 = non-temporal ones; blocks_per_cu = workgroups
- * per compute unit (0 = one workgroup per 8 KiB). */
+ * mode 0 = plain accesses, 1 = non-temporal ones; 2 and 3 = the loads of 0
+ * and 1 without the stores (the yardstick for kernels that only stream a
+ * weight matrix; `dst` then needs 4 writable bytes and stays untouched);
+ * blocks_per_cu = workgroups per compute unit (0 = one workgroup per 8 KiB). */
 IREE_AMD_UK_EXPORT int iree_amd_uk_copy_probe(const void* src, void* dst,
                                               iree_amd_uk_index_t bytes, int32_t mode,
                                               int32_t blocks_per_cu, void* stream);

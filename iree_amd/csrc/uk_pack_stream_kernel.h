@@ -55,7 +55,12 @@ struct Pow2Args {
 // (non-temporal loads: pack 4.5 TB/s) and are pieces of DRAM pages that
 // non-temporal stores no longer merge (unpack 3.0 TB/s). A plain copy with
 // 8 KiB runs on both sides reaches 5.3-5.5 TB/s with ordinary and 6.0-6.2 with
-// non-temporal accesses on the same machine.
+// non-temporal accesses on the same machine. Staging 32 rows x 1 KiB per
+// workgroup through LDS, so that every wave instruction moves 1 KiB of one
+// matrix row or of consecutive tile memory, was slower in all four
+// combinations of non-temporal sides (pack 4.4-5.0, unpack 4.2-4.5 TB/s):
+// longer runs per instruction do not pay for the barrier and the fewer, larger
+// workgroups.
 template <int ES, bool kPack, bool kNtLoad = !kPack, bool kNtStore = kPack>
 __device__ __forceinline__ void stream_pow2_body(const Pow2Args a) {
   constexpr int CE = 16 / ES;

@@ -113,7 +113,7 @@ __global__ __launch_bounds__(kThreads) void dequant_matmul_i4_kernel(I4Args a) {
   // it requests the same span of the NEXT tile, which so streams from HBM
   // while the later spans of x still arrive.
   // activations: rows m_base + mh*16 + nl, this wave's K slice; rows past M
-  // are read from the last row and zeroed.
+  // are zeros.
   int nt = blockIdx.x;
   Meta meta_next;
   load_meta(nt < a.n_tiles ? nt : a.n_tiles - 1, meta_next);
@@ -126,11 +126,26 @@ __global__ __launch_bounds__(kThreads) void dequant_matmul_i4_kernel(I4Args a) {
     for (int sp = 0; sp < SP; ++sp) {
 #pragma unroll
       for (int mh = 0; mh < MH; ++mh) {
+        // (lanes of rows past M load nothing: with one row of activations the
+        // texture path would otherwise spend twice the time on 16 copies of
+        // that row that it spends on the tile's weights)
+        // With 32 rows (nearly all of them live) the loads are unconditional,
+        // rows past M read the last row and are zeroed below: the branch
+        // measured 5 % slower there.
         const int m = a.m_base + mh * 16 + nl;
         const int mr = m < a.M ? m : a.M - 1;
         const uint16_t* row = a.x + (size_t)mr * a.K + k_slice + kc * ckc;
+        if constexpr (MH == 1) {
 #pragma unroll
-        for (int q = 0; q < 4; ++q) xraw[mh][sp][q] = *(const u32x4*)(row + sp * 128 + q * cq);
+          for (int q = 0; q < 4; ++q) xraw[mh][sp][q] = u32x4{0u, 0u, 0u, 0u};
+          if (m < a.M) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) xraw[mh][sp][q] = *(const u32x4*)(row + sp * 128 + q * cq);
+          }
+        } else {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) xraw[mh][sp][q] = *(const u32x4*)(row + sp * 128 + q * cq);
+        }
       }
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -160,11 +175,11 @@ __global__ __launch_bounds__(kThreads) void dequant_matmul_i4_kernel(I4Args a) {
       if constexpr (kFirst) {
 #pragma unroll
         for (int mh = 0; mh < MH; ++mh) {
-          const uint32_t keep = a.m_base + mh * 16 + nl < a.M ? 0xFFFFFFFFu : 0u;
+          const uint32_t keep = MH == 1 || a.m_base + mh * 16 + nl < a.M ? 0xFFFFFFFFu : 0u;
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
             u32x4 v = xraw[mh][sp][q];
-            v.x &= keep; v.y &= keep; v.z &= keep; v.w &= keep;
+            if constexpr (MH != 1) { v.x &= keep; v.y &= keep; v.z &= keep; v.w &= keep; }
             xf[mh][sp][q] = permute_x(v);
           }
         }

@@ -255,7 +255,8 @@ def mfma_probe(type_flag, operands, iters, sink, stream=None):
 
 def copy_probe(src, dst, nbytes, mode=0, blocks_per_cu=0, stream=None):
     """Plain out-of-place copy of ``nbytes`` (whole 8 KiB chunks): the yardstick
-    for the pack / unpack streams. A measurement aid, not part of the
+    for the pack / unpack streams; modes 2 and 3 only read (the yardstick for
+    the weight-streaming kernels). A measurement aid, not part of the
     reference's interface."""
     _check(load_library().iree_amd_uk_copy_probe(_ptr(src), _ptr(dst), nbytes, mode, blocks_per_cu,
                                                  _stream(stream)))

@@ -130,3 +130,27 @@ def test_full_size_f16_8191x5001_pack_unpack_round_trip(uk, cuda):
     b = back.cpu().numpy().view(np.uint16)
     assert np.array_equal(b[:R * Cc], x)
     assert (b[R * Cc:] == 0x1234).all()
+
+
+def test_copy_and_read_probes(uk, cuda):
+    """The yardstick kernels bench.py times next to pack / unpack and the
+    weight-streaming kernels: modes 0 and 1 copy every byte, modes 2 and 3 read
+    only and leave the destination alone; sizes that are not whole 8 KiB chunks
+    are refused."""
+    import torch
+    n = 8192 * 37
+    src = torch.from_numpy(np.random.default_rng(5).integers(0, 256, n, dtype=np.uint8)).to(cuda)
+    for mode in (0, 1):
+        for bpc in (0, 2):
+            dst = torch.zeros(n, dtype=torch.uint8, device=cuda)
+            uk.copy_probe(src, dst, n, mode, bpc)
+            torch.cuda.synchronize()
+            assert torch.equal(src, dst)
+    sink = torch.full((16,), 7, dtype=torch.int32, device=cuda)
+    for mode in (2, 3):
+        uk.copy_probe(src, sink, n, mode, 0)
+        uk.copy_probe(src, sink, n, mode, 4)
+    torch.cuda.synchronize()
+    assert bool((sink == 7).all())
+    with pytest.raises(uk.UkError):
+        uk.copy_probe(src, sink, 8192 * 3 + 16, 0, 0)
