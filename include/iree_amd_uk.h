@@ -436,6 +436,17 @@ IREE_AMD_UK_EXPORT int iree_amd_uk_quantize_f16_to_f8e4m3(
     const void* in_f16, void* out_fp8, iree_amd_uk_index_t n, float inv_scale,
     void* stream);
 
+/* The same conversion and the pack of its result in one pass: f16 row-major
+ * [rows][cols] (row pitch `ld` elements) -> e4m3 left-hand-side tiles
+ * [ceil(rows/32)][cols/16][32][16] with outer pitch `out_stride0` bytes; rows
+ * past `rows` are zero. Bit-identical to iree_amd_uk_quantize_f16_to_f8e4m3
+ * followed by iree_amd_uk_pack (8-bit, tiles 32x16, padding 0). cols must be
+ * whole tiles of 16. */
+IREE_AMD_UK_EXPORT int iree_amd_uk_quantize_pack_f8e4m3(
+    const void* in_f16, iree_amd_uk_index_t ld, void* out_tiles,
+    iree_amd_uk_index_t out_stride0, iree_amd_uk_index_t rows,
+    iree_amd_uk_index_t cols, float inv_scale, void* stream);
+
 /* out_fp8[m][n] = e4m3fn( silu(gate[m][n]*gate_scale) * (up[m][n]*up_scale)
  *                          * inv_out_scale ), gate/up f32 row-major [rows][cols]
  * with row pitch `ld` elements. */

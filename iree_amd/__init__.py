@@ -25,6 +25,7 @@ from .ukernel import (  # noqa: F401
     pack,
     pack_i4_weights,
     quantize_f16_to_f8e4m3,
+    quantize_pack_f8e4m3,
     query_tile_sizes_2d,
     scale_f32,
     silu_mul_quantize,

@@ -109,6 +109,8 @@ def _declare(lib):
     lib.iree_amd_uk_pack_i4_weights.argtypes = [vp, vp, i64, i64, vp]
     lib.iree_amd_uk_quantize_f16_to_f8e4m3.restype = C.c_int
     lib.iree_amd_uk_quantize_f16_to_f8e4m3.argtypes = [vp, vp, i64, C.c_float, vp]
+    lib.iree_amd_uk_quantize_pack_f8e4m3.restype = C.c_int
+    lib.iree_amd_uk_quantize_pack_f8e4m3.argtypes = [vp, i64, vp, i64, i64, i64, C.c_float, vp]
     lib.iree_amd_uk_silu_mul_quantize.restype = C.c_int
     lib.iree_amd_uk_silu_mul_quantize.argtypes = [vp, vp, vp, i64, i64, i64,
                                                    C.c_float, C.c_float, C.c_float, vp]

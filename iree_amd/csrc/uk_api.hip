@@ -470,6 +470,19 @@ extern "C" int iree_amd_uk_quantize_f16_to_f8e4m3(const void* in_f16,
   return launch_quantize_f16_to_f8e4m3(in_f16, out_fp8, n, inv_scale, (hipStream_t)stream);
 }
 
+extern "C" int iree_amd_uk_quantize_pack_f8e4m3(const void* in_f16, iree_amd_uk_index_t ld, void* out_tiles,
+                                               iree_amd_uk_index_t out_stride0, iree_amd_uk_index_t rows,
+                                               iree_amd_uk_index_t cols, float inv_scale, void* stream) {
+  if (rows < 0 || cols < 0 || ld < cols || cols % 16)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "quantize_pack: cols must be whole tiles of 16 and ld >= cols");
+  if (rows == 0 || cols == 0) return 0;
+  if (!in_f16 || !out_tiles) return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "quantize_pack: null buffer");
+  if (out_stride0 < cols * 32 || out_stride0 % 16 || ((uintptr_t)out_tiles & 15))
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT,
+                "quantize_pack: the tiled buffer must be 16-byte aligned with an outer pitch of whole 16 bytes, at least cols * 32");
+  return launch_quantize_pack_f8e4m3(in_f16, ld, out_tiles, out_stride0, rows, cols, inv_scale, (hipStream_t)stream);
+}
+
 extern "C" int iree_amd_uk_silu_mul_quantize(
     const void* gate_f32, const void* up_f32, void* out_fp8,
     iree_amd_uk_index_t rows, iree_amd_uk_index_t cols, iree_amd_uk_index_t ld,

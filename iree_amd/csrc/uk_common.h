@@ -150,6 +150,8 @@ int launch_quantize_groups_i16(const void* x, void* q, void* scale_x, void* grou
 int launch_pack_i4_weights(const void* src, void* dst, int64_t N, int64_t K, hipStream_t s);
 int launch_quantize_f16_to_f8e4m3(const void* in, void* out, int64_t n,
                                   float inv_scale, hipStream_t s);
+int launch_quantize_pack_f8e4m3(const void* in, int64_t ld, void* out, int64_t out_stride0, int64_t rows,
+                                int64_t cols, float inv_scale, hipStream_t s);
 int launch_silu_mul_quantize(const void* gate, const void* up, void* out,
                              int64_t rows, int64_t cols, int64_t ld,
                              float gate_scale, float up_scale,

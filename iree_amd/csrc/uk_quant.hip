@@ -464,6 +464,41 @@ __global__ __launch_bounds__(256) void quantize_f16_kernel(const uint16_t* in, u
   }
 }
 
+// Quantisation and the pack of the result in one pass: f16 row-major
+// [rows][cols] -> e4m3 left-hand-side tiles [ceil(rows/32)][cols/16][32][16],
+// rows past `rows` zero (the padding value of that pack). A lane makes one
+// 16-byte tile row from 32 bytes of a matrix row; lane = (row in block) * 8 +
+// (tile column in block) as in the streaming pack, so a wave reads 8 row
+// pieces of 256 bytes and writes 8 runs of 128 bytes, and a workgroup's four
+// waves complete 8 whole tiles.
+typedef u32x4 u32x4_align2 __attribute__((aligned(2)));
+__global__ __launch_bounds__(256) void quantize_pack_f8_kernel(const uint16_t* in, int64_t ld, uint8_t* out,
+                                                               int64_t out_stride0, int64_t rows, int64_t k_tiles,
+                                                               float inv_scale) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t kt = (int64_t)blockIdx.x * 8 + (lane & 7);
+  const int row_in_tile = wave * 8 + (lane >> 3);
+  const int64_t row = (int64_t)blockIdx.y * 32 + row_in_tile;
+  if (kt >= k_tiles) return;
+  u32x2 q0 = {0u, 0u}, q1 = {0u, 0u};
+  if (row < rows) {
+    const uint16_t* src = in + row * ld + kt * 16;
+    const u32x4 a = *(const u32x4_align2*)src, b = *(const u32x4_align2*)(src + 8);
+    float f[16];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      f[2 * j] = __half2float(__ushort_as_half((uint16_t)(a[j] & 0xFFFF))) * inv_scale;
+      f[2 * j + 1] = __half2float(__ushort_as_half((uint16_t)(a[j] >> 16))) * inv_scale;
+      f[8 + 2 * j] = __half2float(__ushort_as_half((uint16_t)(b[j] & 0xFFFF))) * inv_scale;
+      f[8 + 2 * j + 1] = __half2float(__ushort_as_half((uint16_t)(b[j] >> 16))) * inv_scale;
+    }
+    q0 = u32x2{pack4_e4m3(f[0], f[1], f[2], f[3]), pack4_e4m3(f[4], f[5], f[6], f[7])};
+    q1 = u32x2{pack4_e4m3(f[8], f[9], f[10], f[11]), pack4_e4m3(f[12], f[13], f[14], f[15])};
+  }
+  uint8_t* dst = out + (int64_t)blockIdx.y * out_stride0 + kt * 512 + row_in_tile * 16;
+  *(u32x4*)dst = u32x4{q0.x, q0.y, q1.x, q1.y};
+}
+
 __global__ __launch_bounds__(256) void quantize_f16_scalar_kernel(const uint16_t* in, uint8_t* out,
                                                                   int64_t n, float inv_scale) {
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
@@ -557,6 +592,16 @@ int launch_quantize_f16_to_f8e4m3(const void* in, void* out, int64_t n, float in
                        (const uint16_t*)in, (uint8_t*)out, n, inv_scale);
   }
   return check_hip(hipGetLastError(), "quantize_f16_to_f8e4m3 launch");
+}
+
+int launch_quantize_pack_f8e4m3(const void* in, int64_t ld, void* out, int64_t out_stride0, int64_t rows,
+                                int64_t cols, float inv_scale, hipStream_t s) {
+  const int64_t k_tiles = cols / 16, row_tiles = ceil_div(rows, 32);
+  if (row_tiles > 65535 || ceil_div(k_tiles, 8) > 0x7FFFFFFF)
+    return fail(IREE_AMD_UK_STATUS_UNIMPLEMENTED, "quantize_pack: more than 65535 outer rows");
+  hipLaunchKernelGGL(quantize_pack_f8_kernel, dim3((unsigned)ceil_div(k_tiles, 8), (unsigned)row_tiles), dim3(256), 0, s,
+                     (const uint16_t*)in, ld, (uint8_t*)out, out_stride0, rows, k_tiles, inv_scale);
+  return check_hip(hipGetLastError(), "quantize_pack launch");
 }
 
 int launch_silu_mul_quantize(const void* gate, const void* up, void* out, int64_t rows,

@@ -172,6 +172,17 @@ def quantize_f16_to_f8e4m3(inp, out, n, inv_scale, stream=None):
         _ptr(inp), _ptr(out), n, inv_scale, _stream(stream)))
 
 
+def quantize_pack_f8e4m3(inp, out_tiles, rows, cols, inv_scale, *, ld=None, out_stride0=None, stream=None):
+    """quantize_f16_to_f8e4m3 and the pack of its result into 32x16 left-hand-side
+    tiles in one pass (rows past ``rows`` zero); strides default to tight."""
+    if ld is None:
+        ld = cols
+    if out_stride0 is None:
+        out_stride0 = cols * 32
+    _check(load_library().iree_amd_uk_quantize_pack_f8e4m3(
+        _ptr(inp), ld, _ptr(out_tiles), out_stride0, rows, cols, inv_scale, _stream(stream)))
+
+
 def silu_mul_quantize(gate, up, out, rows, cols, ld, gate_scale, up_scale,
                       inv_out_scale, stream=None):
     _check(load_library().iree_amd_uk_silu_mul_quantize(
@@ -404,8 +415,11 @@ class Fp8Mlp:
             raise ValueError("M must be a multiple of 32 within max_tokens")
         M1, F1, H1 = M // 32, ffn // 32, hidden // 32
         mm = F.MMT4D_TYPE_F8E4M3F8E4M3F32
-        quantize_f16_to_f8e4m3(x_f16, self.xq, M * hidden, 1.0 / self.sx)
-        pack(self.xq, self.x_tiles, M, hidden, M1, hidden // 16, 32, 16, 0, F.PACK_TYPE_I8I8)
+        if self.fused:
+            quantize_pack_f8e4m3(x_f16, self.x_tiles, M, hidden, 1.0 / self.sx)
+        else:
+            quantize_f16_to_f8e4m3(x_f16, self.xq, M * hidden, 1.0 / self.sx)
+            pack(self.xq, self.x_tiles, M, hidden, M1, hidden // 16, 32, 16, 0, F.PACK_TYPE_I8I8)
         if self.fused:
             mmt4d_silu_mul_f8e4m3(self.x_tiles, self.wgu, self.h_tiles, M1, 2 * F1, hidden // 16, 16, mm,
                                   self.sx * self.sg, self.sx * self.su, 1.0 / self.sh)

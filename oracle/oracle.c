@@ -141,7 +141,18 @@ static uint16_t f32_to_f16_ieee(float f) {
   return sign | (uint16_t)(((uint32_t)(e + 15) << 10) + (q - 0x400));
 }
 
-float oracle_f8e4m3_to_f32(uint8_t v, int ieee) {
+static float f8e4m3_decode_one(uint8_t v, int ieee);
+/* The matmul loops decode two operands per multiply-add: the 2 x 256 values
+ * are tabulated when the library is loaded. */
+static float f8e4m3_table[2][256];
+__attribute__((constructor)) static void f8e4m3_table_init(void) {
+  for (int ieee = 0; ieee < 2; ++ieee)
+    for (int v = 0; v < 256; ++v) f8e4m3_table[ieee][v] = f8e4m3_decode_one((uint8_t)v, ieee);
+}
+
+float oracle_f8e4m3_to_f32(uint8_t v, int ieee) { return f8e4m3_table[ieee ? 1 : 0][v]; }
+
+static float f8e4m3_decode_one(uint8_t v, int ieee) {
   const int s = v >> 7, e = (v >> 3) & 0xF, m = v & 7;
   float mag;
   if (e == 15 && m == 7) return bits_to_f32(((uint32_t)s << 31) | 0x7FFFFFFFu);

@@ -99,6 +99,44 @@ def test_quantize_ragged_and_unaligned(uk, cuda):
         assert np.all(got[:off] == 0xAA) and np.all(got[off + n:] == 0xAA)
 
 
+@pytest.mark.parametrize("rows,cols,ld,loose", [(64, 256, 256, False), (45, 48, 56, True), (1, 16, 16, False),
+                                                (33, 2064, 2064, False), (2048, 4096, 4096, False)])
+def test_quantize_pack_in_one_pass(uk, cuda, rows, cols, ld, loose):
+    """The fused quantisation + pack: bit-exact against the oracle encoder laid
+    out by the pack oracle's rule (tile (i, j) row r = matrix row 32 i + r,
+    columns 16 j .. 16 j + 16, rows past the end zero), and equal to the two
+    separate entry points; all f16 bit patterns occur in the first case; memory
+    between outer rows of a loose tiled buffer stays untouched."""
+    import torch
+    if rows * cols >= 65536:
+        x = np.resize(np.arange(65536, dtype=np.uint16), rows * ld)
+        x = np.where((x & 0x7C00) == 0x7C00, x & 0x83FF, x).astype(np.uint16)     # no Inf / NaN here
+    else:
+        x = synth.normal_f16(rows + cols, rows * ld, 30.0).view(np.uint16)
+    inv_scale = 0.37
+    M1, K1 = -(-rows // 32), cols // 16
+    stride = cols * 32 + (64 if loose else 0)
+    src = torch.from_numpy(x.view(np.int16)).cuda()
+    out = torch.full((M1 * stride,), 0xAA, dtype=torch.uint8, device="cuda")
+    uk.quantize_pack_f8e4m3(src, out, rows, cols, inv_scale, ld=ld, out_stride0=stride)
+    q = torch.zeros(rows * ld, dtype=torch.uint8, device="cuda")
+    uk.quantize_f16_to_f8e4m3(src, q, rows * ld, inv_scale)
+    two = torch.full((M1 * stride,), 0xAA, dtype=torch.uint8, device="cuda")
+    uk.pack(q, two, rows, cols, M1, K1, 32, 16, 0, F.PACK_TYPE_I8I8, in_stride0=ld, out_stride0=stride)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    assert np.array_equal(got, two.cpu().numpy())
+    xm = x.view(np.float16).reshape(rows, ld)[:, :cols].astype(np.float32) * np.float32(inv_scale)
+    want = np.zeros((M1 * 32, cols), np.uint8)
+    want[:rows] = quantize_np(xm.reshape(-1)).reshape(rows, cols)
+    want = want.reshape(M1, 32, K1, 16).transpose(0, 2, 1, 3).reshape(M1, cols * 32)
+    g = got.reshape(M1, stride)
+    assert np.array_equal(g[:, :cols * 32], want)
+    assert np.all(g[:, cols * 32:] == 0xAA)
+    with pytest.raises(uk.UkError):
+        uk.quantize_pack_f8e4m3(src, out, rows, cols - 3, inv_scale, ld=ld, out_stride0=stride)
+
+
 def _acceptable_codes(v64):
     """Codes an implementation accurate to 1e-5 relative may produce."""
     lo = quantize_np(v64 * (1 - 1e-5) - 1e-12)
@@ -239,6 +277,7 @@ def test_fp8_mlp_block_small(uk, cuda):
     y2 = torch.full((M * H,), 7.0, dtype=torch.float32, device="cuda")
     fused(dev(x.view(np.int16)), y2, M)
     torch.cuda.synchronize()
+    assert np.array_equal(fused.x_tiles.cpu().numpy(), mlp.x_tiles.cpu().numpy())   # one-pass quantise + pack
     assert np.array_equal(fused.h_tiles.cpu().numpy(), mlp.h_tiles.cpu().numpy())
     assert np.array_equal(y2.cpu().numpy(), y.cpu().numpy())
     # x codes: bit-exact
@@ -349,7 +388,8 @@ def test_fp8_mlp_block_full_size_sampled_tokens(uk, cuda):
     y = torch.zeros(M * H, dtype=torch.float32, device="cuda")
     mlp(x, y, M)
     torch.cuda.synchronize()
-    assert np.array_equal(mlp.xq.cpu().numpy().reshape(M, H)[rows], xq)
+    xt = mlp.x_tiles.cpu().numpy().reshape(M // 32, H // 16, 32, 16).transpose(0, 2, 1, 3).reshape(M, H)
+    assert np.array_equal(xt[rows], xq)
     hq = mlp.h_tiles.cpu().numpy().reshape(M // 32, Fn // 16, 32, 16).transpose(0, 2, 1, 3).reshape(M, Fn)[rows]
     eg = 4e-5 * (np.abs(X) @ np.abs(wg).T) * (sx * sg)
     eu = 4e-5 * (np.abs(X) @ np.abs(wu).T) * (sx * su)
