@@ -270,17 +270,17 @@ __global__ __launch_bounds__(kStreamThreads) void unpack_stream_kernel(StreamArg
 }
 
 template <int ES, bool kPack>
-__global__ __launch_bounds__(kStreamThreads) void stream_pow2_kernel(Pow2Args a) {
+__global__ __launch_bounds__(kPow2Waves * 64) void stream_pow2_kernel(Pow2Args a) {
   stream_pow2_body<ES, kPack>(a);
 }
 
 // The 32-bit per-lane offsets of stream_pow2_kernel must not overflow.
 bool pow2_eligible(const StreamArgs& a, int es) {
   if (!a.pow2) return false;
-  const int64_t rows = kBlockRows * kStreamUnroll;
+  const int64_t rows = kPow2Rows * kPow2Unroll;
   const int64_t pitch = a.m_stride0 * es;
-  if (pitch * rows + 128 >= (1ll << 31)) return false;
-  const int64_t panels = rows / a.tile_rows + 2, cols = kBlockChunks / a.cpr + 2;
+  if (pitch * rows + 256 >= (1ll << 31)) return false;
+  const int64_t panels = rows / a.tile_rows + 2, cols = (64 / kPow2Rows) / a.cpr + 2;
   if (a.t_stride_row_bytes * panels + a.t_stride_col_bytes * cols + (1ll << 20) >= (1ll << 31)) return false;
   if ((int64_t)a.tile_rows * a.cpr * 16 >= (1ll << 20)) return false;
   return true;
@@ -298,11 +298,11 @@ int launch_stream_pow2(const StreamArgs& a, hipStream_t s) {
   p.padding = a.padding;
   const int64_t cols = kPack ? a.padded_chunks_per_row : a.chunks_per_row;
   const int64_t rows = kPack ? a.padded_rows : a.m_size0;
-  const int64_t bx = ceil_div(cols, 4 * kBlockChunks);
-  const int64_t by = ceil_div(rows, kBlockRows * kStreamUnroll);
+  const int64_t bx = ceil_div(cols, kPow2WavesX * (64 / kPow2Rows));
+  const int64_t by = ceil_div(rows, kPow2Rows * kPow2Unroll * (kPow2Waves / kPow2WavesX));
   if (bx < 1 || by < 1 || bx * by > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
   p.blocks_x = (uint32_t)bx; p.blocks_y = (uint32_t)by;
-  hipLaunchKernelGGL((stream_pow2_kernel<ES, kPack>), dim3((unsigned)(bx * by)), dim3(kStreamThreads), 0, s, p);
+  hipLaunchKernelGGL((stream_pow2_kernel<ES, kPack>), dim3((unsigned)(bx * by)), dim3(kPow2Waves * 64), 0, s, p);
   return check_hip(hipGetLastError(), "stream_pow2 launch");
 }
 

@@ -20,16 +20,27 @@ template <> struct Chunk<4> { typedef u32x4 aligned_t __attribute__((aligned(4))
 constexpr int kStreamThreads = 256;
 constexpr int kStreamUnroll = 2;
 
-// Both kernels walk the MATRIX in blocks of 8 rows x 8 chunks (128 bytes of
-// each row) per wave instruction: lane = (row in block) * 8 + (chunk in block).
-// On the matrix side every row segment is 128 contiguous bytes; on the tiled
-// side the 8 rows of one tile column are contiguous as well (8 tile rows of
-// cpr chunks each), so neither side moves less than a cache line at a time.
-// A wave takes kStreamUnroll vertically adjacent blocks; the 4 waves of a
-// workgroup take 4 horizontally adjacent column strips. (Measured on MI355X:
-// two blocks per wave beat four and eight - more waves in flight matter more
-// than more bytes per wave.)
+// The streaming kernels walk the MATRIX in blocks of R rows x 64 / R chunks
+// per wave instruction: lane = (row in block) * (64 / R) + (chunk in block).
+// On the matrix side every row segment is 1024 / R contiguous bytes; on the
+// tiled side the R rows of one tile column are contiguous as well (R tile rows
+// of cpr chunks each), so neither side moves less than a cache line at a time.
+// The kernels for general tile geometry (uk_pack.hip) use R = 8 with
+// kStreamUnroll vertically adjacent blocks per wave and 4 waves side by side:
 constexpr int kBlockRows = 8, kBlockChunks = 8;
+// The power-of-two kernel below takes its block shape as template parameters:
+// kRowsPerBlock rows x 64 / kRowsPerBlock chunks per wave instruction, kUnroll
+// vertically adjacent blocks per wave, kWaves waves per workgroup of which kWX
+// side by side. Measured on MI355X (f16 8191 x 5001 <-> 32x16 tiles, TB/s,
+// pack / unpack): 8 rows x 8 chunks, 2 blocks, 4 waves side by side 5.31 /
+// 4.78; one block per wave 5.50 / 5.10; 4 rows x 16 chunks (256 bytes of a
+// row), one block 5.50-5.54 / 5.24-5.30, as 2 x 2 waves 5.54 / 5.35, as one
+// wave per workgroup 5.61 / 5.38 (the library's choice: the smallest unit of
+// work, 4 KiB, scheduled on its own); 2 rows x 32 chunks 4.82 / 4.78; 16 rows
+// x 4 chunks 5.42 / 4.87; more blocks per wave lose in every shape. Longer row
+// pieces halve the partly written cache lines of ragged rows, which is what
+// unpack gains from.
+constexpr int kPow2Rows = 4, kPow2Unroll = 1, kPow2WavesX = 1, kPow2Waves = 1;
 
 // Power-of-two tile geometry (every gfx950 tile shape): the same 8x8 block walk
 // with all 64-bit address arithmetic done once per wave on the scalar unit and
@@ -61,9 +72,11 @@ struct Pow2Args {
 // combinations of non-temporal sides (pack 4.4-5.0, unpack 4.2-4.5 TB/s):
 // longer runs per instruction do not pay for the barrier and the fewer, larger
 // workgroups.
-template <int ES, bool kPack, bool kNtLoad = !kPack, bool kNtStore = kPack>
+template <int ES, bool kPack, bool kNtLoad = !kPack, bool kNtStore = kPack, int kBlockRows = kPow2Rows,
+          int kStreamUnroll = kPow2Unroll, int kWX = kPow2WavesX, int kWaves = kPow2Waves>
 __device__ __forceinline__ void stream_pow2_body(const Pow2Args a) {
   constexpr int CE = 16 / ES;
+  constexpr int kBlockChunks = 64 / kBlockRows;
   constexpr int kRows = kBlockRows * kStreamUnroll;
   typedef typename Chunk<ES>::aligned_t mat_vec_t;
   const uint32_t lane = threadIdx.x & 63;
@@ -81,14 +94,14 @@ __device__ __forceinline__ void stream_pow2_body(const Pow2Args a) {
     by = logical / a.blocks_x;
     bx = logical - by * a.blocks_x;
   }
-  const uint32_t j0 = (bx * 4 + wave) * kBlockChunks;
+  const uint32_t j0 = (bx * kWX + wave % kWX) * kBlockChunks;
   const uint32_t col_limit = kPack ? a.padded_chunks_per_row : a.chunks_per_row;
   if (j0 >= col_limit) return;
   const int64_t row_limit = kPack ? a.padded_rows : a.m_size0;
-  const int64_t r0 = (int64_t)by * kRows;
+  const int64_t r0 = ((int64_t)by * (kWaves / kWX) + wave / kWX) * kRows;
   if (r0 >= row_limit) return;
   const uint32_t tile_rows = 1u << a.log2_tile_rows, cpr = 1u << a.log2_cpr;
-  const uint32_t jl = lane & 7, rl = lane >> 3;
+  const uint32_t jl = lane % kBlockChunks, rl = lane / kBlockChunks;
   // Scalar bases of this wave's block on both sides.
   const char* mat_base = a.mat + r0 * a.m_pitch_bytes + (int64_t)j0 * 16;
   char* tiled_base = a.tiled + (r0 >> a.log2_tile_rows) * a.t_stride_row_bytes +
