@@ -575,7 +575,9 @@ IREE_AMD_UK_EXPORT int iree_amd_uk_mfma_probe(uint32_t type_flag,
  * (REF runtime/src/iree/builtins/ukernel/tools/memcpy_benchmark.c:24-52).
  * mode 0 = plain accesses, 1 = non-temporal ones; 2 and 3 = the loads of 0
  * and 1 without the stores (the yardstick for kernels that only stream a
- * weight matrix; `dst` then needs 4 writable bytes and stays untouched);
+ * weight matrix; `dst` then needs 4 writable bytes and stays untouched); + 4 =
+ * the same four in single-wave workgroups of 1 KiB per step (the pack / unpack
+ * kernels' unit of work) instead of 256 threads and 8 KiB;
  * blocks_per_cu = workgroups per compute unit (0 = one workgroup per 8 KiB). */
 IREE_AMD_UK_EXPORT int iree_amd_uk_copy_probe(const void* src, void* dst,
                                               iree_amd_uk_index_t bytes, int32_t mode,

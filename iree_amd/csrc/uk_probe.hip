@@ -58,20 +58,22 @@ __global__ __launch_bounds__(256) void mfma_probe_kernel(const char* operands, i
 // runtime/src/iree/builtins/ukernel/tools/memcpy_benchmark.c:24-52). Every lane
 // moves 16 bytes per access; a wave keeps kCopyUnroll accesses of 1 KiB in
 // flight; workgroups walk contiguous chunks, XCD by XCD, like the pack kernel.
-constexpr int kCopyUnroll = 2;
-template <bool kNonTemporal>
-__global__ __launch_bounds__(256) void copy_probe_kernel(const u32x4p* src, u32x4p* dst, int64_t chunks) {
-  // chunk = kCopyUnroll * 256 lanes * 16 bytes
+// Two geometries: 256 threads with two accesses in flight per lane (8 KiB per
+// workgroup and step), and single waves with one (1 KiB: the unit of work the
+// pack / unpack kernels settled on).
+template <bool kNonTemporal, int kThreads, int kCopyUnroll>
+__global__ __launch_bounds__(kThreads) void copy_probe_kernel(const u32x4p* src, u32x4p* dst, int64_t chunks) {
+  // chunk = kCopyUnroll * kThreads lanes * 16 bytes
   for (int64_t c = blockIdx.x; c < chunks; c += gridDim.x) {
-    const int64_t base = c * (kCopyUnroll * 256) + threadIdx.x;
+    const int64_t base = c * (kCopyUnroll * kThreads) + threadIdx.x;
     u32x4p v[kCopyUnroll];
 #pragma unroll
     for (int u = 0; u < kCopyUnroll; ++u)
-      v[u] = kNonTemporal ? __builtin_nontemporal_load(src + base + u * 256) : src[base + u * 256];
+      v[u] = kNonTemporal ? __builtin_nontemporal_load(src + base + u * kThreads) : src[base + u * kThreads];
 #pragma unroll
     for (int u = 0; u < kCopyUnroll; ++u) {
-      if (kNonTemporal) __builtin_nontemporal_store(v[u], dst + base + u * 256);
-      else dst[base + u * 256] = v[u];
+      if (kNonTemporal) __builtin_nontemporal_store(v[u], dst + base + u * kThreads);
+      else dst[base + u * kThreads] = v[u];
     }
   }
 }
@@ -80,19 +82,35 @@ __global__ __launch_bounds__(256) void copy_probe_kernel(const u32x4p* src, u32x
 // weights against a few activation rows) can reach. Every workgroup folds what
 // it reads into one word and stores it only if it has a value that the data
 // never produce in practice, so the loads stay and nothing is written.
-template <bool kNonTemporal>
-__global__ __launch_bounds__(256) void read_probe_kernel(const u32x4p* src, uint32_t* sink, int64_t chunks) {
+template <bool kNonTemporal, int kThreads, int kCopyUnroll>
+__global__ __launch_bounds__(kThreads) void read_probe_kernel(const u32x4p* src, uint32_t* sink, int64_t chunks) {
   uint32_t fold = 0;
   for (int64_t c = blockIdx.x; c < chunks; c += gridDim.x) {
-    const int64_t base = c * (kCopyUnroll * 256) + threadIdx.x;
+    const int64_t base = c * (kCopyUnroll * kThreads) + threadIdx.x;
     u32x4p v[kCopyUnroll];
 #pragma unroll
     for (int u = 0; u < kCopyUnroll; ++u)
-      v[u] = kNonTemporal ? __builtin_nontemporal_load(src + base + u * 256) : src[base + u * 256];
+      v[u] = kNonTemporal ? __builtin_nontemporal_load(src + base + u * kThreads) : src[base + u * kThreads];
 #pragma unroll
     for (int u = 0; u < kCopyUnroll; ++u) fold ^= v[u].x ^ (v[u].y * 3u) ^ (v[u].z * 5u) ^ (v[u].w * 7u);
   }
   if (fold == 0x9E3779B9u) sink[0] = fold;
+}
+
+template <int kThreads, int kCopyUnroll>
+int launch_copy_geometry(const void* src, void* dst, int64_t bytes, int mode, int blocks_per_cu, hipStream_t s) {
+  const int64_t chunks = bytes / ((int64_t)kCopyUnroll * kThreads * 16);
+  int64_t blocks = blocks_per_cu > 0 ? (int64_t)device_cu_count() * blocks_per_cu : chunks;
+  if (blocks > chunks) blocks = chunks;
+  if (blocks > 0x7FFFFFFF) blocks = 0x7FFFFFFF;
+  const dim3 g((unsigned)blocks), b(kThreads);
+  switch (mode & 3) {
+    case 0: hipLaunchKernelGGL((copy_probe_kernel<false, kThreads, kCopyUnroll>), g, b, 0, s, (const u32x4p*)src, (u32x4p*)dst, chunks); break;
+    case 1: hipLaunchKernelGGL((copy_probe_kernel<true, kThreads, kCopyUnroll>), g, b, 0, s, (const u32x4p*)src, (u32x4p*)dst, chunks); break;
+    case 2: hipLaunchKernelGGL((read_probe_kernel<false, kThreads, kCopyUnroll>), g, b, 0, s, (const u32x4p*)src, (uint32_t*)dst, chunks); break;
+    default: hipLaunchKernelGGL((read_probe_kernel<true, kThreads, kCopyUnroll>), g, b, 0, s, (const u32x4p*)src, (uint32_t*)dst, chunks); break;
+  }
+  return check_hip(hipGetLastError(), "copy_probe launch");
 }
 
 template <typename Cfg>
@@ -124,26 +142,15 @@ int launch_mfma_probe(uint32_t type_flag, const void* operands, int64_t iters, v
 }
 
 // bytes: a multiple of 8 KiB; mode 0 = plain accesses, 1 = non-temporal, 2 and
-// 3 = the same two without the stores (dst then needs 4 bytes only);
+// 3 = the same two without the stores (dst then needs 4 bytes only), + 4 = the
+// same in single-wave workgroups of 1 KiB per step;
 // blocks_per_cu workgroups per compute unit (0 = one workgroup per chunk).
 int launch_copy_probe(const void* src, void* dst, int64_t bytes, int mode, int blocks_per_cu, hipStream_t s) {
-  const int64_t chunk_bytes = (int64_t)kCopyUnroll * 256 * 16;
-  if (bytes <= 0 || bytes % chunk_bytes || ((uintptr_t)src | (uintptr_t)dst) % 16)
-    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "copy_probe: bytes must be whole chunks of %lld and buffers 16-byte aligned",
-                (long long)chunk_bytes);
-  const int64_t chunks = bytes / chunk_bytes;
-  int64_t blocks = blocks_per_cu > 0 ? (int64_t)device_cu_count() * blocks_per_cu : chunks;
-  if (blocks > chunks) blocks = chunks;
-  if (blocks > 0x7FFFFFFF) blocks = 0x7FFFFFFF;
-  if (mode == 2)
-    hipLaunchKernelGGL(read_probe_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, s, (const u32x4p*)src, (uint32_t*)dst, chunks);
-  else if (mode == 3)
-    hipLaunchKernelGGL(read_probe_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, s, (const u32x4p*)src, (uint32_t*)dst, chunks);
-  else if (mode == 1)
-    hipLaunchKernelGGL(copy_probe_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, s, (const u32x4p*)src, (u32x4p*)dst, chunks);
-  else
-    hipLaunchKernelGGL(copy_probe_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, s, (const u32x4p*)src, (u32x4p*)dst, chunks);
-  return check_hip(hipGetLastError(), "copy_probe launch");
+  if (bytes <= 0 || bytes % 8192 || ((uintptr_t)src | (uintptr_t)dst) % 16 || mode < 0 || mode > 7)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT,
+                "copy_probe: bytes must be whole chunks of 8192, buffers 16-byte aligned, mode 0..7");
+  if (mode & 4) return launch_copy_geometry<64, 1>(src, dst, bytes, mode, blocks_per_cu, s);
+  return launch_copy_geometry<256, 2>(src, dst, bytes, mode, blocks_per_cu, s);
 }
 
 }  // namespace uk

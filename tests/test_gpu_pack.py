@@ -140,17 +140,19 @@ def test_copy_and_read_probes(uk, cuda):
     import torch
     n = 8192 * 37
     src = torch.from_numpy(np.random.default_rng(5).integers(0, 256, n, dtype=np.uint8)).to(cuda)
-    for mode in (0, 1):
+    for mode in (0, 1, 4, 5):
         for bpc in (0, 2):
             dst = torch.zeros(n, dtype=torch.uint8, device=cuda)
             uk.copy_probe(src, dst, n, mode, bpc)
             torch.cuda.synchronize()
             assert torch.equal(src, dst)
     sink = torch.full((16,), 7, dtype=torch.int32, device=cuda)
-    for mode in (2, 3):
+    for mode in (2, 3, 6, 7):
         uk.copy_probe(src, sink, n, mode, 0)
         uk.copy_probe(src, sink, n, mode, 4)
     torch.cuda.synchronize()
     assert bool((sink == 7).all())
     with pytest.raises(uk.UkError):
         uk.copy_probe(src, sink, 8192 * 3 + 16, 0, 0)
+    with pytest.raises(uk.UkError):
+        uk.copy_probe(src, sink, n, 8, 0)
