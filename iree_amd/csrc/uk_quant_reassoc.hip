@@ -425,25 +425,39 @@ int launch_dequant_matmul_i4_reassoc(const void* x, const void* w, const void* s
     }
     return 0;
   }
-  // Everything else: the element-wise kernel on plain quantised activations.
-  const size_t q_bytes = ((size_t)M * K * 2 + 15) & ~(size_t)15;
-  const size_t t_bytes = (size_t)M * a.G * sizeof(float);
+  // Everything else: the element-wise kernel on plain quantised activations,
+  // in passes of as many rows as 64 MiB of scratch memory hold (the passes
+  // follow one another on the stream, so they can share the buffer).
+  const size_t row_bytes = (size_t)K * 2 + 2 * (size_t)a.G * sizeof(float) + 32;
+  int64_t pass_rows = (int64_t)(((size_t)64 << 20) / row_bytes);
+  if (pass_rows < 1) pass_rows = 1;
+  if (pass_rows > M) pass_rows = M;
+  const size_t q_bytes = ((size_t)pass_rows * K * 2 + 15) & ~(size_t)15;
+  const size_t t_bytes = (size_t)pass_rows * a.G * sizeof(float);
   ScratchLease lease(s, q_bytes + 2 * t_bytes);
   if (!lease.ptr()) return fail(8 /* RESOURCE_EXHAUSTED */, "dequant_matmul_i4: no scratch memory for the quantised activations");
   ReassocArgs r = {};
   r.q_plain = (int16_t*)lease.ptr();
   r.scale_plain = (float*)((char*)lease.ptr() + q_bytes);
-  r.sum_plain = r.scale_plain + (size_t)M * a.G;
-  hipLaunchKernelGGL(quantize_groups_i16_kernel, dim3(quantize_blocks(M, a.G)), dim3(256), 0, s, a.x, a.M,
-                     a.K, a.G, (int)group_size, 0, a.M, r);
-  UK_RETURN_IF_HIP(hipGetLastError());
-  const int64_t total = M * N;
-  int64_t blocks = ceil_div(total, 256);
-  const int64_t max_blocks = (int64_t)cus * 32;
-  if (blocks > max_blocks) blocks = max_blocks;
-  hipLaunchKernelGGL(dequant_matmul_i4_reassoc_generic_kernel, dim3((unsigned)blocks), dim3(256), 0, s, a, r,
-                     (int)group_size);
-  return check_hip(hipGetLastError(), "dequant_matmul_i4_reassoc_generic launch");
+  r.sum_plain = r.scale_plain + (size_t)pass_rows * a.G;
+  for (int64_t m0 = 0; m0 < M; m0 += pass_rows) {
+    const int rows = (int)(M - m0 < pass_rows ? M - m0 : pass_rows);
+    I4Args ap = a;
+    ap.x = a.x + (size_t)m0 * K;
+    ap.out = a.out + (size_t)m0 * N;
+    ap.M = rows;
+    hipLaunchKernelGGL(quantize_groups_i16_kernel, dim3(quantize_blocks(rows, a.G)), dim3(256), 0, s, ap.x, rows,
+                       a.K, a.G, (int)group_size, 0, rows, r);
+    UK_RETURN_IF_HIP(hipGetLastError());
+    const int64_t total = (int64_t)rows * N;
+    int64_t blocks = ceil_div(total, 256);
+    const int64_t max_blocks = (int64_t)cus * 32;
+    if (blocks > max_blocks) blocks = max_blocks;
+    hipLaunchKernelGGL(dequant_matmul_i4_reassoc_generic_kernel, dim3((unsigned)blocks), dim3(256), 0, s, ap, r,
+                       (int)group_size);
+    UK_RETURN_IF_HIP(hipGetLastError());
+  }
+  return 0;
 }
 
 }  // namespace uk
