@@ -75,6 +75,28 @@ __device__ __forceinline__ half8 dequant_dword(uint32_t w, half2v lo, half2v hi)
   return half8{r0.x, r0.y, r1.x, r1.y, r2.x, r2.y, r3.x, r3.y};
 }
 
+// The cheaper form, used where the register file has room for the group sums
+// of the activations: the nibbles go to the matrix cores as f16 SUBNORMALS.
+// w & 0x000F000F is the pair (n0, n4) * 2^-24 and w & 0x00F000F0 the pair
+// (n1, n5) * 16 * 2^-24 (v_mfma_f32_16x16x32_f16 takes subnormal inputs at full
+// precision, and a subnormal times an f16 is exact in f32), so 8 weights cost
+// one shift and four ANDs. The activations that meet the second kind are
+// divided by 16 beforehand (permute_x_for_subnormals), and the zero point
+// leaves the inner loop altogether: sum_k x (n - zp) = sum_k x n - zp sum_k x,
+// with the group sums of x taken once per workgroup.
+__device__ __forceinline__ half8 nibbles_as_subnormals(uint32_t w) {
+  union { uint32_t u[4]; half8 h; } r;
+  const uint32_t w8 = w >> 8;
+  r.u[0] = w & 0x000F000Fu;     // nibbles 0, 4
+  r.u[1] = w & 0x00F000F0u;     // nibbles 1, 5 (x16)
+  r.u[2] = w8 & 0x000F000Fu;    // nibbles 2, 6
+  r.u[3] = w8 & 0x00F000F0u;    // nibbles 3, 7 (x16)
+  return r.h;
+}
+// What the products of that operand have to be multiplied by.
+constexpr float kSubnormalUnit = 5.9604644775390625e-8f;      // 2^-24
+constexpr float kSubnormalRescale = 16777216.0f;              // 2^24
+
 // The two offsets for a packed uint4 zero point zp (0..15), as f16 pairs:
 // 1024 + zp = 0x6400 | zp and 64 + zp = 0x5400 | (zp << 4) (ulp 1/16 at 64).
 __device__ __forceinline__ uint32_t offset_lo_bits(uint32_t zp) { return 0x64006400u | zp | (zp << 16); }
@@ -90,6 +112,24 @@ __device__ __forceinline__ half8 permute_x(u32x4 v) {
   r.u[2] = __builtin_amdgcn_perm(v.w, v.y, 0x05040100);  // (h2, h6)
   r.u[3] = __builtin_amdgcn_perm(v.w, v.y, 0x07060302);  // (h3, h7)
   return r.h;
+}
+
+// The same, with the halves that meet nibbles held 16-fold (positions 2, 3, 6,
+// 7 of the permuted order) divided by 16: exact down to 2^-10, below that the
+// quotient is rounded to the subnormal grid (an absolute error of at most
+// 2^-25 per activation).
+__device__ __forceinline__ half8 permute_x_for_subnormals(u32x4 v) {
+  union { half8 h; half2v p[4]; } r;
+  r.h = permute_x(v);
+  const half2v sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
+  r.p[1] = r.p[1] * sixteenth;
+  r.p[3] = r.p[3] * sixteenth;
+  return r.h;
+}
+// The constant operand whose product with such activations is their plain sum.
+__device__ __forceinline__ half8 ones_for_subnormal_sums() {
+  return half8{(_Float16)1.f, (_Float16)1.f, (_Float16)16.f, (_Float16)16.f,
+               (_Float16)1.f, (_Float16)1.f, (_Float16)16.f, (_Float16)16.f};
 }
 
 // NB bytes (1 .. 16 naturally aligned, 32 aligned to 16) into NB/4 (at least 1) dwords.

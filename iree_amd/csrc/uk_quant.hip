@@ -64,6 +64,10 @@ __global__ __launch_bounds__(kThreads) void dequant_matmul_i4_kernel(I4Args a) {
   constexpr int SB = GW * 2;                 // bytes of scales per lane, tile and half
   constexpr int ZB = kZpU4 ? (GW >= 2 ? GW / 2 : 1) : GW * 2;
   constexpr int SW = (SB + 3) / 4, ZW = (ZB + 3) / 4;
+  // Nibbles as f16 subnormals and the zero point applied through the group sums
+  // of the activations (see nibbles_as_subnormals), where those sums fit the
+  // register file: up to 8 accumulators of 4 registers.
+  constexpr bool kSubnormal = GW * MH <= 8;
   __shared__ float partial[2][kWaves][2 * MH * 4][64];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -154,6 +158,16 @@ __global__ __launch_bounds__(kThreads) void dequant_matmul_i4_kernel(I4Args a) {
     }
   }
   half8 xf[MH][SP][4];
+  // (kSubnormal) the sum of the activations of row r (accumulator layout: every
+  // column the same) over group g of this wave's K slice; complete when the
+  // first tile reaches the end of the group, which is where it is used
+  floatx4 xsum[kSubnormal ? MH : 1][kSubnormal ? GW : 1];
+  if constexpr (kSubnormal) {
+#pragma unroll
+    for (int mh = 0; mh < MH; ++mh)
+#pragma unroll
+      for (int g = 0; g < GW; ++g) xsum[mh][g] = floatx4{0.f, 0.f, 0.f, 0.f};
+  }
 
   int parity = 0;
   // One tile; `first`: the workgroup's first, which turns each span of x into
@@ -180,14 +194,21 @@ __global__ __launch_bounds__(kThreads) void dequant_matmul_i4_kernel(I4Args a) {
           for (int q = 0; q < 4; ++q) {
             u32x4 v = xraw[mh][sp][q];
             if constexpr (MH != 1) { v.x &= keep; v.y &= keep; v.z &= keep; v.w &= keep; }
-            xf[mh][sp][q] = permute_x(v);
+            if constexpr (kSubnormal) {
+              xf[mh][sp][q] = permute_x_for_subnormals(v);
+              const int g = (sp * 128 + q * 32) >> L;
+              xsum[mh][g] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xf[mh][sp][q], ones_for_subnormal_sums(),
+                                                                  xsum[mh][g], 0, 0, 0);
+            } else {
+              xf[mh][sp][q] = permute_x(v);
+            }
           }
         }
       }
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
         const u32x4 wv = wreg[sp][h];
-        float sc = 0.f;
+        float sc = 0.f, zq = 0.f;
         union { uint32_t u; half2v h; } lo, hi, zf;
         lo.u = hi.u = zf.u = 0;
 #pragma unroll
@@ -200,10 +221,20 @@ __global__ __launch_bounds__(kThreads) void dequant_matmul_i4_kernel(I4Args a) {
             // decode the group's parameters
             const uint32_t sbits = (mt.s[h][g >> 1] >> ((g & 1) * 16)) & 0xFFFF;
             sc = __half2float(__ushort_as_half((uint16_t)sbits));
-            // Packed uint4 zero points fold into the offsets (1024 + zp and
-            // 64 + zp are exact). f16 zero points may carry a fraction, which
-            // such a sum would round away: they are subtracted in a second step.
-            if (kZpU4) {
+            if constexpr (kSubnormal) {
+              // the products come in units of 2^-24; zq = -zp in those units
+              sc *= kSubnormalRescale;
+              if (kZpU4) {
+                const uint32_t zb = (mt.z[h][g >> 3] >> ((g & 7) * 4 + mt.zsh[h])) & 0xF;
+                zq = -(float)zb * kSubnormalUnit;
+              } else {
+                const uint32_t zb = (mt.z[h][g >> 1] >> ((g & 1) * 16)) & 0xFFFF;
+                zq = -__half2float(__ushort_as_half((uint16_t)zb)) * kSubnormalUnit;
+              }
+            } else if (kZpU4) {
+              // Packed uint4 zero points fold into the offsets (1024 + zp and
+              // 64 + zp are exact). f16 zero points may carry a fraction, which
+              // such a sum would round away: they are subtracted in a second step.
               const uint32_t zb = (mt.z[h][g >> 3] >> ((g & 7) * 4 + mt.zsh[h])) & 0xF;
               lo.u = offset_lo_bits(zb);
               hi.u = offset_hi_bits(zb);
@@ -218,10 +249,15 @@ __global__ __launch_bounds__(kThreads) void dequant_matmul_i4_kernel(I4Args a) {
 #pragma unroll
             for (int mh = 0; mh < MH; ++mh) part[h][mh] = floatx4{0.f, 0.f, 0.f, 0.f};
           }
-          half8 wq = dequant_dword(wv[q], lo.h, hi.h);
-          if (!kZpU4) {
-            const half8 zsub2 = {zf.h.x, zf.h.x, zf.h.x, zf.h.x, zf.h.x, zf.h.x, zf.h.x, zf.h.x};
-            wq = wq - zsub2;
+          half8 wq;
+          if constexpr (kSubnormal) {
+            wq = nibbles_as_subnormals(wv[q]);
+          } else {
+            wq = dequant_dword(wv[q], lo.h, hi.h);
+            if (!kZpU4) {
+              const half8 zsub2 = {zf.h.x, zf.h.x, zf.h.x, zf.h.x, zf.h.x, zf.h.x, zf.h.x, zf.h.x};
+              wq = wq - zsub2;
+            }
           }
 #pragma unroll
           for (int mh = 0; mh < MH; ++mh)
@@ -230,7 +266,11 @@ __global__ __launch_bounds__(kThreads) void dequant_matmul_i4_kernel(I4Args a) {
 #pragma unroll
             for (int mh = 0; mh < MH; ++mh)
 #pragma unroll
-              for (int r = 0; r < 4; ++r) acc[h][mh][r] = __builtin_fmaf(part[h][mh][r], sc, acc[h][mh][r]);
+              for (int r = 0; r < 4; ++r) {
+                float p = part[h][mh][r];
+                if constexpr (kSubnormal) p = __builtin_fmaf(zq, xsum[mh][g][r], p);     // - zp * sum of x
+                acc[h][mh][r] = __builtin_fmaf(p, sc, acc[h][mh][r]);
+              }
           }
         }
         // The slab's registers are free: request the same slab of the next
