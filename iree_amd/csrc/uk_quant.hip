@@ -56,8 +56,23 @@ namespace {
 //            MFMAs in the tiled layout (MFMA q covers k = q*32 .. +32 of the
 //            span); in the row-major one that only holds for groups of 128
 //            and more, so smaller groups are served from tiled weights only.
-template <int KB, int MH, bool kZpU4, int kLog2Gs>
+//   kStageX  (16-row form, at most kStageRows rows) the wave fetches its K
+//            slice of the activations with one full-width load per KiB into
+//            LDS and takes its operand fragments from there. Fetching them
+//            straight into the operand layout costs 16 load instructions per
+//            wave whatever the number of rows, and the kernel's start is bound
+//            by the rate at which the texture path takes instructions (about
+//            16 cycles each, 8 waves): with one row the weights of the first
+//            tile are requested 0.9 us earlier this way.
+constexpr int kStageRows = 8;
+template <int KB>
+constexpr int stage_row_pitch() { return KB * 128 + 16; }      // bytes; the 16 spread the rows over the banks
+template <int KB>
+constexpr int stage_lds_bytes() { return kWaves * kStageRows * stage_row_pitch<KB>(); }
+
+template <int KB, int MH, bool kZpU4, int kLog2Gs, bool kStageX = false>
 __global__ __launch_bounds__(kThreads) void dequant_matmul_i4_kernel(I4Args a) {
+  static_assert(!kStageX || MH == 1, "staged activations: 16-row form only");
   constexpr int SP = KB / 2;                 // spans of 128 k per wave
   constexpr int L = kLog2Gs >= 9 ? 30 : kLog2Gs;
   constexpr int GW = ((KB * 64) >> L) > 0 ? ((KB * 64) >> L) : 1;   // groups per wave slice
@@ -123,7 +138,46 @@ __global__ __launch_bounds__(kThreads) void dequant_matmul_i4_kernel(I4Args a) {
   load_meta(nt < a.n_tiles ? nt : a.n_tiles - 1, meta_next);
   u32x4 xraw[MH][SP][4];
   u32x4 wreg[SP][2];
-  {
+  if constexpr (kStageX) {
+    extern __shared__ __attribute__((aligned(16))) char stage_all[];
+    constexpr int kPitch = stage_row_pitch<KB>();
+    constexpr int kLanesPerRow = KB * 8;                 // 16-byte chunks of a row's slice
+    char* stage = stage_all + wave * kStageRows * kPitch;
+    const int rows = a.M - a.m_base;                     // (the host chose this form for rows <= kStageRows)
+    const int cq = a.tiled ? 32 : 8, ckc = a.tiled ? 8 : 32;   // chunk strides in k
+    const __amdgpu_buffer_rsrc_t rsrc = tile_rsrc(nt);
+    // One direct-to-LDS load per row (lane l: bytes [16 l, 16 l + 16) of the
+    // row's slice), as many as there are rows, nothing waited for in between;
+    // then the first tile's weights; then the wait for the rows only (loads
+    // return in order: all but the weight loads issued since).
+    const __amdgpu_buffer_rsrc_t xsrc = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)(a.x + (size_t)a.m_base * a.K + k_slice), 0, 0x7FFFFFFF, 0x00020000);
+    if (lane < kLanesPerRow) {
+#pragma unroll 1
+      for (int r = 0; r < rows; ++r)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(xsrc, (__attribute__((address_space(3))) void*)(stage + r * kPitch), 16,
+                                                 lane * 16, r * a.K * 2, 0, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int sp = 0; sp < SP; ++sp)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) wreg[sp][h] = load_slab(rsrc, sp, h);
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(SP * 2) : "memory");
+    // (the wave reads only what it loaded itself: no barrier)
+#pragma unroll
+    for (int sp = 0; sp < SP; ++sp)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) xraw[0][sp][q] = u32x4{0u, 0u, 0u, 0u};
+    if (nl < rows) {
+#pragma unroll
+      for (int sp = 0; sp < SP; ++sp)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          xraw[0][sp][q] = *(const u32x4*)(stage + nl * kPitch + (sp * 128 + q * cq + kc * ckc) * 2);
+    }
+  } else {
     const int cq = a.tiled ? 32 : 8, ckc = a.tiled ? 8 : 32;   // chunk strides in k
     const __amdgpu_buffer_rsrc_t rsrc = tile_rsrc(nt);
 #pragma unroll
@@ -356,15 +410,32 @@ __global__ __launch_bounds__(256) void dequant_matmul_i4_generic_kernel(I4Args a
   }
 }
 
-template <int KB, int MH, bool kZpU4>
-void launch_one(const I4Args& a, int blocks, hipStream_t s) {
-  const dim3 g(blocks), b(kThreads);
+template <int KB, int MH, bool kZpU4, int kLog2Gs, bool kStageX>
+int launch_instance(const I4Args& a, int blocks, hipStream_t s) {
+  void (*kernel)(I4Args) = dequant_matmul_i4_kernel<KB, MH, kZpU4, kLog2Gs, kStageX>;
+  const size_t lds = kStageX ? stage_lds_bytes<KB>() : 0;
+  if (kStageX) {
+    // (with the kernel's static 32 KiB this is more than the 64 KiB a kernel gets by default)
+    static unsigned long long attr_set_on = 0;
+    int dev = 0;
+    UK_RETURN_IF_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= 64 || !((attr_set_on >> dev) & 1)) {
+      UK_RETURN_IF_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+      if (dev >= 0 && dev < 64) attr_set_on |= 1ull << dev;
+    }
+  }
+  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kThreads), lds, s, a);
+  return check_hip(hipGetLastError(), "dequant_matmul_i4 launch");
+}
+
+template <int KB, int MH, bool kZpU4, bool kStageX = false>
+int launch_one(const I4Args& a, int blocks, hipStream_t s) {
   switch (a.log2_gs) {
-    case 5: hipLaunchKernelGGL((dequant_matmul_i4_kernel<KB, MH, kZpU4, 5>), g, b, 0, s, a); break;
-    case 6: hipLaunchKernelGGL((dequant_matmul_i4_kernel<KB, MH, kZpU4, 6>), g, b, 0, s, a); break;
-    case 7: hipLaunchKernelGGL((dequant_matmul_i4_kernel<KB, MH, kZpU4, 7>), g, b, 0, s, a); break;
-    case 8: hipLaunchKernelGGL((dequant_matmul_i4_kernel<KB, MH, kZpU4, 8>), g, b, 0, s, a); break;
-    default: hipLaunchKernelGGL((dequant_matmul_i4_kernel<KB, MH, kZpU4, 9>), g, b, 0, s, a); break;
+    case 5: return launch_instance<KB, MH, kZpU4, 5, kStageX>(a, blocks, s);
+    case 6: return launch_instance<KB, MH, kZpU4, 6, kStageX>(a, blocks, s);
+    case 7: return launch_instance<KB, MH, kZpU4, 7, kStageX>(a, blocks, s);
+    case 8: return launch_instance<KB, MH, kZpU4, 8, kStageX>(a, blocks, s);
+    default: return launch_instance<KB, MH, kZpU4, 9, kStageX>(a, blocks, s);
   }
 }
 
@@ -377,14 +448,18 @@ int launch_fast(I4Args a, hipStream_t s) {
     // One workgroup per compute unit (two of the 16-row kernel would fit, and
     // measure slower: 12.4 against 9.9 us on the decode shape).
     const int blocks = a.n_tiles < cus ? a.n_tiles : cus;
+    int st;
     if (a.M - m_base > 16) {
-      if (a.zp_u4) launch_one<KB, 2, true>(a, blocks, s); else launch_one<KB, 2, false>(a, blocks, s);
+      st = a.zp_u4 ? launch_one<KB, 2, true>(a, blocks, s) : launch_one<KB, 2, false>(a, blocks, s);
       m_base += 32;
+    } else if (a.M - m_base <= kStageRows) {
+      st = a.zp_u4 ? launch_one<KB, 1, true, true>(a, blocks, s) : launch_one<KB, 1, false, true>(a, blocks, s);
+      m_base += 16;
     } else {
-      if (a.zp_u4) launch_one<KB, 1, true>(a, blocks, s); else launch_one<KB, 1, false>(a, blocks, s);
+      st = a.zp_u4 ? launch_one<KB, 1, true>(a, blocks, s) : launch_one<KB, 1, false>(a, blocks, s);
       m_base += 16;
     }
-    UK_RETURN_IF_HIP(hipGetLastError());
+    UK_RETURN_IF_ERROR(st);
   }
   return 0;
 }
