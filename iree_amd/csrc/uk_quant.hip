@@ -20,14 +20,18 @@
 //     workgroup each own one eighth of K and hold their slice of x as MFMA A
 //     operands for the whole kernel, so no LDS or cache bandwidth is spent on
 //     re-reading x (which would be 4 bytes per weight byte);
-//   * dequantises in registers ahead of the MFMA: a nibble n becomes the f16
-//     value 1024+n (or 1024+16n for the upper nibble of a byte, no shift
-//     needed) by OR-ing it into the mantissa of 0x6400, the offset and the zero
-//     point are removed with exact packed-f16 arithmetic, the small integers
-//     go through v_mfma_f32_16x16x32_f16 (products are exact), and the
-//     per-group f32 partial sums are scaled by s[n][g] with one f32 FMA per
-//     accumulator register (the lane owns column n, so the scale is a
-//     per-lane scalar);
+//   * dequantises in registers ahead of the MFMA with as few vector
+//     instructions as the format allows, because the tile loop is bound by
+//     them: the nibbles go to v_mfma_f32_16x16x32_f16 as f16 subnormals (one
+//     shift and four ANDs per 8 weights, every product exact in f32), the zero
+//     point is applied through per-group sums of the activations that the
+//     matrix cores take once per workgroup, and the per-group f32 partial sums
+//     are scaled by s[n][g] with one f32 FMA per accumulator register (the lane
+//     owns column n, so scale and zero point are per-lane scalars). Instances
+//     without register room for the group sums turn a nibble n into the f16
+//     value 1024+n (or 1024+16n for the upper nibble of a byte) by OR-ing it
+//     into the mantissa of 0x6400 and remove offset and zero point with exact
+//     packed-f16 arithmetic;
 //   * sums the 8 K-slices through LDS in a fixed order (deterministic).
 #include "uk_common.h"
 #include "uk_fp8.h"
