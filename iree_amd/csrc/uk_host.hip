@@ -191,7 +191,7 @@ class SlotLease {
       std::lock_guard<std::mutex> lock(pool_->mutex);
       slot_->busy = false;
     }
-    pool_->freed.notify_one();
+    pool_->freed.notify_all();     // (waiters may be after slots of different devices)
   }
   int acquire() {
     int device = 0;
