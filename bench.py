@@ -446,6 +446,13 @@ def extras(args, torch, iree_amd, F, synth, lhs, rhs, out, ex):
     _, t = gpu_time(torch, lambda: iree_amd.mmt4d(li, ri, oi, M1, N1, K1, 32, 32, 16, F.MMT4D_TYPE_S8S8S32),
                     steps, warm)
     ex["mmt4d_i8_tops"] = round(flops / t / 1e12, 2)
+    # the same problem with a signed 4-bit right-hand side (S8S4S32): widened
+    # to int8 in scratch memory, then the kernel above; two launches per call
+    r4 = torch.from_numpy(synth.uniform_u4_packed(3, N1 * K1 * 32 * 16)).cuda()
+    _, t = gpu_time(torch, lambda: iree_amd.mmt4d(li, r4, oi, M1, N1, K1, 32, 32, 16, F.MMT4D_TYPE_S8S4S32),
+                    steps, warm)
+    ex["mmt4d_s8s4_tops"] = round(flops / t / 1e12, 2)
+    del r4
     ex["mmt4d_i8_frac_of_peak"] = round(flops / t / 1e12 / PEAK_I8_TOPS, 4)
     del li, ri, oi
 

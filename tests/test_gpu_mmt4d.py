@@ -100,6 +100,30 @@ def test_mfma_macro_tile_variants_bit_exact(uk, cuda, type_flag, K0, M, N):
         assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), (hex(type_flag), M, N, K, acc)
 
 
+@pytest.mark.parametrize("K0", [16, 32])
+def test_s8s4_on_the_matrix_cores_bit_exact(uk, cuda, K0):
+    """S8S4S32 (signed 4-bit right-hand side, mmt4d_tile_generic.c:81-142) at the
+    gfx950 tiles: the library widens the right-hand side to int8 in scratch
+    memory and runs the s8 x s8 matrix-core kernels; mmt4d_info reports an
+    architecture tile and the generic fallback is NOT allowed in these calls.
+    Bits of the oracle for macro-tile and narrow shapes, accumulate, a partial
+    last K step, loose strides; operands the widening pass cannot take (an odd
+    element offset into the packed nibbles) go through the element-wise kernel
+    with the same bits."""
+    tf = F.MMT4D_TYPE_S8S4S32
+    rng = np.random.default_rng(9100 + K0)
+    assert uk.mmt4d_info(32, 32, K0, tf) == 1
+    assert uk.mmt4d_info(8, 32, K0, tf) == 1
+    assert uk.mmt4d_info(16, 16, 2, tf) == 0
+    for M0, M, N, K, acc in ((32, 3, 5, 7, False), (32, 16, 9, 12, True), (32, 64, 64, 5, False),
+                             (8, 1, 300, 26, True), (1, 1, 40, 64, False)):
+        case = ukref.Mmt4dCase(rng, tf, M, N, K, M0, 32, K0, accumulate=acc)
+        got = gpucase.run_mmt4d(case, flags=case.flags & ~F.MMT4D_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION)
+        assert np.array_equal(got, case.run_oracle()), (M0, M, N, K, acc)
+    case = ukref.Mmt4dCase(rng, tf, 5, 6, 9, 32, 32, K0, accumulate=True, loose_strides=True, offsets=True)
+    assert np.array_equal(gpucase.run_mmt4d(case), case.run_oracle())
+
+
 @pytest.mark.parametrize("type_flag,K0", [(F.MMT4D_TYPE_F16F16F32, 8), (F.MMT4D_TYPE_F16F16F32, 16),
                                           (F.MMT4D_TYPE_BF16BF16F32, 8), (F.MMT4D_TYPE_S8S8S32, 16),
                                           (F.MMT4D_TYPE_S8S8S32, 32), (F.MMT4D_TYPE_F32F32F32, 4),
