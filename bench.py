@@ -61,7 +61,7 @@ def parse_args():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--only", default="", help="run only the named kernel in a loop (for profilers): "
                     "mmt4d_f16 | mmt4d_f16_acc | mmt4d_i8 | mmt4d_fp8 | mmt4d_f16_ksplit | mlp_fp8 | pack | unpack | "
-                    "pack_transpose | dequant_i4[_m8|_m32] | dequant_i4_reassoc[_m8|_m32] | batch_mmt4d_f16 | "
+                    "pack_transpose | unpack_transpose | dequant_i4[_m8|_m32] | dequant_i4_reassoc[_m8|_m32] | batch_mmt4d_f16 | "
                     "batch_mmt4d_f16_narrow | mmt4d_f16_narrow_m1 | mmt4d_f16_narrow_m8 | mmt4d_f16_narrow_n8 | "
                     "chain_i8_1024 | copy | copy_rotating | copy_rotating_nt | copy_rotating_nt_single_waves | read_only_29mb")
     return ap.parse_args()
@@ -844,6 +844,18 @@ def run_only(args, torch, iree_amd, F, synth, mm_step):
             st["i"] += 1
             iree_amd.pack(b, pb[k], size, size, size // 32, size // 8, 32, 8, 0,
                           F.PACK_TYPE_F16F16 | F.PACK_TRANSPOSE_INNER | F.PACK_TRANSPOSE_OUTER)
+    elif args.only == "unpack_transpose":
+        # a 4096 x 4096 f32 result held as 32x32 tiles stored column by column (inner transposed)
+        size = 4096
+        tiles = torch.from_numpy(synth.normal_f32(3, size * size, 1.0)).cuda()
+        mats = [torch.empty(size * size, dtype=torch.float32, device="cuda") for _ in range(4)]
+        st = {"i": 0}
+
+        def fn():
+            k = st["i"] % 4
+            st["i"] += 1
+            iree_amd.unpack(tiles, mats[k], size // 32, size // 32, 32, 32, size, size,
+                            F.UNPACK_TYPE_F32F32 | F.UNPACK_TRANSPOSE_INNER)
     elif args.only == "mlp_fp8":
         mlp, xm, ym, Mt, _, _ = make_fp8_mlp(torch, iree_amd)
         fn = lambda: mlp(xm, ym, Mt)  # noqa: E731

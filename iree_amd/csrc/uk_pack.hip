@@ -397,6 +397,73 @@ __global__ __launch_bounds__(256) void pack_transpose_kernel(TransArgs a) {
   }
 }
 
+// The reverse: unpack of tiles stored column by column (the transposed result
+// tiles of a matmul whose narrow dimension was exchanged, reference
+// unpack.c:190-247). One thread takes one 16-byte chunk of the tiled buffer
+// (CE consecutive matrix rows of one column) and stores its CE elements; the
+// lanes of a wave hold 64 consecutive columns, so every store instruction
+// writes 64 consecutive elements of a matrix row. Same block walk as the pack.
+template <int ES>
+__global__ __launch_bounds__(256) void unpack_transpose_kernel(TransArgs a) {
+  constexpr int CE = 16 / ES;
+  typedef typename Chunk<ES>::elem_t elem_t;
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  uint32_t bx, by;
+  {
+    constexpr uint32_t kXcds = 8;
+    const uint32_t total = a.blocks_x * a.blocks_y;
+    const uint32_t per = total / kXcds, rem = total % kXcds;
+    const uint32_t xcd = blockIdx.x % kXcds, idx = blockIdx.x / kXcds;
+    const uint32_t logical = xcd * per + (xcd < rem ? xcd : rem) + idx;
+    by = logical / a.blocks_x;
+    bx = logical - by * a.blocks_x;
+  }
+  const int64_t c = (int64_t)bx * 64 + lane;                 // matrix column
+  const int64_t g0 = ((int64_t)by * 4 + wave) * kTransUnroll;  // first row group of this wave
+  if (g0 >= a.row_groups || c >= a.m_size1 || c >= a.padded_cols) return;
+  const uint32_t cc = (uint32_t)c;
+  const uint32_t ocol = a.by_tile_cols.div(cc), d2 = cc - ocol * a.tile_cols;
+  const char* in_col = a.tiled + (int64_t)ocol * a.t_stride_ocol_bytes + (int64_t)d2 * a.tile_rows * ES;
+  union { elem_t e[CE]; u32x4 vec; } chunk[kTransUnroll];
+#pragma unroll
+  for (int u = 0; u < kTransUnroll; ++u) {
+    const int64_t g = g0 + u;
+    chunk[u].vec = u32x4{0u, 0u, 0u, 0u};
+    if (g < a.row_groups) {
+      int64_t orow;
+      uint32_t grp;
+      if (g < 0x7FFFFFFF) {
+        orow = a.by_groups.div((uint32_t)g);
+        grp = (uint32_t)g - (uint32_t)orow * a.groups_per_tile;
+      } else {
+        orow = g / a.groups_per_tile;
+        grp = (uint32_t)(g - orow * a.groups_per_tile);
+      }
+      chunk[u].vec = *(const u32x4*)(in_col + orow * a.t_stride_orow_bytes + (int64_t)grp * 16);
+    }
+  }
+  char* dst = (char*)a.mat + c * ES;
+#pragma unroll
+  for (int u = 0; u < kTransUnroll; ++u)
+#pragma unroll
+    for (int i = 0; i < CE; ++i) {
+      const int64_t r = (g0 + u) * CE + i;
+      if (r < a.m_size0) *(elem_t*)(dst + r * a.m_pitch_bytes) = chunk[u].e[i];
+    }
+}
+
+template <int ES>
+int launch_unpack_transpose(TransArgs a, hipStream_t s) {
+  const int64_t cols = a.m_size1 < a.padded_cols ? a.m_size1 : a.padded_cols;
+  const int64_t bx = ceil_div(cols, (int64_t)64);
+  const int64_t by = ceil_div(a.row_groups, (int64_t)(4 * kTransUnroll));
+  if (bx < 1 || by < 1 || bx * by > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  a.blocks_x = (uint32_t)bx; a.blocks_y = (uint32_t)by;
+  hipLaunchKernelGGL((unpack_transpose_kernel<ES>), dim3((unsigned)(bx * by)), dim3(256), 0, s, a);
+  return check_hip(hipGetLastError(), "unpack_transpose launch");
+}
+
 template <int ES>
 int launch_pack_transpose(TransArgs a, hipStream_t s) {
   const int64_t bx = ceil_div(a.padded_cols, (int64_t)64);
@@ -572,6 +639,30 @@ int launch_unpack(const iree_amd_uk_unpack_params_t& p, hipStream_t s) {
     a.padding = 0;
     fill_stream_geometry(&a, es);
     int st = es == 2 ? launch_unpack_stream<2>(a, s) : launch_unpack_stream<4>(a, s);
+    if (st != IREE_AMD_UK_STATUS_NOT_FOUND) return st;
+  }
+
+  // Transposed inner tiles whose stored rows are whole 16-byte chunks.
+  const int ce = 16 / es;
+  if (ti && p.out_stride1 == 1 && p.in_size3 > 0 && p.in_size3 % ce == 0 && p.in_size2 > 0 &&
+      ((uintptr_t)tiled % 16) == 0 && (p.in_stride0 * es) % 16 == 0 && (tile_elems * es) % 16 == 0 &&
+      p.out_size1 < (1ll << 31) && (to ? p.in_size0 : p.in_size1) * p.in_size2 < (1ll << 31)) {
+    TransArgs a;
+    a.mat = mat; a.tiled = (char*)tiled;
+    a.m_size0 = p.out_size0; a.m_size1 = p.out_size1; a.m_pitch_bytes = p.out_stride0 * es;
+    a.tile_rows = (int)p.in_size3; a.tile_cols = (int)p.in_size2;
+    a.groups_per_tile = a.tile_rows / ce;
+    const int64_t outer_rows = to ? p.in_size1 : p.in_size0;
+    const int64_t outer_cols = to ? p.in_size0 : p.in_size1;
+    a.row_groups = outer_rows * a.groups_per_tile;
+    a.padded_cols = outer_cols * a.tile_cols;
+    a.t_stride_orow_bytes = (to ? tile_elems : p.in_stride0) * es;
+    a.t_stride_ocol_bytes = (to ? p.in_stride0 : tile_elems) * es;
+    a.by_tile_cols = make_fastdiv((uint32_t)a.tile_cols);
+    a.by_groups = make_fastdiv((uint32_t)a.groups_per_tile);
+    a.padding = 0;
+    a.blocks_x = a.blocks_y = 0;
+    int st = es == 2 ? launch_unpack_transpose<2>(a, s) : launch_unpack_transpose<4>(a, s);
     if (st != IREE_AMD_UK_STATUS_NOT_FOUND) return st;
   }
 

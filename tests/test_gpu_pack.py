@@ -98,6 +98,29 @@ def test_transposing_pack_with_ragged_edges(uk, cuda, type_flag, tr, tc, rows, c
         assert np.array_equal(gpucase.run_pack(loose), loose.run_oracle()), (to, "loose")
 
 
+@pytest.mark.parametrize("type_flag,tr,tc,rows,cols", [
+    (F.UNPACK_TYPE_F32F32, 32, 32, 333, 1001),
+    (F.UNPACK_TYPE_I32I32, 32, 8, 95, 257),      # the transposed result tiles of a narrow matmul
+    (F.UNPACK_TYPE_F16F16, 16, 32, 129, 1003),
+    (F.UNPACK_TYPE_BF16BF16, 24, 5, 123, 77),    # odd tile width, three row groups
+    (F.UNPACK_TYPE_F32F32, 8, 32, 4096, 70),
+])
+def test_transposing_unpack_with_ragged_edges(uk, cuda, type_flag, tr, tc, rows, cols):
+    """Unpacks of tiles stored column by column (matrix tiles of tr rows x tc
+    columns): the fast kernel for whole 16-byte stored rows; the whole
+    destination buffer is compared, so nothing outside the matrix is touched."""
+    rng = np.random.default_rng(rows * 3 + cols)
+    orows, ocols = -(-rows // tr), -(-cols // tc)
+    for to in (0, 1):
+        case = ukref.UnpackCase(rng, type_flag, orows, ocols, tr, tc, transpose_inner=1,
+                                transpose_outer=to, out_size=(rows, cols))
+        assert np.array_equal(gpucase.run_unpack(case), case.run_oracle()), (to,)
+        loose = ukref.UnpackCase(rng, type_flag, orows, ocols, tr, tc, transpose_inner=1,
+                                 transpose_outer=to, out_size=(rows, cols), loose_strides=True,
+                                 offsets=True)
+        assert np.array_equal(gpucase.run_unpack(loose), loose.run_oracle()), (to, "loose")
+
+
 def test_full_size_f16_8191x5001_pack_unpack_round_trip(uk, cuda):
     """The bandwidth workload at its real size: packed bytes equal the oracle's
     (and the committed SHA-256 produced by the reference library), the padded
