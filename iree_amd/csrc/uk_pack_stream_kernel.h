@@ -58,21 +58,23 @@ struct Pow2Args {
   uint64_t padding;
 };
 
-// Non-temporal accesses on the TILED side only (measured on MI355X, f16
-// 8191 x 5001 <-> 32x16 tiles): its pieces are whole 256-byte runs that nobody
-// else touches, and streaming them past the caches gives pack 5.25 instead of
-// 4.95 TB/s and unpack 4.76 instead of 4.69. On the matrix side they lose:
-// its 128-byte row segments share cache lines with the neighbouring waves
-// (non-temporal loads: pack 4.5 TB/s) and are pieces of DRAM pages that
-// non-temporal stores no longer merge (unpack 3.0 TB/s). A plain copy with
-// 8 KiB runs on both sides reaches 5.3-5.5 TB/s with ordinary and 6.0-6.2 with
-// non-temporal accesses on the same machine. Staging 32 rows x 1 KiB per
+// Non-temporal accesses (measured on MI355X, f16 8191 x 5001 <-> 32x16 tiles).
+// The tiled side's pieces are whole runs that nobody else touches: streaming
+// them past the caches always pays (pack stores, unpack loads). On the matrix
+// side it depends on the length of the row pieces. With 256-byte pieces (the
+// library's block shape) non-temporal LOADS pay too (pack 5.65 -> 5.82 TB/s),
+// non-temporal STORES still lose (unpack 5.41 -> 5.22: pieces of DRAM pages
+// that are no longer merged); with the earlier 128-byte pieces, which share
+// both their cache lines with neighbouring waves, the loads lost as well (pack
+// 5.25 -> 4.5) and the stores were ruinous (unpack 4.76 -> 3.0). A plain copy
+// with 8 KiB runs on both sides reaches 5.3-5.5 TB/s with ordinary and 6.0-6.4
+// with non-temporal accesses on the same machine. Staging 32 rows x 1 KiB per
 // workgroup through LDS, so that every wave instruction moves 1 KiB of one
 // matrix row or of consecutive tile memory, was slower in all four
 // combinations of non-temporal sides (pack 4.4-5.0, unpack 4.2-4.5 TB/s):
 // longer runs per instruction do not pay for the barrier and the fewer, larger
 // workgroups.
-template <int ES, bool kPack, bool kNtLoad = !kPack, bool kNtStore = kPack, int kBlockRows = kPow2Rows,
+template <int ES, bool kPack, bool kNtLoad = true, bool kNtStore = kPack, int kBlockRows = kPow2Rows,
           int kStreamUnroll = kPow2Unroll, int kWX = kPow2WavesX, int kWaves = kPow2Waves>
 __device__ __forceinline__ void stream_pow2_body(const Pow2Args a) {
   constexpr int CE = 16 / ES;

@@ -189,7 +189,7 @@ __device__ __forceinline__ void hal_pack(const void* mat, void* tiled, int size0
   if (blockIdx.x >= a.blocks_x * a.blocks_y) return;
   // (blocks of 16 rows x 32 chunks per 256 threads, as the export's workgroup
   // count says: 2 x 2 waves of 2 blocks of 4 rows x 16 chunks)
-  stream_pow2_body<ES, kPack, !kPack, kPack, 4, 2, 2, 4>(a);
+  stream_pow2_body<ES, kPack, true, kPack, 4, 2, 2, 4>(a);
 }
 
 }  // namespace
