@@ -170,14 +170,15 @@ def test_every_tile_the_query_returns_has_an_architecture_kernel():
             for n in sizes:
                 m0, n0 = q(op | F.QUERY_ROLE_RESULT, m, n)
                 assert m0 == 32 or n0 == 32, (m, n, m0, n0)
-                # the operand queries a caller makes for this matmul: the wider
-                # of two narrow dimensions is passed as dynamic
-                m_arg = m if m0 < 32 or n0 == 32 else dyn
-                n_arg = n if n0 < 32 or m0 == 32 else dyn
-                if m0 < 32:
-                    n_arg = dyn if 0 < n < 32 else n
-                if n0 < 32:
-                    m_arg = dyn if 0 < m < 32 else m
+                # The operand queries a caller makes for this matmul. Only one
+                # dimension is narrowed; a caller passes the other one, when it
+                # is below 32 too, as dynamic, so that its operand keeps the
+                # full tile.
+                m_arg, n_arg = m, n
+                if m0 < 32 and 0 < n < 32:
+                    n_arg = dyn
+                if n0 < 32 and 0 < m < 32:
+                    m_arg = dyn
                 lm0, k0 = q(op | F.QUERY_ROLE_LHS, m_arg, 4096)
                 rn0, rk0 = q(op | F.QUERY_ROLE_RHS, n_arg, 4096)
                 assert (lm0, rn0, rk0) == (m0, n0, k0), (m, n)
