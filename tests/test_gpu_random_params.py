@@ -1,0 +1,82 @@
+"""Seeded random sweeps over the parameter space of the three ukernels: every
+type tuple, the gfx950 tiles (full, narrow on either side) and arbitrary small
+tiles, ragged outer sizes, accumulate, loose strides and offsets, both
+transposes of pack / unpack and every padding regime. Each case is compared
+with the oracle bit for bit (the operands follow the reference's own test
+generator, tools/util.c:122-168: small integers for the float types, so every
+kernel the dispatcher may choose gives the same bits)."""
+import numpy as np
+import pytest
+
+import gpucase
+import ukref
+from iree_amd import flags as F
+
+pytestmark = pytest.mark.gpu
+
+MMT4D_TYPES = [F.MMT4D_TYPE_F32F32F32, F.MMT4D_TYPE_S8S8S32, F.MMT4D_TYPE_F16F16F32, F.MMT4D_TYPE_F16F16F16,
+               F.MMT4D_TYPE_BF16BF16F32, F.MMT4D_TYPE_BF16BF16BF16, F.MMT4D_TYPE_S16S16S32,
+               F.MMT4D_TYPE_S16U4S32, F.MMT4D_TYPE_S16S8S32, F.MMT4D_TYPE_S8S4S32,
+               F.MMT4D_TYPE_F8E4M3F8E4M3F32]
+# K0 values that make a packed tile row 16 bytes (and twice that) per type
+ARCH_K0 = {F.MMT4D_TYPE_F32F32F32: (4,), F.MMT4D_TYPE_S8S8S32: (16, 32), F.MMT4D_TYPE_F16F16F32: (8, 16),
+           F.MMT4D_TYPE_F16F16F16: (8, 16), F.MMT4D_TYPE_BF16BF16F32: (8, 16), F.MMT4D_TYPE_BF16BF16BF16: (8, 16),
+           F.MMT4D_TYPE_S16S16S32: (8,), F.MMT4D_TYPE_S16U4S32: (8,), F.MMT4D_TYPE_S16S8S32: (8,),
+           F.MMT4D_TYPE_S8S4S32: (16, 32), F.MMT4D_TYPE_F8E4M3F8E4M3F32: (16,)}
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_mmt4d_calls_bit_exact(uk, cuda, seed):
+    rng = np.random.default_rng(424200 + seed)
+    for _ in range(150):
+        tf = MMT4D_TYPES[int(rng.integers(0, len(MMT4D_TYPES)))]
+        shape = int(rng.integers(0, 4))
+        if shape == 0:       # the full gfx950 tile
+            M0, N0, K0 = 32, 32, int(rng.choice(ARCH_K0[tf]))
+        elif shape == 1:     # narrow left-hand side
+            M0, N0, K0 = int(rng.choice([1, 2, 4, 8, 16])), 32, int(rng.choice(ARCH_K0[tf]))
+        elif shape == 2:     # narrow right-hand side
+            M0, N0, K0 = 32, int(rng.choice([1, 2, 4, 8, 16])), int(rng.choice(ARCH_K0[tf]))
+        else:                # anything small (even K0 for the 4-bit operands)
+            M0, N0 = int(rng.integers(1, 9)), int(rng.integers(1, 9))
+            K0 = int(rng.integers(1, 5)) * (2 if tf in (F.MMT4D_TYPE_S16U4S32, F.MMT4D_TYPE_S8S4S32) else 1)
+        narrow = shape in (1, 2)
+        M = 1 if shape == 1 and rng.integers(0, 4) else int(rng.integers(1, 7))
+        N = 1 if shape == 2 and rng.integers(0, 4) else int(rng.integers(1, 40 if narrow else 7))
+        K = int(rng.integers(1, 70 if narrow else 20))
+        loose = bool(rng.integers(0, 3) == 0)
+        case = ukref.Mmt4dCase(rng, tf, M, N, K, M0, N0, K0, accumulate=bool(rng.integers(0, 2)),
+                               loose_strides=loose, offsets=loose and bool(rng.integers(0, 2)))
+        got = gpucase.run_mmt4d(case)
+        want = case.run_oracle(ukref.F16_IEEE)
+        assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), \
+            (seed, hex(tf), M, N, K, M0, N0, K0, case.flags, loose)
+
+
+PACK_TYPES = [F.PACK_TYPE_F32F32, F.PACK_TYPE_I8I8, F.PACK_TYPE_I32I32, F.PACK_TYPE_F16F16, F.PACK_TYPE_BF16BF16]
+UNPACK_TYPES = [F.UNPACK_TYPE_F32F32, F.UNPACK_TYPE_I32I32, F.UNPACK_TYPE_F16F16, F.UNPACK_TYPE_BF16BF16]
+PADS = ["none", "one_incomplete_tile", "a_lot"]
+
+
+def _random_tile(rng):
+    if rng.integers(0, 2):
+        return int(rng.choice([1, 2, 4, 8, 16, 32])), int(rng.choice([4, 8, 16, 32, 64]))
+    return int(rng.integers(1, 20)), int(rng.integers(1, 20))
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_pack_and_unpack_calls_bit_exact(uk, cuda, seed):
+    rng = np.random.default_rng(515100 + seed)
+    for _ in range(150):
+        t0, t1 = _random_tile(rng)
+        o0, o1 = int(rng.integers(1, 12)), int(rng.integers(1, 40))
+        loose = bool(rng.integers(0, 3) == 0)
+        kw = dict(transpose_inner=int(rng.integers(0, 2)), transpose_outer=int(rng.integers(0, 2)),
+                  pad=PADS[int(rng.integers(0, 3))], loose_strides=loose, offsets=loose and bool(rng.integers(0, 2)))
+        pc = ukref.PackCase(rng, PACK_TYPES[int(rng.integers(0, 5))], o0, o1, t0, t1,
+                            in_stride1=1 + int(rng.integers(0, 6) == 0), **kw)
+        assert np.array_equal(gpucase.run_pack(pc), pc.run_oracle()), (seed, "pack", o0, o1, t0, t1, kw)
+        uc = ukref.UnpackCase(rng, UNPACK_TYPES[int(rng.integers(0, 4))], o0, o1, t0, t1,
+                              out_stride1=1 + int(rng.integers(0, 6) == 0), **kw)
+        # (the whole destination buffer is compared: nothing outside the matrix may change)
+        assert np.array_equal(gpucase.run_unpack(uc), uc.run_oracle()), (seed, "unpack", o0, o1, t0, t1, kw)
