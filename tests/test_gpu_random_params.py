@@ -80,3 +80,25 @@ def test_random_pack_and_unpack_calls_bit_exact(uk, cuda, seed):
                               out_stride1=1 + int(rng.integers(0, 6) == 0), **kw)
         # (the whole destination buffer is compared: nothing outside the matrix may change)
         assert np.array_equal(gpucase.run_unpack(uc), uc.run_oracle()), (seed, "unpack", o0, o1, t0, t1, kw)
+
+
+@pytest.mark.parametrize("seed", range(3))
+def test_random_int4_dequant_matmul_calls_within_tolerance(uk, cuda, seed):
+    """The grouped int4 dequantising matmul over random row counts (both sides of
+    every kernel boundary: 8, 16, 32 rows), column counts, K (the matrix-core
+    kernels' 2048 / 4096, longer K in whole 2048s, and K only the element-wise
+    kernel takes), group sizes, zero-point forms and weight layouts, in the
+    plain and the reassociated form: the tolerances of test_gpu_dequant.py."""
+    from test_gpu_dequant import run_case, run_reassoc_case
+    rng = np.random.default_rng(616000 + seed)
+    for _ in range(40):
+        K = int(rng.choice([256, 384, 1024, 2048, 2048, 4096, 4096, 6144]))
+        gs_options = [g for g in (32, 64, 128, 256, 512, K) if K % g == 0]
+        gs = int(rng.choice(gs_options))
+        tiled = bool(rng.integers(0, 2)) and K % 128 == 0
+        N = 32 * int(rng.integers(1, 7)) if tiled else int(rng.integers(1, 200))
+        M = int(rng.choice([1, 2, 3, 7, 8, 9, 15, 16, 17, 31, 32, 33, 40]))
+        zp_u4 = bool(rng.integers(0, 2))
+        run_case(uk, M, N, K, gs, zp_u4, tiled, seed=int(rng.integers(0, 1 << 20)))
+        if rng.integers(0, 2):
+            run_reassoc_case(uk, min(M, 17), N, K, gs, zp_u4, tiled, seed=int(rng.integers(0, 1 << 20)))
