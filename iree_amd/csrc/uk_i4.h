@@ -32,6 +32,7 @@ struct I4Args {
   int tiled;
   int n_tiles;            // ceil(N / 32)
   int m_base;             // first activation row of this pass
+  int stage_rows;         // rows the LDS staging area of a wave holds (8 or 16), 16-row form
   // weight addressing of the fast kernel: byte offset of the 16 bytes that
   // lane (nl, kc) reads for column c of tile nt in 128-k span s is
   //   nt * K * 16 + s * span_stride + c * col_stride + kc * 16

@@ -60,23 +60,28 @@ namespace {
 //            MFMAs in the tiled layout (MFMA q covers k = q*32 .. +32 of the
 //            span); in the row-major one that only holds for groups of 128
 //            and more, so smaller groups are served from tiled weights only.
-//   kStageX  (16-row form, at most kStageRows rows) the wave fetches its K
-//            slice of the activations with one full-width load per KiB into
-//            LDS and takes its operand fragments from there. Fetching them
-//            straight into the operand layout costs 16 load instructions per
-//            wave whatever the number of rows, and the kernel's start is bound
-//            by the rate at which the texture path takes instructions (about
-//            16 cycles each, 8 waves): with one row the weights of the first
-//            tile are requested 0.9 us earlier this way.
-constexpr int kStageRows = 8;
+//   kStageX  (the 16-row form) the wave fetches its K slice of the activations
+//            with one full-width direct-to-LDS load per row and takes its
+//            operand fragments from there. Fetching them straight into the
+//            operand layout costs 16 load instructions per wave whatever the
+//            number of rows, and the kernel's start is bound by the rate at
+//            which the compute unit takes load instructions (about 30 cycles
+//            each, 8 waves): with one row the weights of the first tile are
+//            requested 0.8 us earlier this way. Row r of a wave's staging
+//            area is stored rotated by r chunks of 16 bytes (lane l fetches
+//            chunk (l + r) mod row length), so that the 16 lanes that read one
+//            chunk column of 16 rows hit 16 different bank groups without any
+//            padding: 16 rows x 8 waves x 1 KiB are 128 KiB, which with the
+//            32 KiB of partial sums is all the LDS there is. The area is sized
+//            for 8 or for 16 rows (a.stage_rows).
+constexpr int kStageRowsMax = 16;
 template <int KB>
-constexpr int stage_row_pitch() { return KB * 128 + 16; }      // bytes; the 16 spread the rows over the banks
-template <int KB>
-constexpr int stage_lds_bytes() { return kWaves * kStageRows * stage_row_pitch<KB>(); }
+constexpr int stage_row_bytes() { return KB * 128; }
+constexpr int stage_rows_for(int rows) { return rows <= 8 ? 8 : 16; }
 
-template <int KB, int MH, bool kZpU4, int kLog2Gs, bool kStageX = false>
+template <int KB, int MH, bool kZpU4, int kLog2Gs>
 __global__ __launch_bounds__(kThreads) void dequant_matmul_i4_kernel(I4Args a) {
-  static_assert(!kStageX || MH == 1, "staged activations: 16-row form only");
+  constexpr bool kStageX = MH == 1;
   constexpr int SP = KB / 2;                 // spans of 128 k per wave
   constexpr int L = kLog2Gs >= 9 ? 30 : kLog2Gs;
   constexpr int GW = ((KB * 64) >> L) > 0 ? ((KB * 64) >> L) : 1;   // groups per wave slice
@@ -144,23 +149,22 @@ __global__ __launch_bounds__(kThreads) void dequant_matmul_i4_kernel(I4Args a) {
   u32x4 wreg[SP][2];
   if constexpr (kStageX) {
     extern __shared__ __attribute__((aligned(16))) char stage_all[];
-    constexpr int kPitch = stage_row_pitch<KB>();
+    constexpr int kRowBytes = stage_row_bytes<KB>();
     constexpr int kLanesPerRow = KB * 8;                 // 16-byte chunks of a row's slice
-    char* stage = stage_all + wave * kStageRows * kPitch;
-    const int rows = a.M - a.m_base;                     // (the host chose this form for rows <= kStageRows)
+    char* stage = stage_all + wave * a.stage_rows * kRowBytes;
+    const int rows = a.M - a.m_base;                     // (at most 16: the host chose this form)
     const int cq = a.tiled ? 32 : 8, ckc = a.tiled ? 8 : 32;   // chunk strides in k
     const __amdgpu_buffer_rsrc_t rsrc = tile_rsrc(nt);
-    // One direct-to-LDS load per row (lane l: bytes [16 l, 16 l + 16) of the
-    // row's slice), as many as there are rows, nothing waited for in between;
-    // then the first tile's weights; then the wait for the rows only (loads
-    // return in order: all but the weight loads issued since).
+    // One direct-to-LDS load per row, as many as there are rows, nothing waited
+    // for in between; then the first tile's weights; then the wait for the rows
+    // only (loads return in order: all but the weight loads issued since).
     const __amdgpu_buffer_rsrc_t xsrc = __builtin_amdgcn_make_buffer_rsrc(
         (void*)(a.x + (size_t)a.m_base * a.K + k_slice), 0, 0x7FFFFFFF, 0x00020000);
     if (lane < kLanesPerRow) {
 #pragma unroll 1
       for (int r = 0; r < rows; ++r)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(xsrc, (__attribute__((address_space(3))) void*)(stage + r * kPitch), 16,
-                                                 lane * 16, r * a.K * 2, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(xsrc, (__attribute__((address_space(3))) void*)(stage + r * kRowBytes), 16,
+                                                 ((lane + r) & (kLanesPerRow - 1)) * 16, r * a.K * 2, 0, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -175,11 +179,14 @@ __global__ __launch_bounds__(kThreads) void dequant_matmul_i4_kernel(I4Args a) {
 #pragma unroll
       for (int q = 0; q < 4; ++q) xraw[0][sp][q] = u32x4{0u, 0u, 0u, 0u};
     if (nl < rows) {
+      const char* my_row = stage + nl * kRowBytes;
 #pragma unroll
       for (int sp = 0; sp < SP; ++sp)
 #pragma unroll
-        for (int q = 0; q < 4; ++q)
-          xraw[0][sp][q] = *(const u32x4*)(stage + nl * kPitch + (sp * 128 + q * cq + kc * ckc) * 2);
+        for (int q = 0; q < 4; ++q) {
+          const int chunk = (sp * 128 + q * cq + kc * ckc) >> 3;      // of 8 elements, within the slice
+          xraw[0][sp][q] = *(const u32x4*)(my_row + ((chunk - nl) & (kLanesPerRow - 1)) * 16);
+        }
     }
   } else {
     const int cq = a.tiled ? 32 : 8, ckc = a.tiled ? 8 : 32;   // chunk strides in k
@@ -188,26 +195,14 @@ __global__ __launch_bounds__(kThreads) void dequant_matmul_i4_kernel(I4Args a) {
     for (int sp = 0; sp < SP; ++sp) {
 #pragma unroll
       for (int mh = 0; mh < MH; ++mh) {
-        // (lanes of rows past M load nothing: with one row of activations the
-        // texture path would otherwise spend twice the time on 16 copies of
-        // that row that it spends on the tile's weights)
-        // With 32 rows (nearly all of them live) the loads are unconditional,
-        // rows past M read the last row and are zeroed below: the branch
-        // measured 5 % slower there.
+        // (32 rows, nearly all of them live: unconditional loads, rows past M
+        // read the last row and are zeroed below; a branch around the loads
+        // measured 5 % slower)
         const int m = a.m_base + mh * 16 + nl;
         const int mr = m < a.M ? m : a.M - 1;
         const uint16_t* row = a.x + (size_t)mr * a.K + k_slice + kc * ckc;
-        if constexpr (MH == 1) {
 #pragma unroll
-          for (int q = 0; q < 4; ++q) xraw[mh][sp][q] = u32x4{0u, 0u, 0u, 0u};
-          if (m < a.M) {
-#pragma unroll
-            for (int q = 0; q < 4; ++q) xraw[mh][sp][q] = *(const u32x4*)(row + sp * 128 + q * cq);
-          }
-        } else {
-#pragma unroll
-          for (int q = 0; q < 4; ++q) xraw[mh][sp][q] = *(const u32x4*)(row + sp * 128 + q * cq);
-        }
+        for (int q = 0; q < 4; ++q) xraw[mh][sp][q] = *(const u32x4*)(row + sp * 128 + q * cq);
       }
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -247,11 +242,11 @@ __global__ __launch_bounds__(kThreads) void dequant_matmul_i4_kernel(I4Args a) {
       if constexpr (kFirst) {
 #pragma unroll
         for (int mh = 0; mh < MH; ++mh) {
-          const uint32_t keep = MH == 1 || a.m_base + mh * 16 + nl < a.M ? 0xFFFFFFFFu : 0u;
+          const uint32_t keep = kStageX || a.m_base + mh * 16 + nl < a.M ? 0xFFFFFFFFu : 0u;
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
             u32x4 v = xraw[mh][sp][q];
-            if constexpr (MH != 1) { v.x &= keep; v.y &= keep; v.z &= keep; v.w &= keep; }
+            if constexpr (!kStageX) { v.x &= keep; v.y &= keep; v.z &= keep; v.w &= keep; }
             if constexpr (kSubnormal) {
               xf[mh][sp][q] = permute_x_for_subnormals(v);
               const int g = (sp * 128 + q * 32) >> L;
@@ -414,17 +409,19 @@ __global__ __launch_bounds__(256) void dequant_matmul_i4_generic_kernel(I4Args a
   }
 }
 
-template <int KB, int MH, bool kZpU4, int kLog2Gs, bool kStageX>
+template <int KB, int MH, bool kZpU4, int kLog2Gs>
 int launch_instance(const I4Args& a, int blocks, hipStream_t s) {
-  void (*kernel)(I4Args) = dequant_matmul_i4_kernel<KB, MH, kZpU4, kLog2Gs, kStageX>;
-  const size_t lds = kStageX ? stage_lds_bytes<KB>() : 0;
-  if (kStageX) {
+  void (*kernel)(I4Args) = dequant_matmul_i4_kernel<KB, MH, kZpU4, kLog2Gs>;
+  constexpr bool kStaged = MH == 1;
+  const size_t lds = kStaged ? (size_t)kWaves * a.stage_rows * stage_row_bytes<KB>() : 0;
+  if (kStaged) {
     // (with the kernel's static 32 KiB this is more than the 64 KiB a kernel gets by default)
     static unsigned long long attr_set_on = 0;
     int dev = 0;
     UK_RETURN_IF_HIP(hipGetDevice(&dev));
     if (dev < 0 || dev >= 64 || !((attr_set_on >> dev) & 1)) {
-      UK_RETURN_IF_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+      UK_RETURN_IF_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           kWaves * kStageRowsMax * stage_row_bytes<KB>()));
       if (dev >= 0 && dev < 64) attr_set_on |= 1ull << dev;
     }
   }
@@ -432,14 +429,14 @@ int launch_instance(const I4Args& a, int blocks, hipStream_t s) {
   return check_hip(hipGetLastError(), "dequant_matmul_i4 launch");
 }
 
-template <int KB, int MH, bool kZpU4, bool kStageX = false>
+template <int KB, int MH, bool kZpU4>
 int launch_one(const I4Args& a, int blocks, hipStream_t s) {
   switch (a.log2_gs) {
-    case 5: return launch_instance<KB, MH, kZpU4, 5, kStageX>(a, blocks, s);
-    case 6: return launch_instance<KB, MH, kZpU4, 6, kStageX>(a, blocks, s);
-    case 7: return launch_instance<KB, MH, kZpU4, 7, kStageX>(a, blocks, s);
-    case 8: return launch_instance<KB, MH, kZpU4, 8, kStageX>(a, blocks, s);
-    default: return launch_instance<KB, MH, kZpU4, 9, kStageX>(a, blocks, s);
+    case 5: return launch_instance<KB, MH, kZpU4, 5>(a, blocks, s);
+    case 6: return launch_instance<KB, MH, kZpU4, 6>(a, blocks, s);
+    case 7: return launch_instance<KB, MH, kZpU4, 7>(a, blocks, s);
+    case 8: return launch_instance<KB, MH, kZpU4, 8>(a, blocks, s);
+    default: return launch_instance<KB, MH, kZpU4, 9>(a, blocks, s);
   }
 }
 
@@ -456,10 +453,8 @@ int launch_fast(I4Args a, hipStream_t s) {
     if (a.M - m_base > 16) {
       st = a.zp_u4 ? launch_one<KB, 2, true>(a, blocks, s) : launch_one<KB, 2, false>(a, blocks, s);
       m_base += 32;
-    } else if (a.M - m_base <= kStageRows) {
-      st = a.zp_u4 ? launch_one<KB, 1, true, true>(a, blocks, s) : launch_one<KB, 1, false, true>(a, blocks, s);
-      m_base += 16;
     } else {
+      a.stage_rows = stage_rows_for(a.M - m_base);
       st = a.zp_u4 ? launch_one<KB, 1, true>(a, blocks, s) : launch_one<KB, 1, false>(a, blocks, s);
       m_base += 16;
     }
@@ -487,6 +482,7 @@ int launch_dequant_matmul_i4(const void* x, const void* w, const void* scale, co
   a.tiled = tiled;
   a.n_tiles = (int)ceil_div(N, 32);
   a.m_base = 0;
+  a.stage_rows = 0;
   a.log2_gs = 0;
   while ((1ll << a.log2_gs) < group_size) ++a.log2_gs;
   const bool gs_pow2 = (1ll << a.log2_gs) == group_size;

@@ -380,6 +380,7 @@ int launch_dequant_matmul_i4_reassoc(const void* x, const void* w, const void* s
   a.tiled = tiled;
   a.n_tiles = (int)ceil_div(N, 32);
   a.m_base = 0;
+  a.stage_rows = 0;
   a.log2_gs = 0;
   while ((1ll << a.log2_gs) < group_size) ++a.log2_gs;
   const bool gs_pow2 = (1ll << a.log2_gs) == group_size;
