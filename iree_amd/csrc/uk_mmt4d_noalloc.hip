@@ -39,6 +39,9 @@ int static_scratch_address(void** out_ptr) {
 }  // namespace
 
 extern "C" int iree_amd_uk_mmt4d_noalloc_p(const iree_amd_uk_mmt4d_params_t* params, void* stream) {
+  if (!params) return uk::fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "mmt4d: null params");
+  // (invalid parameters are reported as by iree_amd_uk_mmt4d_p, before any device call)
+  UK_RETURN_IF_ERROR(uk::validate_mmt4d(*params));
   void* ptr = nullptr;
   UK_RETURN_IF_ERROR(static_scratch_address(&ptr));
   // Every scratch request of the call is served from the static array or

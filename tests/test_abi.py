@@ -225,4 +225,16 @@ def test_validation_happens_before_any_device_work():
     assert mp(one, 0, 64, one, 0, 2048, one, 0, 64, 33, 64, 40, 16, 2, f1, None) == 12      # K not whole tiles
     assert mp(None, 0, 64, None, 0, 2048, None, 0, 64, 0, 64, 64, 16, 2, f1, None) == 0
     assert lib.iree_amd_uk_mfma_probe(2, None, 1, None, None, None) == 3
+    # the newer entry points: sizes are checked before buffers, buffers before any launch
+    assert lib.iree_amd_uk_quantize_groups_i16(one, one, one, one, 2, 100, 32, None) == 3        # K not whole groups
+    assert lib.iree_amd_uk_quantize_groups_i16(None, None, None, None, 0, 128, 32, None) == 0
+    assert lib.iree_amd_uk_quantize_groups_i16(None, one, one, one, 2, 128, 32, None) == 3
+    assert lib.iree_amd_uk_quantize_pack_f8e4m3(one, 40, one, 40 * 32, 3, 40, f1, None) == 3    # cols not whole tiles
+    assert lib.iree_amd_uk_quantize_pack_f8e4m3(one, 16, one, 32 * 32, 3, 32, f1, None) == 3    # pitch below a row
+    assert lib.iree_amd_uk_quantize_pack_f8e4m3(None, 32, None, 32 * 32, 0, 32, f1, None) == 0
+    assert lib.iree_amd_uk_quantize_pack_f8e4m3(one, 32, None, 32 * 32, 3, 32, f1, None) == 3
+    assert lib.iree_amd_uk_copy_probe(None, one, 8192, 0, 0, None) == 3
+    assert lib.iree_amd_uk_dequant_matmul_i4(one, one, one, one, one, 1, 8, 128, 32, 0x8, None) == 3   # unknown flag bit
+    assert lib.iree_amd_uk_mmt4d_noalloc_p(None, None) == 3
+    assert lib.iree_amd_uk_release_scratch() == 0
     assert lib.iree_amd_uk_version() >= 1
