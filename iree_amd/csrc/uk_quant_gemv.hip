@@ -25,11 +25,13 @@
 // walks all of K for its columns alone (about 8 us of dependent latency and
 // dequantisation); it is therefore used only for the K that kernel cannot take.
 //
-// A nibble n becomes the f16 value 1024+n (or 1024+16n for the upper nibble of
-// a byte) by OR-ing it into 0x6400, offset and zero point are removed with
-// exact packed-f16 arithmetic, v_mfma_f32_16x16x32_f16 multiplies exact small
-// integers, and per-group f32 partial sums are scaled by the group's scale (the
-// lane owns output column n, so the scale is a per-lane scalar).
+// The nibbles go to v_mfma_f32_16x16x32_f16 as f16 subnormals (one shift and
+// four ANDs per 8 weights, every product exact in f32; uk_i4.h), the
+// activations that meet the 16-fold pairs are divided by 16 when they are
+// staged, the zero point multiplies the group's sum of activations, which a
+// second MFMA against a constant operand takes alongside, and the per-group f32
+// partial sums are scaled by the group's scale (the lane owns output column n,
+// so scale and zero point are per-lane scalars).
 #include "uk_common.h"
 #include "uk_i4.h"
 
@@ -156,7 +158,47 @@ __global__ __launch_bounds__(kThreads) void dequant_gemv_i4_kernel(GemvArgs a) {
   };
   auto word_of = [](const u32x4* v, int i) -> uint32_t { return v[i >> 2][i & 3]; };
 
-  // ---- request the first slabs and parameters, then stage x -----------------
+  // ---- stage x, then request the first slabs and parameters ----------------
+  // x -> LDS in MFMA A-operand order: the 16 bytes that lane (row m, kc) feeds
+  // MFMA number `step` (= span * 4 + q) lie at ((step * 4 + kc) * m_eff + m) * 16,
+  // permuted to the k order of the weight dwords. Which 8 k those are depends
+  // on the weight layout (see the other kernel): chunk q*4+kc of the span for
+  // tiled weights, kc*4+q for row-major ones.
+  // The activations go first, four loads in flight per thread: loads return in
+  // order, so behind the 16 slabs of weights (which come from HBM) every round
+  // of this loop would wait for all of them, and the loop is what the barrier
+  // below waits for. (Measured inside the kernel at one row, K = 14336: staged
+  // at 5.4 us with the weights requested first.)
+  {
+    const int chunks_per_row = my_chunks * 256;        // 8-element pieces of this row's K range
+    const int total = a.m_eff * chunks_per_row;
+    constexpr int kBatch = 4;
+    for (int c0x = threadIdx.x; c0x < total; c0x += kThreads * kBatch) {
+      u32x4 v[kBatch];
+#pragma unroll
+      for (int b = 0; b < kBatch; ++b) {
+        const int c = c0x + b * kThreads;
+        v[b] = u32x4{0u, 0u, 0u, 0u};
+        if (c < total) {
+          const int m = c / chunks_per_row, kchunk = c - m * chunks_per_row;
+          v[b] = *(const u32x4*)(a.x + (size_t)(a.m_base + m) * a.K + (size_t)chunk_base * 2048 + kchunk * 8);
+        }
+      }
+#pragma unroll
+      for (int b = 0; b < kBatch; ++b) {
+        const int c = c0x + b * kThreads;
+        if (c < total) {
+          const int m = c / chunks_per_row, kchunk = c - m * chunks_per_row;
+          const int span = kchunk >> 4, r = kchunk & 15;
+          const int q = a.tiled ? (r >> 2) : (r & 3), kcc = a.tiled ? (r & 3) : (r >> 2);
+          union { half8 h; u32x4 u; } p;
+          p.h = permute_x_for_subnormals(v[b]);
+          *(u32x4*)(x_lds + (((span * 4 + q) * 4 + kcc) * a.m_eff + m) * 16) = p.u;
+        }
+      }
+    }
+  }
+  __builtin_amdgcn_sched_barrier(0);
   u32x4 ring[kRingDepth];
   Meta meta_next;
   {
@@ -166,34 +208,19 @@ __global__ __launch_bounds__(kThreads) void dequant_gemv_i4_kernel(GemvArgs a) {
     for (int d = 0; d < kRingDepth; ++d) ring[d] = load_slab(r0, (chunk_base + c0) * kChunkSpans + d);
   }
   __builtin_amdgcn_sched_barrier(0);
-  // x -> LDS in MFMA A-operand order: the 16 bytes that lane (row m, kc) feeds
-  // MFMA number `step` (= span * 4 + q) lie at ((step * 4 + kc) * m_eff + m) * 16,
-  // permuted to the k order of the weight dwords. Which 8 k those are depends
-  // on the weight layout (see the other kernel): chunk q*4+kc of the span for
-  // tiled weights, kc*4+q for row-major ones.
-  {
-    const int chunks_per_row = my_chunks * 256;        // 8-element pieces of this row's K range
-    const int total = a.m_eff * chunks_per_row;
-    for (int c = threadIdx.x; c < total; c += kThreads) {
-      const int m = c / chunks_per_row, kchunk = c - m * chunks_per_row;
-      const int span = kchunk >> 4, r = kchunk & 15;
-      const int q = a.tiled ? (r >> 2) : (r & 3), kcc = a.tiled ? (r & 3) : (r >> 2);
-      const u32x4 v = *(const u32x4*)(a.x + (size_t)(a.m_base + m) * a.K + (size_t)chunk_base * 2048 + kchunk * 8);
-      union { half8 h; u32x4 u; } p;
-      p.h = permute_x(v);
-      *(u32x4*)(x_lds + (((span * 4 + q) * 4 + kcc) * a.m_eff + m) * 16) = p.u;
-    }
-  }
   __syncthreads();
   // Lanes of rows past m_eff read the last row: a row of A only reaches the
   // same row of the result, and those rows are never stored.
   const char* x_lane = x_lds + (kc * a.m_eff + (nl < a.m_eff ? nl : a.m_eff - 1)) * 16;
   const int x_step_bytes = 4 * a.m_eff * 16;
 
-  floatx4 acc = {0.f, 0.f, 0.f, 0.f}, part = {0.f, 0.f, 0.f, 0.f};
-  float run_scale = 0.f;                       // kRuntimeGroups: scale of the open group
-  union { uint32_t u; half2v h; } run_lo, run_hi, run_zf;
-  run_lo.u = 0x64006400u; run_hi.u = 0x54005400u; run_zf.u = 0;
+  // `part`: the products of the open group in units of 2^-24 (the nibbles are
+  // f16 subnormals, see nibbles_as_subnormals); `xs`: the sum of the group's
+  // activations, taken by a second MFMA against a constant operand (every
+  // column the same), which is what the zero point multiplies.
+  floatx4 acc = {0.f, 0.f, 0.f, 0.f}, part = {0.f, 0.f, 0.f, 0.f}, xs = {0.f, 0.f, 0.f, 0.f};
+  float run_scale = 0.f, run_zq = 0.f;         // kRuntimeGroups: parameters of the open group
+  const half8 ones = ones_for_subnormal_sums();
   floatx4* partial = (floatx4*)(x_lds + a.x_bytes);   // [2][kWaves][64], ksplit > 1 only
   int unit = unit0, chunk = c0, parity = 0;
   for (int pair = 0; pair < n_pairs; ++pair) {
@@ -212,9 +239,7 @@ __global__ __launch_bounds__(kThreads) void dequant_gemv_i4_kernel(GemvArgs a) {
 #pragma unroll
     for (int s = 0; s < kChunkSpans; ++s) {
       const u32x4 wv = ring[s % kRingDepth];
-      float sc = 0.f;
-      union { uint32_t u; half2v h; } lo, hi, zf;
-      lo.u = hi.u = zf.u = 0;
+      float sc = 0.f, zq = 0.f;
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const int k_in_chunk = s * 128 + q * 32;
@@ -226,56 +251,48 @@ __global__ __launch_bounds__(kThreads) void dequant_gemv_i4_kernel(GemvArgs a) {
           if (group_start) {
             const uint32_t sg = (uint32_t)n * a.G + (uint32_t)(k_abs >> a.log2_gs);
             const uint32_t sbits = __builtin_amdgcn_raw_buffer_load_b32(scale_rsrc, (sg * 2) & ~3u, 0, 0);
-            run_scale = __half2float(__ushort_as_half((uint16_t)(sbits >> ((sg & 1) * 16))));
+            run_scale = __half2float(__ushort_as_half((uint16_t)(sbits >> ((sg & 1) * 16)))) * kSubnormalRescale;
             if (kZpU4) {
               const uint32_t zw = __builtin_amdgcn_raw_buffer_load_b32(zp_rsrc, (sg >> 1) & ~3u, 0, 0);
               const uint32_t zb = (zw >> (((sg >> 1) & 3) * 8 + (sg & 1) * 4)) & 0xF;
-              run_lo.u = offset_lo_bits(zb);
-              run_hi.u = offset_hi_bits(zb);
+              run_zq = -(float)zb * kSubnormalUnit;
             } else {
               const uint32_t zw = __builtin_amdgcn_raw_buffer_load_b32(zp_rsrc, (sg * 2) & ~3u, 0, 0);
               const uint32_t zb = (zw >> ((sg & 1) * 16)) & 0xFFFF;
-              run_lo.u = 0x64006400u;
-              run_hi.h = half2v{(_Float16)64.0f, (_Float16)64.0f};
-              run_zf.u = zb | (zb << 16);
+              run_zq = -__half2float(__ushort_as_half((uint16_t)zb)) * kSubnormalUnit;
             }
           }
-          sc = run_scale; lo.u = run_lo.u; hi.u = run_hi.u; zf.u = run_zf.u;
+          sc = run_scale; zq = run_zq;
         } else {
           constexpr int L = kLog2Gs;
           const int g = k_in_chunk >> L;                 // group within the chunk
           group_start = (k_in_chunk & ((1 << L) - 1)) == 0;
           group_end = ((k_in_chunk + 32) & ((1 << L) - 1)) == 0;
           if (group_start || q == 0) {
+            // the group's scale, times 2^24, and minus its zero point in units of 2^-24
             const uint32_t sbits = (word_of(mt.s, g >> 1) >> ((g & 1) * 16)) & 0xFFFF;
-            sc = __half2float(__ushort_as_half((uint16_t)sbits));
-            // Packed uint4 zero points fold into the offsets (1024 + zp and
-            // 64 + zp are exact); f16 zero points may carry a fraction, which
-            // such a sum would round away: they are subtracted in a second step.
+            sc = __half2float(__ushort_as_half((uint16_t)sbits)) * kSubnormalRescale;
             if (kZpU4) {
               const uint32_t zb = (word_of(mt.z, g >> 3) >> ((g & 7) * 4)) & 0xF;
-              lo.u = offset_lo_bits(zb);
-              hi.u = offset_hi_bits(zb);
+              zq = -(float)zb * kSubnormalUnit;
             } else {
               const uint32_t zb = (word_of(mt.z, g >> 1) >> ((g & 1) * 16)) & 0xFFFF;
-              lo.u = 0x64006400u;
-              hi.h = half2v{(_Float16)64.0f, (_Float16)64.0f};
-              zf.u = zb | (zb << 16);
+              zq = -__half2float(__ushort_as_half((uint16_t)zb)) * kSubnormalUnit;
             }
           }
         }
-        if (group_start) part = floatx4{0.f, 0.f, 0.f, 0.f};
-        half8 wq = dequant_dword(wv[q], lo.h, hi.h);
-        if (!kZpU4) {
-          const half8 zsub2 = {zf.h.x, zf.h.x, zf.h.x, zf.h.x, zf.h.x, zf.h.x, zf.h.x, zf.h.x};
-          wq = wq - zsub2;
+        if (group_start) {
+          part = floatx4{0.f, 0.f, 0.f, 0.f};
+          xs = floatx4{0.f, 0.f, 0.f, 0.f};
         }
+        const half8 wq = nibbles_as_subnormals(wv[q]);
         union { half8 h; u32x4 u; } xa;
         xa.u = *(const u32x4*)(x_chunk + (s * 4 + q) * x_step_bytes);
         part = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa.h, wq, part, 0, 0, 0);
+        xs = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa.h, ones, xs, 0, 0, 0);
         if (group_end) {
 #pragma unroll
-          for (int r = 0; r < 4; ++r) acc[r] = __builtin_fmaf(part[r], sc, acc[r]);
+          for (int r = 0; r < 4; ++r) acc[r] = __builtin_fmaf(__builtin_fmaf(zq, xs[r], part[r]), sc, acc[r]);
         }
       }
       // The slab's registers are free: request the slab kRingDepth further on,
