@@ -63,6 +63,10 @@ struct SkinnyArgs {
   // z * {lhs,rhs,out}_batch_bytes further on (one plane and zeros without one)
   int batch;
   int64_t lhs_batch_bytes, rhs_batch_bytes, out_batch_bytes;
+  // > 0: every wave fetches the left-hand side of its K slice (one contiguous
+  // piece of the packed row) with direct-to-LDS loads of 1 KiB into its own
+  // area of so many bytes of the dynamic LDS and reads its fragments from there
+  int stage_wave_bytes;
 };
 
 // SP: K steps per wave held in registers (compile-time bound; a.steps_per_wave <= SP).
@@ -133,32 +137,66 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
     return sp >= count ? make_frag(zero, zero) : f;
   };
 
-  // ---- first blocks of the first tile, then the left-hand side -------------
+  // ---- the left-hand side and the first blocks of the first tile ------------
   int j = kPerWave ? blockIdx.x * kWaves + wave : blockIdx.x;
   const int j_step = kPerWave ? gridDim.x * kWaves : gridDim.x;
   frag_t ring[kDepth];
-#pragma unroll
-  for (int d = 0; d < kDepth; ++d) ring[d] = load_block(j, d);
-  __builtin_amdgcn_sched_barrier(0);
   frag_t xf[SP];
+  // bytes of the packed left-hand side per K step: its K tiles are consecutive
+  const int step_bytes = (kSub == 2 ? 4 : a.half_k0 ? 2 : 1) * a.lhs_tile_bytes;
+  // this lane's first piece inside a step (the second one, fp8, a tile further)
+  const int piece_off = kSub == 2 ? 2 * kh * a.lhs_tile_bytes + m0 * 16
+                        : a.half_k0 ? kh * a.lhs_tile_bytes + m0 * 16 : m0 * 32 + kh * 16;
+  if (a.stage_wave_bytes > 0) {
+    // Fetching the fragments straight into registers costs one load
+    // instruction per K step and wave whatever M0 is (with M0 = 1 each moves
+    // 32 bytes), and the compute unit takes a load instruction only every 30
+    // cycles or so: 256 of them held the first tile up by 3 us. The slice is
+    // contiguous in the packed row, so a few full-width loads bring it to LDS
+    // (bytes past its end read as zeros: the descriptor ends there); the
+    // right-hand side is requested right behind and only the slice is waited
+    // for (loads return in order).
+    extern __shared__ __attribute__((aligned(16))) char stage_all[];
+    char* stage = stage_all + wave * a.stage_wave_bytes;
+    const int slice = count * step_bytes;
+    const __amdgpu_buffer_rsrc_t xsrc = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)(a.lhs + (int64_t)(count > 0 ? first : 0) * step_bytes), 0, slice, 0x00020000);
+#pragma unroll 1
+    for (int off = 0; off < slice; off += 1024)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(xsrc, (__attribute__((address_space(3))) void*)(stage + off), 16,
+                                               lane * 16, off, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-  for (int sp = 0; sp < SP; ++sp) {
-    const int s = first + (sp < count ? sp : 0);
-    // K tile(s) of step s: two tiles of K0 = half the MFMA extent, or one;
-    // fp8: four tiles, two per lane half.
-    int4v lo = {0, 0, 0, 0}, hi = {0, 0, 0, 0};
-    if (m0 < a.M0 && sp < count) {
-      if constexpr (kSub == 2) {
-        const char* p = a.lhs + (int64_t)(4 * s + 2 * kh) * a.lhs_tile_bytes + m0 * 16;
+    for (int d = 0; d < kDepth; ++d) ring[d] = load_block(j, d);
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kDepth * kSub) : "memory");
+#pragma unroll
+    for (int sp = 0; sp < SP; ++sp) {
+      int4v lo = {0, 0, 0, 0}, hi = {0, 0, 0, 0};
+      if (m0 < a.M0 && sp < count) {
+        const char* p = stage + sp * step_bytes + piece_off;
         lo = *(const int4v*)p;
-        hi = *(const int4v*)(p + a.lhs_tile_bytes);
-      } else {
-        const int64_t off = a.half_k0 ? ((int64_t)(2 * s + kh) * a.lhs_tile_bytes + m0 * 16)
-                                      : ((int64_t)s * a.lhs_tile_bytes + m0 * 32 + kh * 16);
-        lo = *(const int4v*)(a.lhs + off);
+        if constexpr (kSub == 2) hi = *(const int4v*)(p + a.lhs_tile_bytes);
       }
+      xf[sp] = make_frag(lo, hi);
     }
-    xf[sp] = make_frag(lo, hi);
+  } else {
+#pragma unroll
+    for (int d = 0; d < kDepth; ++d) ring[d] = load_block(j, d);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int sp = 0; sp < SP; ++sp) {
+      const int s = first + (sp < count ? sp : 0);
+      // K tile(s) of step s: two tiles of K0 = half the MFMA extent, or one;
+      // fp8: four tiles, two per lane half.
+      int4v lo = {0, 0, 0, 0}, hi = {0, 0, 0, 0};
+      if (m0 < a.M0 && sp < count) {
+        const char* p = a.lhs + (int64_t)s * step_bytes + piece_off;
+        lo = *(const int4v*)p;
+        if constexpr (kSub == 2) hi = *(const int4v*)(p + a.lhs_tile_bytes);
+      }
+      xf[sp] = make_frag(lo, hi);
+    }
   }
 
   int parity = 0;
@@ -218,6 +256,32 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
 
 // chunks: workgroup rows, each taking a.chunk_steps K steps; with more than one
 // the results are partial sums in the accumulator's type.
+// One launch of the form that splits K over the waves, with the left-hand side
+// staged through LDS when the slices of the 8 waves fit 64 KiB of it (narrow
+// tiles of up to 8 rows at the longest K a launch takes).
+template <typename Cfg, int SP, bool kPartialOut>
+int launch_split_form(SkinnyArgs a, dim3 grid, hipStream_t s) {
+  void (*kernel)(SkinnyArgs) = mmt4d_skinny_kernel<Cfg, SP, kPartialOut>;
+  const int step_bytes = (Cfg::kSub == 2 ? 4 : a.half_k0 ? 2 : 1) * a.lhs_tile_bytes;
+  const int wave_bytes = (SP * step_bytes + 1023) / 1024 * 1024;
+  size_t lds = 0;
+  a.stage_wave_bytes = 0;
+  if (kWaves * wave_bytes <= 64 * 1024) {
+    a.stage_wave_bytes = wave_bytes;
+    lds = (size_t)kWaves * wave_bytes;
+    // (with the kernel's static partial sums this is more than the default 64 KiB)
+    static unsigned long long attr_set_on = 0;
+    int dev = 0;
+    UK_RETURN_IF_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= 64 || !((attr_set_on >> dev) & 1)) {
+      UK_RETURN_IF_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024));
+      if (dev >= 0 && dev < 64) attr_set_on |= 1ull << dev;
+    }
+  }
+  hipLaunchKernelGGL(kernel, grid, dim3(kThreads), lds, s, a);
+  return check_hip(hipGetLastError(), "mmt4d_skinny launch");
+}
+
 template <typename Cfg>
 int launch_cfg(SkinnyArgs a, int chunks, hipStream_t s) {
   const int cus = device_cu_count();
@@ -234,6 +298,7 @@ int launch_cfg(SkinnyArgs a, int chunks, hipStream_t s) {
     // a short K and enough outer columns to give every compute unit 8 of
     // them: one outer column per wave
     a.steps_per_wave = a.chunk_steps;
+    a.stage_wave_bytes = 0;
     const dim3 grid(groups < per_plane ? groups : per_plane, 1, a.batch > 1 ? a.batch : 1);
     if (a.chunk_steps <= 8) {
       hipLaunchKernelGGL((mmt4d_skinny_kernel<Cfg, 8, false, true>), grid, dim3(kThreads), 0, s, a);
@@ -246,26 +311,23 @@ int launch_cfg(SkinnyArgs a, int chunks, hipStream_t s) {
   const int blocks = a.N < per_plane ? a.N : per_plane;
   const int per = (a.chunk_steps + kWaves - 1) / kWaves;
   a.steps_per_wave = per;
-  const dim3 grid(blocks, chunks, a.batch > 1 ? a.batch : 1), block(kThreads);
+  const dim3 grid(blocks, chunks, a.batch > 1 ? a.batch : 1);
   if (chunks > 1 && kNarrowOut) {
     if constexpr (kNarrowOut) {
-      if (per <= 8) hipLaunchKernelGGL((mmt4d_skinny_kernel<Cfg, 8, true>), grid, block, 0, s, a);
-      else if (per <= 16) hipLaunchKernelGGL((mmt4d_skinny_kernel<Cfg, 16, true>), grid, block, 0, s, a);
-      else if (per <= 32) hipLaunchKernelGGL((mmt4d_skinny_kernel<Cfg, 32, true>), grid, block, 0, s, a);
-      else return IREE_AMD_UK_STATUS_NOT_FOUND;
+      if (per <= 8) return launch_split_form<Cfg, 8, true>(a, grid, s);
+      if (per <= 16) return launch_split_form<Cfg, 16, true>(a, grid, s);
+      if (per <= 32) return launch_split_form<Cfg, 32, true>(a, grid, s);
     }
-  } else if (per <= 8) {
-    hipLaunchKernelGGL((mmt4d_skinny_kernel<Cfg, 8>), grid, block, 0, s, a);
-  } else if (per <= 16) {
-    hipLaunchKernelGGL((mmt4d_skinny_kernel<Cfg, 16>), grid, block, 0, s, a);
-  } else if (per <= 32) {
-    // (32 fp8 steps of 8 registers each would not fit the register file)
-    if constexpr (Cfg::kSub == 2) return IREE_AMD_UK_STATUS_NOT_FOUND;
-    else hipLaunchKernelGGL((mmt4d_skinny_kernel<Cfg, 32>), grid, block, 0, s, a);
-  } else {
     return IREE_AMD_UK_STATUS_NOT_FOUND;
   }
-  return check_hip(hipGetLastError(), "mmt4d_skinny launch");
+  if (per <= 8) return launch_split_form<Cfg, 8, false>(a, grid, s);
+  if (per <= 16) return launch_split_form<Cfg, 16, false>(a, grid, s);
+  if (per <= 32) {
+    // (32 fp8 steps of 8 registers each would not fit the register file)
+    if constexpr (Cfg::kSub == 2) return IREE_AMD_UK_STATUS_NOT_FOUND;
+    else return launch_split_form<Cfg, 32, false>(a, grid, s);
+  }
+  return IREE_AMD_UK_STATUS_NOT_FOUND;
 }
 
 int mfma_k_of(uint32_t flags) {
