@@ -453,6 +453,18 @@ def extras(args, torch, iree_amd, F, synth, lhs, rhs, out, ex):
                     steps, warm)
     ex["mmt4d_s8s4_tops"] = round(flops / t / 1e12, 2)
     del r4
+    # 16-bit left-hand sides (S16S8S32, S16S16S32): int8 digit planes in scratch
+    # memory, one s8 x s8 mmt4d of 2 (4) times the work, one pass that adds the
+    # digit products; rate in 16-bit operations
+    l16 = torch.from_numpy(synth.uniform_int8(4, 2 * M1 * K1 * 32 * 16)).cuda().view(torch.int16)
+    _, t = gpu_time(torch, lambda: iree_amd.mmt4d(l16, ri, oi, M1, N1, K1, 32, 32, 16, F.MMT4D_TYPE_S16S8S32),
+                    max(steps // 4, 5), max(warm // 4, 2))
+    ex["mmt4d_s16s8_tops"] = round(flops / t / 1e12, 2)
+    r16 = torch.from_numpy(synth.uniform_int8(5, 2 * N1 * K1 * 32 * 16)).cuda().view(torch.int16)
+    _, t = gpu_time(torch, lambda: iree_amd.mmt4d(l16, r16, oi, M1, N1, K1, 32, 32, 16, F.MMT4D_TYPE_S16S16S32),
+                    max(steps // 4, 5), max(warm // 4, 2))
+    ex["mmt4d_s16s16_tops"] = round(flops / t / 1e12, 2)
+    del l16, r16
     ex["mmt4d_i8_frac_of_peak"] = round(flops / t / 1e12 / PEAK_I8_TOPS, 4)
     del li, ri, oi
 

@@ -190,8 +190,11 @@ IREE_AMD_UK_EXPORT int iree_amd_uk_mmt4d_p(
  * split needs more than the array holds fails with status 8
  * (RESOURCE_EXHAUSTED) and has launched nothing; iree_amd_uk_last_error says how
  * many bytes it needed. Calls that do not split K (most) use no scratch at all;
- * the one other user is S8S4S32 at the gfx950 tiles, whose right-hand side is
- * widened to int8 in the same array (one byte per weight, same limit).
+ * the other users are S8S4S32 at the gfx950 tiles, whose right-hand side is
+ * widened to int8 in the same array (one byte per weight, same limit), and the
+ * types with a 16-bit left-hand side, whose int8 digit planes and their product
+ * go there when they fit (otherwise those run the element-wise kernel, which
+ * needs no scratch memory).
  * All calls on one GPU share that GPU's array and nothing in it needs to start
  * at zero (every partial sum is written before it is read), but calls whose
  * kernels overlap on one GPU - two streams, two host threads - race on it:

@@ -233,6 +233,11 @@ extern "C" int iree_amd_uk_mmt4d_p(const iree_amd_uk_mmt4d_params_t* params,
     if (st != IREE_AMD_UK_STATUS_NOT_FOUND) return st;
     return launch_mmt4d_generic(p, s);     // (an architecture tile all the same)
   }
+  if (mmt4d_s16_planes_supported(p.flags, p.M0, p.N0, p.K0)) {
+    int st = launch_mmt4d_s16_planes(p, s);
+    if (st != IREE_AMD_UK_STATUS_NOT_FOUND) return st;
+    return launch_mmt4d_generic(p, s);     // (likewise)
+  }
   if (!(p.flags & IREE_AMD_UK_FLAG_MMT4D_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION)) {
     // The reference asserts here (mmt4d.c:128-138); a release build would
     // crash on a null tile function. Report instead.
@@ -302,7 +307,7 @@ extern "C" uint32_t iree_amd_uk_mmt4d_info(int32_t M0, int32_t N0, int32_t K0,
                                            const uint64_t* cpu_data) {
   (void)cpu_data;
   return (mmt4d_mfma_supported(flags, M0, N0, K0) || mmt4d_skinny_supported(flags, M0, N0, K0) ||
-          mmt4d_s8s4_widened_supported(flags, M0, N0, K0))
+          mmt4d_s8s4_widened_supported(flags, M0, N0, K0) || mmt4d_s16_planes_supported(flags, M0, N0, K0))
              ? IREE_AMD_UK_FLAG_MMT4D_INFO_HAVE_ARCHITECTURE_SPECIFIC_TILE_FUNCTION
              : 0u;
 }

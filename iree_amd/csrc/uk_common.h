@@ -60,6 +60,11 @@ int launch_mmt4d_skinny(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s);
 // (uk_mmt4d_s8s4.hip); NOT_FOUND when the call must take the element-wise kernel.
 bool mmt4d_s8s4_widened_supported(uint32_t flags, int M0, int N0, int K0);
 int launch_mmt4d_s8s4_widened(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s);
+// 16-bit left-hand sides as int8 digit planes on the matrix cores
+// (uk_mmt4d_s16.hip); NOT_FOUND when the call must take the element-wise kernel
+// (small problems, no scratch memory).
+bool mmt4d_s16_planes_supported(uint32_t flags, int M0, int N0, int K0);
+int launch_mmt4d_s16_planes(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s);
 // Also needs alignment / stride properties of the actual call; returns
 // NOT_FOUND (without recording an error) when the call must take the generic
 // kernel instead.

@@ -1,0 +1,198 @@
+// mmt4d with a 16-bit left-hand side (S16S16S32, S16S8S32, S16U4S32; reference
+// runtime/src/iree/builtins/ukernel/mmt4d_tile_generic.c:11-51,108-142,
+// exported_bits.h:29-41) on the int8 matrix cores, by digit planes.
+//
+// A 16-bit value is x = 256 h + l + 128 with h = x >> 8 and l = (x & 255) - 128,
+// both int8. The left-hand side becomes a tiled int8 operand of 2 M + 1 outer
+// rows: the M rows of h, the M rows of l, and one row of the constant 64; a
+// 16-bit right-hand side likewise 2 N + 1 outer rows (an 8- or 4-bit one is
+// copied, the 4-bit one widened). One s8 x s8 mmt4d multiplies them into a
+// tiled int32 product P in scratch memory, and a last pass adds the digit
+// products with their weights:
+//
+//   8-bit rhs:  out = 256 P[h] + P[l] + 2 P[64]               (128 sum y = 2 * 64 sum y)
+//   16-bit rhs: out = 65536 P[h,h] + 256 (P[h,l] + P[l,h]) + P[l,l]
+//                     + 512 P[h,64] + 2 P[l,64] + 512 P[64,h] + 2 P[64,l] + 4 P[64,64]
+//
+// All of it is arithmetic modulo 2^32, like the reference's int32 accumulators,
+// so the results are those of the element-wise kernel bit for bit. The planes
+// are re-tiled to K0 = 16 on the way (any K0 of the call; the K positions past
+// the end of a ragged K are zero in every plane, the constant one included), so
+// the matrix-core kernel always sees its preferred tile.
+#include "uk_common.h"
+
+namespace uk {
+namespace {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+enum SourceKind { kSourceS16 = 0, kSourceS8 = 1, kSourceU4 = 2 };
+
+struct RetileArgs {
+  const void* src;        // element 0 of the buffer (offsets are in elements)
+  int64_t offset, stride0;
+  int64_t outer, K;       // outer rows and K tiles of the source
+  int K0;
+  int64_t k16;            // K tiles of the result: ceil(K * K0 / 16)
+  uint8_t* dst;           // outer rows of k16 tiles of 32 x 16 bytes
+};
+
+// One thread makes row r of result tile (o, t): 16 consecutive K positions of
+// source row 32 o + r. A 16-bit source writes its two digit planes (outer rows o
+// and outer + o) and, from the threads of o = 0, the constant row 2 outer.
+template <int kKind>
+__global__ __launch_bounds__(256) void retile_planes_kernel(const RetileArgs a) {
+  const int64_t total = a.outer * a.k16 * 32;
+  const int64_t kk0 = a.K * a.K0;
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (int64_t)gridDim.x * blockDim.x) {
+    const int r = (int)(idx & 31);
+    const int64_t t = (idx >> 5) % a.k16, o = (idx >> 5) / a.k16;
+    const int64_t k_first = t * 16;
+    int64_t kt = k_first / a.K0;
+    int k0 = (int)(k_first - kt * a.K0);
+    const int64_t base = a.offset + o * a.stride0;
+    uint32_t hi[4] = {0, 0, 0, 0}, lo[4] = {0, 0, 0, 0}, cst[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      if (k_first + e < kk0) {
+        const int64_t i = base + (kt * 32 + r) * a.K0 + k0;
+        const int sh = 8 * (e & 3);
+        if (kKind == kSourceS16) {
+          const int v = ((const int16_t*)a.src)[i];
+          hi[e >> 2] |= (uint32_t)((v >> 8) & 255) << sh;
+          lo[e >> 2] |= (uint32_t)(((v & 255) - 128) & 255) << sh;
+          cst[e >> 2] |= 64u << sh;
+        } else if (kKind == kSourceS8) {
+          hi[e >> 2] |= (uint32_t)((const uint8_t*)a.src)[i] << sh;
+        } else {
+          const uint8_t b = ((const uint8_t*)a.src)[i >> 1];
+          hi[e >> 2] |= (uint32_t)((i & 1) ? (b >> 4) : (b & 15)) << sh;
+        }
+      }
+      if (++k0 == a.K0) { k0 = 0; ++kt; }
+    }
+    uint8_t* d = a.dst + ((o * a.k16 + t) * 32 + r) * 16;
+    *(u32x4*)d = u32x4{hi[0], hi[1], hi[2], hi[3]};
+    if (kKind == kSourceS16) {
+      const int64_t plane = a.outer * a.k16 * 512;
+      *(u32x4*)(d + plane) = u32x4{lo[0], lo[1], lo[2], lo[3]};
+      if (o == 0) *(u32x4*)(d + 2 * plane) = u32x4{cst[0], cst[1], cst[2], cst[3]};
+    }
+  }
+}
+
+struct CombineArgs {
+  const uint32_t* product;   // (2 M + 1) x cols tiles of 32 x 32
+  int64_t M, N, cols;        // cols = N (narrow rhs) or 2 N + 1
+  uint32_t* out;             // offset applied
+  int64_t out_stride0;
+  int accumulate;
+};
+
+// One thread: 4 consecutive columns of one row of one result tile.
+template <bool kWideRhs>
+__global__ __launch_bounds__(256) void combine_planes_kernel(const CombineArgs a) {
+  const int64_t total = a.M * a.N * 256;
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (int64_t)gridDim.x * blockDim.x) {
+    const int in_tile = (int)(idx & 255);            // row * 8 + group of 4 columns
+    const int r = in_tile >> 3, c = (in_tile & 7) * 4;
+    const int64_t j = (idx >> 8) % a.N, i = (idx >> 8) / a.N;
+    auto tile = [&](int64_t ti, int64_t tj) { return a.product + (ti * a.cols + tj) * 1024; };
+    auto four = [&](const uint32_t* t, int row) { return *(const u32x4*)(t + row * 32 + c); };
+    u32x4 v;
+    if (!kWideRhs) {
+      v = four(tile(i, j), r) * 256u + four(tile(a.M + i, j), r) + four(tile(2 * a.M, j), 0) * 2u;
+    } else {
+      const int64_t cj = 2 * a.N;                    // the constant column
+      v = four(tile(i, j), r) * 65536u + (four(tile(i, a.N + j), r) + four(tile(a.M + i, j), r)) * 256u +
+          four(tile(a.M + i, a.N + j), r) + four(tile(2 * a.M, j), 0) * 512u +
+          four(tile(2 * a.M, a.N + j), 0) * 2u;
+      v += tile(i, cj)[r * 32] * 512u + tile(a.M + i, cj)[r * 32] * 2u + tile(2 * a.M, cj)[0] * 4u;
+    }
+    uint32_t* o = a.out + i * a.out_stride0 + j * 1024 + r * 32 + c;
+    // (the result buffer is only element-aligned)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = a.accumulate ? o[e] + v[e] : v[e];
+  }
+}
+
+template <typename Kernel, typename Args>
+int launch_grid_stride(Kernel kernel, const Args& args, int64_t threads, hipStream_t s, const char* what) {
+  int64_t blocks = ceil_div(threads, (int64_t)256);
+  const int64_t max_blocks = (int64_t)device_cu_count() * 32;
+  if (blocks > max_blocks) blocks = max_blocks;
+  hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(256), 0, s, args);
+  return check_hip(hipGetLastError(), what);
+}
+
+inline size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
+
+// Below this many multiply-accumulates the three extra launches cost more than
+// the element-wise kernel takes.
+constexpr int64_t kMinMacs = (int64_t)1 << 24;
+
+}  // namespace
+
+bool mmt4d_s16_planes_supported(uint32_t flags, int M0, int N0, int K0) {
+  const uint32_t type = flags & IREE_AMD_UK_FLAG_MMT4D_TYPE_MASK;
+  if (type != IREE_AMD_UK_FLAG_MMT4D_TYPE_S16S16S32 && type != IREE_AMD_UK_FLAG_MMT4D_TYPE_S16S8S32 &&
+      type != IREE_AMD_UK_FLAG_MMT4D_TYPE_S16U4S32)
+    return false;
+  return M0 == 32 && N0 == 32 && K0 >= 1 &&
+         mmt4d_mfma_supported(IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32, 32, 32, 16);
+}
+
+int launch_mmt4d_s16_planes(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) {
+  if (!mmt4d_s16_planes_supported(p.flags, p.M0, p.N0, p.K0) || p.K == 0) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  const uint32_t type = p.flags & IREE_AMD_UK_FLAG_MMT4D_TYPE_MASK;
+  const bool wide_rhs = type == IREE_AMD_UK_FLAG_MMT4D_TYPE_S16S16S32;
+  const int64_t kk0 = p.K * p.K0;
+  if (p.M * p.N * 1024 < ceil_div(kMinMacs, kk0)) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  const int64_t k16 = ceil_div(kk0, (int64_t)16);
+  const int64_t lhs_rows = 2 * p.M + 1, rhs_rows = wide_rhs ? 2 * p.N + 1 : p.N;
+  if (lhs_rows > 0x7FFFFFFF / 64 || rhs_rows > 0x7FFFFFFF / 64) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  const size_t lhs_bytes = align256((size_t)lhs_rows * k16 * 512), rhs_bytes = align256((size_t)rhs_rows * k16 * 512);
+  const size_t product_bytes = (size_t)lhs_rows * rhs_rows * 4096;
+  const size_t bytes = lhs_bytes + rhs_bytes + product_bytes;
+  ScratchLease lease(s, bytes);
+  // (no memory, or a caller that brings too little of its own: the element-wise
+  // kernel needs none)
+  if (!lease.ptr()) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  uint8_t* lhs8 = (uint8_t*)lease.ptr();
+  uint8_t* rhs8 = lhs8 + lhs_bytes;
+  uint32_t* product = (uint32_t*)(rhs8 + rhs_bytes);
+
+  const RetileArgs la = {p.lhs_buffer, p.lhs_offset, p.lhs_stride0, p.M, p.K, p.K0, k16, lhs8};
+  UK_RETURN_IF_ERROR(launch_grid_stride(retile_planes_kernel<kSourceS16>, la, p.M * k16 * 32, s,
+                                        "mmt4d digit planes (lhs) launch"));
+  const RetileArgs ra = {p.rhs_buffer, p.rhs_offset, p.rhs_stride0, p.N, p.K, p.K0, k16, rhs8};
+  if (wide_rhs) {
+    UK_RETURN_IF_ERROR(launch_grid_stride(retile_planes_kernel<kSourceS16>, ra, p.N * k16 * 32, s,
+                                          "mmt4d digit planes (rhs) launch"));
+  } else if (type == IREE_AMD_UK_FLAG_MMT4D_TYPE_S16S8S32) {
+    UK_RETURN_IF_ERROR(launch_grid_stride(retile_planes_kernel<kSourceS8>, ra, p.N * k16 * 32, s,
+                                          "mmt4d 8-bit rhs re-tiling launch"));
+  } else {
+    UK_RETURN_IF_ERROR(launch_grid_stride(retile_planes_kernel<kSourceU4>, ra, p.N * k16 * 32, s,
+                                          "mmt4d 4-bit rhs widening launch"));
+  }
+
+  iree_amd_uk_mmt4d_params_t q = {lhs8, 0, k16 * 512, rhs8, 0, k16 * 512, product, 0, rhs_rows * 1024,
+                                  lhs_rows, rhs_rows, k16, 32, 32, 16, IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32,
+                                  nullptr};
+  {
+    // The stream's scratch buffer holds the operands and the product: the
+    // matmul itself runs without scratch memory (no K split).
+    ScratchOverride none(nullptr, 0, /*strict=*/false);
+    UK_RETURN_IF_ERROR(iree_amd_uk_mmt4d_p(&q, s));
+  }
+  const CombineArgs ca = {product, p.M, p.N, rhs_rows, (uint32_t*)p.out_buffer + p.out_offset, p.out_stride0,
+                          (p.flags & IREE_AMD_UK_FLAG_MMT4D_ACCUMULATE) ? 1 : 0};
+  if (wide_rhs)
+    return launch_grid_stride(combine_planes_kernel<true>, ca, p.M * p.N * 256, s, "mmt4d digit combine launch");
+  return launch_grid_stride(combine_planes_kernel<false>, ca, p.M * p.N * 256, s, "mmt4d digit combine launch");
+}
+
+}  // namespace uk

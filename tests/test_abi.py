@@ -147,7 +147,11 @@ def test_mmt4d_info_reports_mfma_tiles():
     assert iree_amd.mmt4d_info(32, 32, 16, F.MMT4D_TYPE_S8S8S32) == have
     assert iree_amd.mmt4d_info(32, 32, 32, F.MMT4D_TYPE_S8S8S32) == have
     assert iree_amd.mmt4d_info(16, 16, 1, F.MMT4D_TYPE_F16F16F32) == 0
-    assert iree_amd.mmt4d_info(32, 32, 8, F.MMT4D_TYPE_S16S16S32) == 0
+    # 16-bit left-hand sides run as int8 digit planes at 32 x 32 tiles of any K0
+    assert iree_amd.mmt4d_info(32, 32, 8, F.MMT4D_TYPE_S16S16S32) == have
+    assert iree_amd.mmt4d_info(32, 32, 2, F.MMT4D_TYPE_S16U4S32) == have
+    assert iree_amd.mmt4d_info(16, 16, 2, F.MMT4D_TYPE_S16S16S32) == 0
+    assert iree_amd.mmt4d_info(1, 32, 8, F.MMT4D_TYPE_S16U4S32) == 0
 
 
 def test_every_tile_the_query_returns_has_an_architecture_kernel():

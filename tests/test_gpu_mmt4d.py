@@ -124,6 +124,49 @@ def test_s8s4_on_the_matrix_cores_bit_exact(uk, cuda, K0):
     assert np.array_equal(gpucase.run_mmt4d(case), case.run_oracle())
 
 
+def _full_range_operand(rng, type_flag, which, n_elems):
+    """Every bit pattern of the element type, the extremes over-represented:
+    sums wrap around modulo 2^32 (the oracle accumulates in uint32_t)."""
+    dt = ukref.mmt4d_operand_dtypes(type_flag)[which]
+    bits = (F.MMT4D_TYPE_BITS[type_flag][0], F.MMT4D_TYPE_BITS[type_flag][1], 32)[which]
+    if bits == 4:
+        return rng.integers(0, 256, size=(n_elems + 1) // 2, dtype=np.uint8)
+    info = np.iinfo(dt)
+    v = rng.integers(info.min, info.max + 1, size=n_elems, dtype=np.int64)
+    edge = rng.random(n_elems) < 0.05
+    v[edge] = rng.choice(np.array([info.min, info.min + 1, -129, -128, -1, 0, 127, 128, 255, 256, info.max - 1,
+                                   info.max]).clip(info.min, info.max), size=int(edge.sum()))
+    return v.astype(dt)
+
+
+@pytest.mark.parametrize("type_flag", [F.MMT4D_TYPE_S16S16S32, F.MMT4D_TYPE_S16S8S32, F.MMT4D_TYPE_S16U4S32])
+def test_s16_on_the_matrix_cores_bit_exact(uk, cuda, type_flag):
+    """16-bit left-hand sides (mmt4d_tile_generic.c:11-51,108-142) at 32 x 32
+    tiles of any K0: above a size threshold the library splits the 16-bit
+    operands into int8 digit planes in scratch memory, runs the s8 x s8
+    matrix-core kernel on them and adds the digit products with their weights,
+    modulo 2^32 like the reference's accumulators. Bits of the oracle for the
+    reference's value ranges and for full-range operands whose sums wrap
+    around; K0 = 2 (the reference's own tile), 8, 16, an odd one that leaves a
+    ragged last 16-wide K tile; accumulate; loose strides and offsets; a
+    problem below the threshold (element-wise kernel, same bits)."""
+    rng = np.random.default_rng(9300 + type_flag)
+    even = type_flag == F.MMT4D_TYPE_S16U4S32          # two 4-bit elements per byte
+    assert uk.mmt4d_info(32, 32, 8, type_flag) == 1
+    assert uk.mmt4d_info(32, 32, 2, type_flag) == 1
+    assert uk.mmt4d_info(16, 16, 2, type_flag) == 0
+    for M, N, K, K0, acc in ((4, 4, 128, 8, False), (3, 7, 100, 8, True), (5, 5, 400, 2, False),
+                             (4, 5, 150 if even else 300, 6 if even else 3, True), (2, 9, 70, 16, False),
+                             (1, 1, 3, 8, True)):
+        for gen in (ukref.random_operand, _full_range_operand):
+            case = ukref.Mmt4dCase(rng, type_flag, M, N, K, 32, 32, K0, accumulate=acc, generator=gen)
+            got = gpucase.run_mmt4d(case, flags=case.flags & ~F.MMT4D_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION)
+            assert np.array_equal(got, case.run_oracle()), (M, N, K, K0, acc, gen.__name__)
+    case = ukref.Mmt4dCase(rng, type_flag, 5, 6, 90, 32, 32, 8, accumulate=True, loose_strides=True, offsets=True,
+                           generator=_full_range_operand)
+    assert np.array_equal(gpucase.run_mmt4d(case), case.run_oracle())
+
+
 @pytest.mark.parametrize("type_flag,K0", [(F.MMT4D_TYPE_F16F16F32, 8), (F.MMT4D_TYPE_F16F16F32, 16),
                                           (F.MMT4D_TYPE_BF16BF16F32, 8), (F.MMT4D_TYPE_S8S8S32, 16),
                                           (F.MMT4D_TYPE_S8S8S32, 32), (F.MMT4D_TYPE_F32F32F32, 4),

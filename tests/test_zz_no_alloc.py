@@ -111,3 +111,32 @@ def test_noalloc_mmt4d_on_random_data_and_beyond_the_limit(uk, cuda):
     gs = out.view(M1, N1, 1024)
     assert torch.equal(gs[:8, :16], wb[:8, :16])
     assert bool((gs[8:] == -5).all()) and bool((gs[:8, 16:] == -5).all())
+
+
+def test_noalloc_mmt4d_with_16_bit_operands(uk, cuda):
+    """The 16-bit left-hand-side types keep their int8 digit planes and the
+    product of the planes in the same array when they fit (4 x 4 and 16 x 16
+    outer tiles) and run the element-wise kernel when they do not (46 x 46:
+    93 x 93 product tiles of 4 KiB): no allocation either way, the bits of
+    iree_amd_uk_mmt4d_p and of the oracle, calls in a row with smaller ones
+    after larger ones."""
+    import torch
+    lib = uk.load_library()
+    rng = np.random.default_rng(616)
+    for type_flag in (F.MMT4D_TYPE_S16S16S32, F.MMT4D_TYPE_S16S8S32):
+        for M, N, K, K0, acc in ((46, 46, 8, 8, False), (16, 16, 64, 8, True), (4, 4, 128, 8, False)):
+            case = ukref.Mmt4dCase(rng, type_flag, M, N, K, 32, 32, K0, accumulate=acc)
+            lhs, rhs, out0 = gpucase._to_dev(case.lhs), gpucase._to_dev(case.rhs), gpucase._to_dev(case.out_init)
+            st_a, want = _run(lib.iree_amd_uk_mmt4d_p, case, lhs, rhs, out0)
+            assert st_a == 0
+            # (the first launch of a kernel in a process makes the HIP runtime
+            # load its code: measured around the second call)
+            st, got = _run(lib.iree_amd_uk_mmt4d_noalloc_p, case, lhs, rhs, out0)
+            assert st == 0, lib.iree_amd_uk_last_error()
+            assert np.array_equal(got, want), (hex(type_flag), M, N, K)
+            free_before = torch.cuda.mem_get_info()[0]
+            st, got = _run(lib.iree_amd_uk_mmt4d_noalloc_p, case, lhs, rhs, out0)
+            assert st == 0, lib.iree_amd_uk_last_error()
+            assert torch.cuda.mem_get_info()[0] == free_before, "the call changed the free device memory"
+            assert np.array_equal(got, want), (hex(type_flag), M, N, K)
+            assert np.array_equal(got, case.run_oracle()), (hex(type_flag), M, N, K)
