@@ -29,6 +29,9 @@
  *       offsets; K a multiple of the matrix-core K extent.
  *   mi355x_pack_*, mi355x_unpack_*          power-of-two tile sizes whose rows
  *       are whole 16-byte chunks, no transposes.
+ *   mi355x_pack_transpose_*, mi355x_unpack_transpose_*   transposed inner
+ *       tiles: power-of-two tile sizes whose stored rows (the tile's matrix
+ *       rows) are whole 16-byte chunks.
  */
 #ifndef IREE_AMD_HAL_EXECUTABLE_H_
 #define IREE_AMD_HAL_EXECUTABLE_H_

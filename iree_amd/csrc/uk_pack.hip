@@ -20,6 +20,7 @@
 //               accesses.
 #include "uk_common.h"
 #include "uk_pack_stream_kernel.h"
+#include "uk_pack_transpose_kernel.h"
 
 namespace uk {
 namespace {
@@ -95,23 +96,6 @@ __global__ __launch_bounds__(256) void unpack_generic_kernel(PackArgs a) {
 // rows of tiles (pack) or groups of matrix rows (unpack).
 //---------------------------------------------------------------------------
 
-
-// n / d for 0 <= n < 2^31 and a fixed d >= 1: (n * mul) >> shift.
-struct FastDiv {
-  uint32_t mul, shift, d;
-  __device__ __forceinline__ uint32_t div(uint32_t n) const {
-    return d == 1 ? n : (uint32_t)(((uint64_t)n * mul) >> shift);
-  }
-};
-FastDiv make_fastdiv(uint32_t d) {
-  FastDiv f;
-  f.d = d;
-  uint32_t l = 0;
-  while ((1ull << l) < d) ++l;
-  f.shift = 31 + l;
-  f.mul = (uint32_t)(((1ull << f.shift) + d - 1) / d);  // < 2^32 for d >= 2
-  return f;
-}
 
 struct StreamArgs {
   const char* mat;
@@ -306,152 +290,10 @@ int launch_stream_pow2(const StreamArgs& a, hipStream_t s) {
   return check_hip(hipGetLastError(), "stream_pow2 launch");
 }
 
-//---------------------------------------------------------------------------
-// Pack with transposed inner tiles (the right-hand side of a matmul given as
-// B[K][N]: every tile is stored column by column). A 16-byte chunk of the tiled
-// buffer is then CE = 16/ES consecutive matrix ROWS of one matrix column. One
-// thread builds one such chunk from CE element-sized loads and stores it with
-// one 128-bit store. Lanes of a wave take 64 consecutive matrix columns, so
-// every load instruction reads 64 consecutive elements of a row and the stores
-// of a wave are whole tiles (or whole rows of chunks of a tile); a wave walks
-// kTransUnroll consecutive row groups so that enough loads are in flight.
-//---------------------------------------------------------------------------
-constexpr int kTransUnroll = 4;
-
-struct TransArgs {
-  const char* mat;
-  char* tiled;
-  int64_t m_size0, m_size1, m_pitch_bytes;
-  int64_t row_groups;            // outer_rows * groups_per_tile
-  int64_t padded_cols;           // outer_cols * tile_cols
-  int64_t t_stride_orow_bytes, t_stride_ocol_bytes;
-  int tile_rows, tile_cols;      // matrix orientation: tile_rows = stored inner size
-  int groups_per_tile;           // tile_rows / CE
-  FastDiv by_tile_cols, by_groups;
-  uint32_t blocks_x, blocks_y;
-  uint64_t padding;
-};
-
 template <int ES>
-__global__ __launch_bounds__(256) void pack_transpose_kernel(TransArgs a) {
-  constexpr int CE = 16 / ES;
-  typedef typename Chunk<ES>::elem_t elem_t;
-  const uint32_t lane = threadIdx.x & 63;
-  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  // Same XCD-compact block order as the streaming kernels.
-  uint32_t bx, by;
-  {
-    constexpr uint32_t kXcds = 8;
-    const uint32_t total = a.blocks_x * a.blocks_y;
-    const uint32_t per = total / kXcds, rem = total % kXcds;
-    const uint32_t xcd = blockIdx.x % kXcds, idx = blockIdx.x / kXcds;
-    const uint32_t logical = xcd * per + (xcd < rem ? xcd : rem) + idx;
-    by = logical / a.blocks_x;
-    bx = logical - by * a.blocks_x;
-  }
-  const int64_t c = (int64_t)bx * 64 + lane;                 // matrix column
-  const int64_t g0 = ((int64_t)by * 4 + wave) * kTransUnroll;  // first row group of this wave
-  if (g0 >= a.row_groups) return;
-  const bool col_in_tiles = c < a.padded_cols;
-  // where column c lands: tile column and row of the (transposed) tile
-  const uint32_t cc = col_in_tiles ? (uint32_t)c : 0;
-  const uint32_t ocol = a.by_tile_cols.div(cc), d2 = cc - ocol * a.tile_cols;
-  char* out_col = a.tiled + (int64_t)ocol * a.t_stride_ocol_bytes + (int64_t)d2 * a.tile_rows * ES;
-  const elem_t pad = (elem_t)a.padding;
-  const bool interior = (int64_t)(bx + 1) * 64 <= a.m_size1 &&
-                        (g0 + kTransUnroll) * CE <= a.m_size0 && g0 + kTransUnroll <= a.row_groups;
-  elem_t v[kTransUnroll][CE];
-  if (interior) {
-    const char* src = a.mat + g0 * CE * a.m_pitch_bytes + c * ES;
-#pragma unroll
-    for (int u = 0; u < kTransUnroll; ++u)
-#pragma unroll
-      for (int i = 0; i < CE; ++i) v[u][i] = *(const elem_t*)(src + (int64_t)(u * CE + i) * a.m_pitch_bytes);
-  } else {
-#pragma unroll
-    for (int u = 0; u < kTransUnroll; ++u)
-#pragma unroll
-      for (int i = 0; i < CE; ++i) {
-        const int64_t r = (g0 + u) * CE + i;
-        v[u][i] = (r < a.m_size0 && c < a.m_size1) ? *(const elem_t*)(a.mat + r * a.m_pitch_bytes + c * ES) : pad;
-      }
-  }
-  if (!col_in_tiles) return;
-#pragma unroll
-  for (int u = 0; u < kTransUnroll; ++u) {
-    const int64_t g = g0 + u;
-    if (g >= a.row_groups) break;
-    int64_t orow;
-    uint32_t grp;
-    if (g < 0x7FFFFFFF) {
-      orow = a.by_groups.div((uint32_t)g);
-      grp = (uint32_t)g - (uint32_t)orow * a.groups_per_tile;
-    } else {
-      orow = g / a.groups_per_tile;
-      grp = (uint32_t)(g - orow * a.groups_per_tile);
-    }
-    union { elem_t e[CE]; u32x4 vec; } chunk;
-#pragma unroll
-    for (int i = 0; i < CE; ++i) chunk.e[i] = v[u][i];
-    *(u32x4*)(out_col + orow * a.t_stride_orow_bytes + (int64_t)grp * 16) = chunk.vec;
-  }
-}
-
-// The reverse: unpack of tiles stored column by column (the transposed result
-// tiles of a matmul whose narrow dimension was exchanged, reference
-// unpack.c:190-247). One thread takes one 16-byte chunk of the tiled buffer
-// (CE consecutive matrix rows of one column) and stores its CE elements; the
-// lanes of a wave hold 64 consecutive columns, so every store instruction
-// writes 64 consecutive elements of a matrix row. Same block walk as the pack.
+__global__ __launch_bounds__(256) void pack_transpose_kernel(TransArgs a) { pack_transpose_body<ES>(a); }
 template <int ES>
-__global__ __launch_bounds__(256) void unpack_transpose_kernel(TransArgs a) {
-  constexpr int CE = 16 / ES;
-  typedef typename Chunk<ES>::elem_t elem_t;
-  const uint32_t lane = threadIdx.x & 63;
-  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  uint32_t bx, by;
-  {
-    constexpr uint32_t kXcds = 8;
-    const uint32_t total = a.blocks_x * a.blocks_y;
-    const uint32_t per = total / kXcds, rem = total % kXcds;
-    const uint32_t xcd = blockIdx.x % kXcds, idx = blockIdx.x / kXcds;
-    const uint32_t logical = xcd * per + (xcd < rem ? xcd : rem) + idx;
-    by = logical / a.blocks_x;
-    bx = logical - by * a.blocks_x;
-  }
-  const int64_t c = (int64_t)bx * 64 + lane;                 // matrix column
-  const int64_t g0 = ((int64_t)by * 4 + wave) * kTransUnroll;  // first row group of this wave
-  if (g0 >= a.row_groups || c >= a.m_size1 || c >= a.padded_cols) return;
-  const uint32_t cc = (uint32_t)c;
-  const uint32_t ocol = a.by_tile_cols.div(cc), d2 = cc - ocol * a.tile_cols;
-  const char* in_col = a.tiled + (int64_t)ocol * a.t_stride_ocol_bytes + (int64_t)d2 * a.tile_rows * ES;
-  union { elem_t e[CE]; u32x4 vec; } chunk[kTransUnroll];
-#pragma unroll
-  for (int u = 0; u < kTransUnroll; ++u) {
-    const int64_t g = g0 + u;
-    chunk[u].vec = u32x4{0u, 0u, 0u, 0u};
-    if (g < a.row_groups) {
-      int64_t orow;
-      uint32_t grp;
-      if (g < 0x7FFFFFFF) {
-        orow = a.by_groups.div((uint32_t)g);
-        grp = (uint32_t)g - (uint32_t)orow * a.groups_per_tile;
-      } else {
-        orow = g / a.groups_per_tile;
-        grp = (uint32_t)(g - orow * a.groups_per_tile);
-      }
-      chunk[u].vec = *(const u32x4*)(in_col + orow * a.t_stride_orow_bytes + (int64_t)grp * 16);
-    }
-  }
-  char* dst = (char*)a.mat + c * ES;
-#pragma unroll
-  for (int u = 0; u < kTransUnroll; ++u)
-#pragma unroll
-    for (int i = 0; i < CE; ++i) {
-      const int64_t r = (g0 + u) * CE + i;
-      if (r < a.m_size0) *(elem_t*)(dst + r * a.m_pitch_bytes) = chunk[u].e[i];
-    }
-}
+__global__ __launch_bounds__(256) void unpack_transpose_kernel(TransArgs a) { unpack_transpose_body<ES>(a); }
 
 template <int ES>
 int launch_unpack_transpose(TransArgs a, hipStream_t s) {

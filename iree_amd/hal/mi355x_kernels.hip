@@ -53,6 +53,17 @@
 //   unpack  bindings 0 in: the tiles (read only), 1 out: the size0 x size1 matrix
 //           push constants size0, size1, tile0, tile1
 //
+// mi355x_pack_transpose_{8,16,32}bit / mi355x_unpack_transpose_{16,32}bit: the same
+// with transposed inner tiles (IREE_UK_FLAG_PACK_TRANSPOSE_INNER, pack.c:131-166,
+// unpack.c:190-247: what the right-hand side B[K][N] of a matmul needs, and
+// the transposed result tiles of a narrow-N matmul): a tile covers tile0 rows
+// x tile1 columns of the matrix and is stored column by column,
+// [ceildiv(size0, tile0)][ceildiv(size1, tile1)][tile1][tile0]; same bindings
+// and push constants; power-of-two tiles with tile0 * bytes >= 16; grid =
+// ceildiv(C, 64) * ceildiv(G, 16) with G = ceildiv(size0, tile0) * tile0 * bytes
+// / 16 (groups of rows that make one 16-byte chunk) and C = the padded columns
+// ceildiv(size1, tile1) * tile1 (pack) or size1 (unpack).
+//
 // 256 threads, no LDS; grid = ceildiv(C, 32) * ceildiv(R, 16) with, for pack,
 // C = ceildiv(size1, tile1) * tile1 * bytes / 16 and R = ceildiv(size0, tile0) *
 // tile0 (the padded extent), for unpack C = ceildiv(size1 * bytes, 16) and
@@ -60,6 +71,7 @@
 // and one outer row of tiles below 2^26 bytes each.
 #include "../csrc/uk_mmt4d_mfma_kernel.h"
 #include "../csrc/uk_pack_stream_kernel.h"
+#include "../csrc/uk_pack_transpose_kernel.h"
 
 namespace {
 
@@ -192,6 +204,48 @@ __device__ __forceinline__ void hal_pack(const void* mat, void* tiled, int size0
   stream_pow2_body<ES, kPack, true, kPack, 4, 2, 2, 4>(a);
 }
 
+// Transposed inner tiles: tile0 rows x tile1 columns of the matrix, stored
+// column by column.
+template <int ES, bool kPack>
+__device__ __forceinline__ void hal_pack_transpose(const void* mat, void* tiled, int size0, int size1,
+                                                   int tile0, int tile1, uint32_t padding) {
+  constexpr int CE = 16 / ES;
+  if (size0 < 1 || size1 < 1 || tile0 < CE || tile1 < 1) return;
+  // power-of-two tiles only (a stored row is then whole 16-byte chunks and the
+  // divisions below are a multiplication by 2^31 and a shift)
+  if ((tile0 & (tile0 - 1)) || (tile1 & (tile1 - 1))) return;
+  auto by_pow2 = [](int d) {
+    FastDiv f;
+    f.d = (uint32_t)d;
+    f.mul = 1u << 31;
+    f.shift = 31 + __builtin_ctz((unsigned)d);
+    return f;
+  };
+  TransArgs a;
+  a.mat = (const char*)mat;
+  a.tiled = (char*)tiled;
+  a.m_size0 = size0;
+  a.m_size1 = size1;
+  a.m_pitch_bytes = (int64_t)size1 * ES;
+  a.tile_rows = tile0;
+  a.tile_cols = tile1;
+  a.groups_per_tile = tile0 / CE;
+  const int64_t outer_rows = ((int64_t)size0 + tile0 - 1) / tile0, outer_cols = ((int64_t)size1 + tile1 - 1) / tile1;
+  a.row_groups = outer_rows * a.groups_per_tile;
+  a.padded_cols = outer_cols * tile1;
+  a.t_stride_ocol_bytes = (int64_t)tile0 * tile1 * ES;
+  a.t_stride_orow_bytes = outer_cols * a.t_stride_ocol_bytes;
+  a.by_tile_cols = by_pow2(tile1);
+  a.by_groups = by_pow2(a.groups_per_tile);
+  a.padding = padding;
+  const int64_t cols = kPack ? a.padded_cols : (int64_t)size1;
+  a.blocks_x = (uint32_t)((cols + 63) / 64);
+  a.blocks_y = (uint32_t)((a.row_groups + 4 * kTransUnroll - 1) / (4 * kTransUnroll));
+  if (blockIdx.x >= a.blocks_x * a.blocks_y) return;
+  if (kPack) pack_transpose_body<ES>(a);
+  else unpack_transpose_body<ES>(a);
+}
+
 }  // namespace
 
 #define MI355X_PACK_EXPORTS(BITS, ES)                                                              \
@@ -206,11 +260,28 @@ __device__ __forceinline__ void hal_pack(const void* mat, void* tiled, int size0
       int tile1) {                                                                                 \
     hal_pack<ES, false>(out, const_cast<void*>(in), size0, size1, tile0, tile1, 0);               \
   }
+#define MI355X_PACK_TRANSPOSE_EXPORTS(BITS, ES)                                                    \
+  extern "C" __global__ __launch_bounds__(256) void mi355x_pack_transpose_##BITS##bit(            \
+      const void* __restrict__ in, void* __restrict__ out, int size0, int size1, int tile0,       \
+      int tile1, unsigned padding) {                                                               \
+    hal_pack_transpose<ES, true>(in, out, size0, size1, tile0, tile1, padding);                   \
+  }
+#define MI355X_UNPACK_TRANSPOSE_EXPORTS(BITS, ES)                                                  \
+  extern "C" __global__ __launch_bounds__(256) void mi355x_unpack_transpose_##BITS##bit(          \
+      const void* __restrict__ in, void* __restrict__ out, int size0, int size1, int tile0,       \
+      int tile1) {                                                                                 \
+    hal_pack_transpose<ES, false>(out, const_cast<void*>(in), size0, size1, tile0, tile1, 0);     \
+  }
 MI355X_PACK_EXPORTS(8, 1)
 MI355X_PACK_EXPORTS(16, 2)
 MI355X_PACK_EXPORTS(32, 4)
 MI355X_UNPACK_EXPORTS(16, 2)
 MI355X_UNPACK_EXPORTS(32, 4)
+MI355X_PACK_TRANSPOSE_EXPORTS(8, 1)
+MI355X_PACK_TRANSPOSE_EXPORTS(16, 2)
+MI355X_PACK_TRANSPOSE_EXPORTS(32, 4)
+MI355X_UNPACK_TRANSPOSE_EXPORTS(16, 2)
+MI355X_UNPACK_TRANSPOSE_EXPORTS(32, 4)
 
 #define MI355X_MATMUL_EXPORT(NAME, CFG, WM, WN, RING, SYNC, OCC, LDS)                              \
   static_assert(uk::mmt4d_mfma_lds_bytes<uk::CFG, WM, WN, RING>() == LDS, "LDS size of the table"); \

@@ -648,6 +648,137 @@ hal.executable.source public @mi355x_mmt4d attributes {
     %x = arith.muli %bx, %by : index
     hal.return %x, %c1, %c1 : index, index, index
   }
+  // pack: in = matrix, out = tiles, tiles of tile0 rows x tile1 columns stored column by column; push constants size0, size1, tile0, tile1, padding; workload (size0, size1, tile0, tile1)
+  // limits: power-of-two tiles with tile0 * 1 >= 16 (else nothing is written)
+  hal.executable.export public @mi355x_pack_transpose_8bit ordinal(35)
+      layout(#hal.pipeline.layout<push_constants = 5, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index]
+  } {
+  ^bb0(%device: !hal.device, %size0: index, %size1: index, %tile0: index, %tile1: index):
+    %c1 = arith.constant 1 : index
+    %c16 = arith.constant 16 : index
+    %c64 = arith.constant 64 : index
+    %bytes = arith.constant 1 : index
+    %o0 = arith.ceildivui %size0, %tile0 : index
+    %tile_bytes = arith.muli %tile0, %bytes : index
+    %per_tile = arith.divui %tile_bytes, %c16 : index
+    %groups = arith.muli %o0, %per_tile : index
+    %o1 = arith.ceildivui %size1, %tile1 : index
+    %cols = arith.muli %o1, %tile1 : index
+    %bx = arith.ceildivui %cols, %c64 : index
+    %by = arith.ceildivui %groups, %c16 : index
+    %x = arith.muli %bx, %by : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  // pack: in = matrix, out = tiles, tiles of tile0 rows x tile1 columns stored column by column; push constants size0, size1, tile0, tile1, padding; workload (size0, size1, tile0, tile1)
+  // limits: power-of-two tiles with tile0 * 2 >= 16 (else nothing is written)
+  hal.executable.export public @mi355x_pack_transpose_16bit ordinal(36)
+      layout(#hal.pipeline.layout<push_constants = 5, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index]
+  } {
+  ^bb0(%device: !hal.device, %size0: index, %size1: index, %tile0: index, %tile1: index):
+    %c1 = arith.constant 1 : index
+    %c16 = arith.constant 16 : index
+    %c64 = arith.constant 64 : index
+    %bytes = arith.constant 2 : index
+    %o0 = arith.ceildivui %size0, %tile0 : index
+    %tile_bytes = arith.muli %tile0, %bytes : index
+    %per_tile = arith.divui %tile_bytes, %c16 : index
+    %groups = arith.muli %o0, %per_tile : index
+    %o1 = arith.ceildivui %size1, %tile1 : index
+    %cols = arith.muli %o1, %tile1 : index
+    %bx = arith.ceildivui %cols, %c64 : index
+    %by = arith.ceildivui %groups, %c16 : index
+    %x = arith.muli %bx, %by : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  // pack: in = matrix, out = tiles, tiles of tile0 rows x tile1 columns stored column by column; push constants size0, size1, tile0, tile1, padding; workload (size0, size1, tile0, tile1)
+  // limits: power-of-two tiles with tile0 * 4 >= 16 (else nothing is written)
+  hal.executable.export public @mi355x_pack_transpose_32bit ordinal(37)
+      layout(#hal.pipeline.layout<push_constants = 5, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index]
+  } {
+  ^bb0(%device: !hal.device, %size0: index, %size1: index, %tile0: index, %tile1: index):
+    %c1 = arith.constant 1 : index
+    %c16 = arith.constant 16 : index
+    %c64 = arith.constant 64 : index
+    %bytes = arith.constant 4 : index
+    %o0 = arith.ceildivui %size0, %tile0 : index
+    %tile_bytes = arith.muli %tile0, %bytes : index
+    %per_tile = arith.divui %tile_bytes, %c16 : index
+    %groups = arith.muli %o0, %per_tile : index
+    %o1 = arith.ceildivui %size1, %tile1 : index
+    %cols = arith.muli %o1, %tile1 : index
+    %bx = arith.ceildivui %cols, %c64 : index
+    %by = arith.ceildivui %groups, %c16 : index
+    %x = arith.muli %bx, %by : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  // unpack: in = tiles, out = matrix, tiles of tile0 rows x tile1 columns stored column by column; push constants size0, size1, tile0, tile1; workload (size0, size1, tile0, tile1)
+  // limits: power-of-two tiles with tile0 * 2 >= 16 (else nothing is written)
+  hal.executable.export public @mi355x_unpack_transpose_16bit ordinal(38)
+      layout(#hal.pipeline.layout<push_constants = 4, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index]
+  } {
+  ^bb0(%device: !hal.device, %size0: index, %size1: index, %tile0: index, %tile1: index):
+    %c1 = arith.constant 1 : index
+    %c16 = arith.constant 16 : index
+    %c64 = arith.constant 64 : index
+    %bytes = arith.constant 2 : index
+    %o0 = arith.ceildivui %size0, %tile0 : index
+    %tile_bytes = arith.muli %tile0, %bytes : index
+    %per_tile = arith.divui %tile_bytes, %c16 : index
+    %groups = arith.muli %o0, %per_tile : index
+    %bx = arith.ceildivui %size1, %c64 : index
+    %by = arith.ceildivui %groups, %c16 : index
+    %x = arith.muli %bx, %by : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  // unpack: in = tiles, out = matrix, tiles of tile0 rows x tile1 columns stored column by column; push constants size0, size1, tile0, tile1; workload (size0, size1, tile0, tile1)
+  // limits: power-of-two tiles with tile0 * 4 >= 16 (else nothing is written)
+  hal.executable.export public @mi355x_unpack_transpose_32bit ordinal(39)
+      layout(#hal.pipeline.layout<push_constants = 4, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index]
+  } {
+  ^bb0(%device: !hal.device, %size0: index, %size1: index, %tile0: index, %tile1: index):
+    %c1 = arith.constant 1 : index
+    %c16 = arith.constant 16 : index
+    %c64 = arith.constant 64 : index
+    %bytes = arith.constant 4 : index
+    %o0 = arith.ceildivui %size0, %tile0 : index
+    %tile_bytes = arith.muli %tile0, %bytes : index
+    %per_tile = arith.divui %tile_bytes, %c16 : index
+    %groups = arith.muli %o0, %per_tile : index
+    %bx = arith.ceildivui %size1, %c64 : index
+    %by = arith.ceildivui %groups, %c16 : index
+    %x = arith.muli %bx, %by : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
 }
 
 // A dispatch site (f16, 4096^3: M = N = 128 outer tiles, K = 512 tiles of K0 = 8):

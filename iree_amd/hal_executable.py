@@ -86,6 +86,25 @@ PACK_EXPORTS = {"mi355x_pack_8bit": (1, True), "mi355x_pack_16bit": (2, True),
                 "mi355x_unpack_32bit": (4, False)}
 
 
+# The same with transposed inner tiles (a tile covers tile0 rows x tile1 columns
+# of the matrix and is stored column by column): power-of-two tiles with
+# tile0 * bytes >= 16.
+PACK_TRANSPOSE_EXPORTS = {"mi355x_pack_transpose_8bit": (1, True), "mi355x_pack_transpose_16bit": (2, True),
+                          "mi355x_pack_transpose_32bit": (4, True),
+                          "mi355x_unpack_transpose_16bit": (2, False),
+                          "mi355x_unpack_transpose_32bit": (4, False)}
+
+
+def pack_transpose_workgroup_count(name, size0, size1, tile0, tile1):
+    """Grid of a transposing pack / unpack export: blocks of 64 columns x 16
+    groups of rows, a group being the 16 / bytes rows of one 16-byte chunk,
+    over the padded columns (pack) or the matrix's own (unpack)."""
+    es, is_pack = PACK_TRANSPOSE_EXPORTS[name]
+    groups = -(-size0 // tile0) * (tile0 * es // 16)
+    cols = -(-size1 // tile1) * tile1 if is_pack else size1
+    return -(-cols // 64) * -(-groups // 16)
+
+
 def pack_workgroup_count(name, size0, size1, tile0, tile1):
     """Grid of a pack / unpack export: blocks of 16 rows x 32 chunks of 16 bytes
     over the padded extent (pack) or the matrix itself (unpack)."""
@@ -121,7 +140,7 @@ class HalExecutable:
 
     def add_export(self, name, block=(WORKGROUP_SIZE, 1, 1), shared_memory_size=None):
         if shared_memory_size is None:
-            shared_memory_size = (0 if name in PACK_EXPORTS else
+            shared_memory_size = (0 if name in PACK_EXPORTS or name in PACK_TRANSPOSE_EXPORTS else
                                   MATMUL_EXPORTS[name].lds if name in MATMUL_EXPORTS else EXPORTS[name].lds)
         ordinal = C.c_int32(-1)
         _check(self._lib.iree_amd_hal_executable_add_export(
@@ -173,6 +192,19 @@ class HalExecutable:
         """mi355x_unpack_*: tiles -> matrix (size0 x size1, dense)."""
         assert not PACK_EXPORTS[name][1]
         self.dispatch(name, pack_workgroup_count(name, size0, size1, tile0, tile1), [tiles, matrix],
+                      [size0, size1, tile0, tile1], stream)
+
+    def pack_transpose(self, name, matrix, tiles, size0, size1, tile0, tile1, padding=0, stream=None):
+        """mi355x_pack_transpose_*: matrix (size0 x size1, dense) -> tiles of
+        tile0 rows x tile1 columns stored column by column."""
+        assert PACK_TRANSPOSE_EXPORTS[name][1]
+        self.dispatch(name, pack_transpose_workgroup_count(name, size0, size1, tile0, tile1), [matrix, tiles],
+                      [size0, size1, tile0, tile1, padding], stream)
+
+    def unpack_transpose(self, name, tiles, matrix, size0, size1, tile0, tile1, stream=None):
+        """mi355x_unpack_transpose_*: tiles stored column by column -> matrix."""
+        assert not PACK_TRANSPOSE_EXPORTS[name][1]
+        self.dispatch(name, pack_transpose_workgroup_count(name, size0, size1, tile0, tile1), [tiles, matrix],
                       [size0, size1, tile0, tile1], stream)
 
     def close(self):
@@ -279,6 +311,39 @@ _MLIR_PACK_EXPORT = """\
   }}
 """
 
+_MLIR_PACK_TRANSPOSE_EXPORT = """\
+  // {what}, tiles of tile0 rows x tile1 columns stored column by column; push constants size0, size1, tile0, tile1{extra}; workload (size0, size1, tile0, tile1)
+  // limits: power-of-two tiles with tile0 * {es} >= 16 (else nothing is written)
+  hal.executable.export public @{name} ordinal({ordinal})
+      layout(#hal.pipeline.layout<push_constants = {constants}, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer>
+        ]>
+      ]>) attributes {{
+    workgroup_size = [{wg} : index, 1 : index, 1 : index]
+  }} {{
+  ^bb0(%device: !hal.device, %size0: index, %size1: index, %tile0: index, %tile1: index):
+    %c1 = arith.constant 1 : index
+    %c16 = arith.constant 16 : index
+    %c64 = arith.constant 64 : index
+    %bytes = arith.constant {es} : index
+    %o0 = arith.ceildivui %size0, %tile0 : index
+    %tile_bytes = arith.muli %tile0, %bytes : index
+    %per_tile = arith.divui %tile_bytes, %c16 : index
+    %groups = arith.muli %o0, %per_tile : index
+{extent}    %bx = arith.ceildivui {cols}, %c64 : index
+    %by = arith.ceildivui %groups, %c16 : index
+    %x = arith.muli %bx, %by : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }}
+"""
+
+_MLIR_PACK_TRANSPOSE_EXTENT = """\
+    %o1 = arith.ceildivui %size1, %tile1 : index
+    %cols = arith.muli %o1, %tile1 : index
+"""
+
 _MLIR_PACK_EXTENT = """\
     %o0 = arith.ceildivui %size0, %tile0 : index
     %rows = arith.muli %o0, %tile0 : index
@@ -321,6 +386,14 @@ def mlir_source():
             extra=", padding" if is_pack else "",
             extent=_MLIR_PACK_EXTENT if is_pack else _MLIR_UNPACK_EXTENT,
             rows="%rows" if is_pack else "%size0"))
+        ordinal += 1
+    for name, (es, is_pack) in PACK_TRANSPOSE_EXPORTS.items():
+        parts.append(_MLIR_PACK_TRANSPOSE_EXPORT.format(
+            name=name, ordinal=ordinal, es=es, wg=WORKGROUP_SIZE, constants=5 if is_pack else 4,
+            what=("pack: in = matrix, out = tiles" if is_pack else "unpack: in = tiles, out = matrix"),
+            extra=", padding" if is_pack else "",
+            extent=_MLIR_PACK_TRANSPOSE_EXTENT if is_pack else "",
+            cols="%cols" if is_pack else "%size1"))
         ordinal += 1
     parts.append(_MLIR_FOOTER)
     return "".join(parts)

@@ -43,6 +43,10 @@ def test_export_table_matches_the_sources():
     assert H.pack_workgroup_count("mi355x_pack_16bit", 8191, 5001, 32, 16) == 20 * 512
     assert H.pack_workgroup_count("mi355x_unpack_16bit", 8191, 5001, 32, 16) == 20 * 512
     assert H.pack_workgroup_count("mi355x_unpack_32bit", 17, 9, 8, 4) == 1 * 2
+    # f16 4096 x 4096 in tiles of 8 rows x 32 columns: one row group per tile row
+    assert H.pack_transpose_workgroup_count("mi355x_pack_transpose_16bit", 4096, 4096, 8, 32) == 64 * 32
+    assert H.pack_transpose_workgroup_count("mi355x_pack_transpose_16bit", 1001, 333, 8, 32) == 6 * 8
+    assert H.pack_transpose_workgroup_count("mi355x_unpack_transpose_32bit", 95, 257, 32, 8) == 5 * 2
     mm = re.findall(r"^MI355X_MATMUL_EXPORT\((\w+), \w+, \d+, \d+, \d+, \d+, \d+, (\d+)\)", src, re.M)
     assert len(mm) == len(H.MATMUL_EXPORTS)
     for name, lds in mm:
@@ -54,7 +58,7 @@ def test_export_table_matches_the_sources():
 def test_code_object_is_built_and_names_every_export():
     with open(H.CODE_OBJECT, "rb") as f:
         image = f.read()
-    for name in list(H.EXPORTS) + list(H.PACK_EXPORTS) + list(H.MATMUL_EXPORTS):
+    for name in list(H.EXPORTS) + list(H.PACK_EXPORTS) + list(H.PACK_TRANSPOSE_EXPORTS) + list(H.MATMUL_EXPORTS):
         assert name.encode() + b"\0" in image, name
 
 
@@ -262,6 +266,65 @@ def test_pack_and_unpack_exports_match_the_closed_form(uk, cuda, exe, name):
             out = got.cpu().numpy()
             assert np.array_equal(out[:size0 * size1 * es], mat.view(np.uint8).reshape(-1)), (name, size0, size1, tile0, tile1)
             assert (out[size0 * size1 * es:] == 0xA5).all()
+
+
+TRANSPOSE_CASES = [  # (size0, size1, tile0 rows, tile1 columns)
+    (1001, 333, 8, 32), (200, 95, 16, 32), (64, 64, 32, 32), (515, 70, 4, 32), (95, 257, 32, 8),
+    (4096, 70, 8, 32), (1, 1, 16, 1), (129, 1003, 16, 4)]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", sorted(H.PACK_TRANSPOSE_EXPORTS))
+def test_transposing_pack_and_unpack_exports_match_the_closed_form(uk, cuda, exe, name):
+    """Tiles of tile0 rows x tile1 columns stored column by column
+    (IREE_UK_FLAG_PACK_TRANSPOSE_INNER, pack.c:131-166; unpack.c:190-247):
+    out[o0][o1][i1][i0] = in[o0 tile0 + i0][o1 tile1 + i1] or the padding
+    element; unpack: the inverse, nothing outside the matrix written. Also
+    bit-identical to the library's iree_amd_uk_pack / _unpack with the flag."""
+    import torch
+    es, is_pack = H.PACK_TRANSPOSE_EXPORTS[name]
+    dt = {1: np.uint8, 2: np.uint16, 4: np.uint32}[es]
+    rng = np.random.default_rng(zlib.crc32(name.encode()))
+    for size0, size1, tile0, tile1 in TRANSPOSE_CASES:
+        if tile0 * es < 16:
+            continue
+        o0, o1 = -(-size0 // tile0), -(-size1 // tile1)
+        pad = int(rng.integers(1, 1 << (8 * es)))
+        mat = rng.integers(0, 1 << (8 * es), (size0, size1), dtype=np.uint64).astype(dt)
+        padded = np.full((o0 * tile0, o1 * tile1), pad, dtype=dt)
+        padded[:size0, :size1] = mat
+        tiles = np.ascontiguousarray(padded.reshape(o0, tile0, o1, tile1).transpose(0, 2, 3, 1))
+        if is_pack:
+            lib_type = {1: F.PACK_TYPE_I8I8, 2: F.PACK_TYPE_F16F16, 4: F.PACK_TYPE_F32F32}[es]
+            src = torch.from_numpy(mat.view(np.uint8).reshape(-1).copy()).cuda()
+            got = torch.full((tiles.size * es,), 0xA5, dtype=torch.uint8, device=cuda)
+            ref = torch.full((tiles.size * es,), 0x5A, dtype=torch.uint8, device=cuda)
+            exe.pack_transpose(name, src, got, size0, size1, tile0, tile1, pad)
+            uk.pack(src, ref, size0, size1, o0, o1, tile1, tile0, pad, lib_type | F.PACK_TRANSPOSE_INNER)
+            torch.cuda.synchronize()
+            assert np.array_equal(got.cpu().numpy(), tiles.view(np.uint8).reshape(-1)), (name, size0, size1, tile0, tile1)
+            assert torch.equal(got, ref)
+        else:
+            lib_type = {2: F.UNPACK_TYPE_F16F16, 4: F.UNPACK_TYPE_F32F32}[es]
+            src = torch.from_numpy(tiles.view(np.uint8).reshape(-1).copy()).cuda()
+            got = torch.full(((size0 + 1) * size1 * es,), 0xA5, dtype=torch.uint8, device=cuda)
+            ref = torch.full(((size0 + 1) * size1 * es,), 0xA5, dtype=torch.uint8, device=cuda)
+            exe.unpack_transpose(name, src, got, size0, size1, tile0, tile1)
+            uk.unpack(src, ref, o0, o1, tile1, tile0, size0, size1, lib_type | F.UNPACK_TRANSPOSE_INNER)
+            torch.cuda.synchronize()
+            out = got.cpu().numpy()
+            assert np.array_equal(out[:size0 * size1 * es], mat.view(np.uint8).reshape(-1)), (name, size0, size1, tile0, tile1)
+            assert (out[size0 * size1 * es:] == 0xA5).all()
+            assert torch.equal(got, ref)
+    # tiles the export does not take leave the destination untouched
+    out = torch.full((4096,), 0xA5, dtype=torch.uint8, device=cuda)
+    src = torch.zeros(4096, dtype=torch.uint8, device=cuda)
+    if is_pack:
+        exe.pack_transpose(name, src, out, 8, 8, 24, 8, 0)
+    else:
+        exe.unpack_transpose(name, src, out, 8, 8, 24, 8)
+    torch.cuda.synchronize()
+    assert bool((out == 0xA5).all())
 
 
 @pytest.mark.gpu
