@@ -520,6 +520,26 @@ IREE_AMD_UK_EXPORT int iree_amd_uk_mmt4d_unpack(
     iree_amd_uk_index_t N, iree_amd_uk_index_t K, int32_t K0, uint32_t flags,
     float out_scale, void* stream);
 
+/* `batch` problems of iree_amd_uk_mmt4d_unpack, entry b on operands lying
+ * b * {lhs,rhs,out}_batch_stride elements after those of entry 0 (what a
+ * linalg.batch_mmt4d followed by the unpack of every entry computes; the
+ * reference runs them entry by entry, REF CPUPrepareUkernels.cpp:23-43,165-245).
+ * One launch whose workgroup planes are the entries; K is not split in it.
+ * Every entry must satisfy what the single call asks of its operands (16-byte
+ * aligned: the operand batch strides are whole 16 bytes, or 0 for an operand
+ * all entries share). Entries must not overlap in `out`; batch == 0 does
+ * nothing. */
+IREE_AMD_UK_EXPORT int iree_amd_uk_batch_mmt4d_unpack(
+    const void* lhs_buffer, iree_amd_uk_index_t lhs_offset,
+    iree_amd_uk_index_t lhs_stride0, const void* rhs_buffer,
+    iree_amd_uk_index_t rhs_offset, iree_amd_uk_index_t rhs_stride0,
+    void* out_buffer, iree_amd_uk_index_t out_offset,
+    iree_amd_uk_index_t out_stride0, iree_amd_uk_index_t out_size0,
+    iree_amd_uk_index_t out_size1, iree_amd_uk_index_t M,
+    iree_amd_uk_index_t N, iree_amd_uk_index_t K, int32_t K0, uint32_t flags,
+    float out_scale, iree_amd_uk_index_t batch, iree_amd_uk_index_t lhs_batch_stride,
+    iree_amd_uk_index_t rhs_batch_stride, iree_amd_uk_index_t out_batch_stride, void* stream);
+
 /* A whole matmul with a pre-packed right-hand side in one kernel: what the
  * reference runs as pack(LHS) -> mmt4d -> unpack
  * (REF compiler/src/iree/compiler/Codegen/Common/CPU/CPULowerToUKernels.cpp:339-480)
@@ -547,6 +567,21 @@ IREE_AMD_UK_EXPORT int iree_amd_uk_matmul_packed_rhs(
     iree_amd_uk_index_t out_stride0, iree_amd_uk_index_t M,
     iree_amd_uk_index_t N, iree_amd_uk_index_t K, int32_t K0, uint32_t flags,
     float out_scale, void* stream);
+
+/* `batch` problems of iree_amd_uk_matmul_packed_rhs (a batch matmul on
+ * row-major left-hand sides, every entry with packed weights of its own, or
+ * rhs_batch_stride = 0 for shared ones), strides in elements as above. One
+ * launch (the left-hand sides are read in the kernel, whatever N is); the same
+ * conditions on every entry as the single call. */
+IREE_AMD_UK_EXPORT int iree_amd_uk_batch_matmul_packed_rhs(
+    const void* lhs_buffer, iree_amd_uk_index_t lhs_offset,
+    iree_amd_uk_index_t lhs_stride0, const void* rhs_buffer,
+    iree_amd_uk_index_t rhs_offset, iree_amd_uk_index_t rhs_stride0,
+    void* out_buffer, iree_amd_uk_index_t out_offset,
+    iree_amd_uk_index_t out_stride0, iree_amd_uk_index_t M,
+    iree_amd_uk_index_t N, iree_amd_uk_index_t K, int32_t K0, uint32_t flags,
+    float out_scale, iree_amd_uk_index_t batch, iree_amd_uk_index_t lhs_batch_stride,
+    iree_amd_uk_index_t rhs_batch_stride, iree_amd_uk_index_t out_batch_stride, void* stream);
 
 /* buf[i] *= scale over n f32 elements, in place (applies the product of the
  * per-tensor scales to an fp8 matmul result). */

@@ -17,7 +17,9 @@ from .ukernel import (  # noqa: F401
     mfma_probe,
     quantize_groups_i16,
     copy_probe,
+    batch_matmul_packed_rhs,
     batch_mmt4d,
+    batch_mmt4d_unpack,
     mmt4d,
     mmt4d_info,
     mmt4d_silu_mul_f8e4m3,

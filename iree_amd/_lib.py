@@ -127,6 +127,14 @@ def _declare(lib):
     lib.iree_amd_uk_matmul_packed_rhs.restype = C.c_int
     lib.iree_amd_uk_matmul_packed_rhs.argtypes = [vp, i64, i64, vp, i64, i64, vp, i64, i64,
                                                   i64, i64, i64, C.c_int32, C.c_uint32, C.c_float, vp]
+    lib.iree_amd_uk_batch_mmt4d_unpack.restype = C.c_int
+    lib.iree_amd_uk_batch_mmt4d_unpack.argtypes = [vp, i64, i64, vp, i64, i64, vp, i64, i64, i64, i64,
+                                                   i64, i64, i64, C.c_int32, C.c_uint32, C.c_float,
+                                                   i64, i64, i64, i64, vp]
+    lib.iree_amd_uk_batch_matmul_packed_rhs.restype = C.c_int
+    lib.iree_amd_uk_batch_matmul_packed_rhs.argtypes = [vp, i64, i64, vp, i64, i64, vp, i64, i64,
+                                                        i64, i64, i64, C.c_int32, C.c_uint32, C.c_float,
+                                                        i64, i64, i64, i64, vp]
     lib.iree_amd_uk_scale_f32.restype = C.c_int
     lib.iree_amd_uk_scale_f32.argtypes = [vp, i64, C.c_float, vp]
     lib.iree_amd_uk_mfma_probe.restype = C.c_int

@@ -563,7 +563,14 @@ extern "C" int iree_amd_uk_mmt4d_silu_mul_f8e4m3(
   return st;
 }
 
-extern "C" int iree_amd_uk_mmt4d_unpack(
+namespace {
+// Entry b of a batch works on operands b * {lhs,rhs,out}_batch_stride elements
+// after those of entry 0; batch = 1 is the plain call.
+struct BatchStrides {
+  iree_amd_uk_index_t batch, lhs, rhs, out;
+};
+
+int mmt4d_unpack_impl(
     const void* lhs_buffer, iree_amd_uk_index_t lhs_offset,
     iree_amd_uk_index_t lhs_stride0, const void* rhs_buffer,
     iree_amd_uk_index_t rhs_offset, iree_amd_uk_index_t rhs_stride0,
@@ -571,7 +578,8 @@ extern "C" int iree_amd_uk_mmt4d_unpack(
     iree_amd_uk_index_t out_stride0, iree_amd_uk_index_t out_size0,
     iree_amd_uk_index_t out_size1, iree_amd_uk_index_t M,
     iree_amd_uk_index_t N, iree_amd_uk_index_t K, int32_t K0, uint32_t flags,
-    float out_scale, void* stream) {
+    float out_scale, const BatchStrides& b, void* stream) {
+  if (b.batch < 0) return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "mmt4d_unpack: negative batch");
   iree_amd_uk_mmt4d_params_t p = {lhs_buffer, lhs_offset, lhs_stride0,
                                   rhs_buffer, rhs_offset, rhs_stride0,
                                   out_buffer, out_offset, out_stride0,
@@ -595,27 +603,70 @@ extern "C" int iree_amd_uk_mmt4d_unpack(
                 "mmt4d_unpack: matrix size does not match the outer tile counts");
   if (out_stride0 < out_size1)
     return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "mmt4d_unpack: out_stride0 smaller than a row");
-  if (M == 0 || N == 0) return 0;
+  if (M == 0 || N == 0 || b.batch == 0) return 0;
   if (!lhs_buffer || !rhs_buffer || !out_buffer)
     return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "mmt4d_unpack: null buffer");
   int st = IREE_AMD_UK_STATUS_NOT_FOUND;
   if (mmt4d_mfma_supported(flags, 32, 32, K0))
-    st = launch_mmt4d_unpack_mfma(p, out_size0, out_size1, out_scale, (hipStream_t)stream);
+    st = launch_mmt4d_unpack_mfma(p, out_size0, out_size1, out_scale, b.batch, b.lhs, b.rhs, b.out,
+                                  (hipStream_t)stream);
+  if (st == IREE_AMD_UK_STATUS_NOT_FOUND && b.batch > 1) {
+    // (batch strides that one launch cannot take: entry by entry)
+    for (iree_amd_uk_index_t e = 0; e < b.batch; ++e) {
+      st = mmt4d_unpack_impl(lhs_buffer, lhs_offset + e * b.lhs, lhs_stride0, rhs_buffer, rhs_offset + e * b.rhs,
+                             rhs_stride0, out_buffer, out_offset + e * b.out, out_stride0, out_size0, out_size1,
+                             M, N, K, K0, flags, out_scale, BatchStrides{1, 0, 0, 0}, stream);
+      if (st) return st;
+    }
+    return 0;
+  }
   if (st == IREE_AMD_UK_STATUS_NOT_FOUND)
     return fail(IREE_AMD_UK_STATUS_UNIMPLEMENTED,
                 "mmt4d_unpack: needs a type and K0 with a matrix-core kernel, K > 0 and "
                 "16-byte aligned operands");
   return st;
 }
+}  // namespace
 
-extern "C" int iree_amd_uk_matmul_packed_rhs(
+extern "C" int iree_amd_uk_mmt4d_unpack(
+    const void* lhs_buffer, iree_amd_uk_index_t lhs_offset,
+    iree_amd_uk_index_t lhs_stride0, const void* rhs_buffer,
+    iree_amd_uk_index_t rhs_offset, iree_amd_uk_index_t rhs_stride0,
+    void* out_buffer, iree_amd_uk_index_t out_offset,
+    iree_amd_uk_index_t out_stride0, iree_amd_uk_index_t out_size0,
+    iree_amd_uk_index_t out_size1, iree_amd_uk_index_t M,
+    iree_amd_uk_index_t N, iree_amd_uk_index_t K, int32_t K0, uint32_t flags,
+    float out_scale, void* stream) {
+  return mmt4d_unpack_impl(lhs_buffer, lhs_offset, lhs_stride0, rhs_buffer, rhs_offset, rhs_stride0, out_buffer,
+                           out_offset, out_stride0, out_size0, out_size1, M, N, K, K0, flags, out_scale,
+                           BatchStrides{1, 0, 0, 0}, stream);
+}
+
+extern "C" int iree_amd_uk_batch_mmt4d_unpack(
+    const void* lhs_buffer, iree_amd_uk_index_t lhs_offset,
+    iree_amd_uk_index_t lhs_stride0, const void* rhs_buffer,
+    iree_amd_uk_index_t rhs_offset, iree_amd_uk_index_t rhs_stride0,
+    void* out_buffer, iree_amd_uk_index_t out_offset,
+    iree_amd_uk_index_t out_stride0, iree_amd_uk_index_t out_size0,
+    iree_amd_uk_index_t out_size1, iree_amd_uk_index_t M,
+    iree_amd_uk_index_t N, iree_amd_uk_index_t K, int32_t K0, uint32_t flags,
+    float out_scale, iree_amd_uk_index_t batch, iree_amd_uk_index_t lhs_batch_stride,
+    iree_amd_uk_index_t rhs_batch_stride, iree_amd_uk_index_t out_batch_stride, void* stream) {
+  return mmt4d_unpack_impl(lhs_buffer, lhs_offset, lhs_stride0, rhs_buffer, rhs_offset, rhs_stride0, out_buffer,
+                           out_offset, out_stride0, out_size0, out_size1, M, N, K, K0, flags, out_scale,
+                           BatchStrides{batch, lhs_batch_stride, rhs_batch_stride, out_batch_stride}, stream);
+}
+
+namespace {
+int matmul_packed_rhs_impl(
     const void* lhs_buffer, iree_amd_uk_index_t lhs_offset,
     iree_amd_uk_index_t lhs_stride0, const void* rhs_buffer,
     iree_amd_uk_index_t rhs_offset, iree_amd_uk_index_t rhs_stride0,
     void* out_buffer, iree_amd_uk_index_t out_offset,
     iree_amd_uk_index_t out_stride0, iree_amd_uk_index_t M,
     iree_amd_uk_index_t N, iree_amd_uk_index_t K, int32_t K0, uint32_t flags,
-    float out_scale, void* stream) {
+    float out_scale, const BatchStrides& b, void* stream) {
+  if (b.batch < 0) return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "matmul_packed_rhs: negative batch");
   if (M < 0 || N < 0 || K < 0 || K0 <= 0)
     return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "matmul_packed_rhs: negative size or K0 <= 0");
   if (K % K0)
@@ -639,17 +690,55 @@ extern "C" int iree_amd_uk_matmul_packed_rhs(
   }
   if (lhs_stride0 < K || out_stride0 < N)
     return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "matmul_packed_rhs: a row pitch smaller than a row");
-  if (M == 0 || N == 0) return 0;
+  if (M == 0 || N == 0 || b.batch == 0) return 0;
   if (!lhs_buffer || !rhs_buffer || !out_buffer)
     return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "matmul_packed_rhs: null buffer");
   int st = IREE_AMD_UK_STATUS_NOT_FOUND;
   if (mmt4d_mfma_supported(flags, 32, 32, K0))
-    st = launch_matmul_packed_rhs_mfma(p, M, N, out_scale, (hipStream_t)stream);
+    st = launch_matmul_packed_rhs_mfma(p, M, N, out_scale, b.batch, b.lhs, b.rhs, b.out, (hipStream_t)stream);
+  if (st == IREE_AMD_UK_STATUS_NOT_FOUND && b.batch > 1) {
+    for (iree_amd_uk_index_t e = 0; e < b.batch; ++e) {
+      st = matmul_packed_rhs_impl(lhs_buffer, lhs_offset + e * b.lhs, lhs_stride0, rhs_buffer,
+                                  rhs_offset + e * b.rhs, rhs_stride0, out_buffer, out_offset + e * b.out,
+                                  out_stride0, M, N, K, K0, flags, out_scale, BatchStrides{1, 0, 0, 0}, stream);
+      if (st) return st;
+    }
+    return 0;
+  }
   if (st == IREE_AMD_UK_STATUS_NOT_FOUND)
     return fail(IREE_AMD_UK_STATUS_UNIMPLEMENTED,
                 "matmul_packed_rhs: needs a type and K0 with a matrix-core kernel, K > 0 in whole "
                 "matrix-core steps and 16-byte aligned rows and tiles");
   return st;
+}
+}  // namespace
+
+extern "C" int iree_amd_uk_matmul_packed_rhs(
+    const void* lhs_buffer, iree_amd_uk_index_t lhs_offset,
+    iree_amd_uk_index_t lhs_stride0, const void* rhs_buffer,
+    iree_amd_uk_index_t rhs_offset, iree_amd_uk_index_t rhs_stride0,
+    void* out_buffer, iree_amd_uk_index_t out_offset,
+    iree_amd_uk_index_t out_stride0, iree_amd_uk_index_t M,
+    iree_amd_uk_index_t N, iree_amd_uk_index_t K, int32_t K0, uint32_t flags,
+    float out_scale, void* stream) {
+  return matmul_packed_rhs_impl(lhs_buffer, lhs_offset, lhs_stride0, rhs_buffer, rhs_offset, rhs_stride0,
+                                out_buffer, out_offset, out_stride0, M, N, K, K0, flags, out_scale,
+                                BatchStrides{1, 0, 0, 0}, stream);
+}
+
+extern "C" int iree_amd_uk_batch_matmul_packed_rhs(
+    const void* lhs_buffer, iree_amd_uk_index_t lhs_offset,
+    iree_amd_uk_index_t lhs_stride0, const void* rhs_buffer,
+    iree_amd_uk_index_t rhs_offset, iree_amd_uk_index_t rhs_stride0,
+    void* out_buffer, iree_amd_uk_index_t out_offset,
+    iree_amd_uk_index_t out_stride0, iree_amd_uk_index_t M,
+    iree_amd_uk_index_t N, iree_amd_uk_index_t K, int32_t K0, uint32_t flags,
+    float out_scale, iree_amd_uk_index_t batch, iree_amd_uk_index_t lhs_batch_stride,
+    iree_amd_uk_index_t rhs_batch_stride, iree_amd_uk_index_t out_batch_stride, void* stream) {
+  return matmul_packed_rhs_impl(lhs_buffer, lhs_offset, lhs_stride0, rhs_buffer, rhs_offset, rhs_stride0,
+                                out_buffer, out_offset, out_stride0, M, N, K, K0, flags, out_scale,
+                                BatchStrides{batch, lhs_batch_stride, rhs_batch_stride, out_batch_stride},
+                                stream);
 }
 
 extern "C" int iree_amd_uk_scale_f32(void* buf_f32, iree_amd_uk_index_t n, float scale,

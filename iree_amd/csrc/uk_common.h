@@ -73,10 +73,14 @@ int launch_batch_mmt4d_skinny(const iree_amd_uk_mmt4d_params_t& p, int64_t batch
                               int64_t rhs_batch_stride, int64_t out_batch_stride, hipStream_t s);
 int launch_batch_mmt4d_mfma(const iree_amd_uk_mmt4d_params_t& p, int64_t batch, int64_t lhs_batch_stride,
                             int64_t rhs_batch_stride, int64_t out_batch_stride, hipStream_t s);
+// (`batch` problems whose operands lie `*_batch_stride` elements apart run as
+// the planes of one launch; NOT_FOUND when the strides are not whole 16 bytes)
 int launch_mmt4d_unpack_mfma(const iree_amd_uk_mmt4d_params_t& p, int64_t out_rows,
-                             int64_t out_cols, float out_scale, hipStream_t s);
+                             int64_t out_cols, float out_scale, int64_t batch, int64_t lhs_batch_stride,
+                             int64_t rhs_batch_stride, int64_t out_batch_stride, hipStream_t s);
 int launch_matmul_packed_rhs_mfma(const iree_amd_uk_mmt4d_params_t& p, int64_t out_rows,
-                                  int64_t out_cols, float out_scale, hipStream_t s);
+                                  int64_t out_cols, float out_scale, int64_t batch, int64_t lhs_batch_stride,
+                                  int64_t rhs_batch_stride, int64_t out_batch_stride, hipStream_t s);
 int launch_mmt4d_silu_mul_mfma(const iree_amd_uk_mmt4d_params_t& p, float gate_scale,
                                float up_scale, float inv_out_scale, hipStream_t s);
 

@@ -253,6 +253,11 @@ int launch_mmt4d_mfma(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) {
 // `batch` mmt4d problems of one shape, operands `*_batch_stride` elements
 // apart: one launch whose workgroup planes are the batch entries (at most
 // 65535 planes a launch).
+namespace {
+int launch_planes(const iree_amd_uk_mmt4d_params_t& p, MfmaArgs a, int64_t batch, int64_t lhs_batch_stride,
+                  int64_t rhs_batch_stride, int64_t out_batch_stride, hipStream_t s);
+}  // namespace
+
 int launch_batch_mmt4d_mfma(const iree_amd_uk_mmt4d_params_t& p, int64_t batch, int64_t lhs_batch_stride,
                             int64_t rhs_batch_stride, int64_t out_batch_stride, hipStream_t s) {
   Mmt4dTypeInfo ti;
@@ -260,6 +265,15 @@ int launch_batch_mmt4d_mfma(const iree_amd_uk_mmt4d_params_t& p, int64_t batch, 
   MfmaArgs a;
   const int st = make_args(p, ti.out_bytes, false, &a);
   if (st) return st;
+  return launch_planes(p, a, batch, lhs_batch_stride, rhs_batch_stride, out_batch_stride, s);
+}
+
+namespace {
+// Launches `a` (any operand form) over `batch` planes.
+int launch_planes(const iree_amd_uk_mmt4d_params_t& p, MfmaArgs a, int64_t batch, int64_t lhs_batch_stride,
+                  int64_t rhs_batch_stride, int64_t out_batch_stride, hipStream_t s) {
+  Mmt4dTypeInfo ti;
+  mmt4d_type_info(p.flags, &ti);
   const int eb = ti.lhs_bits / 8;
   a.lhs_batch_bytes = lhs_batch_stride * eb;
   a.rhs_batch_bytes = rhs_batch_stride * eb;
@@ -277,13 +291,15 @@ int launch_batch_mmt4d_mfma(const iree_amd_uk_mmt4d_params_t& p, int64_t batch, 
   }
   return 0;
 }
+}  // namespace
 
 // mmt4d whose result goes to a row-major out_rows x out_cols matrix (element
 // pitch p.out_stride0 between rows) instead of tiles: what mmt4d followed by
 // an unpack without transposes writes, and reads when accumulating; float
 // results are multiplied by out_scale on the store.
 int launch_mmt4d_unpack_mfma(const iree_amd_uk_mmt4d_params_t& p, int64_t out_rows,
-                             int64_t out_cols, float out_scale, hipStream_t s) {
+                             int64_t out_cols, float out_scale, int64_t batch, int64_t lhs_batch_stride,
+                             int64_t rhs_batch_stride, int64_t out_batch_stride, hipStream_t s) {
   Mmt4dTypeInfo ti;
   mmt4d_type_info(p.flags, &ti);
   MfmaArgs a;
@@ -294,6 +310,7 @@ int launch_mmt4d_unpack_mfma(const iree_amd_uk_mmt4d_params_t& p, int64_t out_ro
   a.out_scale = out_scale;
   a.out_rows = (int)out_rows;
   a.out_cols = (int)out_cols;
+  if (batch > 1) return launch_planes(p, a, batch, lhs_batch_stride, rhs_batch_stride, out_batch_stride, s);
   return launch_typed(p, a, s);
 }
 
@@ -302,7 +319,8 @@ int launch_mmt4d_unpack_mfma(const iree_amd_uk_mmt4d_params_t& p, int64_t out_ro
 // p.lhs_buffer / lhs_offset / lhs_stride0 are the out_rows x (K * K0) matrix,
 // its first element and its row pitch in elements.
 int launch_matmul_packed_rhs_mfma(const iree_amd_uk_mmt4d_params_t& p, int64_t out_rows,
-                                  int64_t out_cols, float out_scale, hipStream_t s) {
+                                  int64_t out_cols, float out_scale, int64_t batch, int64_t lhs_batch_stride,
+                                  int64_t rhs_batch_stride, int64_t out_batch_stride, hipStream_t s) {
   Mmt4dTypeInfo ti;
   mmt4d_type_info(p.flags, &ti);
   MfmaArgs a;
@@ -327,6 +345,11 @@ int launch_matmul_packed_rhs_mfma(const iree_amd_uk_mmt4d_params_t& p, int64_t o
   // other (K is only ever split for problems of few macro tiles).
   const int eb = ti.lhs_bits / 8;
   const int64_t packed_bytes = p.M * p.K * 32 * p.K0 * eb;
+  if (batch > 1) {
+    // (a batch reads its row-major left-hand sides in the kernel)
+    a.lhs_row_major = 1;
+    return launch_planes(p, a, batch, lhs_batch_stride, rhs_batch_stride, out_batch_stride, s);
+  }
   if (out_cols >= 8192 && out_rows >= 512) {
     // (held until the matmul that reads the packed copy has been queued)
     ScratchLease lease(s, (size_t)packed_bytes);

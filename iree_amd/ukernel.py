@@ -250,6 +250,53 @@ def matmul_packed_rhs(lhs, rhs_packed, out, M, N, K, K0, flags, *, lhs_offset=0,
         _ptr(out), out_offset, out_stride0, M, N, K, K0, flags, out_scale, _stream(stream)))
 
 
+def batch_mmt4d_unpack(lhs_buffer, rhs_buffer, out_buffer, batch, out_size0, out_size1, M, N, K, K0, flags, *,
+                       lhs_offset=0, lhs_stride0=None, rhs_offset=0, rhs_stride0=None, out_offset=0,
+                       out_stride0=None, lhs_batch_stride=None, rhs_batch_stride=None,
+                       out_batch_stride=None, out_scale=1.0, stream=None):
+    """``batch`` problems of ``mmt4d_unpack`` in one launch; strides default to tight."""
+    if lhs_stride0 is None:
+        lhs_stride0 = K * 32 * K0
+    if rhs_stride0 is None:
+        rhs_stride0 = K * 32 * K0
+    if out_stride0 is None:
+        out_stride0 = out_size1
+    if lhs_batch_stride is None:
+        lhs_batch_stride = M * lhs_stride0
+    if rhs_batch_stride is None:
+        rhs_batch_stride = N * rhs_stride0
+    if out_batch_stride is None:
+        out_batch_stride = out_size0 * out_stride0
+    _check(load_library().iree_amd_uk_batch_mmt4d_unpack(
+        _ptr(lhs_buffer), lhs_offset, lhs_stride0, _ptr(rhs_buffer), rhs_offset, rhs_stride0,
+        _ptr(out_buffer), out_offset, out_stride0, out_size0, out_size1, M, N, K, K0, flags,
+        out_scale, batch, lhs_batch_stride, rhs_batch_stride, out_batch_stride, _stream(stream)))
+
+
+def batch_matmul_packed_rhs(lhs, rhs_packed, out, batch, M, N, K, K0, flags, *, lhs_offset=0,
+                            lhs_stride0=None, rhs_offset=0, rhs_stride0=None, out_offset=0,
+                            out_stride0=None, lhs_batch_stride=None, rhs_batch_stride=None,
+                            out_batch_stride=None, out_scale=1.0, stream=None):
+    """``batch`` problems of ``matmul_packed_rhs`` in one launch; strides default
+    to tight (``rhs_batch_stride=0`` shares one packed right-hand side)."""
+    if lhs_stride0 is None:
+        lhs_stride0 = K
+    if rhs_stride0 is None:
+        rhs_stride0 = K * 32
+    if out_stride0 is None:
+        out_stride0 = N
+    if lhs_batch_stride is None:
+        lhs_batch_stride = M * lhs_stride0
+    if rhs_batch_stride is None:
+        rhs_batch_stride = -(-N // 32) * rhs_stride0
+    if out_batch_stride is None:
+        out_batch_stride = M * out_stride0
+    _check(load_library().iree_amd_uk_batch_matmul_packed_rhs(
+        _ptr(lhs), lhs_offset, lhs_stride0, _ptr(rhs_packed), rhs_offset, rhs_stride0,
+        _ptr(out), out_offset, out_stride0, M, N, K, K0, flags, out_scale, batch,
+        lhs_batch_stride, rhs_batch_stride, out_batch_stride, _stream(stream)))
+
+
 def scale_f32(buf, n, scale, stream=None):
     _check(load_library().iree_amd_uk_scale_f32(_ptr(buf), n, scale, _stream(stream)))
 

@@ -228,6 +228,15 @@ def test_validation_happens_before_any_device_work():
     assert mp(one, 0, 63, one, 0, 2048, one, 0, 64, 33, 64, 64, 16, 2, f1, None) == 3       # lhs pitch below a row
     assert mp(one, 0, 64, one, 0, 2048, one, 0, 64, 33, 64, 40, 16, 2, f1, None) == 12      # K not whole tiles
     assert mp(None, 0, 64, None, 0, 2048, None, 0, 64, 0, 64, 64, 16, 2, f1, None) == 0
+    # their batch forms: the same checks, a negative batch, an empty batch
+    bmu = lib.iree_amd_uk_batch_mmt4d_unpack
+    assert bmu(one, 0, 512, one, 0, 512, one, 0, 64, 33, 64, 2, 2, 2, 16, 2, f1, -1, 0, 0, 0, None) == 3
+    assert bmu(one, 0, 512, one, 0, 512, one, 0, 63, 33, 64, 2, 2, 2, 16, 2, f1, 3, 0, 0, 0, None) == 3
+    assert bmu(None, 0, 512, None, 0, 512, None, 0, 64, 33, 64, 2, 2, 2, 16, 2, f1, 0, 0, 0, 0, None) == 0
+    bmp = lib.iree_amd_uk_batch_matmul_packed_rhs
+    assert bmp(one, 0, 64, one, 0, 2048, one, 0, 64, 33, 64, 64, 16, 2, f1, -2, 0, 0, 0, None) == 3
+    assert bmp(one, 0, 64, one, 0, 2048, one, 0, 64, 33, 64, 40, 16, 2, f1, 2, 0, 0, 0, None) == 12
+    assert bmp(None, 0, 64, None, 0, 2048, None, 0, 64, 33, 64, 64, 16, 2, f1, 0, 0, 0, 0, None) == 0
     assert lib.iree_amd_uk_mfma_probe(2, None, 1, None, None, None) == 3
     # the newer entry points: sizes are checked before buffers, buffers before any launch
     assert lib.iree_amd_uk_quantize_groups_i16(one, one, one, one, 2, 100, 32, None) == 3        # K not whole groups

@@ -978,3 +978,69 @@ def test_batch_mmt4d_large_entries_match_single_calls(uk, cuda):
         one = torch.zeros(M, N, 32, 32, device="cuda")
         ukernel.mmt4d(lhs[b], rhs[b], one, M, N, K, 32, 32, K0, F.MMT4D_TYPE_F16F16F32)
         assert torch.equal(out[b], one), b
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("type_flag,K0,dt", [(F.MMT4D_TYPE_S8S8S32, 16, np.int8), (F.MMT4D_TYPE_F16F16F32, 8, np.float16),
+                                             (F.MMT4D_TYPE_F32F32F32, 4, np.float32)])
+@pytest.mark.parametrize("accumulate", [False, True])
+def test_batch_forms_of_the_fused_entry_points_match_single_calls(uk, cuda, type_flag, K0, dt, accumulate):
+    """batch_mmt4d_unpack and batch_matmul_packed_rhs (one launch, entries as
+    workgroup planes) against one call of mmt4d_unpack / matmul_packed_rhs per
+    entry, which the tests above pin to the oracle: the same bits, ragged M and
+    N, gaps between the entries of every operand (whole 16 bytes for the
+    operands, whose entries must be aligned like those of a single call; any
+    for `out`), gaps in `out` untouched; a shared right-hand side (batch
+    stride 0); batch 0 and 1; an entry that is not 16-byte aligned is refused
+    like the single call refuses it."""
+    import torch
+    rng = np.random.default_rng(31 + K0)
+    out_dt = np.int32 if dt is np.int8 else np.float32
+    flags = type_flag | (F.MMT4D_ACCUMULATE if accumulate else 0)
+    mfma_k = {np.int8: 32, np.float16: 32, np.float32: 8}[dt]
+
+    def values(n):
+        if dt is np.int8:
+            return rng.integers(-128, 128, n).astype(np.int8)
+        return rng.integers(-4, 5, n).astype(dt)
+
+    for batch, M, N, K, gap in ((5, 70, 100, 3 * mfma_k, 64), (3, 200, 333, 9 * mfma_k, 0), (9, 32, 64, 2 * mfma_k, 16),
+                                (2, 40, 40, 4 * mfma_k, 48), (1, 33, 65, mfma_k, 0), (0, 33, 65, mfma_k, 0)):
+        M1, N1, K1 = -(-M // 32), -(-N // 32), K // K0
+        lhs_bs, rhs_bs = M1 * K1 * 32 * K0 + gap, N1 * K1 * 32 * K0 + gap
+        a_bs, out_bs = M * K + gap, M * N + gap + 7
+        nb = max(batch, 1)
+        lhs_t = torch.from_numpy(values(nb * lhs_bs)).cuda()       # packed left-hand sides
+        rhs_t = torch.from_numpy(values(nb * rhs_bs)).cuda()       # packed right-hand sides
+        a_rm = torch.from_numpy(values(nb * a_bs)).cuda()          # row-major left-hand sides
+        out0 = torch.from_numpy(rng.integers(-50, 50, nb * out_bs).astype(out_dt)).cuda()
+        for shared_rhs in (False, True):
+            rbs = 0 if shared_rhs else rhs_bs
+            # mmt4d_unpack
+            got, want = out0.clone(), out0.clone()
+            uk.batch_mmt4d_unpack(lhs_t, rhs_t, got, batch, M, N, M1, N1, K1, K0, flags,
+                                  lhs_batch_stride=lhs_bs, rhs_batch_stride=rbs, out_batch_stride=out_bs)
+            for b in range(batch):
+                uk.mmt4d_unpack(lhs_t, rhs_t, want, M, N, M1, N1, K1, K0, flags, lhs_offset=b * lhs_bs,
+                                rhs_offset=b * rbs, out_offset=b * out_bs)
+            torch.cuda.synchronize()
+            assert torch.equal(got.view(torch.int32), want.view(torch.int32)), (batch, M, N, K, gap, shared_rhs)
+            if batch:
+                assert not torch.equal(got.view(torch.int32), out0.view(torch.int32))
+            # matmul_packed_rhs
+            got, want = out0.clone(), out0.clone()
+            uk.batch_matmul_packed_rhs(a_rm, rhs_t, got, batch, M, N, K, K0, flags,
+                                       lhs_batch_stride=a_bs, rhs_batch_stride=rbs, out_batch_stride=out_bs)
+            for b in range(batch):
+                uk.matmul_packed_rhs(a_rm, rhs_t, want, M, N, K, K0, flags, lhs_offset=b * a_bs,
+                                     rhs_offset=b * rbs, out_offset=b * out_bs)
+            torch.cuda.synchronize()
+            assert torch.equal(got.view(torch.int32), want.view(torch.int32)), (batch, M, N, K, gap, shared_rhs)
+    with pytest.raises(uk.UkError):
+        uk.batch_mmt4d_unpack(lhs_t, rhs_t, out0, -1, 33, 65, 2, 3, K1, K0, flags)
+    lhs_t = torch.from_numpy(values(2 * (2 * K1 * 32 * K0) + 3)).cuda()
+    rhs_t = torch.from_numpy(values(3 * K1 * 32 * K0)).cuda()
+    out = torch.zeros(2 * 33 * 65, dtype=out0.dtype, device=cuda)
+    with pytest.raises(uk.UkError):
+        uk.batch_mmt4d_unpack(lhs_t, rhs_t, out, 2, 33, 65, 2, 3, K1, K0, flags,
+                              lhs_batch_stride=2 * K1 * 32 * K0 + 3, rhs_batch_stride=0)
