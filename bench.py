@@ -60,7 +60,7 @@ def parse_args():
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary measurements")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--only", default="", help="run only the named kernel in a loop (for profilers): "
-                    "mmt4d_f16 | mmt4d_f16_acc | mmt4d_i8 | mmt4d_fp8 | mmt4d_f16_ksplit | mlp_fp8 | pack | unpack | "
+                    "mmt4d_f16 | mmt4d_f16_acc | mmt4d_i8 | mmt4d_s16s8 | mmt4d_s16s16 | mmt4d_fp8 | mmt4d_f16_ksplit | mlp_fp8 | pack | unpack | "
                     "pack_transpose | unpack_transpose | dequant_i4[_m8|_m32] | dequant_i4_reassoc[_m8|_m32] | batch_mmt4d_f16 | "
                     "batch_mmt4d_f16_narrow | mmt4d_f16_narrow_m1 | mmt4d_f16_narrow_m8 | mmt4d_f16_narrow_n8 | "
                     "chain_i8_1024 | copy | copy_rotating | copy_rotating_nt | copy_rotating_nt_single_waves | read_only_29mb")
@@ -752,6 +752,20 @@ def run_only(args, torch, iree_amd, F, synth, mm_step):
         ri = torch.from_numpy(synth.uniform_int8(2, N1 * K1 * 512)).cuda()
         oi = torch.empty(M1 * N1 * 1024, dtype=torch.int32, device="cuda")
         fn = lambda: iree_amd.mmt4d(li, ri, oi, M1, N1, K1, 32, 32, 16, F.MMT4D_TYPE_S8S8S32)  # noqa: E731
+    elif args.only in ("mmt4d_s16s8", "mmt4d_s16s16"):
+        # 16-bit left-hand side at 4096^3: digit planes, one s8 x s8 mmt4d, the combining pass
+        size = 4096
+        M1 = N1 = size // 32
+        K1 = size // 16
+        l16 = torch.from_numpy(synth.uniform_int8(4, 2 * M1 * K1 * 512)).cuda().view(torch.int16)
+        if args.only == "mmt4d_s16s8":
+            r = torch.from_numpy(synth.uniform_int8(2, N1 * K1 * 512)).cuda()
+            tf = F.MMT4D_TYPE_S16S8S32
+        else:
+            r = torch.from_numpy(synth.uniform_int8(5, 2 * N1 * K1 * 512)).cuda().view(torch.int16)
+            tf = F.MMT4D_TYPE_S16S16S32
+        oi = torch.empty(M1 * N1 * 1024, dtype=torch.int32, device="cuda")
+        fn = lambda: iree_amd.mmt4d(l16, r, oi, M1, N1, K1, 32, 32, 16, tf)  # noqa: E731
     elif args.only in ("pack", "unpack"):
         R, Cc, T0, T1 = 8191, 5001, 32, 16
         O0, O1 = -(-R // T0), -(-Cc // T1)

@@ -82,6 +82,37 @@ __global__ __launch_bounds__(256) void retile_planes_kernel(const RetileArgs a) 
   }
 }
 
+// The same for a 16-bit source whose K0 is a multiple of 8 and whose rows of 8
+// elements are 16-byte aligned, with K * K0 whole 16-wide tiles: a thread's 16
+// positions are two runs of 8 consecutive elements, loaded 16 bytes at a time;
+// the high bytes of 4 elements are gathered with one byte permute, the low ones
+// likewise and moved by 128 with an XOR ((b - 128) mod 256 = b ^ 0x80).
+__global__ __launch_bounds__(256) void retile_planes_s16_wide_kernel(const RetileArgs a) {
+  const int64_t total = a.outer * a.k16 * 32;
+  const int64_t plane = a.outer * a.k16 * 512;
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (int64_t)gridDim.x * blockDim.x) {
+    const int r = (int)(idx & 31);
+    const int64_t t = (idx >> 5) % a.k16, o = (idx >> 5) / a.k16;
+    const int64_t base = a.offset + o * a.stride0;
+    uint32_t hi[4], lo[4];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int64_t k = t * 16 + j * 8, kt = k / a.K0;
+      const int k0 = (int)(k - kt * a.K0);
+      const u32x4 v = *(const u32x4*)((const int16_t*)a.src + base + (kt * 32 + r) * a.K0 + k0);
+      hi[2 * j] = __builtin_amdgcn_perm(v.y, v.x, 0x07050301u);
+      hi[2 * j + 1] = __builtin_amdgcn_perm(v.w, v.z, 0x07050301u);
+      lo[2 * j] = __builtin_amdgcn_perm(v.y, v.x, 0x06040200u) ^ 0x80808080u;
+      lo[2 * j + 1] = __builtin_amdgcn_perm(v.w, v.z, 0x06040200u) ^ 0x80808080u;
+    }
+    uint8_t* d = a.dst + ((o * a.k16 + t) * 32 + r) * 16;
+    *(u32x4*)d = u32x4{hi[0], hi[1], hi[2], hi[3]};
+    *(u32x4*)(d + plane) = u32x4{lo[0], lo[1], lo[2], lo[3]};
+    if (o == 0) *(u32x4*)(d + 2 * plane) = u32x4{0x40404040u, 0x40404040u, 0x40404040u, 0x40404040u};
+  }
+}
+
 struct CombineArgs {
   const uint32_t* product;   // (2 M + 1) x cols tiles of 32 x 32
   int64_t M, N, cols;        // cols = N (narrow rhs) or 2 N + 1
@@ -164,13 +195,34 @@ int launch_mmt4d_s16_planes(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) 
   uint8_t* rhs8 = lhs8 + lhs_bytes;
   uint32_t* product = (uint32_t*)(rhs8 + rhs_bytes);
 
+  // whole 16-byte runs of a 16-bit operand, 16-byte aligned, no ragged last tile
+  auto wide = [&](const void* buffer, int64_t offset, int64_t stride0) {
+    return p.K0 % 8 == 0 && kk0 % 16 == 0 && offset % 8 == 0 && stride0 % 8 == 0 && (uintptr_t)buffer % 16 == 0;
+  };
   const RetileArgs la = {p.lhs_buffer, p.lhs_offset, p.lhs_stride0, p.M, p.K, p.K0, k16, lhs8};
-  UK_RETURN_IF_ERROR(launch_grid_stride(retile_planes_kernel<kSourceS16>, la, p.M * k16 * 32, s,
-                                        "mmt4d digit planes (lhs) launch"));
+  if (wide(p.lhs_buffer, p.lhs_offset, p.lhs_stride0)) {
+    UK_RETURN_IF_ERROR(launch_grid_stride(retile_planes_s16_wide_kernel, la, p.M * k16 * 32, s,
+                                          "mmt4d digit planes (lhs) launch"));
+  } else {
+    UK_RETURN_IF_ERROR(launch_grid_stride(retile_planes_kernel<kSourceS16>, la, p.M * k16 * 32, s,
+                                          "mmt4d digit planes (lhs) launch"));
+  }
   const RetileArgs ra = {p.rhs_buffer, p.rhs_offset, p.rhs_stride0, p.N, p.K, p.K0, k16, rhs8};
+  const uint8_t* rhs_operand = rhs8;
+  int64_t rhs_operand_stride = k16 * 512;
   if (wide_rhs) {
-    UK_RETURN_IF_ERROR(launch_grid_stride(retile_planes_kernel<kSourceS16>, ra, p.N * k16 * 32, s,
-                                          "mmt4d digit planes (rhs) launch"));
+    if (wide(p.rhs_buffer, p.rhs_offset, p.rhs_stride0)) {
+      UK_RETURN_IF_ERROR(launch_grid_stride(retile_planes_s16_wide_kernel, ra, p.N * k16 * 32, s,
+                                            "mmt4d digit planes (rhs) launch"));
+    } else {
+      UK_RETURN_IF_ERROR(launch_grid_stride(retile_planes_kernel<kSourceS16>, ra, p.N * k16 * 32, s,
+                                            "mmt4d digit planes (rhs) launch"));
+    }
+  } else if (type == IREE_AMD_UK_FLAG_MMT4D_TYPE_S16S8S32 && p.K0 == 16 && p.rhs_offset % 16 == 0 &&
+             p.rhs_stride0 % 16 == 0 && (uintptr_t)p.rhs_buffer % 16 == 0) {
+    // (already what the matrix-core kernel takes: used where it lies)
+    rhs_operand = (const uint8_t*)p.rhs_buffer + p.rhs_offset;
+    rhs_operand_stride = p.rhs_stride0;
   } else if (type == IREE_AMD_UK_FLAG_MMT4D_TYPE_S16S8S32) {
     UK_RETURN_IF_ERROR(launch_grid_stride(retile_planes_kernel<kSourceS8>, ra, p.N * k16 * 32, s,
                                           "mmt4d 8-bit rhs re-tiling launch"));
@@ -179,7 +231,7 @@ int launch_mmt4d_s16_planes(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) 
                                           "mmt4d 4-bit rhs widening launch"));
   }
 
-  iree_amd_uk_mmt4d_params_t q = {lhs8, 0, k16 * 512, rhs8, 0, k16 * 512, product, 0, rhs_rows * 1024,
+  iree_amd_uk_mmt4d_params_t q = {lhs8, 0, k16 * 512, rhs_operand, 0, rhs_operand_stride, product, 0, rhs_rows * 1024,
                                   lhs_rows, rhs_rows, k16, 32, 32, 16, IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32,
                                   nullptr};
   {

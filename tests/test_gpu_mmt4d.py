@@ -155,7 +155,7 @@ def test_s16_on_the_matrix_cores_bit_exact(uk, cuda, type_flag):
     assert uk.mmt4d_info(32, 32, 8, type_flag) == 1
     assert uk.mmt4d_info(32, 32, 2, type_flag) == 1
     assert uk.mmt4d_info(16, 16, 2, type_flag) == 0
-    for M, N, K, K0, acc in ((4, 4, 128, 8, False), (3, 7, 100, 8, True), (5, 5, 400, 2, False),
+    for M, N, K, K0, acc in ((4, 4, 128, 8, False), (3, 7, 100, 8, True), (4, 5, 129, 8, True), (5, 5, 400, 2, False),
                              (4, 5, 150 if even else 300, 6 if even else 3, True), (2, 9, 70, 16, False),
                              (1, 1, 3, 8, True)):
         for gen in (ukref.random_operand, _full_range_operand):
