@@ -70,10 +70,11 @@ def test_decode_shape_llama_ffn(uk, cuda, M, tiled):
                                   (4096, 1024), (4096, 4096)])
 @pytest.mark.parametrize("zp_u4", [False, True])
 def test_mfma_kernel_group_sizes_and_zero_point_forms(uk, cuda, K, gs, zp_u4):
-    # (rows: up to 8 stage the activations through LDS, 9..16 and 17..32 fetch
-    # them into registers; 40 = a pass of 32 and one of 8 from row 32 on)
+    # (rows: up to 16 stage the activations through LDS in one go, 8 or 16 rows
+    # per wave; 17..32 in phases of 8 rows, three phases up to 24 rows and four
+    # beyond; 40 = a pass of 32 and one of 8 from row 32 on)
     for M, N, tiled in [(3, 96, True), (32, 64, False), (40, 100, False), (17, 160, True), (12, 64, True),
-                        (8, 32, False), (9, 64, False)]:
+                        (8, 32, False), (9, 64, False), (24, 96, False), (25, 64, True), (31, 64, False)]:
         run_case(uk, M, N, K, gs, zp_u4, tiled, seed=K + gs)
 
 
