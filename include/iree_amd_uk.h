@@ -322,6 +322,40 @@ IREE_AMD_UK_EXPORT int iree_amd_uk_unpack_p(
     const iree_amd_uk_unpack_params_t* params, void* stream);
 
 /*===------------------------------------------------------------------------===
+ * The compile-time side of tile selection, as two host-only functions with the
+ * structure of the reference's (a compiler that materialises encodings for
+ * gfx950 would call these where the CPU one calls its own).
+ *
+ * enumerate_matmul_tiles: the tiles the gfx950 kernels serve for an operation
+ * (an IREE_AMD_UK_FLAG_QUERY_TILE_SIZES_OPERATION_* value): the full
+ * 32 x 32 x K0 tile first, then its truncations in M to 16, 8, 4, 2, 1
+ * (REF CPUMaterializeEncodingPass.cpp:168-281 enumerateMatmulTile*: every
+ * target lists the tile aimed at its instruction and "Truncation of the above"
+ * entries). Writes at most `capacity` tiles, *out_count = how many there are.
+ *
+ * choose_matmul_tile: REF CPUMaterializeEncodingPass.cpp:284-377
+ * chooseMatmulTile, rule for rule. narrow_m / narrow_n: the static size of a
+ * narrow dimension, 0 when it is not narrow. A narrow N that is narrower than
+ * M (or the only narrow one) is reduced to the narrow-M case and the chosen
+ * tile's M and N are exchanged. Tiles beyond `upper_bound` (3 values M, N, K;
+ * NULL = none) are skipped; of the rest, those with the least padding penalty
+ * max(tile.M - PowerOf2Ceil(narrow_m), 0) are kept, and of those the first
+ * with the largest M * N * K wins. NOT_FOUND when every tile was skipped.
+ * iree_amd_uk_query_tile_sizes_2d below answers with exactly these choices.
+ *===------------------------------------------------------------------------===*/
+typedef struct iree_amd_uk_matmul_tile_t {
+  int32_t M, N, K;
+} iree_amd_uk_matmul_tile_t;
+
+IREE_AMD_UK_EXPORT int iree_amd_uk_enumerate_matmul_tiles(
+    uint32_t operation, iree_amd_uk_matmul_tile_t* tiles, int32_t capacity, int32_t* out_count);
+
+IREE_AMD_UK_EXPORT int iree_amd_uk_choose_matmul_tile(
+    const iree_amd_uk_matmul_tile_t* tiles, int32_t count, iree_amd_uk_index_t narrow_m,
+    iree_amd_uk_index_t narrow_n, const iree_amd_uk_index_t* upper_bound,
+    iree_amd_uk_matmul_tile_t* out_tile);
+
+/*===------------------------------------------------------------------------===
  * query_tile_sizes_2d: (operation, operand role) -> (tile_size0, tile_size1).
  * LHS -> (M0,K0), RHS -> (N0,K0), RESULT -> (M0,N0) of the matmul tile chosen
  * for gfx950 (REF query_tile_sizes.c:43-63 for the role mapping).

@@ -18,6 +18,8 @@ from .ukernel import (  # noqa: F401
     quantize_groups_i16,
     copy_probe,
     batch_matmul_packed_rhs,
+    choose_matmul_tile,
+    enumerate_matmul_tiles,
     batch_mmt4d,
     batch_mmt4d_unpack,
     mmt4d,

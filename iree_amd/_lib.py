@@ -59,6 +59,11 @@ class UnpackParams(C.Structure):
     ]
 
 
+class MatmulTile(C.Structure):
+    """iree_amd_uk_matmul_tile_t."""
+    _fields_ = [("M", C.c_int32), ("N", C.c_int32), ("K", C.c_int32)]
+
+
 class QueryParams(C.Structure):
     _fields_ = [("flags", C.c_uint32), ("size0", index_t), ("size1", index_t),
                 ("cpu_data", C.c_void_p)]
@@ -97,6 +102,12 @@ def _declare(lib):
                                         i64, i64, i64, i64, i64, i64, u32, vp, vp]
     lib.iree_amd_uk_unpack_p.restype = C.c_int
     lib.iree_amd_uk_unpack_p.argtypes = [C.POINTER(UnpackParams), vp]
+    lib.iree_amd_uk_enumerate_matmul_tiles.restype = C.c_int
+    lib.iree_amd_uk_enumerate_matmul_tiles.argtypes = [C.c_uint32, C.POINTER(MatmulTile), C.c_int32,
+                                                       C.POINTER(C.c_int32)]
+    lib.iree_amd_uk_choose_matmul_tile.restype = C.c_int
+    lib.iree_amd_uk_choose_matmul_tile.argtypes = [C.POINTER(MatmulTile), C.c_int32, i64, i64,
+                                                   C.POINTER(C.c_int64), C.POINTER(MatmulTile)]
     lib.iree_amd_uk_query_tile_sizes_2d.restype = C.c_int
     lib.iree_amd_uk_query_tile_sizes_2d.argtypes = [C.POINTER(QueryParams),
                                                      C.POINTER(QueryOutParams)]

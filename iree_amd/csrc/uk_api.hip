@@ -417,6 +417,73 @@ extern "C" int iree_amd_uk_query_tile_sizes_2d(
   }
 }
 
+extern "C" int iree_amd_uk_enumerate_matmul_tiles(uint32_t operation, iree_amd_uk_matmul_tile_t* tiles,
+                                                  int32_t capacity, int32_t* out_count) {
+  if (!out_count || capacity < 0 || (capacity > 0 && !tiles))
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "enumerate_matmul_tiles: null argument or negative capacity");
+  MatmulTile t;
+  if (!matmul_tile_for_op(operation & IREE_AMD_UK_FLAG_QUERY_TILE_SIZES_OPERATION_MASK, &t))
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "enumerate_matmul_tiles: unknown operation 0x%x", operation);
+  int32_t n = 0;
+  for (int m = t.M0; m >= 1; m >>= 1, ++n)
+    if (n < capacity) tiles[n] = {m, t.N0, t.K0};
+  *out_count = n;
+  return 0;
+}
+
+namespace {
+int64_t power_of_2_ceil(int64_t v) {
+  int64_t p = 1;
+  while (p < v) p <<= 1;
+  return p;
+}
+}  // namespace
+
+extern "C" int iree_amd_uk_choose_matmul_tile(const iree_amd_uk_matmul_tile_t* tiles, int32_t count,
+                                              iree_amd_uk_index_t narrow_m, iree_amd_uk_index_t narrow_n,
+                                              const iree_amd_uk_index_t* upper_bound,
+                                              iree_amd_uk_matmul_tile_t* out_tile) {
+  if (!tiles || !out_tile || count <= 0 || narrow_m < 0 || narrow_n < 0)
+    return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "choose_matmul_tile: null argument, no tiles or a negative size");
+  // narrow N: reduce to narrow M, exchange M and N of the answer
+  if (narrow_n && (!narrow_m || narrow_n < narrow_m)) {
+    const int st = iree_amd_uk_choose_matmul_tile(tiles, count, narrow_n, 0, upper_bound, out_tile);
+    if (st) return st;
+    const int32_t m = out_tile->M;
+    out_tile->M = out_tile->N;
+    out_tile->N = m;
+    return 0;
+  }
+  int64_t best_penalty = INT64_MAX;
+  for (int pass = 0; pass < 2; ++pass) {
+    int64_t best_product = 0;
+    bool found = false;
+    for (int32_t i = 0; i < count; ++i) {
+      const iree_amd_uk_matmul_tile_t& t = tiles[i];
+      if (upper_bound && (t.M > upper_bound[0] || t.N > upper_bound[1] || t.K > upper_bound[2])) continue;
+      int64_t penalty = 0;
+      if (narrow_m) {
+        penalty = (int64_t)t.M - power_of_2_ceil(narrow_m);
+        if (penalty < 0) penalty = 0;
+      }
+      if (pass == 0) {
+        if (penalty < best_penalty) best_penalty = penalty;
+        found = true;
+      } else if (penalty == best_penalty) {
+        const int64_t product = (int64_t)t.M * t.N * t.K;
+        if (best_product < product) {
+          best_product = product;
+          *out_tile = t;
+          found = true;
+        }
+      }
+    }
+    if (!found)
+      return fail(IREE_AMD_UK_STATUS_NOT_FOUND, "choose_matmul_tile: no tile within the upper bound");
+  }
+  return 0;
+}
+
 //===----------------------------------------------------------------------===//
 // int4 dequant matmul, fp8 helpers
 //===----------------------------------------------------------------------===//

@@ -12,7 +12,7 @@ import ctypes as C
 import torch
 
 from . import flags as F
-from ._lib import (Mmt4dParams, PackParams, QueryOutParams, QueryParams,
+from ._lib import (MatmulTile, Mmt4dParams, PackParams, QueryOutParams, QueryParams,
                    UnpackParams, load_library)
 
 
@@ -144,6 +144,27 @@ def query_tile_sizes_2d(flags, size0=_INT64_MIN, size1=_INT64_MIN):
     o = QueryOutParams()
     _check(load_library().iree_amd_uk_query_tile_sizes_2d(C.byref(p), C.byref(o)))
     return int(o.tile_size0), int(o.tile_size1)
+
+
+def enumerate_matmul_tiles(operation):
+    """The (M, N, K) tiles the gfx950 kernels serve for a QUERY_OP_* operation:
+    the full tile and its truncations in M (the reference's
+    enumerateMatmulTile*, CPUMaterializeEncodingPass.cpp:168-281)."""
+    n = C.c_int32(0)
+    _check(load_library().iree_amd_uk_enumerate_matmul_tiles(operation, None, 0, C.byref(n)))
+    tiles = (MatmulTile * n.value)()
+    _check(load_library().iree_amd_uk_enumerate_matmul_tiles(operation, tiles, n.value, C.byref(n)))
+    return [(t.M, t.N, t.K) for t in tiles]
+
+
+def choose_matmul_tile(tiles, narrow_m=0, narrow_n=0, upper_bound=None):
+    """The reference's chooseMatmulTile (CPUMaterializeEncodingPass.cpp:284-377)
+    over a list of (M, N, K) tiles; returns the chosen (M, N, K)."""
+    arr = (MatmulTile * max(len(tiles), 1))(*[MatmulTile(*t) for t in tiles])
+    ub = (C.c_int64 * 3)(*upper_bound) if upper_bound is not None else None
+    out = MatmulTile()
+    _check(load_library().iree_amd_uk_choose_matmul_tile(arr, len(tiles), narrow_m, narrow_n, ub, C.byref(out)))
+    return out.M, out.N, out.K
 
 
 def dequant_matmul_i4(x, w, scale, zp, out, M, N, K, group_size, flags=0,

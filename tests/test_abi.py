@@ -154,6 +154,75 @@ def test_mmt4d_info_reports_mfma_tiles():
     assert iree_amd.mmt4d_info(1, 32, 8, F.MMT4D_TYPE_S16U4S32) == 0
 
 
+def test_enumerated_tiles_and_the_chooser_follow_the_reference():
+    """enumerate_matmul_tiles / choose_matmul_tile against what
+    CPUMaterializeEncodingPass.cpp:168-377 documents: tile lists are the full
+    tile and its truncations in M; the example of its comment (narrow M = 7 with
+    tiles of M = 8, 4, 2, 1 keeps M = 8); the reference's own avx512 f32 list
+    for matvec / vecmat shapes; narrow N reduced to narrow M with M and N
+    exchanged; upper bounds; and a brute-force restatement of the rating rule
+    on random tile lists. query_tile_sizes_2d answers with the chooser's tile."""
+    import itertools
+    import random
+    assert iree_amd.enumerate_matmul_tiles(F.QUERY_OP_MATMUL_F16F16F32) == [
+        (32, 32, 8), (16, 32, 8), (8, 32, 8), (4, 32, 8), (2, 32, 8), (1, 32, 8)]
+    assert iree_amd.enumerate_matmul_tiles(F.QUERY_OP_MATMUL_I8I8I32)[0] == (32, 32, 16)
+    assert iree_amd.enumerate_matmul_tiles(F.QUERY_OP_MATMUL_F32F32F32)[-1] == (1, 32, 4)
+    with pytest.raises(iree_amd.UkError):
+        iree_amd.enumerate_matmul_tiles(0x7F)
+    ch = iree_amd.choose_matmul_tile
+    assert ch([(8, 8, 1), (4, 8, 1), (2, 8, 1), (1, 8, 1)], narrow_m=7) == (8, 8, 1)
+    avx512 = [(16, 16, 1), (8, 16, 1), (4, 16, 1), (2, 16, 1), (1, 16, 1)]     # its lines 195-201
+    assert ch(avx512) == (16, 16, 1)
+    assert ch(avx512, narrow_m=1) == (1, 16, 1)
+    assert ch(avx512, narrow_n=1) == (16, 1, 1)
+    assert ch(avx512, narrow_m=3) == (4, 16, 1)
+    assert ch(avx512, narrow_m=5, narrow_n=2) == (16, 2, 1)      # N the narrower: exchanged
+    assert ch(avx512, narrow_m=2, narrow_n=5) == (2, 16, 1)
+    assert ch(avx512, narrow_m=4, narrow_n=4) == (4, 16, 1)      # a tie stays a narrow-M problem
+    assert ch(avx512, upper_bound=(4, 16, 1)) == (4, 16, 1)
+    assert ch(avx512, narrow_m=1, upper_bound=(8, 16, 1)) == (1, 16, 1)
+    with pytest.raises(iree_amd.UkError):
+        ch(avx512, upper_bound=(16, 8, 1))
+
+    def pow2ceil(v):
+        return 1 << (v - 1).bit_length() if v > 1 else 1
+
+    def restated(tiles, nm, nn, ub):
+        if nn and (not nm or nn < nm):
+            m, n, k = restated(tiles, nn, 0, ub)
+            return n, m, k
+        ok = [t for t in tiles if ub is None or (t[0] <= ub[0] and t[1] <= ub[1] and t[2] <= ub[2])]
+        pen = [max(t[0] - pow2ceil(nm), 0) if nm else 0 for t in ok]
+        best = [t for t, p in zip(ok, pen) if p == min(pen)]
+        return max(best, key=lambda t: t[0] * t[1] * t[2])       # (max keeps the first of equals)
+
+    rnd = random.Random(5)
+    for _ in range(300):
+        tiles = [(rnd.choice([1, 2, 4, 8, 16, 32]), rnd.choice([4, 8, 16, 32]), rnd.choice([1, 2, 4, 8, 16]))
+                 for _ in range(rnd.randint(1, 7))]
+        nm, nn = rnd.choice([0, 0, 1, 3, 7, 8, 20]), rnd.choice([0, 0, 1, 2, 5, 16])
+        ub = rnd.choice([None, None, (32, 32, 16), (8, 32, 16)])
+        try:
+            want = restated(tiles, nm, nn, ub)
+        except ValueError:
+            with pytest.raises(iree_amd.UkError):
+                ch(tiles, nm, nn, ub)
+            continue
+        assert ch(tiles, nm, nn, ub) == want, (tiles, nm, nn, ub)
+    # the run-time query is this chooser on the enumerated tiles
+    q = iree_amd.query_tile_sizes_2d
+    for op in (F.QUERY_OP_MATMUL_I8I8I32, F.QUERY_OP_MATMUL_F16F16F32, F.QUERY_OP_MATMUL_F32F32F32,
+               F.QUERY_OP_MATMUL_F8E4M3F8E4M3F32):
+        tiles = iree_amd.enumerate_matmul_tiles(op)
+        for m, n in itertools.product([1, 2, 3, 7, 8, 15, 17, 31, 32, 500], repeat=2):
+            narrow_m, narrow_n = (m if m < 32 else 0), (n if n < 32 else 0)
+            M0, N0, K0 = ch(tiles, narrow_m, narrow_n)
+            assert q(op | F.QUERY_ROLE_RESULT, m, n) == (M0, N0), (hex(op), m, n)
+            assert q(op | F.QUERY_ROLE_LHS, m if M0 < 32 else -2 ** 63, 4096) == (M0, K0)
+            assert q(op | F.QUERY_ROLE_RHS, n if N0 < 32 else -2 ** 63, 4096) == (N0, K0)
+
+
 def test_every_tile_the_query_returns_has_an_architecture_kernel():
     """mmt4d_info reports a matrix-core kernel for each tile
     query_tile_sizes_2d can hand out: full tiles, narrow M0 (static M < 32) and
