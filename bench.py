@@ -349,11 +349,15 @@ def extras(args, torch, iree_amd, F, synth, lhs, rhs, out, ex):
     lib = iree_amd.load_library()
     pool = C.c_void_p()
     assert lib.iree_amd_uk_host_pool_create(C.byref(pool)) == 0
-    assert lib.iree_amd_uk_mmt4d_host_pooled(pool, C.byref(hp)) == 0
-    t0 = time.perf_counter()
-    for _ in range(5):
+    # (the first calls pay for the first touch of the result's pages and for the
+    # staging buffers the runtime sets up per copying thread: 4-5 ms each
+    # against 2.8 ms from about the sixth call on)
+    for _ in range(6):
         assert lib.iree_amd_uk_mmt4d_host_pooled(pool, C.byref(hp)) == 0
-    ex["mmt4d_f16_host_pointers_tflops"] = round(flops / ((time.perf_counter() - t0) / 5) / 1e12, 2)
+    t0 = time.perf_counter()
+    for _ in range(10):
+        assert lib.iree_amd_uk_mmt4d_host_pooled(pool, C.byref(hp)) == 0
+    ex["mmt4d_f16_host_pointers_tflops"] = round(flops / ((time.perf_counter() - t0) / 10) / 1e12, 2)
     assert np.array_equal(oh, out.cpu().numpy()), "host-pointer mmt4d differs from the device entry point"
     lib.iree_amd_uk_host_pool_destroy(pool)
     oh[:] = 0
