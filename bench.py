@@ -863,28 +863,30 @@ def run_only(args, torch, iree_amd, F, synth, mm_step):
         fn = lambda: iree_amd.matmul_data_tiled(a8, b8, c8, n1k, n1k, n1k, F.MMT4D_TYPE_S8S8S32,  # noqa: E731
                                                 workspace=ws8)
     elif args.only == "pack_transpose":
-        # the right-hand side of the 4096^3 f16 matmul given as B[K][N]: 32x8 tiles, inner and outer transposed
+        # the right-hand side of the 4096^3 f16 matmul given as B[K][N]: 32x8 tiles, inner and outer
+        # transposed; 8 rotating buffer sets (512 MiB) so that the 256 MiB last-level cache serves nothing
         size = 4096
-        b = torch.from_numpy(synth.normal_f16(2, size * size, 1 / 64).view(np.int16)).cuda()
-        pb = [torch.empty(size * size, dtype=torch.int16, device="cuda") for _ in range(4)]
+        bs = [torch.from_numpy(synth.normal_f16(2 + i, size * size, 1 / 64).view(np.int16)).cuda() for i in range(8)]
+        pb = [torch.empty(size * size, dtype=torch.int16, device="cuda") for _ in range(8)]
         st = {"i": 0}
 
         def fn():
-            k = st["i"] % 4
+            k = st["i"] % 8
             st["i"] += 1
-            iree_amd.pack(b, pb[k], size, size, size // 32, size // 8, 32, 8, 0,
+            iree_amd.pack(bs[k], pb[k], size, size, size // 32, size // 8, 32, 8, 0,
                           F.PACK_TYPE_F16F16 | F.PACK_TRANSPOSE_INNER | F.PACK_TRANSPOSE_OUTER)
     elif args.only == "unpack_transpose":
-        # a 4096 x 4096 f32 result held as 32x32 tiles stored column by column (inner transposed)
+        # a 4096 x 4096 f32 result held as 32x32 tiles stored column by column (inner transposed);
+        # 4 rotating buffer sets (512 MiB)
         size = 4096
-        tiles = torch.from_numpy(synth.normal_f32(3, size * size, 1.0)).cuda()
+        tiles = [torch.from_numpy(synth.normal_f32(3 + i, size * size, 1.0)).cuda() for i in range(4)]
         mats = [torch.empty(size * size, dtype=torch.float32, device="cuda") for _ in range(4)]
         st = {"i": 0}
 
         def fn():
             k = st["i"] % 4
             st["i"] += 1
-            iree_amd.unpack(tiles, mats[k], size // 32, size // 32, 32, 32, size, size,
+            iree_amd.unpack(tiles[k], mats[k], size // 32, size // 32, 32, 32, size, size,
                             F.UNPACK_TYPE_F32F32 | F.UNPACK_TRANSPOSE_INNER)
     elif args.only == "mlp_fp8":
         mlp, xm, ym, Mt, _, _ = make_fp8_mlp(torch, iree_amd)

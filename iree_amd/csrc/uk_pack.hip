@@ -294,6 +294,8 @@ template <int ES>
 __global__ __launch_bounds__(256) void pack_transpose_kernel(TransArgs a) { pack_transpose_body<ES>(a); }
 template <int ES>
 __global__ __launch_bounds__(256) void unpack_transpose_kernel(TransArgs a) { unpack_transpose_body<ES>(a); }
+template <int ES>
+__global__ __launch_bounds__(256) void pack_transpose_wide_kernel(TransArgs a) { pack_transpose_wide_body<ES>(a); }
 
 template <int ES>
 int launch_unpack_transpose(TransArgs a, hipStream_t s) {
@@ -308,10 +310,20 @@ int launch_unpack_transpose(TransArgs a, hipStream_t s) {
 
 template <int ES>
 int launch_pack_transpose(TransArgs a, hipStream_t s) {
-  const int64_t bx = ceil_div(a.padded_cols, (int64_t)64);
+  // 1- and 2-byte elements: dword loads where every row starts on a 4-byte
+  // boundary and tiles are whole dwords of columns
+  constexpr int W = ES < 4 ? 4 / ES : 1;
+  const bool wide = W > 1 && a.tile_cols % W == 0 && (uintptr_t)a.mat % 4 == 0 && a.m_pitch_bytes % 4 == 0;
+  const int64_t bx = ceil_div(a.padded_cols, (int64_t)64 * (wide ? W : 1));
   const int64_t by = ceil_div(a.row_groups, (int64_t)(4 * kTransUnroll));
   if (bx < 1 || by < 1 || bx * by > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
   a.blocks_x = (uint32_t)bx; a.blocks_y = (uint32_t)by;
+  if constexpr (W > 1) {
+    if (wide) {
+      hipLaunchKernelGGL((pack_transpose_wide_kernel<ES>), dim3((unsigned)(bx * by)), dim3(256), 0, s, a);
+      return check_hip(hipGetLastError(), "pack_transpose launch");
+    }
+  }
   hipLaunchKernelGGL((pack_transpose_kernel<ES>), dim3((unsigned)(bx * by)), dim3(256), 0, s, a);
   return check_hip(hipGetLastError(), "pack_transpose launch");
 }

@@ -82,6 +82,11 @@ def test_streaming_shapes_with_ragged_edges(uk, cuda, type_flag, t0, t1, rows, c
     (F.PACK_TYPE_I8I8, 32, 32, 4096, 64),
     (F.PACK_TYPE_F32F32, 4, 32, 515, 70),
     (F.PACK_TYPE_BF16BF16, 24, 5, 123, 77),    # odd tile width, three row groups
+    # rows that start on 4-byte boundaries: the kernel with dword loads, whole and ragged blocks
+    (F.PACK_TYPE_F16F16, 8, 32, 1000, 520),
+    (F.PACK_TYPE_I8I8, 16, 32, 1003, 772),
+    (F.PACK_TYPE_BF16BF16, 16, 64, 300, 1028),
+    (F.PACK_TYPE_I8I8, 32, 8, 200, 1024),
 ])
 def test_transposing_pack_with_ragged_edges(uk, cuda, type_flag, tr, tc, rows, cols):
     """Packs with transposed inner tiles (what the right-hand side B[K][N] of a
