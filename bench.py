@@ -375,6 +375,26 @@ def extras(args, torch, iree_amd, F, synth, lhs, rhs, out, ex):
                     steps, warm)
     ex["mmt4d_f16_accumulate_tflops"] = round(flops / t / 1e12, 2)
 
+    # Reference points from the vendor library (hipBLASLt through torch) on the
+    # same operand bits, viewed as row-major A[4096][4096] and B[4096][4096]
+    # (C = A B^T): the same contraction with an f32 result, which is the
+    # headline operation, and with an f16 result; and this library's f16 -> f16.
+    # Comparisons only: nothing of this library runs through torch's matmul.
+    a2, b2 = lhs.view(size, size), rhs.view(size, size)
+    try:
+        _, t = gpu_time(torch, lambda: torch.mm(a2, b2.t(), out_dtype=torch.float32), steps, warm)
+        ex["vendor_gemm_f16_f32out_tflops"] = round(flops / t / 1e12, 2)
+    except Exception:       # (a torch without out_dtype)
+        pass
+    _, t = gpu_time(torch, lambda: torch.matmul(a2, b2.t()), steps, warm)
+    ex["vendor_gemm_f16_f16out_tflops"] = round(flops / t / 1e12, 2)
+    out16 = torch.empty(M1 * N1 * 1024, dtype=torch.float16, device="cuda")
+    f16_flags = F.MMT4D_TYPE_F16F16F16 | F.MMT4D_SKIP_INTERMEDIATE_ROUNDINGS
+    _, t = gpu_time(torch, lambda: iree_amd.mmt4d(lhs, rhs, out16, M1, N1, size // 8, 32, 32, 8, f16_flags),
+                    steps, warm)
+    ex["mmt4d_f16f16f16_tflops"] = round(flops / t / 1e12, 2)
+    del out16, a2, b2
+
     # A shape of few macro tiles and a long K (256 rows of activations against a
     # 4096 x 14336 down projection): K is split over workgroup rows.
     Ms, Ns, Ks = 256, 4096, 14336
