@@ -95,8 +95,8 @@ __global__ __launch_bounds__(kThreads) void dequant_matmul_i4_kernel(I4Args a) {
   constexpr int SW = (SB + 3) / 4, ZW = (ZB + 3) / 4;
   // Nibbles as f16 subnormals and the zero point applied through the group sums
   // of the activations (see nibbles_as_subnormals), where those sums fit the
-  // register file: up to 8 accumulators of 4 registers.
-  constexpr bool kSubnormal = GW * MH <= 8;
+  // register file: up to 8 accumulators of 4 registers, 16 in the 16-row form.
+  constexpr bool kSubnormal = GW * MH <= 8 || (MH == 1 && GW <= 16);
   // Both forms stage the activations through dynamic LDS. The 16-row form keeps
   // the per-wave partial sums in static LDS next to it; in the 32-row form they
   // take over the staging area once the first tile has been multiplied.
