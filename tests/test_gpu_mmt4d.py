@@ -165,6 +165,15 @@ def test_s16_on_the_matrix_cores_bit_exact(uk, cuda, type_flag):
     case = ukref.Mmt4dCase(rng, type_flag, 5, 6, 90, 32, 32, 8, accumulate=True, loose_strides=True, offsets=True,
                            generator=_full_range_operand)
     assert np.array_equal(gpucase.run_mmt4d(case), case.run_oracle())
+    # random K0, outer counts, strides and offsets, every case above the size threshold
+    for _ in range(10):
+        K0 = int(rng.choice([2, 4, 6, 8, 10, 16, 24, 32])) if even else int(rng.choice([1, 2, 3, 4, 5, 8, 16, 17, 32]))
+        M, N = int(rng.integers(1, 9)), int(rng.integers(1, 9))
+        K = -(-(1 << 24) // (M * N * 1024 * K0)) + int(rng.integers(0, 5))
+        case = ukref.Mmt4dCase(rng, type_flag, M, N, K, 32, 32, K0, accumulate=bool(rng.integers(0, 2)),
+                               loose_strides=bool(rng.integers(0, 2)), offsets=bool(rng.integers(0, 2)),
+                               generator=_full_range_operand)
+        assert np.array_equal(gpucase.run_mmt4d(case), case.run_oracle()), (M, N, K, K0)
 
 
 @pytest.mark.parametrize("type_flag,K0", [(F.MMT4D_TYPE_F16F16F32, 8), (F.MMT4D_TYPE_F16F16F32, 16),
