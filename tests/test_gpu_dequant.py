@@ -228,8 +228,11 @@ def run_reassoc_case(uk, M, N, K, gs, zp_u4, tiled, seed=0):
     pf = plain.view(np.float16).astype(np.float64)
     dev = np.abs(got - pf)
     assert np.all(dev <= 2 * ATOL + RTOL * np.abs(pf)), (M, N, K, gs, float(dev.max()))
-    # (the share grows with the number of truncated terms: K = 16384 gives 2e-4)
-    assert np.mean(dev > ATOL + RTOL * np.abs(pf)) <= 1e-4 * max(1, K // 4096), (M, N, K, gs)
+    # (the share grows with the number of truncated terms: K = 16384 gives 2e-4;
+    # a small result may hold one such element whatever its size: 1 of 2520
+    # at 15 x 168, where the oracle of the rewrite has the same one)
+    outside = int(np.count_nonzero(dev > ATOL + RTOL * np.abs(pf)))
+    assert outside <= max(1, int(1e-4 * max(1, K // 4096) * dev.size)), (M, N, K, gs, outside)
 
 
 @pytest.mark.parametrize("M", [1, 8, 32])
