@@ -221,18 +221,22 @@ def run_reassoc_case(uk, M, N, K, gs, zp_u4, tiled, seed=0):
     # Against the plain (unreassociated) float64 oracle: the rewrite itself
     # loses precision (16-bit activations, truncated; the reference says so,
     # FuseDequantizationMatmul.cpp:746-748), about 5e-4 absolute at these
-    # magnitudes, so results near zero can leave the stated bound by a hair
-    # (the oracle of the rewrite does the same: 1 of 114688 at 8 rows). Held:
-    # the stated bound for all but one in ten thousand (per 4096 of K), twice its absolute
-    # part for every element.
+    # magnitudes for groups of 128 and K = 4096, more with longer K (more
+    # truncated terms) and with larger groups (truncation biases every term of a
+    # group the same way, and one scale serves more activations: a single
+    # group of 6144 reached 0.016). So results near zero can leave the stated
+    # bound, and the oracle of the rewrite leaves it at the same elements.
+    # Held: for every element twice the absolute part of the stated bound,
+    # scaled by K / 4096 and by the group size / 512 where those exceed 1; the
+    # stated bound itself for all but two in a thousand (1 of 114688 at the
+    # decode shape; running the random sweeps under 160 other seeds gave up to
+    # 3 of 3247), and a small result may hold three whatever its size.
     pf = plain.view(np.float16).astype(np.float64)
     dev = np.abs(got - pf)
-    assert np.all(dev <= 2 * ATOL + RTOL * np.abs(pf)), (M, N, K, gs, float(dev.max()))
-    # (the share grows with the number of truncated terms: K = 16384 gives 2e-4;
-    # a small result may hold one such element whatever its size: 1 of 2520
-    # at 15 x 168, where the oracle of the rewrite has the same one)
+    scale = max(1, K // 4096) * max(1, gs // 512)
+    assert np.all(dev <= 2 * ATOL * scale + RTOL * np.abs(pf)), (M, N, K, gs, float(dev.max()))
     outside = int(np.count_nonzero(dev > ATOL + RTOL * np.abs(pf)))
-    assert outside <= max(1, int(1e-4 * max(1, K // 4096) * dev.size)), (M, N, K, gs, outside)
+    assert outside <= max(3, int(2e-3 * dev.size)), (M, N, K, gs, outside)
 
 
 @pytest.mark.parametrize("M", [1, 8, 32])
