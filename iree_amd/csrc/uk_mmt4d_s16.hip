@@ -19,6 +19,11 @@
 // are re-tiled to K0 = 16 on the way (any K0 of the call; the K positions past
 // the end of a ragged K are zero in every plane, the constant one included), so
 // the matrix-core kernel always sees its preferred tile.
+//
+// Narrow left-hand side tiles (one outer row of 1..15 rows against an 8- or
+// 4-bit right-hand side: the reference's own s16 x u4 tile is 1 x 32 x 8,
+// arch/x86_64/mmt4d_x86_64_tiles.inl:75) take the same route through the narrow
+// matrix-core kernel: the planes are the 2 M0 + 1 rows of one int8 tile.
 #include "uk_common.h"
 
 namespace uk {
@@ -113,6 +118,26 @@ __global__ __launch_bounds__(256) void retile_planes_s16_wide_kernel(const Retil
   }
 }
 
+// The 4-bit right-hand side in tiles of K0 = 8 (the reference's s16 x u4 tile):
+// a tile row is one dword of 8 nibbles, and rows r of two consecutive K tiles
+// make one 16-byte row of the int8 tile. One thread per such row: two dword
+// loads, the nibbles spread over bytes with two ANDs and two byte permutes
+// each, one 16-byte store.
+__global__ __launch_bounds__(256) void retile_u4_k8_kernel(const RetileArgs a) {
+  const int64_t total = a.outer * a.k16 * 32;
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (int64_t)gridDim.x * blockDim.x) {
+    const int r = (int)(idx & 31);
+    const int64_t t = (idx >> 5) % a.k16, o = (idx >> 5) / a.k16;
+    const uint32_t* row = (const uint32_t*)((const uint8_t*)a.src + (a.offset + o * a.stride0) / 2) + (2 * t * 32 + r);
+    const uint32_t w0 = 2 * t < a.K ? row[0] : 0u, w1 = 2 * t + 1 < a.K ? row[32] : 0u;
+    const uint32_t lo0 = w0 & 0x0F0F0F0Fu, hi0 = (w0 >> 4) & 0x0F0F0F0Fu;
+    const uint32_t lo1 = w1 & 0x0F0F0F0Fu, hi1 = (w1 >> 4) & 0x0F0F0F0Fu;
+    *(u32x4*)(a.dst + idx * 16) = u32x4{__builtin_amdgcn_perm(hi0, lo0, 0x05010400u), __builtin_amdgcn_perm(hi0, lo0, 0x07030602u),
+                                        __builtin_amdgcn_perm(hi1, lo1, 0x05010400u), __builtin_amdgcn_perm(hi1, lo1, 0x07030602u)};
+  }
+}
+
 struct CombineArgs {
   const uint32_t* product;   // (2 M + 1) x cols tiles of 32 x 32
   int64_t M, N, cols;        // cols = N (narrow rhs) or 2 N + 1
@@ -149,6 +174,81 @@ __global__ __launch_bounds__(256) void combine_planes_kernel(const CombineArgs a
   }
 }
 
+// Narrow left-hand side tiles (M0 < 16 rows, one outer row: the reference's own
+// s16 x u4 tile is 1 x 32 x 8): the digit planes become the ROWS of one int8
+// tile of 2 M0 + 1 rows (h rows, l rows, the constant row), which the narrow
+// matrix-core kernel takes as it is.
+struct RetileNarrowArgs {
+  const int16_t* src;     // element 0 of the buffer
+  int64_t offset;         // of the single outer row
+  int64_t K;
+  int K0, M0;
+  int64_t k16;
+  uint8_t* dst;           // k16 tiles of (2 M0 + 1) rows x 16 bytes
+};
+
+__global__ __launch_bounds__(256) void retile_planes_narrow_kernel(const RetileNarrowArgs a) {
+  const int rows = 2 * a.M0 + 1;
+  const int64_t total = a.k16 * rows;
+  const int64_t kk0 = a.K * a.K0;
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (int64_t)gridDim.x * blockDim.x) {
+    const int r = (int)(idx % rows);
+    const int64_t t = idx / rows;
+    const int src_row = r < a.M0 ? r : r - a.M0;       // (unused for the constant row)
+    int64_t kt = (t * 16) / a.K0;
+    int k0 = (int)(t * 16 - kt * a.K0);
+    uint32_t out[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      if (t * 16 + e < kk0) {
+        uint32_t byte;
+        if (r == 2 * a.M0) {
+          byte = 64;
+        } else {
+          const int v = a.src[a.offset + (kt * a.M0 + src_row) * a.K0 + k0];
+          byte = r < a.M0 ? (uint32_t)((v >> 8) & 255) : (uint32_t)(((v & 255) - 128) & 255);
+        }
+        out[e >> 2] |= byte << (8 * (e & 3));
+      }
+      if (++k0 == a.K0) { k0 = 0; ++kt; }
+    }
+    *(u32x4*)(a.dst + idx * 16) = u32x4{out[0], out[1], out[2], out[3]};
+  }
+}
+
+struct CombineNarrowArgs {
+  const uint32_t* product;   // N tiles of (2 M0 + 1) x 32
+  int64_t N;
+  int M0;
+  uint32_t* out;             // N tiles of M0 x 32, offset applied
+  int accumulate;
+};
+
+__global__ __launch_bounds__(256) void combine_planes_narrow_kernel(const CombineNarrowArgs a) {
+  const int64_t total = a.N * a.M0 * 32;
+  const int rows = 2 * a.M0 + 1;
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (int64_t)gridDim.x * blockDim.x) {
+    const int c = (int)(idx & 31);
+    const int r = (int)((idx >> 5) % a.M0);
+    const int64_t j = (idx >> 5) / a.M0;
+    const uint32_t* t = a.product + j * rows * 32 + c;
+    const uint32_t v = t[r * 32] * 256u + t[(a.M0 + r) * 32] + t[2 * a.M0 * 32] * 2u;
+    a.out[idx] = a.accumulate ? a.out[idx] + v : v;
+  }
+}
+
+template <typename Kernel, typename Args>
+int launch_grid_stride(Kernel kernel, const Args& args, int64_t threads, hipStream_t s, const char* what);
+
+// The 4-bit right-hand side as int8 tiles of K0 = 16.
+int widen_u4_rhs(const RetileArgs& ra, hipStream_t s) {
+  const bool dwords = ra.K0 == 8 && ra.offset % 8 == 0 && ra.stride0 % 8 == 0 && (uintptr_t)ra.src % 4 == 0;
+  if (dwords) return launch_grid_stride(retile_u4_k8_kernel, ra, ra.outer * ra.k16 * 32, s, "mmt4d 4-bit rhs widening launch");
+  return launch_grid_stride(retile_planes_kernel<kSourceU4>, ra, ra.outer * ra.k16 * 32, s, "mmt4d 4-bit rhs widening launch");
+}
+
 template <typename Kernel, typename Args>
 int launch_grid_stride(Kernel kernel, const Args& args, int64_t threads, hipStream_t s, const char* what) {
   int64_t blocks = ceil_div(threads, (int64_t)256);
@@ -171,12 +271,54 @@ bool mmt4d_s16_planes_supported(uint32_t flags, int M0, int N0, int K0) {
   if (type != IREE_AMD_UK_FLAG_MMT4D_TYPE_S16S16S32 && type != IREE_AMD_UK_FLAG_MMT4D_TYPE_S16S8S32 &&
       type != IREE_AMD_UK_FLAG_MMT4D_TYPE_S16U4S32)
     return false;
-  return M0 == 32 && N0 == 32 && K0 >= 1 &&
-         mmt4d_mfma_supported(IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32, 32, 32, 16);
+  if (N0 != 32 || K0 < 1) return false;
+  if (M0 == 32) return mmt4d_mfma_supported(IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32, 32, 32, 16);
+  // narrow left-hand sides with an 8- or 4-bit right-hand side: 2 M0 + 1 plane rows in one narrow tile
+  return type != IREE_AMD_UK_FLAG_MMT4D_TYPE_S16S16S32 && M0 >= 1 && M0 <= 15 &&
+         mmt4d_skinny_supported(IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32, 2 * M0 + 1, 32, 16);
 }
+
+namespace {
+int launch_narrow(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) {
+  const uint32_t type = p.flags & IREE_AMD_UK_FLAG_MMT4D_TYPE_MASK;
+  const int64_t kk0 = p.K * p.K0;
+  if (p.M != 1 || p.K == 0 || (int64_t)p.M0 * 32 * p.N < ceil_div(kMinMacs / 2, kk0)) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  // (whole matrix-core steps of 32: the narrow kernel takes nothing else; the
+  // positions past the end of K are zero in every plane)
+  const int64_t k16 = 2 * ceil_div(kk0, (int64_t)32);
+  const int rows = 2 * p.M0 + 1;
+  const size_t lhs_bytes = align256((size_t)k16 * rows * 16), rhs_bytes = align256((size_t)p.N * k16 * 512);
+  const size_t product_bytes = (size_t)p.N * rows * 32 * 4;
+  ScratchLease lease(s, lhs_bytes + rhs_bytes + product_bytes);
+  if (!lease.ptr()) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  uint8_t* lhs8 = (uint8_t*)lease.ptr();
+  uint8_t* rhs8 = lhs8 + lhs_bytes;
+  uint32_t* product = (uint32_t*)(rhs8 + rhs_bytes);
+  const RetileNarrowArgs la = {(const int16_t*)p.lhs_buffer, p.lhs_offset, p.K, p.K0, p.M0, k16, lhs8};
+  UK_RETURN_IF_ERROR(launch_grid_stride(retile_planes_narrow_kernel, la, k16 * rows, s,
+                                        "mmt4d digit planes (narrow lhs) launch"));
+  const RetileArgs ra = {p.rhs_buffer, p.rhs_offset, p.rhs_stride0, p.N, p.K, p.K0, k16, rhs8};
+  if (type == IREE_AMD_UK_FLAG_MMT4D_TYPE_S16S8S32) {
+    UK_RETURN_IF_ERROR(launch_grid_stride(retile_planes_kernel<kSourceS8>, ra, p.N * k16 * 32, s,
+                                          "mmt4d 8-bit rhs re-tiling launch"));
+  } else {
+    UK_RETURN_IF_ERROR(widen_u4_rhs(ra, s));
+  }
+  iree_amd_uk_mmt4d_params_t q = {lhs8, 0, k16 * rows * 16, rhs8, 0, k16 * 512, product, 0, p.N * rows * 32,
+                                  1, p.N, k16, rows, 32, 16, IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32, nullptr};
+  {
+    ScratchOverride none(nullptr, 0, /*strict=*/false);   // (the buffer is taken: no K split in there)
+    UK_RETURN_IF_ERROR(iree_amd_uk_mmt4d_p(&q, s));
+  }
+  const CombineNarrowArgs ca = {product, p.N, p.M0, (uint32_t*)p.out_buffer + p.out_offset,
+                                (p.flags & IREE_AMD_UK_FLAG_MMT4D_ACCUMULATE) ? 1 : 0};
+  return launch_grid_stride(combine_planes_narrow_kernel, ca, p.N * p.M0 * 32, s, "mmt4d digit combine launch");
+}
+}  // namespace
 
 int launch_mmt4d_s16_planes(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) {
   if (!mmt4d_s16_planes_supported(p.flags, p.M0, p.N0, p.K0) || p.K == 0) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  if (p.M0 != 32) return launch_narrow(p, s);
   const uint32_t type = p.flags & IREE_AMD_UK_FLAG_MMT4D_TYPE_MASK;
   const bool wide_rhs = type == IREE_AMD_UK_FLAG_MMT4D_TYPE_S16S16S32;
   const int64_t kk0 = p.K * p.K0;
@@ -227,8 +369,7 @@ int launch_mmt4d_s16_planes(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) 
     UK_RETURN_IF_ERROR(launch_grid_stride(retile_planes_kernel<kSourceS8>, ra, p.N * k16 * 32, s,
                                           "mmt4d 8-bit rhs re-tiling launch"));
   } else {
-    UK_RETURN_IF_ERROR(launch_grid_stride(retile_planes_kernel<kSourceU4>, ra, p.N * k16 * 32, s,
-                                          "mmt4d 4-bit rhs widening launch"));
+    UK_RETURN_IF_ERROR(widen_u4_rhs(ra, s));
   }
 
   iree_amd_uk_mmt4d_params_t q = {lhs8, 0, k16 * 512, rhs_operand, 0, rhs_operand_stride, product, 0, rhs_rows * 1024,
