@@ -32,6 +32,10 @@
  *   mi355x_pack_transpose_*, mi355x_unpack_transpose_*   transposed inner
  *       tiles: power-of-two tile sizes whose stored rows (the tile's matrix
  *       rows) are whole 16-byte chunks.
+ *   mi355x_dequant_matmul_i4_k4096_g128_r16, _r32   1..16 or 1..32 rows of
+ *       4096 f16 activations; N a multiple of 32; weights in the layout
+ *       iree_amd_uk_pack_i4_weights writes, f16 scales and packed uint4 zero
+ *       points [N][32]; 512 threads and 131072 bytes of dynamic shared memory.
  */
 #ifndef IREE_AMD_HAL_EXECUTABLE_H_
 #define IREE_AMD_HAL_EXECUTABLE_H_

@@ -37,6 +37,7 @@
 #include "uk_common.h"
 #include "uk_fp8.h"
 #include "uk_i4.h"
+#include "uk_i4_kernel.h"
 
 #include <hip/hip_fp16.h>
 
@@ -44,398 +45,9 @@ namespace uk {
 using namespace i4;
 namespace {
 
-// Work decomposition. A tile is 32 columns (n) of the output. Wave w of the
-// workgroup owns k in [w*KB*64, (w+1)*KB*64), walked in KB/2 spans of 128: in
-// one span lane (nl = l % 16, kc = l / 16) loads, for each half h of the
-// tile's columns, 16 bytes of column h*16+nl, so that one wave load
-// instruction moves a 16-column x 128-k slab (1 KiB, contiguous in the tiled
-// layout). Its 4 dwords feed 4 MFMAs 16x16x32 (A = x rows m, B = weight
-// columns n). Which k a dword holds depends on the layout: chunk (8 k) number
-// q*4 + kc of the span in the tiled layout, kc*4 + q in the row-major one; the
-// activation fragments are loaded to match (a.tiled), which in the tiled case
-// makes each wave load of x cover 64 contiguous bytes of 16 rows.
-//   MH       16-row halves of activations held (1: M <= 16, 2: M <= 32)
-//   kZpU4    zero points are packed uint4 (else f16)
-//   kLog2Gs  log2 of the group size, 5..8, or 9 for "at least the wave's K
-//            slice" (one group per wave and tile). A group never straddles
-//            MFMAs in the tiled layout (MFMA q covers k = q*32 .. +32 of the
-//            span); in the row-major one that only holds for groups of 128
-//            and more, so smaller groups are served from tiled weights only.
-//   kStageX  (the 16-row form) the wave fetches its K slice of the activations
-//            with one full-width direct-to-LDS load per row and takes its
-//            operand fragments from there. Fetching them straight into the
-//            operand layout costs 16 load instructions per wave whatever the
-//            number of rows, and the kernel's start is bound by the rate at
-//            which the compute unit takes load instructions (about 30 cycles
-//            each, 8 waves): with one row the weights of the first tile are
-//            requested 0.8 us earlier this way. Row r of a wave's staging
-//            area is stored rotated by r chunks of 16 bytes (lane l fetches
-//            chunk (l + r) mod row length), so that the 16 lanes that read one
-//            chunk column of 16 rows hit 16 different bank groups without any
-//            padding: 16 rows x 8 waves x 1 KiB are 128 KiB, which with the
-//            32 KiB of partial sums is all the LDS there is. The area is sized
-//            for 8 or for 16 rows (a.stage_rows). The 32-row form stages in
-//            four phases of 8 rows through two buffers of 8 rows per wave (the
-//            same 128 KiB, which its partial sums take over afterwards): 256
-//            row loads per compute unit instead of 256 gathers of 16 half
-//            cache lines each (32 rows: 14.4 -> 12.2 us).
-constexpr int kStageRowsMax = 16;
-template <int KB>
-constexpr int stage_row_bytes() { return KB * 128; }
-constexpr int stage_rows_for(int rows) { return rows <= 8 ? 8 : 16; }
-
 template <int KB, int MH, bool kZpU4, int kLog2Gs>
 __global__ __launch_bounds__(kThreads) void dequant_matmul_i4_kernel(I4Args a) {
-  constexpr bool kStageX = MH == 1;
-  constexpr int SP = KB / 2;                 // spans of 128 k per wave
-  constexpr int L = kLog2Gs >= 9 ? 30 : kLog2Gs;
-  constexpr int GW = ((KB * 64) >> L) > 0 ? ((KB * 64) >> L) : 1;   // groups per wave slice
-  constexpr int SB = GW * 2;                 // bytes of scales per lane, tile and half
-  constexpr int ZB = kZpU4 ? (GW >= 2 ? GW / 2 : 1) : GW * 2;
-  constexpr int SW = (SB + 3) / 4, ZW = (ZB + 3) / 4;
-  // Nibbles as f16 subnormals and the zero point applied through the group sums
-  // of the activations (see nibbles_as_subnormals), where those sums fit the
-  // register file: up to 8 accumulators of 4 registers, 16 in the 16-row form.
-  constexpr bool kSubnormal = GW * MH <= 8 || (MH == 1 && GW <= 16);
-  // Both forms stage the activations through dynamic LDS. The 16-row form keeps
-  // the per-wave partial sums in static LDS next to it; in the 32-row form they
-  // take over the staging area once the first tile has been multiplied.
-  extern __shared__ __attribute__((aligned(16))) char stage_all[];
-  typedef float Partial[kWaves][2 * MH * 4][64];
-  Partial* partial;
-  if constexpr (MH == 1) {
-    __shared__ Partial partial_static[2];
-    partial = partial_static;
-  } else {
-    partial = (Partial*)stage_all;
-  }
-  const int lane = threadIdx.x & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int nl = lane & 15, kc = lane >> 4;
-  const int k_slice = wave * KB * 64;
-  const int g_first = k_slice >> a.log2_gs;  // first group of this wave's slice
-  const uint32_t tile_bytes = (uint32_t)a.K * 16;
-  const uint32_t voff = nl * a.col_stride + kc * 16;
-  const uint32_t soff_wave = wave * SP * a.span_stride;
-  const uint32_t half_stride = 16 * a.col_stride;
-
-  // Raw group parameters of this lane's two columns for the wave's K slice
-  // (zsh: position of a lone packed zero point inside its byte).
-  struct Meta { uint32_t s[2][SW], z[2][ZW], zsh[2]; };
-  auto load_meta = [&](int nt, Meta& m) {
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      int n = nt * 32 + h * 16 + nl;
-      n = n < a.N ? n : a.N - 1;
-      const size_t sg = (size_t)n * a.G + g_first;
-      load_bits<SB>(a.scale + sg, m.s[h]);
-      if (kZpU4) load_bits<ZB>((const uint8_t*)a.zp + (sg >> 1), m.z[h]);
-      else load_bits<ZB>((const uint16_t*)a.zp + sg, m.z[h]);
-      m.zsh[h] = (kZpU4 && GW == 1) ? (uint32_t)(sg & 1) * 4 : 0;
-    }
-  };
-  // Weights of one tile: loads past the end of the buffer (a tile after the
-  // last one, columns past N) return zeros without touching memory.
-  auto tile_rsrc = [&](int nt) {
-    const uint32_t off = (uint32_t)nt * tile_bytes;   // the host checked that this fits
-    const uint32_t left = nt < a.n_tiles ? a.w_bytes - off : 0;
-    return __builtin_amdgcn_make_buffer_rsrc((void*)(a.w + off), 0, left, 0x00020000);
-  };
-  auto load_slab = [&](__amdgpu_buffer_rsrc_t rsrc, int sp, int h) -> u32x4 {
-    // (non-temporal: the weights are read once; measured 9.2 -> 8.8 us at one row)
-    return __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, soff_wave + sp * a.span_stride + h * half_stride, 2);
-  };
-
-  // ---- request the first tile's parameters, x and the first tile's weights --
-  // Loads return in order, and a compute unit takes a load instruction only
-  // every 30-50 cycles: with 8 waves each fetching 32 rows that is what bounds
-  // the start of the kernel (every workgroup reads all of x, from L2: 256 KiB
-  // at 32 rows). Both forms therefore fetch x with full-width direct-to-LDS
-  // loads, one row of the wave's slice per instruction, request the first
-  // tile's weights behind the first rows, and pick the rows out of LDS as MFMA
-  // operand fragments. While the first tile multiplies, it requests slab by
-  // slab the weights of the NEXT tile as it frees their registers.
-  // activations: rows m_base + mh*16 + nl, this wave's K slice; rows past M
-  // are zeros.
-  int nt = blockIdx.x;
-  Meta meta_next;
-  load_meta(nt < a.n_tiles ? nt : a.n_tiles - 1, meta_next);
-  u32x4 xraw[MH][SP][4];
-  u32x4 wreg[SP][2];
-  if constexpr (kStageX) {
-    constexpr int kRowBytes = stage_row_bytes<KB>();
-    constexpr int kLanesPerRow = KB * 8;                 // 16-byte chunks of a row's slice
-    char* stage = stage_all + wave * a.stage_rows * kRowBytes;
-    const int rows = a.M - a.m_base;                     // (at most 16: the host chose this form)
-    const int cq = a.tiled ? 32 : 8, ckc = a.tiled ? 8 : 32;   // chunk strides in k
-    const __amdgpu_buffer_rsrc_t rsrc = tile_rsrc(nt);
-    // One direct-to-LDS load per row, as many as there are rows, nothing waited
-    // for in between; then the first tile's weights; then the wait for the rows
-    // only (loads return in order: all but the weight loads issued since).
-    const __amdgpu_buffer_rsrc_t xsrc = __builtin_amdgcn_make_buffer_rsrc(
-        (void*)(a.x + (size_t)a.m_base * a.K + k_slice), 0, 0x7FFFFFFF, 0x00020000);
-    if (lane < kLanesPerRow) {
-#pragma unroll 1
-      for (int r = 0; r < rows; ++r)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(xsrc, (__attribute__((address_space(3))) void*)(stage + r * kRowBytes), 16,
-                                                 ((lane + r) & (kLanesPerRow - 1)) * 16, r * a.K * 2, 0, 0);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int sp = 0; sp < SP; ++sp)
-#pragma unroll
-      for (int h = 0; h < 2; ++h) wreg[sp][h] = load_slab(rsrc, sp, h);
-    __builtin_amdgcn_sched_barrier(0);
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(SP * 2) : "memory");
-    // (the wave reads only what it loaded itself: no barrier)
-#pragma unroll
-    for (int sp = 0; sp < SP; ++sp)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) xraw[0][sp][q] = u32x4{0u, 0u, 0u, 0u};
-    if (nl < rows) {
-      const char* my_row = stage + nl * kRowBytes;
-#pragma unroll
-      for (int sp = 0; sp < SP; ++sp)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int chunk = (sp * 128 + q * cq + kc * ckc) >> 3;      // of 8 elements, within the slice
-          xraw[0][sp][q] = *(const u32x4*)(my_row + ((chunk - nl) & (kLanesPerRow - 1)) * 16);
-        }
-    }
-  } else {
-    // 32 rows: 8 rows at a time through two buffers of 8 rows per wave (16 rows
-    // of every wave's slice fill the LDS), the same full-width loads and rotated
-    // rows. Phases 0 and 1 and the first tile's weights are requested at once;
-    // a phase's rows go to registers as soon as they have landed (lanes whose
-    // row nl lies in the phase: 8 (p & 1) .. + 8 of half p / 2) and the phase
-    // after next is requested into the buffer so freed. Rows past M fetch the
-    // last row (so that every phase is 8 loads and the waits below can count)
-    // and are zeroed when the first tile turns them into operands.
-    constexpr int kRowBytes = stage_row_bytes<KB>();
-    constexpr int kLanesPerRow = KB * 8;
-    constexpr int kPhaseRows = 8;
-    static_assert(MH == 2, "four phases of 8 rows");
-    char* stage = stage_all + wave * 2 * kPhaseRows * kRowBytes;
-    const int last_row = (a.M - a.m_base < 32 ? a.M - a.m_base : 32) - 1;
-    const int cq = a.tiled ? 32 : 8, ckc = a.tiled ? 8 : 32;   // chunk strides in k
-    const __amdgpu_buffer_rsrc_t rsrc = tile_rsrc(nt);
-    const __amdgpu_buffer_rsrc_t xsrc = __builtin_amdgcn_make_buffer_rsrc(
-        (void*)(a.x + (size_t)a.m_base * a.K + k_slice), 0, 0x7FFFFFFF, 0x00020000);
-    auto request_phase = [&](int p) {
-      if (lane < kLanesPerRow) {
-#pragma unroll
-        for (int r = 0; r < kPhaseRows; ++r) {
-          int row = p * kPhaseRows + r;
-          row = row < last_row ? row : last_row;
-          __builtin_amdgcn_raw_ptr_buffer_load_lds(
-              xsrc, (__attribute__((address_space(3))) void*)(stage + ((p & 1) * kPhaseRows + r) * kRowBytes), 16,
-              ((lane + r) & (kLanesPerRow - 1)) * 16, row * a.K * 2, 0, 0);
-        }
-      }
-      __builtin_amdgcn_sched_barrier(0);
-    };
-    auto take_phase = [&](auto phase) {
-      constexpr int p = decltype(phase)::value;
-      if ((nl >> 3) == (p & 1)) {
-        const int r = nl & 7;
-        const char* my_row = stage + ((p & 1) * kPhaseRows + r) * kRowBytes;
-#pragma unroll
-        for (int sp = 0; sp < SP; ++sp)
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const int chunk = (sp * 128 + q * cq + kc * ckc) >> 3;      // of 8 elements, within the slice
-            xraw[p >> 1][sp][q] = *(const u32x4*)(my_row + ((chunk - r) & (kLanesPerRow - 1)) * 16);
-          }
-      }
-      // the reads have left LDS before anything is loaded over them
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-      __builtin_amdgcn_sched_barrier(0);
-    };
-    request_phase(0);
-    request_phase(1);
-#pragma unroll
-    for (int sp = 0; sp < SP; ++sp)
-#pragma unroll
-      for (int h = 0; h < 2; ++h) wreg[sp][h] = load_slab(rsrc, sp, h);
-    __builtin_amdgcn_sched_barrier(0);
-    // (loads return in order: waiting for all but the n youngest)
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kPhaseRows + SP * 2) : "memory");   // phase 0
-    take_phase(std::integral_constant<int, 0>());
-    request_phase(2);
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kPhaseRows + SP * 2) : "memory");   // phase 1
-    take_phase(std::integral_constant<int, 1>());
-    if (last_row >= 3 * kPhaseRows) {
-      request_phase(3);
-      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kPhaseRows) : "memory");          // the weights and phase 2
-      take_phase(std::integral_constant<int, 2>());
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                           // phase 3
-      take_phase(std::integral_constant<int, 3>());
-    } else {
-      // (at most 24 rows: the last phase's rows do not exist; their lanes keep
-      // whatever their registers hold, which the first tile zeroes)
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      take_phase(std::integral_constant<int, 2>());
-    }
-  }
-  half8 xf[MH][SP][4];
-  // (kSubnormal) the sum of the activations of row r (accumulator layout: every
-  // column the same) over group g of this wave's K slice; complete when the
-  // first tile reaches the end of the group, which is where it is used
-  floatx4 xsum[kSubnormal ? MH : 1][kSubnormal ? GW : 1];
-  if constexpr (kSubnormal) {
-#pragma unroll
-    for (int mh = 0; mh < MH; ++mh)
-#pragma unroll
-      for (int g = 0; g < GW; ++g) xsum[mh][g] = floatx4{0.f, 0.f, 0.f, 0.f};
-  }
-
-  int parity = 0;
-  // One tile; `first`: the workgroup's first, which turns each span of x into
-  // MFMA operands when it gets to it.
-  auto tile = [&](auto first) {
-    constexpr bool kFirst = decltype(first)::value;
-    const int next = nt + gridDim.x;
-    const Meta mt = meta_next;
-    load_meta(next < a.n_tiles ? next : a.n_tiles - 1, meta_next);
-    const __amdgpu_buffer_rsrc_t rsrc_next = tile_rsrc(next < a.n_tiles ? next : a.n_tiles);
-    __builtin_amdgcn_sched_barrier(0);
-    floatx4 acc[2][MH], part[2][MH];
-#pragma unroll
-    for (int h = 0; h < 2; ++h)
-#pragma unroll
-      for (int mh = 0; mh < MH; ++mh) acc[h][mh] = part[h][mh] = floatx4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int sp = 0; sp < SP; ++sp) {
-      if constexpr (kFirst) {
-#pragma unroll
-        for (int mh = 0; mh < MH; ++mh) {
-          const uint32_t keep = kStageX || a.m_base + mh * 16 + nl < a.M ? 0xFFFFFFFFu : 0u;
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            u32x4 v = xraw[mh][sp][q];
-            if constexpr (!kStageX) { v.x &= keep; v.y &= keep; v.z &= keep; v.w &= keep; }
-            if constexpr (kSubnormal) {
-              xf[mh][sp][q] = permute_x_for_subnormals(v);
-              const int g = (sp * 128 + q * 32) >> L;
-              xsum[mh][g] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xf[mh][sp][q], ones_for_subnormal_sums(),
-                                                                  xsum[mh][g], 0, 0, 0);
-            } else {
-              xf[mh][sp][q] = permute_x(v);
-            }
-          }
-        }
-      }
-#pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        const u32x4 wv = wreg[sp][h];
-        float sc = 0.f, zq = 0.f;
-        union { uint32_t u; half2v h; } lo, hi, zf;
-        lo.u = hi.u = zf.u = 0;
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int k_lo = sp * 128 + q * 32;                 // within the wave's slice
-          const int g = k_lo >> L;
-          const bool group_start = kLog2Gs >= 9 ? k_lo == 0 : (k_lo & ((1 << L) - 1)) == 0;
-          const bool group_end = kLog2Gs >= 9 ? k_lo + 32 == KB * 64 : ((k_lo + 32) & ((1 << L) - 1)) == 0;
-          if (group_start || q == 0) {
-            // decode the group's parameters
-            const uint32_t sbits = (mt.s[h][g >> 1] >> ((g & 1) * 16)) & 0xFFFF;
-            sc = __half2float(__ushort_as_half((uint16_t)sbits));
-            if constexpr (kSubnormal) {
-              // the products come in units of 2^-24; zq = -zp in those units
-              sc *= kSubnormalRescale;
-              if (kZpU4) {
-                const uint32_t zb = (mt.z[h][g >> 3] >> ((g & 7) * 4 + mt.zsh[h])) & 0xF;
-                zq = -(float)zb * kSubnormalUnit;
-              } else {
-                const uint32_t zb = (mt.z[h][g >> 1] >> ((g & 1) * 16)) & 0xFFFF;
-                zq = -__half2float(__ushort_as_half((uint16_t)zb)) * kSubnormalUnit;
-              }
-            } else if (kZpU4) {
-              // Packed uint4 zero points fold into the offsets (1024 + zp and
-              // 64 + zp are exact). f16 zero points may carry a fraction, which
-              // such a sum would round away: they are subtracted in a second step.
-              const uint32_t zb = (mt.z[h][g >> 3] >> ((g & 7) * 4 + mt.zsh[h])) & 0xF;
-              lo.u = offset_lo_bits(zb);
-              hi.u = offset_hi_bits(zb);
-            } else {
-              const uint32_t zb = (mt.z[h][g >> 1] >> ((g & 1) * 16)) & 0xFFFF;
-              lo.u = 0x64006400u;
-              hi.h = half2v{(_Float16)64.0f, (_Float16)64.0f};
-              zf.u = zb | (zb << 16);
-            }
-          }
-          if (group_start) {
-#pragma unroll
-            for (int mh = 0; mh < MH; ++mh) part[h][mh] = floatx4{0.f, 0.f, 0.f, 0.f};
-          }
-          half8 wq;
-          if constexpr (kSubnormal) {
-            wq = nibbles_as_subnormals(wv[q]);
-          } else {
-            wq = dequant_dword(wv[q], lo.h, hi.h);
-            if (!kZpU4) {
-              const half8 zsub2 = {zf.h.x, zf.h.x, zf.h.x, zf.h.x, zf.h.x, zf.h.x, zf.h.x, zf.h.x};
-              wq = wq - zsub2;
-            }
-          }
-#pragma unroll
-          for (int mh = 0; mh < MH; ++mh)
-            part[h][mh] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xf[mh][sp][q], wq, part[h][mh], 0, 0, 0);
-          if (group_end) {
-#pragma unroll
-            for (int mh = 0; mh < MH; ++mh)
-#pragma unroll
-              for (int r = 0; r < 4; ++r) {
-                float p = part[h][mh][r];
-                if constexpr (kSubnormal) p = __builtin_fmaf(zq, xsum[mh][g][r], p);     // - zp * sum of x
-                acc[h][mh][r] = __builtin_fmaf(p, sc, acc[h][mh][r]);
-              }
-          }
-        }
-        // The slab's registers are free: request the same slab of the next
-        // tile. The fences keep the requests in slab order, which is what
-        // makes every wait in the loop a wait for the OLDEST outstanding load.
-        __builtin_amdgcn_sched_barrier(0);
-        wreg[sp][h] = load_slab(rsrc_next, sp, h);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-    }
-    // ---- sum the 8 K-slices in wave order and store ----------------------
-    float (*buf)[2 * MH * 4][64] = partial[parity];
-    if constexpr (MH == 2 && kFirst) {
-      // the partial sums overwrite the staging area: every wave has taken its
-      // rows out of it by the time it gets here
-      __builtin_amdgcn_s_barrier();
-    }
-#pragma unroll
-    for (int h = 0; h < 2; ++h)
-#pragma unroll
-      for (int mh = 0; mh < MH; ++mh)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) buf[wave][(h * MH + mh) * 4 + r][lane] = acc[h][mh][r];
-    __syncthreads();
-#pragma unroll
-    for (int rep = 0; rep < MH; ++rep) {
-      const int flat = rep * kThreads + threadIdx.x;     // (h*MH + mh)*256 + r*64 + lane
-      const int l = flat & 63, slot = flat >> 6;         // slot = (h*MH + mh)*4 + r
-      float sum = 0.f;
-#pragma unroll
-      for (int w = 0; w < kWaves; ++w) sum += buf[w][slot][l];
-      const int r = slot & 3, hm = slot >> 2, h = hm / MH, mh = hm % MH;
-      const int m = a.m_base + mh * 16 + 4 * (l >> 4) + r;
-      const int n = nt * 32 + h * 16 + (l & 15);
-      if (m < a.M && n < a.N) a.out[(size_t)m * a.N + n] = __half_as_ushort(__float2half_rn(sum));
-    }
-    // The other half of `partial` is used by the next tile; this half is
-    // rewritten only two tiles later, after the next tile's barrier.
-  };
-  if (nt < a.n_tiles) {
-    tile(std::true_type{});
-    nt += gridDim.x;
-    parity ^= 1;
-  }
-  for (; nt < a.n_tiles; nt += gridDim.x, parity ^= 1) tile(std::false_type{});
+  dequant_matmul_i4_body<KB, MH, kZpU4, kLog2Gs>(a);
 }
 
 // Row-major [N][K/2] bytes -> the tiled layout (one thread per dword).

@@ -64,6 +64,18 @@
 // / 16 (groups of rows that make one 16-byte chunk) and C = the padded columns
 // ceildiv(size1, tile1) * tile1 (pack) or size1 (unpack).
 //
+// mi355x_dequant_matmul_i4_k4096_g128_{r16,r32}: the grouped int4-weight
+// dequantising matmul of the decode step (the dispatch
+// compiler/src/iree/compiler/GlobalOptimization/FuseDequantizationMatmul.cpp:53-159
+// forms; no ukernel in the reference): out[M][N] f16 = x[M][4096] f16 times
+// weights of N columns in groups of 128 along K with f16 scales and packed
+// uint4 zero points. Bindings 0 x, 1 the weights in the library's tiled layout
+// (iree_amd_uk_pack_i4_weights), 2 scales [N][32] f16, 3 zero points [N][32]
+// packed two to a byte (all read only), 4 out; push constants M, N. N a
+// multiple of 32; _r16 takes 1..16 rows, _r32 1..32 (anything else writes
+// nothing). 512 threads, 128 KiB of dynamic LDS (plus 32 KiB static in _r16),
+// grid = min(N / 32, 256).
+//
 // 256 threads, no LDS; grid = ceildiv(C, 32) * ceildiv(R, 16) with, for pack,
 // C = ceildiv(size1, tile1) * tile1 * bytes / 16 and R = ceildiv(size0, tile0) *
 // tile0 (the padded extent), for unpack C = ceildiv(size1 * bytes, 16) and
@@ -72,6 +84,7 @@
 #include "../csrc/uk_mmt4d_mfma_kernel.h"
 #include "../csrc/uk_pack_stream_kernel.h"
 #include "../csrc/uk_pack_transpose_kernel.h"
+#include "../csrc/uk_i4_kernel.h"
 
 namespace {
 
@@ -246,7 +259,43 @@ __device__ __forceinline__ void hal_pack_transpose(const void* mat, void* tiled,
   else unpack_transpose_body<ES>(a);
 }
 
+// The decode configuration of the int4 dequantising matmul: K = 4096, groups
+// of 128, packed uint4 zero points, tiled weights.
+template <int MH>
+__device__ __forceinline__ void hal_dequant_matmul_i4(const void* x, const void* w, const void* scale,
+                                                      const void* zp, void* out, int M, int N) {
+  constexpr int K = 4096;
+  if (M < 1 || M > 16 * MH || N < 32 || N % 32 || (int64_t)N * (K / 2) + K * 16 >= (1ll << 32)) return;
+  i4::I4Args a;
+  a.x = (const uint16_t*)x;
+  a.w = (const uint8_t*)w;
+  a.scale = (const uint16_t*)scale;
+  a.zp = zp;
+  a.out = (uint16_t*)out;
+  a.M = M; a.N = N; a.K = K; a.G = K / 128;
+  a.log2_gs = 7;
+  a.zp_u4 = 1;
+  a.tiled = 1;
+  a.n_tiles = N / 32;
+  a.m_base = 0;
+  a.stage_rows = i4::stage_rows_for(M);
+  a.span_stride = 2048;
+  a.col_stride = 64;
+  a.w_bytes = (uint32_t)((int64_t)N * (K / 2));
+  if ((int)blockIdx.x >= a.n_tiles) return;
+  i4::dequant_matmul_i4_body<8, MH, true, 7>(a);
+}
+
 }  // namespace
+
+#define MI355X_DEQUANT_I4_EXPORT(NAME, MH)                                                         \
+  extern "C" __global__ __launch_bounds__(512) void mi355x_dequant_matmul_i4_k4096_g128_##NAME(    \
+      const void* __restrict__ x, const void* __restrict__ w, const void* __restrict__ scale,      \
+      const void* __restrict__ zp, void* __restrict__ out, int M, int N) {                         \
+    hal_dequant_matmul_i4<MH>(x, w, scale, zp, out, M, N);                                        \
+  }
+MI355X_DEQUANT_I4_EXPORT(r16, 1)
+MI355X_DEQUANT_I4_EXPORT(r32, 2)
 
 #define MI355X_PACK_EXPORTS(BITS, ES)                                                              \
   extern "C" __global__ __launch_bounds__(256) void mi355x_pack_##BITS##bit(                      \

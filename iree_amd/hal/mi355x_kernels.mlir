@@ -1,5 +1,5 @@
 // hal.executable.source for iree_amd/hal/mi355x_kernels_gfx950.co: the gfx950
-// mmt4d, pack and unpack kernels as hand-written dispatches on a HIP device, after the
+// mmt4d, pack, unpack and int4 dequantising matmul kernels as hand-written dispatches on a HIP device, after the
 // reference's samples/custom_dispatch/hip/kernels/example.mlir:16-118.
 // Written by iree_amd.hal_executable.mlir_source(); NOT compiled here (this
 // build has no iree-compile).
@@ -777,6 +777,52 @@ hal.executable.source public @mi355x_mmt4d attributes {
     %bx = arith.ceildivui %size1, %c64 : index
     %by = arith.ceildivui %groups, %c16 : index
     %x = arith.muli %bx, %by : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  // out[M][N] f16 = x[M][4096] f16 * int4 weights (tiled), groups of 128: f16 scales [N][32], packed uint4 zero points [N][32]
+  // push constants M, N; workload (N); limits: 1 <= M <= 16, N a multiple of 32 (else nothing is written)
+  hal.executable.export public @mi355x_dequant_matmul_i4_k4096_g128_r16 ordinal(40)
+      layout(#hal.pipeline.layout<push_constants = 2, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer, ReadOnly>,
+            <2, storage_buffer, ReadOnly>,
+            <3, storage_buffer, ReadOnly>,
+            <4, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [512 : index, 1 : index, 1 : index],
+    workgroup_local_memory = 131072 : index
+  } {
+  ^bb0(%device: !hal.device, %n: index):
+    %c1 = arith.constant 1 : index
+    %c32 = arith.constant 32 : index
+    %cmax = arith.constant 256 : index
+    %tiles = arith.divui %n, %c32 : index
+    %x = arith.minui %tiles, %cmax : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  // out[M][N] f16 = x[M][4096] f16 * int4 weights (tiled), groups of 128: f16 scales [N][32], packed uint4 zero points [N][32]
+  // push constants M, N; workload (N); limits: 1 <= M <= 32, N a multiple of 32 (else nothing is written)
+  hal.executable.export public @mi355x_dequant_matmul_i4_k4096_g128_r32 ordinal(41)
+      layout(#hal.pipeline.layout<push_constants = 2, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer, ReadOnly>,
+            <2, storage_buffer, ReadOnly>,
+            <3, storage_buffer, ReadOnly>,
+            <4, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [512 : index, 1 : index, 1 : index],
+    workgroup_local_memory = 131072 : index
+  } {
+  ^bb0(%device: !hal.device, %n: index):
+    %c1 = arith.constant 1 : index
+    %c32 = arith.constant 32 : index
+    %cmax = arith.constant 256 : index
+    %tiles = arith.divui %n, %c32 : index
+    %x = arith.minui %tiles, %cmax : index
     hal.return %x, %c1, %c1 : index, index, index
   }
 }

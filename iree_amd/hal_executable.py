@@ -118,6 +118,21 @@ def pack_workgroup_count(name, size0, size1, tile0, tile1):
     return -(-cols // 32) * -(-rows // 16)
 
 
+# The int4-weight dequantising matmul of the decode step (K = 4096, groups of
+# 128, packed uint4 zero points, tiled weights): name -> rows served.
+DEQUANT_EXPORTS = {"mi355x_dequant_matmul_i4_k4096_g128_r16": 16,
+                   "mi355x_dequant_matmul_i4_k4096_g128_r32": 32}
+DEQUANT_WORKGROUP_SIZE = 512
+DEQUANT_LDS = 128 * 1024
+DEQUANT_MAX_WORKGROUPS = 256
+
+
+def dequant_workgroup_count(N):
+    """Grid of the dequant exports: one workgroup per compute unit at most,
+    each walking tiles of 32 columns."""
+    return min(N // 32, DEQUANT_MAX_WORKGROUPS)
+
+
 def workgroup_count(export, M, N):
     """Grid of an export for M x N outer tiles: what its count region returns."""
     t = EXPORTS[export].tile if isinstance(export, str) else export.tile
@@ -141,7 +156,10 @@ class HalExecutable:
     def add_export(self, name, block=(WORKGROUP_SIZE, 1, 1), shared_memory_size=None):
         if shared_memory_size is None:
             shared_memory_size = (0 if name in PACK_EXPORTS or name in PACK_TRANSPOSE_EXPORTS else
+                                  DEQUANT_LDS if name in DEQUANT_EXPORTS else
                                   MATMUL_EXPORTS[name].lds if name in MATMUL_EXPORTS else EXPORTS[name].lds)
+        if name in DEQUANT_EXPORTS and block == (WORKGROUP_SIZE, 1, 1):
+            block = (DEQUANT_WORKGROUP_SIZE, 1, 1)
         ordinal = C.c_int32(-1)
         _check(self._lib.iree_amd_hal_executable_add_export(
             self._handle, name.encode(), block[0], block[1], block[2], shared_memory_size,
@@ -207,6 +225,13 @@ class HalExecutable:
         self.dispatch(name, pack_transpose_workgroup_count(name, size0, size1, tile0, tile1), [tiles, matrix],
                       [size0, size1, tile0, tile1], stream)
 
+    def dequant_matmul_i4(self, name, x, w_tiled, scale, zp, out, M, N, stream=None):
+        """mi355x_dequant_matmul_i4_k4096_g128_*: out[M][N] f16 = x[M][4096] f16
+        times int4 weights (tiled layout) with f16 scales [N][32] and packed
+        uint4 zero points [N][32]."""
+        assert 1 <= M <= DEQUANT_EXPORTS[name] and N >= 32 and N % 32 == 0
+        self.dispatch(name, dequant_workgroup_count(N), [x, w_tiled, scale, zp, out], [M, N], stream)
+
     def close(self):
         if self._handle:
             self._lib.iree_amd_hal_executable_release(self._handle)
@@ -221,7 +246,7 @@ class HalExecutable:
 
 _MLIR_HEADER = """\
 // hal.executable.source for iree_amd/hal/mi355x_kernels_gfx950.co: the gfx950
-// mmt4d, pack and unpack kernels as hand-written dispatches on a HIP device, after the
+// mmt4d, pack, unpack and int4 dequantising matmul kernels as hand-written dispatches on a HIP device, after the
 // reference's samples/custom_dispatch/hip/kernels/example.mlir:16-118.
 // Written by iree_amd.hal_executable.mlir_source(); NOT compiled here (this
 // build has no iree-compile).
@@ -339,6 +364,32 @@ _MLIR_PACK_TRANSPOSE_EXPORT = """\
   }}
 """
 
+_MLIR_DEQUANT_EXPORT = """\
+  // out[M][N] f16 = x[M][4096] f16 * int4 weights (tiled), groups of 128: f16 scales [N][32], packed uint4 zero points [N][32]
+  // push constants M, N; workload (N); limits: 1 <= M <= {rows}, N a multiple of 32 (else nothing is written)
+  hal.executable.export public @{name} ordinal({ordinal})
+      layout(#hal.pipeline.layout<push_constants = 2, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer, ReadOnly>,
+            <2, storage_buffer, ReadOnly>,
+            <3, storage_buffer, ReadOnly>,
+            <4, storage_buffer>
+        ]>
+      ]>) attributes {{
+    workgroup_size = [{wg} : index, 1 : index, 1 : index],
+    workgroup_local_memory = {lds} : index
+  }} {{
+  ^bb0(%device: !hal.device, %n: index):
+    %c1 = arith.constant 1 : index
+    %c32 = arith.constant 32 : index
+    %cmax = arith.constant {max_wg} : index
+    %tiles = arith.divui %n, %c32 : index
+    %x = arith.minui %tiles, %cmax : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }}
+"""
+
 _MLIR_PACK_TRANSPOSE_EXTENT = """\
     %o1 = arith.ceildivui %size1, %tile1 : index
     %cols = arith.muli %o1, %tile1 : index
@@ -394,6 +445,11 @@ def mlir_source():
             extra=", padding" if is_pack else "",
             extent=_MLIR_PACK_TRANSPOSE_EXTENT if is_pack else "",
             cols="%cols" if is_pack else "%size1"))
+        ordinal += 1
+    for name, rows in DEQUANT_EXPORTS.items():
+        parts.append(_MLIR_DEQUANT_EXPORT.format(name=name, ordinal=ordinal, rows=rows,
+                                                 wg=DEQUANT_WORKGROUP_SIZE, lds=DEQUANT_LDS,
+                                                 max_wg=DEQUANT_MAX_WORKGROUPS))
         ordinal += 1
     parts.append(_MLIR_FOOTER)
     return "".join(parts)

@@ -53,12 +53,15 @@ def test_export_table_matches_the_sources():
         assert H.MATMUL_EXPORTS["mi355x_matmul_packed_rhs_" + name].lds == int(lds)
     assert H.matmul_workgroup_count("mi355x_matmul_packed_rhs_s8s8s32_t4x8", 200, 333) == 2 * 2
     assert H.matmul_workgroup_count("mi355x_matmul_packed_rhs_s8s8s32_t8x8", 4096, 4096) == 16 * 16
+    assert sorted(re.findall(r"^MI355X_DEQUANT_I4_EXPORT\((\w+), \d\)", src, re.M)) == ["r16", "r32"]
+    assert H.dequant_workgroup_count(14336) == 256 and H.dequant_workgroup_count(96) == 3
 
 
 def test_code_object_is_built_and_names_every_export():
     with open(H.CODE_OBJECT, "rb") as f:
         image = f.read()
-    for name in list(H.EXPORTS) + list(H.PACK_EXPORTS) + list(H.PACK_TRANSPOSE_EXPORTS) + list(H.MATMUL_EXPORTS):
+    for name in (list(H.EXPORTS) + list(H.PACK_EXPORTS) + list(H.PACK_TRANSPOSE_EXPORTS) + list(H.MATMUL_EXPORTS) +
+                 list(H.DEQUANT_EXPORTS)):
         assert name.encode() + b"\0" in image, name
 
 
@@ -325,6 +328,53 @@ def test_transposing_pack_and_unpack_exports_match_the_closed_form(uk, cuda, exe
         exe.unpack_transpose(name, src, out, 8, 8, 24, 8)
     torch.cuda.synchronize()
     assert bool((out == 0xA5).all())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", sorted(H.DEQUANT_EXPORTS))
+def test_dequant_exports_equal_the_library_entry_point(uk, cuda, exe, name):
+    """mi355x_dequant_matmul_i4_k4096_g128_*: the bits of
+    iree_amd_uk_dequant_matmul_i4 (same kernel body) on the decode shape and on
+    a narrow one, and within the stated tolerance of the oracle; row counts the
+    export does not take leave the result untouched."""
+    import torch
+    from iree_amd import synth
+    from test_gpu_dequant import ATOL, RTOL, tile_weights
+    K, gs = 4096, 128
+    G = K // gs
+    rows = H.DEQUANT_EXPORTS[name]
+    for N, Ms in ((14336, [1, 8, rows - 7, rows]), (96, [rows - 1])):
+        w = synth.uniform_u4_packed(2, N * K)
+        s = synth.uniform_f16(4, N * G, 0.005, 0.02)
+        zp = synth.uniform_u4_packed(5, N * G)
+        wd = torch.from_numpy(tile_weights(w, N, K)).cuda()
+        sd = torch.from_numpy(s.view(np.int16)).cuda()
+        zd = torch.from_numpy(zp).cuda()
+        for M in Ms:
+            x = synth.normal_f16(M, M * K)
+            xd = torch.from_numpy(x.view(np.int16)).cuda()
+            one = torch.full((M * N,), 0x7E00, dtype=torch.int16, device=cuda)
+            two = torch.full((M * N,), 0x7E00, dtype=torch.int16, device=cuda)
+            exe.dequant_matmul_i4(name, xd, wd, sd, zd, one, M, N)
+            uk.dequant_matmul_i4(xd, wd, sd, zd, two, M, N, K, gs,
+                                 F.DEQUANT_MATMUL_ZP_U4 | F.DEQUANT_MATMUL_W_TILED)
+            torch.cuda.synchronize()
+            assert torch.equal(one, two), (name, M, N)
+            if N == 96 or M == 1:
+                want = np.zeros(M * N, np.uint16)
+                assert ukref.oracle().oracle_dequant_matmul_i4(
+                    ukref.ptr(x.view(np.uint16)), ukref.ptr(w), ukref.ptr(s.view(np.uint16)), ukref.ptr(zp),
+                    ukref.ptr(want), M, N, K, gs, 1) == 0
+                got = one.cpu().numpy().view(np.float16).astype(np.float64)
+                wantf = want.view(np.float16).astype(np.float64)
+                assert np.all(np.abs(got - wantf) <= ATOL + RTOL * np.abs(wantf)), (name, M, N)
+        out = torch.full((64 * N,), 0x7E00, dtype=torch.int16, device=cuda)
+        xd = torch.zeros(64 * K, dtype=torch.int16, device=cuda)
+        for bad_m in (0, rows + 1):
+            exe.dispatch(name, H.dequant_workgroup_count(N), [xd, wd, sd, zd, out], [bad_m, N])
+        exe.dispatch(name, 1, [xd, wd, sd, zd, out], [1, 48])
+        torch.cuda.synchronize()
+        assert bool((out == 0x7E00).all())
 
 
 @pytest.mark.gpu
