@@ -470,6 +470,7 @@ def extras(args, torch, iree_amd, F, synth, lhs, rhs, out, ex):
     _, t = gpu_time(torch, lambda: iree_amd.mmt4d(li, ri, oi, M1, N1, K1, 32, 32, 16, F.MMT4D_TYPE_S8S8S32),
                     steps, warm)
     ex["mmt4d_i8_tops"] = round(flops / t / 1e12, 2)
+    ex["mmt4d_i8_frac_of_peak"] = round(flops / t / 1e12 / PEAK_I8_TOPS, 4)
     # the same problem with a signed 4-bit right-hand side (S8S4S32): widened
     # to int8 in scratch memory, then the kernel above; two launches per call
     r4 = torch.from_numpy(synth.uniform_u4_packed(3, N1 * K1 * 32 * 16)).cuda()
@@ -489,7 +490,6 @@ def extras(args, torch, iree_amd, F, synth, lhs, rhs, out, ex):
                     max(steps // 4, 5), max(warm // 4, 2))
     ex["mmt4d_s16s16_tops"] = round(flops / t / 1e12, 2)
     del l16, r16
-    ex["mmt4d_i8_frac_of_peak"] = round(flops / t / 1e12 / PEAK_I8_TOPS, 4)
     del li, ri, oi
 
     # f32 x f32 -> f32 at 4096^3, tile 32x32x4 (the reference's primary type)
