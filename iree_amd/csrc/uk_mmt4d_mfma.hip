@@ -335,14 +335,17 @@ int launch_matmul_packed_rhs_mfma(const iree_amd_uk_mmt4d_params_t& p, int64_t o
   a.out_rows = (int)out_rows;
   a.out_cols = (int)out_cols;
   a.out_scale = out_scale;
-  // Reading the row-major matrix inside the matmul costs 7-15 % of the matmul's
-  // time (half or quarter cache lines per row and K-step, fetched again by
-  // every column of macro tiles); packing it first costs one pass over it.
-  // With 8192 result columns and more the pass is the cheaper of the two
-  // (measured break-even near 4096): the left-hand side is then packed into
-  // the stream's scratch buffer and the packed-operand kernel runs. That buffer
-  // is also where a K split keeps its partial sums, so the two exclude each
-  // other (K is only ever split for problems of few macro tiles).
+  // Reading the row-major matrix inside the matmul costs 1-4 % of the matmul's
+  // time (half cache lines per row and K-step, fetched again by every column
+  // of macro tiles); packing it first costs one pass over it. With 16384
+  // result columns and more the pass is the cheaper of the two (measured,
+  // f16 / i8 / fp8: 2048 x 28672 x 4096 411 / 247 / 219 us packed first
+  // against 422 / 252 / 227; 4096 x 14336 x 4096 410 / 242 / 205 against
+  // 418 / 239 / 204; 8192^3 886 / 526 / 489 against 834 / 517 / 481): the
+  // left-hand side is then packed into the stream's scratch buffer and the
+  // packed-operand kernel runs. That buffer is also where a K split keeps its
+  // partial sums, so the two exclude each other (K is only ever split for
+  // problems of few macro tiles).
   const int eb = ti.lhs_bits / 8;
   const int64_t packed_bytes = p.M * p.K * 32 * p.K0 * eb;
   if (batch > 1) {
@@ -350,7 +353,7 @@ int launch_matmul_packed_rhs_mfma(const iree_amd_uk_mmt4d_params_t& p, int64_t o
     a.lhs_row_major = 1;
     return launch_planes(p, a, batch, lhs_batch_stride, rhs_batch_stride, out_batch_stride, s);
   }
-  if (out_cols >= 8192 && out_rows >= 512) {
+  if (out_cols >= 16384 && out_rows >= 512) {
     // (held until the matmul that reads the packed copy has been queued)
     ScratchLease lease(s, (size_t)packed_bytes);
     void* packed = lease.ptr();

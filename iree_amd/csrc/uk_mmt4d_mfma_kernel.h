@@ -286,12 +286,36 @@ __device__ __forceinline__ void mmt4d_mfma_body(const MfmaArgs a, const int bid 
   __amdgpu_buffer_rsrc_t a_src[kARowsPerWave], b_src[kBRowsPerWave];
   // Left-hand side: per-lane offset inside a row block, bytes between K-steps
   // and between the two pieces of a wide block. Packed: as the right-hand side.
-  // Row-major: lane l reads row l % 32 (clamped to the last matrix row), the
-  // 16 * kSub bytes of half l / 32 of the K-step: the same bytes in the same
-  // lane order, so LDS and everything behind it are unchanged.
-  uint32_t a_lane_off[kARowsPerWave], b_lane_off[kBRowsPerWave];
+  // Row-major: the load writes LDS in lane order, so which bytes a lane loads
+  // decides where they lie. In the fragment's own lane order adjacent lanes
+  // are adjacent ROWS, and a load instruction then looks up 64 different cache
+  // lines where the packed form looks up 8. Instead 4 (2 where a K-step is 32
+  // bytes of a row) adjacent lanes load the 16-byte chunks of ONE row's
+  // K-step, 64 or 32 contiguous bytes, and a block lies in LDS row by row;
+  // the chunks of a row are rotated by row / (rows per 256 bytes) so that the
+  // 16 lanes of a fragment read that take one chunk of 16 consecutive rows
+  // still hit every bank once. Two pieces per lane (fp8, a K-step is 64 bytes
+  // of a row): piece j of a block holds rows 16 j .. 16 j + 15, all four
+  // chunks of each, and a lane's two chunks (2 h and 2 h + 1 for K half h) are
+  // read from the piece its row lies in.
+  constexpr bool kLhsQuads = lhs_row_major;
+  constexpr int kRowChunks = kChunks * kSub;          // 16-byte chunks of a row's K-step
+  constexpr int kRotRows = 16 / kRowChunks;           // rows that share 256 bytes of LDS
+  const int quad_row = lane / kRowChunks;             // (of the piece)
+  const int quad_chunk = (lane % kRowChunks + 4 * kRowChunks - quad_row / kRotRows) % kRowChunks;
+  auto lhs_read_off = [&](int chunk) -> uint32_t {
+    if constexpr (kSub == 2) {
+      const int q = frag_row % 16;
+      return (uint32_t)((frag_row / 16) * kPieceBytes + q * 64 + ((chunk + q / 4) % 4) * 16);
+    } else {
+      return (uint32_t)(frag_row * 16 * kChunks + ((chunk + frag_row / kRotRows) % kChunks) * 16);
+    }
+  };
+  const uint32_t a_read_off = !kLhsQuads ? (uint32_t)lane * 16 : lhs_read_off(frag_chunk * kSub);
+  const uint32_t a_read_off_hi = !kLhsQuads ? (uint32_t)lane * 16 + kPieceBytes
+                                            : kSub == 2 ? lhs_read_off(frag_chunk * kSub + 1) : 0u;
+  uint32_t a_lane_off[kARowsPerWave][kSub], b_lane_off[kBRowsPerWave];
   const uint32_t a_step_bytes = lhs_row_major ? kChunks * 16 * kSub : kStepBytes;
-  const uint32_t a_piece_stride = lhs_row_major ? 16 : kPieceStride;
 #pragma unroll
   for (int r = 0; r < kARowsPerWave; ++r) {
     const int blk = i_base + wave * kARowsPerWave + r;
@@ -299,13 +323,17 @@ __device__ __forceinline__ void mmt4d_mfma_body(const MfmaArgs a, const int bid 
     const int sub = blk % kPerTile;
     i = i < a.M ? i : a.M - 1;
     if (lhs_row_major) {
-      int row = i * 32 + sub * R + frag_row;
-      row = row < a.out_rows ? row : a.out_rows - 1;
       a_src[r] = row_descriptor(a.lhs);
-      a_lane_off[r] = (uint32_t)row * (uint32_t)a.lhs_stride_bytes + frag_chunk * 16 * kSub;
+#pragma unroll
+      for (int j = 0; j < kSub; ++j) {
+        int row = i * 32 + sub * R + j * 16 + quad_row;
+        row = row < a.out_rows ? row : a.out_rows - 1;
+        a_lane_off[r][j] = (uint32_t)row * (uint32_t)a.lhs_stride_bytes + quad_chunk * 16;
+      }
     } else {
       a_src[r] = row_descriptor(a.lhs + (int64_t)i * a.lhs_stride_bytes);
-      a_lane_off[r] = packed_lane_off(sub);
+#pragma unroll
+      for (int j = 0; j < kSub; ++j) a_lane_off[r][j] = packed_lane_off(sub) + j * kPieceStride;
     }
   }
 #pragma unroll
@@ -395,7 +423,7 @@ __device__ __forceinline__ void mmt4d_mfma_body(const MfmaArgs a, const int bid 
     char* base = lds + slot * kSlotBytes;
     const int r = d / kSub, j = d % kSub;
     if (r < kARowsPerWave) {
-      load_block_to_lds(a_src[r], a_lane_off[r], (uint32_t)ks * a_step_bytes + j * a_piece_stride,
+      load_block_to_lds(a_src[r], a_lane_off[r][j], (uint32_t)ks * a_step_bytes,
                         base + (wave * kARowsPerWave + r) * kBlockBytes + j * kPieceBytes);
     } else {
       const int rb = r - kARowsPerWave;
@@ -415,6 +443,14 @@ __device__ __forceinline__ void mmt4d_mfma_body(const MfmaArgs a, const int bid 
       return frag_t{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
     }
   };
+  auto read_frag_at = [&](const char* block, uint32_t lo_off, uint32_t hi_off) -> frag_t {
+    if constexpr (kSub == 1) {
+      return *(const frag_t*)(block + lo_off);
+    } else {
+      const int4v lo = *(const int4v*)(block + lo_off), hi = *(const int4v*)(block + hi_off);
+      return frag_t{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    }
+  };
   // Fragment `r` (of kFrags) of this wave for the K-step in `slot`: its WN
   // blocks of B, then its WM blocks of A. The MFMAs run over A blocks in the
   // outer loop, so the fragments read last (A blocks 1..) are needed last.
@@ -424,7 +460,7 @@ __device__ __forceinline__ void mmt4d_mfma_body(const MfmaArgs a, const int bid 
     const bool is_b = kOuterB ? r >= WM : r < WN;
     const int idx = kOuterB ? (r < WM ? r : r - WM) : (r < WN ? r : r - WN);
     if (is_b) fb[idx] = read_frag(s0 + kABytes + (wn * WN + idx) * kBlockBytes);
-    else fa[idx] = read_frag(s0 + (wm * WM + idx) * kBlockBytes);
+    else fa[idx] = read_frag_at(lds + slot * kSlotBytes + (wm * WM + idx) * kBlockBytes, a_read_off, a_read_off_hi);
   };
   auto read_frags = [&](int slot, frag_t (&fa)[WM], frag_t (&fb)[WN]) {
 #pragma unroll

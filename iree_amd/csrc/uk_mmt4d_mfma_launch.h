@@ -126,19 +126,25 @@ int launch_variant(const MfmaArgs& a0, hipStream_t s) {
   const int64_t blocks = (int64_t)a.tiles_m * a.tiles_n;
   if (blocks > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
   // one kernel instance per operand form (the forms the entry points produce)
+  constexpr bool kPackedLhs = !RowMajorLhsOnly<Cfg>::value;
   if constexpr (!kSiluMul) {
     if (a.k_slices > 1 && a.row_major_out) return IREE_AMD_UK_STATUS_NOT_FOUND;
     if (a.lhs_row_major && a.row_major_out)
       return launch_form<Cfg, WM, WN, kRing, kSync, kOcc, kSiluMul, kWavesN, 2>(a, (unsigned)blocks, s);
-    if (a.row_major_out)
-      return launch_form<Cfg, WM, WN, kRing, kSync, kOcc, kSiluMul, kWavesN, 1>(a, (unsigned)blocks, s);
+    if constexpr (kPackedLhs) {
+      if (a.row_major_out)
+        return launch_form<Cfg, WM, WN, kRing, kSync, kOcc, kSiluMul, kWavesN, 1>(a, (unsigned)blocks, s);
+    }
   }
   if constexpr (!kSiluMul) {
     if (a.lhs_row_major)   // (tiled result: the partial sums of a K split)
       return launch_form<Cfg, WM, WN, kRing, kSync, kOcc, kSiluMul, kWavesN, 3>(a, (unsigned)blocks, s);
   }
   if (a.lhs_row_major || a.row_major_out) return IREE_AMD_UK_STATUS_NOT_FOUND;
-  return launch_form<Cfg, WM, WN, kRing, kSync, kOcc, kSiluMul, kWavesN, 0>(a, (unsigned)blocks, s);
+  if constexpr (kPackedLhs)
+    return launch_form<Cfg, WM, WN, kRing, kSync, kOcc, kSiluMul, kWavesN, 0>(a, (unsigned)blocks, s);
+  else
+    return IREE_AMD_UK_STATUS_NOT_FOUND;
 }
 
 // The four macro tiles (in outer tiles of 32 rows: 8x8, 8x4, 4x8, 4x4) with
@@ -252,14 +258,15 @@ int launch_cfg(const MfmaArgs& a, hipStream_t s) {
       cost += resident * work / (resident == t.occ ? t.eff_full : t.eff_alone);
     }
     // A row-major left-hand side is the dearer operand to fetch (half or
-    // quarter cache lines per row and K-step): tiles with more rows than
-    // columns pay most. Measured at 2048 x 4096 x 4096 against the packed
-    // operand: 256x256 1.10 (f16) and 1.22 (i8), 256x128 1.27 and 1.36,
-    // 128x256 1.07 and 1.06, 128x128 1.30 and 1.28.
+    // quarter cache lines per row and K-step, each line asked for again on the
+    // next step): tiles with more rows than columns pay most. Measured at
+    // 2048 x 4096 x 4096 against the packed operand, K-steps of 64 bytes of a
+    // row (f16, i8 with two instructions per step; fp8 alike): 256x256 1.01,
+    // 256x128 1.09-1.14, 128x256 1.02-1.03, 128x128 1.13; K-steps of 32 bytes
+    // (i8 otherwise): 1.16, 1.37, 1.06, 1.28.
     if (a.lhs_row_major) {
-      // (a K-step is 64 bytes of a row for f16 / bf16 / fp8, 32 for i8 and f32)
       constexpr bool kHalfLines = Cfg::kRows == 16 || Cfg::kSub == 2;
-      static const double penalty[2][4] = {{1.22, 1.36, 1.06, 1.28}, {1.09, 1.27, 1.07, 1.30}};
+      static const double penalty[2][4] = {{1.16, 1.37, 1.06, 1.28}, {1.02, 1.13, 1.03, 1.13}};
       cost *= penalty[kHalfLines][v];
     }
     return cost;

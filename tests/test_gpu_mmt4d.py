@@ -616,13 +616,15 @@ def test_fused_unpack_applies_the_output_scale(uk, cuda):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("M,N,K", [(1024, 1024, 1024), (123, 456, 800), (81, 19, 64), (1, 1000, 992),
-                                   (300, 257, 32)])
+                                   (300, 257, 32), (77, 130, 1088), (530, 290, 2112)])
 @pytest.mark.parametrize("accumulate", [False, True])
 def test_i8_matmul_with_packed_rhs_in_one_kernel_is_bit_exact(uk, cuda, M, N, K, accumulate):
     """matmul_packed_rhs: row-major LHS read by the matmul itself, pre-packed
     RHS, row-major result. Against the plain integer matmul of the oracle; row
     pitches of A and C wider than a row (the bytes between rows of C must stay
-    untouched), ragged M and N, K in whole matrix-core steps of 32."""
+    untouched), ragged M and N, K in whole matrix-core steps of 32 (an even
+    number of them runs the kernel with two instructions per 64-byte step, an
+    odd number the one with 32-byte steps)."""
     import torch
     lda, ldc = K + 16, N + 5
     A = synth.uniform_int8(1, M * K).reshape(M, K)
@@ -886,11 +888,11 @@ def test_random_outer_shapes_i8_exact(uk, cuda):
 @pytest.mark.gpu
 @pytest.mark.parametrize("accumulate", [False, True])
 def test_matmul_packed_rhs_wide_result_packs_the_lhs_first(uk, cuda, accumulate):
-    """8192 result columns and more (and 512 rows): matmul_packed_rhs packs its
+    """16384 result columns and more (and 512 rows): matmul_packed_rhs packs its
     left-hand side into the stream's scratch buffer and runs the packed-operand
     kernel. Ragged M and N, a row pitch wider than the row, exact integers."""
     import torch
-    M, N, K = 530, 8200, 160
+    M, N, K = 530, 16400, 160
     lda, ldc = K + 16, N + 8
     rng = np.random.default_rng(31)
     a_pad = rng.integers(-128, 128, (M, lda), dtype=np.int8)
