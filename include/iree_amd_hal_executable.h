@@ -26,7 +26,8 @@
  *       (32 x K elements) below 2 GiB; K whole K0 tiles; dense operands.
  *   mi355x_matmul_packed_rhs_*              the row-major left-hand side
  *       (M x K elements) below 2 GiB: its rows are addressed with 32-bit byte
- *       offsets; K a multiple of the matrix-core K extent.
+ *       offsets; K a multiple of the matrix-core K extent (s8s8s32_k64: of
+ *       64, with K0 = 16: the faster i8 form).
  *   mi355x_pack_*, mi355x_unpack_*          power-of-two tile sizes whose rows
  *       are whole 16-byte chunks, no transposes.
  *   mi355x_pack_transpose_*, mi355x_unpack_transpose_*   transposed inner

@@ -37,7 +37,8 @@
 // only), 1 rhs, packed [ceildiv(N, 32)][K / K0][32][K0] (read only: weights
 // packed ahead of time), 2 out, the dense row-major M x N matrix; push
 // constants M, N, K (ELEMENTS; K a whole number of matrix-core K-steps: 32 for
-// f16 / bf16 / i8, 8 for f32, 64 for fp8), K0, flags. Macro tiles of 128 x 256
+// f16 / bf16 / i8, 8 for f32, 64 for fp8 and the s8s8s32_k64 exports, which
+// take K0 = 16 only and are the faster i8 form), K0, flags. Macro tiles of 128 x 256
 // (_t4x8: the cheaper one for a row-major left-hand side, two workgroups per
 // compute unit) or 256 x 256 (_t8x8); grid = ceildiv(ceildiv(M, 32), 4 or 8) *
 // ceildiv(ceildiv(N, 32), 8).
@@ -151,6 +152,7 @@ __device__ __forceinline__ void hal_matmul_packed_rhs(const void* lhs, const voi
   static_assert(TM % kPerTile == 0 && TN % kPerTile == 0, "macro tile of whole outer tiles");
   typedef typename Cfg::out_t out_t;
   if (M < 1 || N < 1 || K < Cfg::kMfmaK || K % Cfg::kMfmaK) return;
+  if (Cfg::kSub == 2 && K0 != 16) return;   // (the two-piece block layout is that of K0 = 16 tiles)
   // The left-hand side is addressed with 32-bit byte offsets: a matrix of 2 GiB
   // or more (the library's entry point refuses it as well) does nothing here.
   if ((int64_t)M * K * Cfg::kElemBytes + 4096 > 0x7FFFFFFFll) return;
@@ -346,6 +348,10 @@ MI355X_MATMUL_EXPORT(bf16bf16f32_t4x8, BF16Cfg16, 4, 8, 3, 1, 2, 73728)
 MI355X_MATMUL_EXPORT(bf16bf16f32_t8x8, BF16Cfg16, 8, 8, 5, 1, 1, 163840)
 MI355X_MATMUL_EXPORT(s8s8s32_t4x8, S8Cfg, 2, 4, 6, 2, 2, 73728)
 MI355X_MATMUL_EXPORT(s8s8s32_t8x8, S8Cfg, 4, 4, 8, 2, 1, 131072)
+// (K0 = 16 and K a multiple of 64: two instructions per 64-byte K-step, so
+// that a lane quad loads 64 contiguous bytes of a row of the left-hand side)
+MI355X_MATMUL_EXPORT(s8s8s32_k64_t4x8, S8Cfg2, 2, 4, 3, 1, 2, 73728)
+MI355X_MATMUL_EXPORT(s8s8s32_k64_t8x8, S8Cfg2, 4, 4, 5, 1, 1, 163840)
 MI355X_MATMUL_EXPORT(f8e4m3f8e4m3f32_t4x8, F8Cfg, 2, 4, 3, 1, 2, 73728)
 MI355X_MATMUL_EXPORT(f8e4m3f8e4m3f32_t8x8, F8Cfg, 4, 4, 5, 1, 1, 163840)
 MI355X_MATMUL_EXPORT(f32f32f32_t4x8, F32Cfg, 2, 4, 6, 2, 2, 73728)

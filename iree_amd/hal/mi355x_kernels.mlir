@@ -451,7 +451,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
   }
   // out[M][N] (+)= lhs[M][K] * rhs (packed); push constants M, N, K (elements), K0, flags; workload (M, N)
   // limits: M * K elements of lhs below 2 GiB, K a multiple of the matrix-core K extent (else nothing is written)
-  hal.executable.export public @mi355x_matmul_packed_rhs_f8e4m3f8e4m3f32_t4x8 ordinal(26)
+  hal.executable.export public @mi355x_matmul_packed_rhs_s8s8s32_k64_t4x8 ordinal(26)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
         <0, bindings = [
             <0, storage_buffer, ReadOnly>,
@@ -469,7 +469,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
   }
   // out[M][N] (+)= lhs[M][K] * rhs (packed); push constants M, N, K (elements), K0, flags; workload (M, N)
   // limits: M * K elements of lhs below 2 GiB, K a multiple of the matrix-core K extent (else nothing is written)
-  hal.executable.export public @mi355x_matmul_packed_rhs_f8e4m3f8e4m3f32_t8x8 ordinal(27)
+  hal.executable.export public @mi355x_matmul_packed_rhs_s8s8s32_k64_t8x8 ordinal(27)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
         <0, bindings = [
             <0, storage_buffer, ReadOnly>,
@@ -487,7 +487,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
   }
   // out[M][N] (+)= lhs[M][K] * rhs (packed); push constants M, N, K (elements), K0, flags; workload (M, N)
   // limits: M * K elements of lhs below 2 GiB, K a multiple of the matrix-core K extent (else nothing is written)
-  hal.executable.export public @mi355x_matmul_packed_rhs_f32f32f32_t4x8 ordinal(28)
+  hal.executable.export public @mi355x_matmul_packed_rhs_f8e4m3f8e4m3f32_t4x8 ordinal(28)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
         <0, bindings = [
             <0, storage_buffer, ReadOnly>,
@@ -505,7 +505,43 @@ hal.executable.source public @mi355x_mmt4d attributes {
   }
   // out[M][N] (+)= lhs[M][K] * rhs (packed); push constants M, N, K (elements), K0, flags; workload (M, N)
   // limits: M * K elements of lhs below 2 GiB, K a multiple of the matrix-core K extent (else nothing is written)
-  hal.executable.export public @mi355x_matmul_packed_rhs_f32f32f32_t8x8 ordinal(29)
+  hal.executable.export public @mi355x_matmul_packed_rhs_f8e4m3f8e4m3f32_t8x8 ordinal(29)
+      layout(#hal.pipeline.layout<push_constants = 5, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer, ReadOnly>,
+            <2, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index],
+    workgroup_local_memory = 163840 : index
+  } {
+  ^bb0(%device: !hal.device, %m: index, %n: index):
+    %x = affine.apply affine_map<()[s0, s1] -> (((s0 ceildiv 32) ceildiv 8) * ((s1 ceildiv 32) ceildiv 8))>()[%m, %n]
+    %c1 = arith.constant 1 : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  // out[M][N] (+)= lhs[M][K] * rhs (packed); push constants M, N, K (elements), K0, flags; workload (M, N)
+  // limits: M * K elements of lhs below 2 GiB, K a multiple of the matrix-core K extent (else nothing is written)
+  hal.executable.export public @mi355x_matmul_packed_rhs_f32f32f32_t4x8 ordinal(30)
+      layout(#hal.pipeline.layout<push_constants = 5, sets = [
+        <0, bindings = [
+            <0, storage_buffer, ReadOnly>,
+            <1, storage_buffer, ReadOnly>,
+            <2, storage_buffer>
+        ]>
+      ]>) attributes {
+    workgroup_size = [256 : index, 1 : index, 1 : index],
+    workgroup_local_memory = 73728 : index
+  } {
+  ^bb0(%device: !hal.device, %m: index, %n: index):
+    %x = affine.apply affine_map<()[s0, s1] -> (((s0 ceildiv 32) ceildiv 4) * ((s1 ceildiv 32) ceildiv 8))>()[%m, %n]
+    %c1 = arith.constant 1 : index
+    hal.return %x, %c1, %c1 : index, index, index
+  }
+  // out[M][N] (+)= lhs[M][K] * rhs (packed); push constants M, N, K (elements), K0, flags; workload (M, N)
+  // limits: M * K elements of lhs below 2 GiB, K a multiple of the matrix-core K extent (else nothing is written)
+  hal.executable.export public @mi355x_matmul_packed_rhs_f32f32f32_t8x8 ordinal(31)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
         <0, bindings = [
             <0, storage_buffer, ReadOnly>,
@@ -523,7 +559,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
   }
   // pack: in = matrix, out = tiles; push constants size0, size1, tile0, tile1, padding; workload (size0, size1, tile0, tile1)
   // limits: power-of-two tiles whose rows are whole 16-byte chunks, no transposes (else nothing is written)
-  hal.executable.export public @mi355x_pack_8bit ordinal(30)
+  hal.executable.export public @mi355x_pack_8bit ordinal(32)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
         <0, bindings = [
             <0, storage_buffer, ReadOnly>,
@@ -550,7 +586,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
   }
   // pack: in = matrix, out = tiles; push constants size0, size1, tile0, tile1, padding; workload (size0, size1, tile0, tile1)
   // limits: power-of-two tiles whose rows are whole 16-byte chunks, no transposes (else nothing is written)
-  hal.executable.export public @mi355x_pack_16bit ordinal(31)
+  hal.executable.export public @mi355x_pack_16bit ordinal(33)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
         <0, bindings = [
             <0, storage_buffer, ReadOnly>,
@@ -577,7 +613,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
   }
   // pack: in = matrix, out = tiles; push constants size0, size1, tile0, tile1, padding; workload (size0, size1, tile0, tile1)
   // limits: power-of-two tiles whose rows are whole 16-byte chunks, no transposes (else nothing is written)
-  hal.executable.export public @mi355x_pack_32bit ordinal(32)
+  hal.executable.export public @mi355x_pack_32bit ordinal(34)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
         <0, bindings = [
             <0, storage_buffer, ReadOnly>,
@@ -604,7 +640,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
   }
   // unpack: in = tiles, out = matrix; push constants size0, size1, tile0, tile1; workload (size0, size1, tile0, tile1)
   // limits: power-of-two tiles whose rows are whole 16-byte chunks, no transposes (else nothing is written)
-  hal.executable.export public @mi355x_unpack_16bit ordinal(33)
+  hal.executable.export public @mi355x_unpack_16bit ordinal(35)
       layout(#hal.pipeline.layout<push_constants = 4, sets = [
         <0, bindings = [
             <0, storage_buffer, ReadOnly>,
@@ -627,7 +663,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
   }
   // unpack: in = tiles, out = matrix; push constants size0, size1, tile0, tile1; workload (size0, size1, tile0, tile1)
   // limits: power-of-two tiles whose rows are whole 16-byte chunks, no transposes (else nothing is written)
-  hal.executable.export public @mi355x_unpack_32bit ordinal(34)
+  hal.executable.export public @mi355x_unpack_32bit ordinal(36)
       layout(#hal.pipeline.layout<push_constants = 4, sets = [
         <0, bindings = [
             <0, storage_buffer, ReadOnly>,
@@ -650,7 +686,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
   }
   // pack: in = matrix, out = tiles, tiles of tile0 rows x tile1 columns stored column by column; push constants size0, size1, tile0, tile1, padding; workload (size0, size1, tile0, tile1)
   // limits: power-of-two tiles with tile0 * 1 >= 16 (else nothing is written)
-  hal.executable.export public @mi355x_pack_transpose_8bit ordinal(35)
+  hal.executable.export public @mi355x_pack_transpose_8bit ordinal(37)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
         <0, bindings = [
             <0, storage_buffer, ReadOnly>,
@@ -677,7 +713,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
   }
   // pack: in = matrix, out = tiles, tiles of tile0 rows x tile1 columns stored column by column; push constants size0, size1, tile0, tile1, padding; workload (size0, size1, tile0, tile1)
   // limits: power-of-two tiles with tile0 * 2 >= 16 (else nothing is written)
-  hal.executable.export public @mi355x_pack_transpose_16bit ordinal(36)
+  hal.executable.export public @mi355x_pack_transpose_16bit ordinal(38)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
         <0, bindings = [
             <0, storage_buffer, ReadOnly>,
@@ -704,7 +740,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
   }
   // pack: in = matrix, out = tiles, tiles of tile0 rows x tile1 columns stored column by column; push constants size0, size1, tile0, tile1, padding; workload (size0, size1, tile0, tile1)
   // limits: power-of-two tiles with tile0 * 4 >= 16 (else nothing is written)
-  hal.executable.export public @mi355x_pack_transpose_32bit ordinal(37)
+  hal.executable.export public @mi355x_pack_transpose_32bit ordinal(39)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
         <0, bindings = [
             <0, storage_buffer, ReadOnly>,
@@ -731,7 +767,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
   }
   // unpack: in = tiles, out = matrix, tiles of tile0 rows x tile1 columns stored column by column; push constants size0, size1, tile0, tile1; workload (size0, size1, tile0, tile1)
   // limits: power-of-two tiles with tile0 * 2 >= 16 (else nothing is written)
-  hal.executable.export public @mi355x_unpack_transpose_16bit ordinal(38)
+  hal.executable.export public @mi355x_unpack_transpose_16bit ordinal(40)
       layout(#hal.pipeline.layout<push_constants = 4, sets = [
         <0, bindings = [
             <0, storage_buffer, ReadOnly>,
@@ -756,7 +792,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
   }
   // unpack: in = tiles, out = matrix, tiles of tile0 rows x tile1 columns stored column by column; push constants size0, size1, tile0, tile1; workload (size0, size1, tile0, tile1)
   // limits: power-of-two tiles with tile0 * 4 >= 16 (else nothing is written)
-  hal.executable.export public @mi355x_unpack_transpose_32bit ordinal(39)
+  hal.executable.export public @mi355x_unpack_transpose_32bit ordinal(41)
       layout(#hal.pipeline.layout<push_constants = 4, sets = [
         <0, bindings = [
             <0, storage_buffer, ReadOnly>,
@@ -781,7 +817,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
   }
   // out[M][N] f16 = x[M][4096] f16 * int4 weights (tiled), groups of 128: f16 scales [N][32], packed uint4 zero points [N][32]
   // push constants M, N; workload (N); limits: 1 <= M <= 16, N a multiple of 32 (else nothing is written)
-  hal.executable.export public @mi355x_dequant_matmul_i4_k4096_g128_r16 ordinal(40)
+  hal.executable.export public @mi355x_dequant_matmul_i4_k4096_g128_r16 ordinal(42)
       layout(#hal.pipeline.layout<push_constants = 2, sets = [
         <0, bindings = [
             <0, storage_buffer, ReadOnly>,
@@ -804,7 +840,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
   }
   // out[M][N] f16 = x[M][4096] f16 * int4 weights (tiled), groups of 128: f16 scales [N][32], packed uint4 zero points [N][32]
   // push constants M, N; workload (N); limits: 1 <= M <= 32, N a multiple of 32 (else nothing is written)
-  hal.executable.export public @mi355x_dequant_matmul_i4_k4096_g128_r32 ordinal(41)
+  hal.executable.export public @mi355x_dequant_matmul_i4_k4096_g128_r32 ordinal(43)
       layout(#hal.pipeline.layout<push_constants = 2, sets = [
         <0, bindings = [
             <0, storage_buffer, ReadOnly>,
