@@ -564,6 +564,15 @@ def extras(args, torch, iree_amd, F, synth, lhs, rhs, out, ex):
                     max(5, steps // 4), 2)
     ex["matmul_f16_pack_mmt4d_fused_unpack_tflops"] = round(flops / t / 1e12, 2)
     assert torch.equal(c, c_two), "fused unpack differs from mmt4d + unpack"
+    # and with the pack of the left-hand side folded into the matmul as well:
+    # the pack of B and one matmul launch
+    c_two = c.clone()
+    _, t = gpu_time(torch, lambda: iree_amd.matmul_data_tiled(a, b, c, size, size, size,
+                                                              F.MMT4D_TYPE_F16F16F32, workspace=ws,
+                                                              fuse_pack_lhs=True),
+                    max(5, steps // 4), 2)
+    ex["matmul_f16_pack_rhs_fused_matmul_tflops"] = round(flops / t / 1e12, 2)
+    assert torch.equal(c, c_two), "the matmul on a row-major left-hand side differs from the chain"
     # and with the right-hand side packed ahead of time (weights) and the
     # left-hand side read row-major by the matmul itself: one launch
     c.fill_(0)

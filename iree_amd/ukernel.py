@@ -382,10 +382,13 @@ def _ceil_div(a, b):
 
 
 def matmul_data_tiled(a, b, c, M, N, K, mmt4d_type, *, accumulate=False,
-                      tile=None, workspace=None, fuse_unpack=False):
+                      tile=None, workspace=None, fuse_unpack=False, fuse_pack_lhs=False):
     """Row-major C[M][N] (+)= A[M][K] * B[K][N] through pack -> mmt4d -> unpack.
     With ``fuse_unpack`` the last two (and the pack of C when accumulating) are
     the one kernel ``mmt4d_unpack``; it needs a tile with a matrix-core kernel.
+    With ``fuse_pack_lhs`` the matmul also reads A row-major itself
+    (``matmul_packed_rhs``): the chain is the pack of B and one matmul launch;
+    K must then be whole matrix-core steps.
 
     ``a``/``b``/``c`` are flat CUDA tensors holding the row-major matrices with
     the element types of ``mmt4d_type``. ``tile`` = (M0, N0, K0); by default the
@@ -403,17 +406,26 @@ def matmul_data_tiled(a, b, c, M, N, K, mmt4d_type, *, accumulate=False,
     in_type = _IN_PACK_TYPE[mmt4d_type]
     out_type = _OUT_PACK_TYPE[mmt4d_type]
     ws = workspace if workspace is not None else {}
-    if "lhs" not in ws:
+    fuse_unpack = fuse_unpack or fuse_pack_lhs
+    if "lhs" not in ws and not fuse_pack_lhs:
         ws["lhs"] = torch.empty(M1 * K1 * M0 * K0, dtype=a.dtype, device=a.device)
     if "rhs" not in ws:
         ws["rhs"] = torch.empty(N1 * K1 * N0 * K0, dtype=b.dtype, device=b.device)
     if "out" not in ws and not fuse_unpack:
         ws["out"] = torch.empty(M1 * N1 * M0 * N0, dtype=c.dtype, device=c.device)
-    pack(a, ws["lhs"], M, K, M1, K1, M0, K0, 0, in_type)
+    if not fuse_pack_lhs:
+        pack(a, ws["lhs"], M, K, M1, K1, M0, K0, 0, in_type)
     pack(b, ws["rhs"], K, N, N1, K1, N0, K0, 0,
          in_type | F.PACK_TRANSPOSE_INNER | F.PACK_TRANSPOSE_OUTER)
     mm_flags = mmt4d_type | F.MMT4D_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION | \
         F.MMT4D_SKIP_INTERMEDIATE_ROUNDINGS
+    if fuse_pack_lhs:
+        if (M0, N0) != (32, 32) or K % K0:
+            raise ValueError("fuse_pack_lhs needs 32x32 tiles and K in whole tiles")
+        if accumulate:
+            mm_flags |= F.MMT4D_ACCUMULATE
+        matmul_packed_rhs(a, ws["rhs"], c, M, N, K, K0, mm_flags)
+        return ws
     if fuse_unpack:
         if (M0, N0) != (32, 32):
             raise ValueError("fuse_unpack needs 32x32 tiles")

@@ -356,6 +356,26 @@ def test_i8_matmul_accumulates_into_seeded_c(uk, cuda):
     assert np.array_equal(c.cpu().numpy().reshape(M, N), want)
 
 
+@pytest.mark.parametrize("M,N,K", [(1024, 1024, 1024), (123, 456, 800), (40, 1000, 992)])
+@pytest.mark.parametrize("accumulate", [False, True])
+def test_i8_matmul_chain_with_the_fused_forms(uk, cuda, M, N, K, accumulate):
+    """The same chain with the unpack, and then also the pack of A, folded into
+    the matmul (pack of B + mmt4d_unpack, pack of B + matmul_packed_rhs): the
+    exact integer product both ways."""
+    import torch
+    A, B = synth.uniform_int8(1, M * K), synth.uniform_int8(2, K * N)
+    c0 = (synth.splitmix64(3, M * N) >> np.uint64(44)).astype(np.int64).astype(np.int32)
+    want = _pack_chain_oracle_i8(A, B, M, N, K)
+    if accumulate:
+        want = want + c0.reshape(M, N)
+    for kw in ({"fuse_unpack": True}, {"fuse_pack_lhs": True}):
+        c = torch.from_numpy(c0.copy()).cuda() if accumulate else torch.zeros(M * N, dtype=torch.int32, device="cuda")
+        uk.matmul_data_tiled(torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda(), c,
+                             M, N, K, F.MMT4D_TYPE_S8S8S32, accumulate=accumulate, **kw)
+        torch.cuda.synchronize()
+        assert np.array_equal(c.cpu().numpy().reshape(M, N), want), kw
+
+
 def _sampled_f64_rows(A, B, rows, K, N):
     return A[rows].astype(np.float64) @ B.astype(np.float64)
 
