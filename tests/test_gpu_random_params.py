@@ -102,3 +102,73 @@ def test_random_int4_dequant_matmul_calls_within_tolerance(uk, cuda, seed):
         run_case(uk, M, N, K, gs, zp_u4, tiled, seed=int(rng.integers(0, 1 << 20)))
         if rng.integers(0, 2):
             run_reassoc_case(uk, min(M, 17), N, K, gs, zp_u4, tiled, seed=int(rng.integers(0, 1 << 20)))
+
+
+# (type, K0 values, elements of K per matrix-core step, integers that the type holds exactly)
+FUSED_TYPES = [(F.MMT4D_TYPE_F16F16F32, (8, 16), 32, 8), (F.MMT4D_TYPE_BF16BF16F32, (8, 16), 32, 8),
+               (F.MMT4D_TYPE_S8S8S32, (16, 32), 32, 128), (F.MMT4D_TYPE_F8E4M3F8E4M3F32, (16,), 64, 8),
+               (F.MMT4D_TYPE_F32F32F32, (4, 8), 8, 8)]
+
+
+def _encode(torch, tf, ints):
+    """Integer-valued matrix -> device tensor of the type's elements."""
+    t = torch.from_numpy(ints.astype(np.float32)).cuda()
+    if tf == F.MMT4D_TYPE_S8S8S32:
+        return torch.from_numpy(ints.astype(np.int8)).cuda()
+    if tf == F.MMT4D_TYPE_F16F16F32:
+        return t.half()
+    if tf == F.MMT4D_TYPE_BF16BF16F32:
+        return t.bfloat16()
+    if tf == F.MMT4D_TYPE_F8E4M3F8E4M3F32:
+        return t.to(torch.float8_e4m3fn).view(torch.uint8)
+    return t
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_fused_matmul_calls_exact(uk, cuda, seed):
+    """mmt4d_unpack and matmul_packed_rhs (the matmul that writes the row-major
+    result itself, and the one that also reads its left-hand side row-major)
+    over random types, shapes, K0, row pitches and accumulate, on small
+    integers: every sum is exact in the accumulator type, so any tile, K-step
+    size or K split the launcher picks must give the integer product."""
+    import torch
+    rng = np.random.default_rng(515100 + seed)
+    pack_type = {1: F.PACK_TYPE_I8I8, 2: F.PACK_TYPE_F16F16, 4: F.PACK_TYPE_F32F32}
+    for _ in range(40):
+        tf, k0s, mfma_k, lim = FUSED_TYPES[int(rng.integers(0, len(FUSED_TYPES)))]
+        K0 = int(rng.choice(k0s))
+        M = int(rng.integers(1, 700)) if rng.integers(0, 4) else int(rng.integers(1, 40))
+        N = int(rng.integers(1, 700)) if rng.integers(0, 4) else int(rng.integers(1, 40))
+        steps = int(rng.integers(1, 12)) if rng.integers(0, 5) else int(rng.integers(64, 160))
+        K = steps * mfma_k
+        acc = bool(rng.integers(0, 2))
+        A = rng.integers(-lim, lim, (M, K))
+        B = rng.integers(-lim, lim, (N, K))
+        C0 = rng.integers(-1000, 1000, (M, N))
+        want = A @ B.T + (C0 if acc else 0)
+        a_dev, b_dev = _encode(torch, tf, A), _encode(torch, tf, B)
+        es = a_dev.element_size()
+        # row pitches: the left-hand side's a multiple of 16 bytes, the result's anything
+        lda = K + int(rng.integers(0, 3)) * (16 // es)
+        ldc = N + int(rng.integers(0, 7))
+        a_pad = torch.zeros(M, lda, dtype=a_dev.dtype, device=cuda)
+        a_pad[:, :K] = a_dev
+        M1, N1, K1 = -(-M // 32), -(-N // 32), K // K0
+        rhs = torch.empty(N1 * K1 * 32 * K0, dtype=b_dev.dtype, device=cuda)
+        lhs = torch.empty(M1 * K1 * 32 * K0, dtype=a_dev.dtype, device=cuda)
+        uk.pack(b_dev, rhs, N, K, N1, K1, 32, K0, 0, pack_type[es])
+        uk.pack(a_dev, lhs, M, K, M1, K1, 32, K0, 0, pack_type[es])
+        odt = torch.int32 if tf == F.MMT4D_TYPE_S8S8S32 else torch.float32
+        flags = tf | (F.MMT4D_ACCUMULATE if acc else 0)
+        for form in ("matmul_packed_rhs", "mmt4d_unpack"):
+            c = torch.full((M, ldc), 77, dtype=odt, device=cuda)
+            c[:, :N] = torch.from_numpy(C0).cuda().to(odt)
+            if form == "matmul_packed_rhs":
+                uk.matmul_packed_rhs(a_pad, rhs, c, M, N, K, K0, flags, lhs_stride0=lda, out_stride0=ldc)
+            else:
+                uk.mmt4d_unpack(lhs, rhs, c, M, N, M1, N1, K1, K0, flags, out_stride0=ldc)
+            torch.cuda.synchronize()
+            got = c.cpu().numpy().astype(np.int64)
+            case = (seed, form, hex(tf), M, N, K, K0, acc, lda, ldc)
+            assert np.array_equal(got[:, :N], want), case
+            assert (got[:, N:] == 77).all(), case
