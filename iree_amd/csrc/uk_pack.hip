@@ -296,6 +296,10 @@ template <int ES>
 __global__ __launch_bounds__(256) void unpack_transpose_kernel(TransArgs a) { unpack_transpose_body<ES>(a); }
 template <int ES>
 __global__ __launch_bounds__(256) void pack_transpose_wide_kernel(TransArgs a) { pack_transpose_wide_body<ES>(a); }
+template <int ES, int kLdsUnroll>
+__global__ __launch_bounds__(256) void pack_transpose_lds_kernel(TransArgs a) {
+  pack_transpose_lds_body<ES, kLdsUnroll>(a);
+}
 
 template <int ES>
 int launch_unpack_transpose(TransArgs a, hipStream_t s) {
@@ -314,6 +318,27 @@ int launch_pack_transpose(TransArgs a, hipStream_t s) {
   // boundary and tiles are whole dwords of columns
   constexpr int W = ES < 4 ? 4 / ES : 1;
   const bool wide = W > 1 && a.tile_cols % W == 0 && (uintptr_t)a.mat % 4 == 0 && a.m_pitch_bytes % 4 == 0;
+  // 2-byte elements, 512 columns and more in tiles of whole 8 columns: 16-byte
+  // loads and an exchange through LDS, 4 row groups per wave where that still
+  // gives every compute unit a workgroup, else 1 (small matrices keep the
+  // finer-grained kernels below)
+  if constexpr (ES == 2) {
+    if (wide && a.tile_cols % 8 == 0 && a.padded_cols >= 512) {
+      const int64_t lx = ceil_div(a.padded_cols, (int64_t)512);
+      const int64_t ly4 = ceil_div(a.row_groups, (int64_t)16), ly1 = ceil_div(a.row_groups, (int64_t)4);
+      const int cus = device_cu_count();
+      if (lx * ly4 >= cus && lx * ly4 <= 0x7FFFFFFF) {
+        a.blocks_x = (uint32_t)lx; a.blocks_y = (uint32_t)ly4;
+        hipLaunchKernelGGL((pack_transpose_lds_kernel<ES, 4>), dim3((unsigned)(lx * ly4)), dim3(256), 0, s, a);
+        return check_hip(hipGetLastError(), "pack_transpose launch");
+      }
+      if (lx * ly1 >= cus && lx * ly1 <= 0x7FFFFFFF) {
+        a.blocks_x = (uint32_t)lx; a.blocks_y = (uint32_t)ly1;
+        hipLaunchKernelGGL((pack_transpose_lds_kernel<ES, 1>), dim3((unsigned)(lx * ly1)), dim3(256), 0, s, a);
+        return check_hip(hipGetLastError(), "pack_transpose launch");
+      }
+    }
+  }
   const int64_t bx = ceil_div(a.padded_cols, (int64_t)64 * (wide ? W : 1));
   const int64_t by = ceil_div(a.row_groups, (int64_t)(4 * kTransUnroll));
   if (bx < 1 || by < 1 || bx * by > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;

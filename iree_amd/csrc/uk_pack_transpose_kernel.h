@@ -199,6 +199,115 @@ __device__ __forceinline__ void pack_transpose_wide_body(const TransArgs& a) {
   }
 }
 
+// 2-byte elements, whole rows of 16 bytes per lane: a wave covers 512 columns
+// of the 8 matrix rows of one row group with 8 load instructions of 1 KiB each
+// (the streaming pack's rate; the dword kernel above needs 32 for the same
+// bytes). A lane then holds an 8 x 8 block, transposes it in registers (one
+// byte permute per dword) into the 8 chunks of its 8 columns, and the wave
+// passes the chunks through its 8 KiB of LDS so that store instruction s takes
+// columns 64 s .. 64 s + 63, one per lane: 1 KiB of whole tiles per store where
+// the lane's own 8 chunks would be 64 pieces of 16 bytes 128 bytes apart. LDS
+// holds lane l's chunk w at 16-byte slot 8 l + (w + l / 2) mod 8: both the
+// writes (lanes 128 bytes apart) and the reads (8 lanes per 128 bytes, two
+// source lanes per 16) then touch every bank once per 16 lanes.
+// kLdsUnroll row groups per wave, all loaded before the first is stored (4:
+// 13.4 us for f16 4096 x 4096 into 32x8 tiles, 1: 14.3; the dword kernel 15.8).
+template <int ES, int kLdsUnroll>
+__device__ __forceinline__ void pack_transpose_lds_body(const TransArgs& a) {
+  static_assert(ES == 2, "2-byte elements");
+  typedef uint32_t u32x4u __attribute__((ext_vector_type(4), aligned(4)));
+  __shared__ u32x4 exchange[4][512];
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  uint32_t bx, by;
+  {
+    constexpr uint32_t kXcds = 8;
+    const uint32_t total = a.blocks_x * a.blocks_y;
+    const uint32_t per = total / kXcds, rem = total % kXcds;
+    const uint32_t xcd = blockIdx.x % kXcds, idx = blockIdx.x / kXcds;
+    const uint32_t logical = xcd * per + (xcd < rem ? xcd : rem) + idx;
+    by = logical / a.blocks_x;
+    bx = logical - by * a.blocks_x;
+  }
+  const int64_t c0 = (int64_t)bx * 512;                       // first column of the wave
+  const int64_t c = c0 + lane * 8;                            // first of this lane's 8 columns
+  const int64_t g0 = ((int64_t)by * 4 + wave) * kLdsUnroll;   // first row group of this wave
+  if (g0 >= a.row_groups) return;
+  u32x4* xw = exchange[wave];
+  const uint32_t pad = (uint16_t)a.padding;
+  // all the loads of the wave's row groups first, so that they are in flight together
+  u32x4 vall[kLdsUnroll][8];
+  if (c0 + 512 <= a.m_size1 && (g0 + kLdsUnroll) * 8 <= a.m_size0) {
+    const char* src = a.mat + g0 * 8 * a.m_pitch_bytes + c * 2;
+#pragma unroll
+    for (int u = 0; u < kLdsUnroll; ++u)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) vall[u][i] = *(const u32x4u*)(src + (int64_t)(u * 8 + i) * a.m_pitch_bytes);
+  } else {
+#pragma unroll
+    for (int u = 0; u < kLdsUnroll; ++u)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int64_t r = (g0 + u) * 8 + i;
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+          uint32_t both = 0;
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            const int64_t col = c + 2 * d + h;
+            const uint32_t e = (r < a.m_size0 && col < a.m_size1)
+                                   ? (uint32_t)*(const uint16_t*)(a.mat + r * a.m_pitch_bytes + col * 2) : pad;
+            both |= e << (16 * h);
+          }
+          vall[u][i][d] = both;
+        }
+      }
+  }
+#pragma unroll
+  for (int u = 0; u < kLdsUnroll; ++u) {
+    const int64_t g = g0 + u;
+    if (g >= a.row_groups) break;
+    const u32x4 (&v)[8] = vall[u];
+    // chunk w: column c + w, rows 0..7 of the group, row 2 j in the low half of dword j
+#pragma unroll
+    for (int w = 0; w < 8; ++w) {
+      const uint32_t sel = (w & 1) ? 0x07060302u : 0x05040100u;
+      u32x4 chunk;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) chunk[j] = __builtin_amdgcn_perm(v[2 * j + 1][w / 2], v[2 * j][w / 2], sel);
+      xw[lane * 8 + ((w + (lane >> 1)) & 7)] = chunk;
+    }
+    // (the wave's own LDS region: lanes run in lockstep and LDS serves a wave's
+    // accesses in order; the fences keep the compiler from reordering them)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    int64_t orow;
+    uint32_t grp;
+    if (g < 0x7FFFFFFF) {
+      orow = a.by_groups.div((uint32_t)g);
+      grp = (uint32_t)g - (uint32_t)orow * a.groups_per_tile;
+    } else {
+      orow = g / a.groups_per_tile;
+      grp = (uint32_t)(g - orow * a.groups_per_tile);
+    }
+    char* out_row = a.tiled + orow * a.t_stride_orow_bytes + (int64_t)grp * 16;
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      const uint32_t from = 8 * s + (lane >> 3);                 // the lane that built this chunk
+      const u32x4 chunk = xw[from * 8 + (((lane & 7) + (from >> 1)) & 7)];
+      const int64_t n = c0 + 64 * s + lane;
+      if (n < a.padded_cols) {
+        const uint32_t ocol = a.by_tile_cols.div((uint32_t)n), d2 = (uint32_t)n - ocol * a.tile_cols;
+        *(u32x4*)(out_row + (int64_t)ocol * a.t_stride_ocol_bytes + (int64_t)d2 * a.tile_rows * 2) = chunk;
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  }
+}
+
 // The reverse: unpack of tiles stored column by column (the transposed result
 // tiles of a matmul whose narrow dimension was exchanged, reference
 // unpack.c:190-247). One thread takes one 16-byte chunk of the tiled buffer

@@ -87,6 +87,12 @@ def test_streaming_shapes_with_ragged_edges(uk, cuda, type_flag, t0, t1, rows, c
     (F.PACK_TYPE_I8I8, 16, 32, 1003, 772),
     (F.PACK_TYPE_BF16BF16, 16, 64, 300, 1028),
     (F.PACK_TYPE_I8I8, 32, 8, 200, 1024),
+    # 2-byte elements, 512 columns and more, enough blocks for every compute unit: the kernel that
+    # loads 16 bytes per lane and passes the chunks through LDS (4 row groups per wave, 1, two row
+    # groups per tile), ragged in both directions
+    (F.PACK_TYPE_F16F16, 8, 32, 4100, 4200),
+    (F.PACK_TYPE_F16F16, 8, 32, 1030, 4200),
+    (F.PACK_TYPE_BF16BF16, 16, 64, 4100, 4130),
 ])
 def test_transposing_pack_with_ragged_edges(uk, cuda, type_flag, tr, tc, rows, cols):
     """Packs with transposed inner tiles (what the right-hand side B[K][N] of a
