@@ -63,6 +63,7 @@ def parse_args():
                     "mmt4d_f16 | mmt4d_f16_acc | mmt4d_i8 | mmt4d_s16s8 | mmt4d_s16s16 | mmt4d_fp8 | mmt4d_f16_ksplit | mlp_fp8 | pack | unpack | "
                     "pack_transpose | unpack_transpose | dequant_i4[_m8|_m32] | dequant_i4_reassoc[_m8|_m32] | batch_mmt4d_f16 | "
                     "batch_mmt4d_f16_narrow | mmt4d_f16_narrow_m1 | mmt4d_f16_narrow_m8 | mmt4d_f16_narrow_n8 | "
+                    "matmul_rowmajor_lhs_f16 | matmul_rowmajor_lhs_i8 | matmul_rowmajor_lhs_fp8 | "
                     "chain_i8_1024 | copy | copy_rotating | copy_rotating_nt | copy_rotating_nt_single_waves | read_only_29mb")
     return ap.parse_args()
 
@@ -883,6 +884,25 @@ def run_only(args, torch, iree_amd, F, synth, mm_step):
                 iree_amd.mmt4d(rn[k], ln, on, Nn // 32, 1, Kn // 8, 32, 8, 8, F.MMT4D_TYPE_F16F16F32)
             else:
                 iree_amd.mmt4d(ln, rn[k], on, 1, Nn // 32, Kn // 8, m0, 32, 8, F.MMT4D_TYPE_F16F16F32)
+    elif args.only in ("matmul_rowmajor_lhs_f16", "matmul_rowmajor_lhs_i8", "matmul_rowmajor_lhs_fp8"):
+        # the whole linear layer at 4096^3: row-major left-hand side read by the
+        # matmul itself, right-hand side packed ahead, row-major result
+        size = 4096
+        if args.only.endswith("_f16"):
+            am = torch.from_numpy(synth.normal_f16(1, size * size, 1 / 64).view(np.int16)).cuda()
+            bm = torch.from_numpy(synth.normal_f16(2, size * size, 1 / 64).view(np.int16)).cuda()
+            k0, tf, odt = 8, F.MMT4D_TYPE_F16F16F32, torch.float32
+        else:
+            am = torch.from_numpy(synth.uniform_int8(1, size * size)).cuda()
+            bm = torch.from_numpy(synth.uniform_int8(2, size * size)).cuda()
+            k0, tf, odt = 16, F.MMT4D_TYPE_S8S8S32, torch.int32
+            if args.only.endswith("_fp8"):
+                # e4m3 codes of moderate magnitude, no NaN
+                am, bm = am.view(torch.uint8) & 0xBF, bm.view(torch.uint8) & 0xBF
+                tf, odt = F.MMT4D_TYPE_F8E4M3F8E4M3F32, torch.float32
+        cm = torch.zeros(size * size, dtype=odt, device="cuda")
+        # (the operand values stand for a packed right-hand side as they are: any bytes do for timing)
+        fn = lambda: iree_amd.matmul_packed_rhs(am, bm, cm, size, size, size, k0, tf)  # noqa: E731
     elif args.only == "chain_i8_1024":
         n1k = 1024
         a8 = torch.from_numpy(synth.uniform_int8(1, n1k * n1k)).cuda()
