@@ -107,7 +107,9 @@ def test_random_int4_dequant_matmul_calls_within_tolerance(uk, cuda, seed):
 # (type, K0 values, elements of K per matrix-core step, integers that the type holds exactly)
 FUSED_TYPES = [(F.MMT4D_TYPE_F16F16F32, (8, 16), 32, 8), (F.MMT4D_TYPE_BF16BF16F32, (8, 16), 32, 8),
                (F.MMT4D_TYPE_S8S8S32, (16, 32), 32, 128), (F.MMT4D_TYPE_F8E4M3F8E4M3F32, (16,), 64, 8),
-               (F.MMT4D_TYPE_F32F32F32, (4, 8), 8, 8)]
+               (F.MMT4D_TYPE_F32F32F32, (4, 8), 8, 8),
+               # results rounded once to the operand type (intermediate roundings skipped)
+               (F.MMT4D_TYPE_F16F16F16, (8, 16), 32, 8), (F.MMT4D_TYPE_BF16BF16BF16, (8, 16), 32, 8)]
 
 
 def _encode(torch, tf, ints):
@@ -115,9 +117,9 @@ def _encode(torch, tf, ints):
     t = torch.from_numpy(ints.astype(np.float32)).cuda()
     if tf == F.MMT4D_TYPE_S8S8S32:
         return torch.from_numpy(ints.astype(np.int8)).cuda()
-    if tf == F.MMT4D_TYPE_F16F16F32:
+    if tf in (F.MMT4D_TYPE_F16F16F32, F.MMT4D_TYPE_F16F16F16):
         return t.half()
-    if tf == F.MMT4D_TYPE_BF16BF16F32:
+    if tf in (F.MMT4D_TYPE_BF16BF16F32, F.MMT4D_TYPE_BF16BF16BF16):
         return t.bfloat16()
     if tf == F.MMT4D_TYPE_F8E4M3F8E4M3F32:
         return t.to(torch.float8_e4m3fn).view(torch.uint8)
@@ -144,7 +146,8 @@ def test_random_fused_matmul_calls_exact(uk, cuda, seed):
         acc = bool(rng.integers(0, 2))
         A = rng.integers(-lim, lim, (M, K))
         B = rng.integers(-lim, lim, (N, K))
-        C0 = rng.integers(-1000, 1000, (M, N))
+        narrow_out = tf in (F.MMT4D_TYPE_F16F16F16, F.MMT4D_TYPE_BF16BF16BF16)
+        C0 = rng.integers(-128, 128, (M, N)) if narrow_out else rng.integers(-1000, 1000, (M, N))
         want = A @ B.T + (C0 if acc else 0)
         a_dev, b_dev = _encode(torch, tf, A), _encode(torch, tf, B)
         es = a_dev.element_size()
@@ -158,8 +161,12 @@ def test_random_fused_matmul_calls_exact(uk, cuda, seed):
         lhs = torch.empty(M1 * K1 * 32 * K0, dtype=a_dev.dtype, device=cuda)
         uk.pack(b_dev, rhs, N, K, N1, K1, 32, K0, 0, pack_type[es])
         uk.pack(a_dev, lhs, M, K, M1, K1, 32, K0, 0, pack_type[es])
-        odt = torch.int32 if tf == F.MMT4D_TYPE_S8S8S32 else torch.float32
-        flags = tf | (F.MMT4D_ACCUMULATE if acc else 0)
+        odt = {F.MMT4D_TYPE_S8S8S32: torch.int32, F.MMT4D_TYPE_F16F16F16: torch.float16,
+               F.MMT4D_TYPE_BF16BF16BF16: torch.bfloat16}.get(tf, torch.float32)
+        flags = tf | (F.MMT4D_ACCUMULATE if acc else 0) | (F.MMT4D_SKIP_INTERMEDIATE_ROUNDINGS if narrow_out else 0)
+        if narrow_out:
+            # the exact sum (it fits f32), rounded once to the result type
+            want = torch.from_numpy(want.astype(np.float32)).to(odt).double().numpy()
         for form in ("matmul_packed_rhs", "mmt4d_unpack"):
             c = torch.full((M, ldc), 77, dtype=odt, device=cuda)
             c[:, :N] = torch.from_numpy(C0).cuda().to(odt)
@@ -168,7 +175,7 @@ def test_random_fused_matmul_calls_exact(uk, cuda, seed):
             else:
                 uk.mmt4d_unpack(lhs, rhs, c, M, N, M1, N1, K1, K0, flags, out_stride0=ldc)
             torch.cuda.synchronize()
-            got = c.cpu().numpy().astype(np.int64)
+            got = c.double().cpu().numpy()
             case = (seed, form, hex(tf), M, N, K, K0, acc, lda, ldc)
-            assert np.array_equal(got[:, :N], want), case
+            assert np.array_equal(got[:, :N], want.astype(np.float64)), case
             assert (got[:, N:] == 77).all(), case
