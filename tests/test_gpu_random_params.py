@@ -83,6 +83,28 @@ def test_random_pack_and_unpack_calls_bit_exact(uk, cuda, seed):
 
 
 @pytest.mark.parametrize("seed", range(3))
+def test_random_large_transposing_packs_bit_exact(uk, cuda, seed):
+    """Transposing packs of 2-byte elements large enough for the kernel that
+    loads 16 bytes per lane and passes the chunks through LDS (512 columns and
+    more, a block for every compute unit), with ragged edges, any padding
+    regime, both outer orders and row pitches that are or are not whole
+    dwords; against the oracle."""
+    rng = np.random.default_rng(626200 + seed)
+    for _ in range(5):
+        t0 = int(rng.choice([8, 16, 32]))
+        t1 = int(rng.choice([8, 16, 32, 64]))
+        rows, cols = int(rng.integers(1030, 4200)), int(rng.integers(600, 4200))
+        # (enough row groups of 8 x 512-column blocks for 256 compute units)
+        if (rows // 8) * (cols // 512 + 1) < 1100:
+            rows = 4100
+        kw = dict(transpose_inner=1, transpose_outer=int(rng.integers(0, 2)), in_size=(rows, cols),
+                  pad=PADS[int(rng.integers(0, 3))], loose_strides=bool(rng.integers(0, 4) == 0))
+        pc = ukref.PackCase(rng, F.PACK_TYPE_F16F16 if rng.integers(0, 2) else F.PACK_TYPE_BF16BF16,
+                            -(-rows // t0), -(-cols // t1), t0, t1, **kw)
+        assert np.array_equal(gpucase.run_pack(pc), pc.run_oracle()), (seed, rows, cols, t0, t1, kw)
+
+
+@pytest.mark.parametrize("seed", range(3))
 def test_random_int4_dequant_matmul_calls_within_tolerance(uk, cuda, seed):
     """The grouped int4 dequantising matmul over random row counts (both sides of
     every kernel boundary: 8, 16, 32 rows), column counts, K (the matrix-core
