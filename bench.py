@@ -713,6 +713,21 @@ def extras(args, torch, iree_amd, F, synth, lhs, rhs, out, ex):
         _, t = gpu_time(torch, do_n, steps, warm)
         ex[f"mmt4d_f16_narrow_m{M0}_gbs"] = round((Nn * Kn * 2 + M0 * Kn * 2 + M0 * Nn * 4) / t / 1e9, 1)
     ex["mmt4d_f16_narrow_m1_frac_of_hbm_peak"] = round(ex["mmt4d_f16_narrow_m1_gbs"] / PEAK_HBM_GBS, 4)
+    # the same shape through the whole-linear-layer entry point: M row-major
+    # rows in, row-major result out (M < 32 runs the kernel above on the rows
+    # themselves; 32 and more the macro-tile kernel)
+    for Mr in (1, 8, 24, 32):
+        ar = torch.from_numpy(synth.normal_f16(62, Mr * Kn).view(np.int16)).cuda()
+        cr = torch.empty(Mr * Nn, dtype=torch.float32, device="cuda")
+        state["i"] = 0
+
+        def do_rows():
+            k = state["i"] % 6
+            state["i"] += 1
+            iree_amd.matmul_packed_rhs(ar, rn[k], cr, Mr, Nn, Kn, 8, F.MMT4D_TYPE_F16F16F32)
+
+        _, t = gpu_time(torch, do_rows, steps, warm)
+        ex[f"matmul_f16_rowmajor_lhs_m{Mr}_n14336_k4096_us"] = round(t * 1e6, 1)
     # the same problem as a narrow RESULT: 14336 rows x 8 columns (32 x 8 result
     # tiles, the wide operand on the left), which the library runs with the
     # operands exchanged and the tiles stored transposed

@@ -761,7 +761,22 @@ int matmul_packed_rhs_impl(
   if (!lhs_buffer || !rhs_buffer || !out_buffer)
     return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "matmul_packed_rhs: null buffer");
   int st = IREE_AMD_UK_STATUS_NOT_FOUND;
-  if (mmt4d_mfma_supported(flags, 32, 32, K0))
+  // One row (the matrix-vector product of a decode step): the row is its own
+  // tile row of 1 x K0 tiles and a row of 1 x 32 result tiles is the row-major
+  // result, so this is the mmt4d with narrow left-hand side tiles that the
+  // tile-size query gives for a static M of 1, which streams the right-hand
+  // side once (N = 14336, K = 4096, f16: 23 us against 28 for the macro-tile
+  // kernel with its K split).
+  if (M == 1 && N % 32 == 0 && b.batch == 1 && out_scale == 1.0f && mmt4d_skinny_supported(flags, 1, 32, K0)) {
+    const iree_amd_uk_mmt4d_params_t row = {lhs_buffer, lhs_offset, K, rhs_buffer, rhs_offset, rhs_stride0,
+                                            out_buffer, out_offset, N, 1, N / 32, K / K0, 1, 32, K0, flags, nullptr};
+    st = launch_mmt4d_skinny(row, (hipStream_t)stream);
+  }
+  // A few rows (2 to 31): the same kernel with the rows of the matrix as the
+  // rows of its one narrow tile, reading them and writing the result row-major.
+  if (st == IREE_AMD_UK_STATUS_NOT_FOUND && M > 1 && M < 32 && b.batch == 1 && out_scale == 1.0f)
+    st = launch_matmul_rows_skinny(p, M, N, (hipStream_t)stream);
+  if (st == IREE_AMD_UK_STATUS_NOT_FOUND && mmt4d_mfma_supported(flags, 32, 32, K0))
     st = launch_matmul_packed_rhs_mfma(p, M, N, out_scale, b.batch, b.lhs, b.rhs, b.out, (hipStream_t)stream);
   if (st == IREE_AMD_UK_STATUS_NOT_FOUND && b.batch > 1) {
     for (iree_amd_uk_index_t e = 0; e < b.batch; ++e) {

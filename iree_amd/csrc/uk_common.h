@@ -56,6 +56,7 @@ int launch_mmt4d_generic(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s);
 bool mmt4d_mfma_supported(uint32_t flags, int M0, int N0, int K0);
 bool mmt4d_skinny_supported(uint32_t flags, int M0, int N0, int K0);
 int launch_mmt4d_skinny(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s);
+int launch_matmul_rows_skinny(const iree_amd_uk_mmt4d_params_t& p, int64_t M, int64_t out_cols, hipStream_t s);
 // S8S4S32 through the s8 x s8 kernels on a widened copy of the right-hand side
 // (uk_mmt4d_s8s4.hip); NOT_FOUND when the call must take the element-wise kernel.
 bool mmt4d_s8s4_widened_supported(uint32_t flags, int M0, int N0, int K0);

@@ -67,6 +67,13 @@ struct SkinnyArgs {
   // piece of the packed row) with direct-to-LDS loads of 1 KiB into its own
   // area of so many bytes of the dynamic LDS and reads its fragments from there
   int stage_wave_bytes;
+  // > 0: the left-hand side is the row-major M0 x K matrix itself, rows so many
+  // bytes apart (instead of one outer row of M0 x K0 tiles), and, with
+  // out_row_pitch_elems > 0, the result the row-major M0 x out_cols matrix
+  // (instead of N tiles of M0 x 32): the whole linear layer on a few rows.
+  int64_t lhs_row_pitch_bytes;
+  int64_t out_row_pitch_elems;
+  int out_cols;
 };
 
 // SP: K steps per wave held in registers (compile-time bound; a.steps_per_wave <= SP).
@@ -143,10 +150,14 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
   frag_t ring[kDepth];
   frag_t xf[SP];
   // bytes of the packed left-hand side per K step: its K tiles are consecutive
-  const int step_bytes = (kSub == 2 ? 4 : a.half_k0 ? 2 : 1) * a.lhs_tile_bytes;
-  // this lane's first piece inside a step (the second one, fp8, a tile further)
+  // (row-major: the bytes of one ROW per K step, 32, or 64 for fp8)
+  const bool rows_lhs = a.lhs_row_pitch_bytes > 0;
+  const int step_bytes = rows_lhs ? 32 * kSub : (kSub == 2 ? 4 : a.half_k0 ? 2 : 1) * a.lhs_tile_bytes;
+  // this lane's first piece inside a step (the second one, fp8, a tile further;
+  // row-major: the next 16 bytes of the row)
   const int piece_off = kSub == 2 ? 2 * kh * a.lhs_tile_bytes + m0 * 16
                         : a.half_k0 ? kh * a.lhs_tile_bytes + m0 * 16 : m0 * 32 + kh * 16;
+  const int hi_off = rows_lhs ? 16 : a.lhs_tile_bytes;
   if (a.stage_wave_bytes > 0) {
     // Fetching the fragments straight into registers costs one load
     // instruction per K step and wave whatever M0 is (with M0 = 1 each moves
@@ -159,12 +170,30 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
     extern __shared__ __attribute__((aligned(16))) char stage_all[];
     char* stage = stage_all + wave * a.stage_wave_bytes;
     const int slice = count * step_bytes;
-    const __amdgpu_buffer_rsrc_t xsrc = __builtin_amdgcn_make_buffer_rsrc(
-        (void*)(a.lhs + (int64_t)(count > 0 ? first : 0) * step_bytes), 0, slice, 0x00020000);
+    // (row-major: the slice of every row, the rows SP steps and 16 bytes apart
+    // in LDS so that the 16-byte reads of up to 16 rows touch every bank once;
+    // a row's last load may run into the next row's place, which the next
+    // row's loads, later in order, overwrite)
+    const int row_stage = SP * step_bytes + 16;
+    if (rows_lhs) {
 #pragma unroll 1
-    for (int off = 0; off < slice; off += 1024)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(xsrc, (__attribute__((address_space(3))) void*)(stage + off), 16,
-                                               lane * 16, off, 0, 0);
+      for (int r = 0; r < a.M0; ++r) {
+        const __amdgpu_buffer_rsrc_t xsrc = __builtin_amdgcn_make_buffer_rsrc(
+            (void*)(a.lhs + r * a.lhs_row_pitch_bytes + (int64_t)(count > 0 ? first : 0) * step_bytes), 0, slice,
+            0x00020000);
+#pragma unroll 1
+        for (int off = 0; off < slice; off += 1024)
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(
+              xsrc, (__attribute__((address_space(3))) void*)(stage + r * row_stage + off), 16, lane * 16, off, 0, 0);
+      }
+    } else {
+      const __amdgpu_buffer_rsrc_t xsrc = __builtin_amdgcn_make_buffer_rsrc(
+          (void*)(a.lhs + (int64_t)(count > 0 ? first : 0) * step_bytes), 0, slice, 0x00020000);
+#pragma unroll 1
+      for (int off = 0; off < slice; off += 1024)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(xsrc, (__attribute__((address_space(3))) void*)(stage + off), 16,
+                                                 lane * 16, off, 0, 0);
+    }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int d = 0; d < kDepth; ++d) ring[d] = load_block(j, d);
@@ -174,9 +203,10 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
     for (int sp = 0; sp < SP; ++sp) {
       int4v lo = {0, 0, 0, 0}, hi = {0, 0, 0, 0};
       if (m0 < a.M0 && sp < count) {
-        const char* p = stage + sp * step_bytes + piece_off;
+        const char* p = rows_lhs ? stage + m0 * row_stage + sp * step_bytes + kh * 16 * kSub
+                                 : stage + sp * step_bytes + piece_off;
         lo = *(const int4v*)p;
-        if constexpr (kSub == 2) hi = *(const int4v*)(p + a.lhs_tile_bytes);
+        if constexpr (kSub == 2) hi = *(const int4v*)(p + hi_off);
       }
       xf[sp] = make_frag(lo, hi);
     }
@@ -191,9 +221,10 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
       // fp8: four tiles, two per lane half.
       int4v lo = {0, 0, 0, 0}, hi = {0, 0, 0, 0};
       if (m0 < a.M0 && sp < count) {
-        const char* p = a.lhs + (int64_t)s * step_bytes + piece_off;
+        const char* p = rows_lhs ? a.lhs + m0 * a.lhs_row_pitch_bytes + (int64_t)s * step_bytes + kh * 16 * kSub
+                                 : a.lhs + (int64_t)s * step_bytes + piece_off;
         lo = *(const int4v*)p;
-        if constexpr (kSub == 2) hi = *(const int4v*)(p + a.lhs_tile_bytes);
+        if constexpr (kSub == 2) hi = *(const int4v*)(p + hi_off);
       }
       xf[sp] = make_frag(lo, hi);
     }
@@ -217,13 +248,16 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
     if constexpr (kPerWave) {
       // (the stores below are divergent and the block's only consumer)
       keep_result_in_all_lanes(acc);
-      store_t* tile = (store_t*)a.out + (int64_t)j * a.out_stride_elems;
+      const bool rows_out = a.out_row_pitch_elems > 0;
+      store_t* tile = (store_t*)a.out + (rows_out ? (int64_t)j * 32 : (int64_t)j * a.out_stride_elems);
       const int mm = lane & 31;
       if (mm < a.M0) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           const int nn = 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-          const int at = a.transpose_out ? nn * a.M0 + mm : mm * 32 + nn;
+          if (rows_out && j * 32 + nn >= a.out_cols) continue;
+          const int64_t at = rows_out ? mm * a.out_row_pitch_elems + nn
+                                      : a.transpose_out ? nn * a.M0 + mm : mm * 32 + nn;
           const sum_t sum = (a.accumulate ? (sum_t)tile[at] : (sum_t)0) + (sum_t)acc[v];
           tile[at] = (store_t)sum;
         }
@@ -235,14 +269,17 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
 #pragma unroll
     for (int v = 0; v < 16; ++v) buf[wave][v][lane] = acc[v];
     __syncthreads();
-    store_t* tile = (store_t*)a.out + blockIdx.y * a.chunk_out_elems + (int64_t)j * a.out_stride_elems;
+    const bool rows_out = a.out_row_pitch_elems > 0;
+    store_t* tile = (store_t*)a.out + blockIdx.y * a.chunk_out_elems +
+                    (rows_out ? (int64_t)j * 32 : (int64_t)j * a.out_stride_elems);
 #pragma unroll
     for (int rep = 0; rep < 2; ++rep) {
       const int flat = rep * kThreads + threadIdx.x;   // v * 64 + lane
       const int l = flat & 63, v = flat >> 6;
       const int mm = l & 31, nn = 8 * (v >> 2) + 4 * (l >> 5) + (v & 3);
-      if (mm < a.M0) {
-        const int at = a.transpose_out ? nn * a.M0 + mm : mm * 32 + nn;
+      if (mm < a.M0 && !(rows_out && j * 32 + nn >= a.out_cols)) {
+        const int64_t at = rows_out ? mm * a.out_row_pitch_elems + nn
+                                    : a.transpose_out ? nn * a.M0 + mm : mm * 32 + nn;
         sum_t sum = a.accumulate ? (sum_t)tile[at] : (sum_t)0;
 #pragma unroll
         for (int w = 0; w < kWaves; ++w) sum += buf[w][v][l];
@@ -262,11 +299,16 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
 template <typename Cfg, int SP, bool kPartialOut>
 int launch_split_form(SkinnyArgs a, dim3 grid, hipStream_t s) {
   void (*kernel)(SkinnyArgs) = mmt4d_skinny_kernel<Cfg, SP, kPartialOut>;
-  const int step_bytes = (Cfg::kSub == 2 ? 4 : a.half_k0 ? 2 : 1) * a.lhs_tile_bytes;
-  const int wave_bytes = (SP * step_bytes + 1023) / 1024 * 1024;
+  const bool rows_lhs = a.lhs_row_pitch_bytes > 0;
+  const int step_bytes = rows_lhs ? 32 * Cfg::kSub : (Cfg::kSub == 2 ? 4 : a.half_k0 ? 2 : 1) * a.lhs_tile_bytes;
+  // (row-major: M0 rows of SP steps and 16 bytes, and room for the last load of the last row)
+  const int wave_bytes = rows_lhs ? (a.M0 * (SP * step_bytes + 16) + 1024 + 1023) / 1024 * 1024
+                                  : (SP * step_bytes + 1023) / 1024 * 1024;
   size_t lds = 0;
   a.stage_wave_bytes = 0;
-  if (kWaves * wave_bytes <= 64 * 1024) {
+  // (the kernel's static partial sums take 64 KiB of the 160)
+  constexpr int kMaxStageBytes = 96 * 1024;
+  if (kWaves * wave_bytes <= (rows_lhs ? kMaxStageBytes : 64 * 1024)) {
     a.stage_wave_bytes = wave_bytes;
     lds = (size_t)kWaves * wave_bytes;
     // (with the kernel's static partial sums this is more than the default 64 KiB)
@@ -274,7 +316,7 @@ int launch_split_form(SkinnyArgs a, dim3 grid, hipStream_t s) {
     int dev = 0;
     UK_RETURN_IF_HIP(hipGetDevice(&dev));
     if (dev < 0 || dev >= 64 || !((attr_set_on >> dev) & 1)) {
-      UK_RETURN_IF_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024));
+      UK_RETURN_IF_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kMaxStageBytes));
       if (dev >= 0 && dev < 64) attr_set_on |= 1ull << dev;
     }
   }
@@ -520,6 +562,9 @@ int launch_chunk(const iree_amd_uk_mmt4d_params_t& p, int chunks, int chunk_step
   a.accumulate = (p.flags & IREE_AMD_UK_FLAG_MMT4D_ACCUMULATE) != 0;
   a.chunk_steps = chunk_steps;
   a.chunk_out_elems = 0;
+  a.lhs_row_pitch_bytes = 0;
+  a.out_row_pitch_elems = 0;
+  a.out_cols = 0;
   a.batch = 1;
   a.lhs_batch_bytes = a.rhs_batch_bytes = a.out_batch_bytes = 0;
   if (batch) {
@@ -547,5 +592,60 @@ int launch_chunk(const iree_amd_uk_mmt4d_params_t& p, int chunks, int chunk_step
   }
 }
 }  // namespace
+
+// The whole linear layer on a few rows: out[M][out_cols] (+)= lhs[M][K] * rhs,
+// lhs and out row-major (`p` describes them as iree_amd_uk_matmul_packed_rhs
+// does: lhs_stride0 and out_stride0 are row pitches in elements), rhs packed
+// 32 x K0 tiles, 1 < M < 32. One launch of the kernel above with the rows of
+// the matrix as the rows of its single narrow tile; NOT_FOUND for what that
+// launch cannot take (a K that one launch row cannot hold in registers, too
+// few outer columns to be worth it, operands that are not 16-byte aligned).
+int launch_matmul_rows_skinny(const iree_amd_uk_mmt4d_params_t& p, int64_t M, int64_t out_cols, hipStream_t s) {
+  if (M < 2 || M > 31 || !mmt4d_skinny_supported(p.flags, 16, 32, p.K0)) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  const int mk = mfma_k_of(p.flags);
+  Mmt4dTypeInfo ti;
+  mmt4d_type_info(p.flags, &ti);
+  const int eb = ti.lhs_bits / 8;
+  const int64_t k_elems = p.K * p.K0;
+  if (p.K == 0 || k_elems % mk || p.N > 0x7FFFFFFF || out_cols > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  const int64_t steps = k_elems / mk;
+  // (a longer K, or a few outer columns only, want K split over workgroup
+  // rows, whose partial sums this form does not write)
+  if (steps > max_steps_per_launch(mk) || p.N * 2 <= device_cu_count()) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  const char* lhs = (const char*)p.lhs_buffer + p.lhs_offset * eb;
+  const char* rhs = (const char*)p.rhs_buffer + p.rhs_offset * eb;
+  if (((uintptr_t)lhs | (uintptr_t)rhs) % 16 || (p.rhs_stride0 * eb) % 16 || (p.lhs_stride0 * eb) % 16)
+    return IREE_AMD_UK_STATUS_NOT_FOUND;
+  if (M * p.lhs_stride0 * eb > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  SkinnyArgs a;
+  a.lhs = lhs; a.rhs = rhs;
+  a.out = (char*)p.out_buffer + p.out_offset * ti.out_bytes;
+  a.rhs_stride_bytes = p.rhs_stride0 * eb;
+  a.transpose_out = 0;
+  a.out_stride_elems = 0;
+  a.N = (int)p.N; a.M0 = (int)M;
+  a.ksteps = (int)steps;
+  a.steps_per_wave = 0;
+  a.lhs_tile_bytes = 0;
+  a.half_k0 = p.K0 * 2 == mk;
+  a.accumulate = (p.flags & IREE_AMD_UK_FLAG_MMT4D_ACCUMULATE) != 0;
+  a.chunk_steps = (int)steps;
+  a.chunk_out_elems = 0;
+  a.lhs_row_pitch_bytes = p.lhs_stride0 * eb;
+  a.out_row_pitch_elems = p.out_stride0;
+  a.out_cols = (int)out_cols;
+  a.batch = 1;
+  a.lhs_batch_bytes = a.rhs_batch_bytes = a.out_batch_bytes = 0;
+  switch (p.flags & IREE_AMD_UK_FLAG_MMT4D_TYPE_MASK) {
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F32: return launch_cfg<F16Cfg>(a, 1, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16F32: return launch_cfg<BF16Cfg>(a, 1, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32: return launch_cfg<S8Cfg>(a, 1, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F32F32F32: return launch_cfg<F32Cfg>(a, 1, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F8E4M3F8E4M3F32: return launch_cfg<F8Cfg>(a, 1, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F16: return launch_cfg<F16F16Cfg>(a, 1, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16BF16: return launch_cfg<BF16BF16Cfg>(a, 1, s);
+    default: return IREE_AMD_UK_STATUS_NOT_FOUND;
+  }
+}
 
 }  // namespace uk

@@ -163,7 +163,17 @@ def test_random_fused_matmul_calls_exact(uk, cuda, seed):
         K0 = int(rng.choice(k0s))
         M = int(rng.integers(1, 700)) if rng.integers(0, 4) else int(rng.integers(1, 40))
         N = int(rng.integers(1, 700)) if rng.integers(0, 4) else int(rng.integers(1, 40))
+        if rng.integers(0, 6) == 0:
+            # one row against whole tiles of columns: the matrix-vector form, which
+            # matmul_packed_rhs hands to the kernel for narrow left-hand side tiles
+            M, N = 1, 32 * int(rng.integers(1, 60))
         steps = int(rng.integers(1, 12)) if rng.integers(0, 5) else int(rng.integers(64, 160))
+        if rng.integers(0, 5) == 0:
+            # a few rows against more than 128 tiles of columns: matmul_packed_rhs runs the
+            # kernel for narrow left-hand side tiles on the row-major matrix itself
+            # (any K that one launch holds: up to 128 steps of 64 bytes per row)
+            M, N = int(rng.integers(2, 32)), int(rng.integers(4100, 5200))
+            steps = int(rng.integers(1, 129))
         K = steps * mfma_k
         acc = bool(rng.integers(0, 2))
         A = rng.integers(-lim, lim, (M, K))
