@@ -767,10 +767,12 @@ int matmul_packed_rhs_impl(
   // tile-size query gives for a static M of 1, which streams the right-hand
   // side once (N = 14336, K = 4096, f16: 23 us against 28 for the macro-tile
   // kernel with its K split).
-  if (M == 1 && N % 32 == 0 && b.batch == 1 && out_scale == 1.0f && mmt4d_skinny_supported(flags, 1, 32, K0)) {
+  if (M == 1 && N % 32 == 0 && out_scale == 1.0f && mmt4d_skinny_supported(flags, 1, 32, K0)) {
     const iree_amd_uk_mmt4d_params_t row = {lhs_buffer, lhs_offset, K, rhs_buffer, rhs_offset, rhs_stride0,
                                             out_buffer, out_offset, N, 1, N / 32, K / K0, 1, 32, K0, flags, nullptr};
-    st = launch_mmt4d_skinny(row, (hipStream_t)stream);
+    // (a batch of such rows, the attention scores of a decode step say: the planes of one launch)
+    st = b.batch == 1 ? launch_mmt4d_skinny(row, (hipStream_t)stream)
+                      : launch_batch_mmt4d_skinny(row, b.batch, b.lhs, b.rhs, b.out, (hipStream_t)stream);
   }
   // A few rows (2 to 31): the same kernel with the rows of the matrix as the
   // rows of its one narrow tile, reading them and writing the result row-major.

@@ -1050,7 +1050,10 @@ def test_batch_forms_of_the_fused_entry_points_match_single_calls(uk, cuda, type
         return rng.integers(-4, 5, n).astype(dt)
 
     for batch, M, N, K, gap in ((5, 70, 100, 3 * mfma_k, 64), (3, 200, 333, 9 * mfma_k, 0), (9, 32, 64, 2 * mfma_k, 16),
-                                (2, 40, 40, 4 * mfma_k, 48), (1, 33, 65, mfma_k, 0), (0, 33, 65, mfma_k, 0)):
+                                (2, 40, 40, 4 * mfma_k, 48), (1, 33, 65, mfma_k, 0), (0, 33, 65, mfma_k, 0),
+                                # one row per entry against whole tiles of columns: the planes of the
+                                # kernel for narrow left-hand side tiles
+                                (4, 1, 96, 4 * mfma_k, 16), (3, 1, 64, 2 * mfma_k, 0)):
         M1, N1, K1 = -(-M // 32), -(-N // 32), K // K0
         lhs_bs, rhs_bs = M1 * K1 * 32 * K0 + gap, N1 * K1 * 32 * K0 + gap
         a_bs, out_bs = M * K + gap, M * N + gap + 7
