@@ -83,7 +83,10 @@ struct SkinnyArgs {
 // is not worth splitting over the waves: every wave takes all of K for an
 // outer column of its own, 8 columns per workgroup at a time, and stores its
 // block itself (no sum through LDS, no barrier).
-template <typename Cfg, int SP, bool kPartialOut = false, bool kPerWave = false>
+// kRows: the row-major forms of left-hand side and result (SkinnyArgs); a
+// compile-time switch so that the tile forms carry none of their address
+// arithmetic (as a run-time one it cost the short-K batch form 16 %).
+template <typename Cfg, int SP, bool kPartialOut = false, bool kPerWave = false, bool kRows = false>
 __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
   typedef typename Cfg::frag_t frag_t;
   typedef typename Cfg::acc_t acc_t;
@@ -151,7 +154,7 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
   frag_t xf[SP];
   // bytes of the packed left-hand side per K step: its K tiles are consecutive
   // (row-major: the bytes of one ROW per K step, 32, or 64 for fp8)
-  const bool rows_lhs = a.lhs_row_pitch_bytes > 0;
+  constexpr bool rows_lhs = kRows;
   const int step_bytes = rows_lhs ? 32 * kSub : (kSub == 2 ? 4 : a.half_k0 ? 2 : 1) * a.lhs_tile_bytes;
   // this lane's first piece inside a step (the second one, fp8, a tile further;
   // row-major: the next 16 bytes of the row)
@@ -248,7 +251,7 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
     if constexpr (kPerWave) {
       // (the stores below are divergent and the block's only consumer)
       keep_result_in_all_lanes(acc);
-      const bool rows_out = a.out_row_pitch_elems > 0;
+      constexpr bool rows_out = kRows;
       store_t* tile = (store_t*)a.out + (rows_out ? (int64_t)j * 32 : (int64_t)j * a.out_stride_elems);
       const int mm = lane & 31;
       if (mm < a.M0) {
@@ -269,7 +272,7 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
 #pragma unroll
     for (int v = 0; v < 16; ++v) buf[wave][v][lane] = acc[v];
     __syncthreads();
-    const bool rows_out = a.out_row_pitch_elems > 0;
+    constexpr bool rows_out = kRows;
     store_t* tile = (store_t*)a.out + blockIdx.y * a.chunk_out_elems +
                     (rows_out ? (int64_t)j * 32 : (int64_t)j * a.out_stride_elems);
 #pragma unroll
@@ -296,10 +299,10 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
 // One launch of the form that splits K over the waves, with the left-hand side
 // staged through LDS when the slices of the 8 waves fit 64 KiB of it (narrow
 // tiles of up to 8 rows at the longest K a launch takes).
-template <typename Cfg, int SP, bool kPartialOut>
+template <typename Cfg, int SP, bool kPartialOut, bool kRows = false>
 int launch_split_form(SkinnyArgs a, dim3 grid, hipStream_t s) {
-  void (*kernel)(SkinnyArgs) = mmt4d_skinny_kernel<Cfg, SP, kPartialOut>;
-  const bool rows_lhs = a.lhs_row_pitch_bytes > 0;
+  void (*kernel)(SkinnyArgs) = mmt4d_skinny_kernel<Cfg, SP, kPartialOut, false, kRows>;
+  constexpr bool rows_lhs = kRows;
   const int step_bytes = rows_lhs ? 32 * Cfg::kSub : (Cfg::kSub == 2 ? 4 : a.half_k0 ? 2 : 1) * a.lhs_tile_bytes;
   // (row-major: M0 rows of SP steps and 16 bytes, and room for the last load of the last row)
   const int wave_bytes = rows_lhs ? (a.M0 * (SP * step_bytes + 16) + 1024 + 1023) / 1024 * 1024
@@ -324,7 +327,7 @@ int launch_split_form(SkinnyArgs a, dim3 grid, hipStream_t s) {
   return check_hip(hipGetLastError(), "mmt4d_skinny launch");
 }
 
-template <typename Cfg>
+template <typename Cfg, bool kRows = false>
 int launch_cfg(SkinnyArgs a, int chunks, hipStream_t s) {
   const int cus = device_cu_count();
   // (a batch: about two workgroups per compute unit over all planes)
@@ -343,10 +346,10 @@ int launch_cfg(SkinnyArgs a, int chunks, hipStream_t s) {
     a.stage_wave_bytes = 0;
     const dim3 grid(groups < per_plane ? groups : per_plane, 1, a.batch > 1 ? a.batch : 1);
     if (a.chunk_steps <= 8) {
-      hipLaunchKernelGGL((mmt4d_skinny_kernel<Cfg, 8, false, true>), grid, dim3(kThreads), 0, s, a);
+      hipLaunchKernelGGL((mmt4d_skinny_kernel<Cfg, 8, false, true, kRows>), grid, dim3(kThreads), 0, s, a);
     } else {
       if constexpr (kPerWaveSteps >= 16)
-        hipLaunchKernelGGL((mmt4d_skinny_kernel<Cfg, 16, false, true>), grid, dim3(kThreads), 0, s, a);
+        hipLaunchKernelGGL((mmt4d_skinny_kernel<Cfg, 16, false, true, kRows>), grid, dim3(kThreads), 0, s, a);
     }
     return check_hip(hipGetLastError(), "mmt4d_skinny launch");
   }
@@ -355,19 +358,19 @@ int launch_cfg(SkinnyArgs a, int chunks, hipStream_t s) {
   a.steps_per_wave = per;
   const dim3 grid(blocks, chunks, a.batch > 1 ? a.batch : 1);
   if (chunks > 1 && kNarrowOut) {
-    if constexpr (kNarrowOut) {
+    if constexpr (kNarrowOut && !kRows) {
       if (per <= 8) return launch_split_form<Cfg, 8, true>(a, grid, s);
       if (per <= 16) return launch_split_form<Cfg, 16, true>(a, grid, s);
       if (per <= 32) return launch_split_form<Cfg, 32, true>(a, grid, s);
     }
     return IREE_AMD_UK_STATUS_NOT_FOUND;
   }
-  if (per <= 8) return launch_split_form<Cfg, 8, false>(a, grid, s);
-  if (per <= 16) return launch_split_form<Cfg, 16, false>(a, grid, s);
+  if (per <= 8) return launch_split_form<Cfg, 8, false, kRows>(a, grid, s);
+  if (per <= 16) return launch_split_form<Cfg, 16, false, kRows>(a, grid, s);
   if (per <= 32) {
     // (32 fp8 steps of 8 registers each would not fit the register file)
     if constexpr (Cfg::kSub == 2) return IREE_AMD_UK_STATUS_NOT_FOUND;
-    else return launch_split_form<Cfg, 32, false>(a, grid, s);
+    else return launch_split_form<Cfg, 32, false, kRows>(a, grid, s);
   }
   return IREE_AMD_UK_STATUS_NOT_FOUND;
 }
@@ -637,13 +640,13 @@ int launch_matmul_rows_skinny(const iree_amd_uk_mmt4d_params_t& p, int64_t M, in
   a.batch = 1;
   a.lhs_batch_bytes = a.rhs_batch_bytes = a.out_batch_bytes = 0;
   switch (p.flags & IREE_AMD_UK_FLAG_MMT4D_TYPE_MASK) {
-    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F32: return launch_cfg<F16Cfg>(a, 1, s);
-    case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16F32: return launch_cfg<BF16Cfg>(a, 1, s);
-    case IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32: return launch_cfg<S8Cfg>(a, 1, s);
-    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F32F32F32: return launch_cfg<F32Cfg>(a, 1, s);
-    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F8E4M3F8E4M3F32: return launch_cfg<F8Cfg>(a, 1, s);
-    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F16: return launch_cfg<F16F16Cfg>(a, 1, s);
-    case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16BF16: return launch_cfg<BF16BF16Cfg>(a, 1, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F32: return launch_cfg<F16Cfg, true>(a, 1, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16F32: return launch_cfg<BF16Cfg, true>(a, 1, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32: return launch_cfg<S8Cfg, true>(a, 1, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F32F32F32: return launch_cfg<F32Cfg, true>(a, 1, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F8E4M3F8E4M3F32: return launch_cfg<F8Cfg, true>(a, 1, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F16: return launch_cfg<F16F16Cfg, true>(a, 1, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16BF16: return launch_cfg<BF16BF16Cfg, true>(a, 1, s);
     default: return IREE_AMD_UK_STATUS_NOT_FOUND;
   }
 }
