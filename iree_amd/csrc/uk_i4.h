@@ -38,6 +38,11 @@ struct I4Args {
   //   nt * K * 16 + s * span_stride + c * col_stride + kc * 16
   uint32_t span_stride, col_stride;
   uint32_t w_bytes;       // size of the weight buffer
+  // A K longer than one workgroup takes (512 KB elements): workgroup row
+  // blockIdx.y multiplies the y-th slice of so many elements and, with more
+  // than one row, stores its f32 sums at partial[(y * M + m) * N + n] for a
+  // second kernel to add in row order (nullptr: one row, f16 results to out).
+  float* partial;
 };
 
 // Position, in the tiled layout, of the byte that holds elements (n, k) and

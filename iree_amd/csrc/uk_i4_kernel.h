@@ -81,11 +81,12 @@ __device__ __forceinline__ void dequant_matmul_i4_body(const I4Args& a) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int nl = lane & 15, kc = lane >> 4;
-  const int k_slice = wave * KB * 64;
+  const int krow = blockIdx.y;               // K slice of this workgroup row (512 KB elements each)
+  const int k_slice = (krow * kWaves + wave) * KB * 64;
   const int g_first = k_slice >> a.log2_gs;  // first group of this wave's slice
   const uint32_t tile_bytes = (uint32_t)a.K * 16;
   const uint32_t voff = nl * a.col_stride + kc * 16;
-  const uint32_t soff_wave = wave * SP * a.span_stride;
+  const uint32_t soff_wave = (krow * kWaves + wave) * SP * a.span_stride;
   const uint32_t half_stride = 16 * a.col_stride;
 
   // Raw group parameters of this lane's two columns for the wave's K slice
@@ -394,7 +395,10 @@ __device__ __forceinline__ void dequant_matmul_i4_body(const I4Args& a) {
       const int r = slot & 3, hm = slot >> 2, h = hm / MH, mh = hm % MH;
       const int m = a.m_base + mh * 16 + 4 * (l >> 4) + r;
       const int n = nt * 32 + h * 16 + (l & 15);
-      if (m < a.M && n < a.N) a.out[(size_t)m * a.N + n] = __half_as_ushort(__float2half_rn(sum));
+      if (m < a.M && n < a.N) {
+        if (a.partial) a.partial[((size_t)krow * a.M + m) * a.N + n] = sum;
+        else a.out[(size_t)m * a.N + n] = __half_as_ushort(__float2half_rn(sum));
+      }
     }
     // The other half of `partial` is used by the next tile; this half is
     // rewritten only two tiles later, after the next tile's barrier.

@@ -39,6 +39,8 @@
 #include "uk_i4.h"
 #include "uk_i4_kernel.h"
 
+#include <memory>
+
 #include <hip/hip_fp16.h>
 
 namespace uk {
@@ -94,7 +96,7 @@ __global__ __launch_bounds__(256) void dequant_matmul_i4_generic_kernel(I4Args a
 }
 
 template <int KB, int MH, bool kZpU4, int kLog2Gs>
-int launch_instance(const I4Args& a, int blocks, hipStream_t s) {
+int launch_instance(const I4Args& a, int blocks, int k_rows, hipStream_t s) {
   void (*kernel)(I4Args) = dequant_matmul_i4_kernel<KB, MH, kZpU4, kLog2Gs>;
   // 16-row form: the rows it stages (8 or 16 per wave); 32-row form: two
   // buffers of 8 rows per wave, and at least the 64 KiB of partial sums that
@@ -114,42 +116,73 @@ int launch_instance(const I4Args& a, int blocks, hipStream_t s) {
       if (dev >= 0 && dev < 64) attr_set_on |= 1ull << dev;
     }
   }
-  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kThreads), lds, s, a);
+  hipLaunchKernelGGL(kernel, dim3(blocks, k_rows), dim3(kThreads), lds, s, a);
   return check_hip(hipGetLastError(), "dequant_matmul_i4 launch");
 }
 
 template <int KB, int MH, bool kZpU4>
-int launch_one(const I4Args& a, int blocks, hipStream_t s) {
+int launch_one(const I4Args& a, int blocks, int k_rows, hipStream_t s) {
+  // (with K rows a group may be longer than a workgroup's slice of K: it is
+  // then "at least the wave's slice" all the same)
   switch (a.log2_gs) {
-    case 5: return launch_instance<KB, MH, kZpU4, 5>(a, blocks, s);
-    case 6: return launch_instance<KB, MH, kZpU4, 6>(a, blocks, s);
-    case 7: return launch_instance<KB, MH, kZpU4, 7>(a, blocks, s);
-    case 8: return launch_instance<KB, MH, kZpU4, 8>(a, blocks, s);
-    default: return launch_instance<KB, MH, kZpU4, 9>(a, blocks, s);
+    case 5: return launch_instance<KB, MH, kZpU4, 5>(a, blocks, k_rows, s);
+    case 6: return launch_instance<KB, MH, kZpU4, 6>(a, blocks, k_rows, s);
+    case 7: return launch_instance<KB, MH, kZpU4, 7>(a, blocks, k_rows, s);
+    case 8: return launch_instance<KB, MH, kZpU4, 8>(a, blocks, k_rows, s);
+    default: return launch_instance<KB, MH, kZpU4, 9>(a, blocks, k_rows, s);
   }
 }
 
+// K = k_rows slices of 512 KB elements. One slice: f16 results straight to the
+// output. More: every workgroup row multiplies its slice into f32 partial sums
+// in the stream's scratch buffer and the K-split reduction kernel adds them in
+// row order and rounds to f16 once (NOT_FOUND without that memory: the caller
+// falls back to the kernel that walks all of K in one workgroup).
 template <int KB>
-int launch_fast(I4Args a, hipStream_t s) {
+int launch_fast(I4Args a, int k_rows, hipStream_t s) {
   const int cus = device_cu_count();
+  std::unique_ptr<ScratchLease> lease;   // held until the reduction has been queued
+  a.partial = nullptr;
+  if (k_rows > 1) {
+    if (((int64_t)a.M * a.N) % 4) return IREE_AMD_UK_STATUS_NOT_FOUND;
+    lease.reset(new ScratchLease(s, (size_t)k_rows * a.M * a.N * 4));
+    a.partial = (float*)lease->ptr();
+    if (!a.partial) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  }
   int m_base = 0;
   while (m_base < a.M) {
     a.m_base = m_base;
     // One workgroup per compute unit (two of the 16-row kernel would fit, and
-    // measure slower: 12.4 against 9.9 us on the decode shape).
-    const int blocks = a.n_tiles < cus ? a.n_tiles : cus;
+    // measure slower: 12.4 against 9.9 us on the decode shape); with K rows,
+    // a row gets its share of the compute units.
+    int blocks = cus / k_rows;
+    blocks = blocks < 1 ? 1 : blocks;
+    blocks = a.n_tiles < blocks ? a.n_tiles : blocks;
     int st;
     if (a.M - m_base > 16) {
-      st = a.zp_u4 ? launch_one<KB, 2, true>(a, blocks, s) : launch_one<KB, 2, false>(a, blocks, s);
+      st = a.zp_u4 ? launch_one<KB, 2, true>(a, blocks, k_rows, s) : launch_one<KB, 2, false>(a, blocks, k_rows, s);
       m_base += 32;
     } else {
       a.stage_rows = stage_rows_for(a.M - m_base);
-      st = a.zp_u4 ? launch_one<KB, 1, true>(a, blocks, s) : launch_one<KB, 1, false>(a, blocks, s);
+      st = a.zp_u4 ? launch_one<KB, 1, true>(a, blocks, k_rows, s) : launch_one<KB, 1, false>(a, blocks, k_rows, s);
       m_base += 16;
     }
     UK_RETURN_IF_ERROR(st);
   }
-  return 0;
+  if (k_rows == 1) return 0;
+  KSplitReduceArgs r;
+  r.partials = a.partial;
+  r.slices = k_rows;
+  r.M = 1; r.N = 1;
+  r.flat_elems = (int64_t)a.M * a.N;
+  r.out = a.out;
+  r.out_stride_bytes = 0;
+  r.accumulate = 0;
+  r.row_major_out = 0; r.out_rows = r.out_cols = 0;
+  r.out_scale = 1.0f;
+  r.acc_is_float = 1;
+  r.out_kind = 1;   // f16
+  return launch_ksplit_reduce(r, s);
 }
 
 }  // namespace
@@ -177,21 +210,31 @@ int launch_dequant_matmul_i4(const void* x, const void* w, const void* scale, co
   const bool gs_pow2 = (1ll << a.log2_gs) == group_size;
   a.span_stride = tiled ? 2048u : 64u;
   a.col_stride = tiled ? 64u : (uint32_t)(K / 2);
-  // Fast path: K = 512 * KB for KB in {4, 8} (every wave owns KB blocks of 64),
+  // Fast path: K in whole slices of 512 * KB for KB in {4, 8} (every wave owns
+  // KB blocks of 64 of its workgroup's slice; more than one slice: workgroup
+  // rows and a second kernel that adds their partial sums),
   // power-of-two groups (below 128 only from tiled weights, where a group never
   // straddles an MFMA), a weight buffer that 32-bit offsets can address (plus
   // one tile, for the offset of the tile after the last), 16-byte aligned
   // operands, and group parameters aligned to what one wave slice loads at once.
-  const int64_t kb = K / 512;
   const int64_t w_bytes = N * K / 2;
-  const bool k_ok = K % 512 == 0 && (kb == 4 || kb == 8);
+  // (a longer K in whole slices of 4096, or else of 2048, over workgroup rows)
+  const int slice_kb = K % 4096 == 0 ? 8 : 4;
+  const int64_t k_rows = K / (512 * slice_kb);
+  const bool k_ok = K % 2048 == 0 && K >= 2048 && k_rows <= 64;
   const bool gs_ok = gs_pow2 && group_size >= (tiled ? 32 : 128);
   const bool size_ok = w_bytes + K * 16 < (1ll << 32);
   const bool aligned = ((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0 &&
                        ((uintptr_t)scale % 16) == 0 && ((uintptr_t)zp % 16) == 0;
-  if (k_ok && gs_ok && size_ok && aligned) {
+  // (one row against few tiles of columns and a split K: the kernel below, in
+  // which a wave walks all of K for its columns, measures a little faster, 11.1
+  // against 11.9 us at N = 4096, K = 14336, and needs no second launch)
+  const bool one_row_few_tiles = M == 1 && k_rows > 1 && a.n_tiles * 2 <= device_cu_count() && K % 2048 == 0 &&
+                                 group_size >= (tiled ? 64 : 128) && group_size <= 256;
+  if (k_ok && gs_ok && size_ok && aligned && !one_row_few_tiles) {
     a.w_bytes = (uint32_t)w_bytes;
-    return kb == 4 ? launch_fast<4>(a, s) : launch_fast<8>(a, s);
+    const int st = slice_kb == 4 ? launch_fast<4>(a, (int)k_rows, s) : launch_fast<8>(a, (int)k_rows, s);
+    if (st != IREE_AMD_UK_STATUS_NOT_FOUND) return st;
   }
   if (gs_pow2 && size_ok && aligned && K > 0) {
     // Other K (whole 2048s): the per-wave-column kernel. It has a longer
@@ -217,6 +260,11 @@ int launch_dequant_matmul_i4(const void* x, const void* w, const void* scale, co
       }
       if (st != IREE_AMD_UK_STATUS_NOT_FOUND) return st;
     }
+  }
+  if (one_row_few_tiles && k_ok && gs_ok && size_ok && aligned) {
+    a.w_bytes = (uint32_t)w_bytes;
+    const int st = slice_kb == 4 ? launch_fast<4>(a, (int)k_rows, s) : launch_fast<8>(a, (int)k_rows, s);
+    if (st != IREE_AMD_UK_STATUS_NOT_FOUND) return st;
   }
   const int64_t total = M * N;
   int64_t blocks = ceil_div(total, 256);

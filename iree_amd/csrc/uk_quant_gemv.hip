@@ -1,6 +1,8 @@
 // Grouped int4-weight dequantising matmul for up to 16 rows of activations and
-// ANY K in whole 2048s (the kernel in uk_quant.hip keeps its slice of the
-// activations in registers and so serves K = 2048 and 4096 only). Same
+// ANY K in whole 2048s (the kernel in uk_quant.hip keeps a slice of 2048 or
+// 4096 of the activations in registers and takes a longer K as workgroup rows
+// plus a second kernel that adds their sums; this one serves what that cannot
+// take, and one row against few columns, where it measures faster). Same
 // arithmetic, different decomposition:
 //
 //   * the activations (at most 16 rows) live in LDS, already in MFMA A-operand

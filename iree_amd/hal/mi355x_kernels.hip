@@ -284,7 +284,8 @@ __device__ __forceinline__ void hal_dequant_matmul_i4(const void* x, const void*
   a.span_stride = 2048;
   a.col_stride = 64;
   a.w_bytes = (uint32_t)((int64_t)N * (K / 2));
-  if ((int)blockIdx.x >= a.n_tiles) return;
+  a.partial = nullptr;
+  if ((int)blockIdx.x >= a.n_tiles || blockIdx.y != 0) return;
   i4::dequant_matmul_i4_body<8, MH, true, 7>(a);
 }
 
