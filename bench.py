@@ -679,9 +679,10 @@ def extras(args, torch, iree_amd, F, synth, lhs, rhs, out, ex):
     assert int(rsink.abs().sum()) == 0
     del rsink
     # the transposed shape (N 4096, K 14336, the same byte counts and buffers):
-    # a K the register-resident kernel cannot take; the activations go through
-    # LDS, 1 row in one pass, 8 rows in two passes over the weights
-    for Mq in (1, 8):
+    # one row runs the kernel that keeps the activations in LDS, more rows the
+    # register-resident kernel as 7 workgroup rows over K slices of 2048 plus
+    # the ordered reduction of their sums
+    for Mq in (1, 8, 32):
         xq = torch.from_numpy(synth.normal_f16(45 + Mq, Mq * Nq).view(np.int16)).cuda()
         oq = torch.empty(Mq * Kq, dtype=torch.int16, device="cuda")
         state["i"] = 0
