@@ -409,7 +409,9 @@ IREE_AMD_UK_EXPORT int iree_amd_uk_query_tile_sizes_2d(
  * form: a floating tensor subtracted after uitofp) or packed uint4 [N][K/gs]
  * (two per byte, even group in the low nibble) when ..._ZP_U4 is set. f32
  * accumulation, result rounded to f16 once (RNE). out: f16 [M][N] row-major.
- * Requires K % group_size == 0, group_size % 32 == 0, 1 <= M.
+ * Requires K % group_size == 0, group_size % 32 == 0, 1 <= M. A K beyond
+ * 4096 is multiplied in slices whose f32 sums go through the stream's scratch
+ * buffer (see iree_amd_uk_mmt4d on that buffer).
  *===------------------------------------------------------------------------===*/
 #define IREE_AMD_UK_FLAG_DEQUANT_MATMUL_ZP_F16 0x0
 #define IREE_AMD_UK_FLAG_DEQUANT_MATMUL_ZP_U4 0x1
