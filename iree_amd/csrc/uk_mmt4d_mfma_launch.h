@@ -302,7 +302,12 @@ int launch_cfg(const MfmaArgs& a, hipStream_t s) {
       // most 4 %).
       double best_us = best_cost * a.ksteps * unit_us * 0.95;
       int split_v = -1, split_n = 0;
-      for (int v = 0; v < 4; ++v)
+      for (int v = 0; v < 4; ++v) {
+        // (up to 64 rows: with the tile and slice count forced, 128x128 tiles
+        // won on every such shape measured, by up to 10 % over what this
+        // estimate picked among the larger tiles, whose rows are as idle and
+        // whose workgroups are half as many)
+        if (a.M <= 2 && v != 3) continue;
         for (int n = 2; n <= 8; ++n) {
           if (a.ksteps / n < 24) break;
           const int64_t tiles = ceil_div((int64_t)a.M, (int64_t)2 * variants[v].wm) *
@@ -312,6 +317,7 @@ int launch_cfg(const MfmaArgs& a, hipStream_t s) {
                             (n + 1 + (a.accumulate ? 1 : 0)) * out_mb / 3.0;
           if (us < best_us) { best_us = us; split_v = v; split_n = n; }
         }
+      }
       if (split_n > 1) {
         const int st = launch_k_split<Cfg>(a, split_v, split_n, s);
         if (st != IREE_AMD_UK_STATUS_NOT_FOUND) return st;
