@@ -28,6 +28,8 @@
 // side in registers and stores every block transposed, as the 32 x N0 tile the
 // caller asked for.
 #include "uk_common.h"
+
+#include <memory>
 #include "uk_mfma_cfg.h"
 
 #include <type_traits>
@@ -358,10 +360,10 @@ int launch_cfg(SkinnyArgs a, int chunks, hipStream_t s) {
   a.steps_per_wave = per;
   const dim3 grid(blocks, chunks, a.batch > 1 ? a.batch : 1);
   if (chunks > 1 && kNarrowOut) {
-    if constexpr (kNarrowOut && !kRows) {
-      if (per <= 8) return launch_split_form<Cfg, 8, true>(a, grid, s);
-      if (per <= 16) return launch_split_form<Cfg, 16, true>(a, grid, s);
-      if (per <= 32) return launch_split_form<Cfg, 32, true>(a, grid, s);
+    if constexpr (kNarrowOut) {
+      if (per <= 8) return launch_split_form<Cfg, 8, true, kRows>(a, grid, s);
+      if (per <= 16) return launch_split_form<Cfg, 16, true, kRows>(a, grid, s);
+      if (per <= 32) return launch_split_form<Cfg, 32, true, kRows>(a, grid, s);
     }
     return IREE_AMD_UK_STATUS_NOT_FOUND;
   }
@@ -612,9 +614,23 @@ int launch_matmul_rows_skinny(const iree_amd_uk_mmt4d_params_t& p, int64_t M, in
   const int64_t k_elems = p.K * p.K0;
   if (p.K == 0 || k_elems % mk || p.N > 0x7FFFFFFF || out_cols > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
   const int64_t steps = k_elems / mk;
-  // (a longer K, or a few outer columns only, want K split over workgroup
-  // rows, whose partial sums this form does not write)
-  if (steps > max_steps_per_launch(mk) || p.N * 2 <= device_cu_count()) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  // (a K longer than one launch row keeps in registers goes to the macro-tile
+  // kernel with its K split, which measures as fast or faster there)
+  if (steps > max_steps_per_launch(mk)) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  // Few outer columns: K is split over workgroup rows as in launch_mmt4d_skinny,
+  // every row writing row-major f32 (s32) sums to the stream's scratch buffer,
+  // which the reduction kernel adds in row order into a result without gaps
+  // between its rows.
+  const int cus = device_cu_count();
+  int64_t chunks = 1;
+  if (p.N * 2 <= cus && steps >= 64) {
+    chunks = cus / p.N;
+    if (chunks > steps / 32) chunks = steps / 32;
+    if (chunks > 8) chunks = 8;
+    if (chunks < 1) chunks = 1;
+  }
+  if (p.N * 2 <= cus && chunks < 2) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  if (chunks > 1 && (p.out_stride0 != out_cols || (M * out_cols) % 4)) return IREE_AMD_UK_STATUS_NOT_FOUND;
   const char* lhs = (const char*)p.lhs_buffer + p.lhs_offset * eb;
   const char* rhs = (const char*)p.rhs_buffer + p.rhs_offset * eb;
   if (((uintptr_t)lhs | (uintptr_t)rhs) % 16 || (p.rhs_stride0 * eb) % 16 || (p.lhs_stride0 * eb) % 16)
@@ -639,16 +655,46 @@ int launch_matmul_rows_skinny(const iree_amd_uk_mmt4d_params_t& p, int64_t M, in
   a.out_cols = (int)out_cols;
   a.batch = 1;
   a.lhs_batch_bytes = a.rhs_batch_bytes = a.out_batch_bytes = 0;
+  std::unique_ptr<ScratchLease> lease;   // held until the reduction has been queued
+  if (chunks > 1) {
+    const int64_t chunk_steps = (steps + chunks - 1) / chunks;
+    chunks = (steps + chunk_steps - 1) / chunk_steps;
+    if (chunks < 2) return IREE_AMD_UK_STATUS_NOT_FOUND;
+    lease.reset(new ScratchLease(s, (size_t)(chunks * M * out_cols * 4)));
+    if (!lease->ptr()) return IREE_AMD_UK_STATUS_NOT_FOUND;
+    a.out = (char*)lease->ptr();
+    a.accumulate = 0;
+    a.chunk_steps = (int)chunk_steps;
+    a.chunk_out_elems = M * out_cols;
+    a.out_row_pitch_elems = out_cols;
+  }
+  int st;
   switch (p.flags & IREE_AMD_UK_FLAG_MMT4D_TYPE_MASK) {
-    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F32: return launch_cfg<F16Cfg, true>(a, 1, s);
-    case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16F32: return launch_cfg<BF16Cfg, true>(a, 1, s);
-    case IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32: return launch_cfg<S8Cfg, true>(a, 1, s);
-    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F32F32F32: return launch_cfg<F32Cfg, true>(a, 1, s);
-    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F8E4M3F8E4M3F32: return launch_cfg<F8Cfg, true>(a, 1, s);
-    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F16: return launch_cfg<F16F16Cfg, true>(a, 1, s);
-    case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16BF16: return launch_cfg<BF16BF16Cfg, true>(a, 1, s);
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F32: st = launch_cfg<F16Cfg, true>(a, (int)chunks, s); break;
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16F32: st = launch_cfg<BF16Cfg, true>(a, (int)chunks, s); break;
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32: st = launch_cfg<S8Cfg, true>(a, (int)chunks, s); break;
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F32F32F32: st = launch_cfg<F32Cfg, true>(a, (int)chunks, s); break;
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F8E4M3F8E4M3F32: st = launch_cfg<F8Cfg, true>(a, (int)chunks, s); break;
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F16: st = launch_cfg<F16F16Cfg, true>(a, (int)chunks, s); break;
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16BF16: st = launch_cfg<BF16BF16Cfg, true>(a, (int)chunks, s); break;
     default: return IREE_AMD_UK_STATUS_NOT_FOUND;
   }
+  if (st || chunks == 1) return st;
+  KSplitReduceArgs r;
+  r.partials = lease->ptr();
+  r.slices = (int)chunks;
+  r.M = 1; r.N = 1;
+  r.flat_elems = M * out_cols;
+  r.out = (char*)p.out_buffer + p.out_offset * ti.out_bytes;
+  r.out_stride_bytes = 0;
+  r.accumulate = (p.flags & IREE_AMD_UK_FLAG_MMT4D_ACCUMULATE) != 0;
+  r.row_major_out = 0; r.out_rows = r.out_cols = 0;
+  r.out_scale = 1.0f;
+  r.acc_is_float = (p.flags & IREE_AMD_UK_FLAG_MMT4D_TYPE_MASK) != IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32;
+  const uint32_t type = p.flags & IREE_AMD_UK_FLAG_MMT4D_TYPE_MASK;
+  r.out_kind = type == IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F16 ? 1
+               : type == IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16BF16 ? 2 : 0;
+  return launch_ksplit_reduce(r, s);
 }
 
 }  // namespace uk
