@@ -63,7 +63,7 @@ def parse_args():
                     "mmt4d_f16 | mmt4d_f16_acc | mmt4d_i8 | mmt4d_s16s8 | mmt4d_s16s16 | mmt4d_fp8 | mmt4d_f16_ksplit | mlp_fp8 | pack | unpack | "
                     "pack_transpose | unpack_transpose | dequant_i4[_m8|_m32] | dequant_i4_reassoc[_m8|_m32] | batch_mmt4d_f16 | "
                     "batch_mmt4d_f16_narrow | mmt4d_f16_narrow_m1 | mmt4d_f16_narrow_m8 | mmt4d_f16_narrow_n8 | "
-                    "matmul_rowmajor_lhs_f16 | matmul_rowmajor_lhs_i8 | matmul_rowmajor_lhs_fp8 | "
+                    "matmul_rowmajor_lhs_f16 | matmul_rowmajor_lhs_i8 | matmul_rowmajor_lhs_fp8 | matmul_rowmajor_lhs_f16_m8 | "
                     "chain_i8_1024 | copy | copy_rotating | copy_rotating_nt | copy_rotating_nt_single_waves | read_only_29mb")
     return ap.parse_args()
 
@@ -919,6 +919,19 @@ def run_only(args, torch, iree_amd, F, synth, mm_step):
         cm = torch.zeros(size * size, dtype=odt, device="cuda")
         # (the operand values stand for a packed right-hand side as they are: any bytes do for timing)
         fn = lambda: iree_amd.matmul_packed_rhs(am, bm, cm, size, size, size, k0, tf)  # noqa: E731
+    elif args.only == "matmul_rowmajor_lhs_f16_m8":
+        # a decode step's linear layer: 8 row-major rows against N 14336, K 4096
+        # (six rotating packed right-hand sides), row-major result
+        Nn, Kn, Mr = 14336, 4096, 8
+        rn = [torch.from_numpy(synth.normal_f16(50 + i, Nn * Kn, 1 / 64).view(np.int16)).cuda() for i in range(6)]
+        ar = torch.from_numpy(synth.normal_f16(62, Mr * Kn).view(np.int16)).cuda()
+        cr = torch.empty(Mr * Nn, dtype=torch.float32, device="cuda")
+        st = {"i": 0}
+
+        def fn():
+            k = st["i"] % 6
+            st["i"] += 1
+            iree_amd.matmul_packed_rhs(ar, rn[k], cr, Mr, Nn, Kn, 8, F.MMT4D_TYPE_F16F16F32)
     elif args.only == "chain_i8_1024":
         n1k = 1024
         a8 = torch.from_numpy(synth.uniform_int8(1, n1k * n1k)).cuda()
