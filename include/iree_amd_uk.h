@@ -592,7 +592,7 @@ IREE_AMD_UK_EXPORT int iree_amd_uk_batch_mmt4d_unpack(
  * otherwise; use the three-call sequence then): K a multiple of the
  * matrix-core K extent (32 for f16/bf16 and i8, 8 for f32, 64 for fp8),
  * K0 as served by iree_amd_uk_mmt4d, 16-byte aligned lhs rows and rhs tiles.
- * Bit-identical to pack + mmt4d + unpack. Fewer than 32 rows (a decode step)
+ * Bit-identical to pack + mmt4d + unpack. Up to 24 rows (32 of 1-byte elements: a decode step)
  * with a K of up to 4096 elements of 2 bytes (8192 of 1 byte) run the kernel
  * for narrow left-hand side tiles on the rows themselves (float sums then
  * come in that kernel's order: the bits of mmt4d on M0 = M tiles). With N >= 16384 (and M >= 512) the

@@ -774,9 +774,9 @@ int matmul_packed_rhs_impl(
     st = b.batch == 1 ? launch_mmt4d_skinny(row, (hipStream_t)stream)
                       : launch_batch_mmt4d_skinny(row, b.batch, b.lhs, b.rhs, b.out, (hipStream_t)stream);
   }
-  // A few rows (2 to 31): the same kernel with the rows of the matrix as the
+  // A few rows (2 to 32): the same kernel with the rows of the matrix as the
   // rows of its one narrow tile, reading them and writing the result row-major.
-  if (st == IREE_AMD_UK_STATUS_NOT_FOUND && M > 1 && M < 32 && b.batch == 1 && out_scale == 1.0f)
+  if (st == IREE_AMD_UK_STATUS_NOT_FOUND && M > 1 && M <= 32 && b.batch == 1 && out_scale == 1.0f)
     st = launch_matmul_rows_skinny(p, M, N, (hipStream_t)stream);
   if (st == IREE_AMD_UK_STATUS_NOT_FOUND && mmt4d_mfma_supported(flags, 32, 32, K0))
     st = launch_matmul_packed_rhs_mfma(p, M, N, out_scale, b.batch, b.lhs, b.rhs, b.out, (hipStream_t)stream);

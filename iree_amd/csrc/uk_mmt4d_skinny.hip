@@ -601,18 +601,22 @@ int launch_chunk(const iree_amd_uk_mmt4d_params_t& p, int chunks, int chunk_step
 // The whole linear layer on a few rows: out[M][out_cols] (+)= lhs[M][K] * rhs,
 // lhs and out row-major (`p` describes them as iree_amd_uk_matmul_packed_rhs
 // does: lhs_stride0 and out_stride0 are row pitches in elements), rhs packed
-// 32 x K0 tiles, 1 < M < 32. One launch of the kernel above with the rows of
+// 32 x K0 tiles, 1 < M <= 32. One launch of the kernel above with the rows of
 // the matrix as the rows of its single narrow tile; NOT_FOUND for what that
 // launch cannot take (a K that one launch row cannot hold in registers, too
 // few outer columns to be worth it, operands that are not 16-byte aligned).
 int launch_matmul_rows_skinny(const iree_amd_uk_mmt4d_params_t& p, int64_t M, int64_t out_cols, hipStream_t s) {
-  if (M < 2 || M > 31 || !mmt4d_skinny_supported(p.flags, 16, 32, p.K0)) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  if (M < 2 || M > 32 || !mmt4d_skinny_supported(p.flags, 16, 32, p.K0)) return IREE_AMD_UK_STATUS_NOT_FOUND;
   const int mk = mfma_k_of(p.flags);
   Mmt4dTypeInfo ti;
   mmt4d_type_info(p.flags, &ti);
   const int eb = ti.lhs_bits / 8;
   const int64_t k_elems = p.K * p.K0;
   if (p.K == 0 || k_elems % mk || p.N > 0x7FFFFFFF || out_cols > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  // (measured at N = 14336, K = 4096: 2-byte elements at 31 / 32 rows 29.0 /
+  // 29.7 us against 28.4 for the macro-tile kernel, 26.9 at 24 rows; 1-byte
+  // elements at 32 rows 15.1 (i8) and 16.7 (fp8) against 17.2 and 17.0)
+  if (eb > 1 && M > 24) return IREE_AMD_UK_STATUS_NOT_FOUND;
   const int64_t steps = k_elems / mk;
   // (a K longer than one launch row keeps in registers goes to the macro-tile
   // kernel with its K split, which measures as fast or faster there)

@@ -172,7 +172,7 @@ def test_random_fused_matmul_calls_exact(uk, cuda, seed):
             # a few rows against more than 128 tiles of columns: matmul_packed_rhs runs the
             # kernel for narrow left-hand side tiles on the row-major matrix itself
             # (any K that one launch holds: up to 128 steps of 64 bytes per row)
-            M, N = int(rng.integers(2, 32)), int(rng.integers(4100, 5200))
+            M, N = int(rng.integers(2, 33)), int(rng.integers(4100, 5200))
             steps = int(rng.integers(1, 129))
         K = steps * mfma_k
         acc = bool(rng.integers(0, 2))
