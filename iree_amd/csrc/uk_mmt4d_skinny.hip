@@ -27,6 +27,12 @@
 // Here the kernel runs with the left-hand side streaming and the right-hand
 // side in registers and stores every block transposed, as the 32 x N0 tile the
 // caller asked for.
+//
+// The same kernel also serves the whole linear layer on a few rows
+// (launch_matmul_rows_skinny: what iree_amd_uk_matmul_packed_rhs runs for a
+// decode step): the left-hand side is then the row-major M x K matrix itself,
+// whose rows take the place of the rows of the one narrow tile, and the result
+// is written row by row (template switch kRows).
 #include "uk_common.h"
 
 #include <memory>
