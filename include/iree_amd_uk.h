@@ -191,10 +191,10 @@ IREE_AMD_UK_EXPORT int iree_amd_uk_mmt4d_p(
  * (RESOURCE_EXHAUSTED) and has launched nothing; iree_amd_uk_last_error says how
  * many bytes it needed. Calls that do not split K (most) use no scratch at all;
  * the other users are S8S4S32 at the gfx950 tiles, whose right-hand side is
- * widened to int8 in the same array (one byte per weight, same limit), and the
- * types with a 16-bit left-hand side, whose int8 digit planes and their product
- * go there when they fit (otherwise those run the element-wise kernel, which
- * needs no scratch memory).
+ * widened to int8 in the same array (one byte per weight), and the types with
+ * a 16-bit left-hand side, whose int8 digit planes and their product go there:
+ * each when it fits, otherwise the call runs the element-wise kernel, which
+ * needs no scratch memory (slow, never an error).
  * All calls on one GPU share that GPU's array and nothing in it needs to start
  * at zero (every partial sum is written before it is read), but calls whose
  * kernels overlap on one GPU - two streams, two host threads - race on it:
@@ -394,6 +394,18 @@ IREE_AMD_UK_EXPORT int iree_amd_uk_query_tile_sizes_2d(
     const iree_amd_uk_query_tile_sizes_2d_params_t* params,
     iree_amd_uk_query_tile_sizes_2d_out_params_t* out_params);
 
+/* The whole tile of one matmul from its three sizes at once (INT64_MIN =
+ * dynamic): enumerate_matmul_tiles + choose_matmul_tile with narrow_m / narrow_n
+ * set from the static sizes below the full tile. The three roles of
+ * iree_amd_uk_query_tile_sizes_2d each see one operand, so LHS and RHS queries
+ * of a matmul whose M AND N are both static and below 32 would narrow both
+ * dimensions; a caller that knows all sizes asks here and gets the one
+ * consistent answer (the narrower dimension narrowed, the other full:
+ * REF CPUMaterializeEncodingPass.cpp:296-303). Host-only. */
+IREE_AMD_UK_EXPORT int iree_amd_uk_query_matmul_tile_sizes(
+    uint32_t operation, iree_amd_uk_index_t M, iree_amd_uk_index_t N, iree_amd_uk_index_t K,
+    iree_amd_uk_matmul_tile_t* out_tile);
+
 /*===------------------------------------------------------------------------===
  * Grouped int4-weight dequantising matmul (the dispatch that quantised LLM
  * inference lowers to; there is no reference ukernel for it, the semantics are
@@ -433,7 +445,10 @@ IREE_AMD_UK_EXPORT int iree_amd_uk_query_tile_sizes_2d(
  * REF runtime/src/iree/builtins/ukernel/arch/x86_64/mmt4d_x86_64_avx512_vnni.c:210-294)
  * and out = sum_g float(acc) * scale_x * s - (zp * s) * sum_k x, all float steps
  * in f32, rounded to f16 once. The quantised activations live in the stream's
- * scratch buffer (see iree_amd_uk_mmt4d). On the matrix cores from tiled
+ * scratch buffer (see iree_amd_uk_mmt4d); where that cannot be leased (the
+ * per-thread default stream, another thread's call holding it) the call takes
+ * its own with hipMallocAsync / hipFreeAsync on `stream`, and returns
+ * RESOURCE_EXHAUSTED only when the device has no memory left. On the matrix cores from tiled
  * weights with K = 2048 or 4096 and power-of-two groups of 128 to K / 8;
  * everything else runs an element-wise kernel. */
 #define IREE_AMD_UK_FLAG_DEQUANT_MATMUL_REASSOCIATE 0x4
@@ -685,6 +700,14 @@ IREE_AMD_UK_EXPORT int iree_amd_uk_stream_synchronize(void* stream);
 IREE_AMD_UK_EXPORT int iree_amd_uk_release_scratch(void);
 /* Human-readable text of the calling thread's last non-OK status ("" if none). */
 IREE_AMD_UK_EXPORT const char* iree_amd_uk_last_error(void);
+/* Name of the kernel family that served the calling thread's last mmt4d or
+ * dequant_matmul_i4 call: "mmt4d:mfma", "mmt4d:mfma-narrow",
+ * "mmt4d:mfma-widened-s4", "mmt4d:mfma-s16-planes", "mmt4d:element-wise",
+ * "dequant_i4:mfma", "dequant_i4:gemv", "dequant_i4:reassociated",
+ * "dequant_i4:element-wise" ("" before the first call). A static string. No
+ * counterpart in the reference, whose tile-function choice is visible through
+ * iree_uk_mmt4d_info only. */
+IREE_AMD_UK_EXPORT const char* iree_amd_uk_last_kernel_path(void);
 /* Library version: (major << 16) | minor. */
 IREE_AMD_UK_EXPORT uint32_t iree_amd_uk_version(void);
 

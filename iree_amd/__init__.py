@@ -20,6 +20,7 @@ from .ukernel import (  # noqa: F401
     batch_matmul_packed_rhs,
     choose_matmul_tile,
     enumerate_matmul_tiles,
+    last_kernel_path,
     batch_mmt4d,
     batch_mmt4d_unpack,
     mmt4d,
@@ -30,6 +31,7 @@ from .ukernel import (  # noqa: F401
     pack_i4_weights,
     quantize_f16_to_f8e4m3,
     quantize_pack_f8e4m3,
+    query_matmul_tile_sizes,
     query_tile_sizes_2d,
     scale_f32,
     silu_mul_quantize,

@@ -108,6 +108,8 @@ def _declare(lib):
     lib.iree_amd_uk_choose_matmul_tile.restype = C.c_int
     lib.iree_amd_uk_choose_matmul_tile.argtypes = [C.POINTER(MatmulTile), C.c_int32, i64, i64,
                                                    C.POINTER(C.c_int64), C.POINTER(MatmulTile)]
+    lib.iree_amd_uk_query_matmul_tile_sizes.restype = C.c_int
+    lib.iree_amd_uk_query_matmul_tile_sizes.argtypes = [C.c_uint32, i64, i64, i64, C.POINTER(MatmulTile)]
     lib.iree_amd_uk_query_tile_sizes_2d.restype = C.c_int
     lib.iree_amd_uk_query_tile_sizes_2d.argtypes = [C.POINTER(QueryParams),
                                                      C.POINTER(QueryOutParams)]
@@ -172,6 +174,8 @@ def _declare(lib):
     lib.iree_amd_uk_stream_synchronize.argtypes = [vp]
     lib.iree_amd_uk_release_scratch.restype = C.c_int
     lib.iree_amd_uk_release_scratch.argtypes = []
+    lib.iree_amd_uk_last_kernel_path.restype = C.c_char_p
+    lib.iree_amd_uk_last_kernel_path.argtypes = []
     lib.iree_amd_uk_last_error.restype = C.c_char_p
     lib.iree_amd_uk_last_error.argtypes = []
     lib.iree_amd_uk_version.restype = u32

@@ -19,6 +19,9 @@ int fail(int status, const char* fmt, ...) {
   return status;
 }
 
+static thread_local const char* g_kernel_path = "";
+void note_kernel_path(const char* name) { g_kernel_path = name; }
+
 int check_hip(hipError_t err, const char* what) {
   if (err == hipSuccess) return 0;
   int status = IREE_AMD_UK_STATUS_INTERNAL;
@@ -212,31 +215,36 @@ extern "C" int iree_amd_uk_mmt4d_p(const iree_amd_uk_mmt4d_params_t* params,
   if (!p.rhs_buffer && p.K && p.K0) return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "mmt4d: null rhs");
   if (!p.out_buffer) return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "mmt4d: null out");
   hipStream_t s = (hipStream_t)stream;
+  // (what served the call is recorded for iree_amd_uk_last_kernel_path)
+  auto generic = [&]() {
+    note_kernel_path("mmt4d:element-wise");
+    return launch_mmt4d_generic(p, s);
+  };
   if (mmt4d_skinny_supported(p.flags, p.M0, p.N0, p.K0)) {
     // Narrow left-hand-side tiles (a matrix of fewer than 32 rows): the
     // streaming MFMA kernel, or the element-wise one for what it cannot take.
     int st = launch_mmt4d_skinny(p, s);
-    if (st != IREE_AMD_UK_STATUS_NOT_FOUND) return st;
-    return launch_mmt4d_generic(p, s);
+    if (st != IREE_AMD_UK_STATUS_NOT_FOUND) { note_kernel_path("mmt4d:mfma-narrow"); return st; }
+    return generic();
   }
   if (mmt4d_mfma_supported(p.flags, p.M0, p.N0, p.K0)) {
     int st = launch_mmt4d_mfma(p, s);
-    if (st != IREE_AMD_UK_STATUS_NOT_FOUND) return st;
+    if (st != IREE_AMD_UK_STATUS_NOT_FOUND) { note_kernel_path("mmt4d:mfma"); return st; }
     // A gfx950 tile whose operands the MFMA kernel cannot take (not 16-byte
     // aligned, or a K extent that is not whole MFMA steps): the tile is still
     // an architecture tile, served by the element-wise kernel whether or not
     // the caller allowed the generic fallback.
-    return launch_mmt4d_generic(p, s);
+    return generic();
   }
   if (mmt4d_s8s4_widened_supported(p.flags, p.M0, p.N0, p.K0)) {
     int st = launch_mmt4d_s8s4_widened(p, s);
-    if (st != IREE_AMD_UK_STATUS_NOT_FOUND) return st;
-    return launch_mmt4d_generic(p, s);     // (an architecture tile all the same)
+    if (st != IREE_AMD_UK_STATUS_NOT_FOUND) { note_kernel_path("mmt4d:mfma-widened-s4"); return st; }
+    return generic();     // (an architecture tile all the same)
   }
   if (mmt4d_s16_planes_supported(p.flags, p.M0, p.N0, p.K0)) {
     int st = launch_mmt4d_s16_planes(p, s);
-    if (st != IREE_AMD_UK_STATUS_NOT_FOUND) return st;
-    return launch_mmt4d_generic(p, s);     // (likewise)
+    if (st != IREE_AMD_UK_STATUS_NOT_FOUND) { note_kernel_path("mmt4d:mfma-s16-planes"); return st; }
+    return generic();     // (likewise)
   }
   if (!(p.flags & IREE_AMD_UK_FLAG_MMT4D_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION)) {
     // The reference asserts here (mmt4d.c:128-138); a release build would
@@ -246,7 +254,7 @@ extern "C" int iree_amd_uk_mmt4d_p(const iree_amd_uk_mmt4d_params_t* params,
                 "generic fallback not allowed",
                 p.flags & 0xFF, p.M0, p.N0, p.K0);
   }
-  return launch_mmt4d_generic(p, s);
+  return generic();
 }
 
 extern "C" int iree_amd_uk_mmt4d(
@@ -406,7 +414,9 @@ extern "C" int iree_amd_uk_query_tile_sizes_2d(
       // other dimension's full tile: CPUMaterializeEncodingPass.cpp:296-303).
       const int m0 = narrow(t.M0, params->size0), n0 = narrow(t.N0, params->size1);
       const bool m_narrow = m0 < t.M0, n_narrow = n0 < t.N0;
-      const bool pick_n = n_narrow && (!m_narrow || params->size1 < params->size0);
+      // (an empty dimension counts as one of size 1, as in the three-size query)
+      const int64_t s0 = params->size0 > 0 ? params->size0 : 1, s1 = params->size1 > 0 ? params->size1 : 1;
+      const bool pick_n = n_narrow && (!m_narrow || s1 < s0);
       out_params->tile_size0 = pick_n ? t.M0 : m0;
       out_params->tile_size1 = pick_n ? n0 : t.N0;
       return 0;
@@ -482,6 +492,23 @@ extern "C" int iree_amd_uk_choose_matmul_tile(const iree_amd_uk_matmul_tile_t* t
       return fail(IREE_AMD_UK_STATUS_NOT_FOUND, "choose_matmul_tile: no tile within the upper bound");
   }
   return 0;
+}
+
+extern "C" int iree_amd_uk_query_matmul_tile_sizes(uint32_t operation, iree_amd_uk_index_t M,
+                                                   iree_amd_uk_index_t N, iree_amd_uk_index_t K,
+                                                   iree_amd_uk_matmul_tile_t* out_tile) {
+  (void)K;   // (no gfx950 tile depends on the size of K)
+  if (!out_tile) return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "query_matmul_tile_sizes: null out_tile");
+  iree_amd_uk_matmul_tile_t tiles[8];
+  int32_t count = 0;
+  UK_RETURN_IF_ERROR(iree_amd_uk_enumerate_matmul_tiles(operation, tiles, 8, &count));
+  if (count > 8) count = 8;
+  // A static size below the widest tile marks the matmul as narrow in that
+  // dimension; the chooser then narrows the narrower of the two only.
+  const int64_t full_m = tiles[0].M, full_n = tiles[0].N;
+  const int64_t narrow_m = (M >= 0 && M < full_m) ? (M > 0 ? M : 1) : 0;
+  const int64_t narrow_n = (N >= 0 && N < full_n) ? (N > 0 ? N : 1) : 0;
+  return iree_amd_uk_choose_matmul_tile(tiles, count, narrow_m, narrow_n, nullptr, out_tile);
 }
 
 //===----------------------------------------------------------------------===//
@@ -903,4 +930,5 @@ extern "C" int iree_amd_uk_release_scratch(void) {
   return 0;
 }
 extern "C" const char* iree_amd_uk_last_error(void) { return g_last_error; }
+extern "C" const char* iree_amd_uk_last_kernel_path(void) { return g_kernel_path; }
 extern "C" uint32_t iree_amd_uk_version(void) { return (0u << 16) | 1u; }

@@ -9,6 +9,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "iree_amd_uk.h"
 
 namespace uk {
@@ -16,6 +18,11 @@ namespace uk {
 // Records a message for iree_amd_uk_last_error() on this thread and returns
 // `status`, so call sites read `return fail(STATUS, "...")`.
 int fail(int status, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+
+// Records which kernel family served the calling thread's last call, for
+// iree_amd_uk_last_kernel_path() (a static string; tests and callers that tune
+// use it to tell a matrix-core kernel from the element-wise one).
+void note_kernel_path(const char* name);
 
 // Converts a hipError_t of a runtime call or of a kernel launch to a status.
 int check_hip(hipError_t err, const char* what);
@@ -31,6 +38,23 @@ int check_hip(hipError_t err, const char* what);
     int uk_status_ = (expr);           \
     if (uk_status_) return uk_status_; \
   } while (0)
+
+// One bit per device ordinal on which a kernel's attributes have been set
+// (hipFuncSetAttribute belongs to the kernel on ONE device). Host threads call
+// concurrently: test() / set() are atomic; two threads may both find the bit
+// clear and both make the idempotent call.
+class PerDeviceOnce {
+ public:
+  bool done(int dev) const {
+    return dev >= 0 && dev < 64 && ((bits_.load(std::memory_order_acquire) >> dev) & 1);
+  }
+  void mark(int dev) {
+    if (dev >= 0 && dev < 64) bits_.fetch_or(1ull << dev, std::memory_order_release);
+  }
+
+ private:
+  std::atomic<unsigned long long> bits_{0};
+};
 
 // Element-type facts of an mmt4d type tuple.
 struct Mmt4dTypeInfo {
@@ -129,6 +153,36 @@ class ScratchLease {
   void* ptr_ = nullptr;
   uint64_t id_ = 0;
   bool overflowed_ = false;
+};
+// Scratch memory a call cannot do without: the stream's cached buffer when it
+// can be leased, otherwise an allocation of the call's own, made and freed in
+// stream order on the caller's stream (hipMallocAsync / hipFreeAsync: some
+// tens of microseconds of host time, which is why it is only the fallback).
+// That covers the per-thread default stream, a buffer another thread holds on
+// the same stream, and a full cache. ptr() is nullptr only under a strict
+// override that is too small, or when the device is out of memory.
+class CallScratch {
+ public:
+  CallScratch(hipStream_t s, size_t bytes) : lease_(s, bytes), stream_(s) {
+    if (!lease_.ptr() && !lease_.overflowed() && bytes) {
+      if (hipMallocAsync(&own_, bytes, s) != hipSuccess) {
+        (void)hipGetLastError();
+        own_ = nullptr;
+      }
+    }
+  }
+  ~CallScratch() {
+    if (own_ && hipFreeAsync(own_, stream_) != hipSuccess) (void)hipGetLastError();
+  }
+  CallScratch(const CallScratch&) = delete;
+  CallScratch& operator=(const CallScratch&) = delete;
+  void* ptr() const { return lease_.ptr() ? lease_.ptr() : own_; }
+  bool overflowed() const { return lease_.overflowed(); }
+
+ private:
+  ScratchLease lease_;
+  void* own_ = nullptr;
+  hipStream_t stream_;
 };
 class ScratchOverride {
  public:

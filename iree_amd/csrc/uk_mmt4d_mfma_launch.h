@@ -97,15 +97,15 @@ int launch_form(const MfmaArgs& a, unsigned blocks, hipStream_t s) {
   }
   if (!kernel) return IREE_AMD_UK_STATUS_NOT_FOUND;
   // The attribute belongs to the kernel on ONE device: set it once per device
-  // ordinal (a benign race: the call is idempotent).
-  static unsigned long long attr_set_on[2] = {0, 0};
-  unsigned long long& set_on = attr_set_on[slices > 1];
+  // ordinal.
+  static PerDeviceOnce attr_set_on[2];
+  PerDeviceOnce& set_on = attr_set_on[slices > 1];
   int dev = 0;
   UK_RETURN_IF_HIP(hipGetDevice(&dev));
-  if (dev < 0 || dev >= 64 || !((set_on >> dev) & 1)) {
+  if (!set_on.done(dev)) {
     UK_RETURN_IF_HIP(hipFuncSetAttribute((const void*)kernel,
                                          hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes));
-    if (dev >= 0 && dev < 64) set_on |= 1ull << dev;
+    set_on.mark(dev);
   }
   MfmaArgs b = a;
   b.batch_by_xcd = a.batch >= 8 && blocks <= 64 ? a.batch / 8 * 8 : 0;

@@ -54,7 +54,11 @@ struct SkinnyArgs {
   int64_t rhs_stride_bytes, out_stride_elems;  // per outer column j
   int N;             // outer columns
   int M0;
-  int ksteps;        // MFMA K steps in total
+  int ksteps;        // MFMA K steps in total (the last one partial when tail_tiles > 0)
+  // K tiles in the last step when K is not whole steps (0 = it is): the lanes
+  // (or lane halves) that stand for the missing tiles of that step contribute
+  // zeros on both sides (kTail kernels only)
+  int tail_tiles;
   int steps_per_wave;
   int lhs_tile_bytes;  // M0 * K0 * element size
   int half_k0;
@@ -94,8 +98,12 @@ struct SkinnyArgs {
 // kRows: the row-major forms of left-hand side and result (SkinnyArgs); a
 // compile-time switch so that the tile forms carry none of their address
 // arithmetic (as a run-time one it cost the short-K batch form 16 %).
-template <typename Cfg, int SP, bool kPartialOut = false, bool kPerWave = false, bool kRows = false>
+// kTail: K ends in a partial step (SkinnyArgs::tail_tiles); a kernel of its own so
+// that whole-step calls carry none of its selects.
+template <typename Cfg, int SP, bool kPartialOut = false, bool kPerWave = false, bool kRows = false,
+          bool kTail = false>
 __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
+  static_assert(!(kTail && kRows), "the row-major forms take whole K steps only");
   typedef typename Cfg::frag_t frag_t;
   typedef typename Cfg::acc_t acc_t;
   typedef typename Cfg::out_t out_t;
@@ -127,6 +135,13 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
   const int lane_off = kSub == 2 ? ((lane >> 5) * 1024 + (lane & 31) * 16)
                        : a.half_k0 ? lane * 16 : ((lane & 31) * 32 + (lane >> 5) * 16);
   const char* rhs_lane = a.rhs + (int64_t)(count > 0 ? first : 0) * kBlock + lane_off;
+  // Partial last step: K tile of this lane's piece(s) inside a step (tiles are
+  // 512 bytes of the right-hand side), whether the last step lacks it, and the
+  // step of this wave's slice that is the last one of K (-1: another wave's).
+  const int tile_lo = kSub == 2 ? 2 * (lane >> 5) : (lane >> 5), tile_hi = tile_lo + 1;
+  const bool lo_missing = kTail && tile_lo >= a.tail_tiles, hi_missing = kTail && tile_hi >= a.tail_tiles;
+  const int tail_s = kTail ? a.ksteps - 1 - (count > 0 ? first : 0) : -1;   // (of the blocks this wave loads)
+  const bool owns_tail = tail_s >= 0 && tail_s < count;
   auto make_frag = [](int4v lo, int4v hi) -> frag_t {
     if constexpr (kSub == 2) {
       return frag_t{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
@@ -143,6 +158,16 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
     const int s = sp < count ? sp : 0;
     const int jj = j < a.N ? j : a.N - 1;
     const char* p = rhs_lane + (int64_t)jj * a.rhs_stride_bytes + (int64_t)s * kBlock;
+    if constexpr (kTail) {
+      // (a piece of a missing tile would lie past the end of the row: it is
+      // fetched from the step's first tile instead and zeroed when consumed)
+      const bool last = s == tail_s;
+      const char* p_lo = p - (last && lo_missing ? tile_lo * 512 : 0);
+      const char* p_hi = p + 512 - (last && hi_missing ? tile_hi * 512 : 0);
+      const int4v lo = __builtin_nontemporal_load((const int4v*)p_lo);
+      const int4v hi = kSub == 2 ? __builtin_nontemporal_load((const int4v*)p_hi) : lo;
+      return make_frag(lo, hi);
+    }
     // (non-temporal: the right-hand side is read once)
     const int4v lo = __builtin_nontemporal_load((const int4v*)p);
     const int4v hi = kSub == 2 ? __builtin_nontemporal_load((const int4v*)(p + 512)) : lo;
@@ -152,6 +177,19 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
   // touching the loaded registers earlier would wait for the load)
   auto live = [&](frag_t f, int sp) -> frag_t {
     const int4v zero = {0, 0, 0, 0};
+    if constexpr (kTail) {
+      if (sp == tail_s) {
+        if constexpr (kSub == 2) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            if (lo_missing) f[e] = 0;
+            if (hi_missing) f[4 + e] = 0;
+          }
+        } else {
+          if (lo_missing) f = make_frag(zero, zero);
+        }
+      }
+    }
     return sp >= count ? make_frag(zero, zero) : f;
   };
 
@@ -180,7 +218,8 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
     // for (loads return in order).
     extern __shared__ __attribute__((aligned(16))) char stage_all[];
     char* stage = stage_all + wave * a.stage_wave_bytes;
-    const int slice = count * step_bytes;
+    // (a partial last step ends after its tail_tiles tiles: what lies beyond reads as zeros)
+    const int slice = count * step_bytes - (owns_tail ? step_bytes - a.tail_tiles * a.lhs_tile_bytes : 0);
     // (row-major: the slice of every row, the rows SP steps and 16 bytes apart
     // in LDS so that the 16-byte reads of up to 16 rows touch every bank once;
     // a row's last load may run into the next row's place, which the next
@@ -216,8 +255,11 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
       if (m0 < a.M0 && sp < count) {
         const char* p = rows_lhs ? stage + m0 * row_stage + sp * step_bytes + kh * 16 * kSub
                                  : stage + sp * step_bytes + piece_off;
-        lo = *(const int4v*)p;
-        if constexpr (kSub == 2) hi = *(const int4v*)(p + hi_off);
+        // (LDS past the staged slice holds whatever was there: a missing tile is not read)
+        if (!(sp == tail_s && lo_missing)) lo = *(const int4v*)p;
+        if constexpr (kSub == 2) {
+          if (!(sp == tail_s && hi_missing)) hi = *(const int4v*)(p + hi_off);
+        }
       }
       xf[sp] = make_frag(lo, hi);
     }
@@ -234,8 +276,10 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
       if (m0 < a.M0 && sp < count) {
         const char* p = rows_lhs ? a.lhs + m0 * a.lhs_row_pitch_bytes + (int64_t)s * step_bytes + kh * 16 * kSub
                                  : a.lhs + (int64_t)s * step_bytes + piece_off;
-        lo = *(const int4v*)p;
-        if constexpr (kSub == 2) hi = *(const int4v*)(p + hi_off);
+        if (!(sp == tail_s && lo_missing)) lo = *(const int4v*)p;
+        if constexpr (kSub == 2) {
+          if (!(sp == tail_s && hi_missing)) hi = *(const int4v*)(p + hi_off);
+        }
       }
       xf[sp] = make_frag(lo, hi);
     }
@@ -307,9 +351,12 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
 // One launch of the form that splits K over the waves, with the left-hand side
 // staged through LDS when the slices of the 8 waves fit 64 KiB of it (narrow
 // tiles of up to 8 rows at the longest K a launch takes).
-template <typename Cfg, int SP, bool kPartialOut, bool kRows = false>
+template <typename Cfg, int SP, bool kPartialOut, bool kRows = false, bool kTail = false>
 int launch_split_form(SkinnyArgs a, dim3 grid, hipStream_t s) {
-  void (*kernel)(SkinnyArgs) = mmt4d_skinny_kernel<Cfg, SP, kPartialOut, false, kRows>;
+  if constexpr (!kRows && !kTail) {
+    if (a.tail_tiles) return launch_split_form<Cfg, SP, kPartialOut, false, true>(a, grid, s);
+  }
+  void (*kernel)(SkinnyArgs) = mmt4d_skinny_kernel<Cfg, SP, kPartialOut, false, kRows, kTail>;
   constexpr bool rows_lhs = kRows;
   const int step_bytes = rows_lhs ? 32 * Cfg::kSub : (Cfg::kSub == 2 ? 4 : a.half_k0 ? 2 : 1) * a.lhs_tile_bytes;
   // (row-major: M0 rows of SP steps and 16 bytes, and room for the last load of the last row)
@@ -323,12 +370,12 @@ int launch_split_form(SkinnyArgs a, dim3 grid, hipStream_t s) {
     a.stage_wave_bytes = wave_bytes;
     lds = (size_t)kWaves * wave_bytes;
     // (with the kernel's static partial sums this is more than the default 64 KiB)
-    static unsigned long long attr_set_on = 0;
+    static PerDeviceOnce attr_set_on;
     int dev = 0;
     UK_RETURN_IF_HIP(hipGetDevice(&dev));
-    if (dev < 0 || dev >= 64 || !((attr_set_on >> dev) & 1)) {
+    if (!attr_set_on.done(dev)) {
       UK_RETURN_IF_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kMaxStageBytes));
-      if (dev >= 0 && dev < 64) attr_set_on |= 1ull << dev;
+      attr_set_on.mark(dev);
     }
   }
   hipLaunchKernelGGL(kernel, grid, dim3(kThreads), lds, s, a);
@@ -353,12 +400,20 @@ int launch_cfg(SkinnyArgs a, int chunks, hipStream_t s) {
     a.steps_per_wave = a.chunk_steps;
     a.stage_wave_bytes = 0;
     const dim3 grid(groups < per_plane ? groups : per_plane, 1, a.batch > 1 ? a.batch : 1);
+    void (*kernel)(SkinnyArgs) = nullptr;
     if (a.chunk_steps <= 8) {
-      hipLaunchKernelGGL((mmt4d_skinny_kernel<Cfg, 8, false, true, kRows>), grid, dim3(kThreads), 0, s, a);
-    } else {
-      if constexpr (kPerWaveSteps >= 16)
-        hipLaunchKernelGGL((mmt4d_skinny_kernel<Cfg, 16, false, true, kRows>), grid, dim3(kThreads), 0, s, a);
+      kernel = mmt4d_skinny_kernel<Cfg, 8, false, true, kRows>;
+      if constexpr (!kRows) {
+        if (a.tail_tiles) kernel = mmt4d_skinny_kernel<Cfg, 8, false, true, false, true>;
+      }
+    } else if constexpr (kPerWaveSteps >= 16) {
+      kernel = mmt4d_skinny_kernel<Cfg, 16, false, true, kRows>;
+      if constexpr (!kRows) {
+        if (a.tail_tiles) kernel = mmt4d_skinny_kernel<Cfg, 16, false, true, false, true>;
+      }
     }
+    if (!kernel) return IREE_AMD_UK_STATUS_NOT_FOUND;
+    hipLaunchKernelGGL(kernel, grid, dim3(kThreads), 0, s, a);
     return check_hip(hipGetLastError(), "mmt4d_skinny launch");
   }
   const int blocks = a.N < per_plane ? a.N : per_plane;
@@ -453,9 +508,9 @@ int launch_batch_mmt4d_skinny(const iree_amd_uk_mmt4d_params_t& p0, int64_t batc
   }
   const int mk = mfma_k_of(p.flags);
   const int64_t k_elems = p.K * p.K0;
-  if (p.M != 1 || p.K == 0 || k_elems % mk || p.N > 0x7FFFFFFF || batch > 65535)
+  if (p.M != 1 || p.K == 0 || p.N > 0x7FFFFFFF || batch > 65535)
     return IREE_AMD_UK_STATUS_NOT_FOUND;
-  const int64_t steps = k_elems / mk;
+  const int64_t steps = (k_elems + mk - 1) / mk;   // (the last one may be partial)
   if (steps > max_steps_per_launch(mk)) return IREE_AMD_UK_STATUS_NOT_FOUND;
   const BatchStrides bs = {batch, lhs_batch_stride, rhs_batch_stride, out_batch_stride};
   return launch_chunk(p, 1, (int)steps, nullptr, s, &bs);
@@ -467,8 +522,9 @@ int launch_mmt4d_skinny(const iree_amd_uk_mmt4d_params_t& p0, hipStream_t s) {
   const bool transposed = (p.flags & kTransposedOut) != 0;
   const int mk = mfma_k_of(p.flags);
   const int64_t k_elems = p.K * p.K0;
-  if (p.M != 1 || p.K == 0 || k_elems % mk || p.N > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
-  const int64_t steps = k_elems / mk;
+  if (p.M != 1 || p.K == 0 || p.N > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  // (a K that is not whole steps ends in a partial one)
+  const int64_t steps = (k_elems + mk - 1) / mk;
   if (steps > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
   const int max_steps = max_steps_per_launch(mk);
   Mmt4dTypeInfo ti;
@@ -533,6 +589,7 @@ int launch_mmt4d_skinny(const iree_amd_uk_mmt4d_params_t& p0, hipStream_t s) {
     iree_amd_uk_mmt4d_params_t q = p;
     const int64_t tile0 = first * tiles_per_step_num / tiles_per_step_den;
     q.K = n * tiles_per_step_num / tiles_per_step_den;
+    if (q.K > p.K - tile0) q.K = p.K - tile0;     // (the last slice ends with K)
     q.lhs_offset += tile0 * p.M0 * p.K0;
     q.rhs_offset += tile0 * p.N0 * p.K0;
     if (first > 0) q.flags |= IREE_AMD_UK_FLAG_MMT4D_ACCUMULATE;
@@ -566,7 +623,8 @@ int launch_chunk(const iree_amd_uk_mmt4d_params_t& p, int chunks, int chunk_step
   a.transpose_out = (p.flags & kTransposedOut) != 0;
   a.out_stride_elems = a.transpose_out ? p.out_stride0 : (int64_t)p.M0 * 32;
   a.N = (int)p.N; a.M0 = p.M0;
-  a.ksteps = (int)(k_elems / mk);
+  a.ksteps = (int)((k_elems + mk - 1) / mk);
+  a.tail_tiles = (int)((k_elems % mk) / p.K0);
   a.steps_per_wave = 0;
   a.lhs_tile_bytes = p.M0 * p.K0 * eb;
   a.half_k0 = p.K0 * 2 == mk;
@@ -654,6 +712,7 @@ int launch_matmul_rows_skinny(const iree_amd_uk_mmt4d_params_t& p, int64_t M, in
   a.out_stride_elems = 0;
   a.N = (int)p.N; a.M0 = (int)M;
   a.ksteps = (int)steps;
+  a.tail_tiles = 0;
   a.steps_per_wave = 0;
   a.lhs_tile_bytes = 0;
   a.half_k0 = p.K0 * 2 == mk;

@@ -107,13 +107,13 @@ int launch_instance(const I4Args& a, int blocks, int k_rows, hipStream_t s) {
   const size_t lds = MH == 1 ? (size_t)kWaves * a.stage_rows * stage_row_bytes<KB>() : kAttrLds;
   {
     // (with the 16-row form's static 32 KiB this is more than the 64 KiB a kernel gets by default)
-    static unsigned long long attr_set_on = 0;
+    static PerDeviceOnce attr_set_on;
     int dev = 0;
     UK_RETURN_IF_HIP(hipGetDevice(&dev));
-    if (dev < 0 || dev >= 64 || !((attr_set_on >> dev) & 1)) {
+    if (!attr_set_on.done(dev)) {
       UK_RETURN_IF_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                                            (int)kAttrLds));
-      if (dev >= 0 && dev < 64) attr_set_on |= 1ull << dev;
+      attr_set_on.mark(dev);
     }
   }
   hipLaunchKernelGGL(kernel, dim3(blocks, k_rows), dim3(kThreads), lds, s, a);
@@ -234,7 +234,7 @@ int launch_dequant_matmul_i4(const void* x, const void* w, const void* scale, co
   if (k_ok && gs_ok && size_ok && aligned && !one_row_few_tiles) {
     a.w_bytes = (uint32_t)w_bytes;
     const int st = slice_kb == 4 ? launch_fast<4>(a, (int)k_rows, s) : launch_fast<8>(a, (int)k_rows, s);
-    if (st != IREE_AMD_UK_STATUS_NOT_FOUND) return st;
+    if (st != IREE_AMD_UK_STATUS_NOT_FOUND) { note_kernel_path("dequant_i4:mfma"); return st; }
   }
   if (gs_pow2 && size_ok && aligned && K > 0) {
     // Other K (whole 2048s): the per-wave-column kernel. It has a longer
@@ -258,18 +258,19 @@ int launch_dequant_matmul_i4(const void* x, const void* w, const void* scale, co
         st = launch_dequant_gemv_i4(a, (int)m0, (int)(M - m0 < rows ? M - m0 : rows), s);
         if (st) break;     // NOT_FOUND can only come from the first pass: nothing has run yet
       }
-      if (st != IREE_AMD_UK_STATUS_NOT_FOUND) return st;
+      if (st != IREE_AMD_UK_STATUS_NOT_FOUND) { note_kernel_path("dequant_i4:gemv"); return st; }
     }
   }
   if (one_row_few_tiles && k_ok && gs_ok && size_ok && aligned) {
     a.w_bytes = (uint32_t)w_bytes;
     const int st = slice_kb == 4 ? launch_fast<4>(a, (int)k_rows, s) : launch_fast<8>(a, (int)k_rows, s);
-    if (st != IREE_AMD_UK_STATUS_NOT_FOUND) return st;
+    if (st != IREE_AMD_UK_STATUS_NOT_FOUND) { note_kernel_path("dequant_i4:mfma"); return st; }
   }
   const int64_t total = M * N;
   int64_t blocks = ceil_div(total, 256);
   const int64_t max_blocks = (int64_t)device_cu_count() * 32;
   if (blocks > max_blocks) blocks = max_blocks;
+  note_kernel_path("dequant_i4:element-wise");
   hipLaunchKernelGGL(dequant_matmul_i4_generic_kernel, dim3((unsigned)blocks), dim3(256), 0, s, a,
                      (int)group_size);
   return check_hip(hipGetLastError(), "dequant_matmul_i4_generic launch");

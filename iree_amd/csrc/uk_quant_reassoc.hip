@@ -324,12 +324,12 @@ int launch_instance(const I4Args& a, const ReassocArgs& r, int blocks, hipStream
   const size_t lds = (size_t)a.G * 32 * 2 * sizeof(float) + (size_t)2 * kWaves * 8 * MH * 64 * sizeof(float);
   void (*kernel)(I4Args, ReassocArgs) = dequant_matmul_i4_reassoc_kernel<KB, MH, kZpU4, kLog2Gs>;
   if (lds > 64 * 1024) {
-    static unsigned long long attr_set_on = 0;
+    static PerDeviceOnce attr_set_on;
     int dev = 0;
     UK_RETURN_IF_HIP(hipGetDevice(&dev));
-    if (dev < 0 || dev >= 64 || !((attr_set_on >> dev) & 1)) {
+    if (!attr_set_on.done(dev)) {
       UK_RETURN_IF_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-      if (dev >= 0 && dev < 64) attr_set_on |= 1ull << dev;
+      attr_set_on.mark(dev);
     }
   }
   hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kThreads), lds, s, a, r);
@@ -399,8 +399,11 @@ int launch_dequant_matmul_i4_reassoc(const void* x, const void* w, const void* s
     const int spans = (int)(K / 128);
     const size_t plane_bytes = (size_t)2 * spans * 4 * 64 * 16;          // 2 row halves, both digits
     const size_t table_bytes = (size_t)a.G * 32 * sizeof(float);
-    ScratchLease lease(s, plane_bytes + 2 * table_bytes);
+    // (held until the last kernel that reads it has been queued)
+    CallScratch lease(s, plane_bytes + 2 * table_bytes);
+    if (lease.overflowed()) return scratch_overflow_status("dequant_matmul_i4: the quantised activations", plane_bytes + 2 * table_bytes);
     if (!lease.ptr()) return fail(8 /* RESOURCE_EXHAUSTED */, "dequant_matmul_i4: no scratch memory for the quantised activations");
+    note_kernel_path("dequant_i4:reassociated");
     for (int m_base = 0; m_base < a.M; m_base += 32) {
       const int rows = a.M - m_base < 32 ? a.M - m_base : 32;
       ReassocArgs r = {};
@@ -435,8 +438,10 @@ int launch_dequant_matmul_i4_reassoc(const void* x, const void* w, const void* s
   if (pass_rows > M) pass_rows = M;
   const size_t q_bytes = ((size_t)pass_rows * K * 2 + 15) & ~(size_t)15;
   const size_t t_bytes = (size_t)pass_rows * a.G * sizeof(float);
-  ScratchLease lease(s, q_bytes + 2 * t_bytes);
+  CallScratch lease(s, q_bytes + 2 * t_bytes);
+  if (lease.overflowed()) return scratch_overflow_status("dequant_matmul_i4: the quantised activations", q_bytes + 2 * t_bytes);
   if (!lease.ptr()) return fail(8 /* RESOURCE_EXHAUSTED */, "dequant_matmul_i4: no scratch memory for the quantised activations");
+  note_kernel_path("dequant_i4:reassociated-element-wise");
   ReassocArgs r = {};
   r.q_plain = (int16_t*)lease.ptr();
   r.scale_plain = (float*)((char*)lease.ptr() + q_bytes);

@@ -49,7 +49,7 @@ class ScratchCache {
   Lease acquire(int device, void* stream, size_t bytes) {
     Lease none;
     if (bytes == 0 || bytes > max_bytes_) return none;
-    std::lock_guard<std::mutex> lock(mutex_);
+    std::unique_lock<std::mutex> lock(mutex_);
     for (Entry& e : entries_) {
       if (e.device != device || e.stream != stream) continue;
       if (e.bytes < bytes) {
@@ -63,20 +63,36 @@ class ScratchCache {
       }
       return lease_of(e);
     }
+    // A new entry. When the table is full the least recently used idle buffer
+    // makes room; it leaves the table here and is freed (a free that waits for
+    // the device) only after the lock has been dropped, so that other threads'
+    // calls do not queue behind that wait.
+    void* evicted = nullptr;
     if (entries_.size() >= max_entries_) {
       size_t victim = entries_.size();
       for (size_t i = 0; i < entries_.size(); ++i)
         if (entries_[i].leases == 0 && (victim == entries_.size() || entries_[i].last_use < entries_[victim].last_use))
           victim = i;
       if (victim == entries_.size()) return none;   // every buffer is in use
-      allocator_.free_now(entries_[victim].ptr, allocator_.user);
+      evicted = entries_[victim].ptr;
       entries_.erase(entries_.begin() + (long)victim);
     }
     const size_t want = bytes < min_bytes_ ? min_bytes_ : bytes;
     void* ptr = allocator_.alloc(want, allocator_.user);
-    if (!ptr) return none;
-    entries_.push_back(Entry{device, stream, ptr, want, 0, 0, next_id_++});
-    return lease_of(entries_.back());
+    if (!ptr && evicted) {
+      // (out of memory with the victim still allocated: free it first after all)
+      allocator_.free_now(evicted, allocator_.user);
+      evicted = nullptr;
+      ptr = allocator_.alloc(want, allocator_.user);
+    }
+    Lease lease;
+    if (ptr) {
+      entries_.push_back(Entry{device, stream, ptr, want, 0, 0, next_id_++});
+      lease = lease_of(entries_.back());
+    }
+    lock.unlock();
+    if (evicted) allocator_.free_now(evicted, allocator_.user);
+    return lease;
   }
 
   void release(const Lease& lease) {
@@ -91,18 +107,21 @@ class ScratchCache {
 
   // Frees every buffer without a lease; returns how many were freed.
   size_t release_idle() {
-    std::lock_guard<std::mutex> lock(mutex_);
-    size_t freed = 0;
-    for (size_t i = 0; i < entries_.size();) {
-      if (entries_[i].leases == 0) {
-        allocator_.free_now(entries_[i].ptr, allocator_.user);
-        entries_.erase(entries_.begin() + (long)i);
-        ++freed;
-      } else {
-        ++i;
+    std::vector<void*> idle;
+    {
+      std::lock_guard<std::mutex> lock(mutex_);
+      for (size_t i = 0; i < entries_.size();) {
+        if (entries_[i].leases == 0) {
+          idle.push_back(entries_[i].ptr);
+          entries_.erase(entries_.begin() + (long)i);
+        } else {
+          ++i;
+        }
       }
     }
-    return freed;
+    // (freed outside the lock: each free waits for the device)
+    for (void* p : idle) allocator_.free_now(p, allocator_.user);
+    return idle.size();
   }
 
   size_t entry_count() {

@@ -62,3 +62,43 @@ def small_int_f16(seed, n, lo=-8, hi=8):
     """Small integers as f16: products and partial sums stay exact."""
     r = (splitmix64(seed, n) >> np.uint64(40)).astype(np.int64)
     return (lo + r % (hi - lo)).astype(np.float16)
+
+
+# ---------------------------------------------------------------------------
+# The operand generator of the reference's end-to-end matmul tests
+# (tools/testing/e2e/test_utils.c:260-267, constants test_utils.h:99-100, used
+# as tools/testing/e2e/iree-e2e-matmul-test.cc:641-660 does): a Lehmer step
+# whose product is taken in 32-bit unsigned arithmetic, i.e. it wraps before
+# the reduction modulo 2^31 - 1, then value = state % range + min.
+# ---------------------------------------------------------------------------
+
+# [min, max] per element type (tools/testing/e2e/test_utils.c:269-319).
+E2E_RANGE = {"i8": (-2, 2), "i32": (-8, 8), "f16": (-4, 4), "bf16": (-2, 2), "f32": (-8, 8)}
+
+
+def e2e_pseudorandom_ints(seed, n, lo, hi):
+    """The n integers in [lo, hi] the reference's test runner draws from `seed`."""
+    out = np.empty(n, dtype=np.int32)
+    state, span = int(seed), hi - lo + 1
+    for i in range(n):
+        state = ((state * 48271) & 0xFFFFFFFF) % 2147483647
+        out[i] = state % span + lo
+    return out
+
+
+def e2e_matrix(seed, n, elem):
+    """n elements of type `elem` ("i8", "i32", "f16", "bf16", "f32") as the
+    reference's generate_random_matrix fills them: small integers, converted
+    exactly (bf16 as its 16 bits in a uint16 array)."""
+    lo, hi = E2E_RANGE[elem]
+    v = e2e_pseudorandom_ints(seed, n, lo, hi)
+    if elem == "i8":
+        return v.astype(np.int8)
+    if elem == "i32":
+        return v
+    if elem == "f16":
+        return v.astype(np.float16)
+    if elem == "f32":
+        return v.astype(np.float32)
+    # bf16: the high half of the f32 (small integers have no low bits)
+    return (v.astype(np.float32).view(np.uint32) >> np.uint32(16)).astype(np.uint16)

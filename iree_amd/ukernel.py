@@ -28,6 +28,12 @@ def _check(status):
         raise UkError(status, msg.decode() if msg else "")
 
 
+def last_kernel_path():
+    """Name of the kernel family that served this thread's last mmt4d or
+    dequant_matmul_i4 call (see include/iree_amd_uk.h)."""
+    return load_library().iree_amd_uk_last_kernel_path().decode()
+
+
 def _ptr(t):
     # (plain ints: the declared argtypes convert them, which is cheaper than
     # building a c_void_p per argument)
@@ -164,6 +170,16 @@ def choose_matmul_tile(tiles, narrow_m=0, narrow_n=0, upper_bound=None):
     ub = (C.c_int64 * 3)(*upper_bound) if upper_bound is not None else None
     out = MatmulTile()
     _check(load_library().iree_amd_uk_choose_matmul_tile(arr, len(tiles), narrow_m, narrow_n, ub, C.byref(out)))
+    return out.M, out.N, out.K
+
+
+def query_matmul_tile_sizes(operation, M=_INT64_MIN, N=_INT64_MIN, K=_INT64_MIN):
+    """The (M0, N0, K0) tile of one matmul from its three sizes at once
+    (``_INT64_MIN`` = dynamic): at most one of M0 and N0 is narrowed, the one of
+    the smaller static size (the reference's chooseMatmulTile,
+    CPUMaterializeEncodingPass.cpp:296-303)."""
+    out = MatmulTile()
+    _check(load_library().iree_amd_uk_query_matmul_tile_sizes(operation, M, N, K, C.byref(out)))
     return out.M, out.N, out.K
 
 
@@ -392,14 +408,16 @@ def matmul_data_tiled(a, b, c, M, N, K, mmt4d_type, *, accumulate=False,
 
     ``a``/``b``/``c`` are flat CUDA tensors holding the row-major matrices with
     the element types of ``mmt4d_type``. ``tile`` = (M0, N0, K0); by default the
-    tile the library's query_tile_sizes_2d reports for gfx950. ``workspace`` may
+    tile the library's query_matmul_tile_sizes reports for these static sizes
+    (narrow for M or N below 32), with ``"dynamic"`` the one for unknown sizes. ``workspace`` may
     carry pre-allocated packed buffers as a dict {"lhs","rhs","out"}.
     Returns the dict of packed buffers used (so callers can reuse them).
     """
     if tile is None:
-        op = _MMT4D_TO_QUERY_OP[mmt4d_type]
-        M0, K0 = query_tile_sizes_2d(op | F.QUERY_ROLE_LHS, M, K)
-        N0, _ = query_tile_sizes_2d(op | F.QUERY_ROLE_RHS, N, K)
+        M0, N0, K0 = query_matmul_tile_sizes(_MMT4D_TO_QUERY_OP[mmt4d_type], M, N, K)
+    elif tile == "dynamic":
+        # (the tile of a matmul whose sizes the compiler did not know)
+        M0, N0, K0 = query_matmul_tile_sizes(_MMT4D_TO_QUERY_OP[mmt4d_type])
     else:
         M0, N0, K0 = tile
     M1, N1, K1 = _ceil_div(M, M0), _ceil_div(N, N0), _ceil_div(K, K0)

@@ -9,8 +9,9 @@
  * How each function is pinned (tests/test_oracle_*.py):
  *   oracle_mmt4d (all integer types)   - against the reference library itself
  *       (oracle/_ref, generic and AVX-512/VNNI tile functions) on the
- *       reference's own shape/tile matrix with its minstd generator; against a
- *       numpy int64 einsum; tile-shape invariance of the row-major result.
+ *       reference's own shape/tile matrix, operands drawn with numpy
+ *       generators over the reference's value ranges; against a numpy int64
+ *       einsum; tile-shape invariance of the row-major result.
  *   oracle_mmt4d (float types)         - same, bit-exact, with the reference's
  *       small-integer value distributions (every partial sum exact); the
  *       no-skip-rounding f16/bf16 variants against oracle/_ref bit-exactly on
@@ -36,6 +37,11 @@
  *       the whole against oracle_dequant_matmul_i4 on inputs the 16-bit
  *       quantisation represents exactly.
  *   oracle_silu_mul                    - libm identity x*sigmoid(x)*u.
+ *   oracle_e2e_reference_matmul        - exact int64 products in numpy on the
+ *       test runner's small-integer operands (every f32 partial sum exact, so
+ *       the order of the additions cannot matter), rounded once by numpy.
+ *   oracle_e2e_pseudorandom_fill       - a big-integer restatement in Python
+ *       and the stream's first values worked out by hand.
  */
 #include "oracle.h"
 
@@ -630,6 +636,71 @@ int oracle_matmul_rowmajor(const void* a, const void* b, void* c, int64_t M,
     return 0;
   }
   return IREE_AMD_UK_STATUS_UNIMPLEMENTED;
+}
+
+/* The reference matmul of the reference's end-to-end test runner: float
+ * accumulation in f32 in k order starting from the accumulator operand (or 0),
+ * the narrow result types rounded once at the end; i8 accumulates in i32. */
+int oracle_e2e_reference_matmul(const void* a, const void* b, const void* acc,
+                                void* c, int64_t M, int64_t N, int64_t K,
+                                uint32_t flags) {
+  const uint32_t type = flags & IREE_AMD_UK_FLAG_MMT4D_TYPE_MASK;
+  if (type == IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32) {
+    const int8_t* A = a;
+    const int8_t* B = b;
+    const int32_t* ACC = acc;
+    int32_t* C = c;
+#pragma omp parallel for
+    for (int64_t m = 0; m < M; ++m)
+      for (int64_t n = 0; n < N; ++n) {
+        uint32_t sum = ACC ? (uint32_t)ACC[m * N + n] : 0u;
+        for (int64_t k = 0; k < K; ++k)
+          sum += (uint32_t)((int32_t)A[m * K + k] * (int32_t)B[k * N + n]);
+        C[m * N + n] = (int32_t)sum;
+      }
+    return 0;
+  }
+  const int out_f16 = type == IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F16;
+  const int out_bf16 = type == IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16BF16;
+  if (!(out_f16 || out_bf16 || type == IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F32 ||
+        type == IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16F32 ||
+        type == IREE_AMD_UK_FLAG_MMT4D_TYPE_F32F32F32))
+    return IREE_AMD_UK_STATUS_UNIMPLEMENTED;
+#pragma omp parallel for
+  for (int64_t m = 0; m < M; ++m)
+    for (int64_t n = 0; n < N; ++n) {
+      const int64_t o = m * N + n;
+      float sum = 0.f;
+      if (acc) {
+        if (out_f16) sum = oracle_f16_to_f32(((const uint16_t*)acc)[o], ORACLE_F16_IEEE);
+        else if (out_bf16) sum = oracle_bf16_to_f32(((const uint16_t*)acc)[o]);
+        else sum = ((const float*)acc)[o];
+      }
+      for (int64_t k = 0; k < K; ++k) {
+        /* (volatile: one rounding per multiply and per add, no contraction) */
+        volatile float prod = load_flt(a, m * K + k, type, ORACLE_F16_IEEE) *
+                              load_flt(b, k * N + n, type, ORACLE_F16_IEEE);
+        sum += prod;
+      }
+      if (out_f16) ((uint16_t*)c)[o] = oracle_f32_to_f16(sum);
+      else if (out_bf16) ((uint16_t*)c)[o] = oracle_f32_to_bf16(sum);
+      else ((float*)c)[o] = sum;
+    }
+  return 0;
+}
+
+/* The pseudorandom stream of the reference's test tools: a Lehmer step whose
+ * product is taken in 32-bit unsigned arithmetic (so it wraps before the
+ * reduction), then value = state % range + min. Returns the final state. */
+uint32_t oracle_e2e_pseudorandom_fill(uint32_t seed, int64_t n, int32_t min,
+                                      int32_t max, int32_t* out) {
+  uint32_t state = seed;
+  const uint32_t range = (uint32_t)(max - min + 1);
+  for (int64_t i = 0; i < n; ++i) {
+    state = (uint32_t)(state * 48271u) % 2147483647u;
+    out[i] = (int32_t)(state % range) + min;
+  }
+  return state;
 }
 
 int oracle_dequant_matmul_i4(const uint16_t* x, const uint8_t* w,

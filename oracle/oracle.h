@@ -67,6 +67,21 @@ uint8_t oracle_f32_to_f8e4m3(float v, int ieee, int saturate);
 int oracle_matmul_rowmajor(const void* a, const void* b, void* c, int64_t M,
                            int64_t N, int64_t K, uint32_t flags);
 
+/* REF tools/testing/e2e/iree-e2e-matmul-test.cc:28-149 (reference_matmul_*):
+ * row-major C[M][N] = (acc ? acc : 0) + A[M][K] * B[K][N]; floats accumulate in
+ * f32 in k order, f16 / bf16 results are rounded once at the end; `acc` may be
+ * NULL and has the result's element type. type = mmt4d type flag value
+ * (S8S8S32, F32F32F32, F16F16F32, F16F16F16, BF16BF16F32, BF16BF16BF16). */
+int oracle_e2e_reference_matmul(const void* a, const void* b, const void* acc,
+                                void* c, int64_t M, int64_t N, int64_t K,
+                                uint32_t flags);
+
+/* REF tools/testing/e2e/test_utils.c:260-267 with the constants of
+ * test_utils.h:99-100, used as iree-e2e-matmul-test.cc:641-660 does: n values
+ * state % (max - min + 1) + min of the stream seeded with `seed`. */
+uint32_t oracle_e2e_pseudorandom_fill(uint32_t seed, int64_t n, int32_t min,
+                                      int32_t max, int32_t* out);
+
 /* REF compiler/src/iree/compiler/GlobalOptimization/FuseDequantizationMatmul.cpp:53-159
  * and GlobalOptimization/test/fuse_dequantization_matmul.mlir:127-158: grouped
  * int4 dequant + matmul, evaluated in double, rounded once to f16. zp_is_u4

@@ -228,6 +228,36 @@ def test_enumerated_tiles_and_the_chooser_follow_the_reference():
             assert q(op | F.QUERY_ROLE_RHS, n if N0 < 32 else -2 ** 63, 4096) == (N0, K0)
 
 
+def test_query_matmul_tile_sizes_gives_one_consistent_tile():
+    """The three-size query: the chooser on the enumerated tiles with the
+    static sizes below 32 as narrow sizes, so at most one of M0 / N0 is
+    narrowed whatever the caller passes, it agrees with the RESULT role, and
+    every answer has a matrix-core kernel."""
+    have = F.MMT4D_INFO_HAVE_ARCHITECTURE_SPECIFIC_TILE_FUNCTION
+    dyn = -2 ** 63
+    qm, q, ch = iree_amd.query_matmul_tile_sizes, iree_amd.query_tile_sizes_2d, iree_amd.choose_matmul_tile
+    assert qm(F.QUERY_OP_MATMUL_F16F16F32, 4, 8, 4096) == (4, 32, 8)     # the wider of two narrow sizes stays full
+    assert qm(F.QUERY_OP_MATMUL_F16F16F32, 8, 4, 4096) == (32, 4, 8)
+    assert qm(F.QUERY_OP_MATMUL_I8I8I32, 1000, 1, 1000) == (32, 1, 16)
+    assert qm(F.QUERY_OP_MATMUL_I8I8I32, 1, 1000, 1000) == (1, 32, 16)
+    assert qm(F.QUERY_OP_MATMUL_F32F32F32) == (32, 32, 4)
+    assert qm(F.QUERY_OP_MATMUL_F32F32F32, 9, dyn, dyn) == (16, 32, 4)
+    for op, type_flag in [(F.QUERY_OP_MATMUL_I8I8I32, F.MMT4D_TYPE_S8S8S32),
+                          (F.QUERY_OP_MATMUL_F16F16F16, F.MMT4D_TYPE_F16F16F16),
+                          (F.QUERY_OP_MATMUL_BF16BF16F32, F.MMT4D_TYPE_BF16BF16F32),
+                          (F.QUERY_OP_MATMUL_F32F32F32, F.MMT4D_TYPE_F32F32F32)]:
+        tiles = iree_amd.enumerate_matmul_tiles(op)
+        for m in (dyn, 0, 1, 2, 3, 9, 10, 15, 16, 31, 32, 81, 1000):
+            for n in (dyn, 0, 1, 3, 7, 10, 16, 19, 32, 41, 1000):
+                M0, N0, K0 = qm(op, m, n, 64)
+                assert (M0, N0, K0) == ch(tiles, max(m, 1) if -1 < m < 32 else 0, max(n, 1) if -1 < n < 32 else 0)
+                assert (M0, N0) == q(op | F.QUERY_ROLE_RESULT, m, n)
+                assert M0 == 32 or N0 == 32
+                assert iree_amd.mmt4d_info(M0, N0, K0, type_flag | F.MMT4D_SKIP_INTERMEDIATE_ROUNDINGS) == have
+    with pytest.raises(iree_amd.UkError):
+        qm(0x7F00, 1, 1, 1)
+
+
 def test_every_tile_the_query_returns_has_an_architecture_kernel():
     """mmt4d_info reports a matrix-core kernel for each tile
     query_tile_sizes_2d can hand out: full tiles, narrow M0 (static M < 32) and

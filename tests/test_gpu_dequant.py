@@ -180,7 +180,7 @@ def test_quantize_groups_i16_equals_the_oracle(uk, cuda):
         assert np.all(np.abs(sm.cpu().numpy().astype(np.float64) - gs0) <= 1e-6 * xf + 1e-12)
 
 
-def run_reassoc_case(uk, M, N, K, gs, zp_u4, tiled, seed=0):
+def run_reassoc_case(uk, M, N, K, gs, zp_u4, tiled, seed=0, stream=None):
     import torch
     G = K // gs
     x = synth.normal_f16(seed + 1, M * K)
@@ -207,7 +207,7 @@ def run_reassoc_case(uk, M, N, K, gs, zp_u4, tiled, seed=0):
     out = torch.full((M * N,), 0x7E00, dtype=torch.int16, device="cuda")
     uk.dequant_matmul_i4(torch.from_numpy(x.view(np.int16)).cuda(), torch.from_numpy(wd).cuda(),
                          torch.from_numpy(s.view(np.int16)).cuda(),
-                         torch.from_numpy(zp.view(np.uint8)).cuda(), out, M, N, K, gs, flags)
+                         torch.from_numpy(zp.view(np.uint8)).cuda(), out, M, N, K, gs, flags, stream=stream)
     torch.cuda.synchronize()
     got = out.cpu().numpy().view(np.float16).astype(np.float64)
     wantf = want.view(np.float16).astype(np.float64)
@@ -244,6 +244,24 @@ def test_reassociated_decode_shape_llama_ffn(uk, cuda, M):
     """The decode configuration through the reassociated form on the matrix
     cores (tiled weights, groups of 128, packed uint4 zero points)."""
     run_reassoc_case(uk, M, 14336, 4096, 128, True, True, seed=50 + M)
+
+
+class _PerThreadStream:
+    """hipStreamPerThread, the handle ((hipStream_t)2) as a stream object."""
+    cuda_stream = 2
+
+
+@pytest.mark.parametrize("M,N,K,gs,tiled", [(8, 256, 4096, 128, True), (3, 40, 384, 64, False)])
+def test_reassociated_on_the_per_thread_default_stream(uk, cuda, M, N, K, gs, tiled):
+    """The library keys its cached scratch buffers by stream and never leases
+    one for the per-thread default stream (one handle, a different stream in
+    every host thread). The reassociated form cannot run without scratch
+    memory: there it takes a buffer of its own in stream order and gives the
+    same result (matrix-core and element-wise kernels)."""
+    import torch
+    torch.cuda.synchronize()
+    run_reassoc_case(uk, M, N, K, gs, True, tiled, seed=900 + M, stream=_PerThreadStream())
+    assert uk.last_kernel_path() == ("dequant_i4:reassociated" if tiled else "dequant_i4:reassociated-element-wise")
 
 
 @pytest.mark.parametrize("M,N,K,gs,zp_u4,tiled", [

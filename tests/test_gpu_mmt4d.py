@@ -200,9 +200,9 @@ def test_narrow_lhs_tiles_bit_exact(uk, cuda, type_flag, K0):
     the tile-size query hands out for a static M below 32) run the streaming
     MFMA kernel: K step counts that fill 8, 16 and 32 register slots per wave,
     ragged splits over the 8 waves, more outer columns than compute units,
-    accumulate, long K. Calls that kernel does not take (two outer rows, an odd
-    K tile count, unaligned operands) must give the same bits through the
-    element-wise kernel."""
+    accumulate, long K. Calls that kernel does not take (two outer rows,
+    unaligned operands) must give the same bits through the element-wise
+    kernel."""
     rng = np.random.default_rng(7000 + type_flag + K0)
     mfma_k = {F.MMT4D_TYPE_S8S8S32: 32, F.MMT4D_TYPE_F32F32F32: 8,
               F.MMT4D_TYPE_F8E4M3F8E4M3F32: 64}.get(type_flag, 16)
@@ -231,6 +231,43 @@ def test_narrow_lhs_tiles_bit_exact(uk, cuda, type_flag, K0):
         case = ukref.Mmt4dCase(rng, type_flag, M, N, K, 8, 32, K0, accumulate=True,
                                loose_strides=True, offsets=True)
         assert np.array_equal(gpucase.run_mmt4d(case), case.run_oracle(ukref.F16_IEEE)), (M, N, K)
+
+
+@pytest.mark.parametrize("type_flag,K0", [(F.MMT4D_TYPE_F16F16F32, 8), (F.MMT4D_TYPE_BF16BF16F32, 8),
+                                          (F.MMT4D_TYPE_S8S8S32, 16), (F.MMT4D_TYPE_F32F32F32, 4),
+                                          (F.MMT4D_TYPE_F16F16F16, 8), (F.MMT4D_TYPE_BF16BF16BF16, 8),
+                                          (F.MMT4D_TYPE_F8E4M3F8E4M3F32, 16)])
+def test_narrow_tiles_with_a_k_that_is_not_whole_instruction_steps(uk, cuda, type_flag, K0):
+    """A packed K is whole tiles of K0, not whole matrix-core steps (two tiles of
+    the queried K0 per step, four for fp8): K = 1000 f16 elements are 125
+    tiles. The narrow-tile kernel ends such a K with a partial step whose
+    missing tiles count as zeros on both sides; nothing may be read past the
+    operands' ends (the right-hand side buffer ends with its last tile). Every
+    tail length, in the one-column-per-wave form, the form that splits K over
+    the waves (staged and direct left-hand sides), the K split over workgroup
+    rows and the narrow right-hand side form; matrix-core kernel asserted."""
+    rng = np.random.default_rng(7300 + type_flag)
+    mfma_k = {F.MMT4D_TYPE_S8S8S32: 32, F.MMT4D_TYPE_F32F32F32: 8,
+              F.MMT4D_TYPE_F8E4M3F8E4M3F32: 64}.get(type_flag, 16)
+    tps = mfma_k // K0
+    no_fallback = ~F.MMT4D_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION
+    for tail in range(1, tps):
+        for M0, N, steps, acc in ((1, 1, 0, False), (1, 1, 0, True), (4, 7, 0, True), (8, 5, 3, False),
+                                  (1, 32, 62, True), (16, 3, 70, False), (2, 2300, 5, True),
+                                  (1, 9, 896, False), (16, 40, 600, True), (4, 300, 13, False)):
+            K = steps * tps + tail
+            case = ukref.Mmt4dCase(rng, type_flag, 1, N, K, M0, 32, K0, accumulate=acc)
+            got = gpucase.run_mmt4d(case, flags=case.flags & no_fallback)
+            assert uk.last_kernel_path() == "mmt4d:mfma-narrow", (hex(type_flag), M0, N, K)
+            assert np.array_equal(got.view(np.uint8), case.run_oracle(ukref.F16_IEEE).view(np.uint8)), \
+                (hex(type_flag), M0, N, K, acc)
+        for N0, M, steps, acc in ((1, 1, 0, False), (1, 1000 // 32 + 1, 62, True), (8, 3, 70, False), (2, 40, 300, True)):
+            K = steps * tps + tail
+            case = ukref.Mmt4dCase(rng, type_flag, M, 1, K, 32, N0, K0, accumulate=acc)
+            got = gpucase.run_mmt4d(case, flags=case.flags & no_fallback)
+            assert uk.last_kernel_path() == "mmt4d:mfma-narrow", (hex(type_flag), N0, M, K)
+            assert np.array_equal(got.view(np.uint8), case.run_oracle(ukref.F16_IEEE).view(np.uint8)), \
+                (hex(type_flag), N0, M, K, acc)
 
 
 @pytest.mark.parametrize("type_flag,K0", [(F.MMT4D_TYPE_F16F16F32, 8), (F.MMT4D_TYPE_F16F16F32, 16),

@@ -140,3 +140,33 @@ def test_noalloc_mmt4d_with_16_bit_operands(uk, cuda):
             assert torch.cuda.mem_get_info()[0] == free_before, "the call changed the free device memory"
             assert np.array_equal(got, want), (hex(type_flag), M, N, K)
             assert np.array_equal(got, case.run_oracle()), (hex(type_flag), M, N, K)
+
+
+def test_noalloc_mmt4d_with_a_4_bit_right_hand_side(uk, cuda):
+    """S8S4S32 at the gfx950 tile widens its right-hand side to int8 in the
+    same array when it fits (one byte per weight) and runs the element-wise
+    kernel when it does not (72 x 1024 tiles of 32 x 16: 37.7 MB against the
+    32 MiB array): no allocation and no error either way, the bits of
+    iree_amd_uk_mmt4d_p and of the oracle, the large call first so that the
+    small one finds the array used."""
+    import torch
+    lib = uk.load_library()
+    rng = np.random.default_rng(404)
+    for M, N, K, acc, path in ((1, 72, 1024, False, "mmt4d:element-wise"),
+                               (4, 8, 64, True, "mmt4d:mfma-widened-s4"),
+                               (2, 3, 10, False, "mmt4d:mfma-widened-s4")):
+        case = ukref.Mmt4dCase(rng, F.MMT4D_TYPE_S8S4S32, M, N, K, 32, 32, 16, accumulate=acc)
+        lhs, rhs, out0 = gpucase._to_dev(case.lhs), gpucase._to_dev(case.rhs), gpucase._to_dev(case.out_init)
+        st_a, want = _run(lib.iree_amd_uk_mmt4d_p, case, lhs, rhs, out0)
+        assert st_a == 0
+        assert uk.last_kernel_path() == "mmt4d:mfma-widened-s4"
+        st, got = _run(lib.iree_amd_uk_mmt4d_noalloc_p, case, lhs, rhs, out0)
+        assert st == 0, lib.iree_amd_uk_last_error()
+        assert np.array_equal(got, want), (M, N, K)
+        free_before = torch.cuda.mem_get_info()[0]
+        st, got = _run(lib.iree_amd_uk_mmt4d_noalloc_p, case, lhs, rhs, out0)
+        assert st == 0, lib.iree_amd_uk_last_error()
+        assert uk.last_kernel_path() == path, (M, N, K)
+        assert torch.cuda.mem_get_info()[0] == free_before, "the call changed the free device memory"
+        assert np.array_equal(got, want), (M, N, K)
+        assert np.array_equal(got, case.run_oracle()), (M, N, K)

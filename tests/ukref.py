@@ -77,6 +77,12 @@ def oracle():
                                                          C.c_void_p, C.c_void_p, C.c_int64,
                                                          C.c_int64, C.c_int64, C.c_int64, C.c_int,
                                                          C.c_void_p]
+        lib.oracle_e2e_reference_matmul.restype = C.c_int
+        lib.oracle_e2e_reference_matmul.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                                    C.c_int64, C.c_int64, C.c_int64, C.c_uint32]
+        lib.oracle_e2e_pseudorandom_fill.restype = C.c_uint32
+        lib.oracle_e2e_pseudorandom_fill.argtypes = [C.c_uint32, C.c_int64, C.c_int32, C.c_int32,
+                                                     C.c_void_p]
         lib.oracle_silu_mul.restype = C.c_double
         lib.oracle_silu_mul.argtypes = [C.c_double, C.c_double]
         _oracle = lib
