@@ -694,6 +694,25 @@ def extras(args, torch, iree_amd, F, synth, lhs, rhs, out, ex):
 
         _, t = gpu_time(torch, do_ql, steps, warm)
         ex[f"dequant_matmul_i4_m{Mq}_n4096_k14336_us"] = round(t * 1e6, 2)
+    # K that is not whole 2048s (common decoder widths; the same buffers taken
+    # as that many bytes): workgroup slices of 2048, the last one shorter
+    for (No, Ko) in ((4096, 11008), (11264, 5120)):
+        Go = Ko // gs
+        for Mq in (1, 8):
+            xq = torch.from_numpy(synth.normal_f16(47 + Mq, Mq * Ko).view(np.int16)).cuda()
+            oq = torch.empty(Mq * No, dtype=torch.int16, device="cuda")
+            obytes = No * Ko // 2 + No * Go * 2 + No * Go // 2 + Mq * Ko * 2 + Mq * No * 2
+            state["i"] = 0
+
+            def do_qo():
+                k = state["i"] % nrot
+                state["i"] += 1
+                iree_amd.dequant_matmul_i4(xq, wq[k], sq, zq, oq, Mq, No, Ko, gs, qflags)
+
+            _, t = gpu_time(torch, do_qo, steps, warm)
+            assert iree_amd.last_kernel_path() == "dequant_i4:mfma", iree_amd.last_kernel_path()
+            ex[f"dequant_matmul_i4_m{Mq}_n{No}_k{Ko}_us"] = round(t * 1e6, 2)
+            ex[f"dequant_matmul_i4_m{Mq}_n{No}_k{Ko}_frac_of_hbm_peak"] = round(obytes / t / 1e9 / PEAK_HBM_GBS, 4)
     del wq, sq, zq
 
     # f16 mmt4d with a narrow left-hand side (decode shape: one outer row of

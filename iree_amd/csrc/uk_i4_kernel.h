@@ -1,5 +1,5 @@
-// The grouped int4-weight dequantising matmul kernel for K = 512 KB (2048 or
-// 4096), as a device function: wrapped in a __global__ by the library
+// The grouped int4-weight dequantising matmul kernel for workgroup slices of
+// K = 512 KB (2048 or 4096; a last slice may be shorter), as a device function: wrapped in a __global__ by the library
 // (uk_quant.hip, which describes the design) and by the code object built for a
 // HAL executable.
 #ifndef IREE_AMD_UK_I4_KERNEL_H_
@@ -43,11 +43,17 @@ namespace {
 //            chunk column of 16 rows hit 16 different bank groups without any
 //            padding: 16 rows x 8 waves x 1 KiB are 128 KiB, which with the
 //            32 KiB of partial sums is all the LDS there is. The area is sized
-//            for 8 or for 16 rows (a.stage_rows). The 32-row form stages in
-//            four phases of 8 rows through two buffers of 8 rows per wave (the
-//            same 128 KiB, which its partial sums take over afterwards): 256
-//            row loads per compute unit instead of 256 gathers of 16 half
-//            cache lines each (32 rows: 14.4 -> 12.2 us).
+//            for 8 or for 16 rows (a.stage_rows). The 32-row form stages span
+//            by span (128 k of all 32 rows at a time) through two buffers of
+//            8 KiB per wave (the same 128 KiB, which its partial sums take
+//            over afterwards), each span just ahead of the first tile's use
+//            of it.
+template <int N>
+__device__ __forceinline__ void i4_wait_vmcnt() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
 constexpr int kStageRowsMax = 16;
 template <int KB>
 constexpr int stage_row_bytes() { return KB * 128; }
@@ -83,9 +89,21 @@ __device__ __forceinline__ void dequant_matmul_i4_body(const I4Args& a) {
   const int nl = lane & 15, kc = lane >> 4;
   const int krow = blockIdx.y;               // K slice of this workgroup row (512 KB elements each)
   const int k_slice = (krow * kWaves + wave) * KB * 64;
-  const int g_first = k_slice >> a.log2_gs;  // first group of this wave's slice
+  // A K that is not whole workgroup slices leaves the last waves of the last
+  // workgroup row without any k (K is whole wave slices: the host checked).
+  // Such a wave runs like the others on zeros: its loads of weights and
+  // activations carry an offset past every buffer's end, which returns zeros
+  // without touching memory, and its group parameters are those of the last
+  // groups that exist (finite numbers, multiplied by sums that are zero).
+  const bool wave_has_k = k_slice < a.K;
+  const uint32_t past_end = wave_has_k ? 0u : 0x80000000u;
+  int g_first = k_slice >> a.log2_gs;        // first group of this wave's slice
+  {
+    constexpr int kGroupsLoaded = ((KB * 64) >> (kLog2Gs >= 9 ? 30 : kLog2Gs)) > 0 ? ((KB * 64) >> (kLog2Gs >= 9 ? 30 : kLog2Gs)) : 1;
+    if (!wave_has_k) g_first = a.G - kGroupsLoaded > 0 ? a.G - kGroupsLoaded : 0;
+  }
   const uint32_t tile_bytes = (uint32_t)a.K * 16;
-  const uint32_t voff = nl * a.col_stride + kc * 16;
+  const uint32_t voff = (nl * a.col_stride + kc * 16) | past_end;
   const uint32_t soff_wave = (krow * kWaves + wave) * SP * a.span_stride;
   const uint32_t half_stride = 16 * a.col_stride;
 
@@ -108,7 +126,7 @@ __device__ __forceinline__ void dequant_matmul_i4_body(const I4Args& a) {
   // last one, columns past N) return zeros without touching memory.
   auto tile_rsrc = [&](int nt) {
     const uint32_t off = (uint32_t)nt * tile_bytes;   // the host checked that this fits
-    const uint32_t left = nt < a.n_tiles ? a.w_bytes - off : 0;
+    const uint32_t left = nt < a.n_tiles ? a.w_bytes - off : 0;   // (columns past N: the buffer ends)
     return __builtin_amdgcn_make_buffer_rsrc((void*)(a.w + off), 0, left, 0x00020000);
   };
   auto load_slab = [&](__amdgpu_buffer_rsrc_t rsrc, int sp, int h) -> u32x4 {
@@ -143,12 +161,12 @@ __device__ __forceinline__ void dequant_matmul_i4_body(const I4Args& a) {
     // for in between; then the first tile's weights; then the wait for the rows
     // only (loads return in order: all but the weight loads issued since).
     const __amdgpu_buffer_rsrc_t xsrc = __builtin_amdgcn_make_buffer_rsrc(
-        (void*)(a.x + (size_t)a.m_base * a.K + k_slice), 0, 0x7FFFFFFF, 0x00020000);
+        (void*)(a.x + (size_t)a.m_base * a.K + (wave_has_k ? k_slice : 0)), 0, 0x7FFFFFFF, 0x00020000);
     if (lane < kLanesPerRow) {
 #pragma unroll 1
       for (int r = 0; r < rows; ++r)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(xsrc, (__attribute__((address_space(3))) void*)(stage + r * kRowBytes), 16,
-                                                 ((lane + r) & (kLanesPerRow - 1)) * 16, r * a.K * 2, 0, 0);
+                                                 (((lane + r) & (kLanesPerRow - 1)) * 16) | past_end, r * a.K * 2, 0, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -172,80 +190,84 @@ __device__ __forceinline__ void dequant_matmul_i4_body(const I4Args& a) {
           xraw[0][sp][q] = *(const u32x4*)(my_row + ((chunk - nl) & (kLanesPerRow - 1)) * 16);
         }
     }
-  } else {
-    // 32 rows: 8 rows at a time through two buffers of 8 rows per wave (16 rows
-    // of every wave's slice fill the LDS), the same full-width loads and rotated
-    // rows. Phases 0 and 1 and the first tile's weights are requested at once;
-    // a phase's rows go to registers as soon as they have landed (lanes whose
-    // row nl lies in the phase: 8 (p & 1) .. + 8 of half p / 2) and the phase
-    // after next is requested into the buffer so freed. Rows past M fetch the
-    // last row (so that every phase is 8 loads and the waits below can count)
-    // and are zeroed when the first tile turns them into operands.
-    constexpr int kRowBytes = stage_row_bytes<KB>();
-    constexpr int kLanesPerRow = KB * 8;
-    constexpr int kPhaseRows = 8;
-    static_assert(MH == 2, "four phases of 8 rows");
-    char* stage = stage_all + wave * 2 * kPhaseRows * kRowBytes;
-    const int last_row = (a.M - a.m_base < 32 ? a.M - a.m_base : 32) - 1;
-    const int cq = a.tiled ? 32 : 8, ckc = a.tiled ? 8 : 32;   // chunk strides in k
+  }
+  // 32 rows: SPAN by span (128 k of the wave's slice, 256 bytes of each of the
+  // 32 rows = 8 KiB) through two buffers per wave, the same full-width loads
+  // (4 rows per instruction) and rotated rows. The first tile walks its spans
+  // in order, so span s of the activations is only needed when that tile gets
+  // to span s: spans 0 and 1 and the first tile's weights are requested at
+  // once, span s + 2 when span s has gone to registers, so that the first
+  // tile multiplies span s while spans s + 1 and s + 2 arrive (staging all
+  // rows up front, in four phases of 8 rows: 12.4 us at 32 rows, this way
+  // 11.8). Timestamps inside the kernel show what bounds it: a compute unit's
+  // 8 waves get a 1 KiB load accepted every 35 cycles or so (29 bytes per
+  // clock), and the 256 KiB of activations plus 128 KiB of weights that each
+  // compute unit pulls in are 5.6 us of that path. Rows past M lie past the
+  // end of the buffer and read as zeros.
+  constexpr int kSpanLoads = 8;                              // load instructions per span and wave
+  constexpr int kSpanBytes = 32 * 256;
+  char* const span_stage = stage_all + wave * 2 * kSpanBytes;
+  const int span_cq = a.tiled ? 32 : 8, span_ckc = a.tiled ? 8 : 32;   // chunk strides in k
+  const int x_rows = a.M - a.m_base < 32 ? a.M - a.m_base : 32;
+  const __amdgpu_buffer_rsrc_t span_src = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(a.x + (size_t)a.m_base * a.K + (wave_has_k ? k_slice : 0)), 0,
+      (uint32_t)(((int64_t)x_rows * a.K - (wave_has_k ? k_slice : 0)) * 2), 0x00020000);
+  auto request_span = [&](int p) {
+#pragma unroll
+    for (int i = 0; i < kSpanLoads; ++i) {
+      const int row = 4 * i + (lane >> 4);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          span_src, (__attribute__((address_space(3))) void*)(span_stage + (p & 1) * kSpanBytes + i * 1024), 16,
+          (row * a.K * 2 + (((lane & 15) + row) & 15) * 16) | past_end, p * 256, 0, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  // Span p has landed when at most the loads issued behind it are outstanding
+  // (loads return in order; a smaller count than the true one only waits longer).
+  // The first tile's order of issue, SP = 4: spans 0, 1, the tile's 8 slabs;
+  // [span 0 taken] span 2; [span 1 taken] span 3, then the next tile's slabs
+  // as the tile consumes its own, those of span 0 first (held back until
+  // span 3 has been requested: a span requested behind loads from memory
+  // would only be seen to land after them). SP = 2: spans 0, 1, 4 slabs, then
+  // the next tile's slabs as usual.
+  auto wait_for_span = [&](int p) {
+    constexpr int kW = SP * 2;
+    static_assert(SP == 2 || SP == 4, "the counts below are those of two or four spans");
+    if constexpr (SP == 4) {
+      if (p == 0) i4_wait_vmcnt<kSpanLoads + kW>();          // span 1, the slabs
+      else if (p == 1) i4_wait_vmcnt<kW + kSpanLoads>();     // the slabs, span 2
+      else if (p == 2) i4_wait_vmcnt<kSpanLoads + 4>();      // span 3, next slabs of spans 0 and 1
+      else i4_wait_vmcnt<6>();                               // next slabs of spans 0 to 2
+    } else {
+      if (p == 0) i4_wait_vmcnt<kSpanLoads + kW>();
+      else i4_wait_vmcnt<kW + 2>();
+    }
+  };
+  auto take_span = [&](int p, u32x4 (&raw)[MH][SP][4]) {
+    const char* buf = span_stage + (p & 1) * kSpanBytes;
+#pragma unroll
+    for (int mh = 0; mh < MH; ++mh) {
+      const int row = mh * 16 + nl;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int chunk = (q * span_cq + kc * span_ckc) >> 3;       // of 8 elements, within the span
+        raw[mh][p][q] = *(const u32x4*)(buf + row * 256 + ((chunk - row) & 15) * 16);
+      }
+    }
+    // the reads have left LDS before anything is loaded over them
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  if constexpr (!kStageX) {
+    static_assert(MH == 2, "the span-wise staging serves the 32-row form");
     const __amdgpu_buffer_rsrc_t rsrc = tile_rsrc(nt);
-    const __amdgpu_buffer_rsrc_t xsrc = __builtin_amdgcn_make_buffer_rsrc(
-        (void*)(a.x + (size_t)a.m_base * a.K + k_slice), 0, 0x7FFFFFFF, 0x00020000);
-    auto request_phase = [&](int p) {
-      if (lane < kLanesPerRow) {
-#pragma unroll
-        for (int r = 0; r < kPhaseRows; ++r) {
-          int row = p * kPhaseRows + r;
-          row = row < last_row ? row : last_row;
-          __builtin_amdgcn_raw_ptr_buffer_load_lds(
-              xsrc, (__attribute__((address_space(3))) void*)(stage + ((p & 1) * kPhaseRows + r) * kRowBytes), 16,
-              ((lane + r) & (kLanesPerRow - 1)) * 16, row * a.K * 2, 0, 0);
-        }
-      }
-      __builtin_amdgcn_sched_barrier(0);
-    };
-    auto take_phase = [&](auto phase) {
-      constexpr int p = decltype(phase)::value;
-      if ((nl >> 3) == (p & 1)) {
-        const int r = nl & 7;
-        const char* my_row = stage + ((p & 1) * kPhaseRows + r) * kRowBytes;
-#pragma unroll
-        for (int sp = 0; sp < SP; ++sp)
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const int chunk = (sp * 128 + q * cq + kc * ckc) >> 3;      // of 8 elements, within the slice
-            xraw[p >> 1][sp][q] = *(const u32x4*)(my_row + ((chunk - r) & (kLanesPerRow - 1)) * 16);
-          }
-      }
-      // the reads have left LDS before anything is loaded over them
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-      __builtin_amdgcn_sched_barrier(0);
-    };
-    request_phase(0);
-    request_phase(1);
+    request_span(0);
+    if constexpr (SP > 1) request_span(1);
 #pragma unroll
     for (int sp = 0; sp < SP; ++sp)
 #pragma unroll
       for (int h = 0; h < 2; ++h) wreg[sp][h] = load_slab(rsrc, sp, h);
     __builtin_amdgcn_sched_barrier(0);
-    // (loads return in order: waiting for all but the n youngest)
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kPhaseRows + SP * 2) : "memory");   // phase 0
-    take_phase(std::integral_constant<int, 0>());
-    request_phase(2);
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kPhaseRows + SP * 2) : "memory");   // phase 1
-    take_phase(std::integral_constant<int, 1>());
-    if (last_row >= 3 * kPhaseRows) {
-      request_phase(3);
-      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kPhaseRows) : "memory");          // the weights and phase 2
-      take_phase(std::integral_constant<int, 2>());
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                           // phase 3
-      take_phase(std::integral_constant<int, 3>());
-    } else {
-      // (at most 24 rows: the last phase's rows do not exist; their lanes keep
-      // whatever their registers hold, which the first tile zeroes)
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      take_phase(std::integral_constant<int, 2>());
-    }
   }
   half8 xf[MH][SP][4];
   // (kSubnormal) the sum of the activations of row r (accumulator layout: every
@@ -276,6 +298,20 @@ __device__ __forceinline__ void dequant_matmul_i4_body(const I4Args& a) {
       for (int mh = 0; mh < MH; ++mh) acc[h][mh] = part[h][mh] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int sp = 0; sp < SP; ++sp) {
+      if constexpr (kFirst && !kStageX) {
+        __builtin_amdgcn_sched_barrier(0);
+        wait_for_span(sp);
+        take_span(sp, xraw);
+        if (sp + 2 < SP) request_span(sp + 2);
+        if (sp + 3 == SP) {
+          // (the next tile's slabs of the spans before this one, held back so far)
+#pragma unroll
+          for (int e = 0; e < sp; ++e)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) wreg[e][h] = load_slab(rsrc_next, e, h);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
       if constexpr (kFirst) {
 #pragma unroll
         for (int mh = 0; mh < MH; ++mh) {
@@ -367,7 +403,7 @@ __device__ __forceinline__ void dequant_matmul_i4_body(const I4Args& a) {
         // tile. The fences keep the requests in slab order, which is what
         // makes every wait in the loop a wait for the OLDEST outstanding load.
         __builtin_amdgcn_sched_barrier(0);
-        wreg[sp][h] = load_slab(rsrc_next, sp, h);
+        if (!(kFirst && !kStageX && sp + 3 < SP)) wreg[sp][h] = load_slab(rsrc_next, sp, h);
         __builtin_amdgcn_sched_barrier(0);
       }
     }

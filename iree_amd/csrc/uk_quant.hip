@@ -99,9 +99,10 @@ template <int KB, int MH, bool kZpU4, int kLog2Gs>
 int launch_instance(const I4Args& a, int blocks, int k_rows, hipStream_t s) {
   void (*kernel)(I4Args) = dequant_matmul_i4_kernel<KB, MH, kZpU4, kLog2Gs>;
   // 16-row form: the rows it stages (8 or 16 per wave); 32-row form: two
-  // buffers of 8 rows per wave, and at least the 64 KiB of partial sums that
-  // later live in the same memory
-  constexpr size_t kMaxLds = (size_t)kWaves * kStageRowsMax * stage_row_bytes<KB>();
+  // buffers of one span (128 k of 32 rows) per wave, and at least the 64 KiB of
+  // partial sums that later live in the same memory
+  constexpr size_t kMaxLds = MH == 2 ? (size_t)kWaves * 2 * 32 * 256    // two spans of 32 rows per wave
+                                     : (size_t)kWaves * kStageRowsMax * stage_row_bytes<KB>();
   constexpr size_t kPartialBytes = MH == 2 ? (size_t)2 * kWaves * 2 * MH * 4 * 64 * sizeof(float) : 0;
   constexpr size_t kAttrLds = kMaxLds > kPartialBytes ? kMaxLds : kPartialBytes;
   const size_t lds = MH == 1 ? (size_t)kWaves * a.stage_rows * stage_row_bytes<KB>() : kAttrLds;
@@ -210,18 +211,21 @@ int launch_dequant_matmul_i4(const void* x, const void* w, const void* scale, co
   const bool gs_pow2 = (1ll << a.log2_gs) == group_size;
   a.span_stride = tiled ? 2048u : 64u;
   a.col_stride = tiled ? 64u : (uint32_t)(K / 2);
-  // Fast path: K in whole slices of 512 * KB for KB in {4, 8} (every wave owns
+  // Fast path: K in slices of 512 * KB for KB in {4, 8} (every wave owns
   // KB blocks of 64 of its workgroup's slice; more than one slice: workgroup
-  // rows and a second kernel that adds their partial sums),
+  // rows and a second kernel that adds their partial sums; K in whole 256s,
+  // the last slice as short as that leaves it),
   // power-of-two groups (below 128 only from tiled weights, where a group never
   // straddles an MFMA), a weight buffer that 32-bit offsets can address (plus
   // one tile, for the offset of the tile after the last), 16-byte aligned
   // operands, and group parameters aligned to what one wave slice loads at once.
   const int64_t w_bytes = N * K / 2;
   // (a longer K in whole slices of 4096, or else of 2048, over workgroup rows)
+  // (any other K in whole wave slices of 256: slices of 2048 whose last one is
+  // shorter, its trailing waves running on zeros)
   const int slice_kb = K % 4096 == 0 ? 8 : 4;
-  const int64_t k_rows = K / (512 * slice_kb);
-  const bool k_ok = K % 2048 == 0 && K >= 2048 && k_rows <= 64;
+  const int64_t k_rows = ceil_div(K, (int64_t)512 * slice_kb);
+  const bool k_ok = K % 256 == 0 && K >= 256 && k_rows <= 64 && (group_size <= 256 || K % 2048 == 0);
   const bool gs_ok = gs_pow2 && group_size >= (tiled ? 32 : 128);
   const bool size_ok = w_bytes + K * 16 < (1ll << 32);
   const bool aligned = ((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0 &&

@@ -20,7 +20,7 @@ def tile_weights(w_bytes, N, K):
     return np.ascontiguousarray(d.transpose(0, 2, 1, 4, 3)).reshape(-1).view(np.uint8)
 
 
-def run_case(uk, M, N, K, gs, zp_u4, tiled, seed=0, frac_zp=False):
+def run_case(uk, M, N, K, gs, zp_u4, tiled, seed=0, frac_zp=False, want_path=None, repeats=0):
     import torch
     G = K // gs
     x = synth.normal_f16(seed + 1, M * K)
@@ -43,11 +43,21 @@ def run_case(uk, M, N, K, gs, zp_u4, tiled, seed=0, frac_zp=False):
     wd = tile_weights(w, N, K) if tiled else w
     flags = (F.DEQUANT_MATMUL_ZP_U4 if zp_u4 else 0) | (F.DEQUANT_MATMUL_W_TILED if tiled else 0)
     out = torch.full((M * N,), 0x7E00, dtype=torch.int16, device="cuda")
-    uk.dequant_matmul_i4(torch.from_numpy(x.view(np.int16)).cuda(), torch.from_numpy(wd).cuda(),
-                         torch.from_numpy(s.view(np.int16)).cuda(),
-                         torch.from_numpy(zp.view(np.uint8)).cuda(), out, M, N, K, gs, flags)
+    xd, wdev = torch.from_numpy(x.view(np.int16)).cuda(), torch.from_numpy(wd).cuda()
+    sd, zd = torch.from_numpy(s.view(np.int16)).cuda(), torch.from_numpy(zp.view(np.uint8)).cuda()
+    uk.dequant_matmul_i4(xd, wdev, sd, zd, out, M, N, K, gs, flags)
     torch.cuda.synchronize()
-    got = out.cpu().numpy().view(np.float16).astype(np.float64)
+    bits = out.cpu().numpy().copy()
+    if want_path is not None:
+        assert uk.last_kernel_path() == want_path, (uk.last_kernel_path(), M, N, K, gs, tiled)
+    for _ in range(repeats):
+        # (the same call again, the result buffer refilled: the sums are added in
+        # a fixed order, so every run gives the same bits)
+        out.fill_(0x7E00)
+        uk.dequant_matmul_i4(xd, wdev, sd, zd, out, M, N, K, gs, flags)
+        torch.cuda.synchronize()
+        assert np.array_equal(out.cpu().numpy(), bits), "two runs of the same call differ"
+    got = bits.view(np.float16).astype(np.float64)
     wantf = want.view(np.float16).astype(np.float64)
     err = np.abs(got - wantf)
     assert np.all(err <= ATOL + RTOL * np.abs(wantf)), (M, N, K, gs, zp_u4, tiled, float(err.max()))
@@ -59,7 +69,7 @@ def run_case(uk, M, N, K, gs, zp_u4, tiled, seed=0, frac_zp=False):
 def test_decode_shape_llama_ffn(uk, cuda, M, tiled):
     """The decode configuration: K = 4096, N = 14336, groups of 128, f16 scales,
     packed uint4 zero points."""
-    err, mag = run_case(uk, M, 14336, 4096, 128, True, tiled)
+    err, mag = run_case(uk, M, 14336, 4096, 128, True, tiled, want_path="dequant_i4:mfma", repeats=3)
     # f32 accumulation of exact products: far inside the stated tolerance, at
     # most one f16 unit in the last place from the correctly rounded result
     assert err <= float(np.spacing(np.float16(max(1.0, mag))))
@@ -76,6 +86,24 @@ def test_mfma_kernel_group_sizes_and_zero_point_forms(uk, cuda, K, gs, zp_u4):
     for M, N, tiled in [(3, 96, True), (32, 64, False), (40, 100, False), (17, 160, True), (12, 64, True),
                         (8, 32, False), (9, 64, False), (24, 96, False), (25, 64, True), (31, 64, False)]:
         run_case(uk, M, N, K, gs, zp_u4, tiled, seed=K + gs)
+
+
+@pytest.mark.parametrize("K", [11008, 5120, 256, 768, 2304, 6400, 13824])
+@pytest.mark.parametrize("gs,zp_u4", [(128, True), (128, False), (256, True), (64, True), (32, False)])
+def test_mfma_kernel_serves_every_k_in_whole_256s(uk, cuda, K, gs, zp_u4):
+    """K is not limited to whole 2048s (the pattern puts no such limit on it:
+    11008 and 5120 are common decoder widths): the matrix-core kernel runs
+    workgroup slices of 2048 whose last one is shorter, the trailing waves of
+    that slice multiplying zeros. One row, few rows, 16, 17 and 32 rows (all
+    staging forms), both weight layouts, against the f64 oracle, the kernel
+    family asserted and two runs bit-identical."""
+    if K % gs:
+        pytest.skip("K is whole groups")
+    for M, N, tiled in [(1, 14336 if K in (11008, 5120) else 96, True), (8, 64, True), (16, 96, False),
+                        (17, 64, True), (32, 160, False), (3, 32, False)]:
+        if gs < 128 and not tiled:
+            continue
+        run_case(uk, M, N, K, gs, zp_u4, tiled, seed=K + gs + M, want_path="dequant_i4:mfma", repeats=1)
 
 
 @pytest.mark.parametrize("K,gs", [(6144, 128), (8192, 64), (14336, 128), (14336, 256), (2048, 64)])
