@@ -302,8 +302,25 @@ __global__ __launch_bounds__(256) void pack_transpose_lds_kernel(TransArgs a) {
 }
 
 template <int ES>
+__global__ __launch_bounds__(64) void unpack_transpose_block_kernel(TransArgs a) {
+  unpack_transpose_block_body<ES>(a);
+}
+
+template <int ES>
 int launch_unpack_transpose(TransArgs a, hipStream_t s) {
   const int64_t cols = a.m_size1 < a.padded_cols ? a.m_size1 : a.padded_cols;
+  // Tiles of whole CE columns and enough columns for a wave's 16 blocks: the
+  // kernel that moves a CE x CE block per lane, one wave per workgroup.
+  constexpr int CE = 16 / ES;
+  if (a.tile_cols % CE == 0 && cols >= 16 * CE) {
+    const int64_t bx = ceil_div(cols, (int64_t)16 * CE);
+    const int64_t by = ceil_div(a.row_groups, (int64_t)4);
+    if (bx >= 1 && by >= 1 && bx * by <= 0x7FFFFFFF) {
+      a.blocks_x = (uint32_t)bx; a.blocks_y = (uint32_t)by;
+      hipLaunchKernelGGL((unpack_transpose_block_kernel<ES>), dim3((unsigned)(bx * by)), dim3(64), 0, s, a);
+      return check_hip(hipGetLastError(), "unpack_transpose launch");
+    }
+  }
   const int64_t bx = ceil_div(cols, (int64_t)64);
   const int64_t by = ceil_div(a.row_groups, (int64_t)(4 * kTransUnroll));
   if (bx < 1 || by < 1 || bx * by > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;

@@ -115,6 +115,10 @@ def test_transposing_pack_with_ragged_edges(uk, cuda, type_flag, tr, tc, rows, c
     (F.UNPACK_TYPE_F16F16, 16, 32, 129, 1003),
     (F.UNPACK_TYPE_BF16BF16, 24, 5, 123, 77),    # odd tile width, three row groups
     (F.UNPACK_TYPE_F32F32, 8, 32, 4096, 70),
+    (F.UNPACK_TYPE_F16F16, 32, 8, 2000, 130),    # lanes whose 8 columns end at the matrix edge
+    (F.UNPACK_TYPE_F32F32, 32, 4, 77, 64),       # exactly one wave of blocks across
+    (F.UNPACK_TYPE_I32I32, 32, 16, 1030, 1000),  # row groups past the matrix in the last quartet
+    (F.UNPACK_TYPE_BF16BF16, 32, 32, 511, 515),
 ])
 def test_transposing_unpack_with_ragged_edges(uk, cuda, type_flag, tr, tc, rows, cols):
     """Unpacks of tiles stored column by column (matrix tiles of tr rows x tc
