@@ -414,7 +414,40 @@ int launch_pack_stream(const StreamArgs& a, hipStream_t s) {
 }
 
 template <int ES>
+__global__ __launch_bounds__(64) void unpack_aligned_kernel(Pow2Args a) { unpack_aligned_body<ES>(a); }
+
+// Rows of at least 1 KiB in power-of-two tiles: the kernel whose stores are
+// aligned cache lines (one wave per workgroup: 4 rows x one 256-byte window).
+template <int ES>
+int launch_unpack_aligned(const StreamArgs& a, hipStream_t s) {
+  const int64_t row_bytes = a.m_size1 * ES;
+  // (32-bit offsets per lane: the same limits as the other power-of-two kernel)
+  if (!pow2_eligible(a, ES) || row_bytes < 1024 || row_bytes + 512 >= (1ll << 31) || a.m_size0 < 1 ||
+      a.m_stride0 * ES * 16 + row_bytes + 512 >= (1ll << 31))
+    return IREE_AMD_UK_STATUS_NOT_FOUND;
+  Pow2Args p;
+  p.mat = a.mat; p.tiled = a.tiled;
+  p.m_size0 = a.m_size0; p.m_size1 = a.m_size1; p.m_pitch_bytes = a.m_stride0 * ES;
+  p.t_stride_row_bytes = a.t_stride_row_bytes; p.t_stride_col_bytes = a.t_stride_col_bytes;
+  p.padded_rows = a.padded_rows;
+  p.chunks_per_row = a.chunks_per_row; p.padded_chunks_per_row = a.padded_chunks_per_row;
+  p.log2_tile_rows = a.log2_tile_rows; p.log2_cpr = a.log2_cpr;
+  p.padding = a.padding;
+  // windows a row can touch: it starts up to 127 bytes into its first line
+  const int64_t bx = (row_bytes + 127 + 255) / 256;
+  const int64_t by = ceil_div(a.m_size0, (int64_t)4);
+  if (bx * by > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  p.blocks_x = (uint32_t)bx; p.blocks_y = (uint32_t)by;
+  hipLaunchKernelGGL((unpack_aligned_kernel<ES>), dim3((unsigned)(bx * by)), dim3(64), 0, s, p);
+  return check_hip(hipGetLastError(), "unpack_aligned launch");
+}
+
+template <int ES>
 int launch_unpack_stream(const StreamArgs& a, hipStream_t s) {
+  {
+    const int st = launch_unpack_aligned<ES>(a, s);
+    if (st != IREE_AMD_UK_STATUS_NOT_FOUND) return st;
+  }
   if (pow2_eligible(a, ES)) return launch_stream_pow2<ES, false>(a, s);
   const int64_t bx = ceil_div(a.chunks_per_row, 4 * kBlockChunks);
   const int64_t row_groups = ceil_div(a.m_size0, kBlockRows * kStreamUnroll);

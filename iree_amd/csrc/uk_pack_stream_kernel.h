@@ -177,6 +177,121 @@ __device__ __forceinline__ void stream_pow2_body(const Pow2Args a) {
   }
 }
 
+// Unpack whose stores are whole, aligned cache lines. The rows of a matrix
+// rarely start on a 128-byte line (8191 x 5001 f16: every row starts 10002
+// bytes after the one before), so a kernel that moves 16-byte chunks from
+// their place in a tile to their place in the row writes pieces that begin and
+// end inside lines it shares with the neighbouring pieces, and non-temporal
+// stores of such pieces lose (measured with the kernel above: 5.40 TB/s with
+// ordinary stores, 5.26 with non-temporal ones; on a matrix whose rows do
+// start on lines 5.61 and 5.94). Here a wave instead owns, for each of 4
+// rows, one 256-byte window of MEMORY that starts on a line: lane (row, t)
+// produces the 16 bytes at window + 16 t, which are bytes o .. o + 16 of the
+// row for an o that is rarely a multiple of 16. It loads the tile chunk o / 16,
+// takes the next one from the next lane (a cross-lane move; the last lane of a
+// row loads its own), shifts the pair right by o % 16 bytes (a dword select by
+// two bits of the shift and a byte align by the other two) and stores 16
+// aligned bytes non-temporally. Only the first and last window of a row write
+// partial chunks, element by element. Same tile geometry as the kernel above
+// (power-of-two tiles, no inner transpose). Measured: 8191 x 5001 f16 from
+// 32x16 tiles 5.78 TB/s (5.40 with the kernel above), 8192 x 5120 6.05; two
+// and four blocks of rows per wave 5.32 and 4.99; loading both chunks per
+// lane 3.7 (non-temporal: the shared chunk comes from memory twice) to 4.1.
+template <int ES, int kU = 1>
+__device__ __forceinline__ void unpack_aligned_body(const Pow2Args a) {
+  typedef typename Chunk<ES>::elem_t elem_t;
+  constexpr int CE = 16 / ES;
+  const uint32_t lane = threadIdx.x & 63;
+  uint32_t bx, by;
+  {
+    constexpr uint32_t kXcds = 8;
+    const uint32_t total = a.blocks_x * a.blocks_y;
+    const uint32_t per = total / kXcds, rem = total % kXcds;
+    const uint32_t xcd = blockIdx.x % kXcds, idx = blockIdx.x / kXcds;
+    const uint32_t logical = xcd * per + (xcd < rem ? xcd : rem) + idx;
+    by = logical / a.blocks_x;
+    bx = logical - by * a.blocks_x;
+  }
+  // All 64-bit arithmetic is the wave's (scalar unit); lanes work with 32-bit
+  // offsets from the wave's first row on both sides.
+  const int64_t r0 = (int64_t)by * (4 * kU);
+  const char* mat_base = a.mat + r0 * a.m_pitch_bytes;
+  const char* tiled_base = a.tiled + (r0 >> a.log2_tile_rows) * a.t_stride_row_bytes;
+  const uint32_t rows_left = (uint32_t)(a.m_size0 - r0 < 4 * kU ? a.m_size0 - r0 : 4 * kU);
+  const uint32_t mat_lo = (uint32_t)(uintptr_t)mat_base;
+  const uint32_t pitch = (uint32_t)a.m_pitch_bytes;
+  const uint32_t srow = (uint32_t)a.t_stride_row_bytes, scol = (uint32_t)a.t_stride_col_bytes;
+  const uint32_t tile_rows = 1u << a.log2_tile_rows, cpr = 1u << a.log2_cpr;
+  const uint32_t trow0 = (uint32_t)r0 & (tile_rows - 1);
+  const int32_t row_bytes = (int32_t)(a.m_size1 * ES);
+  const int32_t last_chunk = (int32_t)a.padded_chunks_per_row - 1;
+  const uint32_t rl = lane >> 4, t = lane & 15;
+  u32x4 lo[kU], hi[kU];
+  int32_t o[kU];
+  uint32_t row_off[kU];
+  bool row_ok[kU];
+  // all the loads of the wave's kU blocks of 4 rows first
+#pragma unroll
+  for (int u = 0; u < kU; ++u) {
+    const uint32_t rloc = u * 4 + rl;
+    row_ok[u] = rloc < rows_left;
+    const uint32_t rr = row_ok[u] ? rloc : rows_left - 1;    // (loads of a row past the end stay inside the buffer)
+    row_off[u] = rr * pitch;
+    // this lane's 16 bytes of memory (bx-th window of the row's first line on) and where in the row they lie
+    const uint32_t head = (mat_lo + row_off[u]) & 127u;
+    o[u] = (int32_t)(bx * 256 + t * 16) - (int32_t)head;     // -127 ..
+    const int32_t q = o[u] >> 4;                             // (floor)
+    const uint32_t r = trow0 + rr;
+    const uint32_t in_panel = (r >> a.log2_tile_rows) * srow + ((r & (tile_rows - 1)) << a.log2_cpr) * 16;
+    auto chunk_at = [&](int32_t qq) -> const u32x4* {
+      qq = qq < 0 ? 0 : (qq > last_chunk ? last_chunk : qq);
+      return (const u32x4*)(tiled_base + (in_panel + ((uint32_t)qq >> a.log2_cpr) * scol + ((uint32_t)qq & (cpr - 1)) * 16));
+    };
+    // The second chunk is the first one of the next lane of the row (fetched
+    // from there across lanes; loading it as well doubled the reads); the
+    // row's last lane loads its own.
+    lo[u] = __builtin_nontemporal_load(chunk_at(q));
+    hi[u] = u32x4{0u, 0u, 0u, 0u};
+    if (t == 15 && (o[u] & 15)) hi[u] = *chunk_at(q + 1);
+  }
+#pragma unroll
+  for (int u = 0; u < kU; ++u) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      // (row_shl:1: lane t of a row of 16 takes lane t + 1's value, lane 15 keeps its own)
+      hi[u][i] = (uint32_t)__builtin_amdgcn_update_dpp((int)hi[u][i], (int)lo[u][i], 0x101, 0xf, 0xf, false);
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < kU; ++u) {
+    // bytes sb .. sb + 16 of lo : hi (everything in named registers: an array
+    // here ends up in LDS)
+    const uint32_t sb = (uint32_t)o[u] & 15;
+    const bool by8 = (sb & 8) != 0, by4 = (sb & 4) != 0;
+    const uint32_t a0 = by8 ? lo[u].z : lo[u].x, a1 = by8 ? lo[u].w : lo[u].y, a2 = by8 ? hi[u].x : lo[u].z,
+                   a3 = by8 ? hi[u].y : lo[u].w, a4 = by8 ? hi[u].z : hi[u].x, a5 = by8 ? hi[u].w : hi[u].y;
+    const uint32_t b0 = by4 ? a1 : a0, b1 = by4 ? a2 : a1, b2 = by4 ? a3 : a2, b3 = by4 ? a4 : a3, b4 = by4 ? a5 : a4;
+    u32x4 out;
+    out.x = __builtin_amdgcn_alignbyte(b1, b0, sb & 3);
+    out.y = __builtin_amdgcn_alignbyte(b2, b1, sb & 3);
+    out.z = __builtin_amdgcn_alignbyte(b3, b2, sb & 3);
+    out.w = __builtin_amdgcn_alignbyte(b4, b3, sb & 3);
+    if (!row_ok[u]) continue;
+    char* dst = (char*)mat_base + row_off[u] + o[u];
+    if (o[u] >= 0 && o[u] + 16 <= row_bytes) {
+      __builtin_nontemporal_store(out, (u32x4*)dst);
+    } else if (o[u] + 16 > 0 && o[u] < row_bytes) {
+      // (row start and row end are whole elements, and so is every piece of a chunk)
+#pragma unroll
+      for (int e = 0; e < CE; ++e) {
+        const int32_t at = o[u] + e * ES;
+        const uint32_t word = e * ES / 4 == 0 ? out.x : e * ES / 4 == 1 ? out.y : e * ES / 4 == 2 ? out.z : out.w;
+        if (at >= 0 && at < row_bytes) ((elem_t*)dst)[e] = (elem_t)(word >> (8 * (e * ES % 4)));
+      }
+    }
+  }
+}
+
 }  // namespace
 }  // namespace uk
 

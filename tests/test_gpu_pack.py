@@ -136,6 +136,34 @@ def test_transposing_unpack_with_ragged_edges(uk, cuda, type_flag, tr, tc, rows,
         assert np.array_equal(gpucase.run_unpack(loose), loose.run_oracle()), (to, "loose")
 
 
+@pytest.mark.parametrize("type_flag,t0,t1,rows,cols", [
+    (F.UNPACK_TYPE_F16F16, 32, 16, 70, 1001),     # rows of 2002 bytes: every alignment of a row start mod 16
+    (F.UNPACK_TYPE_F16F16, 32, 16, 9, 512),       # exactly 1 KiB per row
+    (F.UNPACK_TYPE_BF16BF16, 8, 8, 37, 3000),
+    (F.UNPACK_TYPE_F32F32, 32, 32, 45, 777),
+    (F.UNPACK_TYPE_I32I32, 32, 32, 130, 257),
+    (F.UNPACK_TYPE_F32F32, 16, 4, 33, 1030),
+])
+def test_unpack_with_line_aligned_stores_every_row_alignment(uk, cuda, type_flag, t0, t1, rows, cols):
+    """Rows of 1 KiB and more in power-of-two tiles run the unpack kernel whose
+    stores are aligned cache lines (every 16 stored bytes are a byte-shifted
+    pair of tile chunks): row pitches and first-element offsets that give every
+    alignment of a row start, rows that end inside their last window, row
+    counts that are not whole blocks of 4; the whole destination buffer is
+    compared, so the bytes before and behind every row are untouched."""
+    rng = np.random.default_rng(rows * 7 + cols)
+    o0, o1 = -(-rows // t0), -(-cols // t1)
+    for to in (0, 1):
+        for extra_pitch, out_offset in ((0, 0), (1, 3), (5, 64), (37, 1), (64, 17)):
+            case = ukref.UnpackCase(rng, type_flag, o0, o1, t0, t1, transpose_outer=to, out_size=(rows, cols))
+            case.out_stride0 = cols + extra_pitch
+            case.out_offset = out_offset
+            info = np.iinfo(case.dtype)
+            case.out_init = rng.integers(0, int(info.max) + 1, size=out_offset + rows * case.out_stride0 + 131,
+                                         dtype=np.uint64).astype(case.dtype)
+            assert np.array_equal(gpucase.run_unpack(case), case.run_oracle()), (to, extra_pitch, out_offset)
+
+
 def test_full_size_f16_8191x5001_pack_unpack_round_trip(uk, cuda):
     """The bandwidth workload at its real size: packed bytes equal the oracle's
     (and the committed SHA-256 produced by the reference library), the padded
