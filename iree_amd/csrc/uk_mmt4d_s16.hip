@@ -23,7 +23,10 @@
 // Narrow left-hand side tiles (one outer row of 1..15 rows against an 8- or
 // 4-bit right-hand side: the reference's own s16 x u4 tile is 1 x 32 x 8,
 // arch/x86_64/mmt4d_x86_64_tiles.inl:75) take the same route through the narrow
-// matrix-core kernel: the planes are the 2 M0 + 1 rows of one int8 tile.
+// matrix-core kernel: the planes are the 2 M0 + 1 rows of one int8 tile. With
+// 16 to 31 rows those rows do not fit one narrow tile, and a 16-bit right-hand
+// side has planes of its own: such tiles (one outer row) run as 32-row planes
+// whose rows past M0 are zeros, the last pass storing M0 rows per tile.
 #include "uk_common.h"
 
 namespace uk {
@@ -40,6 +43,7 @@ struct RetileArgs {
   int K0;
   int64_t k16;            // K tiles of the result: ceil(K * K0 / 16)
   uint8_t* dst;           // outer rows of k16 tiles of 32 x 16 bytes
+  int src_rows;           // rows of a source tile: 32, or fewer (the result's rows beyond them are zeros)
 };
 
 // One thread makes row r of result tile (o, t): 16 consecutive K positions of
@@ -60,14 +64,14 @@ __global__ __launch_bounds__(256) void retile_planes_kernel(const RetileArgs a) 
     uint32_t hi[4] = {0, 0, 0, 0}, lo[4] = {0, 0, 0, 0}, cst[4] = {0, 0, 0, 0};
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
-      if (k_first + e < kk0) {
-        const int64_t i = base + (kt * 32 + r) * a.K0 + k0;
+      if (k_first + e < kk0 && r < a.src_rows) {
+        const int64_t i = base + (kt * a.src_rows + r) * a.K0 + k0;
         const int sh = 8 * (e & 3);
         if (kKind == kSourceS16) {
           const int v = ((const int16_t*)a.src)[i];
           hi[e >> 2] |= (uint32_t)((v >> 8) & 255) << sh;
           lo[e >> 2] |= (uint32_t)(((v & 255) - 128) & 255) << sh;
-          cst[e >> 2] |= 64u << sh;
+          cst[e >> 2] |= 64u << sh;       // (row 0 is the one the last pass reads; it always exists)
         } else if (kKind == kSourceS8) {
           hi[e >> 2] |= (uint32_t)((const uint8_t*)a.src)[i] << sh;
         } else {
@@ -144,6 +148,7 @@ struct CombineArgs {
   uint32_t* out;             // offset applied
   int64_t out_stride0;
   int accumulate;
+  int rows;                  // rows of a result tile: 32, or the M0 of a narrow left-hand side
 };
 
 // One thread: 4 consecutive columns of one row of one result tile.
@@ -154,6 +159,7 @@ __global__ __launch_bounds__(256) void combine_planes_kernel(const CombineArgs a
        idx += (int64_t)gridDim.x * blockDim.x) {
     const int in_tile = (int)(idx & 255);            // row * 8 + group of 4 columns
     const int r = in_tile >> 3, c = (in_tile & 7) * 4;
+    if (r >= a.rows) continue;
     const int64_t j = (idx >> 8) % a.N, i = (idx >> 8) / a.N;
     auto tile = [&](int64_t ti, int64_t tj) { return a.product + (ti * a.cols + tj) * 1024; };
     auto four = [&](const uint32_t* t, int row) { return *(const u32x4*)(t + row * 32 + c); };
@@ -167,7 +173,7 @@ __global__ __launch_bounds__(256) void combine_planes_kernel(const CombineArgs a
           four(tile(2 * a.M, a.N + j), 0) * 2u;
       v += tile(i, cj)[r * 32] * 512u + tile(a.M + i, cj)[r * 32] * 2u + tile(2 * a.M, cj)[0] * 4u;
     }
-    uint32_t* o = a.out + i * a.out_stride0 + j * 1024 + r * 32 + c;
+    uint32_t* o = a.out + i * a.out_stride0 + j * (a.rows * 32) + r * 32 + c;
     // (the result buffer is only element-aligned)
 #pragma unroll
     for (int e = 0; e < 4; ++e) o[e] = a.accumulate ? o[e] + v[e] : v[e];
@@ -272,10 +278,11 @@ bool mmt4d_s16_planes_supported(uint32_t flags, int M0, int N0, int K0) {
       type != IREE_AMD_UK_FLAG_MMT4D_TYPE_S16U4S32)
     return false;
   if (N0 != 32 || K0 < 1) return false;
-  if (M0 == 32) return mmt4d_mfma_supported(IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32, 32, 32, 16);
-  // narrow left-hand sides with an 8- or 4-bit right-hand side: 2 M0 + 1 plane rows in one narrow tile
-  return type != IREE_AMD_UK_FLAG_MMT4D_TYPE_S16S16S32 && M0 >= 1 && M0 <= 15 &&
-         mmt4d_skinny_supported(IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32, 2 * M0 + 1, 32, 16);
+  // 32 rows, and narrow left-hand sides of 1 to 31 (one outer row): up to 15
+  // rows against an 8- or 4-bit right-hand side as the 2 M0 + 1 plane rows of
+  // one narrow tile, the others as 32-row planes whose rows past M0 are zeros
+  return M0 >= 1 && M0 <= 32 && mmt4d_mfma_supported(IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32, 32, 32, 16) &&
+         mmt4d_skinny_supported(IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32, 31, 32, 16);
 }
 
 namespace {
@@ -297,7 +304,7 @@ int launch_narrow(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) {
   const RetileNarrowArgs la = {(const int16_t*)p.lhs_buffer, p.lhs_offset, p.K, p.K0, p.M0, k16, lhs8};
   UK_RETURN_IF_ERROR(launch_grid_stride(retile_planes_narrow_kernel, la, k16 * rows, s,
                                         "mmt4d digit planes (narrow lhs) launch"));
-  const RetileArgs ra = {p.rhs_buffer, p.rhs_offset, p.rhs_stride0, p.N, p.K, p.K0, k16, rhs8};
+  const RetileArgs ra = {p.rhs_buffer, p.rhs_offset, p.rhs_stride0, p.N, p.K, p.K0, k16, rhs8, 32};
   if (type == IREE_AMD_UK_FLAG_MMT4D_TYPE_S16S8S32) {
     UK_RETURN_IF_ERROR(launch_grid_stride(retile_planes_kernel<kSourceS8>, ra, p.N * k16 * 32, s,
                                           "mmt4d 8-bit rhs re-tiling launch"));
@@ -318,11 +325,18 @@ int launch_narrow(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) {
 
 int launch_mmt4d_s16_planes(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) {
   if (!mmt4d_s16_planes_supported(p.flags, p.M0, p.N0, p.K0) || p.K == 0) return IREE_AMD_UK_STATUS_NOT_FOUND;
-  if (p.M0 != 32) return launch_narrow(p, s);
   const uint32_t type = p.flags & IREE_AMD_UK_FLAG_MMT4D_TYPE_MASK;
   const bool wide_rhs = type == IREE_AMD_UK_FLAG_MMT4D_TYPE_S16S16S32;
+  if (p.M0 != 32) {
+    // narrow tiles exist for a single outer row only
+    if (p.M != 1) return IREE_AMD_UK_STATUS_NOT_FOUND;
+    if (!wide_rhs && p.M0 <= 15) return launch_narrow(p, s);
+    // 16 to 31 rows (their 2 M0 + 1 plane rows do not fit one narrow tile),
+    // and every narrow tile against a 16-bit right-hand side: the planes of
+    // the 32-row form below, rows past M0 zero; the last pass stores M0 rows
+  }
   const int64_t kk0 = p.K * p.K0;
-  if (p.M * p.N * 1024 < ceil_div(kMinMacs, kk0)) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  if (p.M * p.N * p.M0 * 32 < ceil_div(kMinMacs, kk0)) return IREE_AMD_UK_STATUS_NOT_FOUND;
   const int64_t k16 = ceil_div(kk0, (int64_t)16);
   const int64_t lhs_rows = 2 * p.M + 1, rhs_rows = wide_rhs ? 2 * p.N + 1 : p.N;
   if (lhs_rows > 0x7FFFFFFF / 64 || rhs_rows > 0x7FFFFFFF / 64) return IREE_AMD_UK_STATUS_NOT_FOUND;
@@ -341,15 +355,15 @@ int launch_mmt4d_s16_planes(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) 
   auto wide = [&](const void* buffer, int64_t offset, int64_t stride0) {
     return p.K0 % 8 == 0 && kk0 % 16 == 0 && offset % 8 == 0 && stride0 % 8 == 0 && (uintptr_t)buffer % 16 == 0;
   };
-  const RetileArgs la = {p.lhs_buffer, p.lhs_offset, p.lhs_stride0, p.M, p.K, p.K0, k16, lhs8};
-  if (wide(p.lhs_buffer, p.lhs_offset, p.lhs_stride0)) {
+  const RetileArgs la = {p.lhs_buffer, p.lhs_offset, p.lhs_stride0, p.M, p.K, p.K0, k16, lhs8, p.M0};
+  if (p.M0 == 32 && wide(p.lhs_buffer, p.lhs_offset, p.lhs_stride0)) {
     UK_RETURN_IF_ERROR(launch_grid_stride(retile_planes_s16_wide_kernel, la, p.M * k16 * 32, s,
                                           "mmt4d digit planes (lhs) launch"));
   } else {
     UK_RETURN_IF_ERROR(launch_grid_stride(retile_planes_kernel<kSourceS16>, la, p.M * k16 * 32, s,
                                           "mmt4d digit planes (lhs) launch"));
   }
-  const RetileArgs ra = {p.rhs_buffer, p.rhs_offset, p.rhs_stride0, p.N, p.K, p.K0, k16, rhs8};
+  const RetileArgs ra = {p.rhs_buffer, p.rhs_offset, p.rhs_stride0, p.N, p.K, p.K0, k16, rhs8, 32};
   const uint8_t* rhs_operand = rhs8;
   int64_t rhs_operand_stride = k16 * 512;
   if (wide_rhs) {
@@ -382,7 +396,7 @@ int launch_mmt4d_s16_planes(const iree_amd_uk_mmt4d_params_t& p, hipStream_t s) 
     UK_RETURN_IF_ERROR(iree_amd_uk_mmt4d_p(&q, s));
   }
   const CombineArgs ca = {product, p.M, p.N, rhs_rows, (uint32_t*)p.out_buffer + p.out_offset, p.out_stride0,
-                          (p.flags & IREE_AMD_UK_FLAG_MMT4D_ACCUMULATE) ? 1 : 0};
+                          (p.flags & IREE_AMD_UK_FLAG_MMT4D_ACCUMULATE) ? 1 : 0, p.M0};
   if (wide_rhs)
     return launch_grid_stride(combine_planes_kernel<true>, ca, p.M * p.N * 256, s, "mmt4d digit combine launch");
   return launch_grid_stride(combine_planes_kernel<false>, ca, p.M * p.N * 256, s, "mmt4d digit combine launch");

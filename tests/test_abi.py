@@ -151,12 +151,12 @@ def test_mmt4d_info_reports_mfma_tiles():
     assert iree_amd.mmt4d_info(32, 32, 8, F.MMT4D_TYPE_S16S16S32) == have
     assert iree_amd.mmt4d_info(32, 32, 2, F.MMT4D_TYPE_S16U4S32) == have
     assert iree_amd.mmt4d_info(16, 16, 2, F.MMT4D_TYPE_S16S16S32) == 0
-    # ... and, against an 8- or 4-bit right-hand side, at narrow tiles of up to 15 rows
-    # (the reference's own s16 x u4 tile is 1 x 32 x 8)
+    # ... and at narrow tiles of 1 to 31 rows (the reference's own s16 x u4 tile is 1 x 32 x 8)
     assert iree_amd.mmt4d_info(1, 32, 8, F.MMT4D_TYPE_S16U4S32) == have
     assert iree_amd.mmt4d_info(15, 32, 8, F.MMT4D_TYPE_S16S8S32) == have
-    assert iree_amd.mmt4d_info(16, 32, 8, F.MMT4D_TYPE_S16S8S32) == 0
-    assert iree_amd.mmt4d_info(4, 32, 8, F.MMT4D_TYPE_S16S16S32) == 0
+    assert iree_amd.mmt4d_info(16, 32, 8, F.MMT4D_TYPE_S16S8S32) == have
+    assert iree_amd.mmt4d_info(4, 32, 8, F.MMT4D_TYPE_S16S16S32) == have
+    assert iree_amd.mmt4d_info(32, 16, 8, F.MMT4D_TYPE_S16S16S32) == 0
 
 
 def test_enumerated_tiles_and_the_chooser_follow_the_reference():

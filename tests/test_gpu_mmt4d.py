@@ -165,20 +165,33 @@ def test_s16_on_the_matrix_cores_bit_exact(uk, cuda, type_flag):
     case = ukref.Mmt4dCase(rng, type_flag, 5, 6, 90, 32, 32, 8, accumulate=True, loose_strides=True, offsets=True,
                            generator=_full_range_operand)
     assert np.array_equal(gpucase.run_mmt4d(case), case.run_oracle())
-    # narrow left-hand side tiles (one outer row of 1..15 rows): the planes are the
-    # rows of one int8 tile for the narrow matrix-core kernel; an odd count of
-    # 16-wide K tiles, accumulate, offsets; a 16-bit right-hand side and 16 rows
-    # stay with the element-wise kernel
-    if type_flag != F.MMT4D_TYPE_S16S16S32:
-        assert uk.mmt4d_info(1, 32, 8, type_flag) == 1
-        for M0, N, K, K0, acc in ((1, 70, 520, 8, False), (1, 448, 512, 8, True), (4, 33, 300, 8, False),
-                                  (2, 40, 521, 8, True), (15, 10, 128, 16, False), (7, 24, 700, 2, True)):
-            for gen in (ukref.random_operand, _full_range_operand):
-                case = ukref.Mmt4dCase(rng, type_flag, 1, N, K, M0, 32, K0, accumulate=acc, offsets=acc, generator=gen)
-                got = gpucase.run_mmt4d(case, flags=case.flags & ~F.MMT4D_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION)
-                assert np.array_equal(got, case.run_oracle()), (M0, N, K, K0, acc, gen.__name__)
-    case = ukref.Mmt4dCase(rng, type_flag, 1, 64, 512, 16, 32, 8, generator=_full_range_operand)
-    assert np.array_equal(gpucase.run_mmt4d(case), case.run_oracle())
+    # narrow left-hand side tiles (one outer row of 1..31 rows). Up to 15 rows
+    # against an 8- or 4-bit right-hand side the planes are the rows of one
+    # int8 tile for the narrow matrix-core kernel; 16 to 31 rows, and every
+    # narrow tile against a 16-bit right-hand side, run as 32-row planes whose
+    # rows past M0 are zeros. An odd count of 16-wide K tiles, accumulate,
+    # offsets; the matrix-core route asserted.
+    assert uk.mmt4d_info(1, 32, 8, type_flag) == 1
+    assert uk.mmt4d_info(16, 32, 8, type_flag) == 1 and uk.mmt4d_info(31, 32, 2, type_flag) == 1
+    for M0, N, K, K0, acc in ((1, 70, 520, 8, False), (1, 448, 512, 8, True), (4, 33, 300, 8, False),
+                              (2, 40, 521, 8, True), (15, 10, 128, 16, False), (7, 24, 700, 2, True),
+                              (16, 64, 512, 8, False), (17, 40, 300, 8, True), (31, 12, 256, 16, False),
+                              (24, 33, 129, 2, True)):
+        for gen in (ukref.random_operand, _full_range_operand):
+            case = ukref.Mmt4dCase(rng, type_flag, 1, N, K, M0, 32, K0, accumulate=acc, offsets=acc, generator=gen)
+            got = gpucase.run_mmt4d(case, flags=case.flags & ~F.MMT4D_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION)
+            # (below 2^24 multiply-accumulates, 2^23 for the one-tile form, the three
+            # extra launches cost more than the element-wise kernel takes)
+            one_tile = M0 <= 15 and type_flag != F.MMT4D_TYPE_S16S16S32
+            planes = M0 * 32 * N * K * K0 >= (1 << 23 if one_tile else 1 << 24)
+            assert uk.last_kernel_path() == ("mmt4d:mfma-s16-planes" if planes else "mmt4d:element-wise"), \
+                (M0, N, K, K0, uk.last_kernel_path())
+            assert np.array_equal(got, case.run_oracle()), (M0, N, K, K0, acc, gen.__name__)
+    # two outer rows of a narrow tile, and a problem below the size threshold: the element-wise kernel
+    for M, M0, N, K in ((2, 16, 64, 512), (1, 16, 2, 8)):
+        case = ukref.Mmt4dCase(rng, type_flag, M, N, K, M0, 32, 8, generator=_full_range_operand)
+        assert np.array_equal(gpucase.run_mmt4d(case), case.run_oracle())
+        assert uk.last_kernel_path() == "mmt4d:element-wise"
     # random K0, outer counts, strides and offsets, every case above the size threshold
     for _ in range(10):
         K0 = int(rng.choice([2, 4, 6, 8, 10, 16, 24, 32])) if even else int(rng.choice([1, 2, 3, 4, 5, 8, 16, 17, 32]))
