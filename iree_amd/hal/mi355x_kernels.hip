@@ -183,15 +183,62 @@ __device__ __forceinline__ void hal_matmul_packed_rhs(const void* lhs, const voi
   mmt4d_mfma_body<Cfg, WM, WN, kRing, kSync, false, 2, 2>(a);
 }
 
+// Any other tile shape (the reference's pack and unpack take every tile size,
+// runtime/src/iree/builtins/ukernel/pack.c:254-313, unpack.c:190-247): element
+// by element over the same grid. A workgroup's block is `block_rows` rows of
+// the (padded) matrix by 32 x 16 bytes of columns; thread (row, span) moves the
+// 16 / ES elements of its span one by one to or from their places in the
+// tiles, which are stored row by row, or column by column with kTransposed.
+template <int ES, bool kPack, bool kTransposed>
+__device__ __forceinline__ void hal_pack_elementwise(const void* mat, void* tiled, int size0, int size1,
+                                                     int tile0, int tile1, uint32_t padding, uint32_t bx,
+                                                     uint32_t by, int rows_per_block, int spans_per_block) {
+  typedef typename Chunk<ES>::elem_t elem_t;
+  constexpr int CE = 16 / ES;
+  const uint32_t outer0 = ((uint32_t)size0 + tile0 - 1) / tile0, outer1 = ((uint32_t)size1 + tile1 - 1) / tile1;
+  const int64_t rows = kPack ? (int64_t)outer0 * tile0 : size0;
+  const int64_t cols = kPack ? (int64_t)outer1 * tile1 : size1;
+  const int64_t tile_elems = (int64_t)tile0 * tile1;
+  const elem_t* m_in = (const elem_t*)mat;
+  elem_t* m_out = (elem_t*)mat;
+  const elem_t* t_in = (const elem_t*)tiled;
+  elem_t* t_out = (elem_t*)tiled;
+  const int threads_per_row = 256 / rows_per_block;          // spans a row of threads covers per pass
+  const int64_t r = (int64_t)by * rows_per_block + threadIdx.x / threads_per_row;
+  if (r >= rows) return;
+  const uint32_t orow = (uint32_t)r / tile0, trow = (uint32_t)r - orow * tile0;
+  for (int sp = threadIdx.x % threads_per_row; sp < spans_per_block; sp += threads_per_row) {
+    const int64_t c0 = ((int64_t)bx * spans_per_block + sp) * CE;
+    for (int e = 0; e < CE; ++e) {
+      const int64_t c = c0 + e;
+      if (c >= cols) break;
+      const uint32_t ocol = (uint32_t)c / tile1, tcol = (uint32_t)c - ocol * tile1;
+      const int64_t at = ((int64_t)orow * outer1 + ocol) * tile_elems +
+                         (kTransposed ? (int64_t)tcol * tile0 + trow : (int64_t)trow * tile1 + tcol);
+      if (kPack) t_out[at] = (r < size0 && c < size1) ? m_in[r * size1 + c] : (elem_t)padding;
+      else m_out[r * size1 + c] = t_in[at];
+    }
+  }
+}
+
 template <int ES, bool kPack>
 __device__ __forceinline__ void hal_pack(const void* mat, void* tiled, int size0, int size1,
                                          int tile0, int tile1, uint32_t padding) {
   constexpr int CE = 16 / ES;
-  if (size0 < 1 || size1 < 1 || tile0 < 1 || tile1 < CE) return;
-  // power-of-two tiles whose rows are whole 16-byte chunks only (the geometry
-  // below is shifts); anything else does nothing
+  if (size0 < 1 || size1 < 1 || tile0 < 1 || tile1 < 1) return;
+  // Power-of-two tiles whose rows are whole 16-byte chunks: the streaming
+  // kernel (the geometry below is shifts). Any other tile: element by element
+  // over the same grid (blocks of 16 rows x 32 spans of 16 bytes).
   const int chunks = tile1 / CE;
-  if ((tile0 & (tile0 - 1)) || tile1 % CE || (chunks & (chunks - 1))) return;
+  if ((tile0 & (tile0 - 1)) || tile1 % CE || (chunks & (chunks - 1))) {
+    const int64_t outer0 = ((int64_t)size0 + tile0 - 1) / tile0, outer1 = ((int64_t)size1 + tile1 - 1) / tile1;
+    const int64_t cols = kPack ? outer1 * tile1 : (int64_t)size1, rows = kPack ? outer0 * tile0 : (int64_t)size0;
+    const uint32_t blocks_x = (uint32_t)(((cols * ES + 15) / 16 + 31) / 32), blocks_y = (uint32_t)((rows + 15) / 16);
+    if (blockIdx.x >= blocks_x * blocks_y) return;
+    hal_pack_elementwise<ES, kPack, false>(mat, tiled, size0, size1, tile0, tile1, padding, blockIdx.x % blocks_x,
+                                           blockIdx.x / blocks_x, 16, 32);
+    return;
+  }
   Pow2Args a;
   a.log2_tile_rows = __builtin_ctz((unsigned)tile0);
   const int cpr = tile1 / CE;
@@ -225,10 +272,24 @@ template <int ES, bool kPack>
 __device__ __forceinline__ void hal_pack_transpose(const void* mat, void* tiled, int size0, int size1,
                                                    int tile0, int tile1, uint32_t padding) {
   constexpr int CE = 16 / ES;
-  if (size0 < 1 || size1 < 1 || tile0 < CE || tile1 < 1) return;
-  // power-of-two tiles only (a stored row is then whole 16-byte chunks and the
-  // divisions below are a multiplication by 2^31 and a shift)
-  if ((tile0 & (tile0 - 1)) || (tile1 & (tile1 - 1))) return;
+  if (size0 < 1 || size1 < 1 || tile0 < 1 || tile1 < 1) return;
+  // Power-of-two tiles of at least 16 bytes of rows (a stored column is then
+  // whole 16-byte chunks and the divisions below are a multiplication by 2^31
+  // and a shift): the chunk kernels. Any other tile: element by element over
+  // the same grid, blocks of 64 columns x 16 groups of CE rows, a tile having
+  // ceil(tile0 / CE) groups.
+  if ((tile0 & (tile0 - 1)) || (tile1 & (tile1 - 1)) || tile0 < CE) {
+    const int64_t outer0 = ((int64_t)size0 + tile0 - 1) / tile0, outer1 = ((int64_t)size1 + tile1 - 1) / tile1;
+    const int64_t cols = kPack ? outer1 * tile1 : (int64_t)size1;
+    const int64_t rows = kPack ? outer0 * tile0 : (int64_t)size0;
+    // (rows rather than groups: 16 groups of CE rows are 16 CE rows of the padded matrix)
+    const uint32_t blocks_x = (uint32_t)((cols + 63) / 64), blocks_y = (uint32_t)((rows + 16 * CE - 1) / (16 * CE));
+    if (blockIdx.x >= blocks_x * blocks_y) return;
+    // 64 columns = 64 / CE spans of CE elements; 16 CE rows per block
+    hal_pack_elementwise<ES, kPack, true>(mat, tiled, size0, size1, tile0, tile1, padding, blockIdx.x % blocks_x,
+                                          blockIdx.x / blocks_x, 16 * CE, 64 / CE);
+    return;
+  }
   auto by_pow2 = [](int d) {
     FastDiv f;
     f.d = (uint32_t)d;

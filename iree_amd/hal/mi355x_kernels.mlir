@@ -558,7 +558,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
     hal.return %x, %c1, %c1 : index, index, index
   }
   // pack: in = matrix, out = tiles; push constants size0, size1, tile0, tile1, padding; workload (size0, size1, tile0, tile1)
-  // limits: power-of-two tiles whose rows are whole 16-byte chunks, no transposes (else nothing is written)
+  // any tile size, no transposes; power-of-two tiles whose rows are whole 16-byte chunks stream 16-byte chunks, others move single elements
   hal.executable.export public @mi355x_pack_8bit ordinal(32)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
         <0, bindings = [
@@ -585,7 +585,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
     hal.return %x, %c1, %c1 : index, index, index
   }
   // pack: in = matrix, out = tiles; push constants size0, size1, tile0, tile1, padding; workload (size0, size1, tile0, tile1)
-  // limits: power-of-two tiles whose rows are whole 16-byte chunks, no transposes (else nothing is written)
+  // any tile size, no transposes; power-of-two tiles whose rows are whole 16-byte chunks stream 16-byte chunks, others move single elements
   hal.executable.export public @mi355x_pack_16bit ordinal(33)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
         <0, bindings = [
@@ -612,7 +612,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
     hal.return %x, %c1, %c1 : index, index, index
   }
   // pack: in = matrix, out = tiles; push constants size0, size1, tile0, tile1, padding; workload (size0, size1, tile0, tile1)
-  // limits: power-of-two tiles whose rows are whole 16-byte chunks, no transposes (else nothing is written)
+  // any tile size, no transposes; power-of-two tiles whose rows are whole 16-byte chunks stream 16-byte chunks, others move single elements
   hal.executable.export public @mi355x_pack_32bit ordinal(34)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
         <0, bindings = [
@@ -639,7 +639,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
     hal.return %x, %c1, %c1 : index, index, index
   }
   // unpack: in = tiles, out = matrix; push constants size0, size1, tile0, tile1; workload (size0, size1, tile0, tile1)
-  // limits: power-of-two tiles whose rows are whole 16-byte chunks, no transposes (else nothing is written)
+  // any tile size, no transposes; power-of-two tiles whose rows are whole 16-byte chunks stream 16-byte chunks, others move single elements
   hal.executable.export public @mi355x_unpack_16bit ordinal(35)
       layout(#hal.pipeline.layout<push_constants = 4, sets = [
         <0, bindings = [
@@ -662,7 +662,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
     hal.return %x, %c1, %c1 : index, index, index
   }
   // unpack: in = tiles, out = matrix; push constants size0, size1, tile0, tile1; workload (size0, size1, tile0, tile1)
-  // limits: power-of-two tiles whose rows are whole 16-byte chunks, no transposes (else nothing is written)
+  // any tile size, no transposes; power-of-two tiles whose rows are whole 16-byte chunks stream 16-byte chunks, others move single elements
   hal.executable.export public @mi355x_unpack_32bit ordinal(36)
       layout(#hal.pipeline.layout<push_constants = 4, sets = [
         <0, bindings = [
@@ -685,7 +685,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
     hal.return %x, %c1, %c1 : index, index, index
   }
   // pack: in = matrix, out = tiles, tiles of tile0 rows x tile1 columns stored column by column; push constants size0, size1, tile0, tile1, padding; workload (size0, size1, tile0, tile1)
-  // limits: power-of-two tiles with tile0 * 1 >= 16 (else nothing is written)
+  // any tile size; power-of-two tiles with tile0 * 1 >= 16 move 16-byte chunks, others single elements
   hal.executable.export public @mi355x_pack_transpose_8bit ordinal(37)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
         <0, bindings = [
@@ -702,7 +702,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
     %bytes = arith.constant 1 : index
     %o0 = arith.ceildivui %size0, %tile0 : index
     %tile_bytes = arith.muli %tile0, %bytes : index
-    %per_tile = arith.divui %tile_bytes, %c16 : index
+    %per_tile = arith.ceildivui %tile_bytes, %c16 : index
     %groups = arith.muli %o0, %per_tile : index
     %o1 = arith.ceildivui %size1, %tile1 : index
     %cols = arith.muli %o1, %tile1 : index
@@ -712,7 +712,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
     hal.return %x, %c1, %c1 : index, index, index
   }
   // pack: in = matrix, out = tiles, tiles of tile0 rows x tile1 columns stored column by column; push constants size0, size1, tile0, tile1, padding; workload (size0, size1, tile0, tile1)
-  // limits: power-of-two tiles with tile0 * 2 >= 16 (else nothing is written)
+  // any tile size; power-of-two tiles with tile0 * 2 >= 16 move 16-byte chunks, others single elements
   hal.executable.export public @mi355x_pack_transpose_16bit ordinal(38)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
         <0, bindings = [
@@ -729,7 +729,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
     %bytes = arith.constant 2 : index
     %o0 = arith.ceildivui %size0, %tile0 : index
     %tile_bytes = arith.muli %tile0, %bytes : index
-    %per_tile = arith.divui %tile_bytes, %c16 : index
+    %per_tile = arith.ceildivui %tile_bytes, %c16 : index
     %groups = arith.muli %o0, %per_tile : index
     %o1 = arith.ceildivui %size1, %tile1 : index
     %cols = arith.muli %o1, %tile1 : index
@@ -739,7 +739,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
     hal.return %x, %c1, %c1 : index, index, index
   }
   // pack: in = matrix, out = tiles, tiles of tile0 rows x tile1 columns stored column by column; push constants size0, size1, tile0, tile1, padding; workload (size0, size1, tile0, tile1)
-  // limits: power-of-two tiles with tile0 * 4 >= 16 (else nothing is written)
+  // any tile size; power-of-two tiles with tile0 * 4 >= 16 move 16-byte chunks, others single elements
   hal.executable.export public @mi355x_pack_transpose_32bit ordinal(39)
       layout(#hal.pipeline.layout<push_constants = 5, sets = [
         <0, bindings = [
@@ -756,7 +756,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
     %bytes = arith.constant 4 : index
     %o0 = arith.ceildivui %size0, %tile0 : index
     %tile_bytes = arith.muli %tile0, %bytes : index
-    %per_tile = arith.divui %tile_bytes, %c16 : index
+    %per_tile = arith.ceildivui %tile_bytes, %c16 : index
     %groups = arith.muli %o0, %per_tile : index
     %o1 = arith.ceildivui %size1, %tile1 : index
     %cols = arith.muli %o1, %tile1 : index
@@ -766,7 +766,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
     hal.return %x, %c1, %c1 : index, index, index
   }
   // unpack: in = tiles, out = matrix, tiles of tile0 rows x tile1 columns stored column by column; push constants size0, size1, tile0, tile1; workload (size0, size1, tile0, tile1)
-  // limits: power-of-two tiles with tile0 * 2 >= 16 (else nothing is written)
+  // any tile size; power-of-two tiles with tile0 * 2 >= 16 move 16-byte chunks, others single elements
   hal.executable.export public @mi355x_unpack_transpose_16bit ordinal(40)
       layout(#hal.pipeline.layout<push_constants = 4, sets = [
         <0, bindings = [
@@ -783,7 +783,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
     %bytes = arith.constant 2 : index
     %o0 = arith.ceildivui %size0, %tile0 : index
     %tile_bytes = arith.muli %tile0, %bytes : index
-    %per_tile = arith.divui %tile_bytes, %c16 : index
+    %per_tile = arith.ceildivui %tile_bytes, %c16 : index
     %groups = arith.muli %o0, %per_tile : index
     %bx = arith.ceildivui %size1, %c64 : index
     %by = arith.ceildivui %groups, %c16 : index
@@ -791,7 +791,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
     hal.return %x, %c1, %c1 : index, index, index
   }
   // unpack: in = tiles, out = matrix, tiles of tile0 rows x tile1 columns stored column by column; push constants size0, size1, tile0, tile1; workload (size0, size1, tile0, tile1)
-  // limits: power-of-two tiles with tile0 * 4 >= 16 (else nothing is written)
+  // any tile size; power-of-two tiles with tile0 * 4 >= 16 move 16-byte chunks, others single elements
   hal.executable.export public @mi355x_unpack_transpose_32bit ordinal(41)
       layout(#hal.pipeline.layout<push_constants = 4, sets = [
         <0, bindings = [
@@ -808,7 +808,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
     %bytes = arith.constant 4 : index
     %o0 = arith.ceildivui %size0, %tile0 : index
     %tile_bytes = arith.muli %tile0, %bytes : index
-    %per_tile = arith.divui %tile_bytes, %c16 : index
+    %per_tile = arith.ceildivui %tile_bytes, %c16 : index
     %groups = arith.muli %o0, %per_tile : index
     %bx = arith.ceildivui %size1, %c64 : index
     %by = arith.ceildivui %groups, %c16 : index

@@ -81,15 +81,16 @@ def matmul_workgroup_count(name, M, N):
 
 
 # pack / unpack without transposes, by element size: name -> (bytes per element,
-# True for pack). Power-of-two tiles whose rows are whole 16-byte chunks.
+# True for pack). Any tile size; power-of-two tiles whose rows are whole
+# 16-byte chunks run the streaming kernel, others move single elements.
 PACK_EXPORTS = {"mi355x_pack_8bit": (1, True), "mi355x_pack_16bit": (2, True),
                 "mi355x_pack_32bit": (4, True), "mi355x_unpack_16bit": (2, False),
                 "mi355x_unpack_32bit": (4, False)}
 
 
 # The same with transposed inner tiles (a tile covers tile0 rows x tile1 columns
-# of the matrix and is stored column by column): power-of-two tiles with
-# tile0 * bytes >= 16.
+# of the matrix and is stored column by column): any tile size; power-of-two
+# tiles with tile0 * bytes >= 16 move 16-byte chunks, others single elements.
 PACK_TRANSPOSE_EXPORTS = {"mi355x_pack_transpose_8bit": (1, True), "mi355x_pack_transpose_16bit": (2, True),
                           "mi355x_pack_transpose_32bit": (4, True),
                           "mi355x_unpack_transpose_16bit": (2, False),
@@ -101,7 +102,7 @@ def pack_transpose_workgroup_count(name, size0, size1, tile0, tile1):
     groups of rows, a group being the 16 / bytes rows of one 16-byte chunk,
     over the padded columns (pack) or the matrix's own (unpack)."""
     es, is_pack = PACK_TRANSPOSE_EXPORTS[name]
-    groups = -(-size0 // tile0) * (tile0 * es // 16)
+    groups = -(-size0 // tile0) * -(-tile0 * es // 16)
     cols = -(-size1 // tile1) * tile1 if is_pack else size1
     return -(-cols // 64) * -(-groups // 16)
 
@@ -111,7 +112,7 @@ def pack_workgroup_count(name, size0, size1, tile0, tile1):
     over the padded extent (pack) or the matrix itself (unpack)."""
     es, is_pack = PACK_EXPORTS[name]
     if is_pack:
-        cols = -(-size1 // tile1) * tile1 * es // 16
+        cols = -(-(-(-size1 // tile1) * tile1 * es) // 16)
         rows = -(-size0 // tile0) * tile0
     else:
         cols = -(-size1 * es // 16)
@@ -313,7 +314,7 @@ _MLIR_MATMUL_EXPORT = """\
 
 _MLIR_PACK_EXPORT = """\
   // {what}; push constants size0, size1, tile0, tile1{extra}; workload (size0, size1, tile0, tile1)
-  // limits: power-of-two tiles whose rows are whole 16-byte chunks, no transposes (else nothing is written)
+  // any tile size, no transposes; power-of-two tiles whose rows are whole 16-byte chunks stream 16-byte chunks, others move single elements
   hal.executable.export public @{name} ordinal({ordinal})
       layout(#hal.pipeline.layout<push_constants = {constants}, sets = [
         <0, bindings = [
@@ -339,7 +340,7 @@ _MLIR_PACK_EXPORT = """\
 
 _MLIR_PACK_TRANSPOSE_EXPORT = """\
   // {what}, tiles of tile0 rows x tile1 columns stored column by column; push constants size0, size1, tile0, tile1{extra}; workload (size0, size1, tile0, tile1)
-  // limits: power-of-two tiles with tile0 * {es} >= 16 (else nothing is written)
+  // any tile size; power-of-two tiles with tile0 * {es} >= 16 move 16-byte chunks, others single elements
   hal.executable.export public @{name} ordinal({ordinal})
       layout(#hal.pipeline.layout<push_constants = {constants}, sets = [
         <0, bindings = [
@@ -356,7 +357,7 @@ _MLIR_PACK_TRANSPOSE_EXPORT = """\
     %bytes = arith.constant {es} : index
     %o0 = arith.ceildivui %size0, %tile0 : index
     %tile_bytes = arith.muli %tile0, %bytes : index
-    %per_tile = arith.divui %tile_bytes, %c16 : index
+    %per_tile = arith.ceildivui %tile_bytes, %c16 : index
     %groups = arith.muli %o0, %per_tile : index
 {extent}    %bx = arith.ceildivui {cols}, %c64 : index
     %by = arith.ceildivui %groups, %c16 : index
