@@ -154,7 +154,7 @@ def test_unpack_with_line_aligned_stores_every_row_alignment(uk, cuda, type_flag
     rng = np.random.default_rng(rows * 7 + cols)
     o0, o1 = -(-rows // t0), -(-cols // t1)
     for to in (0, 1):
-        for extra_pitch, out_offset in ((0, 0), (1, 3), (5, 64), (37, 1), (64, 17)):
+        for extra_pitch, out_offset in ((0, 0), (0, 3), (0, 17), (0, 63), (1, 3), (5, 64), (37, 1), (64, 17)):
             case = ukref.UnpackCase(rng, type_flag, o0, o1, t0, t1, transpose_outer=to, out_size=(rows, cols))
             case.out_stride0 = cols + extra_pitch
             case.out_offset = out_offset
