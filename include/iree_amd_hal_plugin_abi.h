@@ -42,12 +42,41 @@ typedef struct iree_amd_hal_status_handle_t* iree_amd_hal_plugin_status_t;
 #define iree_amd_hal_plugin_status_from_code(code) \
   ((iree_amd_hal_plugin_status_t)((uintptr_t)(code) & 0x1Fu))
 
+/* Sanitizer the plugin was compiled with (executable_plugin.h:76-100); the
+ * runtime refuses a plugin whose sanitizer it was not built with itself. */
+#define IREE_AMD_HAL_PLUGIN_SANITIZER_NONE 0
+#define IREE_AMD_HAL_PLUGIN_SANITIZER_ADDRESS 1
+#define IREE_AMD_HAL_PLUGIN_SANITIZER_MEMORY 2
+#define IREE_AMD_HAL_PLUGIN_SANITIZER_THREAD 3
+#define IREE_AMD_HAL_PLUGIN_SANITIZER_UNDEFINED 4
+/* The kind in force for the translation unit that includes this header, for
+ * the header's `sanitizer` field (executable_plugin.h:102-121): clang reports
+ * it through __has_feature, gcc through __SANITIZE_ADDRESS__ / _THREAD__. */
+#if defined(__has_feature)
+#if __has_feature(address_sanitizer)
+#define IREE_AMD_HAL_PLUGIN_SANITIZER_KIND IREE_AMD_HAL_PLUGIN_SANITIZER_ADDRESS
+#elif __has_feature(memory_sanitizer)
+#define IREE_AMD_HAL_PLUGIN_SANITIZER_KIND IREE_AMD_HAL_PLUGIN_SANITIZER_MEMORY
+#elif __has_feature(thread_sanitizer)
+#define IREE_AMD_HAL_PLUGIN_SANITIZER_KIND IREE_AMD_HAL_PLUGIN_SANITIZER_THREAD
+#endif
+#endif
+#if !defined(IREE_AMD_HAL_PLUGIN_SANITIZER_KIND) && defined(__SANITIZE_ADDRESS__)
+#define IREE_AMD_HAL_PLUGIN_SANITIZER_KIND IREE_AMD_HAL_PLUGIN_SANITIZER_ADDRESS
+#endif
+#if !defined(IREE_AMD_HAL_PLUGIN_SANITIZER_KIND) && defined(__SANITIZE_THREAD__)
+#define IREE_AMD_HAL_PLUGIN_SANITIZER_KIND IREE_AMD_HAL_PLUGIN_SANITIZER_THREAD
+#endif
+#if !defined(IREE_AMD_HAL_PLUGIN_SANITIZER_KIND)
+#define IREE_AMD_HAL_PLUGIN_SANITIZER_KIND IREE_AMD_HAL_PLUGIN_SANITIZER_NONE
+#endif
+
 typedef struct iree_amd_hal_plugin_header_t {
   uint32_t version;
   const char* name;
   const char* description;
   uint32_t features;
-  int32_t sanitizer; /* 0 = none */
+  int32_t sanitizer; /* IREE_AMD_HAL_PLUGIN_SANITIZER_* */
   uint64_t reserved[8];
 } iree_amd_hal_plugin_header_t;
 

@@ -252,7 +252,7 @@ iree_hal_executable_plugin_query(uint32_t max_version, void* reserved) {
       .name = "mi355x_uk",
       .description = "MI355X (gfx950) data-tiled matmul microkernels: iree_uk_mmt4d / pack / unpack",
       .features = 0, /* not standalone: opens a shared library and the GPU driver */
-      .sanitizer = 0,
+      .sanitizer = IREE_AMD_HAL_PLUGIN_SANITIZER_KIND,
   };
   static const iree_amd_hal_plugin_v0_t plugin = {
       .header = &header,

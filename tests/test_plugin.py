@@ -126,6 +126,29 @@ def test_query_reports_version_and_refuses_newer_hosts(host):
     assert not host.query(2)                                 # host asks for a newer interface
 
 
+@pytest.mark.parametrize("flags,kind", [([], 0), (["-fsanitize=address"], 1), (["-fsanitize=thread"], 3)])
+def test_header_names_the_sanitizer_it_was_compiled_with(flags, kind):
+    """The header's sanitizer field is whatever the compiler says is in force
+    for the plugin's translation unit (the reference runtime refuses a plugin
+    built with a sanitizer it does not run itself,
+    runtime/src/iree/hal/local/executable_plugin.h:76-121): the macro the
+    plugin initialises the field with, expanded by the preprocessor under each
+    sanitizer switch."""
+    import shutil
+    import subprocess
+    include = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include")
+    src = '#include "iree_amd_hal_plugin_abi.h"\nKIND_IS IREE_AMD_HAL_PLUGIN_SANITIZER_KIND\n'
+    compilers = [c for c in ("gcc", "/opt/rocm/llvm/bin/clang") if shutil.which(c)]
+    assert compilers
+    for cc in compilers:
+        out = subprocess.run([cc, "-E", "-P", "-x", "c", "-I", include, *flags, "-"], input=src, text=True,
+                             capture_output=True, check=True).stdout
+        line = [l for l in out.splitlines() if l.startswith("KIND_IS")][0]
+        assert line.split()[1] == str(kind), (cc, flags, line)
+    with open(os.path.join(os.path.dirname(PLUGIN), "mi355x_uk_plugin.c")) as f:
+        assert ".sanitizer = IREE_AMD_HAL_PLUGIN_SANITIZER_KIND" in f.read()
+
+
 def test_load_resolve_unload_protocol(host):
     plugin = host.query().contents
     status, self_ptr = host.load(plugin, [(b"uk_library", _lib.library_path().encode())])
