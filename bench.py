@@ -39,7 +39,7 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # x 1.0): 192 MiB read (each of the 8 XCD L2s fetches its own operand panels,
 # 12 panels of 2 MiB each: most of it is served by the 256 MiB memory-side
 # cache; 192-212 MiB from run to run) + 64 MiB written.
-MEASURED_TRAFFIC_BYTES = {"mmt4d_f16_4096": 268.7e6}
+MEASURED_TRAFFIC_BYTES = {"mmt4d_f16_4096": 268.8e6}
 
 
 # After an idle spell (or CPU-only work) the GPU's power management needs about
@@ -61,7 +61,7 @@ def parse_args():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--only", default="", help="run only the named kernel in a loop (for profilers): "
                     "mmt4d_f16 | mmt4d_f16_acc | mmt4d_i8 | mmt4d_s16s8 | mmt4d_s16s16 | mmt4d_fp8 | mmt4d_f16_ksplit | mlp_fp8 | pack | unpack | "
-                    "pack_transpose | unpack_transpose | dequant_i4[_m8|_m32] | dequant_i4_reassoc[_m8|_m32] | batch_mmt4d_f16 | "
+                    "pack_transpose | unpack_transpose | dequant_i4[_k11008|_k5120][_m8|_m32] | dequant_i4_reassoc[_m8|_m32] | batch_mmt4d_f16 | "
                     "batch_mmt4d_f16_narrow | mmt4d_f16_narrow_m1 | mmt4d_f16_narrow_m8 | mmt4d_f16_narrow_n8 | "
                     "matmul_rowmajor_lhs_f16 | matmul_rowmajor_lhs_i8 | matmul_rowmajor_lhs_fp8 | matmul_rowmajor_lhs_f16_m8 | "
                     "chain_i8_1024 | copy | copy_rotating | copy_rotating_nt | copy_rotating_nt_single_waves | read_only_29mb")
@@ -865,6 +865,10 @@ def run_only(args, torch, iree_amd, F, synth, mm_step):
         fn = lambda: iree_amd.mmt4d(l8, r8, o8, M1, N1, K1, 32, 32, 16, F.MMT4D_TYPE_F8E4M3F8E4M3F32)  # noqa: E731
     elif args.only.startswith("dequant_i4"):
         Nq, Kq, gs = 14336, 4096, 128
+        if "_k11008" in args.only:
+            Nq, Kq = 4096, 11008
+        elif "_k5120" in args.only:
+            Nq, Kq = 11264, 5120
         G = Kq // gs
         Mq = 32 if args.only.endswith("_m32") else 8 if args.only.endswith("_m8") else 1
         qflags = F.DEQUANT_MATMUL_ZP_U4 | F.DEQUANT_MATMUL_W_TILED
