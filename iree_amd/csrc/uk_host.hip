@@ -21,6 +21,7 @@
 // busy at the same time with a thread for each.
 #include "uk_common.h"
 
+#include <algorithm>
 #include <condition_variable>
 #include <deque>
 #include <mutex>
@@ -209,14 +210,24 @@ class SlotLease {
         }
       }
       if (on_device < kMaxSlots) {
+        // The new slot is entered as busy first and set up (a stream is
+        // created) with the pool unlocked, so other threads' calls do not
+        // wait behind the driver.
         HostSlot* s = new HostSlot();
-        const int st = s->init();
-        if (st) {
-          delete s;
-          return st;
-        }
+        s->device = device;
         s->busy = true;
         pool_->slots.push_back(s);
+        lock.unlock();
+        const int st = s->init();
+        if (st) {
+          lock.lock();
+          auto& v = pool_->slots;
+          v.erase(std::remove(v.begin(), v.end(), s), v.end());
+          lock.unlock();
+          delete s;
+          pool_->freed.notify_all();
+          return st;
+        }
         slot_ = s;
         return 0;
       }
