@@ -36,7 +36,15 @@ PACK_CASES = [
     ("pack_vnni_rhs_large", "i8", 256, 512, 2, 16, True, True, None),
     ("pack_vnni_lhs_large_with_pad", "i8", 127, 255, 16, 2, False, False, 0),
     ("pack_vnni_rhs_large_with_pad", "i8", 255, 511, 2, 16, True, True, 0),
+    # tests/e2e/regression/pack_pad_transpose_1x9_into_2x4x8x4_issue_12546.mlir: a 1 x 9 row of
+    # 1..9 into 2x4x8x4 with both transposes (matrix tiles of 4 rows x 8 columns) and padding 0,
+    # the result written out in the file: the nine values head the columns of the first tiles
+    ("pack_pad_transpose_1x9_into_2x4x8x4", "i8", 1, 9, 4, 8, True, True, 0),
 ]
+
+# Result tensors with more outer tiles than the source needs (whole tiles of
+# padding): name -> (outer rows, outer columns) in matrix orientation.
+PACK_OUTER = {"pack_pad_transpose_1x9_into_2x4x8x4": (4, 2)}
 
 PACK_LITERALS = {
     "pack_simple": [[[[0, 1], [4, 5]], [[2, 3], [6, 7]]], [[[8, 9], [12, 13]], [[10, 11], [14, 15]]]],
@@ -71,7 +79,16 @@ UNPACK_LITERALS = {
 NP = {"i32": np.int32, "i8": np.int8}
 
 
+def _issue_12546_result():
+    out = np.zeros((2, 4, 8, 4), dtype=np.int8)
+    out[0, 0, :, 0] = np.arange(1, 9)
+    out[1, 0, 0, 0] = 9
+    return out
+
+
 def pack_source(elem, rows, cols):
+    if (elem, rows, cols) == ("i8", 1, 9):
+        return np.arange(1, 10, dtype=np.int8).reshape(1, 9)
     lin = np.arange(rows * cols, dtype=np.int64).reshape(rows, cols)
     return (lin % 256).astype(np.uint8).view(np.int8) if elem == "i8" else lin.astype(np.int32)
 
@@ -82,6 +99,8 @@ def pack_expected(name, src, tr, tc, ti, to, padding):
     columns) and linalg.transpose into the result's order."""
     if name in PACK_LITERALS:
         return np.array(PACK_LITERALS[name], dtype=src.dtype)
+    if name == "pack_pad_transpose_1x9_into_2x4x8x4":
+        return _issue_12546_result()
     rows, cols = src.shape
     o0, o1 = -(-rows // tr), -(-cols // tc)
     padded = np.full((o0 * tr, o1 * tc), 0 if padding is None else padding, dtype=src.dtype)

@@ -13,7 +13,8 @@ PACK_FLAG = {"i32": F.PACK_TYPE_I32I32, "i8": F.PACK_TYPE_I8I8}
 
 def make_pack_case(name, elem, rows, cols, tr, tc, ti, to, padding):
     src = T.pack_source(elem, rows, cols)
-    case = ukref.PackCase(np.random.default_rng(1), PACK_FLAG[elem], -(-rows // tr), -(-cols // tc), tr, tc,
+    o0, o1 = T.PACK_OUTER.get(name, (-(-rows // tr), -(-cols // tc)))
+    case = ukref.PackCase(np.random.default_rng(1), PACK_FLAG[elem], o0, o1, tr, tc,
                           transpose_inner=ti, transpose_outer=to, in_size=(rows, cols))
     case.inp = np.ascontiguousarray(src).reshape(-1).view(case.dtype).copy()
     case.padding_value = 0 if padding is None else padding
