@@ -301,9 +301,9 @@ __global__ __launch_bounds__(256) void pack_transpose_lds_kernel(TransArgs a) {
   pack_transpose_lds_body<ES, kLdsUnroll>(a);
 }
 
-template <int ES>
+template <int ES, int kLX, bool kNt = false>
 __global__ __launch_bounds__(64) void unpack_transpose_block_kernel(TransArgs a) {
-  unpack_transpose_block_body<ES>(a);
+  unpack_transpose_block_body<ES, kLX, kNt>(a);
 }
 
 template <int ES>
@@ -313,11 +313,20 @@ int launch_unpack_transpose(TransArgs a, hipStream_t s) {
   // kernel that moves a CE x CE block per lane, one wave per workgroup.
   constexpr int CE = 16 / ES;
   if (a.tile_cols % CE == 0 && cols >= 16 * CE) {
-    const int64_t bx = ceil_div(cols, (int64_t)16 * CE);
-    const int64_t by = ceil_div(a.row_groups, (int64_t)4);
+    // Tiles of 8 row groups and more (stored columns of at least 128 bytes): a
+    // wave takes 8 blocks across and 8 row groups, so that it consumes whole
+    // lines of the stored columns by itself (16 across and 4 row groups leave
+    // the other half of every line to another wave, and a line that two waves
+    // load non-temporally comes from memory twice: 1.15 x the traffic). f32
+    // 4096 x 4096 from 32x32 tiles: 27.1 -> 24.3 us.
+    const bool tall = a.groups_per_tile % 8 == 0;
+    const int lx = tall ? 8 : 16, gy = 64 / lx;
+    const int64_t bx = ceil_div(cols, (int64_t)lx * CE);
+    const int64_t by = ceil_div(a.row_groups, (int64_t)gy);
     if (bx >= 1 && by >= 1 && bx * by <= 0x7FFFFFFF) {
       a.blocks_x = (uint32_t)bx; a.blocks_y = (uint32_t)by;
-      hipLaunchKernelGGL((unpack_transpose_block_kernel<ES>), dim3((unsigned)(bx * by)), dim3(64), 0, s, a);
+      if (tall) hipLaunchKernelGGL((unpack_transpose_block_kernel<ES, 8>), dim3((unsigned)(bx * by)), dim3(64), 0, s, a);
+      else hipLaunchKernelGGL((unpack_transpose_block_kernel<ES, 16>), dim3((unsigned)(bx * by)), dim3(64), 0, s, a);
       return check_hip(hipGetLastError(), "unpack_transpose launch");
     }
   }

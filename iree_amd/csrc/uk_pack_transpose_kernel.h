@@ -379,11 +379,15 @@ __device__ __forceinline__ void unpack_transpose_body(const TransArgs& a) {
 // whole CE columns (the host checks). Measured, f32 4096 x 4096 from 32x32
 // tiles stored column by column: 31.7 us with the kernel above, 27.0 with
 // this one; with two quartets per wave 31.0, as four waves per workgroup
-// 32.9, non-temporal stores 27.9, ordinary loads 28.5.
-template <int ES>
+// 32.9, non-temporal stores 27.9, ordinary loads 28.5. kLX = 8: 8 blocks
+// across and 8 row groups per wave, for tiles of 8 row groups and more, whose
+// stored columns are whole 128-byte lines that the wave then reads alone:
+// 24.3 us (25.7 with non-temporal stores).
+template <int ES, int kLX = 16, bool kNtStore = false>
 __device__ __forceinline__ void unpack_transpose_block_body(const TransArgs& a) {
-  constexpr int kU = 1, kWavesPerGroup = 1;
-  constexpr bool kNtStore = false, kNtLoad = true;
+  // kLX blocks across and kGY = 64 / kLX row groups per wave
+  constexpr int kU = 1, kWavesPerGroup = 1, kGY = 64 / kLX;
+  constexpr bool kNtLoad = true;
   static_assert(ES == 2 || ES == 4, "results are 16- or 32-bit");
   constexpr int CE = 16 / ES;
   typedef typename Chunk<ES>::elem_t elem_t;
@@ -400,10 +404,10 @@ __device__ __forceinline__ void unpack_transpose_block_body(const TransArgs& a) 
     by = logical / a.blocks_x;
     bx = logical - by * a.blocks_x;
   }
-  const uint32_t lc = lane & 15, lg = lane >> 4;
+  const uint32_t lc = lane % kLX, lg = lane / kLX;
   const int64_t cols = a.m_size1 < a.padded_cols ? a.m_size1 : a.padded_cols;
-  const int64_t c = ((int64_t)bx * 16 + lc) * CE;              // first of this lane's CE columns
-  const int64_t g0 = ((int64_t)by * kWavesPerGroup + wave) * 4 * kU;   // first row group of this wave
+  const int64_t c = ((int64_t)bx * kLX + lc) * CE;             // first of this lane's CE columns
+  const int64_t g0 = ((int64_t)by * kWavesPerGroup + wave) * kGY * kU;   // first row group of this wave
   if (g0 >= a.row_groups || c >= cols) return;
   const uint32_t cc = (uint32_t)c;
   const uint32_t ocol = a.by_tile_cols.div(cc), d2 = cc - ocol * a.tile_cols;
@@ -440,19 +444,19 @@ __device__ __forceinline__ void unpack_transpose_block_body(const TransArgs& a) 
   // Interior waves (all 16 blocks across lie inside the matrix, all row groups
   // exist and end inside it): straight-line code, every load issued before the
   // first store.
-  const bool interior = ((int64_t)bx * 16 + 16) * CE <= cols && g0 + 4 * kU <= a.row_groups &&
-                        (g0 + 4 * kU) * CE <= a.m_size0;
+  const bool interior = ((int64_t)bx * kLX + kLX) * CE <= cols && g0 + kGY * kU <= a.row_groups &&
+                        (g0 + kGY * kU) * CE <= a.m_size0;
   if (interior) {
 #pragma unroll
     for (int u = 0; u < kU; ++u) {
-      const char* src = source_of(g0 + u * 4 + lg);
+      const char* src = source_of(g0 + u * kGY + lg);
 #pragma unroll
       for (int j = 0; j < CE; ++j)
         v[u][j] = kNtLoad ? __builtin_nontemporal_load((const u32x4*)(src + j * col_pitch)) : *(const u32x4*)(src + j * col_pitch);
     }
 #pragma unroll
     for (int u = 0; u < kU; ++u) {
-      char* p = dst + (g0 + u * 4 + lg) * CE * a.m_pitch_bytes;
+      char* p = dst + (g0 + u * kGY + lg) * CE * a.m_pitch_bytes;
 #pragma unroll
       for (int i = 0; i < CE; ++i) {
         if (kNtStore) __builtin_nontemporal_store((mat_vec_t)block_row(v[u], i), (mat_vec_t*)(p + i * a.m_pitch_bytes));
@@ -463,7 +467,7 @@ __device__ __forceinline__ void unpack_transpose_block_body(const TransArgs& a) 
   }
 #pragma unroll 1
   for (int u = 0; u < kU; ++u) {
-    const int64_t g = g0 + u * 4 + lg;
+    const int64_t g = g0 + u * kGY + lg;
     if (g >= a.row_groups) continue;
     const char* src = source_of(g);
 #pragma unroll

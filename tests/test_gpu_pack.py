@@ -119,6 +119,10 @@ def test_transposing_pack_with_ragged_edges(uk, cuda, type_flag, tr, tc, rows, c
     (F.UNPACK_TYPE_F32F32, 32, 4, 77, 64),       # exactly one wave of blocks across
     (F.UNPACK_TYPE_I32I32, 32, 16, 1030, 1000),  # row groups past the matrix in the last quartet
     (F.UNPACK_TYPE_BF16BF16, 32, 32, 511, 515),
+    # stored columns of 128 bytes and more: a wave takes 8 row groups and 8 blocks across
+    (F.UNPACK_TYPE_F32F32, 64, 32, 333, 1001),
+    (F.UNPACK_TYPE_F16F16, 64, 16, 1000, 130),
+    (F.UNPACK_TYPE_I32I32, 32, 32, 4100, 37),
 ])
 def test_transposing_unpack_with_ragged_edges(uk, cuda, type_flag, tr, tc, rows, cols):
     """Unpacks of tiles stored column by column (matrix tiles of tr rows x tc
