@@ -253,15 +253,15 @@ __global__ __launch_bounds__(kStreamThreads) void unpack_stream_kernel(StreamArg
   }
 }
 
-template <int ES, bool kPack>
+template <int ES, bool kPack, int kRows = kPow2Rows>
 __global__ __launch_bounds__(kPow2Waves * 64) void stream_pow2_kernel(Pow2Args a) {
-  stream_pow2_body<ES, kPack>(a);
+  stream_pow2_body<ES, kPack, true, kPack, kRows>(a);
 }
 
 // The 32-bit per-lane offsets of stream_pow2_kernel must not overflow.
 bool pow2_eligible(const StreamArgs& a, int es) {
   if (!a.pow2) return false;
-  const int64_t rows = kPow2Rows * kPow2Unroll;
+  const int64_t rows = 8 * kPow2Unroll;      // (the taller of the two block shapes)
   const int64_t pitch = a.m_stride0 * es;
   if (pitch * rows + 256 >= (1ll << 31)) return false;
   const int64_t panels = rows / a.tile_rows + 2, cols = (64 / kPow2Rows) / a.cpr + 2;
@@ -282,11 +282,23 @@ int launch_stream_pow2(const StreamArgs& a, hipStream_t s) {
   p.padding = a.padding;
   const int64_t cols = kPack ? a.padded_chunks_per_row : a.chunks_per_row;
   const int64_t rows = kPack ? a.padded_rows : a.m_size0;
-  const int64_t bx = ceil_div(cols, kPow2WavesX * (64 / kPow2Rows));
-  const int64_t by = ceil_div(rows, kPow2Rows * kPow2Unroll * (kPow2Waves / kPow2WavesX));
+  // Tiles whose rows are a single chunk (f16 32x8, i8 32x16, f32 32x4: the
+  // operand tiles of mmt4d): 8 rows x 8 chunks per wave, so that the wave's
+  // piece of a tile is a whole 128-byte line (4 rows x 16 chunks leave half of
+  // each line to the wave below, and both sides are accessed non-temporally).
+  // Measured (TB/s, 4 rows x 16 chunks -> 8 x 8): pack i8 8192^2 into 32x16
+  // 4.75 -> 5.62, f16 8192 x 4096 into 32x8 4.75 -> 5.62, f32 4096^2 into 32x4
+  // 4.50 -> 5.55; unpack f16 from 32x8 5.65 -> 6.09 (8191 x 5001: 5.02 -> 5.20).
+  const bool tall = a.cpr == 1 && a.tile_rows >= 8;
+  const int block_rows = tall ? 8 : kPow2Rows;
+  const int64_t bx = ceil_div(cols, kPow2WavesX * (64 / block_rows));
+  const int64_t by = ceil_div(rows, block_rows * kPow2Unroll * (kPow2Waves / kPow2WavesX));
   if (bx < 1 || by < 1 || bx * by > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
   p.blocks_x = (uint32_t)bx; p.blocks_y = (uint32_t)by;
-  hipLaunchKernelGGL((stream_pow2_kernel<ES, kPack>), dim3((unsigned)(bx * by)), dim3(kPow2Waves * 64), 0, s, p);
+  if (tall)
+    hipLaunchKernelGGL((stream_pow2_kernel<ES, kPack, 8>), dim3((unsigned)(bx * by)), dim3(kPow2Waves * 64), 0, s, p);
+  else
+    hipLaunchKernelGGL((stream_pow2_kernel<ES, kPack>), dim3((unsigned)(bx * by)), dim3(kPow2Waves * 64), 0, s, p);
   return check_hip(hipGetLastError(), "stream_pow2 launch");
 }
 
@@ -431,6 +443,10 @@ template <int ES>
 int launch_unpack_aligned(const StreamArgs& a, hipStream_t s) {
   const int64_t row_bytes = a.m_size1 * ES;
   // (32-bit offsets per lane: the same limits as the other power-of-two kernel)
+  // (tiles whose rows are a single chunk: 4 rows of one tile are half a line,
+  // the other kernel's 8-row blocks read whole ones: 6.09 against 5.41 TB/s
+  // for f16 8192 x 4096 from 32x8 tiles)
+  if (a.cpr == 1) return IREE_AMD_UK_STATUS_NOT_FOUND;
   if (!pow2_eligible(a, ES) || row_bytes < 1024 || row_bytes + 512 >= (1ll << 31) || a.m_size0 < 1 ||
       a.m_stride0 * ES * 16 + row_bytes + 512 >= (1ll << 31))
     return IREE_AMD_UK_STATUS_NOT_FOUND;
