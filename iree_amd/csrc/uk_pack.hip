@@ -447,6 +447,14 @@ int launch_unpack_aligned(const StreamArgs& a, hipStream_t s) {
   // the other kernel's 8-row blocks read whole ones: 6.09 against 5.41 TB/s
   // for f16 8192 x 4096 from 32x8 tiles)
   if (a.cpr == 1) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  // Tile rows of 64 bytes and more: the other kernel's row pieces are then long
+  // runs on the tiled side as well (4 rows x 256 bytes of a 32x32 f32 tile are
+  // 512 contiguous bytes), and it measures faster than this one, whose windows
+  // cut tile rows at arbitrary chunks: f32 4096^2 from 32x32 tiles 5.94 against
+  // 5.60 TB/s (4095 x 4099: 6.03 against 5.44), f16 8192 x 4096 from 32x32
+  // 6.10 against 5.79. With 32-byte tile rows (f16 32x16) this kernel wins:
+  // 6.08 against 5.57 (8191 x 5001: 5.77 against 5.39).
+  if (a.cpr >= 4) return IREE_AMD_UK_STATUS_NOT_FOUND;
   if (!pow2_eligible(a, ES) || row_bytes < 1024 || row_bytes + 512 >= (1ll << 31) || a.m_size0 < 1 ||
       a.m_stride0 * ES * 16 + row_bytes + 512 >= (1ll << 31))
     return IREE_AMD_UK_STATUS_NOT_FOUND;

@@ -147,6 +147,9 @@ def test_transposing_unpack_with_ragged_edges(uk, cuda, type_flag, tr, tc, rows,
     (F.UNPACK_TYPE_F32F32, 32, 32, 45, 777),
     (F.UNPACK_TYPE_I32I32, 32, 32, 130, 257),
     (F.UNPACK_TYPE_F32F32, 16, 4, 33, 1030),
+    # (that kernel serves tile rows of 32 bytes; the other shapes here take the kernels around it)
+    (F.UNPACK_TYPE_F32F32, 32, 8, 50, 1000),
+    (F.UNPACK_TYPE_BF16BF16, 16, 16, 37, 3000),
 ])
 def test_unpack_with_line_aligned_stores_every_row_alignment(uk, cuda, type_flag, t0, t1, rows, cols):
     """Rows of 1 KiB and more in power-of-two tiles run the unpack kernel whose
