@@ -228,6 +228,7 @@ int make_args(const iree_amd_uk_mmt4d_params_t& p, int out_elem_bytes, bool silu
   a.k_slices = 0; a.slice_ksteps = 0; a.slice_out_bytes = 0;
   a.batch = 1; a.lhs_batch_bytes = a.rhs_batch_bytes = a.out_batch_bytes = 0;
   a.batch_by_xcd = 0;
+  a.stream_out = p.M * p.N * 1024 * out_elem_bytes > (32ll << 20);
   a.accumulate = (p.flags & IREE_AMD_UK_FLAG_MMT4D_ACCUMULATE) != 0;
   a.k0_div = sv.mfma_k / p.K0;
   a.row_major_out = 0; a.out_rows = a.out_cols = 0;
@@ -283,6 +284,7 @@ int launch_planes(const iree_amd_uk_mmt4d_params_t& p, MfmaArgs a, int64_t batch
   for (int64_t b0 = 0; b0 < batch; b0 += kPlanes) {
     MfmaArgs c = a;
     c.batch = (int)(batch - b0 < kPlanes ? batch - b0 : kPlanes);
+    c.stream_out = p.M * p.N * 1024 * (int64_t)ti.out_bytes * c.batch > (32ll << 20);
     c.lhs = a.lhs + b0 * a.lhs_batch_bytes;
     c.rhs = a.rhs + b0 * a.rhs_batch_bytes;
     c.out = a.out + b0 * a.out_batch_bytes;

@@ -98,6 +98,8 @@ struct MfmaArgs {
   int64_t lhs_batch_bytes, rhs_batch_bytes, out_batch_bytes;
   // this many leading planes are dealt to the XCDs whole (see the __global__ wrapper)
   int batch_by_xcd;
+  // the tiled result is larger than the L2s together: write it past the caches
+  int stream_out;
 };
 
 namespace {
@@ -191,8 +193,11 @@ __device__ __forceinline__ void tile_coord(int bid, int tiles_m, int tiles_n,
 // sums of a K split). (An instance compiled for one form has constant step sizes
 // in its loop and one epilogue: measured 2 % (f16) to 6 % (i8) faster at 4096^3
 // than one that reads the form from its arguments.)
+// kStreamOut: the tiled result is not read again soon and may be written past
+// the caches (off for the partial sums of a K split, which the reduction
+// kernel reads next).
 template <typename Cfg, int WM, int WN, int kRing, int kSync, bool kSiluMul = false, int kWavesN = 2,
-          int kForm = 0>
+          int kForm = 0, bool kStreamOut = true>
 __device__ __forceinline__ void mmt4d_mfma_body(const MfmaArgs a, const int bid = blockIdx.x) {
   static_assert(kForm >= 0 && kForm <= 3 && (!kSiluMul || kForm == 0), "unknown operand form");
   constexpr bool lhs_row_major = kForm >= 2;
@@ -707,8 +712,24 @@ __device__ __forceinline__ void mmt4d_mfma_body(const MfmaArgs a, const int bid 
       if (i < a.M && j < a.N) {
         out_t* t = (out_t*)(a.out + (int64_t)i * a.out_stride_bytes) + (int64_t)j * 1024 +
                    (bi % kPerTile) * R * 32 + (bj % kPerTile) * R;
+        // 32-row blocks write whole 128-byte lines per instruction; a result
+        // larger than the L2s goes past the caches (i8 4096^3: 65.3 -> 64.4 us,
+        // fp8 56.65 -> 56.4); the 64-byte row pieces of 16-row blocks lose that
+        // way (f16 110.4 -> 114.9), and a small result is what the next kernel
+        // reads.
+        bool streamed = false;
+        if constexpr (R == 32 && kStreamOut) {
+          if (a.stream_out) {
+            streamed = true;
 #pragma unroll
-        for (int v = 0; v < kAccRegs; ++v) t[acc_row(v) * 32 + acc_col] = acc[x][y][v];
+            for (int v = 0; v < kAccRegs; ++v)
+              __builtin_nontemporal_store((out_t)acc[x][y][v], &t[acc_row(v) * 32 + acc_col]);
+          }
+        }
+        if (!streamed) {
+#pragma unroll
+          for (int v = 0; v < kAccRegs; ++v) t[acc_row(v) * 32 + acc_col] = acc[x][y][v];
+        }
       }
     }
 }

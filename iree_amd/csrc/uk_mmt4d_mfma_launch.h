@@ -72,7 +72,7 @@ __global__ __launch_bounds__(128 * kWavesN, kOcc) void mmt4d_mfma_ksplit_kernel(
     a.ksteps = a.slice_ksteps;
     a.tail_tiles = 0;
   }
-  mmt4d_mfma_body<Cfg, WM, WN, kRing, kSync, false, kWavesN, kForm>(a);
+  mmt4d_mfma_body<Cfg, WM, WN, kRing, kSync, false, kWavesN, kForm, false>(a);
 }
 
 template <typename Cfg, int WM, int WN, int kRing, int kSync, int kOcc, bool kSiluMul, int kWavesN,

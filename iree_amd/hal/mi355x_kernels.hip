@@ -118,6 +118,7 @@ __device__ __forceinline__ void hal_mmt4d(const void* lhs, const void* rhs, void
   a.out_cols = out_cols;
   a.lhs_row_major = 0;
   a.k_slices = 0; a.batch = 1; a.batch_by_xcd = 0;
+  a.stream_out = (int64_t)M * N * 1024 * (int64_t)sizeof(out_t) > (32ll << 20);
   a.slice_ksteps = 0;
   a.slice_out_bytes = 0;
   a.k0_div = Cfg::kMfmaK / K0;
@@ -175,6 +176,7 @@ __device__ __forceinline__ void hal_matmul_packed_rhs(const void* lhs, const voi
   a.out_cols = N;
   a.lhs_row_major = 1;
   a.k_slices = 0; a.batch = 1; a.batch_by_xcd = 0;
+  a.stream_out = 0;   // (row-major result)
   a.slice_ksteps = 0;
   a.slice_out_bytes = 0;
   a.k0_div = Cfg::kMfmaK / K0;
