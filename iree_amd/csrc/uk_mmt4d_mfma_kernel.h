@@ -715,8 +715,11 @@ __device__ __forceinline__ void mmt4d_mfma_body(const MfmaArgs a, const int bid 
         // 32-row blocks write whole 128-byte lines per instruction; a result
         // larger than the L2s goes past the caches (i8 4096^3: 65.3 -> 64.4 us,
         // fp8 56.65 -> 56.4); the 64-byte row pieces of 16-row blocks lose that
-        // way (f16 110.4 -> 114.9), and a small result is what the next kernel
-        // reads.
+        // way (f16 110.4 -> 114.9; exchanging lane rows between the two blocks
+        // of a tile first (v_permlane16_swap), so that they too write whole
+        // lines past the caches, measured the same as their ordinary stores:
+        // 103.8-104.7 against 104.4 us), and a small result is what the next
+        // kernel reads.
         bool streamed = false;
         if constexpr (R == 32 && kStreamOut) {
           if (a.stream_out) {
