@@ -13,7 +13,7 @@
 // w-th eighth of the K steps and keeps its part of the left-hand side in
 // registers for the whole kernel, as the B operand of v_mfma_*_32x32 (column
 // m0 of the block, zero beyond M0). The right-hand side streams through a
-// rolling register buffer of 8 blocks of 1 KiB per wave (A operand: a packed
+// rolling register buffer of 8 or 16 blocks of 1 KiB per wave (A operand: a packed
 // tile is already in operand order), the request for block q+8 issued as block
 // q is consumed, across tile boundaries, so the stream never drains. The 8
 // partial 32x32 blocks are summed through LDS in wave order (deterministic)
@@ -45,7 +45,9 @@ namespace {
 
 constexpr int kWaves = 8;
 constexpr int kThreads = kWaves * 64;
-constexpr int kDepth = 8;   // right-hand-side blocks in flight per wave
+// right-hand-side blocks in flight per wave: 16 where a tile's steps are whole
+// 16s, else 8 (N = 14336, K = 4096 f16: 22.84 -> 22.55 us at one row, 23.6 -> 23.1 at 8)
+constexpr int kDepthMax = 16;
 
 struct SkinnyArgs {
   const char* lhs;   // offsets applied
@@ -107,6 +109,7 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
   typedef typename Cfg::frag_t frag_t;
   typedef typename Cfg::acc_t acc_t;
   typedef typename Cfg::out_t out_t;
+  constexpr int kDepth = (SP % kDepthMax == 0) ? kDepthMax : 8;
   static_assert(SP % kDepth == 0, "the rolling buffer must divide the steps of a tile");
   // partial sums keep the accumulator's type (f32, or s32 for integer inputs)
   typedef typename std::conditional<std::is_same<out_t, int32_t>::value, int32_t, float>::type sum_t;
@@ -416,6 +419,9 @@ int launch_cfg(SkinnyArgs a, int chunks, hipStream_t s) {
     hipLaunchKernelGGL(kernel, grid, dim3(kThreads), 0, s, a);
     return check_hip(hipGetLastError(), "mmt4d_skinny launch");
   }
+  // (one workgroup per compute unit walking its tiles: giving every tile a
+  // workgroup of its own, two resident per compute unit, so that 448 tiles on
+  // 256 compute units all stream at once, measured 24.0 against 22.8 us)
   const int blocks = a.N < per_plane ? a.N : per_plane;
   const int per = (a.chunk_steps + kWaves - 1) / kWaves;
   a.steps_per_wave = per;
