@@ -135,9 +135,43 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
   // tiles 2, 3 as two 16-byte pieces), block of (j, step).
   constexpr int kSub = Cfg::kSub;
   constexpr int kBlock = kSub * 1024;
-  const int lane_off = kSub == 2 ? ((lane >> 5) * 1024 + (lane & 31) * 16)
-                       : a.half_k0 ? lane * 16 : ((lane & 31) * 32 + (lane >> 5) * 16);
-  const char* rhs_lane = a.rhs + (int64_t)(count > 0 ? first : 0) * kBlock + lane_off;
+  // Which columns a workgroup multiplies. The form that splits K over the waves
+  // deals the 32 N columns to the workgroups of a launch row in units of 8, a
+  // contiguous range of as equal a length as that allows each (448 outer
+  // columns on 256 compute units: 56 columns each, where whole outer columns
+  // were 1.75 a unit, paid as 2), and walks its range in windows of 32: lane
+  // row n of a window at column c0 is column c0 + n, which may lie in the next
+  // outer column (8 columns are whole cache lines of a K tile either way).
+  // Columns past the range repeat its last column (the same bytes as a lane
+  // that needs them: no further traffic) and their sums are not stored. The
+  // per-wave form takes whole outer columns, one per wave.
+  int c0, c_step, c_lim;
+  if constexpr (kPerWave) {
+    c0 = (blockIdx.x * kWaves + wave) * 32;
+    c_step = gridDim.x * kWaves * 32;
+    c_lim = a.N * 32;
+  } else {
+    const int units = a.N * 4, groups = (int)gridDim.x, bx = (int)blockIdx.x;
+    const int base = units / groups, rem = units - base * groups;
+    const int u0 = bx * base + (bx < rem ? bx : rem);
+    c0 = u0 * 8;
+    c_step = 32;
+    c_lim = (u0 + base + (bx < rem ? 1 : 0)) * 8;
+  }
+  const char* const rhs_wave = a.rhs + (int64_t)(count > 0 ? first : 0) * kBlock;
+  // this lane's piece of the first block of the window at column `at`
+  auto window_ptr = [&](int at) -> const char* {
+    int c = at + (lane & 31);
+    c = c < c_lim ? c : c_lim - 1;
+    c = c < a.N * 32 ? c : a.N * 32 - 1;        // (a window past the last one: any valid block)
+    c = c < 0 ? 0 : c;
+    const int r = c & 31;
+    const int off = kSub == 2 ? ((lane >> 5) * 1024 + r * 16)
+                    : a.half_k0 ? ((lane >> 5) * 512 + r * 16) : (r * 32 + (lane >> 5) * 16);
+    return rhs_wave + (int64_t)(c >> 5) * a.rhs_stride_bytes + off;
+  };
+  const char* rhs_cur = window_ptr(c0);
+  const char* rhs_next = window_ptr(c0 + c_step);
   // Partial last step: K tile of this lane's piece(s) inside a step (tiles are
   // 512 bytes of the right-hand side), whether the last step lacks it, and the
   // step of this wave's slice that is the last one of K (-1: another wave's).
@@ -157,10 +191,9 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
   // Steps past this wave's count still issue a load (of a valid block, so the
   // number of loads in flight stays constant) but contribute zeros, whatever
   // that block holds.
-  auto load_block = [&](int j, int sp) -> frag_t {
+  auto load_block = [&](const char* window, int sp) -> frag_t {
     const int s = sp < count ? sp : 0;
-    const int jj = j < a.N ? j : a.N - 1;
-    const char* p = rhs_lane + (int64_t)jj * a.rhs_stride_bytes + (int64_t)s * kBlock;
+    const char* p = window + (int64_t)s * kBlock;
     if constexpr (kTail) {
       // (a piece of a missing tile would lie past the end of the row: it is
       // fetched from the step's first tile instead and zeroed when consumed)
@@ -197,8 +230,6 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
   };
 
   // ---- the left-hand side and the first blocks of the first tile ------------
-  int j = kPerWave ? blockIdx.x * kWaves + wave : blockIdx.x;
-  const int j_step = kPerWave ? gridDim.x * kWaves : gridDim.x;
   frag_t ring[kDepth];
   frag_t xf[SP];
   // bytes of the packed left-hand side per K step: its K tiles are consecutive
@@ -249,7 +280,7 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
     }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int d = 0; d < kDepth; ++d) ring[d] = load_block(j, d);
+    for (int d = 0; d < kDepth; ++d) ring[d] = load_block(rhs_cur, d);
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kDepth * kSub) : "memory");
 #pragma unroll
@@ -268,7 +299,7 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
     }
   } else {
 #pragma unroll
-    for (int d = 0; d < kDepth; ++d) ring[d] = load_block(j, d);
+    for (int d = 0; d < kDepth; ++d) ring[d] = load_block(rhs_cur, d);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int sp = 0; sp < SP; ++sp) {
@@ -289,8 +320,7 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
   }
 
   int parity = 0;
-  for (; j < a.N; j += j_step, parity ^= 1) {
-    const int next = j + j_step;
+  for (; c0 < c_lim; c0 += c_step, parity ^= 1) {
     acc_t acc;
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc[v] = 0;
@@ -300,13 +330,16 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
       else acc = Cfg::mfma(live(ring[sp % kDepth], sp), xf[sp], acc);
       // refill the slot: kDepth steps ahead, wrapping into the next tile
       __builtin_amdgcn_sched_barrier(0);
-      ring[sp % kDepth] = sp + kDepth < SP ? load_block(j, sp + kDepth) : load_block(next, sp + kDepth - SP);
+      ring[sp % kDepth] = sp + kDepth < SP ? load_block(rhs_cur, sp + kDepth) : load_block(rhs_next, sp + kDepth - SP);
       __builtin_amdgcn_sched_barrier(0);
     }
+    rhs_cur = rhs_next;
+    rhs_next = window_ptr(c0 + 2 * c_step);
     if constexpr (kPerWave) {
       // (the stores below are divergent and the block's only consumer)
       keep_result_in_all_lanes(acc);
       constexpr bool rows_out = kRows;
+      const int j = c0 >> 5;      // (whole outer columns in this form)
       store_t* tile = (store_t*)a.out + (rows_out ? (int64_t)j * 32 : (int64_t)j * a.out_stride_elems);
       const int mm = lane & 31;
       if (mm < a.M0) {
@@ -328,14 +361,16 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
     for (int v = 0; v < 16; ++v) buf[wave][v][lane] = acc[v];
     __syncthreads();
     constexpr bool rows_out = kRows;
-    store_t* tile = (store_t*)a.out + blockIdx.y * a.chunk_out_elems +
-                    (rows_out ? (int64_t)j * 32 : (int64_t)j * a.out_stride_elems);
+    store_t* const out_row = (store_t*)a.out + blockIdx.y * a.chunk_out_elems;
 #pragma unroll
     for (int rep = 0; rep < 2; ++rep) {
       const int flat = rep * kThreads + threadIdx.x;   // v * 64 + lane
       const int l = flat & 63, v = flat >> 6;
-      const int mm = l & 31, nn = 8 * (v >> 2) + 4 * (l >> 5) + (v & 3);
-      if (mm < a.M0 && !(rows_out && j * 32 + nn >= a.out_cols)) {
+      const int mm = l & 31;
+      const int c = c0 + 8 * (v >> 2) + 4 * (l >> 5) + (v & 3);       // this sum's column
+      const int nn = c & 31;                                          // ... inside its outer column
+      if (mm < a.M0 && c < c_lim && !(rows_out && c >= a.out_cols)) {
+        store_t* tile = out_row + (rows_out ? (int64_t)(c - nn) : (int64_t)(c >> 5) * a.out_stride_elems);
         const int64_t at = rows_out ? mm * a.out_row_pitch_elems + nn
                                     : a.transpose_out ? nn * a.M0 + mm : mm * 32 + nn;
         sum_t sum = a.accumulate ? (sum_t)tile[at] : (sum_t)0;
