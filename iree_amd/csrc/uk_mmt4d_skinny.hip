@@ -549,7 +549,8 @@ int launch_batch_mmt4d_skinny(const iree_amd_uk_mmt4d_params_t& p0, int64_t batc
   }
   const int mk = mfma_k_of(p.flags);
   const int64_t k_elems = p.K * p.K0;
-  if (p.M != 1 || p.K == 0 || p.N > 0x7FFFFFFF || batch > 65535)
+  // (the kernel counts columns, 32 per outer column, in 32 bits)
+  if (p.M != 1 || p.K == 0 || p.N > 0x3FFFFFF || batch > 65535)
     return IREE_AMD_UK_STATUS_NOT_FOUND;
   const int64_t steps = (k_elems + mk - 1) / mk;   // (the last one may be partial)
   if (steps > max_steps_per_launch(mk)) return IREE_AMD_UK_STATUS_NOT_FOUND;
@@ -563,7 +564,7 @@ int launch_mmt4d_skinny(const iree_amd_uk_mmt4d_params_t& p0, hipStream_t s) {
   const bool transposed = (p.flags & kTransposedOut) != 0;
   const int mk = mfma_k_of(p.flags);
   const int64_t k_elems = p.K * p.K0;
-  if (p.M != 1 || p.K == 0 || p.N > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  if (p.M != 1 || p.K == 0 || p.N > 0x3FFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
   // (a K that is not whole steps ends in a partial one)
   const int64_t steps = (k_elems + mk - 1) / mk;
   if (steps > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
@@ -650,7 +651,7 @@ int launch_chunk(const iree_amd_uk_mmt4d_params_t& p, int chunks, int chunk_step
   const int eb = ti.lhs_bits / 8;
   const int64_t k_elems = p.K * p.K0;
   // 16-byte aligned operands
-  if (p.N > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  if (p.N > 0x3FFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
   const char* lhs = (const char*)p.lhs_buffer + p.lhs_offset * eb;
   const char* rhs = (const char*)p.rhs_buffer + p.rhs_offset * eb;
   if (((uintptr_t)lhs | (uintptr_t)rhs) % 16 || (p.rhs_stride0 * eb) % 16 || (p.M0 * p.K0 * eb) % 16)
@@ -717,7 +718,7 @@ int launch_matmul_rows_skinny(const iree_amd_uk_mmt4d_params_t& p, int64_t M, in
   mmt4d_type_info(p.flags, &ti);
   const int eb = ti.lhs_bits / 8;
   const int64_t k_elems = p.K * p.K0;
-  if (p.K == 0 || k_elems % mk || p.N > 0x7FFFFFFF || out_cols > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
+  if (p.K == 0 || k_elems % mk || p.N > 0x3FFFFFF || out_cols > 0x7FFFFFFF) return IREE_AMD_UK_STATUS_NOT_FOUND;
   // (measured at N = 14336, K = 4096: 2-byte elements at 31 / 32 rows 29.0 /
   // 29.7 us against 28.4 for the macro-tile kernel, 26.9 at 24 rows; 1-byte
   // elements at 32 rows 15.1 (i8) and 16.7 (fp8) against 17.2 and 17.0)
