@@ -264,8 +264,11 @@ __device__ __forceinline__ void hal_pack(const void* mat, void* tiled, int size0
   a.padding = padding;
   if (blockIdx.x >= a.blocks_x * a.blocks_y) return;
   // (blocks of 16 rows x 32 chunks per 256 threads, as the export's workgroup
-  // count says: 2 x 2 waves of 2 blocks of 4 rows x 16 chunks)
-  stream_pow2_body<ES, kPack, true, kPack, 4, 2, 2, 4>(a);
+  // count says: 2 x 2 waves of 2 blocks of 4 rows x 16 chunks; tiles whose rows
+  // are one chunk: 4 waves side by side, each 2 blocks of 8 rows x 8 chunks, so
+  // that a wave's piece of a tile is a whole cache line)
+  if (cpr == 1 && tile0 >= 8) stream_pow2_body<ES, kPack, true, kPack, 8, 2, 4, 4>(a);
+  else stream_pow2_body<ES, kPack, true, kPack, 4, 2, 2, 4>(a);
 }
 
 // Transposed inner tiles: tile0 rows x tile1 columns of the matrix, stored

@@ -227,7 +227,7 @@ def test_matmul_exports_equal_the_library_entry_point(uk, cuda, exe, name):
 
 PACK_CASES = [  # size0, size1, tile0, tile1 (elements)
     (1, 1, 1, 16), (33, 70, 32, 16), (100, 257, 8, 32), (64, 64, 32, 32), (17, 500, 16, 64),
-    (300, 33, 1, 16), (129, 1000, 32, 16),
+    (300, 33, 1, 16), (129, 1000, 32, 16), (200, 300, 32, 8), (77, 130, 32, 4), (45, 260, 8, 8),
     # tiles that are not powers of two, or whose rows are not whole 16-byte chunks (single elements)
     (50, 77, 24, 16), (123, 200, 12, 48), (9, 9, 3, 5), (130, 95, 7, 1), (40, 300, 32, 6), (65, 64, 5, 24)]
 
