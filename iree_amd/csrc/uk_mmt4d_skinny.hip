@@ -153,7 +153,16 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
     c_step = gridDim.x * kWaves * 32;
     c_lim = a.N * 32;
   } else {
-    const int units = a.N * 4, groups = (int)gridDim.x, bx = (int)blockIdx.x;
+    // (workgroup ids go round-robin over the 8 XCDs: XCD x takes the x-th
+    // contiguous slice of the ranges, so that neighbouring ranges, which share
+    // the pair of cache lines at their boundary, meet in one L2)
+    const int units = a.N * 4, groups = (int)gridDim.x;
+    int bx;
+    {
+      const int per = groups / 8, more = groups % 8;
+      const int xcd = (int)blockIdx.x % 8, idx = (int)blockIdx.x / 8;
+      bx = xcd * per + (xcd < more ? xcd : more) + idx;
+    }
     const int base = units / groups, rem = units - base * groups;
     const int u0 = bx * base + (bx < rem ? bx : rem);
     c0 = u0 * 8;
