@@ -479,7 +479,16 @@ int launch_cfg(SkinnyArgs a, int chunks, hipStream_t s) {
   // (one workgroup per compute unit walking its tiles: giving every tile a
   // workgroup of its own, two resident per compute unit, so that 448 tiles on
   // 256 compute units all stream at once, measured 24.0 against 22.8 us)
-  const int blocks = a.N < per_plane ? a.N : per_plane;
+  int blocks = a.N < per_plane ? a.N : per_plane;
+  // K split over workgroup rows: the rows share the compute units, one round in
+  // all, each workgroup walking more columns (N = 4096, K = 14336 f16 at 8 rows:
+  // 4 rows of 128 workgroups, two rounds, 27.8 us; 4 rows of 64: 25.65; N = 8192,
+  // K = 7168: 27.3 -> 24.5).
+  if (chunks > 1 && a.batch <= 1) {
+    int share = cus / chunks;
+    share = share < 1 ? 1 : share;
+    blocks = blocks < share ? blocks : share;
+  }
   const int per = (a.chunk_steps + kWaves - 1) / kWaves;
   a.steps_per_wave = per;
   const dim3 grid(blocks, chunks, a.batch > 1 ? a.batch : 1);
