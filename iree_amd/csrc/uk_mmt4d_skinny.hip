@@ -360,18 +360,34 @@ __global__ __launch_bounds__(kThreads) void mmt4d_skinny_kernel(SkinnyArgs a) {
       constexpr bool rows_out = kRows;
       const int j = rotated(c0 >> 5);      // (whole outer columns in this form)
       store_t* tile = (store_t*)a.out + (rows_out ? (int64_t)j * 32 : (int64_t)j * a.out_stride_elems);
-      const int mm = lane & 31;
-      if (mm < a.M0) {
+      // Register v of lane l is row l % 32, column 8 (v / 4) + 4 (l / 32) + v % 4:
+      // stored from there, the M0 x 32 sums of a narrow tile are 16 store
+      // instructions with 2 M0 lanes each, and a compute unit takes a memory
+      // instruction only every 30-50 cycles whatever it moves: with M0 = 1 the
+      // stores of this form cost twice what its 8 loads per outer column do.
+      // The wave passes the block through its own part of LDS instead (no
+      // barrier: a wave's LDS accesses are served in order) and stores element
+      // e = 64 i + lane of the tile from lane `lane`: M0 / 2 instructions.
+      sum_t (*mine)[64] = partial[0][wave];
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const int nn = 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-          if (rows_out && j * 32 + nn >= a.out_cols) continue;
-          const int64_t at = rows_out ? mm * a.out_row_pitch_elems + nn
-                                      : a.transpose_out ? nn * a.M0 + mm : mm * 32 + nn;
-          const sum_t sum = (a.accumulate ? (sum_t)tile[at] : (sum_t)0) + (sum_t)acc[v];
-          tile[at] = (store_t)sum;
-        }
+      for (int v = 0; v < 16; ++v) mine[v][lane] = acc[v];
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      const int elems = a.M0 * 32;
+#pragma unroll 1
+      for (int e = lane; e < elems; e += 64) {
+        // (tiles stored transposed hold element (mm, nn) at nn * M0 + mm)
+        const int mm = a.transpose_out ? e % a.M0 : e >> 5, nn = a.transpose_out ? e / a.M0 : e & 31;
+        if (rows_out && j * 32 + nn >= a.out_cols) continue;
+        const int v = ((nn >> 3) << 2) | (nn & 3), l = mm + 32 * ((nn >> 2) & 1);
+        const int64_t at = rows_out ? mm * a.out_row_pitch_elems + nn : e;
+        const sum_t sum = (a.accumulate ? (sum_t)tile[at] : (sum_t)0) + mine[v][l];
+        tile[at] = (store_t)sum;
       }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
       continue;
     }
     // ---- sum the 8 K slices in wave order and store -----------------------
