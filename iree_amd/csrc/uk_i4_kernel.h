@@ -110,17 +110,37 @@ __device__ __forceinline__ void dequant_matmul_i4_body(const I4Args& a) {
   // Raw group parameters of this lane's two columns for the wave's K slice
   // (zsh: position of a lone packed zero point inside its byte).
   struct Meta { uint32_t s[2][SW], z[2][ZW], zsh[2]; };
-  auto load_meta = [&](int nt, Meta& m) {
+  // They are fetched with lane l % 32 taking column l % 32 of the tile, one
+  // load instruction for the scales and one for the zero points of all 32
+  // columns, and handed to the lanes that need them across the wave when the
+  // tile begins (a compute unit takes a memory instruction only every 30 to 50
+  // cycles whatever it moves: a load per column half, four per tile and wave
+  // beside its eight of weights, was a third of the kernel's memory
+  // instructions at one row).
+  struct MetaRaw { uint32_t s[SW], z[ZW]; };
+  auto load_meta = [&](int nt, MetaRaw& m) {
+    int n = nt * 32 + (lane & 31);
+    n = n < a.N ? n : a.N - 1;
+    const size_t sg = (size_t)n * a.G + g_first;
+    load_bits<SB>(a.scale + sg, m.s);
+    if (kZpU4) load_bits<ZB>((const uint8_t*)a.zp + (sg >> 1), m.z);
+    else load_bits<ZB>((const uint16_t*)a.zp + sg, m.z);
+  };
+  auto spread_meta = [&](const MetaRaw& raw, int nt) -> Meta {
+    Meta m;
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
+      const int from = (h * 16 + nl) * 4;       // (byte address of the source lane)
+#pragma unroll
+      for (int i = 0; i < SW; ++i) m.s[h][i] = (uint32_t)__builtin_amdgcn_ds_bpermute(from, (int)raw.s[i]);
+#pragma unroll
+      for (int i = 0; i < ZW; ++i) m.z[h][i] = (uint32_t)__builtin_amdgcn_ds_bpermute(from, (int)raw.z[i]);
       int n = nt * 32 + h * 16 + nl;
       n = n < a.N ? n : a.N - 1;
       const size_t sg = (size_t)n * a.G + g_first;
-      load_bits<SB>(a.scale + sg, m.s[h]);
-      if (kZpU4) load_bits<ZB>((const uint8_t*)a.zp + (sg >> 1), m.z[h]);
-      else load_bits<ZB>((const uint16_t*)a.zp + sg, m.z[h]);
       m.zsh[h] = (kZpU4 && GW == 1) ? (uint32_t)(sg & 1) * 4 : 0;
     }
+    return m;
   };
   // Weights of one tile: loads past the end of the buffer (a tile after the
   // last one, columns past N) return zeros without touching memory.
@@ -146,8 +166,9 @@ __device__ __forceinline__ void dequant_matmul_i4_body(const I4Args& a) {
   // activations: rows m_base + mh*16 + nl, this wave's K slice; rows past M
   // are zeros.
   int nt = blockIdx.x;
-  Meta meta_next;
-  load_meta(nt < a.n_tiles ? nt : a.n_tiles - 1, meta_next);
+  MetaRaw meta_next;
+  int meta_next_tile = nt < a.n_tiles ? nt : a.n_tiles - 1;
+  load_meta(meta_next_tile, meta_next);
   u32x4 xraw[MH][SP][4];
   u32x4 wreg[SP][2];
   if constexpr (kStageX) {
@@ -287,8 +308,9 @@ __device__ __forceinline__ void dequant_matmul_i4_body(const I4Args& a) {
   auto tile = [&](auto first) {
     constexpr bool kFirst = decltype(first)::value;
     const int next = nt + gridDim.x;
-    const Meta mt = meta_next;
-    load_meta(next < a.n_tiles ? next : a.n_tiles - 1, meta_next);
+    const Meta mt = spread_meta(meta_next, meta_next_tile);
+    meta_next_tile = next < a.n_tiles ? next : a.n_tiles - 1;
+    load_meta(meta_next_tile, meta_next);
     const __amdgpu_buffer_rsrc_t rsrc_next = tile_rsrc(next < a.n_tiles ? next : a.n_tiles);
     __builtin_amdgcn_sched_barrier(0);
     floatx4 acc[2][MH], part[2][MH];
