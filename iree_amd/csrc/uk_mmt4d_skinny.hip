@@ -495,7 +495,13 @@ int launch_cfg(SkinnyArgs a, int chunks, hipStream_t s) {
   // (one workgroup per compute unit walking its tiles: giving every tile a
   // workgroup of its own, two resident per compute unit, so that 448 tiles on
   // 256 compute units all stream at once, measured 24.0 against 22.8 us)
+  // Workgroups of a launch row: one per compute unit at most, and at least 16
+  // columns each (fewer outer columns than compute units are dealt out in
+  // halves: N = 4096, K = 4096 f16 as 256 workgroups of 16 columns 8.4 us, as
+  // 128 of 32 with K split over two rows and the launch that adds them 10.85;
+  // K = 1024: 4.8 against 7.4).
   int blocks = a.N < per_plane ? a.N : per_plane;
+  if (a.batch <= 1) blocks = a.N * 2 < per_plane ? a.N * 2 : per_plane;
   // K split over workgroup rows: the rows share the compute units, one round in
   // all, each workgroup walking more columns (N = 4096, K = 14336 f16 at 8 rows:
   // 4 rows of 128 workgroups, two rounds, 27.8 us; 4 rows of 64: 25.65; N = 8192,
@@ -629,8 +635,10 @@ int launch_mmt4d_skinny(const iree_amd_uk_mmt4d_params_t& p0, hipStream_t s) {
   // (partial sums and result are dense arrays there: transposed tiles must
   // follow each other without gaps)
   const bool dense_out = !transposed || p.N == 1 || p.out_stride0 == (int64_t)p.M0 * 32;
-  if (dense_out && p.N * chunks * 2 <= cus && steps >= 64) {
-    int64_t more = cus / p.N;
+  // (column blocks of a launch row: see launch_cfg)
+  const int64_t col_blocks = p.N * 2 < cus ? p.N * 2 : cus;
+  if (dense_out && col_blocks * chunks * 2 <= cus && steps >= 64) {
+    int64_t more = cus / col_blocks;
     if (more > steps / 32) more = steps / 32;
     if (more > 8) more = 8;
     if (more > chunks) chunks = more;
