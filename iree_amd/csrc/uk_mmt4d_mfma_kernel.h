@@ -100,6 +100,8 @@ struct MfmaArgs {
   int batch_by_xcd;
   // the tiled result is larger than the L2s together: write it past the caches
   int stream_out;
+  // macro-tile rows of one column panel of the workgroup order (see tile_coord)
+  int panel_rows;
 };
 
 namespace {
@@ -158,10 +160,15 @@ __device__ __forceinline__ void spread_issue() {
 // Maps the hardware workgroup id to a macro-tile coordinate. Workgroup ids go
 // round-robin over the 8 XCDs; give XCD x the x-th contiguous slice of the
 // logical tile sequence, and order that sequence in column-panels of `kGroup`
-// macro-tile rows so that a slice is a compact 2-D block.
-__device__ __forceinline__ void tile_coord(int bid, int tiles_m, int tiles_n,
+// macro-tile rows so that a slice is a compact 2-D block. What an XCD's L2
+// fetches for the r x c tiles it holds at a time is r tile heights of the
+// left-hand side plus c tile widths of the right-hand side: 4 rows suit the
+// square tile (32 resident per XCD: 4 x 8) and the tall one (64: 4 x 16 of
+// 256 x 128), 8 rows the wide one (8 x 8 of 128 x 256; in panels of 4 rows
+// every right-hand-side panel is fetched by twice as many XCD slices).
+__device__ __forceinline__ void tile_coord(int bid, int tiles_m, int tiles_n, int kGroup,
                                            int* tm, int* tn) {
-  constexpr int kXcds = 8, kGroup = 4;
+  constexpr int kXcds = 8;
   const int total = tiles_m * tiles_n;
   const int per = total / kXcds, rem = total % kXcds;
   const int xcd = bid % kXcds, idx = bid / kXcds;
@@ -266,7 +273,7 @@ __device__ __forceinline__ void mmt4d_mfma_body(const MfmaArgs a, const int bid 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wm = wave / kWavesN, wn = wave % kWavesN;
   int tm, tn;
-  tile_coord(bid, a.tiles_m, a.tiles_n, &tm, &tn);
+  tile_coord(bid, a.tiles_m, a.tiles_n, a.panel_rows, &tm, &tn);
   const int i_base = tm * TM, j_base = tn * TN;
   const int T = a.ksteps;
 

@@ -121,6 +121,9 @@ int launch_variant(const MfmaArgs& a0, hipStream_t s) {
   constexpr int kPerTile = 32 / Cfg::kRows;
   constexpr int TM = 2 * WM, TN = kWavesN * WN;   // blocks of Cfg::kRows rows
   static_assert(TM % kPerTile == 0 && TN % kPerTile == 0, "a workgroup covers whole outer tiles");
+  // (the fp8 MLP block, whose matmuls run on 128 x 256 tiles: 289-292 us in
+  // panels of 4 rows, 286-288 in panels of 8, 309 in panels of 16)
+  a.panel_rows = WM < WN ? 8 : 4;
   a.tiles_m = (a.M * kPerTile + TM - 1) / TM;
   a.tiles_n = (a.N * kPerTile + TN - 1) / TN;
   const int64_t blocks = (int64_t)a.tiles_m * a.tiles_n;

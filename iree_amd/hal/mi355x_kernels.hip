@@ -108,6 +108,7 @@ __device__ __forceinline__ void hal_mmt4d(const void* lhs, const void* rhs, void
                                  : (int64_t)N * 1024 * (int64_t)sizeof(out_t);
   a.M = M;
   a.N = N;
+  a.panel_rows = 4;
   a.ksteps = (int)(k_elems / Cfg::kMfmaK);
   a.tail_tiles = (int)((k_elems % Cfg::kMfmaK) / K0);
   a.tiles_m = (M * kPerTile + TM - 1) / TM;
@@ -166,6 +167,7 @@ __device__ __forceinline__ void hal_matmul_packed_rhs(const void* lhs, const voi
   a.out_stride_bytes = (int64_t)N * (int64_t)sizeof(out_t);
   a.M = (M + 31) / 32;
   a.N = (N + 31) / 32;
+  a.panel_rows = 4;
   a.ksteps = K / Cfg::kMfmaK;
   a.tail_tiles = 0;
   a.tiles_m = (a.M * kPerTile + TM - 1) / TM;
