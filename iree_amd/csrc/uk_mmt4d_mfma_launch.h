@@ -261,14 +261,15 @@ int launch_cfg(const MfmaArgs& a, hipStream_t s) {
       cost += resident * work / (resident == t.occ ? t.eff_full : t.eff_alone);
     }
     // Of the two half-size tiles the one with more columns than rows is the
-    // faster one when the accumulators are held transposed (row-major result,
-    // SiLU form) on the 32-row instructions: fp8 2048 x 4096 x 14336 91.5 ->
-    // 86.9 us, 1024 x 8192 x 8192 57.7 -> 53.7 (i8 65.0 -> 62.8), the gate/up
-    // matmul with the SiLU epilogue 171.3 -> 167.0; tiled results measure the
-    // other way round (fp8 84.4 against 89.6) and the 16-row shapes the same.
-    // (Measured in bursts of 20 launches; under sustained load, where the
-    // clock follows the power limit, the MLP block measures the same either way.)
-    if ((a.row_major_out || kSiluMul) && Cfg::kRows == 32 && v == 1) cost *= 1.03;
+    // faster one for the SiLU form (the gate/up matmul of the fp8 MLP block
+    // alone, sustained: 187.7 -> 180.0 us; inside the block 292 -> 289). For
+    // row-major results on the 32-row instructions the two measure either way:
+    // 128x256 ahead by 3-7 % when the call is repeated on operands that stay
+    // in the last-level cache (fp8 2048 x 4096 x 14336 100.6 -> 97.4 us),
+    // 256x128 ahead by 2 % inside the MLP block, where the weights come from
+    // memory every time (block 289 -> 283 us): the latter is what a model does,
+    // so those keep the first of the two.
+    if (kSiluMul && Cfg::kRows == 32 && v == 1) cost *= 1.03;
     // A row-major left-hand side is the dearer operand to fetch (half or
     // quarter cache lines per row and K-step, each line asked for again on the
     // next step): tiles with more rows than columns pay most. Measured at
