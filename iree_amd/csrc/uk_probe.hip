@@ -131,7 +131,7 @@ int launch_mfma_probe(uint32_t type_flag, const void* operands, int64_t iters, v
     // (the shapes the mmt4d kernel uses for each type)
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_F16F16F32: st = launch<F16Cfg16>(operands, iters, sink, blocks, s); k = 32; break;
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_BF16BF16F32: st = launch<BF16Cfg16>(operands, iters, sink, blocks, s); k = 32; break;
-    case IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32: st = launch<S8Cfg>(operands, iters, sink, blocks, s); k = 32; break;
+    case IREE_AMD_UK_FLAG_MMT4D_TYPE_S8S8S32: st = launch<S8Cfg16>(operands, iters, sink, blocks, s); k = 64; break;
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_F8E4M3F8E4M3F32: st = launch<F8Cfg>(operands, iters, sink, blocks, s); k = 64; break;
     case IREE_AMD_UK_FLAG_MMT4D_TYPE_F32F32F32: st = launch<F32Cfg>(operands, iters, sink, blocks, s); k = 8; break;
     default: return fail(IREE_AMD_UK_STATUS_INVALID_ARGUMENT, "mfma_probe: type has no MFMA kernel");

@@ -569,7 +569,7 @@ def test_mfma_probe_runs_and_counts_operations(uk, cuda):
     ops = torch.zeros(64 * 1024, dtype=torch.uint8, device=cuda)
     sink = torch.zeros(256, dtype=torch.float32, device=cuda)
     cus = torch.cuda.get_device_properties(0).multi_processor_count
-    for flag, k in ((F.MMT4D_TYPE_F16F16F32, 32), (F.MMT4D_TYPE_BF16BF16F32, 32), (F.MMT4D_TYPE_S8S8S32, 32),
+    for flag, k in ((F.MMT4D_TYPE_F16F16F32, 32), (F.MMT4D_TYPE_BF16BF16F32, 32), (F.MMT4D_TYPE_S8S8S32, 64),
                     (F.MMT4D_TYPE_F8E4M3F8E4M3F32, 64), (F.MMT4D_TYPE_F32F32F32, 8)):
         n = uk.mfma_probe(flag, ops, 7, sink)
         assert n == cus * 4 * 7 * 2 * 128 * 128 * k       # a 128 x 128 x k update per wave and step
