@@ -417,10 +417,11 @@ MI355X_MATMUL_EXPORT(bf16bf16f32_t4x8, BF16Cfg16, 4, 8, 3, 1, 2, 73728)
 MI355X_MATMUL_EXPORT(bf16bf16f32_t8x8, BF16Cfg16, 8, 8, 5, 1, 1, 163840)
 MI355X_MATMUL_EXPORT(s8s8s32_t4x8, S8Cfg, 2, 4, 6, 2, 2, 73728)
 MI355X_MATMUL_EXPORT(s8s8s32_t8x8, S8Cfg, 4, 4, 8, 2, 1, 131072)
-// (K0 = 16 and K a multiple of 64: two instructions per 64-byte K-step, so
-// that a lane quad loads 64 contiguous bytes of a row of the left-hand side)
-MI355X_MATMUL_EXPORT(s8s8s32_k64_t4x8, S8Cfg2, 2, 4, 3, 1, 2, 73728)
-MI355X_MATMUL_EXPORT(s8s8s32_k64_t8x8, S8Cfg2, 4, 4, 5, 1, 1, 163840)
+// (K0 = 16 and K a multiple of 64: the 16-row instruction, whose K-step is 64
+// bytes of a row, so that a lane quad loads 64 contiguous bytes of a row of
+// the left-hand side)
+MI355X_MATMUL_EXPORT(s8s8s32_k64_t4x8, S8Cfg16, 4, 8, 3, 1, 2, 73728)
+MI355X_MATMUL_EXPORT(s8s8s32_k64_t8x8, S8Cfg16, 8, 8, 5, 1, 1, 163840)
 MI355X_MATMUL_EXPORT(f8e4m3f8e4m3f32_t4x8, F8Cfg, 2, 4, 3, 1, 2, 73728)
 MI355X_MATMUL_EXPORT(f8e4m3f8e4m3f32_t8x8, F8Cfg, 4, 4, 5, 1, 1, 163840)
 MI355X_MATMUL_EXPORT(f32f32f32_t4x8, F32Cfg, 2, 4, 6, 2, 2, 73728)
@@ -446,8 +447,8 @@ MI355X_MATMUL_EXPORT(f32f32f32_t8x8, F32Cfg, 4, 4, 8, 2, 1, 131072)
 // f16f16f32_t8   (256x256)  F16Cfg16      8 x 8        5    1   1     8   163840      8, 16
 // f16f16f32_t4   (128x128)  F16Cfg16      4 x 4        4    1   1     4    65536      8, 16
 // bf16bf16f32_t8 / _t4      BF16Cfg16     as f16
-// s8s8s32_t8     (256x256)  S8Cfg         4 x 4        8    2   1     8   131072      16, 32
-// s8s8s32_t4     (128x128)  S8Cfg         2 x 2        8    2   1     4    65536      16, 32
+// s8s8s32_t8     (256x256)  S8Cfg16       8 x 8        5    1   1     8   163840      16, 32
+// s8s8s32_t4     (128x128)  S8Cfg16       4 x 4        4    1   1     4    65536      16, 32
 // f8e4m3f8e4m3f32_t8        F8Cfg         4 x 4        5    1   1     8   163840      16
 // f8e4m3f8e4m3f32_t4        F8Cfg         2 x 2        8    2   1     4   131072      16
 // f32f32f32_t8              F32Cfg        4 x 4        8    2   1     8   131072      4, 8
@@ -456,8 +457,8 @@ MI355X_MMT4D_EXPORTS(f16f16f32_t8, F16Cfg16, 8, 8, 5, 1, 1, 163840)
 MI355X_MMT4D_EXPORTS(f16f16f32_t4, F16Cfg16, 4, 4, 4, 1, 1, 65536)
 MI355X_MMT4D_EXPORTS(bf16bf16f32_t8, BF16Cfg16, 8, 8, 5, 1, 1, 163840)
 MI355X_MMT4D_EXPORTS(bf16bf16f32_t4, BF16Cfg16, 4, 4, 4, 1, 1, 65536)
-MI355X_MMT4D_EXPORTS(s8s8s32_t8, S8Cfg, 4, 4, 8, 2, 1, 131072)
-MI355X_MMT4D_EXPORTS(s8s8s32_t4, S8Cfg, 2, 2, 8, 2, 1, 65536)
+MI355X_MMT4D_EXPORTS(s8s8s32_t8, S8Cfg16, 8, 8, 5, 1, 1, 163840)
+MI355X_MMT4D_EXPORTS(s8s8s32_t4, S8Cfg16, 4, 4, 4, 1, 1, 65536)
 MI355X_MMT4D_EXPORTS(f8e4m3f8e4m3f32_t8, F8Cfg, 4, 4, 5, 1, 1, 163840)
 MI355X_MMT4D_EXPORTS(f8e4m3f8e4m3f32_t4, F8Cfg, 2, 2, 8, 2, 1, 131072)
 MI355X_MMT4D_EXPORTS(f32f32f32_t8, F32Cfg, 4, 4, 8, 2, 1, 131072)

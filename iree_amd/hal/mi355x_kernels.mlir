@@ -158,7 +158,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
         ]>
       ]>) attributes {
     workgroup_size = [256 : index, 1 : index, 1 : index],
-    workgroup_local_memory = 131072 : index
+    workgroup_local_memory = 163840 : index
   } {
   ^bb0(%device: !hal.device, %m: index, %n: index, %batch: index):
     %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 8) * (s1 ceildiv 8))>()[%m, %n]
@@ -174,7 +174,7 @@ hal.executable.source public @mi355x_mmt4d attributes {
         ]>
       ]>) attributes {
     workgroup_size = [256 : index, 1 : index, 1 : index],
-    workgroup_local_memory = 131072 : index
+    workgroup_local_memory = 163840 : index
   } {
   ^bb0(%device: !hal.device, %m: index, %n: index, %batch: index):
     %x = affine.apply affine_map<()[s0, s1] -> ((s0 ceildiv 8) * (s1 ceildiv 8))>()[%m, %n]

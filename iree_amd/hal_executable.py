@@ -34,7 +34,7 @@ def _exports():
     rows = [
         ("f16f16f32", F.MMT4D_TYPE_F16F16F32, 160 * kib, 64 * kib, (8, 16), 2, 4),
         ("bf16bf16f32", F.MMT4D_TYPE_BF16BF16F32, 160 * kib, 64 * kib, (8, 16), 2, 4),
-        ("s8s8s32", F.MMT4D_TYPE_S8S8S32, 128 * kib, 64 * kib, (16, 32), 1, 4),
+        ("s8s8s32", F.MMT4D_TYPE_S8S8S32, 160 * kib, 64 * kib, (16, 32), 1, 4),
         ("f8e4m3f8e4m3f32", F.MMT4D_TYPE_F8E4M3F8E4M3F32, 160 * kib, 128 * kib, (16,), 1, 4),
         ("f32f32f32", F.MMT4D_TYPE_F32F32F32, 128 * kib, 64 * kib, (4, 8), 4, 4),
     ]
