@@ -135,7 +135,7 @@ struct S8Cfg {
 // sustains 3.47 (both 4.92 on zeros): the smaller block costs less energy per
 // operation, as with f16.
 struct S8Cfg16 {
-  static constexpr float kStepUs = 0.72f;
+  static constexpr float kStepUs = 0.65f;
   static constexpr int kRows = 16;
   typedef int4v frag_t;
   typedef intx4 acc_t;
