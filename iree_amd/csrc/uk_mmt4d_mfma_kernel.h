@@ -9,7 +9,8 @@
 //   type            MFMA                         K per MFMA   K0 served
 //   f16 x f16 -> f32  v_mfma_f32_16x16x32_f16        32         8, 16
 //   bf16 x bf16 -> f32 v_mfma_f32_16x16x32_bf16      32         8, 16
-//   s8 x s8 -> s32    v_mfma_i32_32x32x32_i8         32         16, 32
+//   s8 x s8 -> s32    v_mfma_i32_16x16x64_i8         64         16, 32
+//   (s8 with a row-major left-hand side and K in whole 32s only: v_mfma_i32_32x32x32_i8, K 32)
 //   f32 x f32 -> f32  4 x v_mfma_f32_32x32x2_f32      8          4, 8
 //   f16 -> f16, bf16 -> bf16 (intermediate roundings skipped): as -> f32, rounded on store
 //   e4m3 x e4m3 -> f32 v_mfma_scale_f32_32x32x64_f8f6f4  64         16
@@ -43,9 +44,12 @@
 // power-limited by operand toggling. With N(0,1) f16 operands a register-only
 // loop of v_mfma_f32_32x32x16_f16 sustains 1.45-1.7 PFLOP/s on MI355X and one
 // of v_mfma_f32_16x16x32_f16 1.8-1.9 (both 2.3-2.4 with all-zero operands),
-// which is why f16 / bf16 run on the 16-row shape; for i8 and fp8 the 32-row
-// shapes are the faster ones. The clock drops under that limit, so every stall
-// cycle costs more time as well.
+// which is why f16 / bf16 run on the 16-row shape, and so does i8 (uniform
+// random bytes: 3.47 POP/s with the 32-row instruction, 4.16 with the 16-row
+// one). fp8 stays on 32x32x64: the 16-row shape is 8 % ahead there as well,
+// but its K-step is 128 bytes of a row, which the LDS rings of the tiles that
+// run two per compute unit cannot hold. The clock drops under that limit, so
+// every stall cycle costs more time as well.
 //
 // This header holds the kernel itself (the body as a device function, so that
 // the library's launcher and the code object built for a HAL executable can
