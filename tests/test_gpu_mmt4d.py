@@ -693,8 +693,8 @@ def test_i8_matmul_with_packed_rhs_in_one_kernel_is_bit_exact(uk, cuda, M, N, K,
     RHS, row-major result. Against the plain integer matmul of the oracle; row
     pitches of A and C wider than a row (the bytes between rows of C must stay
     untouched), ragged M and N, K in whole matrix-core steps of 32 (an even
-    number of them runs the kernel with two instructions per 64-byte step, an
-    odd number the one with 32-byte steps)."""
+    number of them runs the 16-row instruction on 64-byte steps, an odd number
+    the 32-row one on 32-byte steps)."""
     import torch
     lda, ldc = K + 16, N + 5
     A = synth.uniform_int8(1, M * K).reshape(M, K)
