@@ -147,28 +147,6 @@ struct S8Cfg16 {
     return __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c, 0, 0, 0);
   }
 };
-// i8 with two instructions per K-step (64 bytes of a row, the fp8 block
-// layout: lane l holds row l % 32, bytes 32 (l / 32) .. + 32 of the step, the
-// first instruction multiplies the low 16 of them, the second the high 16).
-// For a row-major left-hand side only: a K-step of 64 bytes lets four adjacent
-// lanes load 64 contiguous bytes of one row, which halves the cache lines a
-// load instruction touches against the 32-byte steps of S8Cfg.
-struct S8Cfg2 {
-  static constexpr float kStepUs = 0.76f;
-  static constexpr int kRows = 32;
-  typedef int8v frag_t;
-  typedef intx16 acc_t;
-  typedef int32_t out_t;
-  static constexpr int kElemBytes = 1;
-  static constexpr int kMfmaK = 64;
-  static constexpr int kSub = 2;
-  static constexpr bool kRowMajorLhsOnly = true;
-  __device__ static acc_t mfma(frag_t a, frag_t b, acc_t c, int = 0) {
-    c = __builtin_amdgcn_mfma_i32_32x32x32_i8(int4v{a[0], a[1], a[2], a[3]}, int4v{b[0], b[1], b[2], b[3]}, c, 0, 0, 0);
-    return __builtin_amdgcn_mfma_i32_32x32x32_i8(int4v{a[4], a[5], a[6], a[7]}, int4v{b[4], b[5], b[6], b[7]}, c, 0, 0, 0);
-  }
-  __device__ static int unit_scales() { return 0; }
-};
 struct F8Cfg {
   static constexpr float kStepUs = 0.86f;
   static constexpr int kRows = 32;     // the instruction's block is kRows x kRows

@@ -274,7 +274,7 @@ int launch_cfg(const MfmaArgs& a, hipStream_t s) {
     // quarter cache lines per row and K-step, each line asked for again on the
     // next step): tiles with more rows than columns pay most. Measured at
     // 2048 x 4096 x 4096 against the packed operand, K-steps of 64 bytes of a
-    // row (f16, i8 with two instructions per step; fp8 alike): 256x256 1.01,
+    // row (f16, i8 on the 16-row instruction; fp8 alike): 256x256 1.01,
     // 256x128 1.09-1.14, 128x256 1.02-1.03, 128x128 1.13; K-steps of 32 bytes
     // (i8 otherwise): 1.16, 1.37, 1.06, 1.28.
     if (a.lhs_row_major) {
