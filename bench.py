@@ -472,6 +472,22 @@ def extras(args, torch, iree_amd, F, synth, lhs, rhs, out, ex):
                     steps, warm)
     ex["mmt4d_i8_tops"] = round(flops / t / 1e12, 2)
     ex["mmt4d_i8_frac_of_peak"] = round(flops / t / 1e12 / PEAK_I8_TOPS, 4)
+    # The same outer sizes with four times the K: what does not depend on K
+    # (the gap between launches, the ring fill, the 64 MiB result: 14-15 us)
+    # weighs a quarter as much, so this is close to the rate of the K loop.
+    K4 = 4 * size
+    # (the operands above, four times along K: every outer row of tiles repeated)
+    li4 = li.view(M1, -1).repeat(1, 4).reshape(-1)
+    ri4 = ri.view(N1, -1).repeat(1, 4).reshape(-1)
+    _, t = gpu_time(torch, lambda: iree_amd.mmt4d(li4, ri4, oi, M1, N1, K4 // 16, 32, 32, 16,
+                                                  F.MMT4D_TYPE_S8S8S32), max(10, steps // 4), 3)
+    ex["mmt4d_i8_4096x4096x16384_tops"] = round(4 * flops / t / 1e12, 2)
+    lf4 = lhs.view(M1, -1).repeat(1, 4).reshape(-1)
+    rf4 = rhs.view(N1, -1).repeat(1, 4).reshape(-1)
+    _, t = gpu_time(torch, lambda: iree_amd.mmt4d(lf4, rf4, out, M1, N1, K4 // 8, 32, 32, 8,
+                                                  F.MMT4D_TYPE_F16F16F32), max(10, steps // 4), 3)
+    ex["mmt4d_f16_4096x4096x16384_tflops"] = round(4 * flops / t / 1e12, 2)
+    del li4, ri4, lf4, rf4
     # the same problem with a signed 4-bit right-hand side (S8S4S32): widened
     # to int8 in scratch memory, then the kernel above; two launches per call
     r4 = torch.from_numpy(synth.uniform_u4_packed(3, N1 * K1 * 32 * 16)).cuda()
